@@ -1,0 +1,390 @@
+"""ctypes binding of ``libcutile_hip.so`` for tests, the smoke check and ``bench.py``.
+
+The product is the C-ABI library (``include/cutile_hip.h``) and the C++ host surface
+above it; this module only marshals ``torch`` tensors (device memory and streams) into
+the ABI's plain records.  The directory name is not a Python identifier, so the package
+is imported through ``__graft_entry__.load_package()`` under the name ``cutile_rs_amd``.
+
+Launcher functions keep the reference's argument order (the ``#[cutile::entry]``
+signatures): outputs are passed as :class:`Partition` objects created with
+:func:`partition`, exactly where the reference takes ``tensor.partition([...])``.
+Nothing here computes on the CPU: if the library is missing, importing fails; if no
+GPU is present, every launch raises :class:`CutileError`.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcutile_hip.so")
+MAX_RANK = 4
+
+# cutile_dtype_t
+(F32, F64, F16, BF16, I8, I16, I32, I64, U8, U16, U32, U64, BOOL, F8E4M3FN, F8E5M2, F8E8M0FNU,
+ DTYPE_COUNT) = range(17)
+
+
+class CutileError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"[{status}] {message}")
+        self.status = status
+        self.message = message
+
+
+class TensorArg(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("dtype", C.c_int), ("rank", C.c_int32),
+                ("shape", C.c_int32 * MAX_RANK), ("strides", C.c_int32 * MAX_RANK)]
+
+
+class PartitionArg(C.Structure):
+    _fields_ = [("tensor", TensorArg), ("partition_shape", C.c_int32 * MAX_RANK),
+                ("partition_strides", C.c_int32 * MAX_RANK), ("prefix_coverage", C.c_int32)]
+
+
+class LaunchOpts(C.Structure):
+    _fields_ = [("grid", C.c_uint32 * 3), ("generics", C.POINTER(C.c_char_p)), ("n_generics", C.c_int32),
+                ("variant", C.c_char_p)]
+
+
+class KernelInfo(C.Structure):
+    _fields_ = [("function", C.c_void_p), ("symbol", C.c_char_p), ("variant", C.c_char_p),
+                ("block", C.c_uint32 * 3), ("lds_bytes", C.c_uint32), ("tile", C.c_int32 * 4)]
+
+
+class SpecBits(C.Structure):
+    _fields_ = [("shape_div", C.c_int32 * MAX_RANK), ("stride_div", C.c_int32 * MAX_RANK),
+                ("stride_one", C.c_int32 * MAX_RANK), ("base_ptr_div", C.c_int32), ("elements_disjoint", C.c_int32)]
+
+
+class DeviceProps(C.Structure):
+    _fields_ = [("compute_units", C.c_int32), ("clock_khz", C.c_int32), ("memory_clock_khz", C.c_int32),
+                ("memory_bus_bits", C.c_int32), ("l2_bytes", C.c_int32), ("lds_bytes_per_block", C.c_int32),
+                ("wavefront_size", C.c_int32), ("reserved", C.c_int32), ("total_memory_bytes", C.c_uint64)]
+
+
+class LaunchRecord(C.Structure):
+    _fields_ = [("symbol", C.c_char_p), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
+                ("shared_mem_bytes", C.c_uint32), ("stream", C.c_void_p), ("args", C.POINTER(C.c_ubyte)),
+                ("args_size", C.c_size_t), ("in_capture", C.c_int32), ("from_graph_replay", C.c_int32)]
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def lib() -> C.CDLL:
+    """The loaded C-ABI library.  Fails loudly when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: run `python cutile-rs_amd/build.py` "
+                              "(or __graft_entry__.build()) first; there is no fallback path")
+        L = C.CDLL(LIB_PATH)
+        L.cutile_last_error_message.restype = C.c_char_p
+        L.cutile_status_name.restype = C.c_char_p
+        L.cutile_status_name.argtypes = [C.c_int32]
+        L.cutile_version.restype = C.c_char_p
+        L.cutile_dtype_name.restype = C.c_char_p
+        L.cutile_dtype_name.argtypes = [C.c_int]
+        L.cutile_dtype_size.restype = C.c_size_t
+        L.cutile_dtype_size.argtypes = [C.c_int]
+        L.cutile_dtype_from_name.restype = C.c_int
+        L.cutile_dtype_from_name.argtypes = [C.c_char_p]
+        L.cutile_module_load_count.restype = C.c_uint64
+        L.cutile_testing_streams_created.restype = C.c_uint64
+        L.cutile_testing_bytes_allocated.restype = C.c_uint64
+        vp, f32, f64, i32, i64 = C.c_void_p, C.c_float, C.c_double, C.c_int32, C.c_int64
+        P = C.POINTER
+        sig = {
+            "cutile_launch_saxpy": [vp, P(PartitionArg), f64, P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_axpy": [vp, P(PartitionArg), f64, P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_add": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_full": [vp, f64, i64, P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_arange": [vp, P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_linspace": [vp, P(PartitionArg), f32, f32, P(LaunchOpts)],
+            "cutile_launch_convert": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
+            "cutile_launch_softmax": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
+            "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
+                                   P(LaunchOpts)],
+            "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
+                                                P(TensorArg), f32, P(LaunchOpts)],
+            "cutile_partition_grid": [P(PartitionArg), P(C.c_uint32 * 3)],
+            "cutile_infer_launch_grid": [P(C.c_uint32 * 3), P(P(PartitionArg)), i32, P(C.c_uint32 * 3)],
+            "cutile_compute_spec": [P(TensorArg), P(SpecBits)],
+            "cutile_kernel_lookup": [vp, C.c_char_p, P(C.c_char_p), i32, C.c_char_p, P(KernelInfo)],
+            "cutile_kernel_set_preferred_variant": [C.c_char_p, C.c_char_p],
+            "cutile_kernel_list": [P(C.c_char_p), i32],
+            "cutile_device_get": [i32, P(vp)],
+            "cutile_device_count": [P(i32)],
+            "cutile_device_name": [vp, C.c_char_p, C.c_size_t],
+            "cutile_device_arch": [vp, C.c_char_p, C.c_size_t],
+            "cutile_device_props": [vp, P(DeviceProps)],
+            "cutile_device_bind_to_thread": [vp],
+            "cutile_device_synchronize": [vp],
+            "cutile_stream_create": [vp, P(vp)],
+            "cutile_stream_release": [vp, vp],
+            "cutile_stream_synchronize": [vp],
+            "cutile_stream_query": [vp, P(i32)],
+            "cutile_event_create": [P(vp)],
+            "cutile_event_record": [vp, vp],
+            "cutile_event_synchronize": [vp],
+            "cutile_event_elapsed_ms": [vp, vp, P(f32)],
+            "cutile_event_destroy": [vp],
+            "cutile_malloc_async": [C.c_size_t, vp, P(vp)],
+            "cutile_free_async": [vp, vp],
+            "cutile_memset_d8_async": [vp, C.c_uint8, C.c_size_t, vp],
+            "cutile_memcpy_htod_async": [vp, vp, C.c_size_t, vp],
+            "cutile_memcpy_dtoh_async": [vp, vp, C.c_size_t, vp],
+            "cutile_memcpy_dtod_async": [vp, vp, C.c_size_t, vp],
+            "cutile_testing_use_fake_hip": [i32],
+            "cutile_testing_get_launch": [i32, P(LaunchRecord)],
+            "cutile_testing_inject_failure": [C.c_char_p, i32, i32],
+        }
+        for name, argtypes in sig.items():
+            fn = getattr(L, name)
+            fn.argtypes = argtypes
+            fn.restype = C.c_int32
+        _lib = L
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise CutileError(status, (lib().cutile_last_error_message() or b"").decode())
+
+
+# ---- torch plumbing -------------------------------------------------------------------------
+def _torch_dtype_code(t) -> int:
+    import torch
+
+    table = {torch.float32: F32, torch.float64: F64, torch.float16: F16, torch.bfloat16: BF16,
+             torch.int8: I8, torch.int16: I16, torch.int32: I32, torch.int64: I64, torch.uint8: U8,
+             torch.bool: BOOL}
+    for name, code in (("float8_e4m3fn", F8E4M3FN), ("float8_e5m2", F8E5M2), ("float8_e8m0fnu", F8E8M0FNU),
+                       ("uint16", U16), ("uint32", U32), ("uint64", U64)):
+        if hasattr(torch, name):
+            table[getattr(torch, name)] = code
+    return table[t.dtype]
+
+
+def tensor_arg(t, dtype: Optional[int] = None) -> TensorArg:
+    """A torch tensor as the ABI's tensor record.  ``dtype`` overrides the element type
+    (e.g. a uint8 tensor holding f8e4m3fn bytes)."""
+    a = TensorArg()
+    a.ptr = t.data_ptr()
+    a.dtype = _torch_dtype_code(t) if dtype is None else dtype
+    a.rank = t.dim()
+    for i in range(t.dim()):
+        a.shape[i] = t.shape[i]
+        a.strides[i] = t.stride(i)
+    return a
+
+
+@dataclass
+class Partition:
+    """``tensor.partition(shape)`` of the reference (cutile/src/tensor.rs:1417-1429): a
+    mutable tensor divided into disjoint tiles; its grid defines the launch grid."""
+    tensor: object
+    shape: Sequence[int]
+    prefix: bool = False          # partition_prefix(): the grid is an upper bound only
+    dtype: Optional[int] = None
+
+    def arg(self) -> PartitionArg:
+        p = PartitionArg()
+        p.tensor = tensor_arg(self.tensor, self.dtype)
+        rank = self.tensor.dim()
+        if len(self.shape) != rank:
+            raise CutileError(-5, f"partition rank {len(self.shape)} does not match tensor rank {rank}")
+        for i in range(rank):
+            p.partition_shape[i] = self.shape[i]
+            # partition strides = tensor strides (cutile/src/tensor.rs:1423-1427)
+            p.partition_strides[i] = self.tensor.stride(i)
+        p.prefix_coverage = int(self.prefix)
+        return p
+
+    def grid(self):
+        g = (C.c_uint32 * 3)()
+        check(lib().cutile_partition_grid(C.byref(self.arg()), C.byref(g)))
+        return tuple(g)
+
+
+def partition(tensor, shape: Sequence[int], prefix: bool = False, dtype: Optional[int] = None) -> Partition:
+    return Partition(tensor, list(shape), prefix, dtype)
+
+
+def _opts(grid=None, generics=None, variant=None):
+    o = LaunchOpts()
+    keep = []
+    if grid is not None:
+        for i in range(3):
+            o.grid[i] = grid[i]
+    if generics is not None:
+        arr = (C.c_char_p * len(generics))(*[str(g).encode() for g in generics])
+        keep.append(arr)
+        o.generics = C.cast(arr, C.POINTER(C.c_char_p))
+        o.n_generics = len(generics)
+    if variant is not None:
+        o.variant = variant.encode()
+    return o, keep
+
+
+def _stream(stream) -> int:
+    if stream is not None:
+        return int(stream)
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream if torch.cuda.is_available() else 0
+
+
+# ---- entry launchers (reference argument order) ---------------------------------------------
+def saxpy(y: Partition, a: float, x, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """y <- a*x + y.  cutile-examples/examples/saxpy.rs:12-17."""
+    o, _k = _opts(grid, generics, variant)
+    xa = tensor_arg(x)
+    check(lib().cutile_launch_saxpy(_stream(stream), C.byref(y.arg()), float(a), C.byref(xa), C.byref(o)))
+
+
+def axpy(z: Partition, a: float, x, y, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """z <- a*x + y (rank 1)."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x), tensor_arg(y)
+    check(lib().cutile_launch_axpy(_stream(stream), C.byref(z.arg()), float(a), C.byref(xa), C.byref(ya), C.byref(o)))
+
+
+def add(z: Partition, x, y, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """z <- x + y.  README.md:29-38 of the reference."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x), tensor_arg(y)
+    check(lib().cutile_launch_add(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), C.byref(o)))
+
+
+def full(value, t: Partition, *, stream=None, grid=None, variant=None) -> None:
+    o, _k = _opts(grid, None, variant)
+    check(lib().cutile_launch_full(_stream(stream), float(value), int(value), C.byref(t.arg()), C.byref(o)))
+
+
+def arange(t: Partition, *, stream=None, grid=None, variant=None) -> None:
+    o, _k = _opts(grid, None, variant)
+    check(lib().cutile_launch_arange(_stream(stream), C.byref(t.arg()), C.byref(o)))
+
+
+def linspace(t: Partition, start: float, step: float, *, stream=None, grid=None) -> None:
+    o, _k = _opts(grid, None, None)
+    check(lib().cutile_launch_linspace(_stream(stream), C.byref(t.arg()), float(start), float(step), C.byref(o)))
+
+
+def convert(src, dst: Partition, *, stream=None, grid=None) -> None:
+    o, _k = _opts(grid, None, None)
+    sa = tensor_arg(src)
+    check(lib().cutile_launch_convert(_stream(stream), C.byref(sa), C.byref(dst.arg()), C.byref(o)))
+
+
+def rms_norm_f16(x, w, out: Partition, eps: float, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """cutile-kernels/src/norms.rs:16-60."""
+    o, _k = _opts(grid, generics, variant)
+    xa, wa = tensor_arg(x), tensor_arg(w)
+    check(lib().cutile_launch_rms_norm_f16(_stream(stream), C.byref(xa), C.byref(wa), C.byref(out.arg()), float(eps),
+                                           C.byref(o)))
+
+
+def softmax(x, y: Partition, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """cutile-benchmarks/benches/softmax.rs:19-35."""
+    o, _k = _opts(grid, generics, variant)
+    xa = tensor_arg(x)
+    check(lib().cutile_launch_softmax(_stream(stream), C.byref(xa), C.byref(y.arg()), C.byref(o)))
+
+
+def gemm(z: Partition, x, y, k: int, *, accumulate: bool = True, stream=None, grid=None, generics=None,
+         variant=None) -> None:
+    """cutile-benchmarks/benches/gemm.rs:20-41 (z is read as the initial accumulator)."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x), tensor_arg(y)
+    check(lib().cutile_launch_gemm(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), int(k),
+                                   int(accumulate), C.byref(o)))
+
+
+def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_group_size: int = 1, *,
+         causal: bool = False, stream=None, grid=None, generics=None, variant=None) -> None:
+    """cutile-examples/examples/flash_attention_causal.rs:19-134."""
+    o, _k = _opts(grid, generics, variant)
+    qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
+    check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
+                                   float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def linear_tile_mxfp8(z: Partition, x, y, x_scales, y_scales, alpha: float = 1.0, *, stream=None, grid=None,
+                      generics=None, variant=None) -> None:
+    """cutile-examples/examples/mxfp8.rs:34-64.  x, y: uint8 (or float8_e4m3fn) tensors of
+    e4m3fn bytes; scales: uint8 (or float8_e8m0fnu) tensors of e8m0 bytes."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x, F8E4M3FN), tensor_arg(y, F8E4M3FN)
+    xsa, ysa = tensor_arg(x_scales, F8E8M0FNU), tensor_arg(y_scales, F8E8M0FNU)
+    check(lib().cutile_launch_linear_tile_mxfp8(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya),
+                                                C.byref(xsa), C.byref(ysa), float(alpha), C.byref(o)))
+
+
+# ---- table / device helpers -------------------------------------------------------------------
+def kernel_list() -> list[str]:
+    n = lib().cutile_kernel_list(None, 0)
+    arr = (C.c_char_p * n)()
+    lib().cutile_kernel_list(arr, n)
+    return [a.decode() for a in arr]
+
+
+def set_preferred_variant(function: str, variant: Optional[str]) -> None:
+    check(lib().cutile_kernel_set_preferred_variant(function.encode(), variant.encode() if variant else None))
+
+
+def device(ordinal: int = 0) -> int:
+    d = C.c_void_p()
+    check(lib().cutile_device_get(ordinal, C.byref(d)))
+    return d.value
+
+
+def device_props(ordinal: int = 0) -> DeviceProps:
+    p = DeviceProps()
+    check(lib().cutile_device_props(device(ordinal), C.byref(p)))
+    return p
+
+
+def device_arch(ordinal: int = 0) -> str:
+    buf = C.create_string_buffer(256)
+    check(lib().cutile_device_arch(device(ordinal), buf, 256))
+    return buf.value.decode()
+
+
+def kernel_lookup(function: str, generics: Sequence[str] = (), variant: Optional[str] = None,
+                  ordinal: int = 0) -> KernelInfo:
+    info = KernelInfo()
+    arr = (C.c_char_p * max(1, len(generics)))(*[str(g).encode() for g in generics])
+    check(lib().cutile_kernel_lookup(device(ordinal), function.encode(), arr, len(generics),
+                                     variant.encode() if variant else None, C.byref(info)))
+    return info
+
+
+class EventTimer:
+    """HIP-event timing on a given stream through the C ABI (cutile/src/bench.rs:162-211)."""
+
+    def __init__(self, stream=None):
+        self.stream = _stream(stream)
+        self.start_ev, self.stop_ev = C.c_void_p(), C.c_void_p()
+        check(lib().cutile_event_create(C.byref(self.start_ev)))
+        check(lib().cutile_event_create(C.byref(self.stop_ev)))
+
+    def start(self):
+        check(lib().cutile_event_record(self.start_ev, self.stream))
+
+    def stop(self) -> float:
+        check(lib().cutile_event_record(self.stop_ev, self.stream))
+        check(lib().cutile_event_synchronize(self.stop_ev))
+        ms = C.c_float()
+        check(lib().cutile_event_elapsed_ms(self.start_ev, self.stop_ev, C.byref(ms)))
+        return ms.value
+
+    def close(self):
+        lib().cutile_event_destroy(self.start_ev)
+        lib().cutile_event_destroy(self.stop_ev)

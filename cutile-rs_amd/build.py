@@ -1,0 +1,113 @@
+"""Builds the gfx950 code objects and the C-ABI host library, in tree.
+
+    python cutile-rs_amd/build.py [--force]
+
+Outputs (git-ignored, carried to the GPU box with the tree):
+    cutile-rs_amd/lib/*.hsaco          one ELF code object per kernel source
+    cutile-rs_amd/lib/libcutile_hip.so host library with the code objects embedded
+
+The device side is compiled by hipcc for gfx950 only; the host side is plain
+C++17 compiled by g++ and binds the HIP runtime with dlopen, so no GPU (and no
+HIP runtime) is needed to build or to load the library.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+KERNEL_DIR = os.path.join(ROOT, "csrc", "kernels")
+HOST_DIR = os.path.join(ROOT, "csrc", "host")
+LIB_DIR = os.path.join(ROOT, "lib")
+BUILD_DIR = os.path.join(ROOT, "build")
+LIB_PATH = os.path.join(LIB_DIR, "libcutile_hip.so")
+
+# image symbol -> kernel source
+IMAGES = {
+    "elementwise": "elementwise.hip",
+    "rowwise": "rowwise.hip",
+    "gemm": "gemm_bf16.hip",
+    "fmha": "fmha.hip",
+    "mxgemm": "mxfp8_gemm.hip",
+}
+HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "fake_hip.cpp"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+CXX = os.environ.get("CXX", "g++")
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950", "--cuda-device-only", "--no-gpu-bundle-output", "-c", "-O3", "-std=c++17",
+    # packed FP32 instructions are kept off on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+HOST_FLAGS = ["-std=c++17", "-O2", "-g0", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
+              "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-pthread"]
+
+
+def _newer(target: str, sources: list[str]) -> bool:
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(s) <= t for s in sources)
+
+
+def _run(cmd: list[str]) -> None:
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + res.stdout)
+        raise RuntimeError(f"build step failed: {cmd[0]} ... {cmd[-1]}")
+
+
+def build_code_objects(force: bool = False) -> dict[str, str]:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    headers = [os.path.join(KERNEL_DIR, f) for f in os.listdir(KERNEL_DIR) if f.endswith(".h")]
+    jobs = []
+    out = {}
+    for name, src in IMAGES.items():
+        src_path = os.path.join(KERNEL_DIR, src)
+        dst = os.path.join(LIB_DIR, name + ".hsaco")
+        out[name] = dst
+        if force or not _newer(dst, [src_path] + headers):
+            jobs.append([HIPCC] + DEVICE_FLAGS + ["-o", dst, src_path])
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        list(ex.map(_run, jobs))
+    return out
+
+
+def build_host_library(images: dict[str, str], force: bool = False) -> str:
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    embed = os.path.join(BUILD_DIR, "embed.S")
+    lines = ['.section .rodata', '']
+    for name, path in images.items():
+        lines += [f".global cutile_img_{name}_start", f".global cutile_img_{name}_end", ".balign 4096",
+                  f"cutile_img_{name}_start:", f'.incbin "{path}"', f"cutile_img_{name}_end:", ""]
+    lines += ['.section .note.GNU-stack,"",@progbits', ""]
+    text = "\n".join(lines)
+    if not os.path.exists(embed) or open(embed).read() != text:
+        with open(embed, "w") as f:
+            f.write(text)
+    sources = [os.path.join(HOST_DIR, s) for s in HOST_SOURCES]
+    deps = sources + [embed] + list(images.values()) + [
+        os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".h")
+    ] + [os.path.join(ROOT, "..", "include", "cutile_hip.h")]
+    if force or not _newer(LIB_PATH, deps):
+        objs = []
+        jobs = []
+        for s in sources + [embed]:
+            o = os.path.join(BUILD_DIR, os.path.basename(s) + ".o")
+            objs.append(o)
+            if force or not _newer(o, deps):
+                jobs.append([CXX] + HOST_FLAGS + ["-c", s, "-o", o])
+        with ThreadPoolExecutor(max_workers=6) as ex:
+            list(ex.map(_run, jobs))
+        _run([CXX, "-shared", "-o", LIB_PATH] + objs + ["-ldl", "-pthread", "-Wl,--no-undefined"])
+    return LIB_PATH
+
+
+def build(force: bool = False) -> str:
+    return build_host_library(build_code_objects(force), force)
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

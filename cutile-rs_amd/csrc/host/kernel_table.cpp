@@ -1,0 +1,249 @@
+// Part B of the C ABI: the table of precompiled gfx950 kernels (see kernel_table.h).
+#include "kernel_table.h"
+
+#include <atomic>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <mutex>
+
+// Code objects, embedded by embed.S (one ELF image per kernel source file).
+extern "C" {
+extern const unsigned char cutile_img_elementwise_start[], cutile_img_elementwise_end[];
+extern const unsigned char cutile_img_rowwise_start[], cutile_img_rowwise_end[];
+extern const unsigned char cutile_img_gemm_start[], cutile_img_gemm_end[];
+extern const unsigned char cutile_img_fmha_start[], cutile_img_fmha_end[];
+extern const unsigned char cutile_img_mxgemm_start[], cutile_img_mxgemm_end[];
+}
+
+namespace cutile {
+namespace {
+
+std::atomic<uint64_t> g_module_loads{0};
+std::mutex g_pref_mutex;
+std::map<std::string, std::string> g_preferred;
+
+struct ImageRef {
+  const unsigned char* start;
+  const unsigned char* end;
+};
+ImageRef image_ref(Image img) {
+  switch (img) {
+    case IMG_ELEMENTWISE: return {cutile_img_elementwise_start, cutile_img_elementwise_end};
+    case IMG_ROWWISE: return {cutile_img_rowwise_start, cutile_img_rowwise_end};
+    case IMG_GEMM: return {cutile_img_gemm_start, cutile_img_gemm_end};
+    case IMG_FMHA: return {cutile_img_fmha_start, cutile_img_fmha_end};
+    case IMG_MXGEMM: return {cutile_img_mxgemm_start, cutile_img_mxgemm_end};
+    default: return {nullptr, nullptr};
+  }
+}
+
+std::vector<KernelEntry> build_table() {
+  std::vector<KernelEntry> t;
+  auto add = [&](const char* fn, const char* variant, const char* symbol, Image img, uint32_t threads,
+                 uint32_t lds, int bm, int bn, int bk, int extra, const char* dtype, int64_t capacity,
+                 int rank) {
+    t.push_back(KernelEntry{fn, variant, symbol, img, {threads, 1, 1}, lds, {bm, bn, bk, extra}, dtype,
+                            capacity, rank});
+  };
+  // ---- elementwise / creation (256 threads, no LDS) ----
+#define EW(fn, dtype, suffix, rank) \
+  add(fn, dtype "_" suffix, fn "_entry__" dtype "_" suffix, IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, dtype, 0, rank)
+  {
+    EW("saxpy", "f32", "r1_flat", 1); EW("saxpy", "f32", "r2_flat", 2);
+    EW("saxpy", "f32", "r1_tiled", 1); EW("saxpy", "f32", "r2_tiled", 2);
+    EW("saxpy", "f16", "r1_flat", 1); EW("saxpy", "f16", "r2_flat", 2);
+    EW("saxpy", "f16", "r1_tiled", 1); EW("saxpy", "f16", "r2_tiled", 2);
+    EW("saxpy", "f64", "r1_flat", 1); EW("saxpy", "f64", "r2_flat", 2);
+    EW("saxpy", "f64", "r1_tiled", 1); EW("saxpy", "f64", "r2_tiled", 2);
+    EW("axpy", "f32", "r1_flat", 1); EW("axpy", "f32", "r1_tiled", 1);
+    EW("axpy", "f16", "r1_flat", 1); EW("axpy", "f16", "r1_tiled", 1);
+    EW("axpy", "f64", "r1_flat", 1); EW("axpy", "f64", "r1_tiled", 1);
+    EW("add", "f32", "r1_flat", 1); EW("add", "f32", "r1_tiled", 1); EW("add", "f32", "r2_tiled", 2);
+    EW("add", "f16", "r1_flat", 1); EW("add", "f16", "r1_tiled", 1); EW("add", "f16", "r2_tiled", 2);
+    EW("add", "bf16", "r1_flat", 1); EW("add", "bf16", "r1_tiled", 1); EW("add", "bf16", "r2_tiled", 2);
+  }
+#undef EW
+  static const char* kCreationTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64", "u8", "u16", "u32"};
+  static std::deque<std::string> names;  // keeps generated strings alive at stable addresses
+  auto keep = [&](std::string s) -> const char* {
+    names.push_back(std::move(s));
+    return names.back().c_str();
+  };
+  for (const char* ty : kCreationTypes) {
+    add("full", ty, keep(std::string("full_entry__") + ty), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, ty, 0, 1);
+    add("arange", ty, keep(std::string("arange_entry__") + ty), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, ty, 0, 1);
+  }
+  add("linspace", "f32", "linspace_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  static const char* kConvertTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64"};
+  for (const char* s : kConvertTypes)
+    for (const char* d : kConvertTypes)
+      add("convert", keep(std::string(s) + "_" + d), keep(std::string("convert_entry__") + s + "_" + d),
+          IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, s, 0, 1);
+
+  // ---- row-wise (256 threads; capacity = elements of one segment held in registers) ----
+  struct RowVariant { int wpr, vpl; };
+  static const RowVariant kRow[] = {{1, 1}, {1, 2}, {1, 4}, {1, 8}, {1, 16}, {2, 8}, {4, 4}, {4, 8}, {4, 16}};
+  for (auto rv : kRow) {
+    std::string v = "w" + std::to_string(rv.wpr) + "v" + std::to_string(rv.vpl);
+    add("rms_norm_f16", keep(v), keep("rms_norm_f16_entry__" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f16",
+        (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
+    add("softmax", keep("f16_" + v), keep("softmax_entry__f16_" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f16",
+        (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
+    add("softmax", keep("f32_" + v), keep("softmax_entry__f32_" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f32",
+        (int64_t)rv.wpr * 64 * rv.vpl * 4, 2);
+  }
+  add("rms_norm_f16", "generic", "rms_norm_f16_entry__generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
+  add("softmax", "f16_generic", "softmax_entry__f16_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
+  add("softmax", "f32_generic", "softmax_entry__f32_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
+
+  // ---- bf16 GEMM: LDS = 2 stages x (BM*BK + BK*BN) x 2 bytes ----
+  auto gemm = [&](const char* dtype, int bm, int bn, int bk, int wvm, int wvn) {
+    std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" +
+                    std::to_string(bk) + "_w" + std::to_string(wvm) + "x" + std::to_string(wvn);
+    add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64),
+        (uint32_t)(2 * (bm * bk + bk * bn) * 2), bm, bn, bk, 0, dtype, 0, 2);
+  };
+  gemm("bf16", 256, 256, 64, 2, 2);
+  gemm("bf16", 256, 256, 64, 2, 4);
+  gemm("bf16", 256, 256, 64, 4, 2);
+  gemm("bf16", 256, 128, 64, 2, 2);
+  gemm("bf16", 128, 256, 64, 2, 2);
+  gemm("bf16", 128, 128, 64, 2, 2);
+  gemm("bf16", 64, 128, 64, 2, 2);
+  gemm("bf16f32", 128, 128, 64, 2, 2);
+  gemm("bf16f32", 256, 256, 64, 2, 2);
+
+  // ---- FMHA: LDS = 2 stages x (K tile + V tile) ----
+  auto fmha = [&](const char* dtype, int bm, int bn, int d) {
+    std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" + std::to_string(d);
+    add("fmha", keep(v), keep("fmha_entry__" + v), IMG_FMHA, (uint32_t)(bm / 32 * 64),
+        (uint32_t)(2 * 2 * bn * d * 2), bm, bn, d, 0, dtype, 0, 3);
+  };
+  fmha("bf16", 128, 64, 128);
+  fmha("bf16", 128, 128, 128);
+  fmha("bf16", 256, 64, 128);
+  fmha("bf16", 128, 64, 64);
+  fmha("bf16", 64, 64, 64);
+  fmha("bf16", 64, 32, 32);
+  fmha("bf16", 32, 32, 32);
+  fmha("f16", 128, 64, 128);
+  fmha("f16", 128, 64, 64);
+  fmha("f16", 32, 32, 32);
+
+  // ---- MXFP8 GEMM: LDS = 2 stages x (BM + BN) x 128 bytes ----
+  auto mx = [&](const char* out, int bm, int bn, int wvm, int wvn) {
+    std::string v = std::string("mxfp8_") + out + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x128_w" +
+                    std::to_string(wvm) + "x" + std::to_string(wvn);
+    add("linear_tile", keep(v), keep("linear_tile_entry__" + v), IMG_MXGEMM, (uint32_t)(wvm * wvn * 64),
+        (uint32_t)(2 * (bm + bn) * 128), bm, bn, 128, 0, out, 0, 2);
+  };
+  mx("bf16", 256, 256, 2, 2);
+  mx("bf16", 256, 256, 2, 4);
+  mx("bf16", 128, 128, 2, 2);
+  mx("f32", 256, 256, 2, 2);
+  mx("f32", 128, 128, 2, 2);
+  mx("f32", 32, 32, 1, 1);
+  mx("f32", 64, 64, 1, 1);
+  return t;
+}
+
+}  // namespace
+
+const std::vector<KernelEntry>& kernel_table() {
+  static const std::vector<KernelEntry> table = build_table();
+  return table;
+}
+
+const KernelEntry* find_entry(const char* function, const std::string& variant) {
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, function) == 0 && variant == e.variant) return &e;
+  return nullptr;
+}
+
+std::string list_variants(const char* function) {
+  std::string s;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, function) == 0) {
+      if (!s.empty()) s += ", ";
+      s += e.variant;
+    }
+  return s;
+}
+
+std::string preferred_variant(const char* function) {
+  std::lock_guard<std::mutex> lock(g_pref_mutex);
+  auto it = g_preferred.find(function);
+  return it == g_preferred.end() ? std::string() : it->second;
+}
+
+void count_module_load() { g_module_loads.fetch_add(1, std::memory_order_relaxed); }
+
+cutile_status_t load_entry(cutile_device_t device, const KernelEntry* entry, hipFunction_t* fn) {
+  CUTILE_REQUIRE(device && entry && fn, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  // The device mutex makes the load single-flight: concurrent first launches of
+  // one kernel load its code object once (tile_kernel.rs:371-399,705-733).
+  std::lock_guard<std::mutex> lock(device->mutex);
+  auto fit = device->functions.find(entry->symbol);
+  if (fit != device->functions.end()) {
+    *fn = fit->second;
+    return CUTILE_SUCCESS;
+  }
+  CUTILE_API_OR_RETURN(api);
+  cutile_module* mod = nullptr;
+  auto mit = device->table_modules.find((int)entry->image);
+  if (mit == device->table_modules.end()) {
+    ImageRef img = image_ref(entry->image);
+    CUTILE_REQUIRE(img.start && img.end > img.start, CUTILE_ERR_KERNEL_NOT_FOUND,
+                   "no code object embedded for kernel %s", entry->symbol);
+    CUTILE_HIP_OR_RETURN(api, hipSetDevice(device->ordinal));
+    hipModule_t m = nullptr;
+    CUTILE_HIP_OR_RETURN(api, hipModuleLoadData(&m, img.start));
+    mod = new cutile_module();
+    mod->device = device;
+    mod->handle = m;
+    device->table_modules[(int)entry->image] = mod;
+    count_module_load();
+  } else {
+    mod = mit->second;
+  }
+  hipFunction_t f = nullptr;
+  CUTILE_HIP_OR_RETURN(api, hipModuleGetFunction(&f, mod->handle, entry->symbol));
+  device->functions[entry->symbol] = f;
+  *fn = f;
+  return CUTILE_SUCCESS;
+}
+
+}  // namespace cutile
+
+using namespace cutile;
+
+extern "C" {
+
+uint64_t cutile_module_load_count(void) { return g_module_loads.load(std::memory_order_relaxed); }
+
+int32_t cutile_kernel_list(const char** names, int32_t cap) {
+  static std::vector<std::string> labels = [] {
+    std::vector<std::string> v;
+    for (const auto& e : kernel_table()) v.push_back(std::string(e.function) + ":" + e.variant);
+    return v;
+  }();
+  for (int32_t i = 0; i < cap && i < (int32_t)labels.size(); ++i) names[i] = labels[i].c_str();
+  return (int32_t)labels.size();
+}
+
+cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const char* variant) {
+  CUTILE_REQUIRE(function, CUTILE_ERR_INVALID_ARGUMENT, "function is null");
+  std::lock_guard<std::mutex> lock(g_pref_mutex);
+  if (!variant) {
+    g_preferred.erase(function);
+    return CUTILE_SUCCESS;
+  }
+  CUTILE_REQUIRE(find_entry(function, variant) != nullptr, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no variant '%s' of kernel '%s'; available: %s", variant, function,
+                 list_variants(function).c_str());
+  g_preferred[function] = variant;
+  return CUTILE_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,846 @@
+// Parts C and D of the C ABI: the launch builder and the per-kernel launchers.
+//
+// A launcher here does what the reference's macro-generated launcher does in
+// execute() (cutile-macro/src/kernel_launcher_generator.rs:821-987): infer or
+// check the generics, validate every tensor against the kernel's signature,
+// infer and validate the launch grid from the output partition
+// (cutile/src/tile_kernel.rs:782-808,934-967), resolve the kernel (here: pick a
+// precompiled variant instead of compiling), push the arguments in signature
+// order (cutile/src/tensor.rs:1723-1739,2005-2016) and launch.  Every check runs
+// before any GPU work, as in the reference.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "common.h"
+#include "kernel_table.h"
+#include "runtime_state.h"
+
+using namespace cutile;
+
+namespace cutile {
+
+cutile_status_t current_device(cutile_device_t* device) {
+  if (cutile_status_t s = ensure_init()) return s;
+  CUTILE_API_OR_RETURN(api);
+  int ord = 0;
+  CUTILE_HIP_OR_RETURN(api, hipGetDevice(&ord));
+  return cutile_device_get(ord, device);
+}
+
+namespace {
+
+struct DTypeInfo {
+  const char* name;
+  size_t size;
+};
+const DTypeInfo kDTypes[CUTILE_DTYPE_COUNT] = {
+    {"f32", 4}, {"f64", 8}, {"f16", 2}, {"bf16", 2}, {"i8", 1},  {"i16", 2},      {"i32", 4},    {"i64", 8},
+    {"u8", 1},  {"u16", 2}, {"u32", 4}, {"u64", 8},  {"bool", 1}, {"f8e4m3fn", 1}, {"f8e5m2", 1}, {"f8e8m0fnu", 1}};
+
+uint16_t f32_to_f16_bits(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint32_t sign = (x >> 16) & 0x8000u, abs = x & 0x7fffffffu;
+  if (abs >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (abs > 0x7f800000u ? 0x0200u : 0));
+  if (abs >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+  if (abs < 0x38800000u) {
+    if (abs < 0x33000000u) return (uint16_t)sign;
+    int e = (int)(abs >> 23);
+    uint32_t man = (abs & 0x7fffffu) | 0x800000u;
+    int shift = 126 - e;
+    uint32_t q = man >> shift, rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+  uint32_t h = (((abs >> 23) - 112u) << 10) | ((abs & 0x7fffffu) >> 13);
+  uint32_t rem = abs & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;
+  return (uint16_t)(sign | h);
+}
+uint16_t f32_to_bf16_bits(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+
+// Encodes a scalar kernel argument of type `dt` from a double (floats) or an
+// int64 (integers).  Returns the number of bytes written, 0 if unsupported.
+size_t scalar_bits(cutile_dtype_t dt, double v, int64_t iv, unsigned char out[8]) {
+  switch (dt) {
+    case CUTILE_DTYPE_F32: { float f = (float)v; memcpy(out, &f, 4); return 4; }
+    case CUTILE_DTYPE_F64: memcpy(out, &v, 8); return 8;
+    case CUTILE_DTYPE_F16: { uint16_t h = f32_to_f16_bits((float)v); memcpy(out, &h, 2); return 2; }
+    case CUTILE_DTYPE_BF16: { uint16_t h = f32_to_bf16_bits((float)v); memcpy(out, &h, 2); return 2; }
+    case CUTILE_DTYPE_I8: case CUTILE_DTYPE_U8: case CUTILE_DTYPE_BOOL: { int8_t x = (int8_t)iv; memcpy(out, &x, 1); return 1; }
+    case CUTILE_DTYPE_I16: case CUTILE_DTYPE_U16: { int16_t x = (int16_t)iv; memcpy(out, &x, 2); return 2; }
+    case CUTILE_DTYPE_I32: case CUTILE_DTYPE_U32: { int32_t x = (int32_t)iv; memcpy(out, &x, 4); return 4; }
+    case CUTILE_DTYPE_I64: case CUTILE_DTYPE_U64: memcpy(out, &iv, 8); return 8;
+    default: return 0;
+  }
+}
+
+// Kernel-argument buffer laid out like the kernarg segment: every value at its
+// natural alignment, in push order.
+struct ArgPacker {
+  std::vector<unsigned char> buf;
+  void push(const void* v, size_t size, size_t align) {
+    size_t off = (buf.size() + align - 1) / align * align;
+    buf.resize(off + size);
+    memcpy(buf.data() + off, v, size);
+  }
+  template <typename T>
+  void push_val(T v) { push(&v, sizeof(T), alignof(T)); }
+  void push_tensor(const cutile_tensor_arg_t& t) {
+    push_val<void*>(t.ptr);
+    for (int i = 0; i < t.rank; ++i) push_val<int32_t>(t.shape[i]);
+    for (int i = 0; i < t.rank; ++i) push_val<int32_t>(t.strides[i]);
+  }
+  void push_partition(const cutile_partition_arg_t& p) {
+    push_tensor(p.tensor);
+    for (int i = 0; i < p.tensor.rank; ++i) push_val<int32_t>(p.partition_shape[i]);
+    for (int i = 0; i < p.tensor.rank; ++i) push_val<int32_t>(p.partition_strides[i]);
+  }
+  void push_tile_grid(const uint32_t g[3]) {
+    uint32_t v[4] = {g[0], g[1], g[2], 0};
+    push(v, sizeof(v), 4);
+  }
+};
+
+cutile_status_t launch_packed(hipFunction_t fn, const uint32_t grid[3], const uint32_t block[3],
+                              uint32_t dyn_lds, cutile_stream_t stream, ArgPacker& args) {
+  CUTILE_API_OR_RETURN(api);
+  CUTILE_REQUIRE(grid[0] > 0 && grid[1] > 0 && grid[2] > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "launch grid (%u, %u, %u) has a zero axis", grid[0], grid[1], grid[2]);
+  size_t size = args.buf.size();
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.buf.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                   HIP_LAUNCH_PARAM_END};
+  CUTILE_HIP_OR_RETURN(api, hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                                  dyn_lds, (hipStream_t)stream, nullptr, extra));
+  return CUTILE_SUCCESS;
+}
+
+// ---- validation helpers --------------------------------------------------------------------
+cutile_status_t check_tensor(const cutile_tensor_arg_t* t, const char* name, int rank_lo, int rank_hi) {
+  CUTILE_REQUIRE(t, CUTILE_ERR_INVALID_ARGUMENT, "%s is null", name);
+  CUTILE_REQUIRE(t->rank >= rank_lo && t->rank <= rank_hi, CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: expected rank %d%s, got %d", name, rank_lo, rank_lo == rank_hi ? "" : "+", t->rank);
+  CUTILE_REQUIRE((unsigned)t->dtype < CUTILE_DTYPE_COUNT, CUTILE_ERR_INVALID_ARGUMENT, "%s: bad dtype", name);
+  for (int i = 0; i < t->rank; ++i)
+    CUTILE_REQUIRE(t->shape[i] > 0, CUTILE_ERR_TENSOR, "%s: Shape dimensions must be positive.", name);
+  CUTILE_REQUIRE(t->ptr, CUTILE_ERR_INVALID_ARGUMENT, "%s: null device pointer", name);
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t check_partition(const cutile_partition_arg_t* p, const char* name, int rank_lo, int rank_hi) {
+  CUTILE_REQUIRE(p, CUTILE_ERR_INVALID_ARGUMENT, "%s is null", name);
+  if (cutile_status_t s = check_tensor(&p->tensor, name, rank_lo, rank_hi)) return s;
+  for (int i = 0; i < p->tensor.rank; ++i)
+    CUTILE_REQUIRE(p->partition_shape[i] > 0, CUTILE_ERR_TENSOR, "%s: partition shape must be positive", name);
+  return CUTILE_SUCCESS;
+}
+
+bool is_contiguous(const cutile_tensor_arg_t& t) {
+  int64_t expect = 1;
+  for (int i = t.rank - 1; i >= 0; --i) {
+    if (t.shape[i] != 1 && t.strides[i] != expect) return false;
+    expect *= t.shape[i];
+  }
+  return true;
+}
+bool same_shape(const cutile_tensor_arg_t& a, const cutile_tensor_arg_t& b) {
+  if (a.rank != b.rank) return false;
+  for (int i = 0; i < a.rank; ++i)
+    if (a.shape[i] != b.shape[i]) return false;
+  return true;
+}
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+int64_t numel(const cutile_tensor_arg_t& t) {
+  int64_t n = 1;
+  for (int i = 0; i < t.rank; ++i) n *= t.shape[i];
+  return n;
+}
+
+// Optional .generics() check: entry i of the caller's list must equal `expect`.
+cutile_status_t check_generic(const cutile_launch_opts_t* o, int i, const std::string& expect, const char* what) {
+  if (!o || !o->generics || i >= o->n_generics) return CUTILE_SUCCESS;
+  CUTILE_REQUIRE(o->generics[i] && expect == o->generics[i], CUTILE_ERR_KERNEL_LAUNCH,
+                 "generic %s: launcher was given '%s' but the arguments imply '%s'", what,
+                 o->generics[i] ? o->generics[i] : "(null)", expect.c_str());
+  return CUTILE_SUCCESS;
+}
+int generic_int(const cutile_launch_opts_t* o, int i, int fallback) {
+  if (!o || !o->generics || i >= o->n_generics || !o->generics[i]) return fallback;
+  return atoi(o->generics[i]);
+}
+
+struct Resolved {
+  const KernelEntry* entry = nullptr;
+  hipFunction_t fn = nullptr;
+  uint32_t tile_grid[3] = {0, 0, 0};
+};
+
+// Infers/validates the tile grid from the output partition and the caller's
+// explicit grid.
+cutile_status_t resolve_grid(const cutile_partition_arg_t* out, const cutile_launch_opts_t* opts, uint32_t grid[3]) {
+  uint32_t explicit_grid[3] = {0, 0, 0};
+  if (opts) memcpy(explicit_grid, opts->grid, sizeof(explicit_grid));
+  const cutile_partition_arg_t* parts[1] = {out};
+  return cutile_infer_launch_grid(explicit_grid, parts, 1, grid);
+}
+
+// Picks the variant: caller's hint, then the pinned preference, then `fallback`.
+cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* opts, const std::string& fallback,
+                              const std::vector<std::string>& acceptable, Resolved* r) {
+  std::string want;
+  if (opts && opts->variant) want = opts->variant;
+  if (want.empty()) {
+    std::string pref = preferred_variant(function);
+    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) want = pref;
+  }
+  if (want.empty()) want = fallback;
+  if (!acceptable.empty() && std::find(acceptable.begin(), acceptable.end(), want) == acceptable.end()) {
+    std::string list;
+    for (auto& a : acceptable) list += (list.empty() ? "" : ", ") + a;
+    return fail(CUTILE_ERR_KERNEL_NOT_FOUND, "variant '%s' of kernel '%s' does not fit these arguments; fitting: %s",
+                want.c_str(), function, list.c_str());
+  }
+  r->entry = find_entry(function, want);
+  CUTILE_REQUIRE(r->entry, CUTILE_ERR_KERNEL_NOT_FOUND, "no variant '%s' of kernel '%s'; available: %s",
+                 want.c_str(), function, list_variants(function).c_str());
+  cutile_device_t dev = nullptr;
+  if (cutile_status_t s = current_device(&dev)) return s;
+  return load_entry(dev, r->entry, &r->fn);
+}
+
+uint32_t div_up(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
+
+const char* float_dtype_name(cutile_dtype_t dt) { return kDTypes[dt].name; }
+
+}  // namespace
+}  // namespace cutile
+
+extern "C" {
+
+// ---- dtypes --------------------------------------------------------------------------------
+const char* cutile_dtype_name(cutile_dtype_t dtype) {
+  return (unsigned)dtype < CUTILE_DTYPE_COUNT ? kDTypes[dtype].name : "?";
+}
+size_t cutile_dtype_size(cutile_dtype_t dtype) { return (unsigned)dtype < CUTILE_DTYPE_COUNT ? kDTypes[dtype].size : 0; }
+cutile_dtype_t cutile_dtype_from_name(const char* name) {
+  if (name)
+    for (int i = 0; i < CUTILE_DTYPE_COUNT; ++i)
+      if (strcmp(kDTypes[i].name, name) == 0) return (cutile_dtype_t)i;
+  return CUTILE_DTYPE_COUNT;
+}
+
+// ---- grid inference ------------------------------------------------------------------------
+cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t grid[3]) {
+  CUTILE_REQUIRE(p && grid, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  const cutile_tensor_arg_t& t = p->tensor;
+  for (int i = 0; i < t.rank; ++i)
+    CUTILE_REQUIRE(t.shape[i] > 0, CUTILE_ERR_TENSOR, "Shape dimensions must be positive.");
+  CUTILE_REQUIRE(t.rank >= 1 && t.rank <= 3, CUTILE_ERR_TENSOR, "Mutable tensor must be at most rank 3.");
+  grid[0] = grid[1] = grid[2] = 1;
+  for (int i = 0; i < t.rank; ++i) {
+    CUTILE_REQUIRE(p->partition_shape[i] > 0, CUTILE_ERR_TENSOR, "partition shape must be positive");
+    grid[i] = div_up((uint32_t)t.shape[i], (uint32_t)p->partition_shape[i]);
+  }
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_infer_launch_grid(const uint32_t explicit_grid[3], const cutile_partition_arg_t* const* partitions,
+                                         int32_t n_partitions, uint32_t grid[3]) {
+  CUTILE_REQUIRE(grid, CUTILE_ERR_INVALID_ARGUMENT, "grid is null");
+  struct Bound { uint32_t g[3]; bool exact; };
+  std::vector<Bound> bounds;
+  for (int i = 0; i < n_partitions; ++i) {
+    Bound b;
+    if (cutile_status_t s = cutile_partition_grid(partitions[i], b.g)) return s;
+    b.exact = !partitions[i]->prefix_coverage;
+    bounds.push_back(b);
+  }
+  auto validate = [&](const uint32_t g[3]) -> cutile_status_t {
+    for (auto& b : bounds)
+      if (b.exact && (b.g[0] != g[0] || b.g[1] != g[1] || b.g[2] != g[2]))
+        return fail(CUTILE_ERR_KERNEL_LAUNCH,
+                    "launch grid (%u, %u, %u) does not match the inferred partition grid (%u, %u, %u)", g[0], g[1],
+                    g[2], b.g[0], b.g[1], b.g[2]);
+    for (auto& b : bounds)
+      if (!b.exact)
+        for (int k = 0; k < 3; ++k)
+          if (g[k] > b.g[k])
+            return fail(CUTILE_ERR_KERNEL_LAUNCH,
+                        "launch grid (%u, %u, %u) exceeds the partial-coverage partition grid (%u, %u, %u) on axis %d",
+                        g[0], g[1], g[2], b.g[0], b.g[1], b.g[2], k);
+    return CUTILE_SUCCESS;
+  };
+  const uint32_t zero[3] = {0, 0, 0};
+  const uint32_t* eg = explicit_grid ? explicit_grid : zero;
+  if (eg[0] || eg[1] || eg[2]) {
+    if (cutile_status_t s = validate(eg)) return s;
+    memcpy(grid, eg, 3 * sizeof(uint32_t));
+    return CUTILE_SUCCESS;
+  }
+  const Bound* first_exact = nullptr;
+  for (auto& b : bounds)
+    if (b.exact) { first_exact = &b; break; }
+  if (!first_exact) {
+    if (bounds.empty()) return fail(CUTILE_ERR_KERNEL_LAUNCH, "Launch grid required.");
+    return fail(CUTILE_ERR_KERNEL_LAUNCH,
+                "Launch grid required: a partial-coverage (partition_prefix) binding only bounds the grid; specify "
+                "the grid explicitly or bind with partition().");
+  }
+  if (cutile_status_t s = validate(first_exact->g)) return s;
+  memcpy(grid, first_exact->g, 3 * sizeof(uint32_t));
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_compute_spec(const cutile_tensor_arg_t* t, cutile_spec_bits_t* spec) {
+  CUTILE_REQUIRE(t && spec, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  CUTILE_REQUIRE(t->rank >= 0 && t->rank <= CUTILE_MAX_RANK, CUTILE_ERR_INVALID_ARGUMENT, "bad rank");
+  auto pow2 = [](int32_t v) -> int32_t {
+    if (v == 0) return 16;
+    int32_t d = v & (int32_t)(0u - (uint32_t)v);
+    return d < 16 && d > 0 ? d : 16;
+  };
+  memset(spec, 0, sizeof(*spec));
+  spec->base_ptr_div = pow2((int32_t)(uint64_t)(uintptr_t)t->ptr);
+  std::vector<std::pair<int32_t, int32_t>> sorted;
+  for (int i = 0; i < t->rank; ++i) {
+    spec->shape_div[i] = pow2(t->shape[i]);
+    spec->stride_div[i] = pow2(t->strides[i]);
+    spec->stride_one[i] = t->strides[i] == 1;
+    sorted.emplace_back(t->strides[i], t->shape[i]);
+  }
+  std::sort(sorted.begin(), sorted.end());
+  spec->elements_disjoint = sorted.empty() ? 1 : sorted[0].first > 0;
+  for (size_t i = 0; i + 1 < sorted.size(); ++i)
+    if (sorted[i + 1].first <= 0 || (int64_t)sorted[i + 1].first < (int64_t)sorted[i].first * sorted[i].second) {
+      spec->elements_disjoint = 0;
+      break;
+    }
+  return CUTILE_SUCCESS;
+}
+
+// ---- Part C: launch builder ----------------------------------------------------------------
+}  // extern "C"
+
+struct cutile_launch {
+  hipFunction_t function = nullptr;
+  ArgPacker args;
+  uint32_t grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+  uint32_t smem = 0;
+  bool configured = false;
+};
+
+extern "C" {
+
+cutile_status_t cutile_launch_create(cutile_function_t function, cutile_launch_t* launch) {
+  CUTILE_REQUIRE(function && launch, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  auto* l = new cutile_launch();
+  l->function = (hipFunction_t)function;
+  *launch = l;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_launch_destroy(cutile_launch_t launch) {
+  delete launch;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_launch_push_arg(cutile_launch_t launch, const void* value, size_t size, size_t align) {
+  CUTILE_REQUIRE(launch && value && size, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  CUTILE_REQUIRE(align && (align & (align - 1)) == 0, CUTILE_ERR_INVALID_ARGUMENT, "alignment must be a power of two");
+  launch->args.push(value, size, align);
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_launch_push_device_ptr(cutile_launch_t launch, void* device_ptr) {
+  CUTILE_REQUIRE(launch, CUTILE_ERR_INVALID_ARGUMENT, "launch is null");
+  launch->args.push_val<void*>(device_ptr);
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_launch_set_config(cutile_launch_t launch, const uint32_t grid[3], const uint32_t block[3],
+                                         uint32_t shared_mem_bytes) {
+  CUTILE_REQUIRE(launch && grid && block, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  memcpy(launch->grid, grid, sizeof(launch->grid));
+  memcpy(launch->block, block, sizeof(launch->block));
+  launch->smem = shared_mem_bytes;
+  launch->configured = true;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_launch_execute(cutile_launch_t launch, cutile_stream_t stream) {
+  CUTILE_REQUIRE(launch, CUTILE_ERR_INVALID_ARGUMENT, "launch is null");
+  CUTILE_REQUIRE(launch->configured, CUTILE_ERR_KERNEL_LAUNCH, "Launch grid required.");
+  return launch_packed(launch->function, launch->grid, launch->block, launch->smem, stream, launch->args);
+}
+
+// ---- Part B: generic lookup ----------------------------------------------------------------
+cutile_status_t cutile_kernel_lookup(cutile_device_t device, const char* function, const char* const* generics,
+                                     int32_t n_generics, const char* variant, cutile_kernel_info_t* info) {
+  CUTILE_REQUIRE(device && function && info, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  const KernelEntry* found = nullptr;
+  std::string want = variant ? variant : preferred_variant(function);
+  for (const auto& e : kernel_table()) {
+    if (strcmp(e.function, function) != 0) continue;
+    if (!want.empty()) {
+      if (want == e.variant) { found = &e; break; }
+      continue;
+    }
+    // Match on generics: a dtype string must equal the entry's dtype; integer
+    // generics are compared against the entry's tile shape, in order.
+    bool ok = true;
+    int tile_i = 0;
+    for (int i = 0; i < n_generics && ok; ++i) {
+      const char* gstr = generics[i];
+      if (!gstr) { ok = false; break; }
+      if (cutile_dtype_from_name(gstr) != CUTILE_DTYPE_COUNT) {
+        ok = strncmp(e.dtype, gstr, strlen(gstr)) == 0;
+      } else if (tile_i < 3 && e.tile[tile_i] != 0) {
+        ok = atoi(gstr) == e.tile[tile_i];
+        ++tile_i;
+      }
+    }
+    if (ok) { found = &e; break; }
+  }
+  if (!found) {
+    std::string key;
+    for (int i = 0; i < n_generics; ++i) key += std::string(i ? ", " : "") + (generics[i] ? generics[i] : "?");
+    return fail(CUTILE_ERR_KERNEL_NOT_FOUND, "no precompiled variant of %s<%s>%s%s; available: %s", function,
+                key.c_str(), want.empty() ? "" : " named ", want.c_str(), list_variants(function).c_str());
+  }
+  hipFunction_t fn = nullptr;
+  if (cutile_status_t s = load_entry(device, found, &fn)) return s;
+  info->function = fn;
+  info->symbol = found->symbol;
+  info->variant = found->variant;
+  memcpy(info->block, found->block, sizeof(info->block));
+  info->lds_bytes = found->lds_bytes;
+  memcpy(info->tile, found->tile, sizeof(info->tile));
+  return CUTILE_SUCCESS;
+}
+
+// ---- Part D: entry launchers ---------------------------------------------------------------
+static cutile_status_t launch_elementwise3(const char* fn_name, cutile_stream_t stream,
+                                           const cutile_partition_arg_t* out, const double* a,
+                                           const cutile_tensor_arg_t* in0, const cutile_tensor_arg_t* in1,
+                                           bool in_place, const cutile_launch_opts_t* opts) {
+  // out <- f(in0, in1) (or f(a, in0, in1)).  For the in-place saxpy, in1 is null
+  // and the second operand is `out` itself.
+  if (cutile_status_t s = check_partition(out, "output", 1, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  const int rank = ot.rank;
+  if (cutile_status_t s = check_tensor(in0, "x", rank, rank)) return s;
+  if (in1)
+    if (cutile_status_t s = check_tensor(in1, "y", rank, rank)) return s;
+  CUTILE_REQUIRE(in0->dtype == ot.dtype && (!in1 || in1->dtype == ot.dtype), CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: all operands must have element type %s", fn_name, cutile_dtype_name(ot.dtype));
+  const std::string dt = cutile_dtype_name(ot.dtype);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  uint32_t full[3];
+  cutile_partition_grid(out, full);
+  const bool full_cover = tg[0] == full[0] && tg[1] == full[1] && tg[2] == full[2];
+
+  bool flat_ok = is_contiguous(ot) && is_contiguous(*in0) && same_shape(ot, *in0) && aligned16(ot.ptr) &&
+                 aligned16(in0->ptr) && (rank == 1 || full_cover);
+  if (in1) flat_ok = flat_ok && is_contiguous(*in1) && same_shape(ot, *in1) && aligned16(in1->ptr);
+  const std::string r = "_r" + std::to_string(rank);
+  std::vector<std::string> acceptable;
+  if (flat_ok && find_entry(fn_name, dt + r + "_flat")) acceptable.push_back(dt + r + "_flat");
+  if (find_entry(fn_name, dt + r + "_tiled")) acceptable.push_back(dt + r + "_tiled");
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND, "no precompiled variant of %s<%s> for rank %d; available: %s",
+                 fn_name, dt.c_str(), rank, list_variants(fn_name).c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry(fn_name, opts, acceptable[0], acceptable, &res)) return s;
+
+  ArgPacker args;
+  args.push_partition(*out);
+  if (a) {
+    unsigned char bits[8];
+    size_t n = scalar_bits(ot.dtype, *a, (int64_t)*a, bits);
+    args.push(bits, n, n);
+  }
+  args.push_tensor(*in0);
+  if (in1) args.push_tensor(*in1);
+  args.push_tile_grid(tg);
+
+  uint32_t grid[3] = {tg[0], tg[1], tg[2]};
+  if (strstr(res.entry->variant, "_flat")) {
+    uint64_t count = rank == 1 ? std::min<uint64_t>((uint64_t)tg[0] * out->partition_shape[0], ot.shape[0]) : (uint64_t)numel(ot);
+    uint64_t per_wg = 256ull * 4ull * (16 / cutile_dtype_size(ot.dtype));
+    grid[0] = std::max<uint32_t>(1, div_up(count, per_wg));
+    grid[1] = grid[2] = 1;
+  }
+  (void)in_place;
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_saxpy(cutile_stream_t stream, const cutile_partition_arg_t* y, double a,
+                                    const cutile_tensor_arg_t* x, const cutile_launch_opts_t* opts) {
+  return launch_elementwise3("saxpy", stream, y, &a, x, nullptr, true, opts);
+}
+cutile_status_t cutile_launch_axpy(cutile_stream_t stream, const cutile_partition_arg_t* z, double a,
+                                   const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                   const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(z && z->tensor.rank == 1, CUTILE_ERR_KERNEL_LAUNCH, "axpy: output must be rank 1");
+  return launch_elementwise3("axpy", stream, z, &a, x, y, false, opts);
+}
+cutile_status_t cutile_launch_add(cutile_stream_t stream, const cutile_partition_arg_t* z, const cutile_tensor_arg_t* x,
+                                  const cutile_tensor_arg_t* y, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(y, CUTILE_ERR_INVALID_ARGUMENT, "y is null");
+  return launch_elementwise3("add", stream, z, nullptr, x, y, false, opts);
+}
+
+static cutile_status_t launch_creation(const char* fn_name, cutile_stream_t stream, const cutile_partition_arg_t* t,
+                                       const unsigned char* scalar, size_t scalar_size, bool scalar_first,
+                                       const float* extra_f32, int n_extra, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(t, "tensor", 1, 1)) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(t, opts, tg)) return s;
+  const std::string dt = cutile_dtype_name(t->tensor.dtype);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry(fn_name, opts, dt, {dt}, &res)) return s;
+  ArgPacker args;
+  if (scalar && scalar_first) args.push(scalar, scalar_size, scalar_size);
+  args.push_partition(*t);
+  for (int i = 0; i < n_extra; ++i) args.push_val<float>(extra_f32[i]);
+  args.push_tile_grid(tg);
+  uint64_t count = std::min<uint64_t>((uint64_t)tg[0] * t->partition_shape[0], t->tensor.shape[0]);
+  uint32_t grid[3] = {std::min<uint32_t>(std::max<uint32_t>(1, div_up(count, 256 * 4)), 16384), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_full(cutile_stream_t stream, double value, int64_t int_value,
+                                   const cutile_partition_arg_t* t, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(t, CUTILE_ERR_INVALID_ARGUMENT, "tensor is null");
+  unsigned char bits[8];
+  size_t n = scalar_bits(t->tensor.dtype, value, int_value, bits);
+  CUTILE_REQUIRE(n, CUTILE_ERR_KERNEL_NOT_FOUND, "full: unsupported element type %s", cutile_dtype_name(t->tensor.dtype));
+  return launch_creation("full", stream, t, bits, n, true, nullptr, 0, opts);
+}
+cutile_status_t cutile_launch_arange(cutile_stream_t stream, const cutile_partition_arg_t* t,
+                                     const cutile_launch_opts_t* opts) {
+  return launch_creation("arange", stream, t, nullptr, 0, false, nullptr, 0, opts);
+}
+cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_partition_arg_t* t, float start, float step,
+                                       const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(t && t->tensor.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_LAUNCH, "linspace: tensor must be f32");
+  float extra[2] = {start, step};
+  return launch_creation("linspace", stream, t, nullptr, 0, false, extra, 2, opts);
+}
+
+cutile_status_t cutile_launch_convert(cutile_stream_t stream, const cutile_tensor_arg_t* src,
+                                      const cutile_partition_arg_t* dst, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(src, "src", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(dst, "dst", 1, 1)) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(dst, opts, tg)) return s;
+  const std::string v = std::string(cutile_dtype_name(src->dtype)) + "_" + cutile_dtype_name(dst->tensor.dtype);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("convert", opts, v, {v}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*src);
+  args.push_partition(*dst);
+  args.push_tile_grid(tg);
+  uint64_t count = std::min<uint64_t>((uint64_t)tg[0] * dst->partition_shape[0], dst->tensor.shape[0]);
+  uint32_t grid[3] = {std::min<uint32_t>(std::max<uint32_t>(1, div_up(count, 256 * 4)), 16384), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+// Row-wise kernels: variants that hold a whole segment in registers, smallest first.
+static std::vector<std::string> fitting_row_variants(const char* fn_name, const std::string& prefix, int64_t seg_len) {
+  std::vector<const KernelEntry*> fit;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, fn_name) == 0 && e.capacity >= seg_len &&
+        strncmp(e.variant, prefix.c_str(), prefix.size()) == 0)
+      fit.push_back(&e);
+  std::stable_sort(fit.begin(), fit.end(), [](const KernelEntry* a, const KernelEntry* b) {
+    if (a->capacity != b->capacity) return a->capacity < b->capacity;
+    return a->tile[3] < b->tile[3];  // fewer wavefronts per segment first
+  });
+  std::vector<std::string> names;
+  for (auto* e : fit) names.push_back(e->variant);
+  return names;
+}
+
+cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                           const cutile_tensor_arg_t* w, const cutile_partition_arg_t* out, float eps,
+                                           const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(w, "w", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 2, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F16 && w->dtype == CUTILE_DTYPE_F16 && ot.dtype == CUTILE_DTYPE_F16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "rms_norm_f16: x, w and out must be f16");
+  const int32_t n = x->shape[1];
+  // Signature: x [-1, N], w [N], out tiles [1, N].
+  CUTILE_REQUIRE(w->shape[0] == n, CUTILE_ERR_KERNEL_LAUNCH, "rms_norm_f16: w has %d elements, expected N = %d", w->shape[0], n);
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == n, CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_f16: out must be partitioned [1, %d], got [%d, %d]", n, out->partition_shape[0],
+                 out->partition_shape[1]);
+  CUTILE_REQUIRE(ot.shape[1] == n && ot.shape[0] <= x->shape[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_f16: out is [%d, %d] but x is [%d, %d]", ot.shape[0], ot.shape[1], x->shape[0], n);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(n), "N")) return s;
+  const int block = generic_int(opts, 1, 0);
+  CUTILE_REQUIRE(block >= 0 && (block == 0 || n % block == 0), CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_f16: N = %d is not a multiple of BLOCK_SIZE = %d", n, block);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+
+  const bool vec_ok = n % 8 == 0 && x->strides[1] == 1 && ot.strides[1] == 1 && w->strides[0] == 1 &&
+                      x->strides[0] % 8 == 0 && ot.strides[0] % 8 == 0 && aligned16(x->ptr) && aligned16(ot.ptr) &&
+                      aligned16(w->ptr);
+  std::vector<std::string> acceptable;
+  if (vec_ok) acceptable = fitting_row_variants("rms_norm_f16", "w", n);
+  acceptable.push_back("generic");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("rms_norm_f16", opts, acceptable[0], acceptable, &res)) return s;
+
+  ArgPacker args;
+  args.push_tensor(*x);
+  args.push_tensor(*w);
+  args.push_partition(*out);
+  args.push_val<float>(eps);
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>(tg[0], ot.shape[0]);
+  uint32_t grid[3] = {1, 1, 1};
+  if (res.entry->capacity > 0) {
+    const int rows_per_wg = 4 / res.entry->tile[3];
+    grid[0] = div_up(rows, rows_per_wg);
+  } else {
+    grid[0] = (uint32_t)std::min<uint64_t>(rows, 1u << 20);
+  }
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                      const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_partition(y, "y", 2, 2)) return s;
+  const cutile_tensor_arg_t& yt = y->tensor;
+  CUTILE_REQUIRE(x->dtype == yt.dtype && (x->dtype == CUTILE_DTYPE_F16 || x->dtype == CUTILE_DTYPE_F32),
+                 CUTILE_ERR_KERNEL_LAUNCH, "softmax: x and y must both be f16 or both f32");
+  const int32_t bm = y->partition_shape[0], bn = y->partition_shape[1];
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bn), "BN")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(y, opts, tg)) return s;
+  const std::string dt = cutile_dtype_name(x->dtype);
+  const int e = 16 / (int)cutile_dtype_size(x->dtype);
+  const uint64_t rows = std::min<uint64_t>((uint64_t)tg[0] * bm, yt.shape[0]);
+  const bool vec_ok = bn % e == 0 && x->shape[1] % e == 0 && yt.shape[1] % e == 0 && x->strides[1] == 1 &&
+                      yt.strides[1] == 1 && x->strides[0] % e == 0 && yt.strides[0] % e == 0 && aligned16(x->ptr) &&
+                      aligned16(yt.ptr) && (uint64_t)x->shape[0] >= rows;
+  std::vector<std::string> acceptable;
+  if (vec_ok) acceptable = fitting_row_variants("softmax", dt + "_w", bn);
+  acceptable.push_back(dt + "_generic");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("softmax", opts, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*x);
+  args.push_partition(*y);
+  args.push_tile_grid(tg);
+  const uint64_t segments = rows * tg[1];
+  uint32_t grid[3] = {1, 1, 1};
+  if (res.entry->capacity > 0)
+    grid[0] = div_up(segments, 4 / res.entry->tile[3]);
+  else
+    grid[0] = (uint32_t)std::min<uint64_t>(segments, 1u << 20);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z, const cutile_tensor_arg_t* x,
+                                   const cutile_tensor_arg_t* y, int32_t k, int32_t accumulate,
+                                   const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(z, "z", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(y, "y", 2, 2)) return s;
+  const cutile_tensor_arg_t& zt = z->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_BF16 && y->dtype == CUTILE_DTYPE_BF16, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "gemm: precompiled variants take bf16 x and y (got %s, %s)", cutile_dtype_name(x->dtype),
+                 cutile_dtype_name(y->dtype));
+  CUTILE_REQUIRE(zt.dtype == CUTILE_DTYPE_BF16 || zt.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "gemm: z must be bf16 or f32");
+  const int32_t bm = z->partition_shape[0], bn = z->partition_shape[1];
+  const int bk_user = generic_int(opts, 3, 64);
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(bn), "BN")) return s;
+  CUTILE_REQUIRE(bk_user > 0, CUTILE_ERR_KERNEL_LAUNCH, "gemm: BK must be positive");
+  CUTILE_REQUIRE(k >= 0, CUTILE_ERR_KERNEL_LAUNCH, "gemm: k must be non-negative");
+  // The tile program runs k / BK whole K tiles (integer division).
+  const int32_t k_total = (k / bk_user) * bk_user;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(z, opts, tg)) return s;
+  CUTILE_REQUIRE(x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
+                     y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
+                     aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
+                     k_total % 8 == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "gemm: precompiled variants need row-major operands with unit inner stride, 16-byte aligned rows "
+                 "and K, N multiples of 8");
+  const std::string dt = zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
+  std::vector<std::string> acceptable;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn)
+      acceptable.push_back(e.variant);
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of gemm<%s, %d, %d, %d>; available: %s", dt.c_str(), bm, bn, bk_user,
+                 list_variants("gemm").c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("gemm", opts, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_tensor(*x);
+  args.push_tensor(*y);
+  args.push_val<int32_t>(k_total);
+  args.push_tile_grid(tg);
+  args.push_val<int32_t>(accumulate ? 1 : 0);
+  uint32_t grid[3] = {tg[0] * tg[1], 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partition_arg_t* out, const cutile_tensor_arg_t* q,
+                                   const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v, float qk_scale,
+                                   int32_t input_pos, int32_t query_group_size, int32_t causal,
+                                   const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(out, "out", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(q, "q", 4, 4)) return s;
+  if (cutile_status_t s = check_tensor(k, "k", 4, 4)) return s;
+  if (cutile_status_t s = check_tensor(v, "v", 4, 4)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE((q->dtype == CUTILE_DTYPE_BF16 || q->dtype == CUTILE_DTYPE_F16) && k->dtype == q->dtype &&
+                     v->dtype == q->dtype && ot.dtype == q->dtype,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "fmha: precompiled variants take bf16 or f16 q, k, v, out of one type");
+  const int32_t b = q->shape[0], h = q->shape[1], m = q->shape[2], d = q->shape[3];
+  const int32_t bm = out->partition_shape[1], dd = out->partition_shape[2];
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && dd == d, CUTILE_ERR_KERNEL_LAUNCH,
+                 "fmha: out must be partitioned [1, BM, %d], got [%d, %d, %d]", d, out->partition_shape[0], bm, dd);
+  CUTILE_REQUIRE(ot.shape[0] == b * h && ot.shape[1] == m && ot.shape[2] == d, CUTILE_ERR_KERNEL_LAUNCH,
+                 "fmha: out is [%d, %d, %d], expected [b*h = %d, m = %d, d = %d]", ot.shape[0], ot.shape[1], ot.shape[2],
+                 b * h, m, d);
+  CUTILE_REQUIRE(query_group_size > 0 && h % query_group_size == 0 && k->shape[1] * query_group_size == h &&
+                     v->shape[1] == k->shape[1],
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha: %d query heads, %d kv heads, query_group_size %d do not agree", h,
+                 k->shape[1], query_group_size);
+  CUTILE_REQUIRE(k->shape[0] == b && v->shape[0] == b && k->shape[3] == d && v->shape[3] == d &&
+                     k->shape[2] == v->shape[2],
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha: k / v shapes do not match q");
+  CUTILE_REQUIRE(input_pos >= 0, CUTILE_ERR_KERNEL_LAUNCH, "fmha: input_pos must be non-negative");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(d), "D")) return s;
+  const int bn_user = generic_int(opts, 1, 0);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  CUTILE_REQUIRE(q->strides[3] == 1 && k->strides[3] == 1 && v->strides[3] == 1 && ot.strides[2] == 1 &&
+                     q->strides[2] % 8 == 0 && k->strides[2] % 8 == 0 && v->strides[2] % 8 == 0 &&
+                     ot.strides[1] % 4 == 0 && aligned16(q->ptr) && aligned16(k->ptr) && aligned16(v->ptr) &&
+                     aligned16(ot.ptr) && q->strides[0] % 8 == 0 && q->strides[1] % 8 == 0 && k->strides[0] % 8 == 0 &&
+                     k->strides[1] % 8 == 0 && v->strides[0] % 8 == 0 && v->strides[1] % 8 == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "fmha: precompiled variants need unit head-dim stride and 16-byte aligned rows");
+  const std::string dt = cutile_dtype_name(q->dtype);
+  std::vector<std::string> acceptable, same_bn;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, "fmha") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[2] == d) {
+      acceptable.push_back(e.variant);
+      if (e.tile[1] == bn_user) same_bn.push_back(e.variant);
+    }
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of fmha<%s, BM=%d, D=%d>; available: %s", dt.c_str(), bm, d,
+                 list_variants("fmha").c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("fmha", opts, same_bn.empty() ? acceptable[0] : same_bn[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*out);
+  args.push_tensor(*q);
+  args.push_tensor(*k);
+  args.push_tensor(*v);
+  args.push_val<float>(qk_scale);
+  args.push_val<int32_t>(input_pos);
+  args.push_val<int32_t>(query_group_size);
+  args.push_val<int32_t>(causal ? 1 : 0);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {tg[0], tg[1], 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                                const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                                const cutile_tensor_arg_t* xs, const cutile_tensor_arg_t* ys, float alpha,
+                                                const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(z, "z", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(y, "y", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(xs, "x_scales", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(ys, "y_scales", 2, 2)) return s;
+  const cutile_tensor_arg_t& zt = z->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F8E4M3FN && y->dtype == CUTILE_DTYPE_F8E4M3FN &&
+                     xs->dtype == CUTILE_DTYPE_F8E8M0FNU && ys->dtype == CUTILE_DTYPE_F8E8M0FNU,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "linear_tile: precompiled variants take f8e4m3fn data with f8e8m0fnu scales");
+  CUTILE_REQUIRE(zt.dtype == CUTILE_DTYPE_F32 || zt.dtype == CUTILE_DTYPE_BF16, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile: z must be f32 or bf16");
+  const int32_t M = x->shape[0], K = x->shape[1], N = y->shape[0];
+  CUTILE_REQUIRE(y->shape[1] == K, CUTILE_ERR_KERNEL_LAUNCH, "linear_tile: x is [%d, %d] but y is [%d, %d]", M, K, N, y->shape[1]);
+  CUTILE_REQUIRE(K % 32 == 0 && xs->shape[0] == M && xs->shape[1] == K / 32 && ys->shape[0] == N && ys->shape[1] == K / 32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "linear_tile: scales must be [M, K/32] and [N, K/32] with K a multiple of 32");
+  CUTILE_REQUIRE(zt.shape[0] == M && zt.shape[1] == N, CUTILE_ERR_KERNEL_LAUNCH, "linear_tile: z is [%d, %d], expected [%d, %d]",
+                 zt.shape[0], zt.shape[1], M, N);
+  const int32_t bm = z->partition_shape[0], bn = z->partition_shape[1];
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bn), "BN")) return s;
+  const int bk_user = generic_int(opts, 2, 128);
+  CUTILE_REQUIRE(bk_user > 0 && bk_user % 32 == 0 && generic_int(opts, 3, bk_user / 32) == bk_user / 32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "linear_tile: BK must be a multiple of 32 and BK_SCALES = BK/32");
+  CUTILE_REQUIRE(K % bk_user == 0, CUTILE_ERR_KERNEL_LAUNCH, "linear_tile: K = %d is not a multiple of BK = %d", K, bk_user);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(z, opts, tg)) return s;
+  uint32_t full[3];
+  cutile_partition_grid(z, full);
+  const bool full_cover = tg[0] == full[0] && tg[1] == full[1];
+  CUTILE_REQUIRE(K % 128 == 0 && x->strides[1] == 1 && y->strides[1] == 1 && xs->strides[1] == 1 && ys->strides[1] == 1 &&
+                     zt.strides[1] == 1 && x->strides[0] % 16 == 0 && y->strides[0] % 16 == 0 && xs->strides[0] % 4 == 0 &&
+                     ys->strides[0] % 4 == 0 && zt.strides[0] % 4 == 0 && zt.shape[1] % 4 == 0 && aligned16(x->ptr) &&
+                     aligned16(y->ptr) && aligned16(zt.ptr) && ((uintptr_t)xs->ptr & 3) == 0 && ((uintptr_t)ys->ptr & 3) == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile: precompiled variants need K a multiple of 128, unit inner strides and aligned rows");
+  const std::string dt = zt.dtype == CUTILE_DTYPE_F32 ? "f32" : "bf16";
+  // A kernel tile that is a whole multiple of the partition tile computes the
+  // same output when the launch covers the whole tensor.
+  std::vector<const KernelEntry*> fit;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, "linear_tile") == 0 && dt == e.dtype &&
+        ((e.tile[0] == bm && e.tile[1] == bn) || (full_cover && e.tile[0] % bm == 0 && e.tile[1] % bn == 0)))
+      fit.push_back(&e);
+  std::stable_sort(fit.begin(), fit.end(), [&](const KernelEntry* a, const KernelEntry* b) {
+    bool ea = a->tile[0] == bm && a->tile[1] == bn, eb = b->tile[0] == bm && b->tile[1] == bn;
+    if (ea != eb) return ea;
+    return a->tile[0] * a->tile[1] < b->tile[0] * b->tile[1];
+  });
+  std::vector<std::string> acceptable;
+  for (auto* e : fit) acceptable.push_back(e->variant);
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of linear_tile<%d, %d, %d, %d> -> %s; available: %s", bm, bn, bk_user,
+                 bk_user / 32, dt.c_str(), list_variants("linear_tile").c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("linear_tile", opts, acceptable[0], acceptable, &res)) return s;
+  uint32_t kg[3] = {tg[0], tg[1], 1};
+  if (res.entry->tile[0] != bm || res.entry->tile[1] != bn) {
+    kg[0] = div_up(M, res.entry->tile[0]);
+    kg[1] = div_up(N, res.entry->tile[1]);
+  }
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_tensor(*x);
+  args.push_tensor(*y);
+  args.push_tensor(*xs);
+  args.push_tensor(*ys);
+  args.push_val<float>(alpha);
+  args.push_tile_grid(kg);
+  uint32_t grid[3] = {kg[0] * kg[1], 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+}  // extern "C"

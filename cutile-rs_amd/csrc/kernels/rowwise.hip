@@ -1,0 +1,338 @@
+// Row-wise bandwidth kernels for gfx950: RMSNorm (f16 IO, f32 math) and softmax
+// over tile rows (f16 or f32 IO, f32 statistics).
+//
+// Bodies follow the reference's tile programs:
+//   rms_norm_f16   cutile-kernels/src/norms.rs:16-60
+//                  ss = sum x^2 (f32); inv = rsqrt(ss/N + eps); out = f16(x * inv * w)
+//   softmax        cutile-examples/examples/softmax.rs:11-24,
+//                  cutile-benchmarks/benches/softmax.rs:19-35
+//                  per tile row: e = exp(x - max); y = e / sum(e)
+//
+// The reference reads each RMSNorm row twice (two loops over BLOCK_SIZE chunks).
+// Here a row is read from HBM exactly once: it is held in registers as 16-byte
+// vectors (one wavefront, or WPR wavefronts, per row; lane-strided so that every
+// access of a wavefront is one contiguous 1 KiB burst), reduced with cross-lane
+// shuffles (plus one LDS exchange when several wavefronts share a row), scaled
+// and written back with 16-byte stores.  Algorithmic traffic is therefore
+// x + out (+ w once per row from L2).
+//
+// A "segment" is one tile row: for RMSNorm a whole tensor row (tile [1, N]); for
+// softmax the BN columns of one row that fall in one [BM, BN] tile (row softmax
+// iff BN == N).  Padding rule for a ragged last tile: lanes beyond the tensor's
+// extent read 0 and take part in max/sum (padding::Zero on load), and are not
+// stored.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include "kernel_args.h"
+
+using namespace cutile;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+template <typename T>
+union Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  u32x4 raw;
+  T v[N];
+  __device__ Vec16() : raw{} {}
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Reduction across the WPR wavefronts that share a segment.  `slot` is the
+// segment's index inside the workgroup, `sub` the wavefront's index inside the
+// segment.  Two buffers alternate so back-to-back reductions need one barrier each.
+template <int WPR, bool IS_MAX>
+__device__ __forceinline__ float group_reduce(float v, float* lds, int slot, int sub) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if constexpr (WPR == 1) {
+    return v;
+  } else {
+    if ((threadIdx.x & 63) == 0) lds[slot * WPR + sub] = v;
+    __syncthreads();
+    float r = lds[slot * WPR];
+#pragma unroll
+    for (int i = 1; i < WPR; ++i) r = IS_MAX ? fmaxf(r, lds[slot * WPR + i]) : r + lds[slot * WPR + i];
+    return r;
+  }
+}
+
+struct SegmentMap {
+  // segment -> (row, first column, valid columns)
+  int32_t n_cols;       // tensor columns
+  int32_t seg_len;      // BN (== tile width)
+  int32_t segs_per_row; // tiles along columns that the launch grid covers
+  int64_t n_segments;
+};
+
+// ---- RMSNorm -----------------------------------------------------------------------------
+template <int WPR, int VPL>
+__device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, int64_t x_row_stride,
+                                              const _Float16* __restrict__ w,
+                                              _Float16* __restrict__ out, int64_t out_row_stride,
+                                              int32_t n, int64_t rows, float eps) {
+  using V = Vec16<_Float16>;
+  constexpr int ROWS_PER_WG = kWaves / WPR;
+  __shared__ float lds[kWaves];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int slot = wave / WPR, sub = wave % WPR;
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + slot;
+  const bool live = row < rows;
+  const int32_t nvec = n >> 3;
+  const int32_t v0 = sub * 64 + lane;
+
+  V xv[VPL];
+  float ss = 0.0f;
+  if (live) {
+    const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * x_row_stride);
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      int32_t vi = v0 + i * (64 * WPR);
+      if (vi < nvec) xv[i].raw = __builtin_nontemporal_load(xr + vi);
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float f = (float)xv[i].v[e];
+        ss = __builtin_fmaf(f, f, ss);
+      }
+    }
+  }
+  ss = group_reduce<WPR, false>(ss, lds, slot, sub);
+  if (!live) return;
+  const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+  u32x4* orow = reinterpret_cast<u32x4*>(out + row * out_row_stride);
+  const u32x4* wr = reinterpret_cast<const u32x4*>(w);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
+    if (vi < nvec) {
+      V wv, ov;
+      wv.raw = wr[vi];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ov.v[e] = (_Float16)(((float)xv[i].v[e] * inv) * (float)wv.v[e]);
+      __builtin_nontemporal_store(ov.raw, orow + vi);
+    }
+  }
+}
+
+// Any N / any strides: one workgroup per row, the row is re-read for the second
+// pass (it is still in L2).
+__device__ __forceinline__ void rms_norm_row_generic(const TensorArg<2>& x, const TensorArg<1>& w,
+                                                     const PartitionArg<2>& out, float eps,
+                                                     int64_t rows) {
+  __shared__ float lds[kWaves];
+  const int wave = threadIdx.x >> 6;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const _Float16* xr = (const _Float16*)x.ptr + row * x.strides[0];
+    const int32_t n = x.shape[1];
+    float ss = 0.0f;
+    for (int32_t j = threadIdx.x; j < n; j += kThreads) {
+      float f = (float)xr[(int64_t)j * x.strides[1]];
+      ss = __builtin_fmaf(f, f, ss);
+    }
+    ss = group_reduce<kWaves, false>(ss, lds, 0, wave);
+    const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+    _Float16* orow = (_Float16*)out.ptr + row * out.strides[0];
+    const int32_t n_out = out.shape[1] < n ? out.shape[1] : n;
+    for (int32_t j = threadIdx.x; j < n_out; j += kThreads) {
+      float f = (float)xr[(int64_t)j * x.strides[1]];
+      float wv = j < w.shape[0] ? (float)((const _Float16*)w.ptr)[(int64_t)j * w.strides[0]] : 0.0f;
+      orow[(int64_t)j * out.strides[1]] = (_Float16)((f * inv) * wv);
+    }
+    __syncthreads();  // lds is reused by the next row
+  }
+}
+
+// ---- softmax -----------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float to_f32(T v) {
+  return (float)v;
+}
+
+template <typename T, int WPR, int VPL>
+__device__ __forceinline__ void softmax_segments(const T* __restrict__ x, int64_t x_row_stride,
+                                                 T* __restrict__ y, int64_t y_row_stride,
+                                                 int32_t x_cols, int32_t y_cols, int32_t seg_len,
+                                                 int32_t segs_per_row, int64_t n_segments) {
+  using V = Vec16<T>;
+  constexpr int E = V::N;
+  constexpr int SEGS_PER_WG = kWaves / WPR;
+  __shared__ float lds[2][kWaves];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int slot = wave / WPR, sub = wave % WPR;
+  const int64_t seg = (int64_t)blockIdx.x * SEGS_PER_WG + slot;
+  const bool live = seg < n_segments;
+  const int64_t row = live ? seg / segs_per_row : 0;
+  const int32_t col0 = live ? (int32_t)(seg % segs_per_row) * seg_len : 0;
+  const int32_t seg_vec = seg_len / E;                 // vectors in a full segment
+  const int32_t x_valid = live ? max(0, min(seg_len, x_cols - col0)) / E : 0;  // readable vectors
+  const int32_t y_valid = live ? max(0, min(seg_len, y_cols - col0)) / E : 0;  // storable vectors
+  const int32_t v0 = sub * 64 + lane;
+
+  V xv[VPL];
+  float m = -INFINITY;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * x_row_stride + col0);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
+    if (vi < x_valid) xv[i].raw = __builtin_nontemporal_load(xr + vi);  // else stays 0 (padding)
+    if (live && vi < seg_vec) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) m = fmaxf(m, to_f32(xv[i].v[e]));
+    }
+  }
+  m = group_reduce<WPR, true>(m, lds[0], slot, sub);
+  const float mb = m * kLog2e;
+  float ev[VPL][E];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
+    if (live && vi < seg_vec) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        ev[i][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(to_f32(xv[i].v[e]), kLog2e, -mb));
+        s += ev[i][e];
+      }
+    }
+  }
+  s = group_reduce<WPR, false>(s, lds[1], slot, sub);
+  if (!live) return;
+  const float inv = 1.0f / s;
+  u32x4* yr = reinterpret_cast<u32x4*>(y + row * y_row_stride + col0);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
+    if (vi < y_valid) {
+      V ov;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if constexpr (sizeof(T) == 4)
+          ov.v[e] = (T)(ev[i][e] / s);
+        else
+          ov.v[e] = (T)(ev[i][e] * inv);
+      }
+      __builtin_nontemporal_store(ov.raw, yr + vi);
+    }
+  }
+}
+
+// Any tile width / any strides: one workgroup per segment, three passes (the
+// segment stays in L2 between them).
+template <typename T>
+__device__ __forceinline__ void softmax_segment_generic(const TensorArg<2>& x,
+                                                        const PartitionArg<2>& y,
+                                                        int32_t segs_per_row, int64_t n_segments) {
+  __shared__ float lds[2][kWaves];
+  const int wave = threadIdx.x >> 6;
+  const int32_t bn = y.pshape[1];
+  for (int64_t seg = blockIdx.x; seg < n_segments; seg += gridDim.x) {
+    const int64_t row = seg / segs_per_row;
+    const int32_t col0 = (int32_t)(seg % segs_per_row) * bn;
+    const bool row_ok = row < x.shape[0];
+    const T* xr = (const T*)x.ptr + row * x.strides[0];
+    auto ld = [&](int32_t j) -> float {
+      int32_t c = col0 + j;
+      return (row_ok && c < x.shape[1]) ? to_f32(xr[(int64_t)c * x.strides[1]]) : 0.0f;
+    };
+    float m = -INFINITY;
+    for (int32_t j = threadIdx.x; j < bn; j += kThreads) m = fmaxf(m, ld(j));
+    m = group_reduce<kWaves, true>(m, lds[0], 0, wave);
+    const float mb = m * kLog2e;
+    float s = 0.0f;
+    for (int32_t j = threadIdx.x; j < bn; j += kThreads)
+      s += __builtin_amdgcn_exp2f(__builtin_fmaf(ld(j), kLog2e, -mb));
+    s = group_reduce<kWaves, false>(s, lds[1], 0, wave);
+    if (row < y.shape[0]) {
+      T* yr = (T*)y.ptr + row * y.strides[0];
+      for (int32_t j = threadIdx.x; j < bn; j += kThreads) {
+        int32_t c = col0 + j;
+        if (c < y.shape[1])
+          yr[(int64_t)c * y.strides[1]] =
+              (T)(__builtin_amdgcn_exp2f(__builtin_fmaf(ld(j), kLog2e, -mb)) / s);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+// rms_norm_f16(x, w, out: [1, N] tiles, eps).  g.x = number of rows the launch covers.
+#define RMS_NORM_KERNEL(WPR, VPL)                                                                   \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      rms_norm_f16_entry__w##WPR##v##VPL(TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out,       \
+                                         float eps, TileGrid g) {                                   \
+    int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);                                       \
+    rms_norm_rows<WPR, VPL>((const _Float16*)x.ptr, x.strides[0], (const _Float16*)w.ptr,          \
+                            (_Float16*)out.ptr, out.strides[0], x.shape[1], rows, eps);            \
+  }
+
+RMS_NORM_KERNEL(1, 1)
+RMS_NORM_KERNEL(1, 2)
+RMS_NORM_KERNEL(1, 4)
+RMS_NORM_KERNEL(1, 8)
+RMS_NORM_KERNEL(1, 16)
+RMS_NORM_KERNEL(2, 8)
+RMS_NORM_KERNEL(4, 4)
+RMS_NORM_KERNEL(4, 8)
+RMS_NORM_KERNEL(4, 16)
+
+extern "C" __global__ void __launch_bounds__(kThreads)
+    rms_norm_f16_entry__generic(TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out, float eps,
+                                TileGrid g) {
+  int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);
+  rms_norm_row_generic(x, w, out, eps, rows);
+}
+
+// softmax(x, y: [BM, BN] tiles).  g.x / g.y = tiles covered along rows / columns.
+#define SOFTMAX_KERNEL(T, NAME, WPR, VPL)                                                           \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      softmax_entry__##NAME##_w##WPR##v##VPL(TensorArg<2> x, PartitionArg<2> y, TileGrid g) {       \
+    int64_t rows = min((int64_t)g.x * y.pshape[0], (int64_t)y.shape[0]);                           \
+    softmax_segments<T, WPR, VPL>((const T*)x.ptr, x.strides[0], (T*)y.ptr, y.strides[0],          \
+                                  x.shape[1], y.shape[1], y.pshape[1], (int32_t)g.y,               \
+                                  rows * (int64_t)g.y);                                            \
+  }
+
+#define SOFTMAX_VARIANTS(T, NAME) \
+  SOFTMAX_KERNEL(T, NAME, 1, 1)   \
+  SOFTMAX_KERNEL(T, NAME, 1, 2)   \
+  SOFTMAX_KERNEL(T, NAME, 1, 4)   \
+  SOFTMAX_KERNEL(T, NAME, 1, 8)   \
+  SOFTMAX_KERNEL(T, NAME, 1, 16)  \
+  SOFTMAX_KERNEL(T, NAME, 2, 8)   \
+  SOFTMAX_KERNEL(T, NAME, 4, 4)   \
+  SOFTMAX_KERNEL(T, NAME, 4, 8)   \
+  SOFTMAX_KERNEL(T, NAME, 4, 16)
+
+SOFTMAX_VARIANTS(_Float16, f16)
+SOFTMAX_VARIANTS(float, f32)
+
+#define SOFTMAX_GENERIC(T, NAME)                                                                    \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      softmax_entry__##NAME##_generic(TensorArg<2> x, PartitionArg<2> y, TileGrid g) {              \
+    int64_t rows = min((int64_t)g.x * y.pshape[0], (int64_t)y.shape[0]);                           \
+    softmax_segment_generic<T>(x, y, (int32_t)g.y, rows * (int64_t)g.y);                           \
+  }
+SOFTMAX_GENERIC(_Float16, f16)
+SOFTMAX_GENERIC(float, f32)

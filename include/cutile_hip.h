@@ -1,0 +1,353 @@
+/*
+ * cutile_hip.h — C ABI of the MI355X (gfx950) tile-kernel path.
+ *
+ * This is the drop-in boundary: the entry points a Rust FFI crate binds in place
+ * of the reference's cuda-bindings / cuda-core / cuda-async crates and of its
+ * Tile-IR JIT.  Plain pointers, integers and POD records only.
+ *
+ *   Part A  driver layer      replaces cuda-bindings + cuda-core
+ *   Part B  kernel table      replaces the JIT: (module, function, generics) ->
+ *                             precompiled gfx950 code object + launch metadata
+ *   Part C  launch builder    replaces cuda-async AsyncKernelLaunch
+ *   Part D  entry launchers   one per #[cutile::entry] kernel on the path; they
+ *                             do what the macro-generated launcher's execute()
+ *                             does: infer generics, validate, infer the grid,
+ *                             pick the kernel, push arguments, launch
+ *   Part E  async runtime     replaces cuda-async: stream pools, completion
+ *                             reactor, graph capture / replay
+ *
+ * Conventions.  Every function returns cutile_status_t: 0 = success, > 0 = the
+ * hipError_t the HIP runtime returned (the reference's DriverError(code),
+ * cuda-core/src/error.rs:17,61-93), < 0 = an error raised by this library before
+ * any GPU work (the reference's Launch / KernelLaunch / Tensor errors,
+ * cutile/src/error.rs:43-56).  cutile_last_error_message() returns the calling
+ * thread's message for the most recent non-zero status; the wording of
+ * validation errors follows the reference where its tests assert on it.
+ * Handles are opaque pointers owned by the library unless stated otherwise.
+ * Nothing here falls back to a CPU implementation: without a HIP runtime and a
+ * gfx950 device every compute entry point fails with CUTILE_ERR_LIBRARY_INIT or
+ * the driver's error.
+ */
+#ifndef CUTILE_HIP_H
+#define CUTILE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t cutile_status_t;
+
+enum {
+  CUTILE_SUCCESS = 0,
+  /* libamdhip64 could not be loaded or a symbol is missing — the reference's
+   * "shared object init failed" (cuda-bindings/src/dyn_load.rs:19-51). */
+  CUTILE_ERR_LIBRARY_INIT = -1,
+  CUTILE_ERR_INVALID_ARGUMENT = -2,
+  /* no precompiled variant for the requested (function, generics) key */
+  CUTILE_ERR_KERNEL_NOT_FOUND = -3,
+  /* launch validation failed (shape / partition / grid / precondition) */
+  CUTILE_ERR_KERNEL_LAUNCH = -4,
+  /* tensor / partition construction error */
+  CUTILE_ERR_TENSOR = -5,
+  /* nested execution, capture misuse and other runtime-state errors */
+  CUTILE_ERR_STATE = -6,
+  CUTILE_ERR_OUT_OF_SLOTS = -7
+};
+
+const char* cutile_last_error_message(void);
+const char* cutile_status_name(cutile_status_t status);
+const char* cutile_version(void);
+
+/* ======================================================================== */
+/* Part A — driver layer                                                     */
+/* ======================================================================== */
+typedef struct cutile_device* cutile_device_t;   /* cuda-core/src/runtime.rs:82-88 Device */
+typedef void* cutile_stream_t;                    /* a hipStream_t; runtime.rs:489-494 Stream */
+typedef void* cutile_event_t;                     /* a hipEvent_t; runtime.rs:534-537 Event */
+typedef struct cutile_module* cutile_module_t;    /* runtime.rs:782-786 Module */
+typedef void* cutile_function_t;                  /* a hipFunction_t; runtime.rs:839-843 Function */
+typedef void* cutile_mempool_t;                   /* a hipMemPool_t; runtime.rs:374-465 MemPool */
+typedef void* cutile_graph_t;                     /* hipGraph_t */
+typedef void* cutile_graph_exec_t;                /* hipGraphExec_t */
+
+/* Loads libamdhip64 (reusing a copy already mapped into the process) and calls
+ * hipInit.  Idempotent; every other entry point calls it lazily.
+ * cuda-bindings/src/dyn_load.rs:121-143. */
+cutile_status_t cutile_init(void);
+/* Device::device_count — runtime.rs:196 */
+cutile_status_t cutile_device_count(int32_t* count);
+/* Device::new(ordinal): process-global handle per ordinal — runtime.rs:126-139 */
+cutile_status_t cutile_device_get(int32_t ordinal, cutile_device_t* device);
+/* Device::name — runtime.rs:214 */
+cutile_status_t cutile_device_name(cutile_device_t device, char* buf, size_t buf_len);
+/* gcnArchName of the device, e.g. "gfx950:sramecc+:xnack-" */
+cutile_status_t cutile_device_arch(cutile_device_t device, char* buf, size_t buf_len);
+/* Device::bind_to_thread — runtime.rs:229 */
+cutile_status_t cutile_device_bind_to_thread(cutile_device_t device);
+/* Device::synchronize — runtime.rs:244 */
+cutile_status_t cutile_device_synchronize(cutile_device_t device);
+/* Device::l2_cache_size_bytes — runtime.rs:597 */
+cutile_status_t cutile_device_l2_cache_size(cutile_device_t device, size_t* bytes);
+typedef struct {
+  int32_t compute_units;
+  int32_t clock_khz;
+  int32_t memory_clock_khz;
+  int32_t memory_bus_bits;
+  int32_t l2_bytes;
+  int32_t lds_bytes_per_block;
+  int32_t wavefront_size;
+  int32_t reserved;
+  uint64_t total_memory_bytes;
+} cutile_device_props_t;
+cutile_status_t cutile_device_props(cutile_device_t device, cutile_device_props_t* props);
+
+/* Device::new_stream: non-blocking stream, taken from a per-device pool and
+ * never destroyed (runtime.rs:249-266,504-509,613-631).  cutile_stream_release
+ * returns it to the pool. */
+cutile_status_t cutile_stream_create(cutile_device_t device, cutile_stream_t* stream);
+cutile_status_t cutile_stream_release(cutile_device_t device, cutile_stream_t stream);
+/* Stream::synchronize / query — runtime.rs:696,706.  *done = 1 when idle. */
+cutile_status_t cutile_stream_synchronize(cutile_stream_t stream);
+cutile_status_t cutile_stream_query(cutile_stream_t stream, int32_t* done);
+/* Stream::launch_host_function — runtime.rs:715-758 */
+typedef void (*cutile_host_fn_t)(void* user);
+cutile_status_t cutile_stream_launch_host_func(cutile_stream_t stream, cutile_host_fn_t fn, void* user);
+/* Stream::begin_capture (relaxed mode) / end_capture — runtime.rs:760-780 */
+cutile_status_t cutile_stream_begin_capture(cutile_stream_t stream);
+cutile_status_t cutile_stream_end_capture(cutile_stream_t stream, cutile_graph_t* graph);
+/* reactor flag write: cuStreamWriteValue32 — cuda-async/src/reactor.rs:154-179 */
+cutile_status_t cutile_stream_write_value32(cutile_stream_t stream, void* device_ptr, uint32_t value);
+
+/* Event — runtime.rs:534-594 */
+cutile_status_t cutile_event_create(cutile_event_t* event);
+cutile_status_t cutile_event_record(cutile_event_t event, cutile_stream_t stream);
+cutile_status_t cutile_event_synchronize(cutile_event_t event);
+cutile_status_t cutile_event_elapsed_ms(cutile_event_t start, cutile_event_t end, float* ms);
+cutile_status_t cutile_event_destroy(cutile_event_t event);
+
+/* Device::load_module_from_bytes: checks the ELF magic first — runtime.rs:309-328 */
+cutile_status_t cutile_module_load_data(cutile_device_t device, const void* image, size_t size,
+                                        cutile_module_t* module);
+cutile_status_t cutile_module_unload(cutile_module_t module);
+/* Module::load_function — runtime.rs:828-835 */
+cutile_status_t cutile_module_get_function(cutile_module_t module, const char* name,
+                                           cutile_function_t* function);
+/* launch_kernel: cuLaunchKernel with a void** parameter array — cuda-core/src/api.rs:48-70 */
+cutile_status_t cutile_launch_kernel(cutile_function_t function, const uint32_t grid[3],
+                                     const uint32_t block[3], uint32_t shared_mem_bytes,
+                                     cutile_stream_t stream, void** kernel_params);
+
+/* malloc_async / malloc_from_pool_async / free_async — cuda-core/src/api.rs:76-119 */
+cutile_status_t cutile_malloc_async(size_t bytes, cutile_stream_t stream, void** device_ptr);
+cutile_status_t cutile_malloc_from_pool_async(size_t bytes, cutile_mempool_t pool,
+                                              cutile_stream_t stream, void** device_ptr);
+cutile_status_t cutile_free_async(void* device_ptr, cutile_stream_t stream);
+/* memset_d8_async / memcpy_{htod,dtoh,dtod}_async — cuda-core/src/api.rs:102-166 */
+cutile_status_t cutile_memset_d8_async(void* device_ptr, uint8_t value, size_t bytes, cutile_stream_t stream);
+cutile_status_t cutile_memcpy_htod_async(void* dst, const void* src, size_t bytes, cutile_stream_t stream);
+cutile_status_t cutile_memcpy_dtoh_async(void* dst, const void* src, size_t bytes, cutile_stream_t stream);
+cutile_status_t cutile_memcpy_dtod_async(void* dst, const void* src, size_t bytes, cutile_stream_t stream);
+/* pinned, mapped host memory for the reactor's completion flags —
+ * cuda-async/src/slot_table.rs (cuMemHostAlloc portable|devicemap) */
+cutile_status_t cutile_host_alloc_mapped(size_t bytes, void** host_ptr, void** device_ptr);
+cutile_status_t cutile_host_free(void* host_ptr);
+
+/* MemPool — runtime.rs:335-465 */
+cutile_status_t cutile_mempool_create(cutile_device_t device, cutile_mempool_t* pool);
+cutile_status_t cutile_mempool_default(cutile_device_t device, cutile_mempool_t* pool);
+cutile_status_t cutile_mempool_destroy(cutile_mempool_t pool);
+cutile_status_t cutile_mempool_set_release_threshold(cutile_mempool_t pool, uint64_t bytes);
+typedef struct {
+  uint64_t reserved_current, reserved_high, used_current, used_high;
+} cutile_pool_mem_stats_t;
+cutile_status_t cutile_mempool_stats(cutile_mempool_t pool, cutile_pool_mem_stats_t* stats);
+cutile_status_t cutile_mempool_reset_used_high(cutile_mempool_t pool);
+cutile_status_t cutile_mempool_reset_reserved_high(cutile_mempool_t pool);
+
+/* graph instantiate / upload / launch / destroy — cuda-async/src/cuda_graph.rs:61-137,179-244 */
+cutile_status_t cutile_graph_instantiate(cutile_graph_t graph, cutile_graph_exec_t* exec);
+cutile_status_t cutile_graph_upload(cutile_graph_exec_t exec, cutile_stream_t stream);
+cutile_status_t cutile_graph_launch(cutile_graph_exec_t exec, cutile_stream_t stream);
+cutile_status_t cutile_graph_exec_destroy(cutile_graph_exec_t exec);
+cutile_status_t cutile_graph_destroy(cutile_graph_t graph);
+
+/* ======================================================================== */
+/* Part B — kernel table                                                     */
+/* ======================================================================== */
+/* What the reference obtains from compile_from_context (cutile/src/tile_kernel.rs:675-756):
+ * a loaded function plus what is needed to launch and validate it.  Here the
+ * function comes from a precompiled gfx950 code object embedded in this library. */
+typedef struct {
+  cutile_function_t function;   /* loaded on the device passed to the lookup */
+  const char* symbol;           /* "<fn>_entry__<variant>" */
+  const char* variant;          /* variant name inside the function family */
+  uint32_t block[3];            /* workgroup shape the kernel was written for */
+  uint32_t lds_bytes;           /* dynamic LDS bytes to pass at launch */
+  int32_t tile[4];              /* tile shape (BM, BN, BK, -) the variant implements; 0 = any */
+} cutile_kernel_info_t;
+
+/* Looks up `function` (e.g. "gemm") with reference-style generics strings
+ * (e.g. {"bf16","256","256","64"}) and a variant hint (NULL = the library's
+ * choice for this key).  Unknown keys fail with CUTILE_ERR_KERNEL_NOT_FOUND and a
+ * message listing the variants that exist.  Loads the code object on first use
+ * (single-flight per device), like the reference's kernel cache
+ * (tile_kernel.rs:371-399,705-733). */
+cutile_status_t cutile_kernel_lookup(cutile_device_t device, const char* function,
+                                     const char* const* generics, int32_t n_generics,
+                                     const char* variant, cutile_kernel_info_t* info);
+/* Number of code-object loads performed so far (the analogue of
+ * jit_compile_count, tile_kernel.rs:45-62). */
+uint64_t cutile_module_load_count(void);
+/* Enumerates the table: returns the number of entries; writes up to `cap`
+ * "function<generics>:variant" C strings (owned by the library). */
+int32_t cutile_kernel_list(const char** names, int32_t cap);
+/* Pins the variant that cutile_launch_* entry points use for `function` when
+ * several fit (the autotuner's output).  variant == NULL restores the default. */
+cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const char* variant);
+
+/* ======================================================================== */
+/* Part C — launch builder                                                   */
+/* ======================================================================== */
+/* AsyncKernelLaunch — cuda-async/src/launch.rs:23-146.  Arguments are pushed in
+ * kernel-signature order; the builder owns copies of the values. */
+typedef struct cutile_launch* cutile_launch_t;
+cutile_status_t cutile_launch_create(cutile_function_t function, cutile_launch_t* launch);
+cutile_status_t cutile_launch_destroy(cutile_launch_t launch);
+/* launch.rs:131-138 push_arg: any POD scalar, by value */
+cutile_status_t cutile_launch_push_arg(cutile_launch_t launch, const void* value, size_t size, size_t align);
+/* launch.rs:117-124 push_device_ptr */
+cutile_status_t cutile_launch_push_device_ptr(cutile_launch_t launch, void* device_ptr);
+/* launch.rs:63-74 LaunchConfig */
+cutile_status_t cutile_launch_set_config(cutile_launch_t launch, const uint32_t grid[3],
+                                         const uint32_t block[3], uint32_t shared_mem_bytes);
+/* launch.rs:95-113 launch on a stream; may be called repeatedly */
+cutile_status_t cutile_launch_execute(cutile_launch_t launch, cutile_stream_t stream);
+
+/* ======================================================================== */
+/* Part D — entry launchers                                                  */
+/* ======================================================================== */
+#define CUTILE_MAX_RANK 4
+
+/* dtype names are the strings the reference passes in .generics
+ * (cuda-core/src/dtype.rs:189-229). */
+typedef enum {
+  CUTILE_DTYPE_F32 = 0, CUTILE_DTYPE_F64, CUTILE_DTYPE_F16, CUTILE_DTYPE_BF16,
+  CUTILE_DTYPE_I8, CUTILE_DTYPE_I16, CUTILE_DTYPE_I32, CUTILE_DTYPE_I64,
+  CUTILE_DTYPE_U8, CUTILE_DTYPE_U16, CUTILE_DTYPE_U32, CUTILE_DTYPE_U64,
+  CUTILE_DTYPE_BOOL, CUTILE_DTYPE_F8E4M3FN, CUTILE_DTYPE_F8E5M2, CUTILE_DTYPE_F8E8M0FNU,
+  CUTILE_DTYPE_COUNT
+} cutile_dtype_t;
+const char* cutile_dtype_name(cutile_dtype_t dtype);
+size_t cutile_dtype_size(cutile_dtype_t dtype);
+/* returns CUTILE_DTYPE_COUNT for an unknown name */
+cutile_dtype_t cutile_dtype_from_name(const char* name);
+
+/* A tensor argument: what KernelInput pushes (cutile/src/tensor.rs:2005-2016). */
+typedef struct {
+  void* ptr;                        /* device pointer (already offset for views) */
+  cutile_dtype_t dtype;
+  int32_t rank;
+  int32_t shape[CUTILE_MAX_RANK];
+  int32_t strides[CUTILE_MAX_RANK]; /* in elements */
+} cutile_tensor_arg_t;
+
+/* An output partition: what KernelOutput pushes (cutile/src/tensor.rs:1723-1739),
+ * plus its coverage mode (GridBound::Exact / AtMost, tensor.rs:1677-1685). */
+typedef struct {
+  cutile_tensor_arg_t tensor;
+  int32_t partition_shape[CUTILE_MAX_RANK];
+  int32_t partition_strides[CUTILE_MAX_RANK];
+  int32_t prefix_coverage;          /* 0 = exact cover, 1 = partition_prefix (at most) */
+} cutile_partition_arg_t;
+
+/* Builder options of the generated launcher (cutile-macro/src/_module.rs:901-923):
+ * .grid(), .generics(), plus the variant hint this build adds. */
+typedef struct {
+  uint32_t grid[3];                 /* (0,0,0) = infer from the partition */
+  const char* const* generics;      /* NULL = infer from argument dtypes / partition shapes */
+  int32_t n_generics;
+  const char* variant;              /* NULL = library's choice */
+} cutile_launch_opts_t;
+
+/* Partition::grid — cutile/src/tensor.rs:447-468 */
+cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t grid[3]);
+/* infer_launch_grid over the bounds of all partition arguments —
+ * cutile/src/tile_kernel.rs:934-967.  `explicit_grid` (0,0,0) = infer. */
+cutile_status_t cutile_infer_launch_grid(const uint32_t explicit_grid[3],
+                                         const cutile_partition_arg_t* const* partitions,
+                                         int32_t n_partitions, uint32_t grid[3]);
+/* SpecializationBits — cutile-compiler/src/specialization.rs:21-174 */
+typedef struct {
+  int32_t shape_div[CUTILE_MAX_RANK];   /* largest power of two <= 16 dividing shape[i] */
+  int32_t stride_div[CUTILE_MAX_RANK];  /* same for strides (elements) */
+  int32_t stride_one[CUTILE_MAX_RANK];  /* stride[i] == 1 */
+  int32_t base_ptr_div;                 /* same for the base pointer (bytes) */
+  int32_t elements_disjoint;
+} cutile_spec_bits_t;
+cutile_status_t cutile_compute_spec(const cutile_tensor_arg_t* t, cutile_spec_bits_t* spec);
+
+/* saxpy<S, T>(y: &mut Tensor<T,S>, a: T, x: &Tensor<T,[-1,-1]>): y <- a*x + y with
+ * one fused multiply-add per element.  Rank 1 or 2.  `a` is passed as f64 and
+ * narrowed to T.  cutile-examples/examples/saxpy.rs:12-17, async_saxpy.rs:21-30. */
+cutile_status_t cutile_launch_saxpy(cutile_stream_t stream, const cutile_partition_arg_t* y,
+                                    double a, const cutile_tensor_arg_t* x,
+                                    const cutile_launch_opts_t* opts);
+/* axpy<B, T>(z: &mut Tensor<T,[B]>, a: T, x, y): z <- a*x + y, rank 1 (the
+ * three-operand form of the same arithmetic; sibling of `add`, README.md:29-38). */
+cutile_status_t cutile_launch_axpy(cutile_stream_t stream, const cutile_partition_arg_t* z, double a,
+                                   const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                   const cutile_launch_opts_t* opts);
+/* add<B>(z, x, y): z <- x + y.  README.md:29-38, cutile/tests/gpu/add_basic.rs:16-25. */
+cutile_status_t cutile_launch_add(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                  const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                  const cutile_launch_opts_t* opts);
+/* creation::full / arange / linspace — cutile/src/kernels/_creation.rs:44-47,79-87,94-108 */
+cutile_status_t cutile_launch_full(cutile_stream_t stream, double value, int64_t int_value,
+                                   const cutile_partition_arg_t* t, const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_arange(cutile_stream_t stream, const cutile_partition_arg_t* t,
+                                     const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_partition_arg_t* t,
+                                       float start, float step, const cutile_launch_opts_t* opts);
+/* conversion::convert — cutile/src/kernels/_conversion.rs:78-85 */
+cutile_status_t cutile_launch_convert(cutile_stream_t stream, const cutile_tensor_arg_t* src,
+                                      const cutile_partition_arg_t* dst, const cutile_launch_opts_t* opts);
+/* rms_norm_f16<N, BLOCK_SIZE>(x, w, out: [1,N] tiles, eps) — cutile-kernels/src/norms.rs:16-60 */
+cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                           const cutile_tensor_arg_t* w,
+                                           const cutile_partition_arg_t* out, float eps,
+                                           const cutile_launch_opts_t* opts);
+/* softmax<BM, BN>(x, y: [BM,BN] tiles), f16 or f32 — cutile-benchmarks/benches/softmax.rs:19-35,
+ * cutile-examples/examples/softmax.rs:11-24 */
+cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                      const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts);
+/* gemm<T, BM, BN, BK>(z: [BM,BN] tiles, x, y, k): z <- z + x·y with f32
+ * accumulation (z is read as the initial accumulator, like the reference bench;
+ * `accumulate` = 0 starts from zero like the example) —
+ * cutile-benchmarks/benches/gemm.rs:20-41, cutile-examples/examples/gemm.rs:20-36 */
+cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                   const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                   int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* fmha<BM, BN, D, H, CAUSAL, EVEN_K>(out: [1,BM,D] tiles, q, k, v, qk_scale,
+ * input_pos, query_group_size) — cutile-examples/examples/flash_attention_causal.rs:19-134,
+ * cutile-benchmarks/benches/fmha.rs:20-145 (non-causal: causal = 0, input_pos = 0) */
+cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partition_arg_t* out,
+                                   const cutile_tensor_arg_t* q, const cutile_tensor_arg_t* k,
+                                   const cutile_tensor_arg_t* v, float qk_scale, int32_t input_pos,
+                                   int32_t query_group_size, int32_t causal,
+                                   const cutile_launch_opts_t* opts);
+/* linear_tile<BM, BN, BK, BK/32>(z: [BM,BN] tiles, x[M,K], y[N,K], x_scales[M,K/32],
+ * y_scales[N,K/32], alpha): z <- alpha * (x·sx) @ (y·sy)^T, e4m3 data, e8m0
+ * scales, f32 accumulation; z is f32 or bf16 — cutile-examples/examples/mxfp8.rs:34-64 */
+cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                                const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                                const cutile_tensor_arg_t* x_scales,
+                                                const cutile_tensor_arg_t* y_scales, float alpha,
+                                                const cutile_launch_opts_t* opts);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUTILE_HIP_H */

@@ -1,0 +1,268 @@
+"""numpy-facing wrapper of the CPU oracle (``liboracle.so``, built by the Makefile here).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``; the shipped library never touches it.
+
+Every function follows the C declaration of the same name in ``oracle.h``, which cites
+the reference file:line it restates.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile liboracle.so with gcc (seconds)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        vp, i64, f32, f64, u64, sz = C.c_void_p, C.c_int64, C.c_float, C.c_double, C.c_uint64, C.c_size_t
+        sigs = {
+            "orc_num_threads": (C.c_int, []),
+            "orc_set_num_threads": (None, [C.c_int]),
+            "orc_f32_to_f16": (C.c_uint16, [f32]),
+            "orc_f16_to_f32": (f32, [C.c_uint16]),
+            "orc_f32_to_bf16": (C.c_uint16, [f32]),
+            "orc_bf16_to_f32": (f32, [C.c_uint16]),
+            "orc_e4m3fn_to_f32": (f32, [C.c_uint8]),
+            "orc_f32_to_e4m3fn": (C.c_uint8, [f32]),
+            "orc_e8m0_to_f32": (f32, [C.c_uint8]),
+            "orc_f32_to_f16_n": (None, [vp, vp, sz]),
+            "orc_f16_to_f32_n": (None, [vp, vp, sz]),
+            "orc_f32_to_bf16_n": (None, [vp, vp, sz]),
+            "orc_bf16_to_f32_n": (None, [vp, vp, sz]),
+            "orc_fill_uniform_f32": (None, [vp, sz, u64, f32, f32]),
+            "orc_fill_normal_f32": (None, [vp, sz, u64, f32, f32]),
+            "orc_saxpy_f32": (None, [sz, f32, vp, vp, vp]),
+            "orc_add_f32": (None, [sz, vp, vp, vp]),
+            "orc_rms_norm_f16": (None, [vp, vp, vp, i64, i64, f32, i64]),
+            "orc_rms_norm_f16_f64": (None, [vp, vp, vp, i64, i64, f64]),
+            "orc_softmax_f32": (None, [vp, vp, i64, i64, i64, i64]),
+            "orc_softmax_f16": (None, [vp, vp, i64, i64, i64, i64]),
+            "orc_cpu_gemm_f32": (None, [vp, vp, vp, i64, i64, i64]),
+            "orc_gemm_bf16": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
+            "orc_gemm_bf16_f32out": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
+            "orc_fmha_ref_cpu": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp, i64]),
+            "orc_mx_quantize_e4m3": (None, [vp, vp, vp, i64, i64]),
+            "orc_mx_dequantize_e4m3": (None, [vp, vp, vp, i64, i64]),
+            "orc_mx_gemm_f32": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, vp, i64]),
+        }
+        for name, (res, args) in sigs.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def num_threads() -> int:
+    return int(lib().orc_num_threads())
+
+
+def set_num_threads(n: int) -> None:
+    lib().orc_set_num_threads(int(n))
+
+
+# ---- codecs -------------------------------------------------------------------------------
+def f32_to_f16_bits(x) -> np.ndarray:
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_f32_to_f16_n(_p(x), _p(out), x.size)
+    return out
+
+
+def f16_bits_to_f32(h) -> np.ndarray:
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().orc_f16_to_f32_n(_p(h), _p(out), h.size)
+    return out
+
+
+def f32_to_bf16_bits(x) -> np.ndarray:
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_f32_to_bf16_n(_p(x), _p(out), x.size)
+    return out
+
+
+def bf16_bits_to_f32(h) -> np.ndarray:
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().orc_bf16_to_f32_n(_p(h), _p(out), h.size)
+    return out
+
+
+def e4m3fn_to_f32(code: int) -> float:
+    return float(lib().orc_e4m3fn_to_f32(int(code)))
+
+
+def f32_to_e4m3fn(v: float) -> int:
+    return int(lib().orc_f32_to_e4m3fn(float(v)))
+
+
+def e8m0_to_f32(code: int) -> float:
+    return float(lib().orc_e8m0_to_f32(int(code)))
+
+
+# ---- seeded inputs ------------------------------------------------------------------------
+def uniform_f32(shape, seed: int, lo: float = -1.0, hi: float = 1.0) -> np.ndarray:
+    out = np.empty(shape, np.float32)
+    lib().orc_fill_uniform_f32(_p(out), out.size, seed, lo, hi)
+    return out
+
+
+def normal_f32(shape, seed: int, mean: float = 0.0, std: float = 1.0) -> np.ndarray:
+    out = np.empty(shape, np.float32)
+    lib().orc_fill_normal_f32(_p(out), out.size, seed, mean, std)
+    return out
+
+
+# ---- K1 -----------------------------------------------------------------------------------
+def saxpy_f32(a: float, x, y) -> np.ndarray:
+    x, y = _c(x, np.float32), _c(y, np.float32)
+    z = np.empty_like(x)
+    lib().orc_saxpy_f32(x.size, a, _p(x), _p(y), _p(z))
+    return z
+
+
+def add_f32(x, y) -> np.ndarray:
+    x, y = _c(x, np.float32), _c(y, np.float32)
+    z = np.empty_like(x)
+    lib().orc_add_f32(x.size, _p(x), _p(y), _p(z))
+    return z
+
+
+# ---- K2 -----------------------------------------------------------------------------------
+def rms_norm_f16(x_bits, w_bits, eps: float, block: int = 0) -> np.ndarray:
+    x, w = _c(x_bits, np.uint16), _c(w_bits, np.uint16)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    lib().orc_rms_norm_f16(_p(x), _p(w), _p(out), rows, n, eps, block or n)
+    return out
+
+
+def rms_norm_f16_f64(x_bits, w_bits, eps: float) -> np.ndarray:
+    x, w = _c(x_bits, np.uint16), _c(w_bits, np.uint16)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    lib().orc_rms_norm_f16_f64(_p(x), _p(w), _p(out), rows, n, eps)
+    return out
+
+
+# ---- K3 -----------------------------------------------------------------------------------
+def softmax_f32(x, bm: int, bn: int) -> np.ndarray:
+    x = _c(x, np.float32)
+    m, n = x.shape
+    y = np.zeros_like(x)
+    lib().orc_softmax_f32(_p(x), _p(y), m, n, bm, bn)
+    return y
+
+
+def softmax_f16(x_bits, bm: int, bn: int) -> np.ndarray:
+    x = _c(x_bits, np.uint16)
+    m, n = x.shape
+    y = np.zeros_like(x)
+    lib().orc_softmax_f16(_p(x), _p(y), m, n, bm, bn)
+    return y
+
+
+# ---- K4 -----------------------------------------------------------------------------------
+def cpu_gemm_f32(x, y) -> np.ndarray:
+    x, y = _c(x, np.float32), _c(y, np.float32)
+    m, k = x.shape
+    k2, n = y.shape
+    assert k == k2
+    z = np.empty((m, n), np.float32)
+    lib().orc_cpu_gemm_f32(_p(x), _p(y), _p(z), m, n, k)
+    return z
+
+
+def _rows_arg(rows):
+    if rows is None:
+        return None, None, 0
+    r = _c(rows, np.int64)
+    return r, _p(r), r.size
+
+
+def gemm_bf16(a_bits, b_bits, rows=None, f32out: bool = False) -> np.ndarray:
+    a, b = _c(a_bits, np.uint16), _c(b_bits, np.uint16)
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2
+    keep, rp, nr = _rows_arg(rows)
+    cnt = nr if rows is not None else m
+    if f32out:
+        c = np.empty((cnt, n), np.float32)
+        lib().orc_gemm_bf16_f32out(_p(a), _p(b), _p(c), m, n, k, rp, nr)
+    else:
+        c = np.empty((cnt, n), np.uint16)
+        lib().orc_gemm_bf16(_p(a), _p(b), _p(c), m, n, k, rp, nr)
+    return c
+
+
+# ---- K5 -----------------------------------------------------------------------------------
+def fmha_ref_cpu(q, k, v, qk_scale: float, input_pos: int = 0, query_group_size: int = 1,
+                 causal: bool = False, rows=None) -> np.ndarray:
+    q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
+    b, h, m, d = q.shape
+    hkv = k.shape[1]
+    keep, rp, nr = _rows_arg(rows)
+    out = np.empty((nr, d) if rows is not None else (b, h, m, d), np.float32)
+    lib().orc_fmha_ref_cpu(_p(q), _p(k), _p(v), _p(out), b, h, hkv, m, d, qk_scale, input_pos,
+                           query_group_size, int(causal), rp, nr)
+    return out
+
+
+# ---- K6 -----------------------------------------------------------------------------------
+def mx_quantize_e4m3(src):
+    src = _c(src, np.float32)
+    rows, k = src.shape
+    assert k % 32 == 0
+    data = np.empty((rows, k), np.uint8)
+    scales = np.empty((rows, k // 32), np.uint8)
+    lib().orc_mx_quantize_e4m3(_p(src), _p(data), _p(scales), rows, k)
+    return data, scales
+
+
+def mx_dequantize_e4m3(data, scales) -> np.ndarray:
+    data, scales = _c(data, np.uint8), _c(scales, np.uint8)
+    rows, k = data.shape
+    dst = np.empty((rows, k), np.float32)
+    lib().orc_mx_dequantize_e4m3(_p(data), _p(scales), _p(dst), rows, k)
+    return dst
+
+
+def mx_gemm_f32(x, y, xs, ys, alpha: float = 1.0, rows=None) -> np.ndarray:
+    x, y, xs, ys = _c(x, np.uint8), _c(y, np.uint8), _c(xs, np.uint8), _c(ys, np.uint8)
+    m, k = x.shape
+    n, k2 = y.shape
+    assert k == k2
+    keep, rp, nr = _rows_arg(rows)
+    z = np.empty((nr if rows is not None else m, n), np.float32)
+    lib().orc_mx_gemm_f32(_p(x), _p(y), _p(xs), _p(ys), _p(z), m, n, k, alpha, rp, nr)
+    return z

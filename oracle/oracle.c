@@ -1,0 +1,452 @@
+/*
+ * CPU oracle for the tile-kernel path.  TEST INFRASTRUCTURE ONLY (see oracle.h):
+ * the shipped library never links or calls this file.
+ *
+ * Build: gcc -O3 -ffp-contract=off -fopenmp (the Makefile beside this file).
+ * -ffp-contract=off keeps `acc += a * b` a separate multiply and add, as the
+ * reference's Rust loops are; the one fused operation is the explicit fmaf in
+ * orc_saxpy_f32.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <omp.h>
+#include <stdlib.h>
+#include <string.h>
+
+int orc_num_threads(void) { return omp_get_max_threads(); }
+void orc_set_num_threads(int n) {
+  if (n > 0) omp_set_num_threads(n);
+}
+
+/* ------------------------------------------------------------------------ */
+/* codecs                                                                    */
+/* ------------------------------------------------------------------------ */
+static inline uint32_t f32_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static inline float bits_f32(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+uint16_t orc_f32_to_f16(float f) {
+  uint32_t x = f32_bits(f);
+  uint32_t sign = (x >> 16) & 0x8000u;
+  uint32_t abs = x & 0x7fffffffu;
+  if (abs >= 0x7f800000u) { /* inf / nan */
+    return (uint16_t)(sign | 0x7c00u | (abs > 0x7f800000u ? 0x0200u | ((abs >> 13) & 0x3ffu) : 0));
+  }
+  if (abs >= 0x477ff000u) { /* rounds to >= 65520 -> inf */
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (abs < 0x38800000u) { /* below the smallest normal half 2^-14: subnormal */
+    if (abs < 0x33000000u) return (uint16_t)sign; /* < 2^-25 -> 0 (ties to even gives 0) */
+    int e = (int)(abs >> 23);                      /* biased f32 exponent */
+    uint32_t man = (abs & 0x7fffffu) | 0x800000u;  /* 24-bit significand */
+    int shift = 126 - e;                           /* bits dropped to reach 2^-24 units */
+    uint32_t q = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+  uint32_t e = (abs >> 23) - 112u; /* rebias 127 -> 15 */
+  uint32_t man = abs & 0x7fffffu;
+  uint32_t h = (e << 10) | (man >> 13);
+  uint32_t rem = man & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++; /* carry may bump the exponent */
+  return (uint16_t)(sign | h);
+}
+
+float orc_f16_to_f32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (e == 0) {
+    if (man == 0) return bits_f32(sign);
+    float v = (float)man * (1.0f / 16777216.0f); /* man * 2^-24 */
+    return sign ? -v : v;
+  }
+  if (e == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+  return bits_f32(sign | ((e + 112u) << 23) | (man << 13));
+}
+
+uint16_t orc_f32_to_bf16(float f) {
+  uint32_t x = f32_bits(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u); /* quiet nan */
+  uint32_t lsb = (x >> 16) & 1u;
+  x += 0x7fffu + lsb;
+  return (uint16_t)(x >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+float orc_e4m3fn_to_f32(uint8_t b) {
+  int sign = b >> 7;
+  int e = (b >> 3) & 0xf;
+  int man = b & 7;
+  float v;
+  if (e == 15 && man == 7) return NAN;
+  if (e == 0)
+    v = ldexpf((float)man, -9); /* man/8 * 2^-6 */
+  else
+    v = ldexpf(1.0f + (float)man / 8.0f, e - 7);
+  return sign ? -v : v;
+}
+
+uint8_t orc_f32_to_e4m3fn(float f) {
+  if (isnan(f)) return 0x7f;
+  uint8_t sign = signbit(f) ? 0x80 : 0;
+  float a = fabsf(f);
+  if (a >= 448.0f) return (uint8_t)(sign | 0x7e); /* saturate (also +-inf) */
+  if (a < 0.015625f) {                              /* < 2^-6: subnormal grid, step 2^-9 */
+    int q = (int)nearbyintf(a * 512.0f);            /* ties-to-even under the default mode */
+    return (uint8_t)(sign | q);                     /* q == 8 is exactly code 0x08 = 2^-6 */
+  }
+  int e;
+  float m = frexpf(a, &e); /* a = m * 2^e, m in [0.5, 1) */
+  m *= 2.0f;
+  e -= 1; /* m in [1, 2) */
+  int q = (int)nearbyintf((m - 1.0f) * 8.0f);
+  if (q == 8) {
+    q = 0;
+    e += 1;
+  }
+  if (e > 8 || (e == 8 && q == 7)) return (uint8_t)(sign | 0x7e);
+  return (uint8_t)(sign | ((e + 7) << 3) | q);
+}
+
+float orc_e8m0_to_f32(uint8_t b) {
+  if (b == 0xff) return NAN;
+  return ldexpf(1.0f, (int)b - 127);
+}
+
+void orc_f32_to_f16_n(const float* src, uint16_t* dst, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = orc_f32_to_f16(src[i]);
+}
+void orc_f16_to_f32_n(const uint16_t* src, float* dst, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = orc_f16_to_f32(src[i]);
+}
+void orc_f32_to_bf16_n(const float* src, uint16_t* dst, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = orc_f32_to_bf16(src[i]);
+}
+void orc_bf16_to_f32_n(const uint16_t* src, float* dst, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = orc_bf16_to_f32(src[i]);
+}
+
+/* ------------------------------------------------------------------------ */
+/* seeded inputs                                                             */
+/* ------------------------------------------------------------------------ */
+/* SplitMix64 evaluated as a counter-based generator: element i depends only on
+ * (seed, i), so fills are identical for any thread count. */
+static inline uint64_t splitmix64_at(uint64_t seed, uint64_t i) {
+  uint64_t z = seed + (i + 1) * 0x9e3779b97f4a7c15ull;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+static inline double u01(uint64_t r) { return (double)(r >> 11) * (1.0 / 9007199254740992.0); }
+
+void orc_fill_uniform_f32(float* dst, size_t n, uint64_t seed, float lo, float hi) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) {
+    double u = u01(splitmix64_at(seed, i));
+    dst[i] = (float)((double)lo + ((double)hi - (double)lo) * u);
+  }
+}
+
+void orc_fill_normal_f32(float* dst, size_t n, uint64_t seed, float mean, float std) {
+  /* Box-Muller, one pair of uniforms per output element (cos branch). */
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) {
+    double u1 = u01(splitmix64_at(seed, 2 * i));
+    double u2 = u01(splitmix64_at(seed, 2 * i + 1));
+    if (u1 < 1e-300) u1 = 1e-300;
+    double r = sqrt(-2.0 * log(u1));
+    dst[i] = (float)((double)mean + (double)std * r * cos(6.283185307179586476925 * u2));
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* K1                                                                        */
+/* ------------------------------------------------------------------------ */
+void orc_saxpy_f32(size_t n, float a, const float* x, const float* y, float* z) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) z[i] = fmaf(a, x[i], y[i]);
+}
+
+void orc_add_f32(size_t n, const float* x, const float* y, float* z) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) z[i] = x[i] + y[i];
+}
+
+/* ------------------------------------------------------------------------ */
+/* K2                                                                        */
+/* ------------------------------------------------------------------------ */
+void orc_rms_norm_f16(const uint16_t* x, const uint16_t* w, uint16_t* out, int64_t rows,
+                      int64_t n, float eps, int64_t block) {
+  if (block <= 0 || block > n) block = n;
+#pragma omp parallel
+  {
+    float* lanes = (float*)malloc(sizeof(float) * (size_t)block);
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+      const uint16_t* xr = x + r * n;
+      for (int64_t l = 0; l < block; l++) lanes[l] = 0.0f;
+      for (int64_t j = 0; j < n; j += block) { /* rms = rms + tx * tx, per lane */
+        int64_t lim = n - j < block ? n - j : block;
+        for (int64_t l = 0; l < lim; l++) {
+          float v = orc_f16_to_f32(xr[j + l]);
+          lanes[l] = lanes[l] + v * v;
+        }
+      }
+      float ss = 0.0f;
+      for (int64_t l = 0; l < block; l++) ss += lanes[l];
+      float inv = 1.0f / sqrtf(ss / (float)n + eps);
+      for (int64_t j = 0; j < n; j++) {
+        float v = orc_f16_to_f32(xr[j]);
+        float o = v * inv * orc_f16_to_f32(w[j]); /* (x * inv) * w */
+        out[r * n + j] = orc_f32_to_f16(o);
+      }
+    }
+    free(lanes);
+  }
+}
+
+void orc_rms_norm_f16_f64(const uint16_t* x, const uint16_t* w, uint16_t* out, int64_t rows,
+                          int64_t n, double eps) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; r++) {
+    const uint16_t* xr = x + r * n;
+    double ss = 0.0;
+    for (int64_t j = 0; j < n; j++) {
+      double v = (double)orc_f16_to_f32(xr[j]);
+      ss += v * v;
+    }
+    double inv = 1.0 / sqrt(ss / (double)n + eps);
+    for (int64_t j = 0; j < n; j++) {
+      double o = (double)orc_f16_to_f32(xr[j]) * inv * (double)orc_f16_to_f32(w[j]);
+      out[r * n + j] = orc_f32_to_f16((float)o);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* K3                                                                        */
+/* ------------------------------------------------------------------------ */
+static void softmax_tile_row(const float* xin, float* yout, int64_t valid, int64_t bn) {
+  /* the tile row has bn lanes; lanes >= valid were zero padded on load */
+  float mx = -INFINITY;
+  for (int64_t j = 0; j < valid; j++) mx = fmaxf(mx, xin[j]);
+  if (valid < bn) mx = fmaxf(mx, 0.0f);
+  float den = 0.0f;
+  for (int64_t j = 0; j < valid; j++) {
+    yout[j] = expf(xin[j] - mx);
+    den += yout[j];
+  }
+  if (valid < bn) den += (float)(bn - valid) * expf(0.0f - mx);
+  for (int64_t j = 0; j < valid; j++) yout[j] = yout[j] / den;
+}
+
+void orc_softmax_f32(const float* x, float* y, int64_t m, int64_t n, int64_t bm, int64_t bn) {
+  (void)bm; /* rows are independent; bm only shapes the launch grid */
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < m; r++) {
+    for (int64_t c0 = 0; c0 < n; c0 += bn) {
+      int64_t valid = n - c0 < bn ? n - c0 : bn;
+      softmax_tile_row(x + r * n + c0, y + r * n + c0, valid, bn);
+    }
+  }
+}
+
+void orc_softmax_f16(const uint16_t* x, uint16_t* y, int64_t m, int64_t n, int64_t bm, int64_t bn) {
+  (void)bm;
+#pragma omp parallel
+  {
+    float* xin = (float*)malloc(sizeof(float) * (size_t)bn * 2);
+    float* yout = xin + bn;
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < m; r++) {
+      for (int64_t c0 = 0; c0 < n; c0 += bn) {
+        int64_t valid = n - c0 < bn ? n - c0 : bn;
+        for (int64_t j = 0; j < valid; j++) xin[j] = orc_f16_to_f32(x[r * n + c0 + j]);
+        softmax_tile_row(xin, yout, valid, bn);
+        for (int64_t j = 0; j < valid; j++) y[r * n + c0 + j] = orc_f32_to_f16(yout[j]);
+      }
+    }
+    free(xin);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* K4                                                                        */
+/* ------------------------------------------------------------------------ */
+void orc_cpu_gemm_f32(const float* x, const float* y, float* z, int64_t m, int64_t n, int64_t k) {
+  /* acc += x[row*k+inner] * y[inner*n+col] with inner ascending.  The loops are
+   * ordered row / inner / col so the compiler can vectorise across col; every
+   * output element still sees the same sequence of operations. */
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < m; row++) {
+    float* acc = z + row * n;
+    for (int64_t col = 0; col < n; col++) acc[col] = 0.0f;
+    for (int64_t inner = 0; inner < k; inner++) {
+      float xv = x[row * k + inner];
+      const float* yr = y + inner * n;
+      for (int64_t col = 0; col < n; col++) acc[col] += xv * yr[col];
+    }
+  }
+}
+
+void orc_gemm_bf16_f32out(const uint16_t* a, const uint16_t* b, float* c, int64_t m, int64_t n,
+                          int64_t k, const int64_t* rows, int64_t n_rows) {
+  int64_t count = rows ? n_rows : m;
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int64_t ri = 0; ri < count; ri++) {
+    int64_t row = rows ? rows[ri] : ri;
+    float* acc = c + ri * n;
+    for (int64_t col = 0; col < n; col++) acc[col] = 0.0f;
+    for (int64_t inner = 0; inner < k; inner++) {
+      float xv = orc_bf16_to_f32(a[row * k + inner]);
+      const uint16_t* br = b + inner * n;
+      for (int64_t col = 0; col < n; col++) acc[col] += xv * orc_bf16_to_f32(br[col]);
+    }
+  }
+}
+
+void orc_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t m, int64_t n,
+                   int64_t k, const int64_t* rows, int64_t n_rows) {
+  int64_t count = rows ? n_rows : m;
+  float* tmp = (float*)malloc(sizeof(float) * (size_t)count * (size_t)n);
+  orc_gemm_bf16_f32out(a, b, tmp, m, n, k, rows, n_rows);
+  orc_f32_to_bf16_n(tmp, c, (size_t)count * (size_t)n);
+  free(tmp);
+}
+
+/* ------------------------------------------------------------------------ */
+/* K5                                                                        */
+/* ------------------------------------------------------------------------ */
+static inline int64_t idx4(int64_t a, int64_t b, int64_t c, int64_t d, int64_t hsz, int64_t m,
+                           int64_t dsz) {
+  return (((a * hsz + b) * m + c) * dsz) + d;
+}
+
+void orc_fmha_ref_cpu(const float* q, const float* k, const float* v, float* out, int64_t bsz,
+                      int64_t hsz, int64_t hkv, int64_t m, int64_t dsz, float qk_scale,
+                      int64_t input_pos, int64_t query_group_size, int causal,
+                      const int64_t* rows, int64_t n_rows) {
+  int64_t count = rows ? n_rows : bsz * hsz * m;
+#pragma omp parallel
+  {
+    float* scores = (float*)malloc(sizeof(float) * (size_t)m);
+#pragma omp for schedule(dynamic, 16)
+    for (int64_t ri = 0; ri < count; ri++) {
+      int64_t g = rows ? rows[ri] : ri;
+      int64_t i = g % m;
+      int64_t h = (g / m) % hsz;
+      int64_t b = g / (m * hsz);
+      int64_t kv_h = h / query_group_size;
+      float max_logit = -INFINITY;
+      for (int64_t j = 0; j < m; j++) {
+        if (causal && j > i + input_pos) {
+          scores[j] = -INFINITY;
+          continue;
+        }
+        float dot = 0.0f;
+        for (int64_t dd = 0; dd < dsz; dd++)
+          dot += q[idx4(b, h, i, dd, hsz, m, dsz)] * k[idx4(b, kv_h, j, dd, hkv, m, dsz)];
+        scores[j] = dot * qk_scale;
+        max_logit = fmaxf(max_logit, scores[j]);
+      }
+      float denom = 0.0f;
+      for (int64_t j = 0; j < m; j++) {
+        scores[j] = expf(scores[j] - max_logit);
+        denom += scores[j];
+      }
+      float* o = rows ? out + ri * dsz : out + idx4(b, h, i, 0, hsz, m, dsz);
+      for (int64_t dd = 0; dd < dsz; dd++) {
+        float val = 0.0f;
+        for (int64_t j = 0; j < m; j++) {
+          float p = scores[j] / denom;
+          val += p * v[idx4(b, kv_h, j, dd, hkv, m, dsz)];
+        }
+        o[dd] = val;
+      }
+    }
+    free(scores);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* K6                                                                        */
+/* ------------------------------------------------------------------------ */
+void orc_mx_quantize_e4m3(const float* src, uint8_t* data, uint8_t* scales, int64_t rows,
+                          int64_t k) {
+  int64_t kb = k / 32;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; r++) {
+    for (int64_t blk = 0; blk < kb; blk++) {
+      const float* s = src + r * k + blk * 32;
+      float amax = 0.0f;
+      for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(s[j]));
+      /* OCP MX v1.0: shared exponent = floor(log2(amax)) - emax(e4m3 = 8),
+       * clamped to the e8m0 range; an all-zero block takes scale 2^0. */
+      int se = 0;
+      if (amax > 0.0f && isfinite(amax)) {
+        int e;
+        frexpf(amax, &e); /* amax = f * 2^e, f in [0.5,1) -> floor(log2) = e-1 */
+        se = (e - 1) - 8;
+        if (se < -127) se = -127;
+        if (se > 127) se = 127;
+      }
+      scales[r * kb + blk] = (uint8_t)(se + 127);
+      float inv = ldexpf(1.0f, -se);
+      for (int j = 0; j < 32; j++) data[r * k + blk * 32 + j] = orc_f32_to_e4m3fn(s[j] * inv);
+    }
+  }
+}
+
+void orc_mx_dequantize_e4m3(const uint8_t* data, const uint8_t* scales, float* dst, int64_t rows,
+                            int64_t k) {
+  int64_t kb = k / 32;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; r++)
+    for (int64_t j = 0; j < k; j++)
+      dst[r * k + j] = orc_e4m3fn_to_f32(data[r * k + j]) * orc_e8m0_to_f32(scales[r * kb + j / 32]);
+}
+
+void orc_mx_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys,
+                     float* z, int64_t m, int64_t n, int64_t k, float alpha, const int64_t* rows,
+                     int64_t n_rows) {
+  int64_t count = rows ? n_rows : m;
+  int64_t kb = k / 32;
+  float lut[256];
+  for (int i = 0; i < 256; i++) lut[i] = orc_e4m3fn_to_f32((uint8_t)i);
+#pragma omp parallel
+  {
+    float* xrow = (float*)malloc(sizeof(float) * (size_t)k);
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t ri = 0; ri < count; ri++) {
+      int64_t row = rows ? rows[ri] : ri;
+      for (int64_t j = 0; j < k; j++)
+        xrow[j] = lut[x[row * k + j]] * orc_e8m0_to_f32(xs[row * kb + j / 32]);
+      for (int64_t col = 0; col < n; col++) {
+        const uint8_t* yr = y + col * k;
+        float acc = 0.0f;
+        for (int64_t blk = 0; blk < kb; blk++) {
+          float sy = orc_e8m0_to_f32(ys[col * kb + blk]);
+          for (int j = 0; j < 32; j++) acc += xrow[blk * 32 + j] * (lut[yr[blk * 32 + j]] * sy);
+        }
+        z[ri * n + col] = alpha * acc;
+      }
+    }
+    free(xrow);
+  }
+}

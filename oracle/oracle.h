@@ -1,0 +1,121 @@
+/*
+ * CPU oracle for the tile-kernel path.  TEST INFRASTRUCTURE ONLY: nothing in the
+ * shipped library links, loads or calls this; it is the checker the GPU kernels
+ * are compared against, and the CPU baseline that is timed next to them.
+ *
+ * Every function restates, from the reference's text, either a naive CPU
+ * reference the reference's own tests/examples use, or (where the reference has
+ * none) the arithmetic of the kernel body itself.  The reference is Rust and
+ * cannot be built in this image, so there is no compiled-reference cross-check;
+ * each function lists what pins it instead.
+ *
+ *   orc_saxpy_f32        cutile-examples/examples/saxpy.rs:47-53 (answer = a*x+y),
+ *                        evaluated with one fused multiply-add.  Pinned by the
+ *                        reference vectors arange(32), a = 2 (exact either way).
+ *   orc_add_f32          cutile/tests/gpu/add_basic.rs:29-43.
+ *   orc_rms_norm_f16     cutile-kernels/src/norms.rs:28-60 (kernel body; the
+ *                        reference has no CPU reference).  Pinned by closed forms
+ *                        and an independent float64 evaluation: parity unpinned
+ *                        by reference tests.
+ *   orc_softmax_*        cutile-examples/examples/softmax.rs:11-24 (kernel body),
+ *                        row sums = 1 (softmax.rs:55-60).  Pinned by closed forms
+ *                        and scipy.special.softmax: parity unpinned by reference
+ *                        tests beyond the row-sum property.
+ *   orc_cpu_gemm_f32     cutile-examples/examples/persistent_gemm.rs:140-152.
+ *   orc_gemm_bf16        the same loop over bf16-decoded inputs, bf16 (RNE) store.
+ *   orc_fmha_ref_cpu     cutile-examples/examples/flash_attention_causal.rs:140-210.
+ *   orc_mx_*             cutile-examples/examples/mxfp8.rs:25-64 (layout, formula),
+ *                        cuda-core/src/dtype.rs:225-227 (0x38 = 1.0, 0x7F = 2^0);
+ *                        codecs pinned against torch.float8_e4m3fn /
+ *                        float8_e8m0fnu over all 256 codes.  The quantiser is not
+ *                        in the reference (OCP MX v1.0 rule): parity unpinned.
+ */
+#ifndef CUTILE_ORACLE_H
+#define CUTILE_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int orc_num_threads(void);
+void orc_set_num_threads(int n);
+
+/* ---- scalar codecs ---------------------------------------------------- */
+uint16_t orc_f32_to_f16(float f);   /* round-to-nearest-even, IEEE binary16 */
+float orc_f16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float f);  /* round-to-nearest-even */
+float orc_bf16_to_f32(uint16_t h);
+float orc_e4m3fn_to_f32(uint8_t b); /* OCP e4m3fn: bias 7, no inf, S.1111.111 = NaN */
+uint8_t orc_f32_to_e4m3fn(float f); /* RNE, saturating to +-448, NaN -> 0x7F */
+float orc_e8m0_to_f32(uint8_t b);   /* 2^(b-127), 0xFF = NaN */
+
+void orc_f32_to_f16_n(const float* src, uint16_t* dst, size_t n);
+void orc_f16_to_f32_n(const uint16_t* src, float* dst, size_t n);
+void orc_f32_to_bf16_n(const float* src, uint16_t* dst, size_t n);
+void orc_bf16_to_f32_n(const uint16_t* src, float* dst, size_t n);
+
+/* ---- seeded host inputs (SplitMix64 counter stream; same bytes feed the
+ *      oracle and the GPU) ------------------------------------------------ */
+void orc_fill_uniform_f32(float* dst, size_t n, uint64_t seed, float lo, float hi);
+void orc_fill_normal_f32(float* dst, size_t n, uint64_t seed, float mean, float std);
+
+/* ---- K1: saxpy / add --------------------------------------------------- */
+void orc_saxpy_f32(size_t n, float a, const float* x, const float* y, float* z);
+void orc_add_f32(size_t n, const float* x, const float* y, float* z);
+
+/* ---- K2: RMSNorm (f16 IO, f32 math) ----------------------------------- */
+/* block: chunk width of the kernel body's [1,BLOCK] accumulator tile; lane l
+ * accumulates columns l, l+block, ... in order, lanes are then summed in
+ * ascending order. */
+void orc_rms_norm_f16(const uint16_t* x, const uint16_t* w, uint16_t* out, int64_t rows,
+                      int64_t n, float eps, int64_t block);
+/* independent float64 evaluation of the same formula (pins the f32 one) */
+void orc_rms_norm_f16_f64(const uint16_t* x, const uint16_t* w, uint16_t* out, int64_t rows,
+                          int64_t n, double eps);
+
+/* ---- K3: softmax over tiles [bm, bn] ---------------------------------- */
+/* f32 IO.  Tile (i, j) covers rows i*bm.., cols j*bn..; every tile row is
+ * normalised on its own (row softmax iff bn == n).  Columns beyond n read as 0
+ * and are not stored (zero padded loads, masked stores). */
+void orc_softmax_f32(const float* x, float* y, int64_t m, int64_t n, int64_t bm, int64_t bn);
+/* f16 IO, f32 statistics */
+void orc_softmax_f16(const uint16_t* x, uint16_t* y, int64_t m, int64_t n, int64_t bm, int64_t bn);
+
+/* ---- K4: GEMM ---------------------------------------------------------- */
+void orc_cpu_gemm_f32(const float* x, const float* y, float* z, int64_t m, int64_t n, int64_t k);
+/* bf16 A[m,k], B[k,n] row-major, f32 accumulate in k order, bf16 C.  If
+ * rows != NULL only the listed n_rows rows of C are computed into c (packed
+ * [n_rows, n]). */
+void orc_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t m, int64_t n,
+                   int64_t k, const int64_t* rows, int64_t n_rows);
+/* same with f32 result (no output rounding) */
+void orc_gemm_bf16_f32out(const uint16_t* a, const uint16_t* b, float* c, int64_t m, int64_t n,
+                          int64_t k, const int64_t* rows, int64_t n_rows);
+
+/* ---- K5: FMHA ---------------------------------------------------------- */
+/* q (b,h,m,d), k/v (b,hkv,m,d), out (b,h,m,d), all f32.  If rows != NULL only
+ * the n_rows listed global query rows (index into b*h*m) are computed, packed
+ * [n_rows, d]. */
+void orc_fmha_ref_cpu(const float* q, const float* k, const float* v, float* out, int64_t bsz,
+                      int64_t hsz, int64_t hkv, int64_t m, int64_t dsz, float qk_scale,
+                      int64_t input_pos, int64_t query_group_size, int causal,
+                      const int64_t* rows, int64_t n_rows);
+
+/* ---- K6: MX block-scaled fp8 GEMM ------------------------------------- */
+/* Quantise src[rows, k] (f32) per 32 contiguous K elements: scale byte e8m0,
+ * data bytes e4m3fn.  scales is [rows, k/32]. */
+void orc_mx_quantize_e4m3(const float* src, uint8_t* data, uint8_t* scales, int64_t rows,
+                          int64_t k);
+void orc_mx_dequantize_e4m3(const uint8_t* data, const uint8_t* scales, float* dst, int64_t rows,
+                            int64_t k);
+/* z[m,n] = alpha * sum_k x[i,k] sx[i,k/32] * y[j,k] sy[j,k/32]; y is stored
+ * [n,k].  f32 accumulate in k order.  Row subset as for orc_gemm_bf16. */
+void orc_mx_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys,
+                     float* z, int64_t m, int64_t n, int64_t k, float alpha, const int64_t* rows,
+                     int64_t n_rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

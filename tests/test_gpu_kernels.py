@@ -1,0 +1,335 @@
+"""GPU parity tests: every hot-path kernel through the C ABI against the CPU oracle on the
+same seeded inputs.  Tolerances: saxpy / add / creation bit exact; RMSNorm and softmax
+f16 within 1 f16 ulp of the oracle (the oracle's f32 sums are ordered differently);
+bf16 GEMM rel-L2 <= 1e-2; FMHA max-abs <= 2e-2; MXFP8 GEMM rel-L2 <= 3e-2 against the
+f32 dequantised reference."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import (f16_ulp_diff, from_dev_bf16_bits, from_dev_f16_bits, normal_bf16_bits, normal_f16_bits, rel_l2,
+                  to_dev_bf16, to_dev_f16)
+
+pytestmark = pytest.mark.gpu
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+# ---- K1: saxpy / add ------------------------------------------------------------------------
+def test_device_is_gfx950(ct, dev):
+    assert "gfx950" in ct.device_arch(0)
+    p = ct.device_props(0)
+    assert p.wavefront_size == 64 and p.compute_units > 0
+
+
+def test_saxpy_reference_vectors(ct, dev):
+    # cutile-examples/examples/saxpy.rs:27-53: arange(32) as [4,8], tiles [2,2], a = 2
+    base = torch.arange(32, dtype=torch.float32, device=dev)
+    x = base.clone().reshape(4, 8)
+    y = base.clone().reshape(4, 8)
+    ct.saxpy(ct.partition(y, [2, 2]), 2.0, x)
+    sync()
+    assert torch.equal(y.flatten(), 2.0 * base + base)
+
+
+@pytest.mark.parametrize("variant", [None, "f32_r1_tiled"])
+@pytest.mark.parametrize("n", [1 << 20, 1000003, 1024, 5])
+def test_saxpy_1d_bit_exact(ct, dev, n, variant):
+    x, y = oracle.uniform_f32(n, 11), oracle.uniform_f32(n, 12)
+    yd = torch.from_numpy(y.copy()).to(dev)
+    ct.saxpy(ct.partition(yd, [1024]), 2.0, torch.from_numpy(x).to(dev), variant=variant)
+    sync()
+    assert np.array_equal(yd.cpu().numpy(), oracle.saxpy_f32(2.0, x, y))
+
+
+def test_axpy_separate_output_bit_exact(ct, dev):
+    n = (1 << 20) + 3
+    x, y = oracle.uniform_f32(n, 21), oracle.uniform_f32(n, 22)
+    zd = torch.empty(n, dtype=torch.float32, device=dev)
+    ct.axpy(ct.partition(zd, [1024]), 2.0, torch.from_numpy(x).to(dev), torch.from_numpy(y).to(dev))
+    sync()
+    assert np.array_equal(zd.cpu().numpy(), oracle.saxpy_f32(2.0, x, y))
+
+
+def test_saxpy_2d_ragged_and_padded_input(ct, dev):
+    # y [37, 53] tiled [8, 16] (ragged both ways); x is smaller: rows/cols beyond it read 0
+    y = oracle.uniform_f32((37, 53), 31)
+    x = oracle.uniform_f32((30, 40), 32)
+    yd = torch.from_numpy(y.copy()).to(dev)
+    ct.saxpy(ct.partition(yd, [8, 16]), 1.5, torch.from_numpy(x).to(dev))
+    sync()
+    xp = np.zeros_like(y)
+    xp[:30, :40] = x
+    assert np.array_equal(yd.cpu().numpy(), oracle.saxpy_f32(1.5, xp, y).reshape(37, 53))
+
+
+def test_saxpy_strided_view(ct, dev):
+    big = torch.from_numpy(oracle.uniform_f32((64, 96), 41)).to(dev)
+    yv = big[:, 16:80]                      # row stride 96, 64 columns
+    x = torch.from_numpy(oracle.uniform_f32((64, 64), 42)).to(dev)
+    expect = torch.from_numpy(oracle.saxpy_f32(3.0, x.cpu().numpy(), yv.cpu().numpy().copy())).reshape(64, 64)
+    untouched = big[:, :16].clone()
+    ct.saxpy(ct.partition(yv, [16, 16]), 3.0, x)
+    sync()
+    assert torch.equal(yv.cpu(), expect) and torch.equal(big[:, :16], untouched)
+
+
+def test_saxpy_prefix_grid_leaves_tail_untouched(ct, dev):
+    n = 8192
+    x, y = oracle.uniform_f32(n, 51), oracle.uniform_f32(n, 52)
+    yd = torch.from_numpy(y.copy()).to(dev)
+    ct.saxpy(ct.partition(yd, [1024], prefix=True), 2.0, torch.from_numpy(x).to(dev), grid=(3, 1, 1))
+    sync()
+    got = yd.cpu().numpy()
+    assert np.array_equal(got[:3072], oracle.saxpy_f32(2.0, x[:3072], y[:3072])) and np.array_equal(got[3072:], y[3072:])
+
+
+def test_add_ones(ct, dev):
+    # cutile/tests/gpu/add_basic.rs:29-43
+    x = torch.ones(4096, device=dev)
+    z = torch.zeros(4096, device=dev)
+    ct.add(ct.partition(z, [128]), x, x)
+    sync()
+    assert torch.equal(z, torch.full_like(z, 2.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_add_16bit(ct, dev, dtype):
+    n = 1 << 18
+    x = torch.from_numpy(oracle.uniform_f32(n, 61)).to(dev).to(dtype)
+    y = torch.from_numpy(oracle.uniform_f32(n, 62)).to(dev).to(dtype)
+    z = torch.zeros_like(x)
+    ct.add(ct.partition(z, [16384]), x, y)
+    sync()
+    assert torch.equal(z, x + y)
+
+
+# ---- K7: creation / conversion --------------------------------------------------------------
+@pytest.mark.parametrize("dtype,value", [(torch.float32, 3.5), (torch.float16, -2.25), (torch.bfloat16, 1.0),
+                                         (torch.int32, 7), (torch.int64, -9), (torch.uint8, 200), (torch.float64, 0.1)])
+def test_full(ct, dev, dtype, value):
+    t = torch.zeros(1000, dtype=dtype, device=dev)
+    ct.full(value, ct.partition(t, [128]))
+    sync()
+    assert torch.equal(t, torch.full_like(t, value))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int32, torch.int64, torch.float16])
+def test_arange(ct, dev, dtype):
+    t = torch.zeros(1000, dtype=dtype, device=dev)
+    ct.arange(ct.partition(t, [128]))
+    sync()
+    assert torch.equal(t, torch.arange(1000, device=dev).to(dtype))
+
+
+def test_linspace(ct, dev):
+    t = torch.zeros(257, device=dev)
+    ct.linspace(ct.partition(t, [128]), 1.0, 0.5)
+    sync()
+    assert torch.equal(t, 1.0 + torch.arange(257, device=dev).float() * 0.5)
+
+
+@pytest.mark.parametrize("src,dst", [(torch.int32, torch.float32), (torch.float32, torch.float16),
+                                     (torch.float32, torch.bfloat16), (torch.float16, torch.float32),
+                                     (torch.float64, torch.int64), (torch.bfloat16, torch.float16)])
+def test_convert(ct, dev, src, dst):
+    s = (torch.from_numpy(oracle.uniform_f32(1024, 71, -100, 100)).to(dev)).to(src)
+    d = torch.zeros(1024, dtype=dst, device=dev)
+    ct.convert(s, ct.partition(d, [128]))
+    sync()
+    assert torch.equal(d, s.to(dst))
+
+
+# ---- K2: RMSNorm ----------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,n,variant", [
+    (64, 512, None), (33, 1024, None), (16, 2048, None), (16, 4096, None), (32, 8192, None),
+    (32, 8192, "w4v4"), (32, 8192, "w2v8"), (32, 8192, "w4v8"), (8, 16384, None), (8, 32768, None),
+    (16, 8192, "generic"), (7, 1000, None), (5, 24, None), (4, 8, None),
+])
+def test_rms_norm_f16(ct, dev, rows, n, variant):
+    xb = normal_f16_bits((rows, n), 101)
+    wb = oracle.f32_to_f16_bits(oracle.uniform_f32(n, 102, 0.5, 1.5))
+    out = torch.zeros(rows, n, dtype=torch.float16, device=dev)
+    ct.rms_norm_f16(to_dev_f16(xb, dev), to_dev_f16(wb, dev), ct.partition(out, [1, n]), 1e-6, variant=variant)
+    sync()
+    ref = oracle.rms_norm_f16(xb, wb, 1e-6)
+    assert f16_ulp_diff(from_dev_f16_bits(out), ref).max() <= 1
+
+
+def test_rms_norm_f16_strided_rows_and_prefix(ct, dev):
+    rows, n = 24, 1024
+    xb = normal_f16_bits((rows, 2 * n), 111)
+    wb = oracle.f32_to_f16_bits(oracle.uniform_f32(n, 112, 0.5, 1.5))
+    xd = to_dev_f16(xb, dev)[:, :n]          # row stride 2n
+    out = torch.zeros(rows, n, dtype=torch.float16, device=dev)
+    ct.rms_norm_f16(xd, to_dev_f16(wb, dev), ct.partition(out, [1, n], prefix=True), 1e-6, grid=(10, 1, 1))
+    sync()
+    ref = oracle.rms_norm_f16(np.ascontiguousarray(xb[:, :n]), wb, 1e-6)
+    got = from_dev_f16_bits(out)
+    assert f16_ulp_diff(got[:10], ref[:10]).max() <= 1 and not got[10:].any()
+
+
+# ---- K3: softmax ----------------------------------------------------------------------------
+@pytest.mark.parametrize("m,n,bm,bn,variant", [
+    (64, 1024, 1, 1024, None), (16, 8192, 1, 8192, None), (16, 8192, 2, 8192, "f16_w4v4"),
+    (16, 8192, 1, 2048, None),          # chunk softmax: four independent tiles per row
+    (9, 4096, 4, 4096, None), (6, 1000, 2, 1000, None), (6, 1000, 2, 512, None),
+    (8, 16384, 1, 16384, None), (16, 4096, 1, 4096, "f16_generic"),
+])
+def test_softmax_f16(ct, dev, m, n, bm, bn, variant):
+    xb = normal_f16_bits((m, n), 201, 2.0)
+    y = torch.zeros(m, n, dtype=torch.float16, device=dev)
+    ct.softmax(to_dev_f16(xb, dev), ct.partition(y, [bm, bn]), variant=variant)
+    sync()
+    ref = oracle.softmax_f16(xb, bm, bn)
+    got = from_dev_f16_bits(y)
+    assert f16_ulp_diff(got, ref).max() <= 1
+
+
+@pytest.mark.parametrize("m,n,bm,bn", [(4, 8, 2, 8), (32, 4096, 2, 4096), (8, 8192, 1, 8192), (5, 100, 1, 100),
+                                       (8, 2048, 1, 512)])
+def test_softmax_f32(ct, dev, m, n, bm, bn):
+    x = oracle.normal_f32((m, n), 211, 0, 2.0) if (m, n) != (4, 8) else np.arange(32, dtype=np.float32).reshape(4, 8)
+    y = torch.zeros(m, n, device=dev)
+    ct.softmax(torch.from_numpy(x).to(dev), ct.partition(y, [bm, bn]))
+    sync()
+    got = y.cpu().numpy()
+    ref = oracle.softmax_f32(x, bm, bn)
+    np.testing.assert_allclose(got, ref, rtol=2e-5, atol=1e-9)
+    if bn == n:  # cutile-examples/examples/softmax.rs:55-60: rows sum to 1
+        np.testing.assert_allclose(got.sum(axis=1), 1.0, atol=1e-4)
+
+
+# ---- K4: bf16 GEMM --------------------------------------------------------------------------
+GEMM_VARIANTS = ["bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
+                 "bf16_128x256x64_w2x2", "bf16_128x128x64_w2x2", "bf16_64x128x64_w2x2"]
+
+
+@pytest.mark.parametrize("variant", GEMM_VARIANTS)
+def test_gemm_bf16_variants(ct, dev, variant):
+    bm, bn = (int(v) for v in variant.split("_")[1].split("x")[:2])
+    m, n, k = 512, 768, 320
+    a, b = normal_bf16_bits((m, k), 301, k ** -0.5), normal_bf16_bits((k, n), 302, k ** -0.5)
+    z = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    ct.gemm(ct.partition(z, [bm, bn]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=False, variant=variant)
+    sync()
+    ref = oracle.gemm_bf16(a, b, f32out=True)
+    got = z.float().cpu().numpy()
+    assert rel_l2(got, ref) <= 1e-2
+    # tighter: bf16 rounding of an f32-accumulated result is within 1 bf16 ulp-ish of the oracle
+    np.testing.assert_allclose(got, ref, rtol=1.6e-2, atol=2e-3)
+
+
+def test_gemm_ones_known_answer_non_divisible(ct, dev):
+    # cutile/tests/slice_non_divisible.rs:459-500: ones x ones = K, M and N not multiples of the tile
+    m, n, k = 200, 264, 128
+    x = torch.ones(m, k, dtype=torch.bfloat16, device=dev)
+    y = torch.ones(k, n, dtype=torch.bfloat16, device=dev)
+    z = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    ct.gemm(ct.partition(z, [128, 128]), x, y, k)
+    sync()
+    assert torch.equal(z.float(), torch.full((m, n), float(k), device=dev))
+
+
+def test_gemm_accumulates_into_z_and_f32_out(ct, dev):
+    m = n = k = 256
+    a, b = normal_bf16_bits((m, k), 311, k ** -0.5), normal_bf16_bits((k, n), 312, k ** -0.5)
+    z0 = oracle.normal_f32((m, n), 313)
+    z = torch.from_numpy(z0.copy()).to(dev)
+    ct.gemm(ct.partition(z, [128, 128]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=True)
+    sync()
+    ref = oracle.gemm_bf16(a, b, f32out=True) + z0
+    np.testing.assert_allclose(z.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_gemm_k_not_multiple_of_kernel_tile(ct, dev):
+    m, n, k = 128, 128, 96                    # three BK=32 tiles of the tile program, 1.5 kernel K tiles
+    a, b = normal_bf16_bits((m, k), 321, k ** -0.5), normal_bf16_bits((k, n), 322, k ** -0.5)
+    z = torch.zeros(m, n, dtype=torch.float32, device=dev)
+    ct.gemm(ct.partition(z, [128, 128]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=False,
+            generics=["bf16", 128, 128, 32])
+    sync()
+    np.testing.assert_allclose(z.cpu().numpy(), oracle.gemm_bf16(a, b, f32out=True), rtol=1e-4, atol=1e-4)
+
+
+# ---- K5: FMHA -------------------------------------------------------------------------------
+def _fmha_case(ct, dev, b, h, hkv, s, d, bm, causal, input_pos, dtype=torch.bfloat16, variant=None, seed=401):
+    rnd = lambda shape, sd: oracle.normal_f32(shape, sd)
+    cast = (lambda x: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(x))) if dtype == torch.bfloat16 else (
+        lambda x: oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(x)))
+    q, k, v = cast(rnd((b, h, s, d), seed)), cast(rnd((b, hkv, s, d), seed + 1)), cast(rnd((b, hkv, s, d), seed + 2))
+    out = torch.zeros(b * h, s, d, dtype=dtype, device=dev)
+    td = lambda t: torch.from_numpy(t).to(dev).to(dtype)
+    scale = 1.0 / np.sqrt(d)
+    ct.fmha(ct.partition(out, [1, bm, d]), td(q), td(k), td(v), scale, input_pos, h // hkv, causal=causal,
+            variant=variant)
+    sync()
+    ref = oracle.fmha_ref_cpu(q, k, v, scale, input_pos, h // hkv, causal).reshape(b * h, s, d)
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    return np.max(np.abs(got - ref))
+
+
+@pytest.mark.parametrize("causal,input_pos", [(False, 0), (True, 5), (True, 0)])
+def test_fmha_reference_example_shape(ct, dev, causal, input_pos):
+    # cutile-examples/examples/flash_attention_causal.rs:216-222: (2, 8, 8, 64, 32), tiles (32, 32)
+    assert _fmha_case(ct, dev, 2, 8, 8, 64, 32, 32, causal, input_pos) <= 2e-2
+
+
+@pytest.mark.parametrize("variant", ["bf16_128x64x128", "bf16_128x128x128", "bf16_256x64x128"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_d128(ct, dev, variant, causal):
+    bm = int(variant.split("_")[1].split("x")[0])
+    assert _fmha_case(ct, dev, 1, 2, 2, 512, 128, bm, causal, 0, variant=variant) <= 2e-2
+
+
+def test_fmha_gqa_and_ragged_lengths(ct, dev):
+    # 4 query heads share 2 kv heads; seq 200 is not a multiple of BM=64 or BN=64
+    assert _fmha_case(ct, dev, 1, 4, 2, 200, 64, 64, True, 0) <= 2e-2
+    assert _fmha_case(ct, dev, 1, 4, 2, 200, 64, 64, False, 0) <= 2e-2
+
+
+def test_fmha_f16(ct, dev):
+    assert _fmha_case(ct, dev, 1, 2, 2, 256, 128, 128, True, 0, dtype=torch.float16) <= 2e-2
+
+
+# ---- K6: MXFP8 GEMM -------------------------------------------------------------------------
+def test_mxfp8_all_ones_known_answer(ct, dev):
+    # cutile-examples/examples/mxfp8.rs:84-135: e4m3 0x38 (1.0), e8m0 0x7F (2^0) -> every output = K
+    m = n = 16
+    k = 128
+    x = torch.full((m, k), 0x38, dtype=torch.uint8, device=dev)
+    y = torch.full((n, k), 0x38, dtype=torch.uint8, device=dev)
+    xs = torch.full((m, k // 32), 0x7F, dtype=torch.uint8, device=dev)
+    ys = torch.full((n, k // 32), 0x7F, dtype=torch.uint8, device=dev)
+    z = torch.zeros(m, n, device=dev)
+    ct.linear_tile_mxfp8(ct.partition(z, [16, 16]), x, y, xs, ys, 1.0, generics=[16, 16, 64, 2])
+    sync()
+    assert torch.allclose(z, torch.full_like(z, float(k)), atol=1e-3)
+
+
+@pytest.mark.parametrize("m,n,k,tile,out_dtype,variant", [
+    (128, 128, 256, 128, torch.float32, None), (256, 256, 512, 256, torch.float32, None),
+    (256, 256, 512, 256, torch.bfloat16, None), (512, 256, 384, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_w2x4"),
+    (96, 160, 256, 32, torch.float32, None), (64, 64, 128, 64, torch.float32, None),
+])
+def test_mxfp8_random_blocks(ct, dev, m, n, k, tile, out_dtype, variant):
+    # per-row scale spread exercises distinct e8m0 codes per 32-block
+    xf = oracle.normal_f32((m, k), 501) * np.exp2(oracle.uniform_f32((m, k // 32), 503, -6, 6)).repeat(32, axis=1)
+    yf = oracle.normal_f32((n, k), 502) * np.exp2(oracle.uniform_f32((n, k // 32), 504, -6, 6)).repeat(32, axis=1)
+    xq, xs = oracle.mx_quantize_e4m3(xf)
+    yq, ys = oracle.mx_quantize_e4m3(yf)
+    assert len(np.unique(xs)) > 4
+    z = torch.zeros(m, n, dtype=out_dtype, device=dev)
+    td = lambda t: torch.from_numpy(t).to(dev)
+    ct.linear_tile_mxfp8(ct.partition(z, [tile, tile]), td(xq), td(yq), td(xs), td(ys), 0.5, variant=variant)
+    sync()
+    ref = oracle.mx_gemm_f32(xq, yq, xs, ys, 0.5)
+    got = z.float().cpu().numpy()
+    tol = 3e-2
+    assert rel_l2(got, ref) <= tol
+    if out_dtype == torch.float32:      # exact products of fp8 values: only summation order differs
+        assert rel_l2(got, ref) <= 1e-5

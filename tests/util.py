@@ -1,0 +1,45 @@
+"""Helpers shared by the GPU parity tests: seeded host inputs from the oracle's PRNG,
+moved to the device as the exact same bytes the oracle sees."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import oracle
+
+
+def to_dev_f16(bits: np.ndarray, dev) -> torch.Tensor:
+    return torch.from_numpy(bits.view(np.float16)).to(dev)
+
+
+def to_dev_bf16(bits: np.ndarray, dev) -> torch.Tensor:
+    return torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.bfloat16)
+
+
+def from_dev_f16_bits(t: torch.Tensor) -> np.ndarray:
+    return t.cpu().numpy().view(np.uint16)
+
+
+def from_dev_bf16_bits(t: torch.Tensor) -> np.ndarray:
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def normal_f16_bits(shape, seed, std=1.0) -> np.ndarray:
+    return oracle.f32_to_f16_bits(oracle.normal_f32(shape, seed, 0.0, std))
+
+
+def normal_bf16_bits(shape, seed, std=1.0) -> np.ndarray:
+    return oracle.f32_to_bf16_bits(oracle.normal_f32(shape, seed, 0.0, std))
+
+
+def f16_ulp_diff(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    """Distance in units of f16 representable values (sign-magnitude -> ordered ints)."""
+    def ordered(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(ordered(a_bits) - ordered(b_bits))
+
+
+def rel_l2(got: np.ndarray, ref: np.ndarray) -> float:
+    return float(np.linalg.norm(got.astype(np.float64) - ref.astype(np.float64)) /
+                 max(np.linalg.norm(ref.astype(np.float64)), 1e-30))
