@@ -1,0 +1,376 @@
+#!/usr/bin/env python3
+"""Throughput of the tile-kernel path on one MI355X, against the kernel's roofline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
+
+A step is one launch of the hot-path kernel over one batch of synthetic input that is
+already resident in HBM.  The headline workload is the bf16 GEMM at M = N = K = 8192
+(the configuration the target fractions are quoted on); every other BASELINE
+configuration is measured the same way and reported under "also" in the same JSON line.
+
+Timing: W untimed launches, then exactly K launches between two device synchronisations
+(wall clock -> ms_per_step / value), and the same K launches bracketed by HIP events on
+the launch stream (-> the kernel's average duration, used for roofline.achieved).
+
+cpu_baseline: the CPU oracle (a port of the reference's naive CPU references), timed on
+this host's cores on a bounded sample of the same workload.  The sampled output is also
+compared against the GPU result ("parity").
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"hbm": (8000.0, "GB/s"), "mfma_bf16": (2500.0, "TFLOP/s"), "mfma_fp8": (5000.0, "TFLOP/s")}
+METRIC = "GEMM/FMHA TFLOP/s + % MFMA peak; RMSNorm GB/s + % HBM peak (1 MI355X)"
+
+
+def _traffic(workload):
+    """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f).get(workload)
+    return None
+
+
+class Workload:
+    name = ""
+    unit = ""
+    dtype = ""
+    bound = "hbm"
+    peak_key = "hbm"
+    work = 0.0          # algorithmic bytes or flops per launch
+    config = {}
+
+    def setup(self, ct, torch, oracle, dev):
+        raise NotImplementedError
+
+    def launch(self):
+        raise NotImplementedError
+
+    def cpu_baseline(self, oracle, np, torch):
+        return None
+
+
+def _td_bf16(torch, np, bits, dev):
+    return torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.bfloat16)
+
+
+class Saxpy(Workload):
+    name, unit, dtype = "saxpy_f32_16777216", "GB/s", "f32"
+    n = 1 << 24
+    work = 12.0 * n
+    config = {"workload": "saxpy fp32 z = a*x + y, n = 16777216, a = 2.0, tiles of 1024"}
+
+    def setup(self, ct, torch, oracle, dev):
+        self.ct = ct
+        self.xh, self.yh = oracle.uniform_f32(self.n, 1), oracle.uniform_f32(self.n, 2)
+        self.x, self.y = torch.from_numpy(self.xh).to(dev), torch.from_numpy(self.yh).to(dev)
+        self.z = torch.empty_like(self.x)
+        self.zp = ct.partition(self.z, [1024])
+
+    def launch(self):
+        self.ct.axpy(self.zp, 2.0, self.x, self.y)
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        reps = 20
+        for _ in range(reps):
+            ref = oracle.saxpy_f32(2.0, self.xh, self.yh)
+        dt = (time.perf_counter() - t0) / reps
+        exact = bool(np.array_equal(self.z.cpu().numpy(), ref))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"full size, {reps} passes"}, {"bit_exact": exact}
+
+
+class Copy(Workload):
+    """A plain copy of known size; used to calibrate the HBM traffic counters."""
+    name, unit, dtype = "copy_f32_67108864", "GB/s", "f32"
+    n = 1 << 26
+    work = 8.0 * n
+    config = {"workload": "plain copy of 2^26 f32 (convert f32 -> f32), calibration for FETCH_SIZE / WRITE_SIZE"}
+
+    def setup(self, ct, torch, oracle, dev):
+        self.ct = ct
+        self.x = torch.arange(self.n, dtype=torch.float32, device=dev)
+        self.z = torch.empty_like(self.x)
+        self.zp = ct.partition(self.z, [128])
+
+    def launch(self):
+        self.ct.convert(self.x, self.zp)
+
+
+class RmsNorm(Workload):
+    name, unit, dtype = "rms_norm_f16_16384x8192", "GB/s", "f16 io / f32 math"
+    m, n = 16384, 8192
+    work = float(2 * m * n * 2 + n * 2)
+    config = {"workload": "RMSNorm fp16 rows [16384, 8192], weight [8192], eps 1e-6"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.xb = oracle.f32_to_f16_bits(oracle.normal_f32((self.m, self.n), 3))
+        self.wb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.n, 4, 0.5, 1.5))
+        self.x = torch.from_numpy(self.xb.view(np.float16)).to(dev)
+        self.w = torch.from_numpy(self.wb.view(np.float16)).to(dev)
+        self.o = torch.empty_like(self.x)
+        self.op = ct.partition(self.o, [1, self.n])
+
+    def launch(self):
+        self.ct.rms_norm_f16(self.x, self.w, self.op, 1e-6)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 2048
+        t0 = time.perf_counter()
+        ref = oracle.rms_norm_f16(self.xb[:rows], self.wb, 1e-6)
+        dt = time.perf_counter() - t0
+        got = self.o[:rows].cpu().numpy().view(np.uint16)
+        d = np.abs(oracle.f16_bits_to_f32(got) - oracle.f16_bits_to_f32(ref))
+        ok = bool(np.all(d <= np.abs(oracle.f16_bits_to_f32(ref)) * 2 ** -10 + 1e-7))
+        return {"value": (2 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                "kind": "port", "sample": f"first {rows} of {self.m} rows"}, {"within_1_f16_ulp": ok}
+
+
+class Softmax(RmsNorm):
+    name = "softmax_f16_16384x8192"
+    work = float(2 * RmsNorm.m * RmsNorm.n * 2)
+    config = {"workload": "row softmax fp16 [16384, 8192], tiles [1, 8192]"}
+
+    def launch(self):
+        self.ct.softmax(self.x, self.op)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 2048
+        t0 = time.perf_counter()
+        ref = oracle.softmax_f16(self.xb[:rows], 1, self.n)
+        dt = time.perf_counter() - t0
+        got = self.o[:rows].cpu().numpy().view(np.uint16)
+        d = np.abs(oracle.f16_bits_to_f32(got) - oracle.f16_bits_to_f32(ref))
+        ok = bool(np.all(d <= np.abs(oracle.f16_bits_to_f32(ref)) * 2 ** -10 + 1e-7))
+        return {"value": (2 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                "kind": "port", "sample": f"first {rows} of {self.m} rows"}, {"within_1_f16_ulp": ok}
+
+
+class Gemm(Workload):
+    unit, dtype, bound, peak_key = "TFLOP/s", "bf16 in / f32 acc / bf16 out", "mfma", "mfma_bf16"
+    tile = (256, 256)
+
+    def __init__(self, s):
+        self.s = s
+        self.name = f"gemm_bf16_{s}"
+        self.work = 2.0 * s ** 3
+        self.config = {"workload": f"GEMM bf16 M=N=K={s}, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 out",
+                       "tile": "256x256x64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        s = self.s
+        self.ct = ct
+        self.ab = oracle.f32_to_bf16_bits(oracle.normal_f32((s, s), 5, 0, s ** -0.5))
+        self.bb = oracle.f32_to_bf16_bits(oracle.normal_f32((s, s), 6, 0, s ** -0.5))
+        self.a, self.b = _td_bf16(torch, np, self.ab, dev), _td_bf16(torch, np, self.bb, dev)
+        self.z = torch.zeros(s, s, dtype=torch.bfloat16, device=dev)
+        self.zp = ct.partition(self.z, list(self.tile))
+
+    def launch(self):
+        self.ct.gemm(self.zp, self.a, self.b, self.s, accumulate=False)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rng = np.random.default_rng(7)
+        rows = np.sort(rng.choice(self.s, size=1024 if self.s >= 8192 else 512, replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        ref = oracle.gemm_bf16(self.ab, self.bb, rows=rows, f32out=True)
+        dt = time.perf_counter() - t0
+        got = self.z[torch.from_numpy(rows).to(self.z.device)].float().cpu().numpy()
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        flops = 2.0 * len(rows) * self.s * self.s
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"{len(rows)} of {self.s} output rows of the same problem (naive f32 loop)"}, \
+               {"rel_l2_sampled_rows": rel, "tolerance": 1e-2, "ok": rel <= 1e-2}
+
+
+class Fmha(Workload):
+    unit, dtype, bound, peak_key = "TFLOP/s", "bf16 io / f32 softmax+acc", "mfma", "mfma_bf16"
+    b, h, s, d = 4, 32, 4096, 128
+    bm = 256
+
+    def __init__(self, causal):
+        self.causal = causal
+        self.name = "fmha_bf16_causal" if causal else "fmha_bf16"
+        self.work = (2.0 if causal else 4.0) * self.s * self.s * self.d * self.h * self.b
+        self.config = {"workload": f"FMHA fwd bf16 b=4 h=32 s=4096 d=128 {'causal' if causal else 'non-causal'}, "
+                                   "scale 1/sqrt(128)", "tile": f"BM={self.bm}"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        shape = (self.b, self.h, self.s, self.d)
+        self.qb, self.kb, self.vb = (oracle.f32_to_bf16_bits(oracle.normal_f32(shape, 8 + i)) for i in range(3))
+        self.q, self.k, self.v = (_td_bf16(torch, np, t, dev) for t in (self.qb, self.kb, self.vb))
+        self.o = torch.zeros(self.b * self.h, self.s, self.d, dtype=torch.bfloat16, device=dev)
+        self.op = ct.partition(self.o, [1, self.bm, self.d])
+
+    def launch(self):
+        self.ct.fmha(self.op, self.q, self.k, self.v, self.d ** -0.5, 0, 1, causal=self.causal)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rng = np.random.default_rng(9)
+        total = self.b * self.h * self.s
+        rows = np.sort(rng.choice(total, size=65536, replace=False)).astype(np.int64)
+        q, k, v = (oracle.bf16_bits_to_f32(t) for t in (self.qb, self.kb, self.vb))
+        t0 = time.perf_counter()
+        ref = oracle.fmha_ref_cpu(q, k, v, self.d ** -0.5, 0, 1, self.causal, rows=rows)
+        dt = time.perf_counter() - t0
+        got = self.o.reshape(total, self.d)[torch.from_numpy(rows).to(self.o.device)].float().cpu().numpy()
+        err = float(np.max(np.abs(got - ref)))
+        flops = len(rows) * 4.0 * self.s * self.d        # the reference evaluates every key, masked or not
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"{len(rows)} of {total} query rows of the same problem"}, \
+               {"max_abs_sampled_rows": err, "tolerance": 2e-2, "ok": err <= 2e-2}
+
+
+class MxGemm(Workload):
+    name, unit, bound, peak_key = "mxfp8_gemm_8192", "TFLOP/s", "mfma", "mfma_fp8"
+    dtype = "fp8 e4m3 x e8m0 block scale / f32 acc / bf16 out"
+    s = 8192
+    work = 2.0 * s ** 3
+    tile = 128
+    config = {"workload": "MX block-scaled fp8 GEMM A[8192,8192] B[8192,8192], e4m3 + e8m0 per 32 K, bf16 out",
+              "tile": "128x128x128"}
+
+    def setup(self, ct, torch, oracle, dev):
+        s = self.s
+        self.ct = ct
+        self.xq, self.xs = oracle.mx_quantize_e4m3(oracle.normal_f32((s, s), 12))
+        self.yq, self.ys = oracle.mx_quantize_e4m3(oracle.normal_f32((s, s), 13))
+        td = lambda t: torch.from_numpy(t).to(dev)
+        self.x, self.y, self.xsd, self.ysd = td(self.xq), td(self.yq), td(self.xs), td(self.ys)
+        self.z = torch.zeros(s, s, dtype=torch.bfloat16, device=dev)
+        self.zp = ct.partition(self.z, [self.tile, self.tile])
+
+    def launch(self):
+        self.ct.linear_tile_mxfp8(self.zp, self.x, self.y, self.xsd, self.ysd, 1.0)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rng = np.random.default_rng(11)
+        rows = np.sort(rng.choice(self.s, size=128, replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        ref = oracle.mx_gemm_f32(self.xq, self.yq, self.xs, self.ys, 1.0, rows=rows)
+        dt = time.perf_counter() - t0
+        got = self.z[torch.from_numpy(rows).to(self.z.device)].float().cpu().numpy()
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        flops = 2.0 * len(rows) * self.s * self.s
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"{len(rows)} of {self.s} output rows, f32 dequantised reference"}, \
+               {"rel_l2_sampled_rows": rel, "tolerance": 3e-2, "ok": rel <= 3e-2}
+
+
+def make_workloads():
+    return [Gemm(8192), Gemm(4096), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm()]
+
+
+EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run
+
+
+def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np):
+    for _ in range(warmup):
+        w.launch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        w.launch()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    timer = ct.EventTimer()
+    timer.start()
+    for _ in range(steps):
+        w.launch()
+    kernel_ms = timer.stop() / steps
+    timer.close()
+    scale = 1e9 if w.unit == "GB/s" else 1e12
+    peak, punit = PEAK[w.peak_key]
+    achieved = w.work / (kernel_ms * 1e-3) / scale
+    rec = {
+        "workload": w.name, "value": w.work / (wall_ms * 1e-3) / scale, "unit": w.unit, "ms_per_step": wall_ms,
+        "dtype": w.dtype, "config": w.config,
+        "roofline": {"bound": w.bound, "achieved": achieved, "peak": peak, "unit": punit, "frac": achieved / peak,
+                     "traffic": _traffic(w.name), "kernel_ms": kernel_ms, "algorithmic_work": w.work},
+    }
+    if with_cpu:
+        res = w.cpu_baseline(oracle, np, torch)
+        if res:
+            rec["cpu_baseline"], rec["parity"] = res
+    return rec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gemm_bf16_8192")
+    ap.add_argument("--only", action="store_true", help="measure only --workload (no 'also' list)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / sampled parity leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (every kernel here is a one-GPU tile kernel; "
+                 "nothing uses a second device) — run with --gpus 1")
+
+    import numpy as np
+    import torch
+
+    import __graft_entry__ as entry
+    import oracle
+
+    ct = entry.load_package()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    workloads = make_workloads()
+    head = next((w for w in workloads if w.name == args.workload), None)
+    if head is None:
+        head = next((c() for c in EXTRA_WORKLOADS if c.name == args.workload), None)
+        args.only = args.only or head is not None
+    if head is None:
+        sys.exit(f"unknown workload {args.workload}; choose from {[w.name for w in workloads]}")
+    order = [head] + ([] if args.only else [w for w in workloads if w is not head])
+    records = []
+    for w in order:
+        w.setup(ct, torch, oracle, dev)
+        with_cpu = not args.no_cpu
+        records.append(measure(w, ct, torch, args.steps, args.warmup, with_cpu, oracle, np))
+        # free device memory before the next workload
+        for k in list(w.__dict__):
+            if hasattr(w.__dict__[k], "is_cuda"):
+                del w.__dict__[k]
+        torch.cuda.empty_cache()
+    h = records[0]
+    line = {
+        "metric": METRIC, "value": h["value"], "unit": h["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": h["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": h["dtype"], "data": "synthetic (seeded host PRNG, same bytes fed to the CPU oracle)",
+        "config": h["config"], "roofline": h["roofline"],
+        "device": ct.device_arch(0),
+    }
+    if "cpu_baseline" in h:
+        line["cpu_baseline"] = h["cpu_baseline"]
+        line["parity"] = h["parity"]
+    if len(records) > 1:
+        line["also"] = records[1:]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

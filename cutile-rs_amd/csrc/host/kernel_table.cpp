@@ -104,9 +104,10 @@ std::vector<KernelEntry> build_table() {
     add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64),
         (uint32_t)(2 * (bm * bk + bk * bn) * 2), bm, bn, bk, 0, dtype, 0, 2);
   };
-  gemm("bf16", 256, 256, 64, 2, 2);
-  gemm("bf16", 256, 256, 64, 2, 4);
+  // first entry of a tile shape = default variant
   gemm("bf16", 256, 256, 64, 4, 2);
+  gemm("bf16", 256, 256, 64, 2, 4);
+  gemm("bf16", 256, 256, 64, 2, 2);
   gemm("bf16", 256, 128, 64, 2, 2);
   gemm("bf16", 128, 256, 64, 2, 2);
   gemm("bf16", 128, 128, 64, 2, 2);
