@@ -1,0 +1,285 @@
+"""CPU tests of the C-ABI library's host side: exported symbols, grid / specialization
+logic against the reference's own unit-test vectors, and the launchers' validation,
+variant selection, grid translation and argument marshalling observed through the
+recording stand-in for the HIP runtime (no kernel runs, nothing is computed)."""
+import ctypes as C
+import os
+import re
+import struct
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(ct):
+    L = ct.lib()
+    declared = set()
+    for h in ("cutile_hip.h", "cutile_hip_testing.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        declared |= set(re.findall(r"\b(cutile_[a-z0-9_]+)\s*\(", text))
+    assert len(declared) > 80
+    missing = [s for s in sorted(declared) if not hasattr(L, s)]
+    assert not missing, missing
+
+
+def test_status_names_and_dtypes(ct):
+    L = ct.lib()
+    assert L.cutile_status_name(0) == b"CUTILE_SUCCESS" and L.cutile_status_name(-4) == b"CUTILE_ERR_KERNEL_LAUNCH"
+    assert L.cutile_status_name(700) == b"DriverError"
+    # names are the strings passed in .generics (cuda-core/src/dtype.rs:189-229)
+    for name, size in [("f32", 4), ("f64", 8), ("f16", 2), ("bf16", 2), ("i32", 4), ("u8", 1), ("f8e4m3fn", 1),
+                       ("f8e8m0fnu", 1), ("bool", 1), ("i64", 8)]:
+        code = L.cutile_dtype_from_name(name.encode())
+        assert code < ct.DTYPE_COUNT and L.cutile_dtype_name(code) == name.encode() and L.cutile_dtype_size(code) == size
+    assert L.cutile_dtype_from_name(b"f128") == ct.DTYPE_COUNT
+
+
+def test_without_a_gpu_compute_entry_points_fail_loudly(ct):
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    y = torch.zeros(8)
+    with pytest.raises(ct.CutileError) as e:
+        ct.saxpy(ct.partition(y, [4]), 2.0, torch.ones(8))
+    assert e.value.status != 0 and "DriverError" in e.value.message or "shared object" in e.value.message
+    assert torch.equal(y, torch.zeros(8))          # nothing was computed on the host
+
+
+# ---- Partition::grid / infer_launch_grid (cutile/src/tensor.rs:447-468, tile_kernel.rs:782-808,934-967) ----
+def test_partition_grid(ct):
+    assert ct.partition(torch.zeros(128, 256), [32, 64]).grid() == (4, 4, 1)       # doc example tensor.rs:440-442
+    assert ct.partition(torch.zeros(1000), [128]).grid() == (8, 1, 1)               # div_ceil
+    assert ct.partition(torch.zeros(4, 5, 6), [1, 2, 4]).grid() == (4, 3, 2)
+    with pytest.raises(ct.CutileError, match="at most rank 3"):
+        ct.partition(torch.zeros(2, 2, 2, 2), [1, 1, 1, 1]).grid()
+
+
+def _infer(ct, explicit, bounds):
+    """bounds: list of (grid tuple, exact?) realised as rank-3 partitions with unit tiles."""
+    parts = []
+    for g, exact in bounds:
+        p = ct.partition(torch.zeros(*g), [1, 1, 1], prefix=not exact).arg()
+        parts.append(p)
+    arr = (C.POINTER(ct.PartitionArg) * max(1, len(parts)))(*[C.pointer(p) for p in parts])
+    eg = (C.c_uint32 * 3)(*explicit)
+    out = (C.c_uint32 * 3)()
+    ct.check(ct.lib().cutile_infer_launch_grid(C.byref(eg), arr, len(parts), C.byref(out)))
+    return tuple(out)
+
+
+def test_infer_launch_grid_truth_table(ct):
+    EX, AM = True, False
+    # tile_kernel.rs:1567-1594
+    with pytest.raises(ct.CutileError, match="partial-coverage"):
+        _infer(ct, (0, 0, 0), [((3, 1, 1), AM)])
+    assert _infer(ct, (0, 0, 0), [((3, 1, 1), EX), ((4, 1, 1), AM)]) == (3, 1, 1)
+    with pytest.raises(ct.CutileError):
+        _infer(ct, (0, 0, 0), [((3, 1, 1), EX), ((2, 1, 1), AM)])
+    assert _infer(ct, (2, 1, 1), [((3, 1, 1), AM)]) == (2, 1, 1)
+    with pytest.raises(ct.CutileError, match="exceeds the partial-coverage"):
+        _infer(ct, (4, 1, 1), [((3, 1, 1), AM)])
+    with pytest.raises(ct.CutileError, match="Launch grid required."):
+        _infer(ct, (0, 0, 0), [])
+    # tile_kernel.rs:1548-1565: per-axis prefix, never total count; exact keeps strict equality
+    for g, ok in [((3, 2, 1), True), ((2, 2, 1), True), ((2, 1, 1), True), ((4, 1, 1), False), ((1, 3, 1), False),
+                  ((6, 1, 1), False)]:
+        if ok:
+            assert _infer(ct, g, [((3, 2, 1), AM)]) == g
+        else:
+            with pytest.raises(ct.CutileError):
+                _infer(ct, g, [((3, 2, 1), AM)])
+    with pytest.raises(ct.CutileError, match="does not match the inferred partition grid"):
+        _infer(ct, (2, 1, 1), [((3, 1, 1), EX), ((3, 1, 1), AM)])
+    assert _infer(ct, (3, 1, 1), [((3, 1, 1), EX), ((4, 1, 1), AM)]) == (3, 1, 1)
+    # tile_kernel.rs:1509-1517: matching / mismatching exact grids
+    assert _infer(ct, (4, 1, 1), [((4, 1, 1), EX)]) == (4, 1, 1)
+    with pytest.raises(ct.CutileError):
+        _infer(ct, (4, 1, 1), [((2, 1, 1), EX)])
+
+
+def _spec(ct, ptr, shape, strides):
+    t = ct.TensorArg()
+    t.ptr, t.rank = ptr, len(shape)
+    for i, (s, st) in enumerate(zip(shape, strides)):
+        t.shape[i], t.strides[i] = s, st
+    sb = ct.SpecBits()
+    ct.check(ct.lib().cutile_compute_spec(C.byref(t), C.byref(sb)))
+    r = len(shape)
+    return list(sb.shape_div)[:r], list(sb.stride_div)[:r], [bool(v) for v in sb.stride_one][:r], sb.base_ptr_div, bool(sb.elements_disjoint)
+
+
+def test_compute_spec_vectors(ct):
+    # cutile-compiler/src/specialization_tests.rs:68-205
+    assert _spec(ct, 0x1000, [1024], [1]) == ([16], [1], [True], 16, True)
+    assert _spec(ct, 0x1000, [128, 256], [256, 1]) == ([16, 16], [16, 1], [False, True], 16, True)
+    assert _spec(ct, 0x1000, [1023], [1])[:3] == ([1], [1], [True])
+    assert _spec(ct, 0x1004, [128], [1])[3] == 4
+    assert _spec(ct, 0x1000, [4, 8], [8, 1])[4] is True
+    assert _spec(ct, 0x1000, [4, 8], [4, 1])[4] is False           # overlapping rows
+    for v, d in [(1, 1), (2, 2), (8, 8), (16, 16), (32, 16), (3, 1), (6, 2), (12, 4), (24, 8), (48, 16), (1023, 1), (0, 16)]:
+        assert _spec(ct, 0x1000, [max(v, 1)], [v])[1] == [d]        # max_pow2_divisor, clamped to 16, 0 -> 16
+
+
+# ---- launchers through the recording runtime ------------------------------------------------
+def _last(fake_hip):
+    n = fake_hip.lib().cutile_testing_launch_count()
+    rec = fake_hip.LaunchRecord()
+    fake_hip.check(fake_hip.lib().cutile_testing_get_launch(n - 1, C.byref(rec)))
+    return rec, bytes(rec.args[:rec.args_size])
+
+
+def test_saxpy_argument_marshalling_and_variant_choice(fake_hip):
+    ct = fake_hip
+    y, x = torch.zeros(4, 8), torch.ones(4, 8)
+    ct.saxpy(ct.partition(y, [2, 2]), 2.0, x)
+    rec, args = _last(ct)
+    assert rec.symbol == b"saxpy_entry__f32_r2_flat" and tuple(rec.block) == (256, 1, 1) and tuple(rec.grid) == (1, 1, 1)
+    # (ptr, shape[2], strides[2], partition_shape[2], partition_strides[2]) a (ptr, shape[2], strides[2]) tile grid
+    # — the push order of cutile/src/tensor.rs:1723-1739, 2005-2016
+    yp, s0, s1, st0, st1, p0, p1, ps0, ps1, a, _pad, xp, xs0, xs1, xst0, xst1, gx, gy, gz, _ = struct.unpack("<Q8ifiQ4i4I", args)
+    assert (yp, xp) == (y.data_ptr(), x.data_ptr()) and (s0, s1, st0, st1) == (4, 8, 8, 1)
+    assert (p0, p1, ps0, ps1) == (2, 2, 8, 1) and a == 2.0 and (xs0, xs1, xst0, xst1) == (4, 8, 8, 1) and (gx, gy, gz) == (2, 4, 1)
+    # a strided view cannot take the flat path; one workgroup per tile
+    big = torch.zeros(4, 16)
+    ct.saxpy(ct.partition(big[:, :8], [2, 2]), 2.0, x)
+    rec, _ = _last(ct)
+    assert rec.symbol == b"saxpy_entry__f32_r2_tiled" and tuple(rec.grid) == (2, 4, 1)
+    # asking for a variant that does not fit the arguments is an error, not a silent switch
+    with pytest.raises(ct.CutileError, match="does not fit"):
+        ct.saxpy(ct.partition(big[:, :8], [2, 2]), 2.0, x, variant="f32_r2_flat")
+
+
+def test_validation_happens_before_any_gpu_work(fake_hip):
+    ct = fake_hip
+    L = ct.lib()
+    L.cutile_testing_clear_log()
+    z = torch.zeros(512, 512, dtype=torch.bfloat16)
+    a, b = torch.zeros(512, 256, dtype=torch.bfloat16), torch.zeros(256, 512, dtype=torch.bfloat16)
+    cases = [
+        (lambda: ct.gemm(ct.partition(z, [256, 256]), a, b, 256, grid=(1, 1, 1)), "does not match the inferred partition grid"),
+        (lambda: ct.gemm(ct.partition(z, [256, 256], prefix=True), a, b, 256), "partial-coverage"),
+        (lambda: ct.gemm(ct.partition(z, [100, 100]), a, b, 256), "no precompiled variant of gemm<bf16, 100, 100, 64>"),
+        (lambda: ct.gemm(ct.partition(z, [256, 256]), a, b, 256, generics=["bf16", 128, 256, 64]), "generic BM"),
+        (lambda: ct.gemm(ct.partition(z, [256, 256]), a.float(), b, 256), "bf16 x and y"),
+        (lambda: ct.rms_norm_f16(torch.zeros(4, 64, dtype=torch.half), torch.zeros(32, dtype=torch.half),
+                                 ct.partition(torch.zeros(4, 64, dtype=torch.half), [1, 64]), 1e-6), "expected N = 64"),
+        (lambda: ct.rms_norm_f16(torch.zeros(4, 64, dtype=torch.half), torch.zeros(64, dtype=torch.half),
+                                 ct.partition(torch.zeros(4, 64, dtype=torch.half), [2, 64]), 1e-6), r"partitioned \[1, 64\]"),
+        (lambda: ct.softmax(torch.zeros(4, 64), ct.partition(torch.zeros(4, 64, dtype=torch.half), [1, 64])), "both be f16 or both f32"),
+        (lambda: ct.fmha(ct.partition(torch.zeros(4, 64, 32, dtype=torch.bfloat16), [1, 32, 32]),
+                         *(torch.zeros(1, 4, 64, 32, dtype=torch.bfloat16) for _ in range(3)), 0.1, 0, 3), "do not agree"),
+        (lambda: ct.saxpy(ct.partition(torch.zeros(8), [4]), 1.0, torch.zeros(8, dtype=torch.float64)), "element type f32"),
+    ]
+    for fn, msg in cases:
+        with pytest.raises(ct.CutileError, match=msg):
+            fn()
+    assert L.cutile_testing_launch_count() == 0
+
+
+def test_grid_translation_per_kernel_family(fake_hip):
+    ct = fake_hip
+    h = torch.half
+    # row-wise: four single-wave rows per workgroup for N <= 8192 in registers
+    x, w, o = torch.zeros(100, 1024, dtype=h), torch.zeros(1024, dtype=h), torch.zeros(100, 1024, dtype=h)
+    ct.rms_norm_f16(x, w, ct.partition(o, [1, 1024]), 1e-6, generics=[1024, 512])
+    rec, _ = _last(ct)
+    assert rec.symbol == b"rms_norm_f16_entry__w1v2" and tuple(rec.grid) == (25, 1, 1)
+    ct.rms_norm_f16(x, w, ct.partition(o, [1, 1024]), 1e-6, variant="w4v4")
+    assert tuple(_last(ct)[0].grid) == (100, 1, 1)
+    # N = 1001 is not a whole number of 16-byte vectors: the any-shape kernel takes it
+    x1, w1, o1 = torch.zeros(8, 1001, dtype=h), torch.zeros(1001, dtype=h), torch.zeros(8, 1001, dtype=h)
+    ct.rms_norm_f16(x1, w1, ct.partition(o1, [1, 1001]), 1e-6)
+    assert _last(ct)[0].symbol == b"rms_norm_f16_entry__generic"
+    # chunk softmax: 16 rows x 4 column tiles = 64 segments of 2048
+    xs, ys = torch.zeros(16, 8192, dtype=h), torch.zeros(16, 8192, dtype=h)
+    ct.softmax(xs, ct.partition(ys, [1, 2048]))
+    rec, _ = _last(ct)
+    assert rec.symbol == b"softmax_entry__f16_w1v4" and tuple(rec.grid) == (16, 1, 1)
+    # GEMM: one workgroup per output tile on a 1-D grid (the kernel remaps ids per XCD)
+    z = torch.zeros(1000, 520, dtype=torch.bfloat16)
+    a, b = torch.zeros(1000, 256, dtype=torch.bfloat16), torch.zeros(256, 520, dtype=torch.bfloat16)
+    ct.gemm(ct.partition(z, [128, 128]), a, b, 256)
+    rec, args = _last(ct)
+    assert rec.symbol == b"gemm_entry__bf16_128x128x64_w2x2" and tuple(rec.grid) == (8 * 5, 1, 1) and tuple(rec.block) == (256, 1, 1)
+    k_total, gx, gy, gz, _, acc = struct.unpack_from("<i4Ii", args, 88)
+    assert (k_total, gx, gy, gz, acc) == (256, 8, 5, 1, 1)
+    # FMHA: (batch*heads, query tiles)
+    q = torch.zeros(2, 4, 512, 128, dtype=torch.bfloat16)
+    out = torch.zeros(8, 512, 128, dtype=torch.bfloat16)
+    ct.fmha(ct.partition(out, [1, 128, 128]), q, q, q, 0.088, 0, 1, causal=True, generics=[128, 64, 128, 4, 1, 1])
+    rec, _ = _last(ct)
+    assert rec.symbol == b"fmha_entry__bf16_128x64x128" and tuple(rec.grid) == (8, 4, 1) and tuple(rec.block) == (256, 1, 1)
+    # MXFP8: the reference example's 16x16 tiles are covered by one 32x32 kernel tile
+    u8 = torch.uint8
+    ct.linear_tile_mxfp8(ct.partition(torch.zeros(16, 16), [16, 16]), torch.zeros(16, 128, dtype=u8), torch.zeros(16, 128, dtype=u8),
+                         torch.zeros(16, 4, dtype=u8), torch.zeros(16, 4, dtype=u8), 1.0, generics=[16, 16, 64, 2])
+    rec, _ = _last(ct)
+    assert rec.symbol == b"linear_tile_entry__mxfp8_f32_32x32x128_w1x1" and tuple(rec.grid) == (1, 1, 1)
+
+
+def test_kernel_table_lookup_and_single_flight_module_load(fake_hip):
+    ct = fake_hip
+    L = ct.lib()
+    before = L.cutile_module_load_count()
+    info = ct.kernel_lookup("gemm", ["bf16", "256", "256", "64"])
+    assert info.symbol.startswith(b"gemm_entry__bf16_256x256x64") and tuple(info.tile)[:3] == (256, 256, 64)
+    info2 = ct.kernel_lookup("gemm", ["bf16", "128", "128", "64"])
+    assert info2.symbol == b"gemm_entry__bf16_128x128x64_w2x2" and tuple(info2.block) == (256, 1, 1)
+    assert L.cutile_module_load_count() == before + 1          # one code object per kernel family per device
+    with pytest.raises(ct.CutileError, match="available: "):
+        ct.kernel_lookup("gemm", ["bf16", "48", "48", "16"])
+    with pytest.raises(ct.CutileError):
+        ct.kernel_lookup("no_such_kernel")
+    names = ct.kernel_list()
+    assert "saxpy:f32_r1_flat" in names and "fmha:bf16_256x64x128" in names and len(set(names)) == len(names)
+    # pinned preference (autotuner output) is honoured and validated
+    ct.set_preferred_variant("gemm", "bf16_256x256x64_w2x2")
+    z = torch.zeros(256, 256, dtype=torch.bfloat16)
+    ct.gemm(ct.partition(z, [256, 256]), z, z, 256)
+    assert _last(ct)[0].symbol == b"gemm_entry__bf16_256x256x64_w2x2"
+    ct.set_preferred_variant("gemm", None)
+    with pytest.raises(ct.CutileError):
+        ct.set_preferred_variant("gemm", "nope")
+
+
+def test_driver_layer_on_the_recording_runtime(fake_hip):
+    ct = fake_hip
+    L = ct.lib()
+    n = C.c_int32()
+    ct.check(L.cutile_device_count(C.byref(n)))
+    assert n.value == 1
+    dev = ct.device(0)
+    assert ct.device(0) == dev                                  # one handle per ordinal
+    with pytest.raises(ct.CutileError, match="DriverError"):
+        ct.device(3)                                            # cuda-async/tests/error_handling.rs:174-190
+    assert "gfx950" in ct.device_arch(0) and ct.device_props(0).wavefront_size == 64
+    # streams are pooled: a released stream is handed out again, never destroyed
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    created = L.cutile_testing_streams_created()
+    ct.check(L.cutile_stream_create(dev, C.byref(s1)))
+    ct.check(L.cutile_stream_release(dev, s1))
+    ct.check(L.cutile_stream_create(dev, C.byref(s2)))
+    assert s1.value == s2.value and L.cutile_testing_streams_created() == created + 1
+    # async alloc / copies / memset round trip
+    p = C.c_void_p()
+    ct.check(L.cutile_malloc_async(64, s2, C.byref(p)))
+    src = (C.c_ubyte * 64)(*range(64))
+    dst = (C.c_ubyte * 64)()
+    ct.check(L.cutile_memcpy_htod_async(p, src, 64, s2))
+    ct.check(L.cutile_memcpy_dtoh_async(dst, p, 64, s2))
+    ct.check(L.cutile_stream_synchronize(s2))
+    assert bytes(dst) == bytes(range(64))
+    ct.check(L.cutile_memset_d8_async(p, 7, 64, s2))
+    ct.check(L.cutile_memcpy_dtoh_async(dst, p, 64, s2))
+    assert bytes(dst) == bytes([7] * 64)
+    ct.check(L.cutile_free_async(p, s2))
+    # a module image that is not ELF is rejected before the driver sees it (runtime.rs:309-328)
+    mod = C.c_void_p()
+    L.cutile_module_load_data.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+    assert L.cutile_module_load_data(dev, b"not an elf image", 16, C.byref(mod)) == -2
+    # driver failures surface as DriverError(code) with the runtime's text
+    ct.check(L.cutile_testing_inject_failure(b"hipMallocAsync", 2, 1))
+    st = L.cutile_malloc_async(64, s2, C.byref(p))
+    assert st == 2 and b"DriverError(2)" in L.cutile_last_error_message()
