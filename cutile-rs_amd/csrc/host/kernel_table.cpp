@@ -98,13 +98,16 @@ std::vector<KernelEntry> build_table() {
   add("softmax", "f32_generic", "softmax_entry__f32_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
 
   // ---- bf16 GEMM: LDS = 2 stages x (BM*BK + BK*BN) x 2 bytes ----
-  auto gemm = [&](const char* dtype, int bm, int bn, int bk, int wvm, int wvn) {
+  auto gemm = [&](const char* dtype, int bm, int bn, int bk, int wvm, int wvn, const char* kind = "w") {
     std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" +
-                    std::to_string(bk) + "_w" + std::to_string(wvm) + "x" + std::to_string(wvn);
+                    std::to_string(bk) + "_" + kind + std::to_string(wvm) + "x" + std::to_string(wvn);
     add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64),
         (uint32_t)(2 * (bm * bk + bk * bn) * 2), bm, bn, bk, 0, dtype, 0, 2);
   };
-  // first entry of a tile shape = default variant
+  // first entry of a tile shape = default variant; "d" = global->LDS direct, pipelined
+  gemm("bf16", 256, 256, 64, 2, 4, "d");
+  gemm("bf16", 256, 256, 64, 4, 2, "d");
+  gemm("bf16", 128, 128, 64, 2, 2, "d");
   gemm("bf16", 256, 256, 64, 4, 2);
   gemm("bf16", 256, 256, 64, 2, 4);
   gemm("bf16", 256, 256, 64, 2, 2);

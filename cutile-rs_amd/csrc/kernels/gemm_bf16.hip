@@ -258,6 +258,227 @@ struct Gemm {
   }
 };
 
+
+// ---- pipelined variant: global -> LDS without passing through registers ------------------
+// Differences from Gemm above:
+//  * tiles are fetched with buffer loads that write straight into LDS (16 bytes
+//    per lane, 1 KiB per wavefront instruction).  The XOR swizzle is applied by
+//    choosing WHICH global unit a lane fetches, because the LDS side of such a
+//    load is always lane-contiguous;
+//  * two LDS stages, and the hand-over point sits before the LAST MFMA block of
+//    a K tile: by then every wavefront holds that tile's last operands in
+//    registers, so after one barrier the stage can be refilled with tile kt+2
+//    while the first operands of tile kt+1 are read under the remaining MFMAs.
+//    A tile's loads are thus in flight for a whole K tile, and neither the
+//    barrier nor LDS latency is exposed;
+//  * operands are read one MFMA block ahead (register double buffering);
+//  * the K advance of the global addresses rides in the scalar offset of the
+//    buffer instruction: no per-iteration address arithmetic in vector registers.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+struct GemmDirect {
+  static constexpr int BK = 64;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int UB = BN / 8;                         // 16-byte units per y-tile row
+  static constexpr int kAInstr = BM / 8 / kWaves;           // 1 KiB = 8 x-tile rows
+  static constexpr int kBRowsPerInstr = 64 / UB;
+  static constexpr int kBInstr = BK / kBRowsPerInstr / kWaves;
+  static constexpr int kABytes = BM * BK * 2, kBBytes = BK * BN * 2;
+  static constexpr int kStageBytes = kABytes + kBBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static_assert(BM % (8 * kWaves) == 0 && BK % (kBRowsPerInstr * kWaves) == 0, "tile must split evenly");
+  static_assert(UB >= 16 && UB <= 64, "y-tile row must be 16..64 units");
+
+  __device__ static __forceinline__ int a_lds_off(int r, int u) { return r * (BK * 2) + ((u ^ ((r >> 1) & 7)) << 4); }
+  __device__ static __forceinline__ int b_lds_off(int r, int u) { return r * (BN * 2) + ((u ^ ((r & 3) << 2)) << 4); }
+
+  struct Frags {
+    bf16x8 a[TM], b[TN];
+  };
+
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                             int32_t k_total, const TileGrid& g, int32_t accumulate) {
+    // Two separately named stages so that the compiler can tell a refill of one
+    // from operand reads of the other.
+    __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStageBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    const int32_t M = x.shape[0], N = y.shape[1];
+    const int32_t lda = x.strides[0], ldb = y.strides[0];
+    const int32_t row0 = pm * BM, col0 = pn * BN;
+    const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)(((int64_t)(M - 1) * lda + x.shape[1]) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)(((int64_t)(y.shape[0] - 1) * ldb + N) * 2));
+    constexpr uint32_t kOob = 0x80000000u;
+
+    // Global side of the tile fetches (per lane, K tile 0; the K advance is scalar).
+    uint32_t a_goff[kAInstr], b_goff[kBInstr];
+    int32_t a_k[kAInstr], b_k[kBInstr];  // K index (within a tile) this lane fetches: for the K tail
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_k[i] = u * 8;
+      a_goff[i] = (row0 + r < M) ? (uint32_t)(((int64_t)(row0 + r) * lda + u * 8) * 2) : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < kBInstr; ++i) {
+      const int r = (wave * kBInstr + i) * kBRowsPerInstr + lane / UB;
+      const int u = (lane % UB) ^ ((r & 3) << 2);
+      b_k[i] = r;
+      b_goff[i] = (col0 + u * 8 < N) ? (uint32_t)(((int64_t)r * ldb + col0 + u * 8) * 2) : kOob;
+    }
+    auto fetch_tile = [&](unsigned char* stage, int32_t k0) {
+      if (k0 + BK > k_valid) {  // uniform; only the last tile can be short: lanes beyond K fetch zeros
+#pragma unroll
+        for (int i = 0; i < kAInstr; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                                   k0 + a_k[i] >= k_valid ? kOob : a_goff[i], k0 * 2, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kBInstr; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(stage + kABytes + (wave * kBInstr + i) * 1024),
+                                                   16, k0 + b_k[i] >= k_valid ? kOob : b_goff[i], k0 * ldb * 2, 0, 0);
+      } else {
+#pragma unroll
+        for (int i = 0; i < kAInstr; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                                   a_goff[i], k0 * 2, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kBInstr; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(stage + kABytes + (wave * kBInstr + i) * 1024),
+                                                   16, b_goff[i], k0 * ldb * 2, 0, 0);
+      }
+    };
+
+    // LDS side of the operand reads (byte offsets inside a stage).
+    const int l32 = lane & 31, khalf = lane >> 5;
+    const int grp = lane >> 4, l16 = lane & 15;
+    const int tr_row = l16 >> 2, tr_col = (l16 & 3) * 4;
+    int a_addr[TM][4], b_addr[TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) a_addr[tm][ks] = a_lds_off(wm * WM + tm * 32 + l32, ks * 2 + khalf);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int n = wn * WN + tn * 32 + (grp & 1) * 16 + tr_col;
+      const int kr = (grp >> 1) * 8 + tr_row;  // (kr & 3) does not depend on ks: the swizzle term is fixed
+      b_addr[tn] = kABytes + b_lds_off(kr, n >> 3) + (n & 7) * 2;
+    }
+    auto read_frags = [&](const unsigned char* stage, int ks, Frags& f) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) f.a[tm] = *reinterpret_cast<const bf16x8*>(stage + a_addr[tm][ks]);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const unsigned char* p = stage + b_addr[tn] + ks * 16 * (BN * 2);
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 4 * (BN * 2)));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        f.b[tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
+    auto mfma_block = [&](const Frags& f) {
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[tn], f.a[tm], acc[tn][tm], 0, 0, 0);
+    };
+
+    const int k_tiles = (k_total + BK - 1) / BK;
+    Frags f0, f1;
+    if (k_tiles > 0) {
+      fetch_tile(stage0, 0);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (k_tiles > 1) fetch_tile(stage1, BK);
+      read_frags(stage0, 0, f0);
+    }
+    // One K tile: `cur` is being multiplied, `nxt` holds (or is receiving) tile kt+1.
+    // sched_barrier(0) pins the order "issue the next operand reads, then the MFMA
+    // block": a wavefront issues in order and each MFMA holds the issue slot until
+    // the matrix pipe accepts it, so reads placed after a block would start late.
+    auto k_tile = [&](unsigned char* cur, unsigned char* nxt, int kt) {
+      read_frags(cur, 1, f1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(f0);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(cur, 2, f0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(f1);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(cur, 3, f1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(f0);
+      __builtin_amdgcn_sched_barrier(0);
+      // Hand-over: this wavefront holds all it needs of `cur`, and its part of
+      // tile kt+1 has landed in `nxt`.
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (kt + 2 < k_tiles) fetch_tile(cur, (kt + 2) * BK);
+      if (kt + 1 < k_tiles) read_frags(nxt, 0, f0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(f1);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int kt = 0; kt < k_tiles; kt += 2) {
+      k_tile(stage0, stage1, kt);
+      if (kt + 1 < k_tiles) k_tile(stage1, stage0, kt + 1);
+    }
+
+    OutT* zp = (OutT*)z.ptr;
+    const int32_t ldz = z.strides[0];
+    const int32_t zM = z.shape[0], zN = z.shape[1];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const int32_t r = row0 + wm * WM + tm * 32 + l32;
+      if (r >= zM) continue;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int32_t c = col0 + wn * WN + tn * 32 + q * 8 + khalf * 4;
+          if (c >= zN) continue;
+          OutT* dst = zp + (int64_t)r * ldz + c;
+          float v0 = acc[tn][tm][q * 4 + 0], v1 = acc[tn][tm][q * 4 + 1];
+          float v2 = acc[tn][tm][q * 4 + 2], v3 = acc[tn][tm][q * 4 + 3];
+          if constexpr (sizeof(OutT) == 2) {
+            if (accumulate) {
+              u32x2 old = *reinterpret_cast<const u32x2*>(dst);
+              v0 += __builtin_bit_cast(float, old.x << 16);
+              v1 += __builtin_bit_cast(float, old.x & 0xffff0000u);
+              v2 += __builtin_bit_cast(float, old.y << 16);
+              v3 += __builtin_bit_cast(float, old.y & 0xffff0000u);
+            }
+            u32x2 o;
+            o.x = pack_bf16x2(v0, v1);
+            o.y = pack_bf16x2(v2, v3);
+            *reinterpret_cast<u32x2*>(dst) = o;
+          } else {
+            f32x4 o = {v0, v1, v2, v3};
+            if (accumulate) o += *reinterpret_cast<const f32x4*>(dst);
+            *reinterpret_cast<f32x4*>(dst) = o;
+          }
+        }
+      }
+    }
+  }
+};
+
 }  // namespace
 
 // gemm<bf16, BM, BN, BK>(z, x, y, k) with trailing launch metadata.
@@ -277,3 +498,14 @@ GEMM_KERNEL(bf16_128x128x64_w2x2, 128, 128, 64, 2, 2, __bf16)
 GEMM_KERNEL(bf16_64x128x64_w2x2, 64, 128, 64, 2, 2, __bf16)
 GEMM_KERNEL(bf16f32_128x128x64_w2x2, 128, 128, 64, 2, 2, float)
 GEMM_KERNEL(bf16f32_256x256x64_w2x2, 256, 256, 64, 2, 2, float)
+
+#define GEMM_DIRECT_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                        \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmDirect<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, k, g, accumulate);                        \
+  }
+
+GEMM_DIRECT_KERNEL(bf16_256x256x64_d4x2, 256, 256, 4, 2, __bf16)
+GEMM_DIRECT_KERNEL(bf16_256x256x64_d2x4, 256, 256, 2, 4, __bf16)
+GEMM_DIRECT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)

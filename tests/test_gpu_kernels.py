@@ -204,7 +204,7 @@ def test_softmax_f32(ct, dev, m, n, bm, bn):
 
 
 # ---- K4: bf16 GEMM --------------------------------------------------------------------------
-GEMM_VARIANTS = ["bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
+GEMM_VARIANTS = ["bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
                  "bf16_128x256x64_w2x2", "bf16_128x128x64_w2x2", "bf16_64x128x64_w2x2"]
 
 

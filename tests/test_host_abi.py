@@ -202,7 +202,7 @@ def test_grid_translation_per_kernel_family(fake_hip):
     a, b = torch.zeros(1000, 256, dtype=torch.bfloat16), torch.zeros(256, 520, dtype=torch.bfloat16)
     ct.gemm(ct.partition(z, [128, 128]), a, b, 256)
     rec, args = _last(ct)
-    assert rec.symbol == b"gemm_entry__bf16_128x128x64_w2x2" and tuple(rec.grid) == (8 * 5, 1, 1) and tuple(rec.block) == (256, 1, 1)
+    assert rec.symbol == b"gemm_entry__bf16_128x128x64_d2x2" and tuple(rec.grid) == (8 * 5, 1, 1) and tuple(rec.block) == (256, 1, 1)
     k_total, gx, gy, gz, _, acc = struct.unpack_from("<i4Ii", args, 88)
     assert (k_total, gx, gy, gz, acc) == (256, 8, 5, 1, 1)
     # FMHA: (batch*heads, query tiles)
@@ -226,7 +226,7 @@ def test_kernel_table_lookup_and_single_flight_module_load(fake_hip):
     info = ct.kernel_lookup("gemm", ["bf16", "256", "256", "64"])
     assert info.symbol.startswith(b"gemm_entry__bf16_256x256x64") and tuple(info.tile)[:3] == (256, 256, 64)
     info2 = ct.kernel_lookup("gemm", ["bf16", "128", "128", "64"])
-    assert info2.symbol == b"gemm_entry__bf16_128x128x64_w2x2" and tuple(info2.block) == (256, 1, 1)
+    assert info2.symbol == b"gemm_entry__bf16_128x128x64_d2x2" and tuple(info2.block) == (256, 1, 1)
     assert L.cutile_module_load_count() == before + 1          # one code object per kernel family per device
     with pytest.raises(ct.CutileError, match="available: "):
         ct.kernel_lookup("gemm", ["bf16", "48", "48", "16"])
