@@ -32,7 +32,7 @@ IMAGES = {
     "fmha": "fmha.hip",
     "mxgemm": "mxfp8_gemm.hip",
 }
-HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "fake_hip.cpp"]
+HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")
@@ -105,8 +105,44 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
     return LIB_PATH
 
 
+CPP_TEST_DIR = os.path.join(ROOT, "..", "tests", "cpp")
+CPP_TESTS = {
+    # binary -> (source, needs the library, extra flags)
+    "test_host_surface": ("test_host_surface.cpp", True, []),
+    "test_gpu_surface": ("test_gpu_surface.cpp", True, []),
+    "test_slot_table": ("test_slot_table.cpp", False, []),
+    "test_slot_table_tsan": ("test_slot_table.cpp", False, ["-fsanitize=thread"]),
+}
+
+
+def build_cpp_tests(force: bool = False) -> str:
+    """Compiles the C++ host-surface test programs (run by tests/test_cpp_surface.py)."""
+    out_dir = os.path.join(CPP_TEST_DIR, "bin")
+    os.makedirs(out_dir, exist_ok=True)
+    include = os.path.join(ROOT, "..", "include")
+    headers = [os.path.join(include, "cutile", f) for f in os.listdir(os.path.join(include, "cutile"))]
+    headers += [os.path.join(include, f) for f in os.listdir(include) if f.endswith(".h")]
+    headers += [os.path.join(CPP_TEST_DIR, "check.hpp"), os.path.join(HOST_DIR, "slot_table.h")]
+    jobs = []
+    for name, (src, needs_lib, extra) in CPP_TESTS.items():
+        dst = os.path.join(out_dir, name)
+        src_path = os.path.join(CPP_TEST_DIR, src)
+        deps = [src_path] + headers + ([LIB_PATH] if needs_lib else [])
+        if force or not _newer(dst, deps):
+            cmd = [CXX, "-std=c++17", "-O1", "-g0", "-I" + include, "-Wall", "-Wextra", "-Wno-unused-parameter"] + extra
+            cmd += [src_path, "-o", dst, "-pthread"]
+            if needs_lib:
+                cmd += ["-L" + LIB_DIR, "-lcutile_hip", "-Wl,-rpath,$ORIGIN/../../../cutile-rs_amd/lib"]
+            jobs.append(cmd)
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        list(ex.map(_run, jobs))
+    return out_dir
+
+
 def build(force: bool = False) -> str:
-    return build_host_library(build_code_objects(force), force)
+    lib = build_host_library(build_code_objects(force), force)
+    build_cpp_tests(force)
+    return lib
 
 
 if __name__ == "__main__":

@@ -38,6 +38,7 @@ cutile_status_t ensure_init() {
 }
 
 void reset_runtime_for_testing() {
+  reset_async_runtime_for_testing();
   std::lock_guard<std::mutex> lock(g_devices_mutex);
   g_devices.clear();
 }

@@ -32,6 +32,7 @@ namespace cutile {
 cutile_status_t ensure_init();
 void count_module_load();
 void reset_runtime_for_testing();
+void reset_async_runtime_for_testing();
 // Device the calling thread is bound to (hipGetDevice), as a handle.
 cutile_status_t current_device(cutile_device_t* device);
 

@@ -1,0 +1,400 @@
+// api::* — lazy tensor constructors and transfers, and the kernel launchers of
+// the hot path.
+//
+// Constructors mirror cutile/src/api.rs:215-735 (zeros/ones/full :483-528,
+// arange :552-559, copy_host_vec_to_device / to_host_vec / dup / memcpy
+// :215-460, convert :654-666, randn :683-719, meta :450-462).  Everything is a
+// DeviceOp: nothing is allocated or launched until the op executes.
+//
+// Launchers mirror the macro-generated unified launcher of each entry kernel
+// (cutile-macro/src/kernel_launcher_generator.rs:1056-1202): arguments may be
+// plain values or DeviceOps, the builder methods .generics() / .grid() are kept,
+// and the output is the tuple of the arguments, in signature order, in the
+// ownership form they were given.
+#pragma once
+#include <array>
+#include <cmath>
+#include <string>
+
+#include "tensor.hpp"
+
+namespace cutile {
+namespace api {
+
+// ---- allocation ----------------------------------------------------------------------------
+template <class T>
+class Uninitialized : public DeviceOp<Uninitialized<T>, Tensor<T>> {
+ public:
+  explicit Uninitialized(std::vector<int32_t> shape) : shape_(std::move(shape)) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    auto n = checked_num_elements(shape_);
+    if (!n) return DeviceError::tensor("Tensor shape contains invalid dimensions or overflows.");
+    auto p = ctx.alloc_async(*n * sizeof(T));  // tensor.rs:1016-1030
+    if (p.is_err()) return p.error();
+    auto strides = contiguous_strides(shape_);
+    return Tensor<T>::from_raw_parts(p.value(), *n * sizeof(T), ctx.device_id(), std::move(shape_), std::move(strides));
+  }
+
+ private:
+  std::vector<int32_t> shape_;
+};
+
+inline cutile_partition_arg_t flat_partition(const cutile_tensor_arg_t& t, size_t n, int32_t tile) {
+  cutile_partition_arg_t p{};
+  p.tensor = t;
+  p.tensor.rank = 1;
+  p.tensor.shape[0] = (int32_t)n;
+  p.tensor.strides[0] = 1;
+  p.partition_shape[0] = tile;
+  p.partition_strides[0] = 1;
+  return p;
+}
+
+// full: allocate, then launch the library kernel creation::full over tiles of 128
+// (api.rs:518-528; kernel cutile/src/kernels/_creation.rs:44-47).
+template <class T>
+class Full : public DeviceOp<Full<T>, Tensor<T>> {
+ public:
+  Full(double v, int64_t iv, std::vector<int32_t> shape) : v_(v), iv_(iv), shape_(std::move(shape)) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<T>(std::move(shape_)).execute(ctx);
+    if (t.is_err()) return t.error();
+    if (t.value().size() == 0) return t;
+    cutile_partition_arg_t p = flat_partition(t.value().arg(), t.value().size(), 128);
+    CUTILE_TRY_STATUS(cutile_launch_full(ctx.stream()->raw(), v_, iv_, &p, nullptr));
+    return t;
+  }
+
+ private:
+  double v_;
+  int64_t iv_;
+  std::vector<int32_t> shape_;
+};
+template <class T> Full<T> full(double value, std::vector<int32_t> shape) { return Full<T>(value, (int64_t)value, std::move(shape)); }
+template <class T> Full<T> zeros(std::vector<int32_t> shape) { return Full<T>(0.0, 0, std::move(shape)); }
+template <class T> Full<T> ones(std::vector<int32_t> shape) { return Full<T>(1.0, 1, std::move(shape)); }
+
+template <class T>
+class Arange : public DeviceOp<Arange<T>, Tensor<T>> {
+ public:
+  explicit Arange(size_t n) : n_(n) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<T>({(int32_t)n_}).execute(ctx);
+    if (t.is_err()) return t.error();
+    cutile_partition_arg_t p = flat_partition(t.value().arg(), n_, 128);
+    CUTILE_TRY_STATUS(cutile_launch_arange(ctx.stream()->raw(), &p, nullptr));
+    return t;
+  }
+
+ private:
+  size_t n_;
+};
+template <class T> Arange<T> arange(size_t n) { return Arange<T>(n); }
+
+class Linspace : public DeviceOp<Linspace, Tensor<float>> {
+ public:
+  Linspace(float start, float stop, size_t n) : start_(start), stop_(stop), n_(n) {}
+  Result<Tensor<float>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<float>({(int32_t)n_}).execute(ctx);
+    if (t.is_err()) return t.error();
+    float step = n_ > 1 ? (stop_ - start_) / (float)(n_ - 1) : 0.0f;
+    cutile_partition_arg_t p = flat_partition(t.value().arg(), n_, 128);
+    CUTILE_TRY_STATUS(cutile_launch_linspace(ctx.stream()->raw(), &p, start_, step, nullptr));
+    return t;
+  }
+
+ private:
+  float start_, stop_;
+  size_t n_;
+};
+inline Linspace linspace(float start, float stop, size_t n) { return Linspace(start, stop, n); }
+
+// meta: shape/stride metadata without memory (api.rs:450-462).
+template <class T> Value<Tensor<T>> meta(std::vector<int32_t> shape) { return value(Tensor<T>::from_meta(std::move(shape))); }
+
+// ---- transfers -----------------------------------------------------------------------------
+template <class T>
+class CopyHostVecToDevice : public DeviceOp<CopyHostVecToDevice<T>, Tensor<T>> {
+ public:
+  explicit CopyHostVecToDevice(std::shared_ptr<std::vector<T>> host) : host_(std::move(host)) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<T>({(int32_t)host_->size()}).execute(ctx);
+    if (t.is_err()) return t.error();
+    CUTILE_TRY_STATUS(cutile_memcpy_htod_async(t.value().device_pointer(), host_->data(), host_->size() * sizeof(T), ctx.stream()->raw()));
+    return t;
+  }
+
+ private:
+  std::shared_ptr<std::vector<T>> host_;  // must stay alive until the stream is synchronised
+};
+template <class T>
+CopyHostVecToDevice<T> copy_host_vec_to_device(std::shared_ptr<std::vector<T>> host) { return CopyHostVecToDevice<T>(std::move(host)); }
+
+// to_host_vec: the vector is valid once the stream has been synchronised.
+template <class Src>
+class ToHostVec : public DeviceOp<ToHostVec<Src>, std::vector<typename std::decay_t<decltype(*std::declval<Src>())>::Elem>> {
+ public:
+  using T = typename std::decay_t<decltype(*std::declval<Src>())>::Elem;
+  explicit ToHostVec(Src src) : src_(std::move(src)) {}
+  Result<std::vector<T>> execute(const ExecutionContext& ctx) && {
+    const Tensor<T>& t = *src_;
+    if (!t.is_contiguous()) return DeviceError::tensor("to_host_vec: tensor must be contiguous");
+    std::vector<T> out(t.size());
+    CUTILE_TRY_STATUS(cutile_memcpy_dtoh_async(out.data(), t.device_pointer(), t.num_bytes(), ctx.stream()->raw()));
+    return out;
+  }
+
+ private:
+  Src src_;  // shared_ptr<Tensor<T>> or const Tensor<T>*
+};
+template <class T> ToHostVec<std::shared_ptr<Tensor<T>>> to_host_vec(std::shared_ptr<Tensor<T>> t) { return ToHostVec<std::shared_ptr<Tensor<T>>>(std::move(t)); }
+template <class T> ToHostVec<const Tensor<T>*> to_host_vec(const Tensor<T>& t) { return ToHostVec<const Tensor<T>*>(&t); }
+// device_op.to_host_vec(): copy the tensor an op produces.
+template <class Op>
+auto to_host_vec_op(Op op) {
+  using T = typename Op::Output::Elem;
+  return std::move(op).then([](Tensor<T> t) { return to_host_vec(std::make_shared<Tensor<T>>(std::move(t))); });
+}
+
+template <class T>
+class Dup : public DeviceOp<Dup<T>, Tensor<T>> {
+ public:
+  explicit Dup(const Tensor<T>* src) : src_(src) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    if (!src_->is_contiguous()) return DeviceError::tensor("dup: tensor must be contiguous");
+    auto t = Uninitialized<T>(src_->shape()).execute(ctx);
+    if (t.is_err()) return t.error();
+    CUTILE_TRY_STATUS(cutile_memcpy_dtod_async(t.value().device_pointer(), src_->device_pointer(), src_->num_bytes(), ctx.stream()->raw()));
+    return t;
+  }
+
+ private:
+  const Tensor<T>* src_;
+};
+template <class T> Dup<T> dup(const Tensor<T>& t) { return Dup<T>(&t); }
+
+// memcpy: device-to-device into an existing tensor; sizes must agree; a graph node (api.rs:298).
+template <class T>
+class Memcpy : public DeviceOp<Memcpy<T>, Unit> {
+ public:
+  Memcpy(Tensor<T>* dst, const Tensor<T>* src) : dst_(dst), src_(src) {
+    if (dst->size() != src->size()) throw std::logic_error("memcpy: source and destination must have the same number of elements");
+  }
+  Result<Unit> execute(const ExecutionContext& ctx) && {
+    return check(cutile_memcpy_dtod_async(dst_->device_pointer(), src_->device_pointer(), src_->num_bytes(), ctx.stream()->raw()));
+  }
+
+ private:
+  Tensor<T>* dst_;
+  const Tensor<T>* src_;
+};
+template <class T> Memcpy<T> memcpy(Tensor<T>& dst, const Tensor<T>& src) { return Memcpy<T>(&dst, &src); }
+
+// convert<From, To>: new tensor of another element type (api.rs:654-666).
+template <class To, class From>
+class Convert : public DeviceOp<Convert<To, From>, Tensor<To>> {
+ public:
+  explicit Convert(std::shared_ptr<Tensor<From>> src) : src_(std::move(src)) {}
+  Result<Tensor<To>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<To>({(int32_t)src_->size()}).execute(ctx);
+    if (t.is_err()) return t.error();
+    cutile_tensor_arg_t s = src_->arg();
+    s.rank = 1; s.shape[0] = (int32_t)src_->size(); s.strides[0] = 1;
+    cutile_partition_arg_t d = flat_partition(t.value().arg(), src_->size(), 128);
+    CUTILE_TRY_STATUS(cutile_launch_convert(ctx.stream()->raw(), &s, &d, nullptr));
+    return std::move(t).unwrap().reshape(src_->shape());
+  }
+
+ private:
+  std::shared_ptr<Tensor<From>> src_;
+};
+template <class To, class From> Convert<To, From> convert(std::shared_ptr<Tensor<From>> src) { return Convert<To, From>(std::move(src)); }
+
+// randn / rand: seeded host generator (SplitMix64 counter stream + Box–Muller),
+// copied to the device.  The reference draws from cuRAND (api.rs:683-719); those
+// streams do not exist on this platform, so only the distribution is kept.
+inline uint64_t splitmix64_at(uint64_t seed, uint64_t i) {
+  uint64_t z = seed + (i + 1) * 0x9e3779b97f4a7c15ull;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+inline CopyHostVecToDevice<float> randn_flat(float mean, float std, size_t n, uint64_t seed) {
+  auto host = std::make_shared<std::vector<float>>(n);
+  for (size_t i = 0; i < n; ++i) {
+    double u1 = (double)(splitmix64_at(seed, 2 * i) >> 11) * (1.0 / 9007199254740992.0);
+    double u2 = (double)(splitmix64_at(seed, 2 * i + 1) >> 11) * (1.0 / 9007199254740992.0);
+    if (u1 < 1e-300) u1 = 1e-300;
+    (*host)[i] = (float)(mean + std * std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2));
+  }
+  return copy_host_vec_to_device(std::move(host));
+}
+inline auto randn(float mean, float std, std::vector<int32_t> shape, uint64_t seed = 0) {
+  size_t n = checked_num_elements(shape).value_or(0);
+  return randn_flat(mean, std, n, seed).then([shape = std::move(shape)](Tensor<float> t) mutable {
+    return value(std::move(t).reshape(std::move(shape)).unwrap());
+  });
+}
+
+}  // namespace api
+
+// reshape on an op's output (api::DeviceOpReshape).
+template <class Op>
+auto reshape_op(Op op, std::vector<int32_t> shape) {
+  using TT = typename Op::Output;
+  return std::move(op).then([shape = std::move(shape)](TT t) mutable { return value(std::move(t).reshape(std::move(shape)).unwrap()); });
+}
+// partition on an op's output (tile_kernel.rs:1236-1316 PartitionOp).
+template <class Op>
+auto partition_op(Op op, std::vector<int32_t> tile) {
+  using TT = typename Op::Output;
+  return std::move(op).then([tile = std::move(tile)](TT t) mutable { return value(std::move(t).partition(std::move(tile))); });
+}
+// unpartition on an op that yields a partition.
+template <class Op>
+auto unpartition_op(Op op) {
+  using P = typename Op::Output;
+  return std::move(op).map([](P p) { return std::move(p).unpartition(); });
+}
+
+// ---- kernel launchers ------------------------------------------------------------------------
+template <class Fn, class... ArgOps>
+class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple<typename ArgOps::Output...>> {
+ public:
+  using Out = std::tuple<typename ArgOps::Output...>;
+  explicit KernelLauncher(ArgOps&&... ops) : ops_(std::move(ops)...) {}
+  KernelLauncher(KernelLauncher&&) = default;
+  // Builder methods of the generated launcher (cutile-macro/src/_module.rs:901-923).
+  KernelLauncher generics(std::vector<std::string> g) && { generics_ = std::move(g); return std::move(*this); }
+  KernelLauncher grid(uint32_t x, uint32_t y, uint32_t z) && { grid_ = {x, y, z}; return std::move(*this); }
+  KernelLauncher variant(std::string v) && { variant_ = std::move(v); return std::move(*this); }
+
+  Result<Out> execute(const ExecutionContext& ctx) && {
+    // 1. run the argument ops in signature order; 2. validate + launch; 3. hand the arguments back.
+    auto args = std::move(ops_).execute(ctx);
+    if (args.is_err()) return args.error();
+    Out vals = std::move(args).unwrap();
+    std::vector<const char*> gptrs;
+    for (auto& s : generics_) gptrs.push_back(s.c_str());
+    cutile_launch_opts_t opts{};
+    opts.grid[0] = grid_[0]; opts.grid[1] = grid_[1]; opts.grid[2] = grid_[2];
+    opts.generics = gptrs.empty() ? nullptr : gptrs.data();
+    opts.n_generics = (int32_t)gptrs.size();
+    opts.variant = variant_.empty() ? nullptr : variant_.c_str();
+    cutile_status_t s = std::apply([&](auto&... a) { return Fn::launch(ctx.stream()->raw(), &opts, a...); }, vals);
+    if (s != CUTILE_SUCCESS) return DeviceError::from_status(s);
+    return vals;
+  }
+
+ private:
+  Zip<ArgOps...> ops_;
+  std::vector<std::string> generics_;
+  std::array<uint32_t, 3> grid_{0, 0, 0};
+  std::string variant_;
+};
+template <class Fn, class... ArgOps>
+struct is_graph_node<KernelLauncher<Fn, ArgOps...>> : std::bool_constant<(is_graph_node_v<ArgOps> && ...)> {};
+
+template <class Fn, class... Xs>
+auto make_launcher(Xs&&... xs) {
+  return KernelLauncher<Fn, into_op_t<Xs>...>(into_op(std::forward<Xs>(xs))...);
+}
+
+namespace kernels {
+struct SaxpyFn {
+  template <class Y, class X>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Y& y, double a, X& x) {
+    auto yp = y.arg();
+    auto xa = input_arg(x);
+    return cutile_launch_saxpy(s, &yp, a, &xa, o);
+  }
+};
+struct AxpyFn {
+  template <class Z, class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, double a, X& x, Yv& y) {
+    auto zp = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y);
+    return cutile_launch_axpy(s, &zp, a, &xa, &ya, o);
+  }
+};
+struct AddFn {
+  template <class Z, class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y) {
+    auto zp = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y);
+    return cutile_launch_add(s, &zp, &xa, &ya, o);
+  }
+};
+struct RmsNormF16Fn {
+  template <class X, class W, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, W& w, O& out, float eps) {
+    auto xa = input_arg(x), wa = input_arg(w);
+    auto op = out.arg();
+    return cutile_launch_rms_norm_f16(s, &xa, &wa, &op, eps, o);
+  }
+};
+struct SoftmaxFn {
+  template <class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, Yv& y) {
+    auto xa = input_arg(x);
+    auto yp = y.arg();
+    return cutile_launch_softmax(s, &xa, &yp, o);
+  }
+};
+template <bool Accumulate>
+struct GemmFn {
+  template <class Z, class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, int32_t k) {
+    auto zp = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y);
+    return cutile_launch_gemm(s, &zp, &xa, &ya, k, Accumulate ? 1 : 0, o);
+  }
+};
+template <bool Causal>
+struct FmhaFn {
+  // fmha(out, q, k, v, qk_scale, input_pos, query_group_size) — flash_attention_causal.rs:32-40
+  template <class O, class Q, class K, class V>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, O& out, Q& q, K& k, V& v, float scale,
+                                int32_t input_pos, int32_t group) {
+    auto op = out.arg();
+    auto qa = input_arg(q), ka = input_arg(k), va = input_arg(v);
+    return cutile_launch_fmha(s, &op, &qa, &ka, &va, scale, input_pos, group, Causal ? 1 : 0, o);
+  }
+};
+struct LinearTileMxfp8Fn {
+  template <class Z, class X, class Yv, class XS, class YS>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, XS& xs, YS& ys, float alpha) {
+    auto zp = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y), xsa = input_arg(xs), ysa = input_arg(ys);
+    return cutile_launch_linear_tile_mxfp8(s, &zp, &xa, &ya, &xsa, &ysa, alpha, o);
+  }
+};
+}  // namespace kernels
+
+// saxpy(y: partition, a, x) -> (y, a, x)        cutile-examples/examples/saxpy.rs:12-17
+template <class Y, class A, class X> auto saxpy(Y&& y, A&& a, X&& x) { return make_launcher<kernels::SaxpyFn>(std::forward<Y>(y), std::forward<A>(a), std::forward<X>(x)); }
+// axpy(z: partition, a, x, y) -> (z, a, x, y)   three-operand form, rank 1
+template <class Z, class A, class X, class Y> auto axpy(Z&& z, A&& a, X&& x, Y&& y) { return make_launcher<kernels::AxpyFn>(std::forward<Z>(z), std::forward<A>(a), std::forward<X>(x), std::forward<Y>(y)); }
+// add(z: partition, x, y) -> (z, x, y)          README.md:29-38
+template <class Z, class X, class Y> auto add(Z&& z, X&& x, Y&& y) { return make_launcher<kernels::AddFn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y)); }
+// rms_norm_f16(x, w, out: partition [1,N], eps) -> (x, w, out, eps)   cutile-kernels/src/norms.rs:22-27
+template <class X, class W, class O> auto rms_norm_f16(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormF16Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
+// softmax(x, y: partition [BM,BN]) -> (x, y)    cutile-benchmarks/benches/softmax.rs:23-26
+template <class X, class Y> auto softmax(X&& x, Y&& y) { return make_launcher<kernels::SoftmaxFn>(std::forward<X>(x), std::forward<Y>(y)); }
+// gemm(z: partition [BM,BN], x, y, k) -> (z, x, y, k): z <- z + x·y   cutile-benchmarks/benches/gemm.rs:25-30
+template <class Z, class X, class Y> auto gemm(Z&& z, X&& x, Y&& y, int32_t k) { return make_launcher<kernels::GemmFn<true>>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), k); }
+// gemm_zero_init: accumulator starts at 0                              cutile-examples/examples/gemm.rs:20-36
+template <class Z, class X, class Y> auto gemm_zero_init(Z&& z, X&& x, Y&& y, int32_t k) { return make_launcher<kernels::GemmFn<false>>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), k); }
+// fmha(out: partition [1,BM,D], q, k, v, qk_scale, input_pos, query_group_size)   flash_attention_causal.rs:32-40
+template <class O, class Q, class K, class V> auto fmha(O&& out, Q&& q, K&& k, V&& v, float scale, int32_t input_pos, int32_t group) { return make_launcher<kernels::FmhaFn<false>>(std::forward<O>(out), std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), scale, input_pos, group); }
+template <class O, class Q, class K, class V> auto fmha_causal(O&& out, Q&& q, K&& k, V&& v, float scale, int32_t input_pos, int32_t group) { return make_launcher<kernels::FmhaFn<true>>(std::forward<O>(out), std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), scale, input_pos, group); }
+// linear_tile(z: partition [BM,BN], x, y, x_scales, y_scales, alpha)   cutile-examples/examples/mxfp8.rs:35-42
+template <class Z, class X, class Y, class XS, class YS> auto linear_tile(Z&& z, X&& x, Y&& y, XS&& xs, YS&& ys, float alpha) { return make_launcher<kernels::LinearTileMxfp8Fn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), std::forward<XS>(xs), std::forward<YS>(ys), alpha); }
+
+namespace api {
+template <class T> struct is_graph_node_memcpy : std::true_type {};
+}
+template <class T>
+struct is_graph_node<api::Memcpy<T>> : std::true_type {};
+
+}  // namespace cutile

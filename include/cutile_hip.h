@@ -185,7 +185,7 @@ typedef struct {
   const char* symbol;           /* "<fn>_entry__<variant>" */
   const char* variant;          /* variant name inside the function family */
   uint32_t block[3];            /* workgroup shape the kernel was written for */
-  uint32_t lds_bytes;           /* dynamic LDS bytes to pass at launch */
+  uint32_t lds_bytes;           /* LDS the kernel uses; it is static (carried by the code object), launches pass 0 */
   int32_t tile[4];              /* tile shape (BM, BN, BK, -) the variant implements; 0 = any */
 } cutile_kernel_info_t;
 
@@ -346,6 +346,55 @@ cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cu
                                                 const cutile_tensor_arg_t* x_scales,
                                                 const cutile_tensor_arg_t* y_scales, float alpha,
                                                 const cutile_launch_opts_t* opts);
+
+/* ======================================================================== */
+/* Part E — asynchronous runtime                                             */
+/* ======================================================================== */
+/* Thread-local execution lock: on a thread only one DeviceOp executes at a time
+ * (cuda-async/src/device_operation.rs:27-55).  Acquiring it twice on one thread
+ * fails with CUTILE_ERR_STATE and the reference's "non-reentrant" message. */
+cutile_status_t cutile_execution_lock_acquire(void);
+void cutile_execution_lock_release(void);
+int32_t cutile_execution_lock_held(void);
+
+/* Thread-local device contexts (cuda-async/src/device_context.rs:139-450).  Each
+ * thread has a default device and, per device, a scheduling policy, a dedicated
+ * deallocator stream and an optional memory pool; tests isolate state by running
+ * on fresh threads, as the reference's do. */
+typedef enum { CUTILE_POLICY_ROUND_ROBIN = 0, CUTILE_POLICY_SINGLE_STREAM = 1 } cutile_policy_kind_t;
+int32_t cutile_get_default_device(void);                      /* device_context.rs:164 */
+void cutile_set_default_device(int32_t ordinal);              /* device_context.rs:363-367 */
+/* init_device_contexts: a second call on a thread fails "Context already
+ * initialized." (device_context.rs:178-195) */
+cutile_status_t cutile_init_device_contexts(int32_t default_device, int32_t num_devices);
+/* init_device with an explicit policy; a second call for the same device fails
+ * "Device is already initialized." (device_context.rs:235-260).  num_streams <= 0
+ * selects the default pool of 4 (device_context.rs:39). */
+cutile_status_t cutile_init_device(int32_t ordinal, cutile_policy_kind_t kind, int32_t num_streams);
+/* with_device_policy(|p| p.next_stream()): ordinal < 0 = the thread's default
+ * device; contexts are created lazily with the round-robin policy
+ * (device_context.rs:315-328,444-450; scheduling_policies.rs:35-87). */
+cutile_status_t cutile_policy_next_stream(int32_t ordinal, cutile_stream_t* stream);
+/* with_deallocator_stream (device_context.rs:330-338): the stream frees are queued on */
+cutile_status_t cutile_deallocator_stream(int32_t ordinal, cutile_stream_t* stream);
+/* set_device_pool / get_device_pool (device_context.rs:396-432); NULL clears */
+cutile_status_t cutile_set_device_pool(int32_t ordinal, cutile_mempool_t pool);
+cutile_status_t cutile_get_device_pool(int32_t ordinal, cutile_mempool_t* pool);
+
+/* Completion notification for work already submitted on `stream`.  `waker(user)`
+ * is called exactly once, from another thread, after that work has completed.
+ * cutile_reactor_register is the flag-write path (cuda-async/src/reactor.rs:154-179):
+ * claim one of 1024 slots, enqueue a 32-bit stream write of 1 into pinned mapped
+ * memory, publish the waker to the scanner thread; CUTILE_ERR_OUT_OF_SLOTS when
+ * all slots are in flight.  cutile_completion_register is the chain
+ * DeviceFuture uses (cuda-async/src/device_future.rs:103-154): reactor first,
+ * hipLaunchHostFunc as fallback (or always, with CUTILE_ASYNC_HOST_SYNC=callback). */
+typedef void (*cutile_waker_fn_t)(void* user);
+cutile_status_t cutile_reactor_register(cutile_stream_t stream, cutile_waker_fn_t waker, void* user);
+cutile_status_t cutile_completion_register(cutile_stream_t stream, cutile_waker_fn_t waker, void* user);
+uint64_t cutile_reactor_registrations(void);
+uint64_t cutile_reactor_wakes(void);
+int32_t cutile_reactor_armed(void);
 
 #ifdef __cplusplus
 }

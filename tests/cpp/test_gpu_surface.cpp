@@ -1,0 +1,218 @@
+// GPU tests of the C++ host surface: the reference's runnable examples, end to end
+// through Tensor / Partition / DeviceOp / graph / future on a real MI355X, with
+// the known answers those examples assert (cutile-examples/examples/saxpy.rs:47-53,
+// softmax.rs:55-60, mxfp8.rs:129-135, cuda_graphs.rs:333-344,
+// cutile/tests/gpu/add_basic.rs:29-43, cutile/tests/slice_non_divisible.rs:459-500).
+#include <cutile/cutile.hpp>
+
+#include <atomic>
+#include <cmath>
+#include <thread>
+
+#include "check.hpp"
+
+using namespace cutile;
+
+static std::shared_ptr<Stream> new_stream() { return Device::create(0).unwrap()->new_stream().unwrap(); }
+
+TEST(device_is_gfx950) {
+  auto dev = Device::create(0).unwrap();
+  CHECK(dev->arch().unwrap().find("gfx950") != std::string::npos);
+  CHECK(dev->props().unwrap().wavefront_size == 64 && dev->l2_cache_size_bytes().unwrap() > 0);
+  CHECK(Device::device_count().unwrap() >= 1 && dev->name().is_ok());
+}
+
+TEST(saxpy_example) {
+  auto stream = new_stream();
+  auto input = std::make_shared<Tensor<float>>(api::arange<float>(32).sync_on(stream).unwrap());
+  auto x = std::make_shared<Tensor<float>>(std::move(api::dup(*input).sync_on(stream).unwrap()).reshape({4, 8}).unwrap());
+  auto y = std::move(api::dup(*input).sync_on(stream).unwrap()).reshape({4, 8}).unwrap().partition({2, 2});
+  auto y_host = api::to_host_vec_op(unpartition_op(saxpy(std::move(y), 2.0f, x).first())).sync_on(stream).unwrap();
+  auto in_host = api::to_host_vec(input).sync_on(stream).unwrap();
+  for (size_t i = 0; i < in_host.size(); ++i) CHECK(y_host[i] == 2.0f * in_host[i] + in_host[i]);
+}
+
+TEST(add_with_lazy_arguments) {
+  auto z = add(partition_op(api::zeros<float>({256}), {64}), api::ones<float>({256}), api::ones<float>({256}));
+  auto host = api::to_host_vec_op(unpartition_op(std::move(z).first())).sync().unwrap();  // default policy stream
+  for (float v : host) CHECK(v == 2.0f);
+}
+
+TEST(softmax_example_rows_sum_to_one) {
+  auto stream = new_stream();
+  auto x = std::make_shared<Tensor<float>>(reshape_op(api::arange<float>(32), {4, 8}).sync_on(stream).unwrap());
+  auto y = partition_op(api::zeros<float>({4, 8}), {2, 8});
+  auto [xo, yo] = softmax(x, std::move(y)).sync_on(stream).unwrap();
+  auto host = api::to_host_vec(std::move(yo).unpartition()).sync_on(stream).unwrap();
+  for (int r = 0; r < 4; ++r) {
+    float sum = 0;
+    for (int c = 0; c < 8; ++c) sum += host[r * 8 + c];
+    CHECK(std::fabs(sum - 1.0f) < 1e-4f);
+  }
+  CHECK(xo.get() == x.get());
+}
+
+TEST(rms_norm_constant_rows) {
+  auto stream = new_stream();
+  auto x = api::full<f16>(3.0, {16, 1024}).sync_on(stream).unwrap();
+  auto w = api::full<f16>(0.5, {1024}).sync_on(stream).unwrap();
+  auto out = api::zeros<f16>({16, 1024}).sync_on(stream).unwrap();
+  CHECK(rms_norm_f16(&x, &w, out.partition_mut({1, 1024}), 0.0f).generics({"1024", "512"}).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 0.5f);  // x == c -> out = w
+}
+
+TEST(gemm_ones_non_divisible) {
+  auto stream = new_stream();
+  const int m = 200, n = 264, k = 128;
+  auto x = api::ones<bf16>({m, k}).sync_on(stream).unwrap();
+  auto y = api::ones<bf16>({k, n}).sync_on(stream).unwrap();
+  auto z = api::zeros<bf16>({m, n}).sync_on(stream).unwrap();
+  CHECK(gemm(z.partition_mut({128, 128}), &x, &y, k).sync_on(stream).is_ok());
+  for (bf16 v : api::to_host_vec(z).sync_on(stream).unwrap()) CHECK(f32_from_bf16(v) == (float)k);
+}
+
+TEST(fmha_uniform_values) {
+  auto stream = new_stream();
+  const int b = 1, h = 2, s = 256, d = 64;
+  // V == 1 -> every output is 1 whatever the scores; Q, K random
+  auto to_bf16 = [&](Tensor<float> t) {
+    auto arc = std::make_shared<Tensor<float>>(std::move(t));
+    return std::move(api::convert<bf16>(arc).sync_on(stream).unwrap()).reshape({b, h, s, d}).unwrap();
+  };
+  auto q = to_bf16(api::randn(0.0f, 1.0f, {b * h * s * d}, 7).sync_on(stream).unwrap());
+  auto k = to_bf16(api::randn(0.0f, 1.0f, {b * h * s * d}, 11).sync_on(stream).unwrap());
+  auto v = api::ones<bf16>({b, h, s, d}).sync_on(stream).unwrap();
+  auto out = api::zeros<bf16>({b * h, s, d}).sync_on(stream).unwrap();
+  CHECK(fmha_causal(out.partition_mut({1, 64, d}), &q, &k, &v, 1.0f / std::sqrt((float)d), 0, 1).sync_on(stream).is_ok());
+  for (bf16 o : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(std::fabs(f32_from_bf16(o) - 1.0f) < 1e-2f);
+}
+
+TEST(mxfp8_example_all_ones) {
+  auto stream = new_stream();
+  const int M = 16, N = 16, K = 128;
+  auto bytes = [&](uint8_t v, int n, std::vector<int32_t> shape) {
+    auto host = std::make_shared<std::vector<uint8_t>>(n, v);
+    return std::make_shared<Tensor<uint8_t>>(std::move(api::copy_host_vec_to_device(host).sync_on(stream).unwrap()).reshape(std::move(shape)).unwrap());
+  };
+  auto x = Tensor<uint8_t>::reinterpret<f8e4m3fn>(bytes(0x38, M * K, {M, K}), {M, K}).unwrap();
+  auto y = Tensor<uint8_t>::reinterpret<f8e4m3fn>(bytes(0x38, N * K, {N, K}), {N, K}).unwrap();
+  auto xs = Tensor<uint8_t>::reinterpret<f8e8m0fnu>(bytes(0x7F, M * K / 32, {M, K / 32}), {M, K / 32}).unwrap();
+  auto ys = Tensor<uint8_t>::reinterpret<f8e8m0fnu>(bytes(0x7F, N * K / 32, {N, K / 32}), {N, K / 32}).unwrap();
+  auto z = partition_op(api::zeros<float>({M, N}), {16, 16});
+  auto res = linear_tile(std::move(z), x, y, xs, ys, 1.0f).generics({"16", "16", "64", "2"}).sync_on(stream).unwrap();
+  auto host = api::to_host_vec(std::move(std::get<0>(res)).unpartition()).sync_on(stream).unwrap();
+  for (float v : host) CHECK(std::fabs(v - (float)K) <= 1e-3f);
+}
+
+TEST(graph_replay_matches_eager) {
+  auto stream = new_stream();
+  const int n = 1 << 16;
+  auto w = api::randn(0.0f, 1.0f, {n}, 3).sync_on(stream).unwrap();
+  auto input = api::zeros<float>({n}).sync_on(stream).unwrap();
+  auto acc = api::zeros<float>({n}).sync_on(stream).unwrap();
+  // graph: acc <- input; acc <- 2*w + acc; acc <- 0.5*w + acc
+  auto graph = HipGraph<Unit>::scope(stream, [&](Scope& s) -> Result<Unit> {
+    CUTILE_TRY(s.record(api::memcpy(acc, input)));
+    CUTILE_TRY(s.record(saxpy(acc.partition_mut({1024}), 2.0f, &w)));
+    CUTILE_TRY(s.record(saxpy(acc.partition_mut({1024}), 0.5f, &w)));
+    return ok();
+  }).unwrap();
+  auto wh = api::to_host_vec(w).sync_on(stream).unwrap();
+  for (int rep = 0; rep < 4; ++rep) {  // several replays with eager work and syncs in between
+    auto fresh = api::full<float>((double)rep, {n}).sync_on(stream).unwrap();
+    CHECK(graph.update(api::memcpy(input, fresh)).is_ok());
+    CHECK(graph.launch().sync_on(stream).is_ok());
+    auto got = api::to_host_vec(acc).sync_on(stream).unwrap();
+    for (int i = 0; i < n; i += 97) {
+      float eager = std::fmaf(0.5f, wh[i], std::fmaf(2.0f, wh[i], (float)rep));
+      CHECK(got[i] == eager);
+    }
+  }
+  // graph_on keeps the captured op's output; launching it again recomputes in place
+  auto y = api::zeros<float>({n}).sync_on(stream).unwrap();
+  auto g2 = saxpy(y.partition_mut({1024}), 1.0f, &w).graph_on(stream).unwrap();
+  CHECK(g2.take_output().has_value());
+  CHECK(g2.launch().sync_on(stream).is_ok());
+  auto yh = api::to_host_vec(y).sync_on(stream).unwrap();
+  for (int i = 0; i < n; i += 101) CHECK(yh[i] == wh[i]);  // one replay after a capture pass that does not execute
+}
+
+TEST(futures_complete_through_the_reactor) {
+  // CUTILE_ASYNC_SPIN_BUDGET_US=0 (set in main) forces the notification path
+  auto stream = new_stream();
+  const int n = 1 << 20;
+  auto w = api::ones<float>({n}).sync_on(stream).unwrap();
+  auto y = api::zeros<float>({n}).sync_on(stream).unwrap();
+  uint64_t before = cutile_reactor_registrations();
+  for (int i = 0; i < 50; ++i) CHECK(saxpy(y.partition_mut({1024}), 1.0f, &w).schedule_on(stream).block_on().is_ok());
+  CHECK(cutile_reactor_registrations() == before + 50 && cutile_reactor_armed() == 0);
+  auto host = api::to_host_vec(y).sync_on(stream).unwrap();
+  CHECK(host[0] == 50.0f && host[n - 1] == 50.0f);
+  // wait() on the default policy, from several threads at once
+  std::atomic<int> okc{0};
+  std::vector<std::thread> ts;
+  for (int t = 0; t < 4; ++t)
+    ts.emplace_back([&] {
+      for (int i = 0; i < 25; ++i)
+        if (api::to_host_vec_op(api::full<float>(3.0, {4096})).wait().unwrap()[4095] == 3.0f) okc.fetch_add(1);
+    });
+  for (auto& t : ts) t.join();
+  CHECK(okc.load() == 100);
+}
+
+TEST(memory_pool_and_streams) {
+  auto dev = Device::create(0).unwrap();
+  auto pool = dev->new_mem_pool().unwrap();
+  CHECK(pool->set_release_threshold(64u << 20).is_ok());
+  CHECK(cutile_set_device_pool(0, pool->raw()) == CUTILE_SUCCESS);
+  auto stream = dev->new_stream().unwrap();
+  {
+    auto t = api::zeros<float>({1 << 20}).sync_on(stream).unwrap();  // allocated from the thread's pool
+    auto st = pool->mem_stats().unwrap();
+    CHECK(st.used_current >= (4u << 20) && st.used_high >= st.used_current);
+  }
+  CHECK(cutile_set_device_pool(0, nullptr) == CUTILE_SUCCESS);
+  CHECK(stream->query().is_ok() && stream->synchronize().is_ok());
+}
+
+TEST(do_bench_and_autotune_pick_a_variant) {
+  auto stream = new_stream();
+  const int rows = 4096, n = 8192;
+  auto x = api::full<f16>(1.0, {rows, n}).sync_on(stream).unwrap();
+  auto w = api::ones<f16>({n}).sync_on(stream).unwrap();
+  auto out = api::zeros<f16>({rows, n}).sync_on(stream).unwrap();
+  bench::BenchOptions bo;
+  bo.warmup = std::chrono::milliseconds(5);
+  bo.rep = std::chrono::milliseconds(20);
+  auto m = bench::do_bench(stream, bo, [&](const std::shared_ptr<Stream>& s) -> Result<Unit> {
+    auto r = rms_norm_f16(&x, &w, out.partition_mut({1, n}), 1e-6f).async_on(s);
+    return r.is_err() ? Result<Unit>(r.error()) : ok();
+  }).unwrap();
+  CHECK(m.reps() >= 5 && m.median_ms() > 0.005f && m.median_ms() < 5.0f && m.min_ms() <= m.median_ms());
+  auto tuned = tune::Autotuner("rms_norm_f16_8192").configs(tune::variant_configs("rms_norm_f16")).bench_options(bo)
+                   .run(stream, [&](const std::shared_ptr<Stream>&, const tune::Config& c) -> Result<bench::BenchFn> {
+                     std::string v = *c.str("variant");
+                     // probe once: variants that cannot hold an 8192-wide row are invalid candidates
+                     auto probe = rms_norm_f16(&x, &w, out.partition_mut({1, n}), 1e-6f).variant(v).sync_on(stream);
+                     if (probe.is_err()) return probe.error();
+                     return bench::BenchFn([&, v](const std::shared_ptr<Stream>& s) -> Result<Unit> {
+                       auto r = rms_norm_f16(&x, &w, out.partition_mut({1, n}), 1e-6f).variant(v).async_on(s);
+                       return r.is_err() ? Result<Unit>(r.error()) : ok();
+                     });
+                   }).unwrap();
+  CHECK(tuned.best.has_value());
+  int invalid = 0;
+  for (auto& t : tuned.trials) invalid += !t.measured;
+  CHECK(invalid >= 4);  // w1v1..w1v8 cannot hold the row
+  std::string best = *tuned.best->str("variant");
+  CHECK(best != "generic");
+  CHECK(cutile_kernel_set_preferred_variant("rms_norm_f16", best.c_str()) == CUTILE_SUCCESS);
+  CHECK(rms_norm_f16(&x, &w, out.partition_mut({1, n}), 1e-6f).sync_on(stream).is_ok());
+  CHECK(cutile_kernel_set_preferred_variant("rms_norm_f16", nullptr) == CUTILE_SUCCESS);
+  printf("     autotune picked rms_norm_f16 variant %s\n", best.c_str());
+}
+
+int main(int argc, char** argv) {
+  setenv("CUTILE_ASYNC_SPIN_BUDGET_US", "0", 1);
+  return run_all_tests(argc, argv);
+}

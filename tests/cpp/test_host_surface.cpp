@@ -1,0 +1,466 @@
+// CPU tests of the C++ host surface on the recording stand-in for the HIP
+// runtime.  They restate, case by case, the reference's host-only and
+// fake-backed tests: cuda-async/tests/{execute_once,error_handling,cuda_graph}.rs,
+// cutile/src/tensor.rs:2161-2202, cutile/src/bench.rs:266-291,
+// cutile/src/tune.rs (FakeOracle tests), cuda-async/src/device_future.rs:325-384.
+#include <cutile/cutile.hpp>
+#include <cutile_hip_testing.h>
+
+#include <atomic>
+#include <thread>
+
+#include "check.hpp"
+
+using namespace cutile;
+
+static std::shared_ptr<Stream> fresh_stream() {
+  auto dev = Device::create(0).unwrap();
+  return dev->new_stream().unwrap();
+}
+static int launches() { return cutile_testing_launch_count(); }
+static std::string last_symbol() {
+  cutile_testing_launch_record_t r;
+  cutile_testing_get_launch(launches() - 1, &r);
+  return r.symbol;
+}
+
+// An op that counts how often it executes (execute_once.rs:24 uses a boxed op the same way).
+struct Counting : DeviceOp<Counting, int> {
+  std::shared_ptr<std::atomic<int>> n;
+  int v;
+  Counting(std::shared_ptr<std::atomic<int>> n, int v) : n(std::move(n)), v(v) {}
+  Result<int> execute(const ExecutionContext&) && {
+    n->fetch_add(1);
+    return v;
+  }
+};
+struct Failing : DeviceOp<Failing, int> {
+  Result<int> execute(const ExecutionContext&) && { return DeviceError::launch("boom"); }
+};
+
+TEST(combinators_compose_and_propagate_errors) {
+  auto s = fresh_stream();
+  CHECK(value(3).map([](int x) { return x + 1; }).sync_on(s).unwrap() == 4);
+  int seen = 0;
+  auto r = value(5).inspect([&](const int& x) { seen = x; }).then([](int x) { return value(x * 2); }).sync_on(s);
+  CHECK(r.unwrap() == 10 && seen == 5);
+  auto z = zip(value(1), 2.5, value(std::string("x"))).sync_on(s).unwrap();
+  CHECK(std::get<0>(z) == 1 && std::get<1>(z) == 2.5 && std::get<2>(z) == "x");
+  CHECK(zip(1, 2, 3).first().sync_on(s).unwrap() == 1);
+  CHECK(zip(1, 2, 3).last().sync_on(s).unwrap() == 3);
+  // an error short-circuits the chain: the closure after it never runs
+  bool ran = false;
+  auto e = Failing{}.then([&](int) { ran = true; return value(0); }).sync_on(s);
+  CHECK(e.is_err() && e.error().kind == DeviceError::Kind::Launch && !ran);
+  auto ez = zip(value(1), Failing{}).sync_on(s);
+  CHECK(ez.is_err());
+}
+
+TEST(shared_and_unzip_execute_once) {
+  auto s = fresh_stream();
+  auto n = std::make_shared<std::atomic<int>>(0);
+  auto sh = Counting(n, 7).shared();
+  auto a = sh;  // clones share the result
+  auto b = sh;
+  CHECK(*std::move(a).sync_on(s).unwrap() == 7);
+  CHECK(*std::move(b).sync_on(s).unwrap() == 7);
+  CHECK(*std::move(sh).sync_on(s).unwrap() == 7);
+  CHECK(n->load() == 1);
+  // unzip: the tuple op runs once, each half takes its element
+  auto m = std::make_shared<std::atomic<int>>(0);
+  auto [x, y] = Counting(m, 1).map([](int v) { return std::make_tuple(v, std::string("s")); }).unzip();
+  CHECK(std::move(y).sync_on(s).unwrap() == "s");
+  CHECK(std::move(x).sync_on(s).unwrap() == 1);
+  CHECK(m->load() == 1);
+  // shared(arc): already computed
+  CHECK(*shared(std::make_shared<int>(9)).sync_on(s).unwrap() == 9);
+  CHECK(unwrap_arc(std::make_shared<int>(4)) == 4);
+  auto two = std::make_shared<int>(4);
+  auto other = two;
+  CHECK_THROWS(unwrap_arc(two), "multiple owners");
+  // boxed ops go into one container
+  std::vector<BoxedDeviceOp<int>> ops;
+  ops.push_back(value(1).boxed());
+  ops.push_back(Counting(n, 2).boxed());
+  int sum = 0;
+  for (auto& o : ops) sum += std::move(o).sync_on(s).unwrap();
+  CHECK(sum == 3);
+}
+
+TEST(execution_is_not_reentrant_on_a_thread) {
+  auto s = fresh_stream();
+  auto s2 = fresh_stream();
+  // sync_on inside a then-closure is rejected (device_operation.rs:27-55; tests/cuda_graph.rs:130-165)
+  std::optional<DeviceError> inner;
+  auto r = value(1).then([&](int x) {
+    auto nested = value(2).sync_on(s2);
+    if (nested.is_err()) inner = nested.error();
+    return value(x);
+  }).sync_on(s);
+  CHECK(r.is_ok() && inner && inner->message.find("non-reentrant") != std::string::npos);
+  CHECK(cutile_execution_lock_held() == 0);  // released after the outer op
+  CHECK(value(1).sync_on(s).is_ok());        // and usable again
+}
+
+TEST(default_policy_round_robins_over_four_streams) {
+  std::vector<cutile_stream_t> seen;
+  for (int i = 0; i < 9; ++i) seen.push_back(next_stream().unwrap()->raw());
+  CHECK(seen[0] != seen[1] && seen[1] != seen[2] && seen[2] != seen[3]);
+  CHECK(seen[4] == seen[0] && seen[5] == seen[1] && seen[8] == seen[0]);
+  // contexts are per thread: another thread gets its own pool
+  cutile_stream_t other = nullptr;
+  std::thread([&] { other = next_stream().unwrap()->raw(); }).join();
+  CHECK(other != nullptr && other != seen[0] && other != seen[1] && other != seen[2] && other != seen[3]);
+  // sync() uses the policy
+  CHECK(value(1).sync().unwrap() == 1);
+}
+
+TEST(explicit_policies_and_double_initialisation) {
+  CHECK(init_device_contexts(0, 1).is_ok());
+  auto again = init_device_contexts(0, 1);  // error_handling.rs:137-156
+  CHECK(again.is_err() && again.error().message.find("Context already initialized.") != std::string::npos);
+  CHECK(init_device(0, PolicyKind::SingleStream).is_ok());
+  auto dup = init_device(0, PolicyKind::StreamPoolRoundRobin, 2);
+  CHECK(dup.is_err() && dup.error().message.find("Device is already initialized.") != std::string::npos);
+  auto a = next_stream().unwrap()->raw();
+  auto b = next_stream().unwrap()->raw();
+  CHECK(a == b);  // SingleStream
+  // invalid device ordinal surfaces as a driver error (error_handling.rs:174-190)
+  auto bad = Device::create(7);
+  CHECK(bad.is_err() && bad.error().kind == DeviceError::Kind::Driver);
+  set_default_device(0);
+  CHECK(get_default_device() == 0);
+}
+
+struct FakeAlloc : DeviceAllocation {  // cutile/src/tensor.rs:2146-2159
+  size_t len;
+  explicit FakeAlloc(size_t l) : len(l) {}
+  void* device_ptr() const override { return (void*)16; }
+  size_t len_bytes() const override { return len; }
+  int device_id() const override { return 0; }
+};
+
+TEST(tensor_extent_validation_vectors) {
+  // tensor.rs:2161-2202
+  CHECK(addressable_bytes<float>({4}, {1}) == 16);
+  CHECK(addressable_bytes<float>({4}, {10}) == 31 * 4);
+  CHECK(addressable_bytes<float>({0}, {1}) == 0);
+  auto ok = Tensor<float>::from_foreign(std::make_shared<FakeAlloc>(124), {4}, {10});
+  CHECK(ok.size() == 4);
+  CHECK_THROWS(Tensor<float>::from_foreign(std::make_shared<FakeAlloc>(16), {4}, {10}), "addressable extent");
+  CHECK_THROWS(Tensor<float>::from_foreign(std::make_shared<FakeAlloc>(16), {INT32_MAX, INT32_MAX}, {INT32_MAX, INT32_MAX}),
+               "addressable extent overflowed");
+  // prod(shape) * sizeof(T) must equal the storage size (tensor.rs:739-752)
+  CHECK_THROWS(Tensor<float>::from_raw_parts((void*)16, 12, 0, {4}, {1}), "storage size");
+}
+
+TEST(meta_tensors_have_metadata_but_no_pointer) {
+  auto m = Tensor<float>::from_meta({128, 256});
+  CHECK(m.is_meta() && m.size() == 128 * 256 && m.strides() == std::vector<int32_t>({256, 1}));
+  CHECK(m.spec().base_ptr_div == 16 && m.spec().shape_div[0] == 16);
+  CHECK_THROWS(m.device_pointer(), "meta tensor");
+}
+
+TEST(tensor_views_reshape_reinterpret_partition) {
+  auto s = fresh_stream();
+  auto t = api::arange<float>(1024).sync_on(s).unwrap();
+  CHECK(t.shape() == std::vector<int32_t>({1024}) && t.is_contiguous() && t.num_bytes() == 4096);
+  // views / slices: offsets accumulate (host-api reference: tensor[110..120])
+  auto inner = t.slice({{100, 200}}).unwrap().slice({{10, 20}}).unwrap();
+  CHECK(inner.offset_bytes() == 110 * 4 && inner.shape()[0] == 10);
+  auto mat = t.view({32, 32}).unwrap();
+  auto block = mat.slice({{1, 3}, {2, 6}}).unwrap();
+  CHECK(block.offset_bytes() == (32 + 2) * 4 && block.shape() == std::vector<int32_t>({2, 4}) && block.strides() == std::vector<int32_t>({32, 1}));
+  CHECK((char*)block.arg().ptr - (char*)t.device_pointer() == (32 + 2) * 4);
+  CHECK(t.view({33, 31}).is_err() && t.slice({{0, 2000}}).is_err());
+  // reshape consumes; reshape_shared and reinterpret share the allocation
+  auto r = std::move(t).reshape({4, 256}).unwrap();
+  CHECK(r.strides() == std::vector<int32_t>({256, 1}));
+  CHECK(std::move(r).reshape({5, 5}).is_err());
+  auto arc = std::make_shared<Tensor<uint32_t>>(api::arange<uint32_t>(4).sync_on(s).unwrap());
+  auto fl = Tensor<uint32_t>::reinterpret<float>(arc, {4}).unwrap();
+  CHECK(fl->device_pointer() == arc->device_pointer() && fl->shape()[0] == 4);
+  CHECK(Tensor<uint32_t>::reinterpret<double>(arc, {4}).is_err());  // byte size must match
+  auto two = Tensor<uint32_t>::reshape_shared(arc, {2, 2}).unwrap();
+  // partition needs unique storage: the allocation is shared by three handles now
+  CHECK(try_partition(arc, {2}).is_err());
+  auto solo = api::zeros<float>({128, 256}).sync_on(s).unwrap();
+  auto p = std::move(solo).partition({32, 64});
+  auto g = p.grid().unwrap();
+  CHECK(g[0] == 4 && g[1] == 4 && g[2] == 1);  // tensor.rs:440-442
+  auto back = std::move(p).unpartition();
+  CHECK(back.size() == 128 * 256);
+  auto one = std::make_shared<Tensor<float>>(std::move(back));
+  CHECK(try_partition(std::move(one), {128, 256}).is_ok());
+}
+
+TEST(transfers_round_trip) {
+  auto s = fresh_stream();
+  auto host = std::make_shared<std::vector<float>>(std::vector<float>{1, 2, 3, 4, 5, 6});
+  auto t = api::copy_host_vec_to_device(host).sync_on(s).unwrap();
+  auto d = api::dup(t).sync_on(s).unwrap();
+  CHECK(d.device_pointer() != t.device_pointer());
+  CHECK(api::to_host_vec(d).sync_on(s).unwrap() == *host);
+  auto dst = api::zeros<float>({6}).sync_on(s).unwrap();
+  CHECK(api::memcpy(dst, t).sync_on(s).is_ok());
+  CHECK(api::to_host_vec(dst).sync_on(s).unwrap() == *host);
+  auto small = api::zeros<float>({3}).sync_on(s).unwrap();
+  CHECK_THROWS(api::memcpy(small, t), "same number of elements");
+  // op-level helpers: reshape / partition / to_host_vec on an op's output
+  auto v = api::to_host_vec_op(reshape_op(api::copy_host_vec_to_device(host), {2, 3})).sync_on(s).unwrap();
+  CHECK(v == *host);
+  // owned storage is released when the tensor goes away
+  uint64_t before = cutile_testing_bytes_allocated();
+  { auto tmp = api::zeros<float>({1024}).sync_on(s).unwrap(); CHECK(cutile_testing_bytes_allocated() == before + 4096); }
+  CHECK(cutile_testing_bytes_allocated() == before);
+}
+
+TEST(launchers_hand_arguments_back_in_the_form_given) {
+  auto s = fresh_stream();
+  cutile_testing_clear_log();
+  auto x = std::make_shared<Tensor<float>>(api::arange<float>(32).sync_on(s).unwrap());
+  auto x2 = Tensor<float>::reshape_shared(x, {4, 8}).unwrap();
+  x.reset();
+  int before = launches();
+  // owned partition + Arc input: cutile-examples/examples/saxpy.rs:27-45
+  auto y = reshape_op(api::arange<float>(32), {4, 8}).sync_on(s).unwrap().partition({2, 2});
+  auto [y_out, a_out, x_out] = saxpy(std::move(y), 2.0f, x2).sync_on(s).unwrap();
+  CHECK(launches() == before + 2);  // arange for y + the saxpy itself
+  CHECK(last_symbol() == "saxpy_entry__f32_r2_flat");
+  CHECK(a_out == 2.0f && x_out.get() == x2.get());
+  Tensor<float> y_back = std::move(y_out).unpartition();
+  CHECK(y_back.shape() == std::vector<int32_t>({4, 8}));
+  // borrowed input and in-place partition: nothing changes hands
+  Tensor<float> w = api::ones<float>({4, 8}).sync_on(s).unwrap();
+  auto res = saxpy(y_back.partition_mut({2, 2}), 1.0f, &w).sync_on(s).unwrap();
+  CHECK(std::get<2>(res) == &w && &std::get<0>(res).tensor() == &y_back);
+  // arguments may themselves be ops; views are passed as pointer + offset
+  auto view = w.slice({{0, 2}}).unwrap();
+  auto r2 = saxpy(partition_op(api::zeros<float>({2, 8}), {2, 8}), 3.0f, view).sync_on(s);
+  CHECK(r2.is_ok());
+  // a launch-time violation is reported before any GPU work
+  int n0 = launches();
+  auto bad = rms_norm_f16(api::zeros<f16>({4, 64}), api::zeros<f16>({32}), partition_op(api::zeros<f16>({4, 64}), {1, 64}), 1e-6f).sync_on(s);
+  CHECK(bad.is_err() && bad.error().kind == DeviceError::Kind::Launch);
+  CHECK(launches() == n0 + 3);  // the three fills ran, the kernel did not
+  auto nokernel = gemm(partition_op(api::zeros<bf16>({64, 64}), {48, 48}), api::zeros<bf16>({64, 64}), api::zeros<bf16>({64, 64}), 64).sync_on(s);
+  CHECK(nokernel.is_err() && nokernel.error().kind == DeviceError::Kind::KernelCache);
+  // builder methods reach the launcher
+  auto g = gemm(partition_op(api::zeros<bf16>({256, 256}), {128, 128}), api::zeros<bf16>({256, 64}), api::zeros<bf16>({64, 256}), 64)
+               .generics({"bf16", "128", "128", "64"}).variant("bf16_128x128x64_w2x2").sync_on(s);
+  CHECK(g.is_ok() && last_symbol() == "gemm_entry__bf16_128x128x64_w2x2");
+  auto wrong = gemm(partition_op(api::zeros<bf16>({256, 256}), {128, 128}), api::zeros<bf16>({256, 64}), api::zeros<bf16>({64, 256}), 64)
+                   .grid(1, 1, 1).sync_on(s);
+  CHECK(wrong.is_err() && wrong.error().message.find("does not match the inferred partition grid") != std::string::npos);
+}
+
+TEST(graph_capture_replay_and_failure_matrix) {
+  auto s = fresh_stream();
+  Tensor<float> out = api::zeros<float>({1024}).sync_on(s).unwrap();
+  Tensor<float> w = api::ones<float>({1024}).sync_on(s).unwrap();
+  Tensor<float> staging = api::zeros<float>({1024}).sync_on(s).unwrap();
+  cutile_testing_clear_log();
+  // scope: two launches recorded, none executed eagerly twice (cuda_graphs.rs example shape)
+  auto graph = HipGraph<Unit>::scope(s, [&](Scope& sc) -> Result<Unit> {
+    CUTILE_TRY(sc.record(saxpy(out.partition_mut({128}), 2.0f, &w)));
+    CUTILE_TRY(sc.record(saxpy(out.partition_mut({64}), 1.0f, &w)));
+    CUTILE_TRY(sc.record(api::memcpy(staging, out)));
+    return ok();
+  }).unwrap();
+  CHECK(launches() == 2);
+  cutile_testing_launch_record_t rec;
+  cutile_testing_get_launch(0, &rec);
+  CHECK(rec.in_capture == 1 && rec.from_graph_replay == 0);
+  CHECK(graph.launch().sync_on(s).is_ok());
+  CHECK(graph.launch().sync_on(s).is_ok());
+  CHECK(launches() == 6);  // each replay re-issues both kernels
+  cutile_testing_get_launch(5, &rec);
+  CHECK(rec.from_graph_replay == 1 && std::string(rec.symbol) == "saxpy_entry__f32_r1_flat");
+  CHECK(cutile_execution_lock_held() == 0);
+  // update runs on the graph's stream without a sync
+  CHECK(graph.update(api::memcpy(staging, w)).is_ok());
+  // graph_on keeps the op's output from the capture pass
+  auto g2 = saxpy(partition_op(api::zeros<float>({256}), {128}), 1.0f, api::ones<float>({256})).graph_on(s);
+  CHECK(g2.is_err());  // allocation inside a capture is refused by the runtime (hipErrorStreamCaptureUnsupported)
+  auto g3 = value(41).map([](int v) { return v + 1; }).graph_on(s).unwrap();
+  CHECK(*g3.take_output() == 42 && !g3.take_output());
+  // failure matrix (cuda_graph.rs:81-104): op fails -> its error, capture still ended
+  auto f1 = Failing{}.graph_on(s);
+  CHECK(f1.is_err() && f1.error().message == "boom");
+  CHECK(value(1).sync_on(s).is_ok());  // the stream is usable: capture was closed
+  cutile_testing_inject_failure("hipStreamEndCapture", 901, 1);
+  auto f2 = value(1).graph_on(s);
+  CHECK(f2.is_err() && f2.error().kind == DeviceError::Kind::Driver && f2.error().code == 901);
+  cutile_testing_inject_failure("hipGraphInstantiateWithFlags", 2, 1);
+  CHECK(value(1).graph_on(s).is_err());
+  cutile_testing_inject_failure("hipGraphUpload", 2, 1);
+  CHECK(value(1).graph_on(s).is_err());
+  // a body that throws still ends the capture and releases the lock (cuda_graph.rs:400-505)
+  bool threw = false;
+  try {
+    (void)HipGraph<Unit>::scope(s, [&](Scope&) -> Result<Unit> { throw std::runtime_error("body panicked"); });
+  } catch (const std::runtime_error&) { threw = true; }
+  CHECK(threw && cutile_execution_lock_held() == 0 && value(1).sync_on(s).is_ok());
+  // nested execution inside a scope is rejected
+  auto nested = HipGraph<Unit>::scope(s, [&](Scope&) -> Result<Unit> {
+    auto r = value(1).sync_on(s);
+    return r.is_err() ? Result<Unit>(r.error()) : ok();
+  });
+  CHECK(nested.is_err() && nested.error().message.find("non-reentrant") != std::string::npos);
+}
+
+TEST(device_future_states) {
+  auto s = fresh_stream();
+  // failed(): first poll yields the error, a second poll is a bug (device_future.rs:88-97,312-316)
+  auto f = DeviceFuture<Value<int>>::failed(DeviceError::scheduling("no stream"));
+  CHECK(f.state() == DeviceFutureState::Failed);
+  auto r = f.poll([] {});
+  CHECK(r && r->is_err() && r->error().kind == DeviceError::Kind::Scheduling && f.state() == DeviceFutureState::Complete);
+  CHECK_THROWS(f.poll([] {}), "Poll called after completion.");
+  // a scheduled future: Idle -> (Executing ->) Complete, result delivered once
+  auto fut = value(5).map([](int v) { return v * 3; }).schedule_on(s);
+  CHECK(fut.state() == DeviceFutureState::Idle);
+  CHECK(fut.block_on().unwrap() == 15 && fut.state() == DeviceFutureState::Complete);
+  // the op's error comes out of the first poll
+  auto bad = Failing{}.schedule_on(s);
+  auto br = bad.poll([] {});
+  CHECK(br && br->is_err() && bad.state() == DeviceFutureState::Complete);
+  // wait() = into_future().block_on() on the policy's stream
+  CHECK(value(2).wait().unwrap() == 2);
+  CHECK(cutile_execution_lock_held() == 0);
+}
+
+TEST(completion_goes_through_the_reactor_when_not_spun) {
+  // CUTILE_ASYNC_SPIN_BUDGET_US=0 is set by main(): every future registers for a notification
+  auto s = fresh_stream();
+  uint64_t before = cutile_reactor_registrations();
+  std::atomic<int> wakes{0};
+  auto fut = value(1).schedule_on(s);
+  auto first = fut.poll([&] { wakes.fetch_add(1); });
+  CHECK(!first && fut.state() == DeviceFutureState::Executing);
+  for (int i = 0; i < 2000 && wakes.load() == 0; ++i) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  CHECK(wakes.load() == 1 && cutile_reactor_registrations() == before + 1);
+  auto second = fut.poll([] {});
+  CHECK(second && second->unwrap() == 1);
+  // many in flight at once, from several threads
+  std::vector<std::thread> ts;
+  std::atomic<int> done{0};
+  for (int t = 0; t < 4; ++t)
+    ts.emplace_back([&] {
+      auto st = Device::create(0).unwrap()->new_stream().unwrap();
+      for (int i = 0; i < 200; ++i)
+        if (value(i).schedule_on(st).block_on().unwrap() == i) done.fetch_add(1);
+    });
+  for (auto& t : ts) t.join();
+  CHECK(done.load() == 800 && cutile_reactor_armed() == 0);
+  // the raw registration API reports exhaustion instead of blocking: hold the stream in capture so flags never fire
+  CHECK(cutile_stream_begin_capture(s->raw()) == CUTILE_SUCCESS);
+  int ok_regs = 0, exhausted = 0;
+  static std::atomic<int> fired{0};
+  for (int i = 0; i < 1100; ++i) {
+    cutile_status_t st = cutile_reactor_register(s->raw(), [](void*) { fired.fetch_add(1); }, nullptr);
+    if (st == CUTILE_SUCCESS) ++ok_regs; else if (st == CUTILE_ERR_OUT_OF_SLOTS) ++exhausted;
+  }
+  CHECK(ok_regs == 1024 && exhausted == 76);
+  // completion_register falls back to a host callback when the reactor is full (device_future.rs:142-153)
+  CHECK(cutile_completion_register(s->raw(), [](void*) { fired.fetch_add(1000000); }, nullptr) == CUTILE_SUCCESS);
+  cutile_graph_t g = nullptr;
+  CHECK(cutile_stream_end_capture(s->raw(), &g) == CUTILE_SUCCESS);
+  cutile_graph_exec_t ge = nullptr;
+  CHECK(cutile_graph_instantiate(g, &ge) == CUTILE_SUCCESS && cutile_graph_launch(ge, s->raw()) == CUTILE_SUCCESS);
+  for (int i = 0; i < 2000 && fired.load() < 1001024; ++i) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  CHECK(fired.load() == 1001024 && cutile_reactor_armed() == 0);
+}
+
+TEST(bench_quantiles) {
+  // cutile/src/bench.rs:266-291
+  bench::Measurement r({4.0f, 1.0f, 3.0f, 2.0f});
+  CHECK(r.min_ms() == 1.0f && r.median_ms() == 2.5f && r.quantile_ms(0.0f) == 1.0f && r.quantile_ms(1.0f) == 4.0f);
+  CHECK(r.quantile_ms(-1.0f) == 1.0f && r.quantile_ms(2.0f) == 4.0f && std::fabs(r.mean_ms() - 2.5f) < 1e-6f);
+  bench::Measurement one({7.0f});
+  CHECK(one.median_ms() == 7.0f && one.quantile_ms(0.25f) == 7.0f);
+  bench::Measurement out({1.0f, 1.0f, 1.0f, 1.0f, 100.0f});
+  CHECK(out.median_ms() == 1.0f && out.mean_ms() > 20.0f);
+  // do_bench on the recording runtime: warm-up at least once, reps within bounds, the closure sees the stream
+  auto s = fresh_stream();
+  int calls = 0;
+  bench::BenchOptions o;
+  o.warmup = std::chrono::milliseconds(0);
+  o.rep = std::chrono::milliseconds(1);
+  o.min_reps = 3;
+  o.max_reps = 3;
+  auto m = bench::do_bench(s, o, [&](const std::shared_ptr<Stream>& st) -> Result<Unit> { CHECK(st.get() == s.get()); ++calls; return ok(); }).unwrap();
+  CHECK(m.reps() == 3 && calls == 1 + 1 + 3);
+}
+
+struct FakeOracle : tune::Oracle {  // cutile/src/tune.rs:1045
+  std::vector<tune::Config> cfgs;
+  std::map<std::string, float> ms;
+  std::vector<std::string> measured;
+  size_t budget = SIZE_MAX;
+  const std::vector<tune::Config>& configs() const override { return cfgs; }
+  bool budget_exhausted() const override { return measured.size() >= budget; }
+  tune::Trial measure(size_t i) override {
+    measured.push_back(cfgs[i].id);
+    auto it = ms.find(cfgs[i].id);
+    if (it == ms.end()) return tune::Trial::invalid(cfgs[i].id, "does not launch");
+    return tune::Trial::ok(cfgs[i].id, it->second, it->second, 5);
+  }
+};
+
+TEST(autotuner_search_semantics) {
+  using tune::Config;
+  auto a = Config::make({{"bm", "128"}, {"bn", "128"}}), b = Config::make({{"bm", "256"}, {"bn", "256"}}), c = Config::make({{"bm", "64"}, {"bn", "64"}});
+  CHECK(a.id == "bm=128,bn=128" && *a.integer("bm") == 128 && !a.integer("zz") && *a.str("bn") == "128");
+  CHECK(tune::space_hash({a, b, c}) == tune::space_hash({c, a, b}) && tune::space_hash({a, b}) != tune::space_hash({a, b, c}));
+  FakeOracle o;
+  o.cfgs = {a, b, c};
+  o.ms = {{a.id, 2.0f}, {b.id, 1.0f}};  // c is invalid: data, not an error
+  auto trials = tune::GridSearch{}.search(o);
+  CHECK(trials.size() == 3 && !trials[2].measured && trials[2].invalid_reason == "does not launch");
+  CHECK(tune::best_config(o.cfgs, trials)->id == b.id);
+  // resume: measured known trials are kept, invalid ones retried, stale configs ignored
+  FakeOracle o2;
+  o2.cfgs = {a, b, c};
+  o2.ms = {{a.id, 2.0f}, {b.id, 1.0f}, {c.id, 0.5f}};
+  std::vector<tune::Trial> known = {tune::Trial::ok(a.id, 2.0f, 2.0f, 5), tune::Trial::invalid(c.id, "transient"), tune::Trial::ok("gone=1", 0.1f, 0.1f, 5)};
+  auto t2 = tune::GridSearch{}.resume(known).search(o2);
+  CHECK(o2.measured == std::vector<std::string>({b.id, c.id}));
+  CHECK(tune::best_config(o2.cfgs, t2)->id == c.id);  // the stale 0.1 ms record neither wins nor shadows
+  // budget: stop measuring when exhausted
+  FakeOracle o3;
+  o3.cfgs = {a, b, c};
+  o3.ms = o2.ms;
+  o3.budget = 1;
+  CHECK(tune::GridSearch{}.search(o3).size() == 1);
+  // end to end on the recording runtime: candidates that fail to set up are recorded as invalid
+  auto s = fresh_stream();
+  bench::BenchOptions bo;
+  bo.warmup = std::chrono::milliseconds(0);
+  bo.rep = std::chrono::milliseconds(1);
+  bo.min_reps = 2;
+  bo.max_reps = 2;
+  bo.clear_l2 = false;
+  std::string log = "/tmp/cutile_tune_test.jsonl";
+  remove(log.c_str());
+  auto run = [&] {
+    return tune::Autotuner("unit").configs({a, b, c}).bench_options(bo).log(log)
+        .prune([](const Config& cfg) { return *cfg.integer("bm") >= 128; })
+        .run(s, [&](const std::shared_ptr<Stream>&, const Config& cfg) -> Result<bench::BenchFn> {
+          if (*cfg.integer("bm") == 256) return DeviceError::launch("tile too large");
+          return bench::BenchFn([](const std::shared_ptr<Stream>&) { return ok(); });
+        }).unwrap();
+  };
+  auto out = run();
+  CHECK(out.best && out.best->id == a.id && out.trials.size() == 2);
+  auto out2 = run();  // resumed from the log: the measured candidate is not measured again
+  CHECK(out2.best->id == a.id);
+  auto variants = tune::variant_configs("gemm", "256x256");
+  CHECK(variants.size() >= 3);
+}
+
+int main(int argc, char** argv) {
+  setenv("CUTILE_ASYNC_SPIN_BUDGET_US", "0", 1);
+  if (cutile_testing_use_fake_hip(1) != CUTILE_SUCCESS) return 2;
+  return run_all_tests(argc, argv);
+}
