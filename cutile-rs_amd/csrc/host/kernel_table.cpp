@@ -81,16 +81,18 @@ std::vector<KernelEntry> build_table() {
       add("convert", keep(std::string(s) + "_" + d), keep(std::string("convert_entry__") + s + "_" + d),
           IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, s, 0, 1);
 
-  // ---- row-wise (256 threads; capacity = elements of one segment held in registers) ----
+  // ---- row-wise (256 threads; capacity = elements of one segment held in registers;
+  //      tile[2] = 16-byte vectors per lane, tile[3] = wavefronts per segment) ----
   struct RowVariant { int wpr, vpl; };
-  static const RowVariant kRow[] = {{1, 1}, {1, 2}, {1, 4}, {1, 8}, {1, 16}, {2, 8}, {4, 4}, {4, 8}, {4, 16}};
+  static const RowVariant kRow[] = {{1, 1}, {1, 2}, {1, 4}, {1, 8}, {1, 16}, {2, 2}, {2, 4}, {2, 8},
+                                    {4, 1}, {4, 2}, {4, 4}, {4, 8}, {4, 16}};
   for (auto rv : kRow) {
     std::string v = "w" + std::to_string(rv.wpr) + "v" + std::to_string(rv.vpl);
-    add("rms_norm_f16", keep(v), keep("rms_norm_f16_entry__" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f16",
+    add("rms_norm_f16", keep(v), keep("rms_norm_f16_entry__" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f16",
         (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
-    add("softmax", keep("f16_" + v), keep("softmax_entry__f16_" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f16",
+    add("softmax", keep("f16_" + v), keep("softmax_entry__f16_" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f16",
         (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
-    add("softmax", keep("f32_" + v), keep("softmax_entry__f32_" + v), IMG_ROWWISE, 256, 0, 0, 0, 0, rv.wpr, "f32",
+    add("softmax", keep("f32_" + v), keep("softmax_entry__f32_" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f32",
         (int64_t)rv.wpr * 64 * rv.vpl * 4, 2);
   }
   add("rms_norm_f16", "generic", "rms_norm_f16_entry__generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);

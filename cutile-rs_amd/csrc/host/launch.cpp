@@ -31,6 +31,19 @@ cutile_status_t current_device(cutile_device_t* device) {
   return cutile_device_get(ord, device);
 }
 
+cutile_status_t compute_units(cutile_device_t device, int* count) {
+  CUTILE_REQUIRE(device && count, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  std::lock_guard<std::mutex> lock(device->mutex);
+  if (device->compute_units <= 0) {
+    CUTILE_API_OR_RETURN(api);
+    int v = 0;
+    CUTILE_HIP_OR_RETURN(api, hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device->ordinal));
+    device->compute_units = v;
+  }
+  *count = device->compute_units;
+  return CUTILE_SUCCESS;
+}
+
 namespace {
 
 struct DTypeInfo {
@@ -183,6 +196,7 @@ struct Resolved {
   const KernelEntry* entry = nullptr;
   hipFunction_t fn = nullptr;
   uint32_t tile_grid[3] = {0, 0, 0};
+  cutile_device_t device = nullptr;
 };
 
 // Infers/validates the tile grid from the output partition and the caller's
@@ -213,9 +227,8 @@ cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* 
   r->entry = find_entry(function, want);
   CUTILE_REQUIRE(r->entry, CUTILE_ERR_KERNEL_NOT_FOUND, "no variant '%s' of kernel '%s'; available: %s",
                  want.c_str(), function, list_variants(function).c_str());
-  cutile_device_t dev = nullptr;
-  if (cutile_status_t s = current_device(&dev)) return s;
-  return load_entry(dev, r->entry, &r->fn);
+  if (cutile_status_t s = current_device(&r->device)) return s;
+  return load_entry(r->device, r->entry, &r->fn);
 }
 
 uint32_t div_up(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
@@ -551,7 +564,10 @@ cutile_status_t cutile_launch_convert(cutile_stream_t stream, const cutile_tenso
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
-// Row-wise kernels: variants that hold a whole segment in registers, smallest first.
+// Row-wise kernels: variants that hold a whole segment in registers, best first.
+// Measured on MI355X: up to 4 vectors (64 bytes) per lane stream at full rate, so
+// among those the smallest capacity wins and wider segments are split over more
+// wavefronts; only segments too long for that take more vectors per lane.
 static std::vector<std::string> fitting_row_variants(const char* fn_name, const std::string& prefix, int64_t seg_len) {
   std::vector<const KernelEntry*> fit;
   for (const auto& e : kernel_table())
@@ -559,12 +575,37 @@ static std::vector<std::string> fitting_row_variants(const char* fn_name, const 
         strncmp(e.variant, prefix.c_str(), prefix.size()) == 0)
       fit.push_back(&e);
   std::stable_sort(fit.begin(), fit.end(), [](const KernelEntry* a, const KernelEntry* b) {
+    const int va = std::max(a->tile[2], 4), vb = std::max(b->tile[2], 4);
+    if (va != vb) return va < vb;
     if (a->capacity != b->capacity) return a->capacity < b->capacity;
     return a->tile[3] < b->tile[3];  // fewer wavefronts per segment first
   });
   std::vector<std::string> names;
   for (auto* e : fit) names.push_back(e->variant);
   return names;
+}
+
+// Launch grid of a row-wise kernel over `segments` tile rows: register-resident
+// variants take 4 / WPR segments per workgroup, the any-layout ones walk the
+// segments with a grid stride.
+static void row_launch_grid(const KernelEntry* e, uint64_t segments, uint32_t grid[3]) {
+  grid[0] = grid[1] = grid[2] = 1;
+  if (e->capacity <= 0)
+    grid[0] = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(segments, 1), 1u << 20);
+  else
+    grid[0] = std::max<uint32_t>(1, div_up(segments, 4 / e->tile[3]));
+}
+
+// RMSNorm moves every byte exactly once, and with all 8 workgroups a compute unit
+// can hold resident far more rows are in flight than HBM needs, which costs
+// bandwidth (measured: 3-6 % at N >= 8192).  Unused dynamic LDS caps residency at
+// about 96 KiB of rows in flight per compute unit, never below 5 workgroups.
+static uint32_t rms_norm_residency_lds(const KernelEntry* e, int32_t n) {
+  if (e->capacity <= 0) return 0;
+  const uint64_t bytes_per_wg = (uint64_t)(4 / e->tile[3]) * (uint64_t)n * 2;
+  const uint64_t wgs = std::min<uint64_t>(8, std::max<uint64_t>(5, (96 * 1024 + bytes_per_wg / 2) / bytes_per_wg));
+  if (wgs >= 8) return 0;
+  return (uint32_t)(160 * 1024 / wgs - 1024);
 }
 
 cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x,
@@ -595,7 +636,7 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
                       x->strides[0] % 8 == 0 && ot.strides[0] % 8 == 0 && aligned16(x->ptr) && aligned16(ot.ptr) &&
                       aligned16(w->ptr);
   std::vector<std::string> acceptable;
-  if (vec_ok) acceptable = fitting_row_variants("rms_norm_f16", "w", n);
+  if (vec_ok) acceptable = fitting_row_variants("rms_norm_f16", "", n);
   acceptable.push_back("generic");
   Resolved res;
   if (cutile_status_t s = resolve_entry("rms_norm_f16", opts, acceptable[0], acceptable, &res)) return s;
@@ -607,14 +648,9 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
   args.push_val<float>(eps);
   args.push_tile_grid(tg);
   const uint64_t rows = std::min<uint64_t>(tg[0], ot.shape[0]);
-  uint32_t grid[3] = {1, 1, 1};
-  if (res.entry->capacity > 0) {
-    const int rows_per_wg = 4 / res.entry->tile[3];
-    grid[0] = div_up(rows, rows_per_wg);
-  } else {
-    grid[0] = (uint32_t)std::min<uint64_t>(rows, 1u << 20);
-  }
-  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+  uint32_t grid[3];
+  row_launch_grid(res.entry, rows, grid);
+  return launch_packed(res.fn, grid, res.entry->block, rms_norm_residency_lds(res.entry, n), stream, args);
 }
 
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
@@ -645,11 +681,8 @@ cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tenso
   args.push_partition(*y);
   args.push_tile_grid(tg);
   const uint64_t segments = rows * tg[1];
-  uint32_t grid[3] = {1, 1, 1};
-  if (res.entry->capacity > 0)
-    grid[0] = div_up(segments, 4 / res.entry->tile[3]);
-  else
-    grid[0] = (uint32_t)std::min<uint64_t>(segments, 1u << 20);
+  uint32_t grid[3];
+  row_launch_grid(res.entry, segments, grid);
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

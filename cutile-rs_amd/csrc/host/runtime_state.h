@@ -21,6 +21,7 @@ struct cutile_device {
   std::mutex mutex;
   std::vector<hipStream_t> idle_streams;  // released streams, reused before creating new ones
   uint64_t streams_created = 0;
+  int compute_units = 0;  // filled on first use by compute_units()
   // Code objects of the kernel table loaded on this device: image id -> module.
   std::map<int, cutile_module*> table_modules;
   // Resolved functions: symbol -> hipFunction_t.
@@ -35,5 +36,7 @@ void reset_runtime_for_testing();
 void reset_async_runtime_for_testing();
 // Device the calling thread is bound to (hipGetDevice), as a handle.
 cutile_status_t current_device(cutile_device_t* device);
+// Compute units of the device (cached).
+cutile_status_t compute_units(cutile_device_t device, int* count);
 
 }  // namespace cutile

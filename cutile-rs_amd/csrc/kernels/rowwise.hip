@@ -292,7 +292,11 @@ RMS_NORM_KERNEL(1, 2)
 RMS_NORM_KERNEL(1, 4)
 RMS_NORM_KERNEL(1, 8)
 RMS_NORM_KERNEL(1, 16)
+RMS_NORM_KERNEL(2, 2)
+RMS_NORM_KERNEL(2, 4)
 RMS_NORM_KERNEL(2, 8)
+RMS_NORM_KERNEL(4, 1)
+RMS_NORM_KERNEL(4, 2)
 RMS_NORM_KERNEL(4, 4)
 RMS_NORM_KERNEL(4, 8)
 RMS_NORM_KERNEL(4, 16)
@@ -320,7 +324,11 @@ extern "C" __global__ void __launch_bounds__(kThreads)
   SOFTMAX_KERNEL(T, NAME, 1, 4)   \
   SOFTMAX_KERNEL(T, NAME, 1, 8)   \
   SOFTMAX_KERNEL(T, NAME, 1, 16)  \
+  SOFTMAX_KERNEL(T, NAME, 2, 2)   \
+  SOFTMAX_KERNEL(T, NAME, 2, 4)   \
   SOFTMAX_KERNEL(T, NAME, 2, 8)   \
+  SOFTMAX_KERNEL(T, NAME, 4, 1)   \
+  SOFTMAX_KERNEL(T, NAME, 4, 2)   \
   SOFTMAX_KERNEL(T, NAME, 4, 4)   \
   SOFTMAX_KERNEL(T, NAME, 4, 8)   \
   SOFTMAX_KERNEL(T, NAME, 4, 16)
