@@ -167,7 +167,7 @@ class Gemm(Workload):
         self.s = s
         self.name = f"gemm_bf16_{s}"
         self.work = 2.0 * s ** 3
-        self.config = {"workload": f"GEMM bf16 M=N=K={s}, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 out",
+        self.config = {"workload": f"GEMM bf16 M=N=K={s}, z += A·B, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 z",
                        "tile": "256x256x64"}
 
     def setup(self, ct, torch, oracle, dev):
@@ -182,11 +182,16 @@ class Gemm(Workload):
         self.zp = ct.partition(self.z, list(self.tile))
 
     def launch(self):
-        self.ct.gemm(self.zp, self.a, self.b, self.s, accumulate=False)
+        # z is read as the initial accumulator and written back, like the reference's
+        # benchmark kernel (cutile-benchmarks/benches/gemm.rs:34-40: z.load(); mma...; z.store()).
+        self.ct.gemm(self.zp, self.a, self.b, self.s, accumulate=True)
 
     def cpu_baseline(self, oracle, np, torch):
         rng = np.random.default_rng(7)
         rows = np.sort(rng.choice(self.s, size=1024 if self.s >= 8192 else 512, replace=False)).astype(np.int64)
+        self.z.zero_()          # the timed launches accumulated into z: one launch from zero for the comparison
+        self.launch()
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         ref = oracle.gemm_bf16(self.ab, self.bb, rows=rows, f32out=True)
         dt = time.perf_counter() - t0

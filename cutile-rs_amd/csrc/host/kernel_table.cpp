@@ -103,13 +103,17 @@ std::vector<KernelEntry> build_table() {
   auto gemm = [&](const char* dtype, int bm, int bn, int bk, int wvm, int wvn, const char* kind = "w") {
     std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" +
                     std::to_string(bk) + "_" + kind + std::to_string(wvm) + "x" + std::to_string(wvn);
-    add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64),
-        (uint32_t)(2 * (bm * bk + bk * bn) * 2), bm, bn, bk, 0, dtype, 0, 2);
+    // "r" = ring of three x stages and two y stages, the others hold two stages of each
+    const uint32_t lds = kind[0] == 'r' ? (uint32_t)((3 * bm * bk + 2 * bk * bn) * 2) : (uint32_t)(2 * (bm * bk + bk * bn) * 2);
+    add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64), lds, bm, bn, bk, 0, dtype, 0, 2);
   };
   // first entry of a tile shape = default variant; "d" = global->LDS direct, pipelined
-  gemm("bf16", 256, 256, 64, 2, 4, "d");
   gemm("bf16", 256, 256, 64, 4, 2, "d");
+  gemm("bf16", 256, 256, 64, 2, 4, "d");
   gemm("bf16", 128, 128, 64, 2, 2, "d");
+  gemm("bf16", 256, 256, 64, 4, 2, "r");
+  gemm("bf16", 256, 256, 64, 2, 4, "r");
+  gemm("bf16", 128, 128, 64, 2, 2, "r");
   gemm("bf16", 256, 256, 64, 4, 2);
   gemm("bf16", 256, 256, 64, 2, 4);
   gemm("bf16", 256, 256, 64, 2, 2);

@@ -716,9 +716,12 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
                  "gemm: precompiled variants need row-major operands with unit inner stride, 16-byte aligned rows "
                  "and K, N multiples of 8");
   const std::string dt = zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
+  // The ring-pipelined variants ("_r") fetch whole K tiles only.
+  const int32_t k_valid = std::min(std::min(x->shape[1], y->shape[0]), k_total);
   std::vector<std::string> acceptable;
   for (const auto& e : kernel_table())
-    if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn)
+    if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
+        (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
       acceptable.push_back(e.variant);
   CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
                  "no precompiled variant of gemm<%s, %d, %d, %d>; available: %s", dt.c_str(), bm, bn, bk_user,

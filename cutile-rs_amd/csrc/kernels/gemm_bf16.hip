@@ -259,6 +259,87 @@ struct Gemm {
 };
 
 
+// Epilogue shared by the pipelined variants: accumulators -> z through LDS.
+// In the MFMA layout a lane owns 4 consecutive columns of one row, so a direct
+// store touches 32 rows with 8 or 16 bytes each and every 128-byte line of z is
+// written in 8 pieces.  Staged through LDS (f32, one 32-row band of the
+// wavefront's sub-tile at a time, wavefront-private so no barrier is needed), the
+// same data leaves as 16-byte stores with consecutive lanes on consecutive
+// columns: whole lines.  `accumulate` adds the old z in f32 before the single
+// rounding, as the tile program does (acc = z.load(); ...; z.store(acc)).
+// `stage` is this wavefront's private region of kEpilogueBytesPerWave<WN> bytes.
+// Rows are WN*4 bytes; 16-byte chunk c of row r sits at chunk c ^ (r & 15), so the 16
+// rows of one write pass fall on distinct banks.
+template <int WN>
+constexpr int kEpilogueBytesPerWave = 32 * WN * 4;
+
+template <int TM, int TN, typename OutT>
+__device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
+                                                  int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
+                                                  int lane, int32_t accumulate) {
+  constexpr int WN = TN * 32;
+  constexpr int PITCH = WN * 4;
+  constexpr int COLS_PER_LANE = sizeof(OutT) == 2 ? 8 : 4;      // 16 bytes of output per lane
+  constexpr int LANES_PER_ROW = WN / COLS_PER_LANE;
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  const int l32 = lane & 31, khalf = lane >> 5;
+  const int rd_row = lane / LANES_PER_ROW, rd_col = (lane % LANES_PER_ROW) * COLS_PER_LANE;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    // write this band in the MFMA layout
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        f32x4 v = {acc[tn][tm][q * 4 + 0], acc[tn][tm][q * 4 + 1], acc[tn][tm][q * 4 + 2], acc[tn][tm][q * 4 + 3]};
+        *reinterpret_cast<f32x4*>(stage + l32 * PITCH + (((tn * 8 + q * 2 + khalf) ^ (l32 & 15)) << 4)) = v;
+      }
+    // read it back row-contiguous and store
+#pragma unroll
+    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+      const int r = pass * ROWS_PER_PASS + rd_row;
+      const int32_t gr = wave_row0 + tm * 32 + r, gc = wave_col0 + rd_col;
+      const unsigned char* src = stage + r * PITCH;
+      f32x4 lo = *reinterpret_cast<const f32x4*>(src + (((rd_col >> 2) ^ (r & 15)) << 4));
+      if constexpr (sizeof(OutT) == 2) {
+        f32x4 hi = *reinterpret_cast<const f32x4*>(src + ((((rd_col >> 2) + 1) ^ (r & 15)) << 4));
+        if (gr < zM && gc < zN) {   // zN is a multiple of 4: a lane's 8 columns are all, or the first 4, inside
+          OutT* dst = zp + (int64_t)gr * ldz + gc;
+          const bool full = gc + 8 <= zN;
+          if (accumulate) {
+            u32x2 o0 = *reinterpret_cast<const u32x2*>(dst);
+            lo[0] += __builtin_bit_cast(float, o0.x << 16);
+            lo[1] += __builtin_bit_cast(float, o0.x & 0xffff0000u);
+            lo[2] += __builtin_bit_cast(float, o0.y << 16);
+            lo[3] += __builtin_bit_cast(float, o0.y & 0xffff0000u);
+            if (full) {
+              u32x2 o1 = *reinterpret_cast<const u32x2*>(dst + 4);
+              hi[0] += __builtin_bit_cast(float, o1.x << 16);
+              hi[1] += __builtin_bit_cast(float, o1.x & 0xffff0000u);
+              hi[2] += __builtin_bit_cast(float, o1.y << 16);
+              hi[3] += __builtin_bit_cast(float, o1.y & 0xffff0000u);
+            }
+          }
+          if (full) {
+            u32x4 o = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
+                       pack_bf16x2(hi[2], hi[3])};
+            *reinterpret_cast<u32x4*>(dst) = o;
+          } else {
+            u32x2 o = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+            *reinterpret_cast<u32x2*>(dst) = o;
+          }
+        }
+      } else {
+        if (gr < zM && gc < zN) {
+          OutT* dst = zp + (int64_t)gr * ldz + gc;
+          if (accumulate) lo += *reinterpret_cast<const f32x4*>(dst);
+          *reinterpret_cast<f32x4*>(dst) = lo;
+        }
+      }
+    }
+  }
+}
+
 // ---- pipelined variant: global -> LDS without passing through registers ------------------
 // Differences from Gemm above:
 //  * tiles are fetched with buffer loads that write straight into LDS (16 bytes
@@ -408,10 +489,72 @@ struct GemmDirect {
       if (k_tiles > 1) fetch_tile(stage1, BK);
       read_frags(stage0, 0, f0);
     }
-    // One K tile: `cur` is being multiplied, `nxt` holds (or is receiving) tile kt+1.
-    // sched_barrier(0) pins the order "issue the next operand reads, then the MFMA
-    // block": a wavefront issues in order and each MFMA holds the issue slot until
-    // the matrix pipe accepts it, so reads placed after a block would start late.
+
+    // ---- steady state: one memory instruction group per MFMA ----------------------------
+    // A wavefront issues in order and an MFMA holds the issue slot until the matrix
+    // pipe accepts it, so whatever follows a run of MFMAs starts late and whatever
+    // precedes it delays the pipe.  Operand reads (one MFMA block ahead) and the
+    // refill of the stage just released are therefore dealt out between the MFMAs,
+    // at most two per MFMA; sched_barrier(0) after every step keeps that order.
+    constexpr int NB = TM * TN;          // MFMAs per block (one 16-wide K step)
+    constexpr int NR = TM + TN;          // operand fragments per block, issue order b0, a0..a(TM-1), b1..
+    auto read_operand = [&](const unsigned char* stage, int ks, Frags& f, int r) {
+      if (r >= 1 && r <= TM) {
+        f.a[r - 1] = *reinterpret_cast<const bf16x8*>(stage + a_addr[r - 1][ks]);
+      } else {
+        const int tn = r == 0 ? 0 : r - TM;
+        const unsigned char* p = stage + b_addr[tn] + ks * 16 * (BN * 2);
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 4 * (BN * 2)));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        f.b[tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+    auto fetch_one = [&](unsigned char* stage, int32_t k0, int i) {
+      if (i < kAInstr)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                                 a_goff[i], k0 * 2, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(stage + kABytes + (wave * kBInstr + (i - kAInstr)) * 1024),
+                                                 16, b_goff[i - kAInstr], k0 * ldb * 2, 0, 0);
+    };
+    // MFMAs of one block on `use`, with the fragments of (rd_stage, rd_ks) read into
+    // `into` during the first READ_SLOTS MFMAs and, if REFILL, tile k0 fetched into
+    // `fill` during the first FETCH_SLOTS.
+    constexpr int READ_SLOTS = NB / 2 > 0 ? NB / 2 : 1;
+    constexpr int NF = kAInstr + kBInstr;
+    constexpr int FETCH_SLOTS = NB / 2 > 0 ? NB / 2 : 1;
+    auto block = [&](const unsigned char* rd_stage, int rd_ks, Frags& into, const Frags& use, bool refill,
+                     unsigned char* fill, int32_t k0) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        if (refill) {
+#pragma unroll
+          for (int i = 0; i < NF; ++i)
+            if (i * FETCH_SLOTS / NF == j) fetch_one(fill, k0, i);
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+          if (r * READ_SLOTS / NR == j) read_operand(rd_stage, rd_ks, into, r);
+        acc[j / TM][j % TM] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    auto k_tile_fast = [&](unsigned char* cur, unsigned char* nxt, int kt) {
+      block(cur, 1, f1, f0, false, nullptr, 0);
+      block(cur, 2, f0, f1, false, nullptr, 0);
+      block(cur, 3, f1, f0, false, nullptr, 0);
+      // Hand-over: all of `cur` is in registers, this wavefront's share of tile
+      // kt+1 has landed in `nxt`.
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      block(nxt, 0, f0, f1, true, cur, (kt + 2) * BK);
+    };
+
+    // One K tile, any position: `cur` is being multiplied, `nxt` holds (or is
+    // receiving) tile kt+1.  Used for the last tiles, where the refill may be short
+    // or absent.
     auto k_tile = [&](unsigned char* cur, unsigned char* nxt, int kt) {
       read_frags(cur, 1, f1);
       __builtin_amdgcn_sched_barrier(0);
@@ -425,8 +568,6 @@ struct GemmDirect {
       __builtin_amdgcn_sched_barrier(0);
       mfma_block(f0);
       __builtin_amdgcn_sched_barrier(0);
-      // Hand-over: this wavefront holds all it needs of `cur`, and its part of
-      // tile kt+1 has landed in `nxt`.
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       if (kt + 2 < k_tiles) fetch_tile(cur, (kt + 2) * BK);
@@ -435,47 +576,263 @@ struct GemmDirect {
       mfma_block(f1);
       __builtin_amdgcn_sched_barrier(0);
     };
-    for (int kt = 0; kt < k_tiles; kt += 2) {
+    // Tiles whose refill (tile kt+2) lies wholly inside K take the fast path.
+    const int fast_end = k_valid / BK - 2;  // kt < fast_end  <=>  (kt + 3) * BK <= k_valid
+    int kt = 0;
+    for (; kt + 1 < fast_end; kt += 2) {
+      k_tile_fast(stage0, stage1, kt);
+      k_tile_fast(stage1, stage0, kt + 1);
+    }
+    for (; kt < k_tiles; kt += 2) {
       k_tile(stage0, stage1, kt);
       if (kt + 1 < k_tiles) k_tile(stage1, stage0, kt + 1);
     }
 
-    OutT* zp = (OutT*)z.ptr;
-    const int32_t ldz = z.strides[0];
-    const int32_t zM = z.shape[0], zN = z.shape[1];
+    // Every wavefront is past its operand reads and every fetch has landed: the
+    // stages are free to carry the output.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    static_assert(kWaves / 2 * kEpilogueBytesPerWave<WN> <= kStageBytes, "the output bands must fit the stages");
+    unsigned char* band = (wave < kWaves / 2 ? stage0 : stage1) + (wave % (kWaves / 2)) * kEpilogueBytesPerWave<WN>;
+    store_tile_staged<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0],
+                                    z.shape[0], z.shape[1], row0 + wm * WM, col0 + wn * WN, lane, accumulate);
+  }
+};
+
+// ---- ring variant: three x stages, two y stages released by halves -----------------------
+// The two-stage pipeline above gives a tile's loads one K tile of time to land,
+// and the matrix pipes were measured waiting on them for about a quarter of the
+// run.  Here every load has at least one and a half K tiles:
+//  * the x tile (K-contiguous rows, consumed by column slices) can only be
+//    released as a whole, so it gets three stages: tile kt+3 is fetched when
+//    tile kt is released, two tiles before its first use;
+//  * the y tile is consumed by rows, so its two stages are released by halves:
+//    K rows 0..31 after the first MFMA block of a tile, K rows 32..63 at the
+//    hand-over before the last block; each half is refilled at once with the
+//    same half of tile kt+2;
+//  * loads complete in issue order, so both barriers of a K tile wait with
+//    vmcnt(kAInstr + kBInstr): exactly the loads needed next have landed, one
+//    tile's worth of younger ones stays in flight;
+//  * fetches past the end of K read zeros through the descriptor's range check,
+//    so the loop has one shape for every tile, including a ragged last one.
+// LDS: 3 * BM*BK*2 + 2 * BK*BN*2 bytes (160 KiB for 256x256).
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+struct GemmRing {
+  static constexpr int BK = 64;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int UB = BN / 8;                         // 16-byte units per y-tile row
+  static constexpr int kAInstr = BM / 8 / kWaves;           // 1 KiB = 8 x-tile rows
+  static constexpr int kBRowsPerInstr = 64 / UB;
+  static constexpr int kBInstr = BK / kBRowsPerInstr / kWaves;
+  static constexpr int kABytes = BM * BK * 2, kBBytes = BK * BN * 2;
+  static constexpr int kLdsBytes = 3 * kABytes + 2 * kBBytes;
+  static_assert(BM % (8 * kWaves) == 0 && BK % (kBRowsPerInstr * kWaves) == 0, "tile must split evenly");
+  static_assert(UB >= 16 && UB <= 64, "y-tile row must be 16..64 units");
+  static_assert(kBInstr % 2 == 0, "each wavefront fetches the same share of both y halves");
+  static_assert(kAInstr + kBInstr <= 15, "the wait count must fit the low vmcnt field");
+
+  __device__ static __forceinline__ int a_lds_off(int r, int u) { return r * (BK * 2) + ((u ^ ((r >> 1) & 7)) << 4); }
+  __device__ static __forceinline__ int b_lds_off(int r, int u) { return r * (BN * 2) + ((u ^ ((r & 3) << 2)) << 4); }
+
+  struct Frags {
+    bf16x8 a[TM], b[TN];
+  };
+
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                             int32_t k_total, const TileGrid& g, int32_t accumulate) {
+    // Separately named stages: the compiler can then tell a refill of one from
+    // operand reads of another and adds no waits of its own.
+    __shared__ __attribute__((aligned(1024))) unsigned char xs0[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs1[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs2[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char ys0a[kBBytes / 2];  // y stage 0, K rows 0..31
+    __shared__ __attribute__((aligned(1024))) unsigned char ys0b[kBBytes / 2];  //            K rows 32..63
+    __shared__ __attribute__((aligned(1024))) unsigned char ys1a[kBBytes / 2];
+    __shared__ __attribute__((aligned(1024))) unsigned char ys1b[kBBytes / 2];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    const int32_t M = x.shape[0], N = y.shape[1];
+    const int32_t lda = x.strides[0], ldb = y.strides[0];
+    const int32_t row0 = pm * BM, col0 = pn * BN;
+    const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)(((int64_t)(M - 1) * lda + x.shape[1]) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)(((int64_t)(y.shape[0] - 1) * ldb + N) * 2));
+    constexpr uint32_t kOob = 0x80000000u;
+
+    // Global side of the fetches (per lane, K tile 0; the K advance is scalar).
+    // y instruction i of this wavefront covers K rows of half i / (kBInstr/2).
+    uint32_t a_goff[kAInstr], b_goff[kBInstr];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-      const int32_t r = row0 + wm * WM + tm * 32 + l32;
-      if (r >= zM) continue;
+    for (int i = 0; i < kAInstr; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_goff[i] = (row0 + r < M) ? (uint32_t)(((int64_t)(row0 + r) * lda + u * 8) * 2) : kOob;
+    }
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
+    for (int i = 0; i < kBInstr; ++i) {
+      const int r = (i * kWaves + wave) * kBRowsPerInstr + lane / UB;
+      const int u = (lane % UB) ^ ((r & 3) << 2);
+      b_goff[i] = (col0 + u * 8 < N) ? (uint32_t)(((int64_t)r * ldb + col0 + u * 8) * 2) : kOob;
+    }
+    // K is a whole number of tiles here (the launcher sends ragged K to the
+    // two-stage variant), so a tile is either wholly inside K or wholly beyond it;
+    // beyond it every lane's offset is out of range and the fetch reads zeros.
+    auto fetch_a = [&](unsigned char* stage, int32_t k0, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                               k0 < k_valid ? a_goff[i] : kOob, k0 * 2, 0, 0);
+    };
+    // `half` = the y half-stage receiving K rows 32*h..32*h+31, h = i / (kBInstr/2)
+    auto fetch_b = [&](unsigned char* half, int32_t k0, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(half + ((i % (kBInstr / 2)) * kWaves + wave) * 1024),
+                                               16, k0 < k_valid ? b_goff[i] : kOob, k0 * ldb * 2, 0, 0);
+    };
+
+    // LDS side of the operand reads (byte offsets inside a stage).
+    const int l32 = lane & 31, khalf = lane >> 5;
+    const int grp = lane >> 4, l16 = lane & 15;
+    const int tr_row = l16 >> 2, tr_col = (l16 & 3) * 4;
+    int a_addr[TM][4], b_addr[TN];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int32_t c = col0 + wn * WN + tn * 32 + q * 8 + khalf * 4;
-          if (c >= zN) continue;
-          OutT* dst = zp + (int64_t)r * ldz + c;
-          float v0 = acc[tn][tm][q * 4 + 0], v1 = acc[tn][tm][q * 4 + 1];
-          float v2 = acc[tn][tm][q * 4 + 2], v3 = acc[tn][tm][q * 4 + 3];
-          if constexpr (sizeof(OutT) == 2) {
-            if (accumulate) {
-              u32x2 old = *reinterpret_cast<const u32x2*>(dst);
-              v0 += __builtin_bit_cast(float, old.x << 16);
-              v1 += __builtin_bit_cast(float, old.x & 0xffff0000u);
-              v2 += __builtin_bit_cast(float, old.y << 16);
-              v3 += __builtin_bit_cast(float, old.y & 0xffff0000u);
-            }
-            u32x2 o;
-            o.x = pack_bf16x2(v0, v1);
-            o.y = pack_bf16x2(v2, v3);
-            *reinterpret_cast<u32x2*>(dst) = o;
-          } else {
-            f32x4 o = {v0, v1, v2, v3};
-            if (accumulate) o += *reinterpret_cast<const f32x4*>(dst);
-            *reinterpret_cast<f32x4*>(dst) = o;
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) a_addr[tm][ks] = a_lds_off(wm * WM + tm * 32 + l32, ks * 2 + khalf);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int n = wn * WN + tn * 32 + (grp & 1) * 16 + tr_col;
+      const int kr = (grp >> 1) * 8 + tr_row;  // (kr & 3) does not depend on ks: the swizzle term is fixed
+      b_addr[tn] = b_lds_off(kr, n >> 3) + (n & 7) * 2;
+    }
+    constexpr int NB = TM * TN;  // MFMAs per block (one 16-wide K step)
+    constexpr int NR = TM + TN;  // operand fragments per block, issue order b0, a0..a(TM-1), b1..
+    // `yh` = the y half-stage holding K step ks (rows 16*ks..16*ks+15 of the tile)
+    auto read_operand = [&](const unsigned char* xs, const unsigned char* yh, int ks, Frags& f, int r) {
+      if (r >= 1 && r <= TM) {
+        f.a[r - 1] = *reinterpret_cast<const bf16x8*>(xs + a_addr[r - 1][ks]);
+      } else {
+        const int tn = r == 0 ? 0 : r - TM;
+        const unsigned char* p = yh + b_addr[tn] + (ks & 1) * 16 * (BN * 2);
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 4 * (BN * 2)));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        f.b[tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
+
+    // One MFMA block on `use`.  Dealt out between its MFMAs, at most two per
+    // MFMA and in this order: refill instructions first..last of the x stage
+    // `fill_x` (if any) and of the y stage `fill_y` (instructions fb0..fb1-1),
+    // then the reads of (rd_x, rd_y, rd_ks) into `into`.  A wavefront issues in
+    // order and an MFMA holds the issue slot until the matrix pipe takes it, so
+    // memory work placed after a run of MFMAs would start late; sched_barrier(0)
+    // after every step keeps the order written here.
+    constexpr int SLOTS = NB / 2 > 0 ? NB / 2 : 1;
+    auto block = [&](const Frags& use, const unsigned char* rd_x, const unsigned char* rd_y, int rd_ks, Frags& into,
+                     unsigned char* fill_x, unsigned char* fill_y, int fb0, int fb1, int32_t k0_x, int32_t k0_y) {
+      const int n_fill = (fill_x ? kAInstr : 0) + (fb1 - fb0);
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+#pragma unroll
+        for (int i = 0; i < kAInstr + kBInstr; ++i) {
+          if (i < n_fill && i * SLOTS / n_fill == j) {
+            if (fill_x && i < kAInstr)
+              fetch_a(fill_x, k0_x, i);
+            else
+              fetch_b(fill_y, k0_y, fb0 + i - (fill_x ? kAInstr : 0));
           }
         }
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+          if (r * SLOTS / NR == j) read_operand(rd_x, rd_y, rd_ks, into, r);
+        acc[j / TM][j % TM] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    };
+    // s_waitcnt immediate of gfx9: vmcnt [3:0] (and [15:14]), expcnt [6:4], lgkmcnt [11:8].
+    constexpr int kWaitOlderLoads = (kAInstr + kBInstr) | (7 << 4) | (0 << 8);
+    constexpr int kWaitPrologue = ((2 * kAInstr + 3 * kBInstr / 2) & 15) | (7 << 4) | (0 << 8) | (((2 * kAInstr + 3 * kBInstr / 2) >> 4) << 14);
+
+    const int k_tiles = (k_total + BK - 1) / BK;
+    Frags f0, f1;
+    // Prologue, in the issue order the steady state would have produced.
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs0, 0, i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys0a, 0, i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs1, BK, i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys0b, 0, i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys1a, BK, i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs2, 2 * BK, i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys1b, BK, i);
+    __builtin_amdgcn_s_waitcnt(kWaitPrologue);  // x tile 0 and the first y half of tile 0 have landed
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_operand(xs0, ys0a, 0, f0, r);
+
+    // Tile kt lives in x_cur and the y halves (ya_cur, yb_cur); tile kt+1 in x_nxt, ya_nxt.
+    auto k_tile = [&](unsigned char* x_cur, unsigned char* ya_cur, unsigned char* yb_cur, const unsigned char* x_nxt,
+                      const unsigned char* ya_nxt, int kt) {
+      block(f0, x_cur, ya_cur, 1, f1, nullptr, nullptr, 0, 0, 0, 0);
+      // First y half of tile kt is in registers everywhere; its second half has landed.
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(f1, x_cur, yb_cur, 2, f0, nullptr, ya_cur, 0, kBInstr / 2, 0, (kt + 2) * BK);
+      block(f0, x_cur, yb_cur, 3, f1, nullptr, nullptr, 0, 0, 0, 0);
+      // Hand-over: all of tile kt is in registers; x tile kt+1 and its first y half have landed.
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(f1, x_nxt, ya_nxt, 0, f0, x_cur, yb_cur, kBInstr / 2, kBInstr, (kt + 3) * BK, (kt + 2) * BK);
+    };
+    // The stage names repeat every 6 tiles (3 x stages, 2 y stages).
+    int kt = 0;
+    for (; kt + 6 <= k_tiles; kt += 6) {
+      k_tile(xs0, ys0a, ys0b, xs1, ys1a, kt);
+      k_tile(xs1, ys1a, ys1b, xs2, ys0a, kt + 1);
+      k_tile(xs2, ys0a, ys0b, xs0, ys1a, kt + 2);
+      k_tile(xs0, ys1a, ys1b, xs1, ys0a, kt + 3);
+      k_tile(xs1, ys0a, ys0b, xs2, ys1a, kt + 4);
+      k_tile(xs2, ys1a, ys1b, xs0, ys0a, kt + 5);
     }
+    const int rest = k_tiles - kt;
+    if (rest > 0) k_tile(xs0, ys0a, ys0b, xs1, ys1a, kt);
+    if (rest > 1) k_tile(xs1, ys1a, ys1b, xs2, ys0a, kt + 1);
+    if (rest > 2) k_tile(xs2, ys0a, ys0b, xs0, ys1a, kt + 2);
+    if (rest > 3) k_tile(xs0, ys1a, ys1b, xs1, ys0a, kt + 3);
+    if (rest > 4) k_tile(xs1, ys0a, ys0b, xs2, ys1a, kt + 4);
+    __builtin_amdgcn_s_waitcnt(0);  // trailing (zero-filling) fetches must not outlive the workgroup's LDS
+
+    // Every wavefront is past its operand reads and every fetch has landed: the
+    // stages are free to carry the output (two wavefronts share an x stage, the
+    // last two take the y stages).
+    __syncthreads();
+    static_assert(2 * kEpilogueBytesPerWave<WN> <= kABytes && kEpilogueBytesPerWave<WN> <= kBBytes / 2 && kWaves <= 10,
+                  "the output bands must fit the stages");
+    unsigned char* band = wave < 2 ? xs0 : wave < 4 ? xs1 : wave < 6 ? xs2 : wave == 6 ? ys0a : wave == 7 ? ys0b : wave == 8 ? ys1a : ys1b;
+    if (wave < 6) band += (wave & 1) * kEpilogueBytesPerWave<WN>;
+    store_tile_staged<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0], z.shape[0], z.shape[1], row0 + wm * WM,
+                                    col0 + wn * WN, lane, accumulate);
   }
 };
 
@@ -509,3 +866,14 @@ GEMM_KERNEL(bf16f32_256x256x64_w2x2, 256, 256, 64, 2, 2, float)
 GEMM_DIRECT_KERNEL(bf16_256x256x64_d4x2, 256, 256, 4, 2, __bf16)
 GEMM_DIRECT_KERNEL(bf16_256x256x64_d2x4, 256, 256, 2, 4, __bf16)
 GEMM_DIRECT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)
+
+#define GEMM_RING_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                          \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmRing<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, k, g, accumulate);                          \
+  }
+
+GEMM_RING_KERNEL(bf16_256x256x64_r2x4, 256, 256, 2, 4, __bf16)
+GEMM_RING_KERNEL(bf16_256x256x64_r4x2, 256, 256, 4, 2, __bf16)
+GEMM_RING_KERNEL(bf16_128x128x64_r2x2, 128, 128, 2, 2, __bf16)

@@ -204,7 +204,7 @@ def test_softmax_f32(ct, dev, m, n, bm, bn):
 
 
 # ---- K4: bf16 GEMM --------------------------------------------------------------------------
-GEMM_VARIANTS = ["bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
+GEMM_VARIANTS = ["bf16_256x256x64_r2x4", "bf16_256x256x64_r4x2", "bf16_128x128x64_r2x2", "bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
                  "bf16_128x256x64_w2x2", "bf16_128x128x64_w2x2", "bf16_64x128x64_w2x2"]
 
 
@@ -221,6 +221,34 @@ def test_gemm_bf16_variants(ct, dev, variant):
     assert rel_l2(got, ref) <= 1e-2
     # tighter: bf16 rounding of an f32-accumulated result is within 1 bf16 ulp-ish of the oracle
     np.testing.assert_allclose(got, ref, rtol=1.6e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("variant", ["bf16_256x256x64_r2x4", "bf16_128x128x64_r2x2"])
+@pytest.mark.parametrize("k_tiles", [1, 2, 3, 6, 7, 13])
+def test_gemm_ring_pipeline_every_loop_shape(ct, dev, variant, k_tiles):
+    # the ring pipeline repeats its stage names every 6 K tiles: cover the unrolled
+    # loop, every remainder, and M, N that are not multiples of the tile
+    bm, bn = (int(v) for v in variant.split("_")[1].split("x")[:2])
+    m, n, k = 328, 520, 64 * k_tiles
+    a, b = normal_bf16_bits((m, k), 331 + k_tiles, k ** -0.5), normal_bf16_bits((k, n), 332 + k_tiles, k ** -0.5)
+    z = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    ct.gemm(ct.partition(z, [bm, bn]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=False, variant=variant)
+    sync()
+    ref = oracle.gemm_bf16(a, b, f32out=True)
+    np.testing.assert_allclose(z.float().cpu().numpy(), ref, rtol=1.6e-2, atol=2e-3)
+
+
+def test_gemm_ring_variant_rejects_ragged_k(ct, dev):
+    m = n = 256
+    k = 96
+    x = torch.ones(m, k, dtype=torch.bfloat16, device=dev)
+    y = torch.ones(k, n, dtype=torch.bfloat16, device=dev)
+    z = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ct.CutileError, match="does not fit"):
+        ct.gemm(ct.partition(z, [256, 256]), x, y, k, generics=["bf16", 256, 256, 32], variant="bf16_256x256x64_r2x4")
+    ct.gemm(ct.partition(z, [256, 256]), x, y, k, generics=["bf16", 256, 256, 32])  # falls back to a two-stage variant
+    sync()
+    assert torch.equal(z.float(), torch.full((m, n), float(k), device=dev))
 
 
 def test_gemm_ones_known_answer_non_divisible(ct, dev):
