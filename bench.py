@@ -321,8 +321,8 @@ def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gemm_bf16_8192")
     ap.add_argument("--only", action="store_true", help="measure only --workload (no 'also' list)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / sampled parity leg")

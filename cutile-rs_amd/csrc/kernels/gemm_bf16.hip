@@ -282,8 +282,33 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
   constexpr int COLS_PER_LANE = sizeof(OutT) == 2 ? 8 : 4;      // 16 bytes of output per lane
   constexpr int LANES_PER_ROW = WN / COLS_PER_LANE;
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  constexpr int PASSES = 32 / ROWS_PER_PASS;
   const int l32 = lane & 31, khalf = lane >> 5;
   const int rd_row = lane / LANES_PER_ROW, rd_col = (lane % LANES_PER_ROW) * COLS_PER_LANE;
+  const int32_t gc = wave_col0 + rd_col;
+  const bool col_ok = gc < zN;
+  const bool full = gc + COLS_PER_LANE <= zN;  // zN is a multiple of 4: otherwise exactly the first 4 columns are inside
+  // Old z, all of it requested before anything is waited for.
+  u32x4 old[TM][PASSES];
+  if (accumulate) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int pass = 0; pass < PASSES; ++pass) {
+        const int32_t gr = wave_row0 + tm * 32 + pass * ROWS_PER_PASS + rd_row;
+        old[tm][pass] = u32x4{0, 0, 0, 0};
+        if (gr < zM && col_ok) {
+          const OutT* src = zp + (int64_t)gr * ldz + gc;
+          if (full) {
+            old[tm][pass] = *reinterpret_cast<const u32x4*>(src);
+          } else {
+            u32x2 h = *reinterpret_cast<const u32x2*>(src);
+            old[tm][pass].x = h.x;
+            old[tm][pass].y = h.y;
+          }
+        }
+      }
+  }
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) {
     // write this band in the MFMA layout
@@ -296,45 +321,38 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
       }
     // read it back row-contiguous and store
 #pragma unroll
-    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+    for (int pass = 0; pass < PASSES; ++pass) {
       const int r = pass * ROWS_PER_PASS + rd_row;
-      const int32_t gr = wave_row0 + tm * 32 + r, gc = wave_col0 + rd_col;
+      const int32_t gr = wave_row0 + tm * 32 + r;
       const unsigned char* src = stage + r * PITCH;
       f32x4 lo = *reinterpret_cast<const f32x4*>(src + (((rd_col >> 2) ^ (r & 15)) << 4));
+      const u32x4 o = old[tm][pass];
       if constexpr (sizeof(OutT) == 2) {
         f32x4 hi = *reinterpret_cast<const f32x4*>(src + ((((rd_col >> 2) + 1) ^ (r & 15)) << 4));
-        if (gr < zM && gc < zN) {   // zN is a multiple of 4: a lane's 8 columns are all, or the first 4, inside
+        if (accumulate) {
+          lo[0] += __builtin_bit_cast(float, o.x << 16);
+          lo[1] += __builtin_bit_cast(float, o.x & 0xffff0000u);
+          lo[2] += __builtin_bit_cast(float, o.y << 16);
+          lo[3] += __builtin_bit_cast(float, o.y & 0xffff0000u);
+          hi[0] += __builtin_bit_cast(float, o.z << 16);
+          hi[1] += __builtin_bit_cast(float, o.z & 0xffff0000u);
+          hi[2] += __builtin_bit_cast(float, o.w << 16);
+          hi[3] += __builtin_bit_cast(float, o.w & 0xffff0000u);
+        }
+        if (gr < zM && col_ok) {
           OutT* dst = zp + (int64_t)gr * ldz + gc;
-          const bool full = gc + 8 <= zN;
-          if (accumulate) {
-            u32x2 o0 = *reinterpret_cast<const u32x2*>(dst);
-            lo[0] += __builtin_bit_cast(float, o0.x << 16);
-            lo[1] += __builtin_bit_cast(float, o0.x & 0xffff0000u);
-            lo[2] += __builtin_bit_cast(float, o0.y << 16);
-            lo[3] += __builtin_bit_cast(float, o0.y & 0xffff0000u);
-            if (full) {
-              u32x2 o1 = *reinterpret_cast<const u32x2*>(dst + 4);
-              hi[0] += __builtin_bit_cast(float, o1.x << 16);
-              hi[1] += __builtin_bit_cast(float, o1.x & 0xffff0000u);
-              hi[2] += __builtin_bit_cast(float, o1.y << 16);
-              hi[3] += __builtin_bit_cast(float, o1.y & 0xffff0000u);
-            }
-          }
           if (full) {
-            u32x4 o = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
+            u32x4 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
                        pack_bf16x2(hi[2], hi[3])};
-            *reinterpret_cast<u32x4*>(dst) = o;
+            *reinterpret_cast<u32x4*>(dst) = w;
           } else {
-            u32x2 o = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
-            *reinterpret_cast<u32x2*>(dst) = o;
+            u32x2 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+            *reinterpret_cast<u32x2*>(dst) = w;
           }
         }
       } else {
-        if (gr < zM && gc < zN) {
-          OutT* dst = zp + (int64_t)gr * ldz + gc;
-          if (accumulate) lo += *reinterpret_cast<const f32x4*>(dst);
-          *reinterpret_cast<f32x4*>(dst) = lo;
-        }
+        if (accumulate) lo += __builtin_bit_cast(f32x4, o);
+        if (gr < zM && col_ok) *reinterpret_cast<f32x4*>(zp + (int64_t)gr * ldz + gc) = lo;
       }
     }
   }
