@@ -57,10 +57,9 @@ struct Elem<__bf16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
-    uint32_t a = __builtin_bit_cast(uint32_t, lo), b = __builtin_bit_cast(uint32_t, hi);
-    a += 0x7fffu + ((a >> 16) & 1u);
-    b += 0x7fffu + ((b >> 16) & 1u);
-    return (a >> 16) | (b & 0xffff0000u);
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo, hi}, b2));  // v_cvt_pk_bf16_f32, RNE
   }
 };
 template <>
@@ -71,8 +70,8 @@ struct Elem<_Float16> {
   }
   __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2 v = {(_Float16)lo, (_Float16)hi};
-    return __builtin_bit_cast(uint32_t, v);
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo, hi}, h2));  // v_cvt_pk_f16_f32
   }
 };
 
@@ -227,10 +226,16 @@ struct Fmha {
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[sb][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      // Statistics are kept in the scaled log2 domain: m = c * rowmax(raw).
-      const float m_new = fmaxf(m_i, mx * c);
+      // Statistics are kept in the scaled log2 domain: m = c * rowmax(raw).  The
+      // reference point m only has to bound the exponents, not equal the maximum:
+      // it moves (and the accumulators are rescaled) only when some row's maximum
+      // rose by more than kSlack, so p stays below 2^kSlack and after the first
+      // tiles the rescale is skipped almost always.
+      constexpr float kSlack = 8.0f;
+      const float m_cand = fmaxf(m_i, mx * c);
+      const bool moved = __builtin_amdgcn_ballot_w64(m_cand > m_i + kSlack) != 0;   // wavefront-uniform
+      const float m_new = moved ? m_cand : m_i;
       const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // fully masked so far: keep exp2 finite
-      const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
       float rs = 0.0f;
       vec8 pf[BN / 16];
 #pragma unroll
@@ -252,12 +257,16 @@ struct Fmha {
         }
       }
       rs += __shfl_xor(rs, 32, 64);
-      l_i = l_i * alpha + rs;
-      m_i = m_new;
+      if (moved) {
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+        l_i *= alpha;
 #pragma unroll
-      for (int i = 0; i < DB; ++i)
+        for (int i = 0; i < DB; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+        m_i = m_new;
+      }
+      l_i += rs;
 
       // Oᵀ += V_jᵀ · Pᵀ.  MFMA step t covers kv rows 16t..16t+15 of the tile; slot
       // (half, jj) of a lane's operand is kv = 16t + 8*(jj/4) + 4*half + jj%4, which is
