@@ -125,11 +125,14 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16f32", 256, 256, 64, 2, 2);
 
   // ---- FMHA: LDS = 2 stages x (K tile + V tile) ----
-  auto fmha = [&](const char* dtype, int bm, int bn, int d) {
-    std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" + std::to_string(d);
+  // "_pp": the two wavefronts of a SIMD run half a tile apart (BM = 256 only)
+  auto fmha = [&](const char* dtype, int bm, int bn, int d, const char* suffix = "") {
+    std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" + std::to_string(d) + suffix;
     add("fmha", keep(v), keep("fmha_entry__" + v), IMG_FMHA, (uint32_t)(bm / 32 * 64),
         (uint32_t)(2 * 2 * bn * d * 2), bm, bn, d, 0, dtype, 0, 3);
   };
+  fmha("bf16", 256, 64, 128, "_pp");
+  fmha("f16", 256, 64, 128, "_pp");
   fmha("bf16", 128, 64, 128);
   fmha("bf16", 128, 128, 128);
   fmha("bf16", 256, 64, 128);

@@ -26,6 +26,8 @@
 // matrix work.  One wavefront owns 32 query rows; a workgroup is BM/32 waves.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernel_args.h"
 
 using namespace cutile;
@@ -307,6 +309,336 @@ struct Fmha {
   }
 };
 
+// ---- ping-pong variant (BM = 256, eight wavefronts) --------------------------------------
+// The kernel above keeps all wavefronts of a workgroup in the same phase: they
+// multiply together (matrix pipes busy, vector ALUs idle) and then run the
+// softmax together (the reverse).  Per KV tile a wavefront needs about as many
+// vector-ALU cycles for the softmax as matrix-pipe cycles for its 32 MFMAs, so
+// here the two wavefronts that share a SIMD (w and w+4) run half a tile apart:
+//   interval:        I0      I1      I2          I3          I4
+//   waves 0..3:      S0      soft0   PV0,S1      soft1       PV1,S2 ...
+//   waves 4..7:      -       S0      soft0       PV0,S1      soft1  ...
+// with one workgroup barrier between intervals, so that on every SIMD one
+// wavefront feeds the matrix pipe while the other feeds the vector ALU.
+//  * K and V tiles go global -> LDS directly (16 bytes per lane), two buffers
+//    each; a buffer is refilled in the interval after both halves of the
+//    workgroup have read it and is waited for two intervals later;
+//  * operand fragments are read from LDS three MFMAs ahead of their use;
+//  * the two 32-row blocks of S^T (and the four of O^T) are independent
+//    accumulators and are issued alternately, so no MFMA waits on the previous one;
+//  * the output leaves through LDS as 16-byte stores of whole 256-byte rows.
+template <typename T, int BN, int D>
+struct FmhaPingPong {
+  using E = Elem<T>;
+  using vec8 = typename E::vec8;
+  static constexpr int BM = 256;
+  static constexpr int kWaves = BM / 32;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int kUnitsPerRow = D / 8;
+  static constexpr int kTileBytes = BN * D * 2;
+  static constexpr int kRowsPerInstr = 1024 / (D * 2);
+  static constexpr int kInstr = kTileBytes / 1024 / kWaves;    // direct loads per wavefront per tile
+  static constexpr int SB = BN / 32, DB = D / 32, KS = D / 16, TS = BN / 16;
+  static constexpr int kLdsBytes = 4 * kTileBytes;
+  static_assert(D == 128 && BN % 32 == 0, "tile shape");
+  static_assert(kInstr >= 1 && kTileBytes % (1024 * kWaves) == 0, "tile must split evenly over the workgroup");
+  static_assert(kWaves * 32 * D * 2 <= kLdsBytes, "the output bands must fit the tile buffers");
+
+  // Same layouts as Fmha: K unit u of row r at u ^ (r & 15); V unit u at u ^ ((r & 3) << 2).
+  __device__ static __forceinline__ int k_off(int r, int u) { return r * (D * 2) + ((u ^ (r & 15)) << 4); }
+  __device__ static __forceinline__ int v_off(int r, int u) { return r * (D * 2) + ((u ^ ((r & 3) << 2)) << 4); }
+
+  __device__ static void run(const PartitionArg<3>& out, const TensorArg<4>& q, const TensorArg<4>& k,
+                             const TensorArg<4>& v, float qk_scale, int32_t input_pos,
+                             int32_t group_size, int32_t causal, const TileGrid& g) {
+    // Separately named buffers: the compiler can tell a refill of one from reads of another.
+    __shared__ __attribute__((aligned(1024))) unsigned char kb0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char kb1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char vb0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char vb1[kTileBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool late = wave >= kWaves / 2;   // the half of the workgroup that runs one interval behind
+    const int l32 = lane & 31, half = lane >> 5;
+    const int grp = lane >> 4, l16 = lane & 15;
+
+    const int32_t H = q.shape[1];
+    const int32_t bh = blockIdx.x;
+    const int32_t q_tile = causal ? (int32_t)(g.y - 1 - blockIdx.y) : (int32_t)blockIdx.y;
+    const int32_t batch = bh / H, head = bh % H, kv_head = head / group_size;
+    const int32_t q_len = q.shape[2], k_len = k.shape[2];
+    const int32_t q0 = q_tile * BM + wave * 32;
+
+    const T* qb = (const T*)q.ptr + (int64_t)batch * q.strides[0] + (int64_t)head * q.strides[1];
+    const T* kb = (const T*)k.ptr + (int64_t)batch * k.strides[0] + (int64_t)kv_head * k.strides[1];
+    const T* vb = (const T*)v.ptr + (int64_t)batch * v.strides[0] + (int64_t)kv_head * v.strides[1];
+    const int32_t q_ld = q.strides[2], k_ld = k.strides[2], v_ld = v.strides[2];
+    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qb, (uint32_t)(((int64_t)(q_len - 1) * q_ld + D) * 2));
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kb, (uint32_t)(((int64_t)(k_len - 1) * k_ld + D) * 2));
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vb, (uint32_t)(((int64_t)(k_len - 1) * v_ld + D) * 2));
+    constexpr uint32_t kOob = 0x80000000u;
+
+    vec8 qf[KS];
+    {
+      const int32_t qr = q0 + l32;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint32_t off = qr < q_len ? (uint32_t)(((int64_t)qr * q_ld + ks * 16 + half * 8) * 2) : kOob;
+        qf[ks] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0));
+      }
+    }
+
+    int32_t tc = (k_len + BN - 1) / BN;
+    int32_t mask_start = k_len / BN;
+    if (causal) {
+      const int32_t m_end = input_pos + (q_tile + 1) * BM;
+      mask_start = min((input_pos + q_tile * BM) / BN, k_len / BN);
+      tc = (min(m_end, k_len) + BN - 1) / BN;
+    }
+
+    // Global side of the tile fetches: the LDS side of a direct load is lane
+    // contiguous, so a lane fetches the unit that belongs at its LDS position.
+    int32_t ld_row[kInstr];
+    uint32_t k_goff[kInstr], v_goff[kInstr];
+#pragma unroll
+    for (int i = 0; i < kInstr; ++i) {
+      const int r = (wave * kInstr + i) * kRowsPerInstr + lane / kUnitsPerRow;
+      const int up = lane % kUnitsPerRow;
+      ld_row[i] = r;
+      k_goff[i] = (uint32_t)(((int64_t)r * k_ld + (up ^ (r & 15)) * 8) * 2);
+      v_goff[i] = (uint32_t)(((int64_t)r * v_ld + (up ^ ((r & 3) << 2)) * 8) * 2);
+    }
+    // Tile j of K (V) into `buf`; rows at or beyond k_len, and every row when
+    // !wanted, use an out-of-range offset and read zeros.
+    auto fetch_k = [&](unsigned char* buf, int32_t j, bool wanted = true) {
+      const int32_t row0 = wanted ? j * BN : 0;
+#pragma unroll
+      for (int i = 0; i < kInstr; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (LDS_PTR(void))(buf + (wave * kInstr + i) * 1024), 16,
+                                                 wanted && row0 + ld_row[i] < k_len ? k_goff[i] : kOob,
+                                                 row0 * k_ld * 2, 0, 0);
+    };
+    auto fetch_v = [&](unsigned char* buf, int32_t j) {
+#pragma unroll
+      for (int i = 0; i < kInstr; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (LDS_PTR(void))(buf + (wave * kInstr + i) * 1024), 16,
+                                                 j * BN + ld_row[i] < k_len ? v_goff[i] : kOob, j * BN * v_ld * 2, 0, 0);
+    };
+
+    // LDS side of the operand reads.
+    int k_addr[KS], v_addr[DB];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_addr[ks] = k_off(l32, ks * 2 + half);          // + sb * 32 rows
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int dcol = db * 32 + (grp & 1) * 16 + (l16 & 3) * 4;
+      const int kr = (grp >> 1) * 4 + (l16 >> 2);                                   // + t * 16 (+ 8) rows
+      v_addr[db] = v_off(kr, dcol >> 3) + (dcol & 7) * 2;
+    }
+    auto read_k = [&](const unsigned char* buf, int n) -> vec8 {   // step n of S^T: ks = n / SB, sb = n % SB
+      return *reinterpret_cast<const vec8*>(buf + k_addr[n / SB] + (n % SB) * 32 * (D * 2));
+    };
+    auto read_v = [&](const unsigned char* buf, int n) -> vec8 {   // step n of O^T: t = n / DB, db = n % DB
+      const unsigned char* p = buf + v_addr[n % DB] + (n / DB) * 16 * (D * 2);
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 8 * (D * 2)));
+      return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+
+    f32x16 o_acc[DB], s[SB];
+    vec8 pf[TS];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
+    float m_i = -INFINITY, l_i = 0.0f;
+    const float c = qk_scale * kLog2e;
+    const int32_t q_pos = q0 + l32 + input_pos;
+
+    // Matrix segments.  Fragments are read kAhead steps before the MFMA that uses
+    // them; sched_barrier(0) after every step keeps reads and MFMAs in this order.
+    constexpr int kAhead = 3, kRing = kAhead + 1;
+    constexpr int NS = SB * KS, NO = TS * DB;   // MFMAs of S^T and of O^T per tile
+    // O^T += V_j^T P_j^T from `vbuf`, then (WITH_S) S^T = K_{j+1} Q^T from `kbuf`.
+    auto matrix_segment = [&](const unsigned char* vbuf, const unsigned char* kbuf, auto with_s) {
+      constexpr int total = NO + (decltype(with_s)::value ? NS : 0);
+      vec8 ring[kRing];
+      auto read_step = [&](int n) -> vec8 { return n < NO ? read_v(vbuf, n) : read_k(kbuf, n - NO); };
+#pragma unroll
+      for (int n = 0; n < kAhead; ++n) ring[n % kRing] = read_step(n);
+#pragma unroll
+      for (int n = 0; n < total; ++n) {
+        if (n + kAhead < total) ring[(n + kAhead) % kRing] = read_step(n + kAhead);
+        if (n < NO) {
+          o_acc[n % DB] = E::mfma(ring[n % kRing], pf[n / DB], o_acc[n % DB]);
+        } else {
+          const int m = n - NO;
+          if (m < SB) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[m % SB][e] = 0.0f;
+          }
+          s[m % SB] = E::mfma(ring[n % kRing], qf[m / SB], s[m % SB]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // S^T = K_0 Q^T alone (first segment).
+    auto first_segment = [&](const unsigned char* kbuf) {
+      vec8 ring[kRing];
+#pragma unroll
+      for (int n = 0; n < kAhead; ++n) ring[n % kRing] = read_k(kbuf, n);
+#pragma unroll
+      for (int m = 0; m < NS; ++m) {
+        if (m + kAhead < NS) ring[(m + kAhead) % kRing] = read_k(kbuf, m + kAhead);
+        if (m < SB) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) s[m % SB][e] = 0.0f;
+        }
+        s[m % SB] = E::mfma(ring[m % kRing], qf[m / SB], s[m % SB]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // Softmax segment of tile j: s -> pf, running statistics, rescale when the reference point moves.
+    auto softmax_segment = [&](int32_t j) {
+      if (j >= mask_start) {
+#pragma unroll
+        for (int sb = 0; sb < SB; ++sb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            int32_t kv = j * BN + sb * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+            bool visible = kv < k_len && (!causal || q_pos >= kv);
+            s[sb][e] = visible ? s[sb][e] : -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int sb = 0; sb < SB; ++sb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[sb][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      constexpr float kSlack = 8.0f;   // see Fmha: the reference point moves only on a rise above 2^kSlack
+      const float m_cand = fmaxf(m_i, mx * c);
+      const bool moved = __builtin_amdgcn_ballot_w64(m_cand > m_i + kSlack) != 0;
+      const float m_new = moved ? m_cand : m_i;
+      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+      float rs = 0.0f;
+#pragma unroll
+      for (int sb = 0; sb < SB; ++sb) {
+        float p[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[sb][e], c, -m_use));
+          rs += p[e];
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          u32x4 w;
+          w.x = E::pack2(p[hh * 8 + 0], p[hh * 8 + 1]);
+          w.y = E::pack2(p[hh * 8 + 2], p[hh * 8 + 3]);
+          w.z = E::pack2(p[hh * 8 + 4], p[hh * 8 + 5]);
+          w.w = E::pack2(p[hh * 8 + 6], p[hh * 8 + 7]);
+          pf[sb * 2 + hh] = __builtin_bit_cast(vec8, w);
+        }
+      }
+      rs += __shfl_xor(rs, 32, 64);
+      if (moved) {
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+        l_i *= alpha;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+        m_i = m_new;
+      }
+      l_i += rs;
+    };
+    auto interval_end = [&]() {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto wait_fetches = [&]() { __builtin_amdgcn_s_waitcnt(0); };   // own fetches landed, own LDS reads done
+    // The two halves of the workgroup run the same segments one interval apart;
+    // each gets its own straight-line copy of the loop.  Tile j: K_j in kc, V_j in
+    // vc, K_{j+1} in kn; refills K_{j+2} -> kc and V_{j+1} -> vn are issued in the
+    // interval after both halves have read those buffers (the early half at the
+    // start of its matrix segment, the late half at the start of its softmax) and
+    // waited for at the end of the following interval.
+    auto pipeline = [&](auto late_tag) {
+      constexpr bool LATE = decltype(late_tag)::value;
+      auto tile = [&](int32_t j, unsigned char* kc, unsigned char* kn, unsigned char* vc, unsigned char* vn,
+                      auto last_tag) {
+        constexpr bool LAST = decltype(last_tag)::value;
+        auto refill = [&]() {
+          fetch_k(kc, j + 2, j + 2 < tc);
+          fetch_v(vn, j + 1);
+        };
+        if (LATE && !LAST) refill();
+        softmax_segment(j);
+        if (!LATE) wait_fetches();
+        interval_end();
+        if (!LATE && !LAST) refill();
+        matrix_segment(vc, kn, std::integral_constant<bool, !LAST>{});
+        if (LATE && !LAST) wait_fetches();
+        interval_end();
+      };
+      fetch_k(kb1, 1, tc > 1);
+      fetch_v(vb0, 0);
+      if (LATE) interval_end();          // this half sits out the first interval
+      first_segment(kb0);
+      if (LATE) wait_fetches();
+      interval_end();
+      int32_t j = 0;
+      for (; j + 2 < tc; j += 2) {
+        tile(j, kb0, kb1, vb0, vb1, std::false_type{});
+        tile(j + 1, kb1, kb0, vb1, vb0, std::false_type{});
+      }
+      if (tc - j == 2) {
+        tile(j, kb0, kb1, vb0, vb1, std::false_type{});
+        tile(j + 1, kb1, kb0, vb1, vb0, std::true_type{});
+      } else {
+        tile(j, kb0, kb1, vb0, vb1, std::true_type{});
+      }
+      if (!LATE) interval_end();         // pairs with the late half's last interval
+    };
+    if (tc > 0) {
+      fetch_k(kb0, 0);
+      wait_fetches();
+      interval_end();
+      if (late)
+        pipeline(std::true_type{});
+      else
+        pipeline(std::false_type{});
+    }
+    interval_end();                      // nobody reads the tile buffers any more
+
+    // out[bh, q, d] = acc / l through LDS: this wavefront's 32 rows x D as T, 16-byte
+    // chunk c of row r at chunk c ^ (r & 15); then whole rows leave as 16-byte stores.
+    unsigned char* band = (wave < 2 ? kb0 : wave < 4 ? kb1 : wave < 6 ? vb0 : vb1) + (wave & 1) * (32 * D * 2);
+    const float inv_l = 1.0f / l_i;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int chunk = db * 4 + qd;   // d = chunk*8 + half*4 .. +3
+        u32x2 w;
+        w.x = E::pack2(o_acc[db][qd * 4 + 0] * inv_l, o_acc[db][qd * 4 + 1] * inv_l);
+        w.y = E::pack2(o_acc[db][qd * 4 + 2] * inv_l, o_acc[db][qd * 4 + 3] * inv_l);
+        *reinterpret_cast<u32x2*>(band + l32 * (D * 2) + ((chunk ^ (l32 & 15)) << 4) + half * 8) = w;
+      }
+    constexpr int kLanesPerRow = D * 2 / 16, kRowsPerPass = 64 / kLanesPerRow;
+    const int rd_row = lane / kLanesPerRow, rd_chunk = lane % kLanesPerRow;
+#pragma unroll
+    for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+      const int r = pass * kRowsPerPass + rd_row;
+      const int32_t qr = q0 + r;
+      u32x4 w = *reinterpret_cast<const u32x4*>(band + r * (D * 2) + ((rd_chunk ^ (r & 15)) << 4));
+      if (qr < out.shape[1] && qr < q_len)
+        *reinterpret_cast<u32x4*>((T*)out.ptr + (int64_t)bh * out.strides[0] + (int64_t)qr * out.strides[1] + rd_chunk * 8) = w;
+    }
+  }
+};
+
 }  // namespace
 
 #define FMHA_KERNEL(NAME, T, BM, BN, D)                                                           \
@@ -327,3 +659,14 @@ FMHA_KERNEL(bf16, __bf16, 32, 32, 32)
 FMHA_KERNEL(f16, _Float16, 128, 64, 128)
 FMHA_KERNEL(f16, _Float16, 128, 64, 64)
 FMHA_KERNEL(f16, _Float16, 32, 32, 32)
+
+#define FMHA_PINGPONG_KERNEL(NAME, T, BN, D)                                                       \
+  extern "C" __global__ void __launch_bounds__(512)                                               \
+      fmha_entry__##NAME##_256x##BN##x##D##_pp(PartitionArg<3> out, TensorArg<4> q, TensorArg<4> k, \
+                                               TensorArg<4> v, float qk_scale, int32_t input_pos,  \
+                                               int32_t query_group_size, int32_t causal, TileGrid g) { \
+    FmhaPingPong<T, BN, D>::run(out, q, k, v, qk_scale, input_pos, query_group_size, causal, g);  \
+  }
+
+FMHA_PINGPONG_KERNEL(bf16, __bf16, 64, 128)
+FMHA_PINGPONG_KERNEL(f16, _Float16, 64, 128)

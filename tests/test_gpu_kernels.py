@@ -307,11 +307,23 @@ def test_fmha_reference_example_shape(ct, dev, causal, input_pos):
     assert _fmha_case(ct, dev, 2, 8, 8, 64, 32, 32, causal, input_pos) <= 2e-2
 
 
-@pytest.mark.parametrize("variant", ["bf16_128x64x128", "bf16_128x128x128", "bf16_256x64x128"])
+@pytest.mark.parametrize("variant", ["bf16_128x64x128", "bf16_128x128x128", "bf16_256x64x128", "bf16_256x64x128_pp"])
 @pytest.mark.parametrize("causal", [False, True])
 def test_fmha_d128(ct, dev, variant, causal):
     bm = int(variant.split("_")[1].split("x")[0])
     assert _fmha_case(ct, dev, 1, 2, 2, 512, 128, bm, causal, 0, variant=variant) <= 2e-2
+
+
+@pytest.mark.parametrize("s,causal,input_pos", [(64, False, 0), (128, True, 0), (192, True, 3), (320, False, 0),
+                                                 (1000, True, 0), (1000, False, 0), (1536, True, 17)])
+def test_fmha_pingpong_every_loop_shape(ct, dev, s, causal, input_pos):
+    # 1, 2, 3, 5 and many KV tiles (the pipeline is unrolled by two and peels its last
+    # tile), ragged sequence ends, causal offsets, two kv heads shared by four query heads
+    assert _fmha_case(ct, dev, 1, 4, 2, s, 128, 256, causal, input_pos, variant="bf16_256x64x128_pp", seed=431) <= 2e-2
+
+
+def test_fmha_pingpong_f16(ct, dev):
+    assert _fmha_case(ct, dev, 1, 2, 2, 640, 128, 256, True, 0, dtype=torch.float16, variant="f16_256x64x128_pp") <= 2e-2
 
 
 def test_fmha_gqa_and_ragged_lengths(ct, dev):
