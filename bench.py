@@ -249,9 +249,9 @@ class MxGemm(Workload):
     dtype = "fp8 e4m3 x e8m0 block scale / f32 acc / bf16 out"
     s = 8192
     work = 2.0 * s ** 3
-    tile = 128
+    tile = 256
     config = {"workload": "MX block-scaled fp8 GEMM A[8192,8192] B[8192,8192], e4m3 + e8m0 per 32 K, bf16 out",
-              "tile": "128x128x128"}
+              "tile": "256x256x128"}
 
     def setup(self, ct, torch, oracle, dev):
         s = self.s

@@ -1,0 +1,152 @@
+// Pieces shared by the GEMM kernels for gfx950 (bf16 and MX fp8): vector types,
+// buffer descriptors, the workgroup -> tile mapping and the LDS-staged epilogue.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "kernel_args.h"
+
+namespace cutile {
+namespace gemm {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define LDS_PTR(T) __attribute__((address_space(3))) T*
+
+constexpr int kNumXcd = 8;
+constexpr int kGroupM = 8;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo, hi}, b2));  // v_cvt_pk_bf16_f32, round to nearest even
+}
+
+// Tile index for this workgroup: XCD-contiguous, then grouped along M.
+__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t* pm,
+                                            uint32_t* pn) {
+  const uint32_t total = tiles_m * tiles_n;
+  uint32_t id = blockIdx.x;
+  // Workgroups are dealt round-robin to the XCDs; give each XCD a contiguous
+  // range of logical tile ids (only when the count divides evenly, otherwise the
+  // plain order is kept so every tile is still covered exactly once).
+  if (total % kNumXcd == 0) id = (id % kNumXcd) * (total / kNumXcd) + id / kNumXcd;
+  const uint32_t per_group = kGroupM * tiles_n;
+  const uint32_t group = id / per_group;
+  const uint32_t first_m = group * kGroupM;
+  const uint32_t rows = min(tiles_m - first_m, (uint32_t)kGroupM);
+  const uint32_t in_group = id % per_group;
+  *pm = first_m + in_group % rows;
+  *pn = in_group / rows;
+}
+
+// Epilogue shared by the pipelined variants: accumulators -> z through LDS.
+// In the MFMA layout a lane owns 4 consecutive columns of one row, so a direct
+// store touches 32 rows with 8 or 16 bytes each and every 128-byte line of z is
+// written in 8 pieces.  Staged through LDS (f32, one 32-row band of the
+// wavefront's sub-tile at a time, wavefront-private so no barrier is needed), the
+// same data leaves as 16-byte stores with consecutive lanes on consecutive
+// columns: whole lines.  `accumulate` adds the old z in f32 before the single
+// rounding, as the tile program does (acc = z.load(); ...; z.store(acc)).
+// `stage` is this wavefront's private region of kEpilogueBytesPerWave<WN> bytes.
+// Rows are WN*4 bytes; 16-byte chunk c of row r sits at chunk c ^ (r & 15), so the 16
+// rows of one write pass fall on distinct banks.
+template <int WN>
+constexpr int kEpilogueBytesPerWave = 32 * WN * 4;
+
+template <int TM, int TN, typename OutT>
+__device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
+                                                  int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
+                                                  int lane, int32_t accumulate) {
+  constexpr int WN = TN * 32;
+  constexpr int PITCH = WN * 4;
+  constexpr int COLS_PER_LANE = sizeof(OutT) == 2 ? 8 : 4;      // 16 bytes of output per lane
+  constexpr int LANES_PER_ROW = WN / COLS_PER_LANE;
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  constexpr int PASSES = 32 / ROWS_PER_PASS;
+  const int l32 = lane & 31, khalf = lane >> 5;
+  const int rd_row = lane / LANES_PER_ROW, rd_col = (lane % LANES_PER_ROW) * COLS_PER_LANE;
+  const int32_t gc = wave_col0 + rd_col;
+  const bool col_ok = gc < zN;
+  const bool full = gc + COLS_PER_LANE <= zN;  // zN is a multiple of 4: otherwise exactly the first 4 columns are inside
+  // Old z, all of it requested before anything is waited for.
+  u32x4 old[TM][PASSES];
+  if (accumulate) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int pass = 0; pass < PASSES; ++pass) {
+        const int32_t gr = wave_row0 + tm * 32 + pass * ROWS_PER_PASS + rd_row;
+        old[tm][pass] = u32x4{0, 0, 0, 0};
+        if (gr < zM && col_ok) {
+          const OutT* src = zp + (int64_t)gr * ldz + gc;
+          if (full) {
+            old[tm][pass] = *reinterpret_cast<const u32x4*>(src);
+          } else {
+            u32x2 h = *reinterpret_cast<const u32x2*>(src);
+            old[tm][pass].x = h.x;
+            old[tm][pass].y = h.y;
+          }
+        }
+      }
+  }
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    // write this band in the MFMA layout
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        f32x4 v = {acc[tn][tm][q * 4 + 0], acc[tn][tm][q * 4 + 1], acc[tn][tm][q * 4 + 2], acc[tn][tm][q * 4 + 3]};
+        *reinterpret_cast<f32x4*>(stage + l32 * PITCH + (((tn * 8 + q * 2 + khalf) ^ (l32 & 15)) << 4)) = v;
+      }
+    // read it back row-contiguous and store
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int r = pass * ROWS_PER_PASS + rd_row;
+      const int32_t gr = wave_row0 + tm * 32 + r;
+      const unsigned char* src = stage + r * PITCH;
+      f32x4 lo = *reinterpret_cast<const f32x4*>(src + (((rd_col >> 2) ^ (r & 15)) << 4));
+      const u32x4 o = old[tm][pass];
+      if constexpr (sizeof(OutT) == 2) {
+        f32x4 hi = *reinterpret_cast<const f32x4*>(src + ((((rd_col >> 2) + 1) ^ (r & 15)) << 4));
+        if (accumulate) {
+          lo[0] += __builtin_bit_cast(float, o.x << 16);
+          lo[1] += __builtin_bit_cast(float, o.x & 0xffff0000u);
+          lo[2] += __builtin_bit_cast(float, o.y << 16);
+          lo[3] += __builtin_bit_cast(float, o.y & 0xffff0000u);
+          hi[0] += __builtin_bit_cast(float, o.z << 16);
+          hi[1] += __builtin_bit_cast(float, o.z & 0xffff0000u);
+          hi[2] += __builtin_bit_cast(float, o.w << 16);
+          hi[3] += __builtin_bit_cast(float, o.w & 0xffff0000u);
+        }
+        if (gr < zM && col_ok) {
+          OutT* dst = zp + (int64_t)gr * ldz + gc;
+          if (full) {
+            u32x4 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
+                       pack_bf16x2(hi[2], hi[3])};
+            *reinterpret_cast<u32x4*>(dst) = w;
+          } else {
+            u32x2 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+            *reinterpret_cast<u32x2*>(dst) = w;
+          }
+        }
+      } else {
+        if (accumulate) lo += __builtin_bit_cast(f32x4, o);
+        if (gr < zM && col_ok) *reinterpret_cast<f32x4*>(zp + (int64_t)gr * ldz + gc) = lo;
+      }
+    }
+  }
+}
+
+}  // namespace gemm
+}  // namespace cutile

@@ -25,45 +25,15 @@
 // stores, XCD-aware grouped tile order.
 #include <hip/hip_runtime.h>
 
+#include "gemm_common.h"
 #include "kernel_args.h"
 
 using namespace cutile;
+using namespace cutile::gemm;
 
 namespace {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int kNumXcd = 8;
-constexpr int kGroupM = 8;
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  uint32_t a = __builtin_bit_cast(uint32_t, lo), b = __builtin_bit_cast(uint32_t, hi);
-  a += 0x7fffu + ((a >> 16) & 1u);
-  b += 0x7fffu + ((b >> 16) & 1u);
-  return (a >> 16) | (b & 0xffff0000u);
-}
-
-__device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t* pm,
-                                            uint32_t* pn) {
-  const uint32_t total = tiles_m * tiles_n;
-  uint32_t id = blockIdx.x;
-  if (total % kNumXcd == 0) id = (id % kNumXcd) * (total / kNumXcd) + id / kNumXcd;
-  const uint32_t per_group = kGroupM * tiles_n;
-  const uint32_t group = id / per_group;
-  const uint32_t first_m = group * kGroupM;
-  const uint32_t rows = min(tiles_m - first_m, (uint32_t)kGroupM);
-  const uint32_t in_group = id % per_group;
-  *pm = first_m + in_group % rows;
-  *pn = in_group / rows;
-}
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
 struct MxGemm {
@@ -249,6 +219,248 @@ struct MxGemm {
   }
 };
 
+// ---- pipelined variant: global -> LDS directly, scales through LDS too ---------------------
+// Same pipeline as the bf16 GEMM's direct variant, adapted to 32-byte operands:
+//  * data tiles AND the tile's scale dwords are fetched with buffer loads that
+//    write straight into LDS (data: 16 bytes per lane with the swizzle applied on
+//    the global side; scales: one dword per row, 256 bytes per instruction), two
+//    stages, refilled one K tile ahead;
+//  * an fp8 operand fragment is 8 registers, so there is one set of fragments,
+//    not two: each fragment is reloaded for the next 64-wide K step right after
+//    the last MFMA that reads it, at least three MFMAs (192 matrix-pipe cycles)
+//    before its next use.  The MFMAs of a step run outer-fragment-major so that
+//    the outer fragments free up one by one and the inner ones during the last
+//    outer iteration;
+//  * the stage hand-over sits after the third MFMA of a tile's second K step: by
+//    then every read of the current stage has completed without being waited for;
+//  * memory instructions are dealt out between MFMAs, sched_barrier(0) keeps
+//    the written order; the epilogue is the shared LDS-staged one.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+struct MxGemmDirect {
+  static constexpr int BK = 128;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int kAInstr = BM / 8 / kWaves, kBInstr = BN / 8 / kWaves;   // 1 KiB = 8 rows of 128 bytes
+  static constexpr int kSInstr = (BM + BN) / 64 / kWaves;                     // 256 bytes = 64 rows of scales
+  static constexpr int kABytes = BM * BK, kBBytes = BN * BK;
+  static constexpr int kScaleBytes = (BM + BN) * 4;
+  static constexpr int kStageBytes = kABytes + kBBytes + kScaleBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr bool kOuterIsN = TN <= TM;          // the operand with fewer fragments is the outer one
+  static constexpr int NO = kOuterIsN ? TN : TM, NI = kOuterIsN ? TM : TN;
+  static constexpr int NB = TM * TN;
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0 && (BM + BN) % (64 * kWaves) == 0 && BM % 64 == 0,
+                "tile must split evenly");
+  static_assert(NI >= 3 && NB >= 6, "the reload distance assumes at least three inner fragments");
+  static_assert(kWaves / 2 * kEpilogueBytesPerWave<WN> <= kStageBytes, "the output bands must fit the stages");
+
+  __device__ static __forceinline__ int lds_off(int r, int u) { return r * BK + ((u ^ ((r >> 1) & 7)) << 4); }
+
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                             const TensorArg<2>& xs, const TensorArg<2>& ys, float alpha, const TileGrid& g) {
+    __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStageBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane & 31, khalf = lane >> 5;
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    const int32_t M = x.shape[0], N = y.shape[0], K = min(x.shape[1], y.shape[1]);
+    const int32_t lda = x.strides[0], ldb = y.strides[0];
+    const int32_t ldsa = xs.strides[0], ldsb = ys.strides[0];
+    const int32_t row0 = pm * BM, col0 = pn * BN;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)((int64_t)(M - 1) * lda + x.shape[1]));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)((int64_t)(N - 1) * ldb + y.shape[1]));
+    const __amdgpu_buffer_rsrc_t rsa = make_rsrc(xs.ptr, (uint32_t)((int64_t)(xs.shape[0] - 1) * ldsa + xs.shape[1]));
+    const __amdgpu_buffer_rsrc_t rsb = make_rsrc(ys.ptr, (uint32_t)((int64_t)(ys.shape[0] - 1) * ldsb + ys.shape[1]));
+    constexpr uint32_t kOob = 0x80000000u;
+    const int k_tiles = K / BK;
+
+    // Global side of the fetches (per lane, K tile 0; the K advance is scalar).
+    uint32_t a_goff[kAInstr], b_goff[kBInstr], s_goff[kSInstr];
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_goff[i] = (row0 + r < M) ? (uint32_t)((int64_t)(row0 + r) * lda + u * 16) : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < kBInstr; ++i) {
+      const int r = (wave * kBInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      b_goff[i] = (col0 + r < N) ? (uint32_t)((int64_t)(col0 + r) * ldb + u * 16) : kOob;
+    }
+    // Scale rows: instruction s covers 64 rows; the first BM/64 instructions are x rows.
+    // Rows beyond the tensor read scale byte 0 (2^-127) against all-zero data: they contribute 0.
+#pragma unroll
+    for (int i = 0; i < kSInstr; ++i) {
+      const int sidx = wave * kSInstr + i;
+      const bool is_x = sidx < BM / 64;
+      const int r = (is_x ? sidx : sidx - BM / 64) * 64 + lane;
+      s_goff[i] = is_x ? ((row0 + r < M) ? (uint32_t)((int64_t)(row0 + r) * ldsa) : kOob)
+                       : ((col0 + r < N) ? (uint32_t)((int64_t)(col0 + r) * ldsb) : kOob);
+    }
+    // Fetch instruction i of tile kt into `stage`: x data, then y data, then scales.
+    constexpr int NF = kAInstr + kBInstr + kSInstr;
+    auto fetch_one = [&](unsigned char* stage, int32_t kt, int i) {
+      const bool wanted = kt < k_tiles;   // past the last tile: out-of-range offsets, zeros
+      const int32_t k0 = wanted ? kt * BK : 0;
+      if (i < kAInstr) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                                 wanted ? a_goff[i] : kOob, k0, 0, 0);
+      } else if (i < kAInstr + kBInstr) {
+        const int b = i - kAInstr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(stage + kABytes + (wave * kBInstr + b) * 1024), 16,
+                                                 wanted ? b_goff[b] : kOob, k0, 0, 0);
+      } else {
+        const int si = i - kAInstr - kBInstr;
+        const int sidx = wave * kSInstr + si;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(sidx < BM / 64 ? rsa : rsb,
+                                                 (LDS_PTR(void))(stage + kABytes + kBBytes + sidx * 256), 4,
+                                                 wanted ? s_goff[si] : kOob, k0 / 32, 0, 0);
+      }
+    };
+
+    // LDS side of the operand reads: a fragment of K step ks is units ks*4+khalf and ks*4+2+khalf.
+    int a_addr[2][2], b_addr[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        a_addr[ks][h] = lds_off(wm * WM + l32, ks * 4 + 2 * h + khalf);                 // + tm * 32 rows
+        b_addr[ks][h] = kABytes + lds_off(wn * WN + l32, ks * 4 + 2 * h + khalf);       // + tn * 32 rows
+      }
+    const int sa_addr = kABytes + kBBytes + (wm * WM + l32) * 4;                        // + tm * 32 rows
+    const int sb_addr = kABytes + kBBytes + BM * 4 + (wn * WN + l32) * 4;               // + tn * 32 rows
+    auto read_a = [&](const unsigned char* stage, int ks, int tm) -> i32x8 {
+      u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[ks][0] + tm * 32 * BK);
+      u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[ks][1] + tm * 32 * BK);
+      return i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    };
+    auto read_b = [&](const unsigned char* stage, int ks, int tn) -> i32x8 {
+      u32x4 lo = *reinterpret_cast<const u32x4*>(stage + b_addr[ks][0] + tn * 32 * BK);
+      u32x4 hi = *reinterpret_cast<const u32x4*>(stage + b_addr[ks][1] + tn * 32 * BK);
+      return i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
+
+    i32x8 af[TM], bfr[TN];               // the one set of operand fragments
+    uint32_t sa_cur[TM], sb_cur[TN];     // scale dwords (4 MX blocks) of the tile whose first K step is next
+    int sas[TM], sbs[TN];                // scales of a tile's second K step, already moved to byte 0
+    // K step ks covers MX blocks 2ks and 2ks+1 of the tile; lanes 0-31 supply the scale
+    // of the first, lanes 32-63 of the second, in byte 0 of the scale operand.
+    const int sh0 = 8 * khalf, sh1 = 8 * (2 + khalf);
+    auto read_scales = [&](const unsigned char* stage) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) sa_cur[tm] = *reinterpret_cast<const uint32_t*>(stage + sa_addr + tm * 32 * 4);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) sb_cur[tn] = *reinterpret_cast<const uint32_t*>(stage + sb_addr + tn * 32 * 4);
+    };
+    // MFMA j of a K step (outer-major) and, after it, the reload of whatever fragment it used last.
+    auto mfma_step = [&](int j, int ks) {
+      const int o = j / NI, i = j % NI;
+      const int tn = kOuterIsN ? o : i, tm = kOuterIsN ? i : o;
+      const int sb = ks == 0 ? (int)(sb_cur[tn] >> sh0) : sbs[tn];
+      const int sa = ks == 0 ? (int)(sa_cur[tm] >> sh0) : sas[tm];
+      acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0, sb, 0, sa);
+    };
+    auto reload_after = [&](int j, const unsigned char* stage, int ks) {
+      const int o = j / NI, i = j % NI;
+      if (i == NI - 1) {        // outer fragment o is done
+        if (kOuterIsN) bfr[o] = read_b(stage, ks, o); else af[o] = read_a(stage, ks, o);
+      }
+      if (o == NO - 1) {        // inner fragment i is done
+        if (kOuterIsN) af[i] = read_a(stage, ks, i); else bfr[i] = read_b(stage, ks, i);
+      }
+    };
+
+    // Prologue: tile 0 (and 1) on their way, first fragments and scales in registers.
+    if (k_tiles > 0) {
+#pragma unroll
+      for (int i = 0; i < NF; ++i) fetch_one(stage0, 0, i);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < NF; ++i) fetch_one(stage1, 1, i);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) af[tm] = read_a(stage0, 0, tm);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) bfr[tn] = read_b(stage0, 0, tn);
+      read_scales(stage0);
+    }
+    constexpr int kHandOverAt = 3;   // MFMAs of the second K step issued before the hand-over
+    auto k_tile = [&](unsigned char* cur, const unsigned char* nxt, int kt) {
+      // K step 0; fragments of step 1 are reloaded from `cur` as they free up.
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        mfma_step(j, 0);
+        __builtin_amdgcn_sched_barrier(0);   // the reload must follow the last reader, or it needs registers of its own
+        reload_after(j, cur, 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // K step 1; after the hand-over, fragments and scales of tile kt+1 come from
+      // `nxt` and tile kt+2 is fetched into `cur`.
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) sas[tm] = (int)(sa_cur[tm] >> sh1);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) sbs[tn] = (int)(sb_cur[tn] >> sh1);
+#pragma unroll
+      for (int j = 0; j < kHandOverAt; ++j) {
+        mfma_step(j, 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_waitcnt(0);   // own reads of `cur` done, own share of tile kt+1 landed
+      __syncthreads();
+      read_scales(nxt);
+#pragma unroll
+      for (int j = kHandOverAt; j < NB; ++j) {
+#pragma unroll
+        for (int i = 0; i < NF; ++i)
+          if (i * (NB - kHandOverAt) / NF == j - kHandOverAt) fetch_one(cur, kt + 2, i);
+        mfma_step(j, 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj)   // reloads that fell before the hand-over are issued with the first MFMA after it
+          if ((jj < kHandOverAt && j == kHandOverAt) || jj == j) reload_after(jj, nxt, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // Whole pairs in the loop, an odd last tile after it: with the second tile
+    // under a condition inside the loop the compiler would have to assume, at the
+    // top of the loop, a refill of stage0 in flight and wait for it before every read.
+    int kt = 0;
+    for (; kt + 2 <= k_tiles; kt += 2) {
+      k_tile(stage0, stage1, kt);
+      k_tile(stage1, stage0, kt + 1);
+    }
+    if (kt < k_tiles) k_tile(stage0, stage1, kt);
+
+    // Every wavefront is past its operand reads and every fetch has landed: the
+    // stages are free to carry the output.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tn][tm][v] *= alpha;
+    unsigned char* band = (wave < kWaves / 2 ? stage0 : stage1) + (wave % (kWaves / 2)) * kEpilogueBytesPerWave<WN>;
+    store_tile_staged<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0], z.shape[0], z.shape[1], row0 + wm * WM,
+                                    col0 + wn * WN, lane, 0);
+  }
+};
+
 }  // namespace
 
 #define MX_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                                   \
@@ -265,3 +477,14 @@ MX_KERNEL(mxfp8_f32_256x256x128_w2x2, 256, 256, 2, 2, float)
 MX_KERNEL(mxfp8_f32_128x128x128_w2x2, 128, 128, 2, 2, float)
 MX_KERNEL(mxfp8_f32_32x32x128_w1x1, 32, 32, 1, 1, float)
 MX_KERNEL(mxfp8_f32_64x64x128_w1x1, 64, 64, 1, 1, float)
+
+#define MX_DIRECT_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                            \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                     \
+      linear_tile_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, TensorArg<2> xs, \
+                                TensorArg<2> ys, float alpha, TileGrid g) {                        \
+    MxGemmDirect<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, xs, ys, alpha, g);                         \
+  }
+
+MX_DIRECT_KERNEL(mxfp8_bf16_256x256x128_d2x4, 256, 256, 2, 4, __bf16)
+MX_DIRECT_KERNEL(mxfp8_bf16_256x256x128_d4x2, 256, 256, 4, 2, __bf16)
+MX_DIRECT_KERNEL(mxfp8_f32_256x256x128_d2x4, 256, 256, 2, 4, float)

@@ -355,6 +355,13 @@ def test_mxfp8_all_ones_known_answer(ct, dev):
     (128, 128, 256, 128, torch.float32, None), (256, 256, 512, 256, torch.float32, None),
     (256, 256, 512, 256, torch.bfloat16, None), (512, 256, 384, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_w2x4"),
     (96, 160, 256, 32, torch.float32, None), (64, 64, 128, 64, torch.float32, None),
+    # the pipelined variants: one, two (a pair), three and seven K tiles; M, N off the tile
+    (256, 256, 128, 256, torch.float32, "mxfp8_f32_256x256x128_d2x4"),
+    (256, 512, 256, 256, torch.float32, "mxfp8_f32_256x256x128_d2x4"),
+    (328, 520, 384, 256, torch.float32, "mxfp8_f32_256x256x128_d2x4"),
+    (520, 328, 896, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_d2x4"),
+    (328, 520, 896, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_d4x2"),
+    (512, 512, 1024, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_w2x2"),
 ])
 def test_mxfp8_random_blocks(ct, dev, m, n, k, tile, out_dtype, variant):
     # per-row scale spread exercises distinct e8m0 codes per 32-block
