@@ -123,6 +123,10 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 64, 128, 64, 2, 2);
   gemm("bf16f32", 128, 128, 64, 2, 2);
   gemm("bf16f32", 256, 256, 64, 2, 2);
+  // any tile shape, strides and extents (tile = 0: not tied to a partition shape); 64x64 outputs per workgroup
+  for (const char* dt : {"bf16", "bf16f32", "f16", "f32"})
+    add("gemm", keep(std::string(dt) + "_generic"), keep(std::string("gemm_entry__") + dt + "_generic"), IMG_GEMM, 256,
+        (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
   // ---- FMHA: LDS = 2 stages x (K tile + V tile) ----
   // "_pp": the two wavefronts of a SIMD run half a tile apart (BM = 256 only)

@@ -693,11 +693,14 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
   if (cutile_status_t s = check_tensor(y, "y", 2, 2)) return s;
   const cutile_tensor_arg_t& zt = z->tensor;
-  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_BF16 && y->dtype == CUTILE_DTYPE_BF16, CUTILE_ERR_KERNEL_NOT_FOUND,
-                 "gemm: precompiled variants take bf16 x and y (got %s, %s)", cutile_dtype_name(x->dtype),
+  const bool in_bf16 = x->dtype == CUTILE_DTYPE_BF16, in_f16 = x->dtype == CUTILE_DTYPE_F16, in_f32 = x->dtype == CUTILE_DTYPE_F32;
+  CUTILE_REQUIRE(x->dtype == y->dtype && (in_bf16 || in_f16 || in_f32), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "gemm: x and y must both be bf16, f16 or f32 (got %s, %s)", cutile_dtype_name(x->dtype),
                  cutile_dtype_name(y->dtype));
-  CUTILE_REQUIRE(zt.dtype == CUTILE_DTYPE_BF16 || zt.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_NOT_FOUND,
-                 "gemm: z must be bf16 or f32");
+  CUTILE_REQUIRE((in_bf16 && (zt.dtype == CUTILE_DTYPE_BF16 || zt.dtype == CUTILE_DTYPE_F32)) ||
+                     (in_f16 && zt.dtype == CUTILE_DTYPE_F16) || (in_f32 && zt.dtype == CUTILE_DTYPE_F32),
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "gemm: no kernel for %s operands with %s z (bf16 -> bf16 | f32, f16 -> f16, f32 -> f32)",
+                 cutile_dtype_name(x->dtype), cutile_dtype_name(zt.dtype));
   const int32_t bm = z->partition_shape[0], bn = z->partition_shape[1];
   const int bk_user = generic_int(opts, 3, 64);
   if (cutile_status_t s = check_generic(opts, 1, std::to_string(bm), "BM")) return s;
@@ -708,24 +711,22 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   const int32_t k_total = (k / bk_user) * bk_user;
   uint32_t tg[3];
   if (cutile_status_t s = resolve_grid(z, opts, tg)) return s;
-  CUTILE_REQUIRE(x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
-                     y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
-                     aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
-                     k_total % 8 == 0,
-                 CUTILE_ERR_KERNEL_NOT_FOUND,
-                 "gemm: precompiled variants need row-major operands with unit inner stride, 16-byte aligned rows "
-                 "and K, N multiples of 8");
-  const std::string dt = zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
+  // The matrix-core variants need row-major operands with unit inner stride, 16-byte
+  // aligned rows and K, N multiples of 8; everything else takes the any-layout kernel.
+  const bool fast_layout = x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
+                           y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
+                           aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
+                           k_total % 8 == 0;
+  const std::string dt = in_f32 ? "f32" : in_f16 ? "f16" : zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
   // The ring-pipelined variants ("_r") fetch whole K tiles only.
   const int32_t k_valid = std::min(std::min(x->shape[1], y->shape[0]), k_total);
   std::vector<std::string> acceptable;
-  for (const auto& e : kernel_table())
-    if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
-        (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
-      acceptable.push_back(e.variant);
-  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
-                 "no precompiled variant of gemm<%s, %d, %d, %d>; available: %s", dt.c_str(), bm, bn, bk_user,
-                 list_variants("gemm").c_str());
+  if (fast_layout)
+    for (const auto& e : kernel_table())
+      if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
+          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
+        acceptable.push_back(e.variant);
+  acceptable.push_back(dt + "_generic");
   Resolved res;
   if (cutile_status_t s = resolve_entry("gemm", opts, acceptable[0], acceptable, &res)) return s;
   ArgPacker args;
@@ -736,6 +737,12 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   args.push_tile_grid(tg);
   args.push_val<int32_t>(accumulate ? 1 : 0);
   uint32_t grid[3] = {tg[0] * tg[1], 1, 1};
+  if (res.entry->tile[0] == 0) {   // any-layout kernel: 64x64 outputs per workgroup over the covered region
+    const uint64_t cover_m = std::min<uint64_t>((uint64_t)tg[0] * bm, zt.shape[0]);
+    const uint64_t cover_n = std::min<uint64_t>((uint64_t)tg[1] * bn, zt.shape[1]);
+    grid[0] = std::max<uint32_t>(1, div_up(cover_m, 64));
+    grid[1] = std::max<uint32_t>(1, div_up(cover_n, 64));
+  }
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

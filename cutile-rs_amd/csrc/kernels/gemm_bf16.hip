@@ -714,6 +714,76 @@ struct GemmRing {
   }
 };
 
+// ---- any-layout variant ---------------------------------------------------------------------
+// The tile program for arbitrary tile shapes, element types (bf16, f16, f32),
+// strides and extents — what the pipelined variants cannot take (rows that are
+// not 16-byte aligned, N or K not a multiple of 8, tile shapes without a
+// precompiled kernel, e.g. the reference tests' 16x16x8).  It computes the same
+// function directly: z[r,c] (+)= sum_k x[r,k] * y[k,c] over the region the launch
+// grid covers, reads outside a tensor contributing 0, f32 accumulation in K
+// order, one rounding on store.  64x64 outputs per workgroup of 256 lanes, 4x4
+// per lane, operands staged through LDS as f32.  Correctness path, not a fast one.
+template <typename T>
+__device__ __forceinline__ float elem_to_f32(T v) { return (float)v; }
+
+template <typename InT, typename OutT>
+__device__ void gemm_any_layout(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                int32_t k_total, const TileGrid& g, int32_t accumulate) {
+  constexpr int TS = 64, KS = 16;
+  __shared__ float xs[TS][KS + 1];
+  __shared__ float ys[KS][TS + 1];
+  const int tid = threadIdx.x;
+  const int tr = tid / 16, tc = tid % 16;             // this lane's 4x4 block inside the 64x64 tile
+  const int64_t cover_m = min((int64_t)g.x * z.pshape[0], (int64_t)z.shape[0]);
+  const int64_t cover_n = min((int64_t)g.y * z.pshape[1], (int64_t)z.shape[1]);
+  const int64_t row0 = (int64_t)blockIdx.x * TS, col0 = (int64_t)blockIdx.y * TS;
+  const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
+  const InT* xp = (const InT*)x.ptr;
+  const InT* yp = (const InT*)y.ptr;
+  float acc[4][4] = {};
+  for (int32_t k0 = 0; k0 < k_valid; k0 += KS) {
+    for (int i = tid; i < TS * KS; i += 256) {
+      const int r = i / KS, kk = i % KS;
+      const int64_t gr = row0 + r;
+      xs[r][kk] = (gr < x.shape[0] && k0 + kk < k_valid)
+                      ? elem_to_f32(xp[gr * x.strides[0] + (int64_t)(k0 + kk) * x.strides[1]]) : 0.0f;
+    }
+    for (int i = tid; i < KS * TS; i += 256) {
+      const int kk = i / TS, c = i % TS;
+      const int64_t gc = col0 + c;
+      ys[kk][c] = (gc < y.shape[1] && k0 + kk < k_valid)
+                      ? elem_to_f32(yp[(int64_t)(k0 + kk) * y.strides[0] + gc * y.strides[1]]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[tr * 4 + i][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ys[kk][tc * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  OutT* zp = (OutT*)z.ptr;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t gr = row0 + tr * 4 + i, gc = col0 + tc * 4 + j;
+      if (gr < cover_m && gc < cover_n) {
+        OutT* dst = zp + gr * z.strides[0] + gc * z.strides[1];
+        float v = acc[i][j];
+        if (accumulate) v += elem_to_f32(*dst);
+        *dst = (OutT)v;
+      }
+    }
+}
+
 }  // namespace
 
 // gemm<bf16, BM, BN, BK>(z, x, y, k) with trailing launch metadata.
@@ -755,3 +825,15 @@ GEMM_DIRECT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)
 GEMM_RING_KERNEL(bf16_256x256x64_r2x4, 256, 256, 2, 4, __bf16)
 GEMM_RING_KERNEL(bf16_256x256x64_r4x2, 256, 256, 4, 2, __bf16)
 GEMM_RING_KERNEL(bf16_128x128x64_r2x2, 128, 128, 2, 2, __bf16)
+
+#define GEMM_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                                \
+  extern "C" __global__ void __launch_bounds__(256)                                            \
+      gemm_entry__##NAME##_generic(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, \
+                                   TileGrid g, int32_t accumulate) {                            \
+    gemm_any_layout<IN_T, OUT_T>(z, x, y, k, g, accumulate);                                    \
+  }
+
+GEMM_ANY_LAYOUT_KERNEL(bf16, __bf16, __bf16)
+GEMM_ANY_LAYOUT_KERNEL(bf16f32, __bf16, float)
+GEMM_ANY_LAYOUT_KERNEL(f16, _Float16, _Float16)
+GEMM_ANY_LAYOUT_KERNEL(f32, float, float)

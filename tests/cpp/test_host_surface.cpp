@@ -243,8 +243,14 @@ TEST(launchers_hand_arguments_back_in_the_form_given) {
   auto bad = rms_norm_f16(api::zeros<f16>({4, 64}), api::zeros<f16>({32}), partition_op(api::zeros<f16>({4, 64}), {1, 64}), 1e-6f).sync_on(s);
   CHECK(bad.is_err() && bad.error().kind == DeviceError::Kind::Launch);
   CHECK(launches() == n0 + 3);  // the three fills ran, the kernel did not
-  auto nokernel = gemm(partition_op(api::zeros<bf16>({64, 64}), {48, 48}), api::zeros<bf16>({64, 64}), api::zeros<bf16>({64, 64}), 64).sync_on(s);
+  // a tile shape without a matrix-core kernel runs on the any-layout kernel ...
+  auto odd_tile = gemm(partition_op(api::zeros<bf16>({64, 64}), {48, 48}), api::zeros<bf16>({64, 64}), api::zeros<bf16>({64, 64}), 64).sync_on(s);
+  CHECK(odd_tile.is_ok() && last_symbol() == "gemm_entry__bf16_generic");
+  // ... and a key nothing was built for is a kernel-cache error that names what exists
+  auto nokernel = fmha(partition_op(api::zeros<bf16>({2, 96, 32}), {1, 48, 32}), api::zeros<bf16>({1, 2, 96, 32}), api::zeros<bf16>({1, 2, 96, 32}),
+                       api::zeros<bf16>({1, 2, 96, 32}), 0.125f, 0, 1).sync_on(s);
   CHECK(nokernel.is_err() && nokernel.error().kind == DeviceError::Kind::KernelCache);
+  CHECK(nokernel.error().message.find("available:") != std::string::npos);
   // builder methods reach the launcher
   auto g = gemm(partition_op(api::zeros<bf16>({256, 256}), {128, 128}), api::zeros<bf16>({256, 64}), api::zeros<bf16>({64, 256}), 64)
                .generics({"bf16", "128", "128", "64"}).variant("bf16_128x128x64_w2x2").sync_on(s);

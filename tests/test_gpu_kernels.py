@@ -262,6 +262,42 @@ def test_gemm_ones_known_answer_non_divisible(ct, dev):
     assert torch.equal(z.float(), torch.full((m, n), float(k), device=dev))
 
 
+def test_gemm_any_layout_reference_f32_case_and_odd_layouts(ct, dev):
+    # cutile/tests/slice_non_divisible.rs:458-497 as the reference runs it: f32, tiles 16x16x8, M = N = 100
+    m, n, k = 100, 100, 64
+    z = torch.zeros(m, n, device=dev)
+    ct.gemm(ct.partition(z, [16, 16]), torch.ones(m, k, device=dev), torch.ones(k, n, device=dev), k,
+            generics=["f32", 16, 16, 8])
+    sync()
+    assert torch.all((z - float(k)).abs() < 1e-3)
+    # random f32 against the oracle's cpu_gemm; y passed as a transposed view (inner stride != 1), z accumulated into
+    m, n, k = 77, 53, 40
+    x, y = oracle.normal_f32((m, k), 341), oracle.normal_f32((k, n), 342)
+    z0 = oracle.normal_f32((m, n), 343)
+    z = torch.from_numpy(z0.copy()).to(dev)
+    yt = torch.from_numpy(np.ascontiguousarray(y.T)).to(dev).t()
+    ct.gemm(ct.partition(z, [32, 16]), torch.from_numpy(x).to(dev), yt, k, accumulate=True, generics=["f32", 32, 16, 8])
+    sync()
+    np.testing.assert_allclose(z.cpu().numpy(), oracle.cpu_gemm_f32(x, y) + z0, rtol=1e-5, atol=1e-5)
+    # bf16 with N not a multiple of 8 (rows not 16-byte aligned): the matrix-core variants cannot take it
+    m, n, k = 130, 100, 96
+    a, b = normal_bf16_bits((m, k), 344, k ** -0.5), normal_bf16_bits((k, n), 345, k ** -0.5)
+    z = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    ct.gemm(ct.partition(z, [128, 128]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=False,
+            generics=["bf16", 128, 128, 32])
+    sync()
+    assert rel_l2(z.float().cpu().numpy(), oracle.gemm_bf16(a, b, f32out=True)) <= 1e-2
+    # f16 in, f16 out; only the first tile row is launched (prefix coverage): the rest of z stays untouched
+    m, n, k = 64, 48, 32
+    xh = torch.from_numpy(oracle.f32_to_f16_bits(oracle.normal_f32((m, k), 346)).view(np.float16)).to(dev)
+    yh = torch.from_numpy(oracle.f32_to_f16_bits(oracle.normal_f32((k, n), 347)).view(np.float16)).to(dev)
+    z = torch.full((m, n), 7.0, dtype=torch.float16, device=dev)
+    ct.gemm(ct.partition(z, [16, 16], prefix=True), xh, yh, k, accumulate=False, grid=(1, 3, 1), generics=["f16", 16, 16, 16])
+    sync()
+    ref = xh.float() @ yh.float()
+    assert torch.allclose(z[:16].float(), ref[:16], rtol=2e-3, atol=2e-3) and torch.all(z[16:] == 7.0)
+
+
 def test_gemm_accumulates_into_z_and_f32_out(ct, dev):
     m = n = k = 256
     a, b = normal_bf16_bits((m, k), 311, k ** -0.5), normal_bf16_bits((k, n), 312, k ** -0.5)

@@ -160,9 +160,10 @@ def test_validation_happens_before_any_gpu_work(fake_hip):
     cases = [
         (lambda: ct.gemm(ct.partition(z, [256, 256]), a, b, 256, grid=(1, 1, 1)), "does not match the inferred partition grid"),
         (lambda: ct.gemm(ct.partition(z, [256, 256], prefix=True), a, b, 256), "partial-coverage"),
-        (lambda: ct.gemm(ct.partition(z, [100, 100]), a, b, 256), "no precompiled variant of gemm<bf16, 100, 100, 64>"),
+        (lambda: ct.gemm(ct.partition(z, [100, 100]), a, b, 256, variant="bf16_256x256x64_d4x2"), "does not fit these arguments"),
         (lambda: ct.gemm(ct.partition(z, [256, 256]), a, b, 256, generics=["bf16", 128, 256, 64]), "generic BM"),
-        (lambda: ct.gemm(ct.partition(z, [256, 256]), a.float(), b, 256), "bf16 x and y"),
+        (lambda: ct.gemm(ct.partition(z, [256, 256]), a.float(), b, 256), "x and y must both be"),
+        (lambda: ct.gemm(ct.partition(z, [256, 256]), a.float(), b.float(), 256), "no kernel for f32 operands with bf16 z"),
         (lambda: ct.rms_norm_f16(torch.zeros(4, 64, dtype=torch.half), torch.zeros(32, dtype=torch.half),
                                  ct.partition(torch.zeros(4, 64, dtype=torch.half), [1, 64]), 1e-6), "expected N = 64"),
         (lambda: ct.rms_norm_f16(torch.zeros(4, 64, dtype=torch.half), torch.zeros(64, dtype=torch.half),
@@ -228,8 +229,9 @@ def test_kernel_table_lookup_and_single_flight_module_load(fake_hip):
     info2 = ct.kernel_lookup("gemm", ["bf16", "128", "128", "64"])
     assert info2.symbol == b"gemm_entry__bf16_128x128x64_d2x2" and tuple(info2.block) == (256, 1, 1)
     assert L.cutile_module_load_count() == before + 1          # one code object per kernel family per device
+    assert ct.kernel_lookup("gemm", ["bf16", "48", "48", "16"]).symbol == b"gemm_entry__bf16_generic"   # any tile shape
     with pytest.raises(ct.CutileError, match="available: "):
-        ct.kernel_lookup("gemm", ["bf16", "48", "48", "16"])
+        ct.kernel_lookup("gemm", ["f64", "48", "48", "16"])
     with pytest.raises(ct.CutileError):
         ct.kernel_lookup("no_such_kernel")
     names = ct.kernel_list()
