@@ -149,12 +149,12 @@ std::vector<KernelEntry> build_table() {
   fmha("f16", 32, 32, 32);
 
   // ---- MXFP8 GEMM: LDS = 2 stages x (BM + BN) x 128 bytes ----
-  // "d" = global->LDS direct, pipelined, scale dwords staged with the data (4 bytes per row)
+  // "d" = global->LDS direct, pipelined; scales staged in blocks of four K tiles (16 bytes per row, two blocks)
   auto mx = [&](const char* out, int bm, int bn, int wvm, int wvn, const char* kind = "w") {
     std::string v = std::string("mxfp8_") + out + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x128_" + kind +
                     std::to_string(wvm) + "x" + std::to_string(wvn);
     add("linear_tile", keep(v), keep("linear_tile_entry__" + v), IMG_MXGEMM, (uint32_t)(wvm * wvn * 64),
-        (uint32_t)(2 * (bm + bn) * (128 + (kind[0] == 'd' ? 4 : 0))), bm, bn, 128, 0, out, 0, 2);
+        (uint32_t)(2 * (bm + bn) * (128 + (kind[0] == 'd' ? 16 : 0))), bm, bn, 128, 0, out, 0, 2);
   };
   mx("bf16", 256, 256, 4, 2, "d");
   mx("bf16", 256, 256, 2, 4, "d");

@@ -25,6 +25,8 @@
 // stores, XCD-aware grouped tile order.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gemm_common.h"
 #include "kernel_args.h"
 
@@ -243,11 +245,11 @@ struct MxGemmDirect {
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int kAInstr = BM / 8 / kWaves, kBInstr = BN / 8 / kWaves;   // 1 KiB = 8 rows of 128 bytes
-  static constexpr int kSInstr = (BM + BN) / 64 / kWaves;                     // 256 bytes = 64 rows of scales
+  static constexpr int kSInstr = (BM + BN) / 64 / kWaves;                     // 1 KiB = 64 rows x 16 scale bytes
   static constexpr int kABytes = BM * BK, kBBytes = BN * BK;
-  static constexpr int kScaleBytes = (BM + BN) * 4;
-  static constexpr int kStageBytes = kABytes + kBBytes + kScaleBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kScaleBytes = (BM + BN) * 16;                          // 4 K tiles of scales per row
+  static constexpr int kStageBytes = kABytes + kBBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes + 2 * kScaleBytes;
   static constexpr bool kOuterIsN = TN <= TM;          // the operand with fewer fragments is the outer one
   static constexpr int NO = kOuterIsN ? TN : TM, NI = kOuterIsN ? TM : TN;
   static constexpr int NB = TM * TN;
@@ -262,6 +264,8 @@ struct MxGemmDirect {
                              const TensorArg<2>& xs, const TensorArg<2>& ys, float alpha, const TileGrid& g) {
     __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStageBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char scales0[kScaleBytes];   // scale blocks 0, 2, 4 ...
+    __shared__ __attribute__((aligned(1024))) unsigned char scales1[kScaleBytes];   // scale blocks 1, 3, 5 ...
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -303,8 +307,13 @@ struct MxGemmDirect {
       s_goff[i] = is_x ? ((row0 + r < M) ? (uint32_t)((int64_t)(row0 + r) * ldsa) : kOob)
                        : ((col0 + r < N) ? (uint32_t)((int64_t)(col0 + r) * ldsb) : kOob);
     }
-    // Fetch instruction i of tile kt into `stage`: x data, then y data, then scales.
-    constexpr int NF = kAInstr + kBInstr + kSInstr;
+    // Fetch instruction i of tile kt into `stage`: x data, then y data; with
+    // WITH_SCALES also this wavefront's share of the scale block of tile kt (the
+    // 16 scale bytes per row that cover tiles kt..kt+3, kt a multiple of 4).  One
+    // dword per row per tile would touch a separate cache line per lane every
+    // tile; a block of four tiles costs the same lines once.
+    constexpr int NF = kAInstr + kBInstr;
+    auto scale_block = [&](int32_t tile) -> unsigned char* { return ((tile >> 2) & 1) ? scales1 : scales0; };
     auto fetch_one = [&](unsigned char* stage, int32_t kt, int i) {
       const bool wanted = kt < k_tiles;   // past the last tile: out-of-range offsets, zeros
       const int32_t k0 = wanted ? kt * BK : 0;
@@ -319,7 +328,7 @@ struct MxGemmDirect {
         const int si = i - kAInstr - kBInstr;
         const int sidx = wave * kSInstr + si;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(sidx < BM / 64 ? rsa : rsb,
-                                                 (LDS_PTR(void))(stage + kABytes + kBBytes + sidx * 256), 4,
+                                                 (LDS_PTR(void))(scale_block(kt) + sidx * 1024), 16,
                                                  wanted ? s_goff[si] : kOob, k0 / 32, 0, 0);
       }
     };
@@ -333,8 +342,8 @@ struct MxGemmDirect {
         a_addr[ks][h] = lds_off(wm * WM + l32, ks * 4 + 2 * h + khalf);                 // + tm * 32 rows
         b_addr[ks][h] = kABytes + lds_off(wn * WN + l32, ks * 4 + 2 * h + khalf);       // + tn * 32 rows
       }
-    const int sa_addr = kABytes + kBBytes + (wm * WM + l32) * 4;                        // + tm * 32 rows
-    const int sb_addr = kABytes + kBBytes + BM * 4 + (wn * WN + l32) * 4;               // + tn * 32 rows
+    const int sa_addr = (wm * WM + l32) * 16;                                           // + tm * 32 rows, + 4 * (tile % 4)
+    const int sb_addr = BM * 16 + (wn * WN + l32) * 16;                                 // + tn * 32 rows
     auto read_a = [&](const unsigned char* stage, int ks, int tm) -> i32x8 {
       u32x4 lo = *reinterpret_cast<const u32x4*>(stage + a_addr[ks][0] + tm * 32 * BK);
       u32x4 hi = *reinterpret_cast<const u32x4*>(stage + a_addr[ks][1] + tm * 32 * BK);
@@ -360,11 +369,12 @@ struct MxGemmDirect {
     // K step ks covers MX blocks 2ks and 2ks+1 of the tile; lanes 0-31 supply the scale
     // of the first, lanes 32-63 of the second, in byte 0 of the scale operand.
     const int sh0 = 8 * khalf, sh1 = 8 * (2 + khalf);
-    auto read_scales = [&](const unsigned char* stage) {
+    auto read_scales = [&](int32_t tile) {
+      const unsigned char* blk = scale_block(tile) + (tile & 3) * 4;
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) sa_cur[tm] = *reinterpret_cast<const uint32_t*>(stage + sa_addr + tm * 32 * 4);
+      for (int tm = 0; tm < TM; ++tm) sa_cur[tm] = *reinterpret_cast<const uint32_t*>(blk + sa_addr + tm * 32 * 16);
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) sb_cur[tn] = *reinterpret_cast<const uint32_t*>(stage + sb_addr + tn * 32 * 4);
+      for (int tn = 0; tn < TN; ++tn) sb_cur[tn] = *reinterpret_cast<const uint32_t*>(blk + sb_addr + tn * 32 * 16);
     };
     // MFMA j of a K step (outer-major) and, after it, the reload of whatever fragment it used last.
     auto mfma_step = [&](int j, int ks) {
@@ -387,7 +397,7 @@ struct MxGemmDirect {
     // Prologue: tile 0 (and 1) on their way, first fragments and scales in registers.
     if (k_tiles > 0) {
 #pragma unroll
-      for (int i = 0; i < NF; ++i) fetch_one(stage0, 0, i);
+      for (int i = 0; i < NF + kSInstr; ++i) fetch_one(stage0, 0, i);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
 #pragma unroll
@@ -396,10 +406,12 @@ struct MxGemmDirect {
       for (int tm = 0; tm < TM; ++tm) af[tm] = read_a(stage0, 0, tm);
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) bfr[tn] = read_b(stage0, 0, tn);
-      read_scales(stage0);
+      read_scales(0);
     }
     constexpr int kHandOverAt = 3;   // MFMAs of the second K step issued before the hand-over
-    auto k_tile = [&](unsigned char* cur, const unsigned char* nxt, int kt) {
+    // `with_scales`: tile kt+2 opens a scale block (kt + 2 is a multiple of 4).
+    auto k_tile = [&](unsigned char* cur, const unsigned char* nxt, int kt, auto with_scales) {
+      constexpr int NFT = NF + (decltype(with_scales)::value ? kSInstr : 0);
       // K step 0; fragments of step 1 are reloaded from `cur` as they free up.
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
@@ -421,12 +433,12 @@ struct MxGemmDirect {
       }
       __builtin_amdgcn_s_waitcnt(0);   // own reads of `cur` done, own share of tile kt+1 landed
       __syncthreads();
-      read_scales(nxt);
+      read_scales(kt + 1);
 #pragma unroll
       for (int j = kHandOverAt; j < NB; ++j) {
 #pragma unroll
-        for (int i = 0; i < NF; ++i)
-          if (i * (NB - kHandOverAt) / NF == j - kHandOverAt) fetch_one(cur, kt + 2, i);
+        for (int i = 0; i < NFT; ++i)
+          if (i * (NB - kHandOverAt) / NFT == j - kHandOverAt) fetch_one(cur, kt + 2, i);
         mfma_step(j, 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -439,11 +451,15 @@ struct MxGemmDirect {
     // under a condition inside the loop the compiler would have to assume, at the
     // top of the loop, a refill of stage0 in flight and wait for it before every read.
     int kt = 0;
-    for (; kt + 2 <= k_tiles; kt += 2) {
-      k_tile(stage0, stage1, kt);
-      k_tile(stage1, stage0, kt + 1);
+    for (; kt + 4 <= k_tiles; kt += 4) {
+      k_tile(stage0, stage1, kt, std::false_type{});
+      k_tile(stage1, stage0, kt + 1, std::false_type{});
+      k_tile(stage0, stage1, kt + 2, std::true_type{});
+      k_tile(stage1, stage0, kt + 3, std::false_type{});
     }
-    if (kt < k_tiles) k_tile(stage0, stage1, kt);
+    if (kt < k_tiles) k_tile(stage0, stage1, kt, std::false_type{});
+    if (kt + 1 < k_tiles) k_tile(stage1, stage0, kt + 1, std::false_type{});
+    if (kt + 2 < k_tiles) k_tile(stage0, stage1, kt + 2, std::true_type{});
 
     // Every wavefront is past its operand reads and every fetch has landed: the
     // stages are free to carry the output.
