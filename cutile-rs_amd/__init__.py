@@ -107,6 +107,14 @@ def lib() -> C.CDLL:
             "cutile_launch_convert": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
             "cutile_launch_softmax": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_add_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
+                                               P(PartitionArg), f32, P(LaunchOpts)],
+            "cutile_launch_qk_norm_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
+                                          f32, i32, P(LaunchOpts)],
+            "cutile_launch_add_2d_f16": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_silu_mul_2d_f16": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_rope_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), i32, P(PartitionArg),
+                                       i32, P(LaunchOpts)],
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
@@ -296,6 +304,55 @@ def softmax(x, y: Partition, *, stream=None, grid=None, generics=None, variant=N
     o, _k = _opts(grid, generics, variant)
     xa = tensor_arg(x)
     check(lib().cutile_launch_softmax(_stream(stream), C.byref(xa), C.byref(y.arg()), C.byref(o)))
+
+
+def add_rms_norm_f16(residual, x, w, out: Partition, residual_out: Partition, eps: float, *, stream=None, grid=None,
+                     generics=None, variant=None) -> None:
+    """combined = residual + x; out = RMSNorm(combined) * w; residual_out = combined (cutile-kernels norms.rs:68-136)"""
+    ra, xa, wa = tensor_arg(residual), tensor_arg(x), tensor_arg(w)
+    o, keep = _opts(grid, generics, variant)
+    check(lib().cutile_launch_add_rms_norm_f16(_stream(stream), C.byref(ra), C.byref(xa), C.byref(wa), C.byref(out.arg()),
+                                               C.byref(residual_out.arg()), C.c_float(eps), C.byref(o)))
+
+
+def qk_norm_f16(q, k, q_weight, k_weight, out: Partition, eps: float, num_q_rows: int, *, stream=None, grid=None,
+                generics=None, variant=None) -> None:
+    """rows < num_q_rows of out: RMSNorm(q) * q_weight; the rest: RMSNorm(k) * k_weight (norms.rs:143-216)"""
+    qa, ka, qw, kw = tensor_arg(q), tensor_arg(k), tensor_arg(q_weight), tensor_arg(k_weight)
+    o, keep = _opts(grid, generics, variant)
+    check(lib().cutile_launch_qk_norm_f16(_stream(stream), C.byref(qa), C.byref(ka), C.byref(qw), C.byref(kw),
+                                          C.byref(out.arg()), C.c_float(eps), int(num_q_rows), C.byref(o)))
+
+
+def add_2d_f16(out: Partition, lhs, rhs, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    la, ra = tensor_arg(lhs), tensor_arg(rhs)
+    o, keep = _opts(grid, generics, variant)
+    check(lib().cutile_launch_add_2d_f16(_stream(stream), C.byref(out.arg()), C.byref(la), C.byref(ra), C.byref(o)))
+
+
+def silu_mul_2d_f16(out: Partition, gate, up, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """out = sigmoid(gate) * gate * up (pointwise.rs:46-78)"""
+    ga, ua = tensor_arg(gate), tensor_arg(up)
+    o, keep = _opts(grid, generics, variant)
+    check(lib().cutile_launch_silu_mul_2d_f16(_stream(stream), C.byref(out.arg()), C.byref(ga), C.byref(ua), C.byref(o)))
+
+
+def rope_f16(out: Partition, x, inv_freq, position_start=0, *, k=None, num_q_heads: int = 0, stream=None, grid=None,
+             generics=None) -> None:
+    """Rotary embedding (positional.rs).  `position_start` is an int (rope_seq_f16) or a one-element
+    uint32/int32 device tensor (the dynpos forms); with `k`, heads >= num_q_heads of out come from k."""
+    xa, fa = tensor_arg(x), tensor_arg(inv_freq)
+    ka = tensor_arg(k) if k is not None else None
+    pos_dev = None
+    pos = 0
+    if isinstance(position_start, int):
+        pos = position_start
+    else:
+        pos_dev = tensor_arg(position_start, dtype=U32)
+    o, keep = _opts(grid, generics, None)
+    check(lib().cutile_launch_rope_f16(_stream(stream), C.byref(xa), C.byref(ka) if ka is not None else None, C.byref(fa),
+                                       C.byref(pos_dev) if pos_dev is not None else None, int(pos), C.byref(out.arg()),
+                                       int(num_q_heads), C.byref(o)))
 
 
 def gemm(z: Partition, x, y, k: int, *, accumulate: bool = True, stream=None, grid=None, generics=None,

@@ -62,7 +62,10 @@ std::vector<KernelEntry> build_table() {
     EW("add", "f32", "r1_flat", 1); EW("add", "f32", "r1_tiled", 1); EW("add", "f32", "r2_tiled", 2);
     EW("add", "f16", "r1_flat", 1); EW("add", "f16", "r1_tiled", 1); EW("add", "f16", "r2_tiled", 2);
     EW("add", "bf16", "r1_flat", 1); EW("add", "bf16", "r1_tiled", 1); EW("add", "bf16", "r2_tiled", 2);
+    EW("add", "f32", "r2_flat", 2); EW("add", "f16", "r2_flat", 2); EW("add", "bf16", "r2_flat", 2);
+    EW("silu_mul_2d_f16", "f16", "r2_flat", 2); EW("silu_mul_2d_f16", "f16", "r2_tiled", 2);
   }
+  add("rope", "f16", "rope_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 #undef EW
   static const char* kCreationTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64", "u8", "u16", "u32"};
   static std::deque<std::string> names;  // keeps generated strings alive at stable addresses
@@ -94,6 +97,16 @@ std::vector<KernelEntry> build_table() {
         (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
     add("softmax", keep("f32_" + v), keep("softmax_entry__f32_" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f32",
         (int64_t)rv.wpr * 64 * rv.vpl * 4, 2);
+  }
+  // the fused row norms of the transformer block share the register-resident row machinery
+  static const RowVariant kFusedRow[] = {{1, 1}, {1, 2}, {1, 4}, {1, 8}, {2, 2}, {2, 4}, {2, 8}, {4, 1}, {4, 2}, {4, 4}, {4, 8}};
+  for (const char* fn : {"add_rms_norm_f16", "qk_norm_f16"}) {
+    for (auto rv : kFusedRow) {
+      std::string v = "w" + std::to_string(rv.wpr) + "v" + std::to_string(rv.vpl);
+      add(fn, keep(v), keep(std::string(fn) + "_entry__" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f16",
+          (int64_t)rv.wpr * 64 * rv.vpl * 8, 2);
+    }
+    add(fn, "generic", keep(std::string(fn) + "_entry__generic"), IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   }
   add("rms_norm_f16", "generic", "rms_norm_f16_entry__generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   add("softmax", "f16_generic", "softmax_entry__f16_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);

@@ -502,6 +502,28 @@ cutile_status_t cutile_launch_axpy(cutile_stream_t stream, const cutile_partitio
   CUTILE_REQUIRE(z && z->tensor.rank == 1, CUTILE_ERR_KERNEL_LAUNCH, "axpy: output must be rank 1");
   return launch_elementwise3("axpy", stream, z, &a, x, y, false, opts);
 }
+// add_2d_f16 / silu_mul_2d_f16: rank-2 f16, output tiles [1, BLOCK_SIZE].
+static cutile_status_t launch_pointwise_2d_f16(const char* name, const char* kernel, cutile_stream_t stream,
+                                               const cutile_partition_arg_t* out, const cutile_tensor_arg_t* a,
+                                               const cutile_tensor_arg_t* b, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(out && out->tensor.rank == 2 && out->tensor.dtype == CUTILE_DTYPE_F16 && out->partition_shape[0] == 1,
+                 CUTILE_ERR_KERNEL_LAUNCH, "%s: out must be a rank-2 f16 tensor partitioned [1, BLOCK_SIZE]", name);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(out->partition_shape[1]), "BLOCK_SIZE")) return s;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;   // validated above; the kernels themselves are keyed by the element type
+  o.n_generics = 0;
+  return launch_elementwise3(kernel, stream, out, nullptr, a, b, false, &o);
+}
+cutile_status_t cutile_launch_add_2d_f16(cutile_stream_t stream, const cutile_partition_arg_t* out,
+                                         const cutile_tensor_arg_t* lhs, const cutile_tensor_arg_t* rhs,
+                                         const cutile_launch_opts_t* opts) {
+  return launch_pointwise_2d_f16("add_2d_f16", "add", stream, out, lhs, rhs, opts);
+}
+cutile_status_t cutile_launch_silu_mul_2d_f16(cutile_stream_t stream, const cutile_partition_arg_t* out,
+                                              const cutile_tensor_arg_t* gate, const cutile_tensor_arg_t* up,
+                                              const cutile_launch_opts_t* opts) {
+  return launch_pointwise_2d_f16("silu_mul_2d_f16", "silu_mul_2d_f16", stream, out, gate, up, opts);
+}
 cutile_status_t cutile_launch_add(cutile_stream_t stream, const cutile_partition_arg_t* z, const cutile_tensor_arg_t* x,
                                   const cutile_tensor_arg_t* y, const cutile_launch_opts_t* opts) {
   CUTILE_REQUIRE(y, CUTILE_ERR_INVALID_ARGUMENT, "y is null");
@@ -651,6 +673,146 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
   uint32_t grid[3];
   row_launch_grid(res.entry, rows, grid);
   return launch_packed(res.fn, grid, res.entry->block, rms_norm_residency_lds(res.entry, n), stream, args);
+}
+
+// The two fused row norms: same shape rules and variant choice as rms_norm_f16.
+static cutile_status_t launch_fused_norm(const char* fn, cutile_stream_t stream, const cutile_tensor_arg_t* a,
+                                         const cutile_tensor_arg_t* b, const cutile_tensor_arg_t* w,
+                                         const cutile_tensor_arg_t* w2, const cutile_partition_arg_t* out,
+                                         const cutile_partition_arg_t* out2, float eps, const int32_t* num_q_rows,
+                                         const cutile_launch_opts_t* opts) {
+  const bool qk = num_q_rows != nullptr;
+  if (cutile_status_t s = check_tensor(a, qk ? "q" : "residual", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(b, qk ? "k" : "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(w, qk ? "q_weight" : "w", 1, 1)) return s;
+  if (w2)
+    if (cutile_status_t s = check_tensor(w2, "k_weight", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 2, 2)) return s;
+  if (out2)
+    if (cutile_status_t s = check_partition(out2, "residual_out", 2, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  const int32_t n = a->shape[1];
+  bool f16 = a->dtype == CUTILE_DTYPE_F16 && b->dtype == CUTILE_DTYPE_F16 && w->dtype == CUTILE_DTYPE_F16 &&
+             ot.dtype == CUTILE_DTYPE_F16 && (!w2 || w2->dtype == CUTILE_DTYPE_F16) &&
+             (!out2 || out2->tensor.dtype == CUTILE_DTYPE_F16);
+  CUTILE_REQUIRE(f16, CUTILE_ERR_KERNEL_LAUNCH, "%s: every tensor must be f16", fn);
+  CUTILE_REQUIRE(b->shape[1] == n && w->shape[0] == n && (!w2 || w2->shape[0] == n) && ot.shape[1] == n,
+                 CUTILE_ERR_KERNEL_LAUNCH, "%s: row length N = %d must be shared by all tensors", fn, n);
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == n &&
+                     (!out2 || (out2->partition_shape[0] == 1 && out2->partition_shape[1] == n)),
+                 CUTILE_ERR_KERNEL_LAUNCH, "%s: outputs must be partitioned [1, %d]", fn, n);
+  if (qk) {
+    CUTILE_REQUIRE(*num_q_rows >= 0 && *num_q_rows <= a->shape[0] && ot.shape[0] <= *num_q_rows + b->shape[0],
+                   CUTILE_ERR_KERNEL_LAUNCH, "%s: out has %d rows but q supplies %d (num_q_rows) and k %d", fn, ot.shape[0],
+                   *num_q_rows, b->shape[0]);
+  } else {
+    CUTILE_REQUIRE(ot.shape[0] <= a->shape[0] && ot.shape[0] <= b->shape[0] && out2->tensor.shape[0] == ot.shape[0] &&
+                       out2->tensor.shape[1] == n,
+                   CUTILE_ERR_KERNEL_LAUNCH, "%s: out is [%d, %d] but residual is [%d, %d] and x [%d, %d]", fn, ot.shape[0],
+                   ot.shape[1], a->shape[0], n, b->shape[0], n);
+  }
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(n), "N")) return s;
+  uint32_t tg[3];
+  if (out2) {
+    uint32_t explicit_grid[3] = {0, 0, 0};
+    if (opts) memcpy(explicit_grid, opts->grid, sizeof(explicit_grid));
+    const cutile_partition_arg_t* parts[2] = {out, out2};
+    if (cutile_status_t s = cutile_infer_launch_grid(explicit_grid, parts, 2, tg)) return s;
+  } else if (cutile_status_t s = resolve_grid(out, opts, tg)) {
+    return s;
+  }
+  auto row_ok = [&](const cutile_tensor_arg_t& t) { return t.strides[1] == 1 && t.strides[0] % 8 == 0 && aligned16(t.ptr); };
+  const bool vec_ok = n % 8 == 0 && row_ok(*a) && row_ok(*b) && row_ok(ot) && (!out2 || row_ok(out2->tensor)) &&
+                      w->strides[0] == 1 && aligned16(w->ptr) && (!w2 || (w2->strides[0] == 1 && aligned16(w2->ptr)));
+  std::vector<std::string> acceptable;
+  if (vec_ok) acceptable = fitting_row_variants(fn, "w", n);
+  acceptable.push_back("generic");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry(fn, opts, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*a);
+  args.push_tensor(*b);
+  args.push_tensor(*w);
+  if (w2) args.push_tensor(*w2);
+  args.push_partition(*out);
+  if (out2) args.push_partition(*out2);
+  args.push_val<float>(eps);
+  if (qk) args.push_val<int32_t>(*num_q_rows);
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>(tg[0], ot.shape[0]);
+  uint32_t grid[3];
+  row_launch_grid(res.entry, rows, grid);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_add_rms_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* residual,
+                                               const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* w,
+                                               const cutile_partition_arg_t* out,
+                                               const cutile_partition_arg_t* residual_out, float eps,
+                                               const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(residual_out, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  return launch_fused_norm("add_rms_norm_f16", stream, residual, x, w, nullptr, out, residual_out, eps, nullptr, opts);
+}
+
+cutile_status_t cutile_launch_qk_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                          const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* q_weight,
+                                          const cutile_tensor_arg_t* k_weight, const cutile_partition_arg_t* out,
+                                          float eps, int32_t num_q_rows, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(k_weight, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  return launch_fused_norm("qk_norm_f16", stream, q, k, q_weight, k_weight, out, nullptr, eps, &num_q_rows, opts);
+}
+
+// Rotary embedding, all three reference forms: `k` may be null (rope_seq*), and
+// the start position comes either by value or from one u32 in device memory.
+cutile_status_t cutile_launch_rope_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                       const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* inv_freq,
+                                       const cutile_tensor_arg_t* position_start_dev, int32_t position_start,
+                                       const cutile_partition_arg_t* out, int32_t num_q_heads,
+                                       const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(q, k ? "q" : "x", 3, 3)) return s;
+  if (k)
+    if (cutile_status_t s = check_tensor(k, "k", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(inv_freq, "inv_freq", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 3, 3)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  const int32_t d = q->shape[2], half = d / 2;
+  CUTILE_REQUIRE(q->dtype == CUTILE_DTYPE_F16 && ot.dtype == CUTILE_DTYPE_F16 && (!k || k->dtype == CUTILE_DTYPE_F16) &&
+                     inv_freq->dtype == CUTILE_DTYPE_F32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "rope: x / q / k / out must be f16 and inv_freq f32");
+  CUTILE_REQUIRE(d % 2 == 0 && inv_freq->shape[0] == half && ot.shape[2] == d && (!k || k->shape[2] == d),
+                 CUTILE_ERR_KERNEL_LAUNCH, "rope: head dimension D = %d needs inv_freq of D/2 = %d entries and matching tensors", d, half);
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == 1 && out->partition_shape[2] == half,
+                 CUTILE_ERR_KERNEL_LAUNCH, "rope: out must be partitioned [1, 1, %d] (HALF_D), got [%d, %d, %d]", half,
+                 out->partition_shape[0], out->partition_shape[1], out->partition_shape[2]);
+  if (!k) num_q_heads = q->shape[1];
+  CUTILE_REQUIRE(num_q_heads >= 0 && num_q_heads <= q->shape[1] && ot.shape[0] <= q->shape[0] &&
+                     ot.shape[1] <= num_q_heads + (k ? k->shape[1] : 0) && (!k || ot.shape[0] <= k->shape[0]),
+                 CUTILE_ERR_KERNEL_LAUNCH, "rope: out [%d, %d, %d] does not fit the inputs", ot.shape[0], ot.shape[1], ot.shape[2]);
+  if (position_start_dev) {
+    if (cutile_status_t s = check_tensor(position_start_dev, "position_start", 1, 1)) return s;
+    CUTILE_REQUIRE(position_start_dev->dtype == CUTILE_DTYPE_U32 && position_start_dev->shape[0] == 1 &&
+                       ((uintptr_t)position_start_dev->ptr & 3) == 0,
+                   CUTILE_ERR_KERNEL_LAUNCH, "rope: position_start must be one aligned u32");
+  }
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(half), "HALF_D")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  CUTILE_REQUIRE(tg[2] == 2, CUTILE_ERR_KERNEL_LAUNCH, "rope: the launch grid must cover both halves of D (grid.z = 2, got %u)", tg[2]);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("rope", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*q);
+  args.push_tensor(k ? *k : *q);
+  args.push_tensor(*inv_freq);
+  args.push_val<const void*>(position_start_dev ? position_start_dev->ptr : nullptr);
+  args.push_partition(*out);
+  args.push_val<int32_t>(position_start);
+  args.push_val<int32_t>(num_q_heads);
+  args.push_tile_grid(tg);
+  const uint64_t lanes = (uint64_t)std::min<uint32_t>(tg[0], ot.shape[0]) * std::min<uint32_t>(tg[1], ot.shape[1]) * ((half + 7) / 8);
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(lanes, 256), 1u << 16)), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,

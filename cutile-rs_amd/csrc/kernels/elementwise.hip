@@ -213,6 +213,96 @@ ADD_KERNELS(float, f32)
 ADD_KERNELS(_Float16, f16)
 ADD_KERNELS(__bf16, bf16)
 
+// rank-2 flat form (add_2d_f16 of cutile-kernels/src/pointwise.rs:15-40 is add<f16> on [1, BLOCK] tiles)
+#define ADD_R2_FLAT(T, NAME)                                                                        \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      add_entry__##NAME##_r2_flat(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, TileGrid g) { \
+    flat_stream3<T>((T*)z.ptr, (const T*)x.ptr, (const T*)y.ptr, (size_t)z.shape[0] * z.shape[1],  \
+                    [](T xv, T yv) { return (T)(xv + yv); });                                      \
+  }
+ADD_R2_FLAT(float, f32)
+ADD_R2_FLAT(_Float16, f16)
+ADD_R2_FLAT(__bf16, bf16)
+
+// ---- silu_mul_2d_f16: out <- sigmoid(gate) * gate * up, f32 math ---------------------------
+// cutile-kernels/src/pointwise.rs:46-78: sigmoid = 1 / (1 + exp(0 - gate)).
+__device__ __forceinline__ _Float16 silu_mul(_Float16 gate, _Float16 up) {
+  const float g = (float)gate, u = (float)up;
+  const float sig = 1.0f / (1.0f + __builtin_amdgcn_exp2f((0.0f - g) * 1.4426950408889634f));
+  return (_Float16)(sig * g * u);
+}
+extern "C" __global__ void __launch_bounds__(kThreads)
+    silu_mul_2d_f16_entry__f16_r2_flat(PartitionArg<2> out, TensorArg<2> gate, TensorArg<2> up, TileGrid g) {
+  flat_stream3<_Float16>((_Float16*)out.ptr, (const _Float16*)gate.ptr, (const _Float16*)up.ptr,
+                         (size_t)out.shape[0] * out.shape[1], [](_Float16 a, _Float16 b) { return silu_mul(a, b); });
+}
+extern "C" __global__ void __launch_bounds__(kThreads)
+    silu_mul_2d_f16_entry__f16_r2_tiled(PartitionArg<2> out, TensorArg<2> gate, TensorArg<2> up, TileGrid g) {
+  for_each_tile_elem<2>(out, [&](const int32_t* idx, int64_t off) {
+    _Float16 gv = load_padded<_Float16>((const _Float16*)gate.ptr, gate.shape, gate.strides, idx, 2);
+    _Float16 uv = load_padded<_Float16>((const _Float16*)up.ptr, up.shape, up.strides, idx, 2);
+    ((_Float16*)out.ptr)[off] = silu_mul(gv, uv);
+  });
+}
+
+// ---- rotary position embedding -------------------------------------------------------------
+// rope_seq_f16 / rope_seq_dynpos_f16 / qk_rope_dynpos_f16 (cutile-kernels/src/positional.rs:13-64,
+// 70-130, 136-230): x [seq, heads, D] split in halves lo = [.., :D/2], hi = [.., D/2:];
+// theta = f32(position_start + s) * inv_freq[i]; y_lo = x_lo cos - x_hi sin; y_hi = x_hi cos + x_lo sin.
+// The reference launches one tile block per (s, head, half) and computes both halves
+// in each; here one lane produces both halves of one rotation pair, 8 pairs per
+// lane (16-byte accesses), a workgroup row per (s, head).  In the q/k form heads
+// >= num_q_heads of `out` come from `k`.  `pos_dev` (if not null) holds the start position.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    rope_entry__f16(TensorArg<3> q, TensorArg<3> k, TensorArg<1> inv_freq, const uint32_t* pos_dev,
+                    PartitionArg<3> out, int32_t position_start, int32_t num_q_heads, TileGrid g) {
+  const int32_t d = q.shape[2], half = d >> 1;
+  const int64_t seq = min((int64_t)g.x, (int64_t)out.shape[0]);
+  const int64_t heads = min((int64_t)g.y, (int64_t)out.shape[1]);
+  const int32_t base = pos_dev ? (int32_t)pos_dev[0] : position_start;
+  const float* freq = (const float*)inv_freq.ptr;
+  const int64_t pairs_per_row = (half + 7) / 8;                 // 8 rotation pairs per lane
+  const int64_t total = seq * heads * pairs_per_row;
+  for (int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
+    const int32_t chunk = (int32_t)(t % pairs_per_row);
+    const int64_t sh = t / pairs_per_row;
+    const int32_t h = (int32_t)(sh % heads);
+    const int64_t s_idx = sh / heads;
+    const bool from_k = h >= num_q_heads;
+    const TensorArg<3>& src = from_k ? k : q;
+    const _Float16* xr = (const _Float16*)src.ptr + s_idx * src.strides[0] + (int64_t)(from_k ? h - num_q_heads : h) * src.strides[1];
+    _Float16* orow = (_Float16*)out.ptr + s_idx * out.strides[0] + (int64_t)h * out.strides[1];
+    const float pos = (float)(base + (int32_t)s_idx);
+    const int32_t i0 = chunk * 8;
+    const bool vec = (half % 8 == 0) && src.strides[2] == 1 && out.strides[2] == 1 && (src.strides[1] % 8 == 0) &&
+                     (src.strides[0] % 8 == 0) && (out.strides[1] % 8 == 0) && (out.strides[0] % 8 == 0) &&
+                     (((uintptr_t)src.ptr | (uintptr_t)out.ptr) & 15) == 0;
+    if (vec) {
+      Vec16<_Float16> lo, hi, ylo, yhi;
+      lo.raw = *reinterpret_cast<const u32x4*>(xr + i0);
+      hi.raw = *reinterpret_cast<const u32x4*>(xr + half + i0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float sn, cs;
+        sincosf(pos * freq[i0 + e], &sn, &cs);
+        const float l = (float)lo.v[e], hv = (float)hi.v[e];
+        ylo.v[e] = (_Float16)(l * cs - hv * sn);
+        yhi.v[e] = (_Float16)(hv * cs + l * sn);
+      }
+      *reinterpret_cast<u32x4*>(orow + i0) = ylo.raw;
+      *reinterpret_cast<u32x4*>(orow + half + i0) = yhi.raw;
+    } else {
+      for (int32_t i = i0; i < min(i0 + 8, half); ++i) {
+        float sn, cs;
+        sincosf(pos * freq[(int64_t)i * inv_freq.strides[0]], &sn, &cs);
+        const float l = (float)xr[(int64_t)i * src.strides[2]], hv = (float)xr[(int64_t)(half + i) * src.strides[2]];
+        orow[(int64_t)i * out.strides[2]] = (_Float16)(l * cs - hv * sn);
+        orow[(int64_t)(half + i) * out.strides[2]] = (_Float16)(hv * cs + l * sn);
+      }
+    }
+  }
+}
+
 // ---- creation ------------------------------------------------------------------------------
 #define CREATION_KERNELS(T, NAME)                                                                   \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \

@@ -8,6 +8,9 @@
 //                  cutile-benchmarks/benches/softmax.rs:19-35
 //                  per tile row: e = exp(x - max); y = e / sum(e)
 //
+// Also here, on the same row machinery: add_rms_norm_f16 and qk_norm_f16
+// (cutile-kernels/src/norms.rs:68-136, 143-216).
+//
 // The reference reads each RMSNorm row twice (two loops over BLOCK_SIZE chunks).
 // Here a row is read from HBM exactly once: it is held in registers as 16-byte
 // vectors (one wavefront, or WPR wavefronts, per row; lane-strided so that every
@@ -83,11 +86,15 @@ struct SegmentMap {
 };
 
 // ---- RMSNorm -----------------------------------------------------------------------------
+// Rows at or beyond `split` come from (x2, w2) instead of (x, w), indexed from 0
+// again: qk_norm_f16's "q rows first, then k rows" (split = rows for plain RMSNorm).
 template <int WPR, int VPL>
 __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, int64_t x_row_stride,
                                               const _Float16* __restrict__ w,
                                               _Float16* __restrict__ out, int64_t out_row_stride,
-                                              int32_t n, int64_t rows, float eps) {
+                                              int32_t n, int64_t rows, float eps,
+                                              const _Float16* __restrict__ x2 = nullptr, int64_t x2_row_stride = 0,
+                                              const _Float16* __restrict__ w2 = nullptr, int64_t split = INT64_MAX) {
   using V = Vec16<_Float16>;
   constexpr int ROWS_PER_WG = kWaves / WPR;
   __shared__ float lds[kWaves];
@@ -100,8 +107,9 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
 
   V xv[VPL];
   float ss = 0.0f;
+  const bool second = row >= split;   // same for all wavefronts of a row
   if (live) {
-    const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * x_row_stride);
+    const u32x4* xr = reinterpret_cast<const u32x4*>(second ? x2 + (row - split) * x2_row_stride : x + row * x_row_stride);
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
       int32_t vi = v0 + i * (64 * WPR);
@@ -120,7 +128,7 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
   if (!live) return;
   const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
   u32x4* orow = reinterpret_cast<u32x4*>(out + row * out_row_stride);
-  const u32x4* wr = reinterpret_cast<const u32x4*>(w);
+  const u32x4* wr = reinterpret_cast<const u32x4*>(second ? w2 : w);
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     int32_t vi = v0 + i * (64 * WPR);
@@ -131,6 +139,113 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
       for (int e = 0; e < 8; ++e) ov.v[e] = (_Float16)(((float)xv[i].v[e] * inv) * (float)wv.v[e]);
       __builtin_nontemporal_store(ov.raw, orow + vi);
     }
+  }
+}
+
+// add_rms_norm_f16: combined = residual + x stays in f32 registers (it is both
+// the normalised quantity and, rounded, the new residual): two rows read, two
+// rows written, each once.
+template <int WPR, int VPL>
+__device__ __forceinline__ void add_rms_norm_rows(const _Float16* __restrict__ residual, int64_t res_row_stride,
+                                                  const _Float16* __restrict__ x, int64_t x_row_stride,
+                                                  const _Float16* __restrict__ w,
+                                                  _Float16* __restrict__ out, int64_t out_row_stride,
+                                                  _Float16* __restrict__ res_out, int64_t res_out_row_stride,
+                                                  int32_t n, int64_t rows, float eps) {
+  using V = Vec16<_Float16>;
+  constexpr int ROWS_PER_WG = kWaves / WPR;
+  __shared__ float lds[kWaves];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int slot = wave / WPR, sub = wave % WPR;
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + slot;
+  const bool live = row < rows;
+  const int32_t nvec = n >> 3;
+  const int32_t v0 = sub * 64 + lane;
+
+  float cv[VPL][8];
+  float ss = 0.0f;
+  if (live) {
+    const u32x4* rr = reinterpret_cast<const u32x4*>(residual + row * res_row_stride);
+    const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * x_row_stride);
+    V rv[VPL], xv[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      int32_t vi = v0 + i * (64 * WPR);
+      if (vi < nvec) {
+        rv[i].raw = __builtin_nontemporal_load(rr + vi);
+        xv[i].raw = __builtin_nontemporal_load(xr + vi);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        cv[i][e] = (float)rv[i].v[e] + (float)xv[i].v[e];
+        ss = __builtin_fmaf(cv[i][e], cv[i][e], ss);
+      }
+    }
+  }
+  ss = group_reduce<WPR, false>(ss, lds, slot, sub);
+  if (!live) return;
+  const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+  u32x4* orow = reinterpret_cast<u32x4*>(out + row * out_row_stride);
+  u32x4* rrow = reinterpret_cast<u32x4*>(res_out + row * res_out_row_stride);
+  const u32x4* wr = reinterpret_cast<const u32x4*>(w);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
+    if (vi < nvec) {
+      V wv, ov, cvh;
+      wv.raw = wr[vi];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ov.v[e] = (_Float16)((cv[i][e] * inv) * (float)wv.v[e]);
+        cvh.v[e] = (_Float16)cv[i][e];
+      }
+      __builtin_nontemporal_store(ov.raw, orow + vi);
+      __builtin_nontemporal_store(cvh.raw, rrow + vi);
+    }
+  }
+}
+
+// Any N / any strides for the two fused forms: one workgroup per row, inputs re-read (L2).
+__device__ __forceinline__ void fused_norm_row_generic(const TensorArg<2>& a, const TensorArg<2>* b_add,
+                                                       const TensorArg<2>* b_alt, const TensorArg<1>& w,
+                                                       const TensorArg<1>* w_alt, const PartitionArg<2>& out,
+                                                       const PartitionArg<2>* out2, float eps, int64_t rows,
+                                                       int64_t split) {
+  // b_add: second addend (add_rms_norm); b_alt / w_alt: source and weight for rows >= split (qk_norm)
+  __shared__ float lds[kWaves];
+  const int wave = threadIdx.x >> 6;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const bool second = b_alt && row >= split;
+    const TensorArg<2>& src = second ? *b_alt : a;
+    const int64_t srow = second ? row - split : row;
+    const TensorArg<1>& wt = second ? *w_alt : w;
+    const _Float16* xr = (const _Float16*)src.ptr + srow * src.strides[0];
+    const _Float16* ar = b_add ? (const _Float16*)b_add->ptr + row * b_add->strides[0] : nullptr;
+    const int32_t n = src.shape[1];
+    auto value = [&](int32_t j) -> float {
+      float f = (float)xr[(int64_t)j * src.strides[1]];
+      return ar ? f + (float)ar[(int64_t)j * b_add->strides[1]] : f;
+    };
+    float ss = 0.0f;
+    for (int32_t j = threadIdx.x; j < n; j += kThreads) {
+      float f = value(j);
+      ss = __builtin_fmaf(f, f, ss);
+    }
+    ss = group_reduce<kWaves, false>(ss, lds, 0, wave);
+    const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+    _Float16* orow = (_Float16*)out.ptr + row * out.strides[0];
+    _Float16* o2row = out2 ? (_Float16*)out2->ptr + row * out2->strides[0] : nullptr;
+    const int32_t n_out = out.shape[1] < n ? out.shape[1] : n;
+    for (int32_t j = threadIdx.x; j < n_out; j += kThreads) {
+      float f = value(j);
+      float wv = j < wt.shape[0] ? (float)((const _Float16*)wt.ptr)[(int64_t)j * wt.strides[0]] : 0.0f;
+      orow[(int64_t)j * out.strides[1]] = (_Float16)((f * inv) * wv);
+      if (o2row && j < out2->shape[1]) o2row[(int64_t)j * out2->strides[1]] = (_Float16)f;
+    }
+    __syncthreads();
   }
 }
 
@@ -300,6 +415,48 @@ RMS_NORM_KERNEL(4, 2)
 RMS_NORM_KERNEL(4, 4)
 RMS_NORM_KERNEL(4, 8)
 RMS_NORM_KERNEL(4, 16)
+
+// add_rms_norm_f16(residual, x, w, out: [1, N] tiles, residual_out: [1, N] tiles, eps)
+#define ADD_RMS_NORM_KERNEL(WPR, VPL)                                                               \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      add_rms_norm_f16_entry__w##WPR##v##VPL(TensorArg<2> residual, TensorArg<2> x, TensorArg<1> w, \
+                                             PartitionArg<2> out, PartitionArg<2> residual_out,     \
+                                             float eps, TileGrid g) {                               \
+    int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);                                       \
+    add_rms_norm_rows<WPR, VPL>((const _Float16*)residual.ptr, residual.strides[0],                \
+                                (const _Float16*)x.ptr, x.strides[0], (const _Float16*)w.ptr,      \
+                                (_Float16*)out.ptr, out.strides[0], (_Float16*)residual_out.ptr,   \
+                                residual_out.strides[0], x.shape[1], rows, eps);                   \
+  }
+// qk_norm_f16(q, k, q_weight, k_weight, out: [1, N] tiles, eps, num_q_rows)
+#define QK_NORM_KERNEL(WPR, VPL)                                                                    \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      qk_norm_f16_entry__w##WPR##v##VPL(TensorArg<2> q, TensorArg<2> k, TensorArg<1> qw,            \
+                                        TensorArg<1> kw, PartitionArg<2> out, float eps,            \
+                                        int32_t num_q_rows, TileGrid g) {                           \
+    int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);                                       \
+    rms_norm_rows<WPR, VPL>((const _Float16*)q.ptr, q.strides[0], (const _Float16*)qw.ptr,         \
+                            (_Float16*)out.ptr, out.strides[0], q.shape[1], rows, eps,             \
+                            (const _Float16*)k.ptr, k.strides[0], (const _Float16*)kw.ptr,         \
+                            (int64_t)num_q_rows);                                                  \
+  }
+#define FUSED_NORM_VARIANTS(M) \
+  M(1, 1) M(1, 2) M(1, 4) M(1, 8) M(2, 2) M(2, 4) M(2, 8) M(4, 1) M(4, 2) M(4, 4) M(4, 8)
+FUSED_NORM_VARIANTS(ADD_RMS_NORM_KERNEL)
+FUSED_NORM_VARIANTS(QK_NORM_KERNEL)
+
+extern "C" __global__ void __launch_bounds__(kThreads)
+    add_rms_norm_f16_entry__generic(TensorArg<2> residual, TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out,
+                                    PartitionArg<2> residual_out, float eps, TileGrid g) {
+  int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);
+  fused_norm_row_generic(x, &residual, nullptr, w, nullptr, out, &residual_out, eps, rows, INT64_MAX);
+}
+extern "C" __global__ void __launch_bounds__(kThreads)
+    qk_norm_f16_entry__generic(TensorArg<2> q, TensorArg<2> k, TensorArg<1> qw, TensorArg<1> kw, PartitionArg<2> out,
+                               float eps, int32_t num_q_rows, TileGrid g) {
+  int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);
+  fused_norm_row_generic(q, nullptr, &k, qw, &kw, out, nullptr, eps, rows, (int64_t)num_q_rows);
+}
 
 extern "C" __global__ void __launch_bounds__(kThreads)
     rms_norm_f16_entry__generic(TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out, float eps,

@@ -369,6 +369,56 @@ struct LinearTileMxfp8Fn {
     return cutile_launch_linear_tile_mxfp8(s, &zp, &xa, &ya, &xsa, &ysa, alpha, o);
   }
 };
+// ---- transformer-block kernels (cutile-kernels/src/{norms,pointwise,positional}.rs) ----
+struct AddRmsNormF16Fn {
+  template <class R, class X, class W, class O, class RO>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, R& residual, X& x, W& w, O& out, RO& residual_out, float eps) {
+    auto ra = input_arg(residual), xa = input_arg(x), wa = input_arg(w);
+    auto op = out.arg(), rop = residual_out.arg();
+    return cutile_launch_add_rms_norm_f16(s, &ra, &xa, &wa, &op, &rop, eps, o);
+  }
+};
+struct QkNormF16Fn {
+  template <class Q, class K, class QW, class KW, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, QW& qw, KW& kw, O& out, float eps, int32_t num_q_rows) {
+    auto qa = input_arg(q), ka = input_arg(k), qwa = input_arg(qw), kwa = input_arg(kw);
+    auto op = out.arg();
+    return cutile_launch_qk_norm_f16(s, &qa, &ka, &qwa, &kwa, &op, eps, num_q_rows, o);
+  }
+};
+template <bool Silu>
+struct Pointwise2dF16Fn {
+  template <class O, class A, class B>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, O& out, A& a, B& b) {
+    auto op = out.arg();
+    auto aa = input_arg(a), ba = input_arg(b);
+    return Silu ? cutile_launch_silu_mul_2d_f16(s, &op, &aa, &ba, o) : cutile_launch_add_2d_f16(s, &op, &aa, &ba, o);
+  }
+};
+struct RopeSeqF16Fn {
+  template <class X, class F, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, F& inv_freq, O& out, int32_t position_start) {
+    auto xa = input_arg(x), fa = input_arg(inv_freq);
+    auto op = out.arg();
+    return cutile_launch_rope_f16(s, &xa, nullptr, &fa, nullptr, position_start, &op, 0, o);
+  }
+};
+struct RopeSeqDynposF16Fn {
+  template <class X, class F, class P, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, F& inv_freq, P& position_start, O& out) {
+    auto xa = input_arg(x), fa = input_arg(inv_freq), pa = input_arg(position_start);
+    auto op = out.arg();
+    return cutile_launch_rope_f16(s, &xa, nullptr, &fa, &pa, 0, &op, 0, o);
+  }
+};
+struct QkRopeDynposF16Fn {
+  template <class Q, class K, class F, class P, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, F& inv_freq, P& position_start, O& out, int32_t num_q_heads) {
+    auto qa = input_arg(q), ka = input_arg(k), fa = input_arg(inv_freq), pa = input_arg(position_start);
+    auto op = out.arg();
+    return cutile_launch_rope_f16(s, &qa, &ka, &fa, &pa, 0, &op, num_q_heads, o);
+  }
+};
 }  // namespace kernels
 
 // saxpy(y: partition, a, x) -> (y, a, x)        cutile-examples/examples/saxpy.rs:12-17
@@ -390,6 +440,19 @@ template <class O, class Q, class K, class V> auto fmha(O&& out, Q&& q, K&& k, V
 template <class O, class Q, class K, class V> auto fmha_causal(O&& out, Q&& q, K&& k, V&& v, float scale, int32_t input_pos, int32_t group) { return make_launcher<kernels::FmhaFn<true>>(std::forward<O>(out), std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), scale, input_pos, group); }
 // linear_tile(z: partition [BM,BN], x, y, x_scales, y_scales, alpha)   cutile-examples/examples/mxfp8.rs:35-42
 template <class Z, class X, class Y, class XS, class YS> auto linear_tile(Z&& z, X&& x, Y&& y, XS&& xs, YS&& ys, float alpha) { return make_launcher<kernels::LinearTileMxfp8Fn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), std::forward<XS>(xs), std::forward<YS>(ys), alpha); }
+// add_rms_norm_f16(residual, x, w, out: [1,N], residual_out: [1,N], eps)      cutile-kernels/src/norms.rs:76-83
+template <class R, class X, class W, class O, class RO> auto add_rms_norm_f16(R&& residual, X&& x, W&& w, O&& out, RO&& residual_out, float eps) { return make_launcher<kernels::AddRmsNormF16Fn>(std::forward<R>(residual), std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), std::forward<RO>(residual_out), eps); }
+// qk_norm_f16(q, k, q_weight, k_weight, out: [1,N], eps, num_q_rows)          cutile-kernels/src/norms.rs:152-160
+template <class Q, class K, class QW, class KW, class O> auto qk_norm_f16(Q&& q, K&& k, QW&& qw, KW&& kw, O&& out, float eps, int32_t num_q_rows) { return make_launcher<kernels::QkNormF16Fn>(std::forward<Q>(q), std::forward<K>(k), std::forward<QW>(qw), std::forward<KW>(kw), std::forward<O>(out), eps, num_q_rows); }
+// add_2d_f16(out: [1,BLOCK], lhs, rhs) / silu_mul_2d_f16(out: [1,BLOCK], gate, up)   cutile-kernels/src/pointwise.rs:20-24, 51-55
+template <class O, class A, class B> auto add_2d_f16(O&& out, A&& lhs, B&& rhs) { return make_launcher<kernels::Pointwise2dF16Fn<false>>(std::forward<O>(out), std::forward<A>(lhs), std::forward<B>(rhs)); }
+template <class O, class A, class B> auto silu_mul_2d_f16(O&& out, A&& gate, B&& up) { return make_launcher<kernels::Pointwise2dF16Fn<true>>(std::forward<O>(out), std::forward<A>(gate), std::forward<B>(up)); }
+// rope_seq_f16(x, inv_freq, out: [1,1,D/2], position_start)                    cutile-kernels/src/positional.rs:18-23
+template <class X, class F, class O> auto rope_seq_f16(X&& x, F&& inv_freq, O&& out, int32_t position_start) { return make_launcher<kernels::RopeSeqF16Fn>(std::forward<X>(x), std::forward<F>(inv_freq), std::forward<O>(out), position_start); }
+// rope_seq_dynpos_f16(x, inv_freq, position_start: [1] u32, out)               positional.rs:75-80
+template <class X, class F, class P, class O> auto rope_seq_dynpos_f16(X&& x, F&& inv_freq, P&& position_start, O&& out) { return make_launcher<kernels::RopeSeqDynposF16Fn>(std::forward<X>(x), std::forward<F>(inv_freq), std::forward<P>(position_start), std::forward<O>(out)); }
+// qk_rope_dynpos_f16(q, k, inv_freq, position_start, out, num_q_heads)         positional.rs:141-148
+template <class Q, class K, class F, class P, class O> auto qk_rope_dynpos_f16(Q&& q, K&& k, F&& inv_freq, P&& position_start, O&& out, int32_t num_q_heads) { return make_launcher<kernels::QkRopeDynposF16Fn>(std::forward<Q>(q), std::forward<K>(k), std::forward<F>(inv_freq), std::forward<P>(position_start), std::forward<O>(out), num_q_heads); }
 
 namespace api {
 template <class T> struct is_graph_node_memcpy : std::true_type {};

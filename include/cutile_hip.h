@@ -323,6 +323,40 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
  * cutile-examples/examples/softmax.rs:11-24 */
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
                                       const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts);
+/* ---- transformer-block kernels of cutile-kernels (f16 IO, f32 math) ------ */
+/* add_rms_norm_f16<N, BLOCK_SIZE>(residual, x, w, out: [1,N] tiles, residual_out: [1,N] tiles, eps):
+ * combined = residual + x; out = RMSNorm(combined) * w; residual_out = combined —
+ * cutile-kernels/src/norms.rs:68-136 */
+cutile_status_t cutile_launch_add_rms_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* residual,
+                                               const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* w,
+                                               const cutile_partition_arg_t* out,
+                                               const cutile_partition_arg_t* residual_out, float eps,
+                                               const cutile_launch_opts_t* opts);
+/* qk_norm_f16<N, BLOCK_SIZE>(q, k, q_weight, k_weight, out: [1,N] tiles, eps, num_q_rows): rows
+ * < num_q_rows of out are RMSNorm(q rows) * q_weight, the rest RMSNorm(k rows) * k_weight —
+ * cutile-kernels/src/norms.rs:143-216 */
+cutile_status_t cutile_launch_qk_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                          const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* q_weight,
+                                          const cutile_tensor_arg_t* k_weight, const cutile_partition_arg_t* out,
+                                          float eps, int32_t num_q_rows, const cutile_launch_opts_t* opts);
+/* add_2d_f16<BLOCK_SIZE>(out: [1,BLOCK] tiles, lhs, rhs) and silu_mul_2d_f16<BLOCK_SIZE>(out, gate, up):
+ * out = sigmoid(gate) * gate * up — cutile-kernels/src/pointwise.rs:15-40, 46-78 */
+cutile_status_t cutile_launch_add_2d_f16(cutile_stream_t stream, const cutile_partition_arg_t* out,
+                                         const cutile_tensor_arg_t* lhs, const cutile_tensor_arg_t* rhs,
+                                         const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_silu_mul_2d_f16(cutile_stream_t stream, const cutile_partition_arg_t* out,
+                                              const cutile_tensor_arg_t* gate, const cutile_tensor_arg_t* up,
+                                              const cutile_launch_opts_t* opts);
+/* Rotary position embedding on [seq, heads, D] with out partitioned [1, 1, D/2] (grid.z = 2).
+ * One entry point for the three reference launchers (cutile-kernels/src/positional.rs):
+ *   rope_seq_f16(x, inv_freq, out, position_start)                 :13-64   k = NULL, position_start_dev = NULL
+ *   rope_seq_dynpos_f16(x, inv_freq, position_start: [1] u32, out)  :70-130  k = NULL
+ *   qk_rope_dynpos_f16(q, k, inv_freq, position_start, out, num_q_heads) :136-230  heads >= num_q_heads of out come from k */
+cutile_status_t cutile_launch_rope_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                       const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* inv_freq,
+                                       const cutile_tensor_arg_t* position_start_dev, int32_t position_start,
+                                       const cutile_partition_arg_t* out, int32_t num_q_heads,
+                                       const cutile_launch_opts_t* opts);
 /* gemm<T, BM, BN, BK>(z: [BM,BN] tiles, x, y, k): z <- z + x·y with f32
  * accumulation (z is read as the initial accumulator, like the reference bench;
  * `accumulate` = 0 starts from zero like the example) —

@@ -54,6 +54,11 @@ def lib() -> C.CDLL:
             "orc_add_f32": (None, [sz, vp, vp, vp]),
             "orc_rms_norm_f16": (None, [vp, vp, vp, i64, i64, f32, i64]),
             "orc_rms_norm_f16_f64": (None, [vp, vp, vp, i64, i64, f64]),
+            "orc_add_rms_norm_f16": (None, [vp, vp, vp, vp, vp, i64, i64, f32, i64]),
+            "orc_qk_norm_f16": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, i64]),
+            "orc_add_f16": (None, [sz, vp, vp, vp]),
+            "orc_silu_mul_f16": (None, [sz, vp, vp, vp]),
+            "orc_rope_seq_f16": (None, [vp, vp, vp, i64, i64, i64, C.c_int32]),
             "orc_softmax_f32": (None, [vp, vp, i64, i64, i64, i64]),
             "orc_softmax_f16": (None, [vp, vp, i64, i64, i64, i64]),
             "orc_cpu_gemm_f32": (None, [vp, vp, vp, i64, i64, i64]),
@@ -171,6 +176,48 @@ def rms_norm_f16_f64(x_bits, w_bits, eps: float) -> np.ndarray:
     rows, n = x.shape
     out = np.empty_like(x)
     lib().orc_rms_norm_f16_f64(_p(x), _p(w), _p(out), rows, n, eps)
+    return out
+
+
+# ---- transformer-block kernels ---------------------------------------------------------------
+def add_rms_norm_f16(residual_bits, x_bits, w_bits, eps: float, block: int = 0):
+    """-> (out, residual_out), both f16 bit patterns"""
+    r, x, w = _c(residual_bits, np.uint16), _c(x_bits, np.uint16), _c(w_bits, np.uint16)
+    rows, n = x.shape
+    out, res = np.empty_like(x), np.empty_like(x)
+    lib().orc_add_rms_norm_f16(_p(r), _p(x), _p(w), _p(out), _p(res), rows, n, eps, block or n)
+    return out, res
+
+
+def qk_norm_f16(q_bits, k_bits, qw_bits, kw_bits, eps: float, block: int = 0) -> np.ndarray:
+    q, k = _c(q_bits, np.uint16), _c(k_bits, np.uint16)
+    qw, kw = _c(qw_bits, np.uint16), _c(kw_bits, np.uint16)
+    n = q.shape[1]
+    out = np.empty((q.shape[0] + k.shape[0], n), np.uint16)
+    lib().orc_qk_norm_f16(_p(q), _p(k), _p(qw), _p(kw), _p(out), q.shape[0], k.shape[0], n, eps, block or n)
+    return out
+
+
+def add_f16(lhs_bits, rhs_bits) -> np.ndarray:
+    a, b = _c(lhs_bits, np.uint16), _c(rhs_bits, np.uint16)
+    out = np.empty_like(a)
+    lib().orc_add_f16(a.size, _p(a), _p(b), _p(out))
+    return out
+
+
+def silu_mul_f16(gate_bits, up_bits) -> np.ndarray:
+    g, u = _c(gate_bits, np.uint16), _c(up_bits, np.uint16)
+    out = np.empty_like(g)
+    lib().orc_silu_mul_f16(g.size, _p(g), _p(u), _p(out))
+    return out
+
+
+def rope_seq_f16(x_bits, inv_freq, position_start: int) -> np.ndarray:
+    x, f = _c(x_bits, np.uint16), _c(inv_freq, np.float32)
+    seq, heads, d = x.shape
+    assert f.size == d // 2
+    out = np.empty_like(x)
+    lib().orc_rope_seq_f16(_p(x), _p(f), _p(out), seq, heads, d, position_start)
     return out
 
 

@@ -240,6 +240,114 @@ void orc_rms_norm_f16_f64(const uint16_t* x, const uint16_t* w, uint16_t* out, i
 }
 
 /* ------------------------------------------------------------------------ */
+/* Transformer-block kernels (cutile-kernels/src/{norms,pointwise,positional}.rs) */
+/* ------------------------------------------------------------------------ */
+/* Lane-wise sum of squares as the kernel bodies do it: a [1, block] f32
+ * accumulator tile, lane l takes columns l, l + block, ...; lanes summed in
+ * ascending order (reduce_sum). */
+static float lane_sum_of_squares(const float* row, int64_t n, int64_t block, float* lanes) {
+  for (int64_t l = 0; l < block; l++) lanes[l] = 0.0f;
+  for (int64_t j = 0; j < n; j += block) {
+    int64_t lim = n - j < block ? n - j : block;
+    for (int64_t l = 0; l < lim; l++) lanes[l] = lanes[l] + row[j + l] * row[j + l];
+  }
+  float ss = 0.0f;
+  for (int64_t l = 0; l < block; l++) ss += lanes[l];
+  return ss;
+}
+
+/* norms.rs:68-136: combined = f32(residual) + f32(x) (kept in f32); rms over combined;
+ * out = f16(combined * inv * w); residual_out = f16(combined). */
+void orc_add_rms_norm_f16(const uint16_t* residual, const uint16_t* x, const uint16_t* w,
+                          uint16_t* out, uint16_t* residual_out, int64_t rows, int64_t n, float eps,
+                          int64_t block) {
+  if (block <= 0 || block > n) block = n;
+#pragma omp parallel
+  {
+    float* lanes = (float*)malloc(sizeof(float) * (size_t)block);
+    float* comb = (float*)malloc(sizeof(float) * (size_t)n);
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+      for (int64_t j = 0; j < n; j++)
+        comb[j] = orc_f16_to_f32(residual[r * n + j]) + orc_f16_to_f32(x[r * n + j]);
+      float ss = lane_sum_of_squares(comb, n, block, lanes);
+      float inv = 1.0f / sqrtf(ss / (float)n + eps);
+      for (int64_t j = 0; j < n; j++) {
+        out[r * n + j] = orc_f32_to_f16(comb[j] * inv * orc_f16_to_f32(w[j]));
+        residual_out[r * n + j] = orc_f32_to_f16(comb[j]);
+      }
+    }
+    free(lanes);
+    free(comb);
+  }
+}
+
+/* norms.rs:143-216: output row r < q_rows is RMSNorm(q[r]) with q_weight, row
+ * q_rows + r is RMSNorm(k[r]) with k_weight. */
+void orc_qk_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qw, const uint16_t* kw,
+                     uint16_t* out, int64_t q_rows, int64_t k_rows, int64_t n, float eps,
+                     int64_t block) {
+  if (block <= 0 || block > n) block = n;
+#pragma omp parallel
+  {
+    float* lanes = (float*)malloc(sizeof(float) * (size_t)block);
+    float* row = (float*)malloc(sizeof(float) * (size_t)n);
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < q_rows + k_rows; r++) {
+      const int is_q = r < q_rows;
+      const uint16_t* src = is_q ? q + r * n : k + (r - q_rows) * n;
+      const uint16_t* wt = is_q ? qw : kw;
+      for (int64_t j = 0; j < n; j++) row[j] = orc_f16_to_f32(src[j]);
+      float ss = lane_sum_of_squares(row, n, block, lanes);
+      float inv = 1.0f / sqrtf(ss / (float)n + eps);
+      for (int64_t j = 0; j < n; j++) out[r * n + j] = orc_f32_to_f16(row[j] * inv * orc_f16_to_f32(wt[j]));
+    }
+    free(lanes);
+    free(row);
+  }
+}
+
+/* pointwise.rs:15-40: f16 + f16 (one rounding: the f32 sum of two f16 values is exact). */
+void orc_add_f16(size_t n, const uint16_t* lhs, const uint16_t* rhs, uint16_t* out) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) out[i] = orc_f32_to_f16(orc_f16_to_f32(lhs[i]) + orc_f16_to_f32(rhs[i]));
+}
+
+/* pointwise.rs:46-78: sigmoid = 1 / (1 + exp(0 - gate)); y = f16(sigmoid * gate * up), f32 math. */
+void orc_silu_mul_f16(size_t n, const uint16_t* gate, const uint16_t* up, uint16_t* out) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) {
+    float g = orc_f16_to_f32(gate[i]), u = orc_f16_to_f32(up[i]);
+    float sig = 1.0f / (1.0f + expf(0.0f - g));
+    out[i] = orc_f32_to_f16(sig * g * u);
+  }
+}
+
+/* positional.rs:13-64 (rope_seq_f16; the dynpos forms differ only in where the
+ * start position comes from): x [seq, heads, d], halves lo = [..., :d/2], hi =
+ * [..., d/2:]; theta = f32(position_start + s) * inv_freq[i];
+ * y_lo = x_lo cos - x_hi sin; y_hi = x_hi cos + x_lo sin. */
+void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, int64_t seq,
+                      int64_t heads, int64_t d, int32_t position_start) {
+  const int64_t half = d / 2;
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < seq; s++) {
+    const float pos = (float)(position_start + (int32_t)s);
+    for (int64_t h = 0; h < heads; h++) {
+      const uint16_t* xr = x + (s * heads + h) * d;
+      uint16_t* orow = out + (s * heads + h) * d;
+      for (int64_t i = 0; i < half; i++) {
+        float theta = pos * inv_freq[i];
+        float c = cosf(theta), sn = sinf(theta);
+        float lo = orc_f16_to_f32(xr[i]), hi = orc_f16_to_f32(xr[half + i]);
+        orow[i] = orc_f32_to_f16(lo * c - hi * sn);
+        orow[half + i] = orc_f32_to_f16(hi * c + lo * sn);
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------ */
 /* K3                                                                        */
 /* ------------------------------------------------------------------------ */
 static void softmax_tile_row(const float* xin, float* yout, int64_t valid, int64_t bn) {

@@ -74,6 +74,22 @@ void orc_rms_norm_f16(const uint16_t* x, const uint16_t* w, uint16_t* out, int64
 void orc_rms_norm_f16_f64(const uint16_t* x, const uint16_t* w, uint16_t* out, int64_t rows,
                           int64_t n, double eps);
 
+/* ---- transformer-block kernels (f16 IO, f32 math) ----------------------- */
+/* add_rms_norm_f16: cutile-kernels/src/norms.rs:68-136 */
+void orc_add_rms_norm_f16(const uint16_t* residual, const uint16_t* x, const uint16_t* w,
+                          uint16_t* out, uint16_t* residual_out, int64_t rows, int64_t n, float eps,
+                          int64_t block);
+/* qk_norm_f16: norms.rs:143-216; out has q_rows + k_rows rows */
+void orc_qk_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qw, const uint16_t* kw,
+                     uint16_t* out, int64_t q_rows, int64_t k_rows, int64_t n, float eps,
+                     int64_t block);
+/* add_2d_f16 / silu_mul_2d_f16: cutile-kernels/src/pointwise.rs:15-40, 46-78 */
+void orc_add_f16(size_t n, const uint16_t* lhs, const uint16_t* rhs, uint16_t* out);
+void orc_silu_mul_f16(size_t n, const uint16_t* gate, const uint16_t* up, uint16_t* out);
+/* rope_seq_f16 (and its dynpos / qk forms): cutile-kernels/src/positional.rs:13-64 */
+void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, int64_t seq,
+                      int64_t heads, int64_t d, int32_t position_start);
+
 /* ---- K3: softmax over tiles [bm, bn] ---------------------------------- */
 /* f32 IO.  Tile (i, j) covers rows i*bm.., cols j*bn..; every tile row is
  * normalised on its own (row softmax iff bn == n).  Columns beyond n read as 0

@@ -61,6 +61,49 @@ TEST(rms_norm_constant_rows) {
   for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 0.5f);  // x == c -> out = w
 }
 
+TEST(transformer_block_kernels_closed_forms) {
+  auto stream = new_stream();
+  // add_rms_norm: residual = 1, x = 2 -> combined = 3 everywhere; out = w, residual_out = 3
+  auto res = api::full<f16>(1.0, {8, 512}).sync_on(stream).unwrap();
+  auto x = api::full<f16>(2.0, {8, 512}).sync_on(stream).unwrap();
+  auto w = api::full<f16>(0.25, {512}).sync_on(stream).unwrap();
+  auto out = api::zeros<f16>({8, 512}).sync_on(stream).unwrap();
+  auto res_out = api::zeros<f16>({8, 512}).sync_on(stream).unwrap();
+  CHECK(add_rms_norm_f16(&res, &x, &w, out.partition_mut({1, 512}), res_out.partition_mut({1, 512}), 0.0f).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 0.25f);
+  for (f16 v : api::to_host_vec(res_out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 3.0f);
+  // qk_norm: q rows take q_weight, k rows k_weight
+  auto q = api::full<f16>(-2.0, {6, 128}).sync_on(stream).unwrap();
+  auto k = api::full<f16>(5.0, {2, 128}).sync_on(stream).unwrap();
+  auto qw = api::full<f16>(1.0, {128}).sync_on(stream).unwrap();
+  auto kw = api::full<f16>(2.0, {128}).sync_on(stream).unwrap();
+  auto qk = api::zeros<f16>({8, 128}).sync_on(stream).unwrap();
+  CHECK(qk_norm_f16(&q, &k, &qw, &kw, qk.partition_mut({1, 128}), 0.0f, 6).sync_on(stream).is_ok());
+  auto qk_host = api::to_host_vec(qk).sync_on(stream).unwrap();
+  for (int i = 0; i < 8 * 128; ++i) CHECK(f32_from_f16(qk_host[i]) == (i < 6 * 128 ? -1.0f : 2.0f));
+  // silu_mul: gate = 0 -> 0; add_2d: 2 + 2 = 4
+  auto gate = api::zeros<f16>({4, 256}).sync_on(stream).unwrap();
+  auto act = api::full<f16>(7.0, {4, 256}).sync_on(stream).unwrap();
+  auto up = api::full<f16>(2.0, {4, 256}).sync_on(stream).unwrap();
+  CHECK(silu_mul_2d_f16(act.partition_mut({1, 64}), &gate, &up).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(act).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 0.0f);
+  CHECK(add_2d_f16(act.partition_mut({1, 64}), &up, &up).generics({"64"}).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(act).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 4.0f);
+  // rope at position 0 is the identity, whichever way the position arrives
+  auto ramp = std::make_shared<Tensor<float>>(api::arange<float>(3 * 2 * 16).sync_on(stream).unwrap());
+  auto xr = reshape_op(api::convert<f16>(ramp), {3, 2, 16}).sync_on(stream).unwrap();
+  auto inv_freq = api::full<float>(0.5, {8}).sync_on(stream).unwrap();
+  auto rot = api::zeros<f16>({1, 2, 16}).sync_on(stream).unwrap();
+  CHECK(rope_seq_f16(&xr, &inv_freq, rot.partition_mut({1, 1, 8}), 0).sync_on(stream).is_ok());
+  auto rot_host = api::to_host_vec(rot).sync_on(stream).unwrap();
+  for (int i = 0; i < 32; ++i) CHECK(f32_from_f16(rot_host[i]) == (float)i);
+  auto pos = api::zeros<uint32_t>({1}).sync_on(stream).unwrap();
+  CHECK(rope_seq_dynpos_f16(&xr, &inv_freq, &pos, rot.partition_mut({1, 1, 8})).sync_on(stream).is_ok());
+  CHECK(qk_rope_dynpos_f16(&xr, &xr, &inv_freq, &pos, rot.partition_mut({1, 1, 8}), 1).sync_on(stream).is_ok());
+  rot_host = api::to_host_vec(rot).sync_on(stream).unwrap();
+  for (int i = 0; i < 16; ++i) CHECK(f32_from_f16(rot_host[16 + i]) == (float)i);   // head 1 of out = head 0 of k
+}
+
 TEST(gemm_ones_non_divisible) {
   auto stream = new_stream();
   const int m = 200, n = 264, k = 128;
