@@ -614,6 +614,8 @@ static void row_launch_grid(const KernelEntry* e, uint64_t segments, uint32_t gr
   grid[0] = grid[1] = grid[2] = 1;
   if (e->capacity <= 0)
     grid[0] = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(segments, 1), 1u << 20);
+  else if (e->tile[1] > 0)   // short-row variants: tile[1] rows per workgroup
+    grid[0] = std::max<uint32_t>(1, div_up(segments, e->tile[1]));
   else
     grid[0] = std::max<uint32_t>(1, div_up(segments, 4 / e->tile[3]));
 }
@@ -725,7 +727,7 @@ static cutile_status_t launch_fused_norm(const char* fn, cutile_stream_t stream,
   const bool vec_ok = n % 8 == 0 && row_ok(*a) && row_ok(*b) && row_ok(ot) && (!out2 || row_ok(out2->tensor)) &&
                       w->strides[0] == 1 && aligned16(w->ptr) && (!w2 || (w2->strides[0] == 1 && aligned16(w2->ptr)));
   std::vector<std::string> acceptable;
-  if (vec_ok) acceptable = fitting_row_variants(fn, "w", n);
+  if (vec_ok) acceptable = fitting_row_variants(fn, "", n);
   acceptable.push_back("generic");
   Resolved res;
   if (cutile_status_t s = resolve_entry(fn, opts, acceptable[0], acceptable, &res)) return s;
@@ -810,8 +812,8 @@ cutile_status_t cutile_launch_rope_f16(cutile_stream_t stream, const cutile_tens
   args.push_val<int32_t>(position_start);
   args.push_val<int32_t>(num_q_heads);
   args.push_tile_grid(tg);
-  const uint64_t lanes = (uint64_t)std::min<uint32_t>(tg[0], ot.shape[0]) * std::min<uint32_t>(tg[1], ot.shape[1]) * ((half + 7) / 8);
-  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(lanes, 256), 1u << 16)), 1, 1};
+  // one workgroup per sequence position (it computes that position's angles once)
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(std::min<uint32_t>(tg[0], ot.shape[0]), 1u << 20)), 1, 1};
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

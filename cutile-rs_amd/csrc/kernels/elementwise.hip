@@ -250,54 +250,72 @@ extern "C" __global__ void __launch_bounds__(kThreads)
 // 70-130, 136-230): x [seq, heads, D] split in halves lo = [.., :D/2], hi = [.., D/2:];
 // theta = f32(position_start + s) * inv_freq[i]; y_lo = x_lo cos - x_hi sin; y_hi = x_hi cos + x_lo sin.
 // The reference launches one tile block per (s, head, half) and computes both halves
-// in each; here one lane produces both halves of one rotation pair, 8 pairs per
-// lane (16-byte accesses), a workgroup row per (s, head).  In the q/k form heads
-// >= num_q_heads of `out` come from `k`.  `pos_dev` (if not null) holds the start position.
+// in each; here a workgroup takes one position s: cos/sin of its D/2 angles are
+// computed once into LDS (they do not depend on the head), then every lane
+// rotates 8 pairs of one head (16-byte accesses).  In the q/k form heads >=
+// num_q_heads of `out` come from `k`.  `pos_dev` (if not null) holds the start position.
 extern "C" __global__ void __launch_bounds__(kThreads)
     rope_entry__f16(TensorArg<3> q, TensorArg<3> k, TensorArg<1> inv_freq, const uint32_t* pos_dev,
                     PartitionArg<3> out, int32_t position_start, int32_t num_q_heads, TileGrid g) {
+  constexpr int kMaxHalf = 1024;                      // angles kept in LDS; longer heads recompute per lane
+  __shared__ float cs_tab[kMaxHalf], sn_tab[kMaxHalf];
   const int32_t d = q.shape[2], half = d >> 1;
   const int64_t seq = min((int64_t)g.x, (int64_t)out.shape[0]);
-  const int64_t heads = min((int64_t)g.y, (int64_t)out.shape[1]);
+  const int32_t heads = (int32_t)min((int64_t)g.y, (int64_t)out.shape[1]);
   const int32_t base = pos_dev ? (int32_t)pos_dev[0] : position_start;
   const float* freq = (const float*)inv_freq.ptr;
-  const int64_t pairs_per_row = (half + 7) / 8;                 // 8 rotation pairs per lane
-  const int64_t total = seq * heads * pairs_per_row;
-  for (int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
-    const int32_t chunk = (int32_t)(t % pairs_per_row);
-    const int64_t sh = t / pairs_per_row;
-    const int32_t h = (int32_t)(sh % heads);
-    const int64_t s_idx = sh / heads;
-    const bool from_k = h >= num_q_heads;
-    const TensorArg<3>& src = from_k ? k : q;
-    const _Float16* xr = (const _Float16*)src.ptr + s_idx * src.strides[0] + (int64_t)(from_k ? h - num_q_heads : h) * src.strides[1];
-    _Float16* orow = (_Float16*)out.ptr + s_idx * out.strides[0] + (int64_t)h * out.strides[1];
+  const int32_t chunks = (half + 7) / 8;               // 8 rotation pairs per lane
+  const bool tab = half <= kMaxHalf;
+  const bool vec_out = (half % 8 == 0) && out.strides[2] == 1 && (out.strides[1] % 8 == 0) && (out.strides[0] % 8 == 0) &&
+                       ((uintptr_t)out.ptr & 15) == 0;
+  auto vec_in = [&](const TensorArg<3>& t) {
+    return t.strides[2] == 1 && (t.strides[1] % 8 == 0) && (t.strides[0] % 8 == 0) && ((uintptr_t)t.ptr & 15) == 0;
+  };
+  const bool vec = vec_out && vec_in(q) && vec_in(k);
+  for (int64_t s_idx = blockIdx.x; s_idx < seq; s_idx += gridDim.x) {
     const float pos = (float)(base + (int32_t)s_idx);
-    const int32_t i0 = chunk * 8;
-    const bool vec = (half % 8 == 0) && src.strides[2] == 1 && out.strides[2] == 1 && (src.strides[1] % 8 == 0) &&
-                     (src.strides[0] % 8 == 0) && (out.strides[1] % 8 == 0) && (out.strides[0] % 8 == 0) &&
-                     (((uintptr_t)src.ptr | (uintptr_t)out.ptr) & 15) == 0;
-    if (vec) {
-      Vec16<_Float16> lo, hi, ylo, yhi;
-      lo.raw = *reinterpret_cast<const u32x4*>(xr + i0);
-      hi.raw = *reinterpret_cast<const u32x4*>(xr + half + i0);
+    if (tab) {
+      __syncthreads();                                 // the previous position's table is no longer read
+      for (int32_t i = threadIdx.x; i < half; i += kThreads)
+        sincosf(pos * freq[(int64_t)i * inv_freq.strides[0]], &sn_tab[i], &cs_tab[i]);
+      __syncthreads();
+    }
+    for (int32_t t = threadIdx.x; t < heads * chunks; t += kThreads) {
+      const int32_t h = t / chunks, i0 = (t % chunks) * 8;
+      const bool from_k = h >= num_q_heads;
+      const TensorArg<3>& src = from_k ? k : q;
+      const _Float16* xr = (const _Float16*)src.ptr + s_idx * src.strides[0] + (int64_t)(from_k ? h - num_q_heads : h) * src.strides[1];
+      _Float16* orow = (_Float16*)out.ptr + s_idx * out.strides[0] + (int64_t)h * out.strides[1];
+      auto angle = [&](int32_t i, float* sn, float* cs) {
+        if (tab) {
+          *sn = sn_tab[i];
+          *cs = cs_tab[i];
+        } else {
+          sincosf(pos * freq[(int64_t)i * inv_freq.strides[0]], sn, cs);
+        }
+      };
+      if (vec) {
+        Vec16<_Float16> lo, hi, ylo, yhi;
+        lo.raw = *reinterpret_cast<const u32x4*>(xr + i0);
+        hi.raw = *reinterpret_cast<const u32x4*>(xr + half + i0);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float sn, cs;
-        sincosf(pos * freq[i0 + e], &sn, &cs);
-        const float l = (float)lo.v[e], hv = (float)hi.v[e];
-        ylo.v[e] = (_Float16)(l * cs - hv * sn);
-        yhi.v[e] = (_Float16)(hv * cs + l * sn);
-      }
-      *reinterpret_cast<u32x4*>(orow + i0) = ylo.raw;
-      *reinterpret_cast<u32x4*>(orow + half + i0) = yhi.raw;
-    } else {
-      for (int32_t i = i0; i < min(i0 + 8, half); ++i) {
-        float sn, cs;
-        sincosf(pos * freq[(int64_t)i * inv_freq.strides[0]], &sn, &cs);
-        const float l = (float)xr[(int64_t)i * src.strides[2]], hv = (float)xr[(int64_t)(half + i) * src.strides[2]];
-        orow[(int64_t)i * out.strides[2]] = (_Float16)(l * cs - hv * sn);
-        orow[(int64_t)(half + i) * out.strides[2]] = (_Float16)(hv * cs + l * sn);
+        for (int e = 0; e < 8; ++e) {
+          float sn, cs;
+          angle(i0 + e, &sn, &cs);
+          const float l = (float)lo.v[e], hv = (float)hi.v[e];
+          ylo.v[e] = (_Float16)(l * cs - hv * sn);
+          yhi.v[e] = (_Float16)(hv * cs + l * sn);
+        }
+        *reinterpret_cast<u32x4*>(orow + i0) = ylo.raw;
+        *reinterpret_cast<u32x4*>(orow + half + i0) = yhi.raw;
+      } else {
+        for (int32_t i = i0; i < min(i0 + 8, half); ++i) {
+          float sn, cs;
+          angle(i, &sn, &cs);
+          const float l = (float)xr[(int64_t)i * src.strides[2]], hv = (float)xr[(int64_t)(half + i) * src.strides[2]];
+          orow[(int64_t)i * out.strides[2]] = (_Float16)(l * cs - hv * sn);
+          orow[(int64_t)(half + i) * out.strides[2]] = (_Float16)(hv * cs + l * sn);
+        }
       }
     }
   }

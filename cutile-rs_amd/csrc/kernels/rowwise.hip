@@ -142,6 +142,45 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
   }
 }
 
+// Short rows (head-dimension norms: N = 64 .. 256): LPR lanes per row, one
+// 16-byte vector per lane, 64 / LPR rows per wavefront; the reduction stays
+// inside the LPR-lane group.  With a wavefront per row most lanes would idle.
+template <int LPR>
+__device__ __forceinline__ void rms_norm_rows_short(const _Float16* __restrict__ x, int64_t x_row_stride,
+                                                    const _Float16* __restrict__ w,
+                                                    _Float16* __restrict__ out, int64_t out_row_stride,
+                                                    int32_t n, int64_t rows, float eps,
+                                                    const _Float16* __restrict__ x2 = nullptr, int64_t x2_row_stride = 0,
+                                                    const _Float16* __restrict__ w2 = nullptr, int64_t split = INT64_MAX) {
+  using V = Vec16<_Float16>;
+  constexpr int RPW = 64 / LPR;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t row = ((int64_t)blockIdx.x * kWaves + wave) * RPW + lane / LPR;
+  const int32_t vi = lane % LPR;
+  const bool live = row < rows && vi < (n >> 3);
+  const bool second = row >= split;
+  V xv;
+  float ss = 0.0f;
+  if (live) {
+    const u32x4* xr = reinterpret_cast<const u32x4*>(second ? x2 + (row - split) * x2_row_stride : x + row * x_row_stride);
+    xv.raw = __builtin_nontemporal_load(xr + vi);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float f = (float)xv.v[e];
+      ss = __builtin_fmaf(f, f, ss);
+    }
+  }
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  if (!live) return;
+  const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+  V wv, ov;
+  wv.raw = reinterpret_cast<const u32x4*>(second ? w2 : w)[vi];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ov.v[e] = (_Float16)(((float)xv.v[e] * inv) * (float)wv.v[e]);
+  __builtin_nontemporal_store(ov.raw, reinterpret_cast<u32x4*>(out + row * out_row_stride) + vi);
+}
+
 // add_rms_norm_f16: combined = residual + x stays in f32 registers (it is both
 // the normalised quantity and, rounded, the new residual): two rows read, two
 // rows written, each once.
@@ -440,6 +479,27 @@ RMS_NORM_KERNEL(4, 16)
                             (const _Float16*)k.ptr, k.strides[0], (const _Float16*)kw.ptr,         \
                             (int64_t)num_q_rows);                                                  \
   }
+#define RMS_NORM_SHORT_KERNEL(LPR)                                                                  \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      rms_norm_f16_entry__s##LPR(TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out, float eps,    \
+                                 TileGrid g) {                                                      \
+    int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);                                       \
+    rms_norm_rows_short<LPR>((const _Float16*)x.ptr, x.strides[0], (const _Float16*)w.ptr,         \
+                             (_Float16*)out.ptr, out.strides[0], x.shape[1], rows, eps);           \
+  }                                                                                                 \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      qk_norm_f16_entry__s##LPR(TensorArg<2> q, TensorArg<2> k, TensorArg<1> qw, TensorArg<1> kw,   \
+                                PartitionArg<2> out, float eps, int32_t num_q_rows, TileGrid g) {   \
+    int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);                                       \
+    rms_norm_rows_short<LPR>((const _Float16*)q.ptr, q.strides[0], (const _Float16*)qw.ptr,        \
+                             (_Float16*)out.ptr, out.strides[0], q.shape[1], rows, eps,            \
+                             (const _Float16*)k.ptr, k.strides[0], (const _Float16*)kw.ptr,        \
+                             (int64_t)num_q_rows);                                                 \
+  }
+RMS_NORM_SHORT_KERNEL(8)
+RMS_NORM_SHORT_KERNEL(16)
+RMS_NORM_SHORT_KERNEL(32)
+
 #define FUSED_NORM_VARIANTS(M) \
   M(1, 1) M(1, 2) M(1, 4) M(1, 8) M(2, 2) M(2, 4) M(2, 8) M(4, 1) M(4, 2) M(4, 4) M(4, 8)
 FUSED_NORM_VARIANTS(ADD_RMS_NORM_KERNEL)
