@@ -113,6 +113,11 @@ def lib() -> C.CDLL:
                                           f32, i32, P(LaunchOpts)],
             "cutile_launch_add_2d_f16": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
             "cutile_launch_silu_mul_2d_f16": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_kv_cache_update_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(PartitionArg),
+                                                  P(TensorArg), i32, i32, P(LaunchOpts)],
+            "cutile_launch_fmha_decode_gqa_split": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
+                                                    P(PartitionArg), f32, P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_splitk_reduce_merge": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_rope_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), i32, P(PartitionArg),
                                        i32, P(LaunchOpts)],
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
@@ -353,6 +358,33 @@ def rope_f16(out: Partition, x, inv_freq, position_start=0, *, k=None, num_q_hea
     check(lib().cutile_launch_rope_f16(_stream(stream), C.byref(xa), C.byref(ka) if ka is not None else None, C.byref(fa),
                                        C.byref(pos_dev) if pos_dev is not None else None, int(pos), C.byref(out.arg()),
                                        int(num_q_heads), C.byref(o)))
+
+
+def kv_cache_update_f16(new_k, new_v, k_cache: Partition, v_cache: Partition, position_start, seq_len: int, *, stream=None,
+                        grid=None, generics=None) -> None:
+    """cache[h, position_start + s] = new[s, h] (kv_cache.rs); position_start: int or one-element device tensor"""
+    ka, va = tensor_arg(new_k), tensor_arg(new_v)
+    pos_dev, pos = (None, int(position_start)) if isinstance(position_start, int) else (tensor_arg(position_start, dtype=U32), 0)
+    o, keep = _opts(grid, generics, None)
+    check(lib().cutile_launch_kv_cache_update_f16(_stream(stream), C.byref(ka), C.byref(va), C.byref(k_cache.arg()),
+                                                  C.byref(v_cache.arg()), C.byref(pos_dev) if pos_dev is not None else None,
+                                                  pos, int(seq_len), C.byref(o)))
+
+
+def fmha_decode_gqa_split(q, k, v, att_out: Partition, lse_out: Partition, qk_scale: float, position_start, *, stream=None,
+                          grid=None, generics=None) -> None:
+    """split-KV decode attention (attention.rs:737-902); position_start: one-element device tensor"""
+    qa, ka, va, pa = tensor_arg(q), tensor_arg(k), tensor_arg(v), tensor_arg(position_start, dtype=U32)
+    o, keep = _opts(grid, generics, None)
+    check(lib().cutile_launch_fmha_decode_gqa_split(_stream(stream), C.byref(qa), C.byref(ka), C.byref(va),
+                                                    C.byref(att_out.arg()), C.byref(lse_out.arg()), C.c_float(qk_scale),
+                                                    C.byref(pa), C.byref(o)))
+
+
+def splitk_reduce_merge(att_partial, lse_partial, out: Partition, *, stream=None, grid=None, generics=None) -> None:
+    aa, la = tensor_arg(att_partial), tensor_arg(lse_partial)
+    o, keep = _opts(grid, generics, None)
+    check(lib().cutile_launch_splitk_reduce_merge(_stream(stream), C.byref(aa), C.byref(la), C.byref(out.arg()), C.byref(o)))
 
 
 def gemm(z: Partition, x, y, k: int, *, accumulate: bool = True, stream=None, grid=None, generics=None,

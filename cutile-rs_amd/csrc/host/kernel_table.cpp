@@ -66,6 +66,7 @@ std::vector<KernelEntry> build_table() {
     EW("silu_mul_2d_f16", "f16", "r2_flat", 2); EW("silu_mul_2d_f16", "f16", "r2_tiled", 2);
   }
   add("rope", "f16", "rope_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
+  add("kv_cache_update", "f16", "kv_cache_update_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 #undef EW
   static const char* kCreationTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64", "u8", "u16", "u32"};
   static std::deque<std::string> names;  // keeps generated strings alive at stable addresses
@@ -166,6 +167,15 @@ std::vector<KernelEntry> build_table() {
   fmha("f16", 128, 64, 128);
   fmha("f16", 128, 64, 64);
   fmha("f16", 32, 32, 32);
+
+  // ---- decode attention: one workgroup per (KV head, split); tile = (GROUP, 0, D) ----
+  for (int d : {64, 128, 256})
+    for (int grp : {1, 2, 4, 8}) {
+      std::string v = "f16_g" + std::to_string(grp) + "_d" + std::to_string(d);
+      add("fmha_decode_gqa_split", keep(v), keep("fmha_decode_gqa_split_entry__" + v), IMG_FMHA, 256,
+          (uint32_t)(4 * grp * (d + 2) * 4), grp, 0, d, 0, "f16", 0, 3);
+    }
+  add("splitk_reduce_merge", "f16", "splitk_reduce_merge_entry__f16", IMG_FMHA, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 
   // ---- MXFP8 GEMM: LDS = 2 stages x (BM + BN) x 128 bytes ----
   // "d" = global->LDS direct, pipelined; scales staged in blocks of four K tiles (16 bytes per row, two blocks)

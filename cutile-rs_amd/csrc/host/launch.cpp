@@ -817,6 +817,168 @@ cutile_status_t cutile_launch_rope_f16(cutile_stream_t stream, const cutile_tens
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// kv_cache_update_seq_f16 / kv_cache_update_seq_dynpos_f16: the start position by value or from device memory.
+cutile_status_t cutile_launch_kv_cache_update_f16(cutile_stream_t stream, const cutile_tensor_arg_t* new_k,
+                                                  const cutile_tensor_arg_t* new_v, const cutile_partition_arg_t* k_cache,
+                                                  const cutile_partition_arg_t* v_cache,
+                                                  const cutile_tensor_arg_t* position_start_dev, int32_t position_start,
+                                                  int32_t seq_len, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(new_k, "new_k", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(new_v, "new_v", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(k_cache, "k_cache", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(v_cache, "v_cache", 3, 3)) return s;
+  const cutile_tensor_arg_t& kc = k_cache->tensor;
+  const cutile_tensor_arg_t& vc = v_cache->tensor;
+  const int32_t d = new_k->shape[2];
+  CUTILE_REQUIRE(new_k->dtype == CUTILE_DTYPE_F16 && new_v->dtype == CUTILE_DTYPE_F16 && kc.dtype == CUTILE_DTYPE_F16 &&
+                     vc.dtype == CUTILE_DTYPE_F16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: every tensor must be f16");
+  CUTILE_REQUIRE(new_v->shape[2] == d && kc.shape[2] == d && vc.shape[2] == d && new_v->shape[0] == new_k->shape[0] &&
+                     new_v->shape[1] == new_k->shape[1] && vc.shape[0] == kc.shape[0] && kc.shape[0] <= new_k->shape[1],
+                 CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: new_k/new_v [seq, heads, D] and the caches [heads, max_seq, D] do not agree");
+  CUTILE_REQUIRE(seq_len >= 0 && seq_len <= new_k->shape[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "kv_cache_update: seq_len = %d but new_k holds %d positions", seq_len, new_k->shape[0]);
+  const int32_t block = k_cache->partition_shape[2];
+  CUTILE_REQUIRE(k_cache->partition_shape[0] == 1 && v_cache->partition_shape[0] == 1 && block > 0 && d % block == 0 &&
+                     v_cache->partition_shape[1] == k_cache->partition_shape[1] && v_cache->partition_shape[2] == block,
+                 CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: caches must be partitioned [1, rows, BLOCK_SIZE] with BLOCK_SIZE dividing D = %d", d);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(block), "BLOCK_SIZE")) return s;
+  uint32_t explicit_grid[3] = {0, 0, 0};
+  if (opts) memcpy(explicit_grid, opts->grid, sizeof(explicit_grid));
+  const cutile_partition_arg_t* parts[2] = {k_cache, v_cache};
+  uint32_t tg[3];
+  if (cutile_status_t s = cutile_infer_launch_grid(explicit_grid, parts, 2, tg)) return s;
+  CUTILE_REQUIRE((int64_t)tg[2] * block >= d, CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: the launch grid must cover all of D");
+  if (position_start_dev) {
+    if (cutile_status_t s = check_tensor(position_start_dev, "position_start", 1, 1)) return s;
+    CUTILE_REQUIRE(position_start_dev->dtype == CUTILE_DTYPE_U32 && position_start_dev->shape[0] == 1 &&
+                       ((uintptr_t)position_start_dev->ptr & 3) == 0,
+                   CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: position_start must be one aligned u32");
+  } else {
+    // kv_cache.rs:27 "_position_start ... asserted == 0 at call site": the prefill form writes rows 0..seq_len
+    CUTILE_REQUIRE(position_start == 0, CUTILE_ERR_KERNEL_LAUNCH,
+                   "kv_cache_update_seq_f16 writes cache rows 0..seq_len; position_start must be 0 (got %d), use the "
+                   "device-position form for other offsets", position_start);
+    CUTILE_REQUIRE((int64_t)seq_len <= std::min(kc.shape[1], vc.shape[1]) &&
+                       (int64_t)seq_len <= (int64_t)tg[1] * k_cache->partition_shape[1],
+                   CUTILE_ERR_KERNEL_LAUNCH, "kv_cache_update: %d rows do not fit the cache rows the launch covers", seq_len);
+  }
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("kv_cache_update", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*new_k);
+  args.push_tensor(*new_v);
+  args.push_partition(*k_cache);
+  args.push_partition(*v_cache);
+  args.push_val<const void*>(position_start_dev ? position_start_dev->ptr : nullptr);
+  args.push_val<int32_t>(position_start);
+  args.push_val<int32_t>(seq_len);
+  args.push_tile_grid(tg);
+  const uint64_t lanes = (uint64_t)seq_len * std::min<uint32_t>(tg[0], kc.shape[0]) * std::max(1, d / 8);
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(lanes, 256), 1u << 16)), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+static bool decode_vec_layout(const cutile_tensor_arg_t& t) {
+  return t.strides[2] == 1 && t.strides[1] % 8 == 0 && t.strides[0] % 8 == 0 && aligned16(t.ptr);
+}
+
+cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                                    const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                                    const cutile_partition_arg_t* att_out,
+                                                    const cutile_partition_arg_t* lse_out, float qk_scale,
+                                                    const cutile_tensor_arg_t* position_start,
+                                                    const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(q, "q", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(k, "k", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(v, "v", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(att_out, "att_out", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(lse_out, "lse_out", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(position_start, "position_start", 1, 1)) return s;
+  const cutile_tensor_arg_t& at = att_out->tensor;
+  const cutile_tensor_arg_t& lt = lse_out->tensor;
+  const int32_t kv_heads = q->shape[0], group = q->shape[1], d = q->shape[2];
+  CUTILE_REQUIRE(q->dtype == CUTILE_DTYPE_F16 && k->dtype == CUTILE_DTYPE_F16 && v->dtype == CUTILE_DTYPE_F16 &&
+                     at.dtype == CUTILE_DTYPE_F16 && lt.dtype == CUTILE_DTYPE_F32 && position_start->dtype == CUTILE_DTYPE_U32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha_decode_gqa_split: q, k, v, att_out are f16, lse_out f32, position_start u32");
+  CUTILE_REQUIRE(k->shape[0] == kv_heads && v->shape[0] == kv_heads && k->shape[2] == d && v->shape[2] == d &&
+                     at.shape[0] == kv_heads && at.shape[2] == d && lt.shape[0] == kv_heads && at.shape[1] == lt.shape[1] &&
+                     at.shape[1] % group == 0 && position_start->shape[0] == 1,
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha_decode_gqa_split: q [kv_heads, GROUP, D], k/v [kv_heads, max_seq, D], "
+                 "att_out [kv_heads, NUM_KV_SPLITS*GROUP, D] and lse_out [kv_heads, NUM_KV_SPLITS*GROUP] do not agree");
+  CUTILE_REQUIRE(att_out->partition_shape[0] == 1 && att_out->partition_shape[1] == group && att_out->partition_shape[2] == d &&
+                     lse_out->partition_shape[0] == 1 && lse_out->partition_shape[1] == group,
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha_decode_gqa_split: att_out must be partitioned [1, %d, %d] and lse_out [1, %d]", group, d, group);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(group), "GROUP")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(d), "D")) return s;
+  const int bn = generic_int(opts, 1, 64);
+  CUTILE_REQUIRE(bn > 0, CUTILE_ERR_KERNEL_LAUNCH, "fmha_decode_gqa_split: BN must be positive");
+  uint32_t explicit_grid[3] = {0, 0, 0};
+  if (opts) memcpy(explicit_grid, opts->grid, sizeof(explicit_grid));
+  const cutile_partition_arg_t* parts[2] = {att_out, lse_out};
+  uint32_t tg[3];
+  if (cutile_status_t s = cutile_infer_launch_grid(explicit_grid, parts, 2, tg)) return s;
+  if (cutile_status_t s = check_generic(opts, 3, std::to_string(tg[1]), "NUM_KV_SPLITS")) return s;
+  CUTILE_REQUIRE(decode_vec_layout(*q) && decode_vec_layout(*k) && decode_vec_layout(*v) && decode_vec_layout(at) &&
+                     ((uintptr_t)position_start->ptr & 3) == 0 && ((uintptr_t)lt.ptr & 3) == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "fmha_decode_gqa_split: precompiled variants need unit head-dim stride and 16-byte aligned rows");
+  const std::string want = "f16_g" + std::to_string(group) + "_d" + std::to_string(d);
+  CUTILE_REQUIRE(find_entry("fmha_decode_gqa_split", want), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of fmha_decode_gqa_split<GROUP=%d, D=%d>; available: %s", group, d,
+                 list_variants("fmha_decode_gqa_split").c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("fmha_decode_gqa_split", opts, want, {want}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*q);
+  args.push_tensor(*k);
+  args.push_tensor(*v);
+  args.push_partition(*att_out);
+  args.push_partition(*lse_out);
+  args.push_val<float>(qk_scale);
+  args.push_val<const void*>(position_start->ptr);
+  args.push_val<int32_t>(bn);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {std::min<uint32_t>(tg[0], (uint32_t)kv_heads), tg[1], 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const cutile_tensor_arg_t* att_partial,
+                                                  const cutile_tensor_arg_t* lse_partial, const cutile_partition_arg_t* out,
+                                                  const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(att_partial, "att_partial", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(lse_partial, "lse_partial", 2, 2)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 3, 3)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  const int32_t group = ot.shape[1], d = ot.shape[2];
+  CUTILE_REQUIRE(att_partial->dtype == CUTILE_DTYPE_F16 && lse_partial->dtype == CUTILE_DTYPE_F32 && ot.dtype == CUTILE_DTYPE_F16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "splitk_reduce_merge: att_partial and out are f16, lse_partial f32");
+  CUTILE_REQUIRE(group > 0 && att_partial->shape[0] >= ot.shape[0] && lse_partial->shape[0] >= ot.shape[0] &&
+                     att_partial->shape[2] == d && att_partial->shape[1] == lse_partial->shape[1] &&
+                     att_partial->shape[1] % group == 0 && att_partial->shape[1] >= group,
+                 CUTILE_ERR_KERNEL_LAUNCH, "splitk_reduce_merge: att_partial [kv_heads, NUM_KV_SPLITS*GROUP, D], lse_partial "
+                 "[kv_heads, NUM_KV_SPLITS*GROUP] and out [kv_heads, GROUP, D] do not agree");
+  const int32_t chunk = out->partition_shape[2];
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == group && chunk > 0 && d % chunk == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "splitk_reduce_merge: out must be partitioned [1, %d, CHUNK_D] with CHUNK_D dividing D = %d", group, d);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(group), "GROUP")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(chunk), "CHUNK_D")) return s;
+  if (cutile_status_t s = check_generic(opts, 3, std::to_string(att_partial->shape[1] / group), "NUM_KV_SPLITS")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  CUTILE_REQUIRE((int64_t)tg[2] * chunk >= d, CUTILE_ERR_KERNEL_LAUNCH, "splitk_reduce_merge: the launch grid must cover all of D");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("splitk_reduce_merge", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*att_partial);
+  args.push_tensor(*lse_partial);
+  args.push_partition(*out);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {std::min<uint32_t>(tg[0], (uint32_t)ot.shape[0]), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
                                       const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts) {
   if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;

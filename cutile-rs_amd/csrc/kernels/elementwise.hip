@@ -245,6 +245,47 @@ extern "C" __global__ void __launch_bounds__(kThreads)
   });
 }
 
+// ---- KV cache update ------------------------------------------------------------------------
+// kv_cache_update_seq_f16 / kv_cache_update_seq_dynpos_f16 (cutile-kernels/src/kv_cache.rs:15-49,
+// 58-97): cache[h, position_start + s, :] = new[s, h, :] for s < seq_len, K and V together.
+// new_* are [seq, heads, D], the caches [heads, max_seq, D].  Rows that would land
+// beyond max_seq are dropped.  16 bytes per lane when the layout allows it.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    kv_cache_update_entry__f16(TensorArg<3> new_k, TensorArg<3> new_v, PartitionArg<3> k_cache, PartitionArg<3> v_cache,
+                               const uint32_t* pos_dev, int32_t position_start, int32_t seq_len, TileGrid g) {
+  const int32_t d = new_k.shape[2], heads = min((int32_t)g.x, k_cache.shape[0]);
+  const int32_t base = pos_dev ? (int32_t)pos_dev[0] : position_start;
+  const int32_t max_seq = min(k_cache.shape[1], v_cache.shape[1]);
+  auto vec_ok = [&](const void* p, const int32_t* st) {
+    return st[2] == 1 && st[1] % 8 == 0 && st[0] % 8 == 0 && ((uintptr_t)p & 15) == 0;
+  };
+  const bool vec = d % 8 == 0 && vec_ok(new_k.ptr, new_k.strides) && vec_ok(new_v.ptr, new_v.strides) &&
+                   vec_ok(k_cache.ptr, k_cache.strides) && vec_ok(v_cache.ptr, v_cache.strides);
+  const int32_t per_row = vec ? d / 8 : d;
+  const int64_t total = (int64_t)seq_len * heads * per_row;
+  for (int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
+    const int32_t c = (int32_t)(t % per_row);
+    const int64_t sh = t / per_row;
+    const int32_t h = (int32_t)(sh % heads);
+    const int64_t sidx = sh / heads;
+    const int64_t pos = base + sidx;
+    if (pos < 0 || pos >= max_seq) continue;
+    const int64_t src_k = sidx * new_k.strides[0] + (int64_t)h * new_k.strides[1];
+    const int64_t src_v = sidx * new_v.strides[0] + (int64_t)h * new_v.strides[1];
+    const int64_t dst_k = (int64_t)h * k_cache.strides[0] + pos * k_cache.strides[1];
+    const int64_t dst_v = (int64_t)h * v_cache.strides[0] + pos * v_cache.strides[1];
+    if (vec) {
+      *reinterpret_cast<u32x4*>((_Float16*)k_cache.ptr + dst_k + c * 8) =
+          *reinterpret_cast<const u32x4*>((const _Float16*)new_k.ptr + src_k + c * 8);
+      *reinterpret_cast<u32x4*>((_Float16*)v_cache.ptr + dst_v + c * 8) =
+          *reinterpret_cast<const u32x4*>((const _Float16*)new_v.ptr + src_v + c * 8);
+    } else {
+      ((_Float16*)k_cache.ptr)[dst_k + (int64_t)c * k_cache.strides[2]] = ((const _Float16*)new_k.ptr)[src_k + (int64_t)c * new_k.strides[2]];
+      ((_Float16*)v_cache.ptr)[dst_v + (int64_t)c * v_cache.strides[2]] = ((const _Float16*)new_v.ptr)[src_v + (int64_t)c * new_v.strides[2]];
+    }
+  }
+}
+
 // ---- rotary position embedding -------------------------------------------------------------
 // rope_seq_f16 / rope_seq_dynpos_f16 / qk_rope_dynpos_f16 (cutile-kernels/src/positional.rs:13-64,
 // 70-130, 136-230): x [seq, heads, D] split in halves lo = [.., :D/2], hi = [.., D/2:];

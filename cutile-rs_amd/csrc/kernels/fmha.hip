@@ -661,6 +661,159 @@ struct FmhaPingPong {
   }
 };
 
+// ---- decode attention: split over the KV sequence, then merge ---------------------------------
+// fmha_decode_gqa_split / splitk_reduce_merge (cutile-kernels/src/attention.rs:737-902, 917-1013).
+// One new token: the GROUP query heads that share KV head h attend to keys
+// 0..input_pos of that head's cache.  A workgroup takes one (KV head, split) and
+// streams its share of the cache once; this is bandwidth work (every K and V
+// byte is used for GROUP dot products), so it runs on the vector ALUs:
+//  * a cache row of D halves is spread over D/8 lanes (16-byte loads), so a
+//    wavefront takes 512/D rows at a time and the four wavefronts interleave;
+//  * every row slot keeps its own online-softmax state (m, l, acc) in the log2
+//    domain; slots are merged by shuffles, wavefronts through LDS;
+//  * the partial result is normalised and stored with its log-sum-exp,
+//    lse = m + log2(l), as the merge kernel expects.  p is rounded to f16
+//    before it multiplies V, as in the tile program; a split with no keys
+//    stores att = 0 and lse = -1e30 + log2(BN) (the tile program's initial state).
+template <int G, int D>
+__device__ __forceinline__ void decode_split(const TensorArg<3>& q, const TensorArg<3>& k, const TensorArg<3>& v,
+                                             const PartitionArg<3>& att_out, const PartitionArg<2>& lse_out,
+                                             float qk_scale, const uint32_t* pos_dev, int32_t bn, const TileGrid& g) {
+  constexpr int LPR = D / 8, RPW = 64 / LPR, kWaves = 4;
+  static_assert(D % 8 == 0 && 64 % LPR == 0 && LPR <= 64, "head dimension");
+  __shared__ float sm[kWaves][G], sl[kWaves][G];
+  __shared__ __attribute__((aligned(16))) float sacc[kWaves][G][D];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int slot = lane / LPR, dl = lane % LPR;
+  const int32_t head = blockIdx.x, split = blockIdx.y, splits = (int32_t)g.y;
+  const int32_t max_seq = min(k.shape[1], v.shape[1]);
+  const int32_t s_kv = min((int32_t)pos_dev[0] + 1, max_seq);
+  const int32_t tiles = (s_kv + bn - 1) / bn, per_split = (tiles + splits - 1) / splits;
+  const int32_t r0 = split * per_split * bn;
+  const int32_t r1 = min(min((split + 1) * per_split, tiles) * bn, s_kv);
+  const float c = qk_scale * kLog2e;
+
+  float qv[G][8];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    const _Float16* qr = (const _Float16*)q.ptr + (int64_t)head * q.strides[0] + (int64_t)gi * q.strides[1] + dl * 8;
+    f16x8 t = *reinterpret_cast<const f16x8*>(qr);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[gi][e] = (float)t[e] * c;   // scale folded into q: s is in the log2 domain
+  }
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    m[gi] = -1.0e30f;
+    l[gi] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[gi][e] = 0.0f;
+  }
+  const _Float16* kb = (const _Float16*)k.ptr + (int64_t)head * k.strides[0] + dl * 8;
+  const _Float16* vb = (const _Float16*)v.ptr + (int64_t)head * v.strides[0] + dl * 8;
+  for (int32_t base = r0 + wave * RPW; base < r1; base += kWaves * RPW) {   // wavefront-uniform trip count
+    const int32_t row = base + slot;
+    const bool valid = row < r1;
+    f16x8 kr = {}, vr = {};
+    if (valid) {
+      kr = *reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1]);
+      vr = *reinterpret_cast<const f16x8*>(vb + (int64_t)row * v.strides[1]);
+    }
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+      float sdot = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sdot = __builtin_fmaf((float)kr[e], qv[gi][e], sdot);
+#pragma unroll
+      for (int o = LPR / 2; o > 0; o >>= 1) sdot += __shfl_xor(sdot, o, 64);
+      const float m_new = valid ? fmaxf(m[gi], sdot) : m[gi];
+      const float alpha = __builtin_amdgcn_exp2f(m[gi] - m_new);
+      const float p = valid ? __builtin_amdgcn_exp2f(sdot - m_new) : 0.0f;
+      l[gi] = l[gi] * alpha + p;
+      const float ph = (float)(_Float16)p;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[gi][e] = __builtin_fmaf((float)vr[e], ph, acc[gi][e] * alpha);
+      m[gi] = m_new;
+    }
+  }
+  // merge the row slots of this wavefront ...
+#pragma unroll
+  for (int o = LPR; o < 64; o <<= 1) {
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+      const float mo = __shfl_xor(m[gi], o, 64), lo = __shfl_xor(l[gi], o, 64);
+      const float m_new = fmaxf(m[gi], mo);
+      const float fs = __builtin_amdgcn_exp2f(m[gi] - m_new), fo = __builtin_amdgcn_exp2f(mo - m_new);
+      l[gi] = l[gi] * fs + lo * fo;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[gi][e] = acc[gi][e] * fs + __shfl_xor(acc[gi][e], o, 64) * fo;
+      m[gi] = m_new;
+    }
+  }
+  // ... and the wavefronts through LDS
+  if (slot == 0) {
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+      if (dl == 0) {
+        sm[wave][gi] = m[gi];
+        sl[wave][gi] = l[gi];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sacc[wave][gi][dl * 8 + e] = acc[gi][e];
+    }
+  }
+  __syncthreads();
+  if (wave == 0 && slot == 0) {
+    _Float16* ab = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + dl * 8;
+    float* lb = (float*)lse_out.ptr + (int64_t)head * lse_out.strides[0];
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+      float mt = sm[0][gi];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) mt = fmaxf(mt, sm[w][gi]);
+      float lt = 0.0f, at[8] = {};
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float f = __builtin_amdgcn_exp2f(sm[w][gi] - mt);
+        lt += sl[w][gi] * f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) at[e] += sacc[w][gi][dl * 8 + e] * f;
+      }
+      if (r0 >= r1) lt = (float)bn;   // no keys in this split: the tile program's untouched l = 1 per lane
+      const float safe = fmaxf(lt, 1.0e-8f);
+      const int64_t orow = (int64_t)split * G + gi;
+      f16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (_Float16)(at[e] / safe);
+      *reinterpret_cast<f16x8*>(ab + orow * att_out.strides[1]) = o;
+      if (dl == 0) lb[orow * lse_out.strides[1]] = mt + __builtin_log2f(safe);
+    }
+  }
+}
+
+// out[h, g, :] = sum_s w[g, s] att[h, s*GROUP + g, :], w = exp2(lse - max_s lse) / max(sum, 1e-8).
+__device__ __forceinline__ void splitk_merge(const TensorArg<3>& att, const TensorArg<2>& lse, const PartitionArg<3>& out) {
+  const int32_t head = blockIdx.x, group = out.shape[1], d = out.shape[2];
+  const int32_t splits = att.shape[1] / group;
+  const _Float16* ab = (const _Float16*)att.ptr + (int64_t)head * att.strides[0];
+  const float* lb = (const float*)lse.ptr + (int64_t)head * lse.strides[0];
+  _Float16* ob = (_Float16*)out.ptr + (int64_t)head * out.strides[0];
+  for (int32_t idx = threadIdx.x; idx < group * d; idx += blockDim.x) {
+    const int32_t gi = idx / d, cidx = idx % d;
+    float mx = -INFINITY, sum = 0.0f;
+    for (int32_t sidx = 0; sidx < splits; ++sidx) mx = fmaxf(mx, lb[(int64_t)(sidx * group + gi) * lse.strides[1]]);
+    for (int32_t sidx = 0; sidx < splits; ++sidx)
+      sum += __builtin_amdgcn_exp2f(lb[(int64_t)(sidx * group + gi) * lse.strides[1]] - mx);
+    const float safe = fmaxf(sum, 1.0e-8f);
+    float o = 0.0f;
+    for (int32_t sidx = 0; sidx < splits; ++sidx) {
+      const float w = __builtin_amdgcn_exp2f(lb[(int64_t)(sidx * group + gi) * lse.strides[1]] - mx) / safe;
+      o += (float)ab[(int64_t)(sidx * group + gi) * att.strides[1] + (int64_t)cidx * att.strides[2]] * w;
+    }
+    ob[(int64_t)gi * out.strides[1] + (int64_t)cidx * out.strides[2]] = (_Float16)o;
+  }
+}
+
 }  // namespace
 
 #define FMHA_KERNEL(NAME, T, BM, BN, D)                                                           \
@@ -692,3 +845,24 @@ FMHA_KERNEL(f16, _Float16, 32, 32, 32)
 
 FMHA_PINGPONG_KERNEL(bf16, __bf16, 64, 128)
 FMHA_PINGPONG_KERNEL(f16, _Float16, 64, 128)
+
+// fmha_decode_gqa_split<GROUP, BN, D, NUM_KV_SPLITS>(q, k, v, att_out: [1,GROUP,D] tiles, lse_out: [1,GROUP] tiles,
+//                                                   qk_scale, position_start); grid (kv_heads, NUM_KV_SPLITS)
+#define DECODE_SPLIT_KERNEL(G, D)                                                                  \
+  extern "C" __global__ void __launch_bounds__(256)                                               \
+      fmha_decode_gqa_split_entry__f16_g##G##_d##D(TensorArg<3> q, TensorArg<3> k, TensorArg<3> v, \
+                                                   PartitionArg<3> att_out, PartitionArg<2> lse_out, \
+                                                   float qk_scale, const uint32_t* position_start, \
+                                                   int32_t bn, TileGrid g) {                       \
+    decode_split<G, D>(q, k, v, att_out, lse_out, qk_scale, position_start, bn, g);               \
+  }
+#define DECODE_SPLIT_GROUPS(D) DECODE_SPLIT_KERNEL(1, D) DECODE_SPLIT_KERNEL(2, D) DECODE_SPLIT_KERNEL(4, D) DECODE_SPLIT_KERNEL(8, D)
+DECODE_SPLIT_GROUPS(64)
+DECODE_SPLIT_GROUPS(128)
+DECODE_SPLIT_GROUPS(256)
+
+// splitk_reduce_merge<GROUP, D, CHUNK_D, NUM_KV_SPLITS, ..>(att_partial, lse_partial, out: [1,GROUP,CHUNK_D] tiles)
+extern "C" __global__ void __launch_bounds__(256)
+    splitk_reduce_merge_entry__f16(TensorArg<3> att_partial, TensorArg<2> lse_partial, PartitionArg<3> out, TileGrid g) {
+  splitk_merge(att_partial, lse_partial, out);
+}

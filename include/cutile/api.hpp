@@ -419,6 +419,38 @@ struct QkRopeDynposF16Fn {
     return cutile_launch_rope_f16(s, &qa, &ka, &fa, &pa, 0, &op, num_q_heads, o);
   }
 };
+struct KvCacheUpdateSeqF16Fn {
+  template <class NK, class NV, class KC, class VC>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, NK& new_k, NV& new_v, KC& k_cache, VC& v_cache, int32_t position_start, int32_t seq_len) {
+    auto ka = input_arg(new_k), va = input_arg(new_v);
+    auto kp = k_cache.arg(), vp = v_cache.arg();
+    return cutile_launch_kv_cache_update_f16(s, &ka, &va, &kp, &vp, nullptr, position_start, seq_len, o);
+  }
+};
+struct KvCacheUpdateSeqDynposF16Fn {
+  template <class NK, class NV, class KC, class VC, class P>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, NK& new_k, NV& new_v, KC& k_cache, VC& v_cache, P& position_start, int32_t seq_len) {
+    auto ka = input_arg(new_k), va = input_arg(new_v), pa = input_arg(position_start);
+    auto kp = k_cache.arg(), vp = v_cache.arg();
+    return cutile_launch_kv_cache_update_f16(s, &ka, &va, &kp, &vp, &pa, 0, seq_len, o);
+  }
+};
+struct FmhaDecodeGqaSplitFn {
+  template <class Q, class K, class V, class A, class L, class P>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, A& att_out, L& lse_out, float qk_scale, P& position_start) {
+    auto qa = input_arg(q), ka = input_arg(k), va = input_arg(v), pa = input_arg(position_start);
+    auto ap = att_out.arg(), lp = lse_out.arg();
+    return cutile_launch_fmha_decode_gqa_split(s, &qa, &ka, &va, &ap, &lp, qk_scale, &pa, o);
+  }
+};
+struct SplitkReduceMergeFn {
+  template <class A, class L, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, A& att_partial, L& lse_partial, O& out) {
+    auto aa = input_arg(att_partial), la = input_arg(lse_partial);
+    auto op = out.arg();
+    return cutile_launch_splitk_reduce_merge(s, &aa, &la, &op, o);
+  }
+};
 }  // namespace kernels
 
 // saxpy(y: partition, a, x) -> (y, a, x)        cutile-examples/examples/saxpy.rs:12-17
@@ -453,6 +485,15 @@ template <class X, class F, class O> auto rope_seq_f16(X&& x, F&& inv_freq, O&& 
 template <class X, class F, class P, class O> auto rope_seq_dynpos_f16(X&& x, F&& inv_freq, P&& position_start, O&& out) { return make_launcher<kernels::RopeSeqDynposF16Fn>(std::forward<X>(x), std::forward<F>(inv_freq), std::forward<P>(position_start), std::forward<O>(out)); }
 // qk_rope_dynpos_f16(q, k, inv_freq, position_start, out, num_q_heads)         positional.rs:141-148
 template <class Q, class K, class F, class P, class O> auto qk_rope_dynpos_f16(Q&& q, K&& k, F&& inv_freq, P&& position_start, O&& out, int32_t num_q_heads) { return make_launcher<kernels::QkRopeDynposF16Fn>(std::forward<Q>(q), std::forward<K>(k), std::forward<F>(inv_freq), std::forward<P>(position_start), std::forward<O>(out), num_q_heads); }
+
+// kv_cache_update_seq_f16(new_k, new_v, k_cache: [1,BM_S,BLOCK], v_cache, position_start (= 0), seq_len)   cutile-kernels/src/kv_cache.rs:21-28
+template <class NK, class NV, class KC, class VC> auto kv_cache_update_seq_f16(NK&& new_k, NV&& new_v, KC&& k_cache, VC&& v_cache, int32_t position_start, int32_t seq_len) { return make_launcher<kernels::KvCacheUpdateSeqF16Fn>(std::forward<NK>(new_k), std::forward<NV>(new_v), std::forward<KC>(k_cache), std::forward<VC>(v_cache), position_start, seq_len); }
+// kv_cache_update_seq_dynpos_f16(new_k, new_v, k_cache: [1,MAX_SEQ,BLOCK], v_cache, position_start: [1] u32, seq_len)   kv_cache.rs:68-79
+template <class NK, class NV, class KC, class VC, class P> auto kv_cache_update_seq_dynpos_f16(NK&& new_k, NV&& new_v, KC&& k_cache, VC&& v_cache, P&& position_start, int32_t seq_len) { return make_launcher<kernels::KvCacheUpdateSeqDynposF16Fn>(std::forward<NK>(new_k), std::forward<NV>(new_v), std::forward<KC>(k_cache), std::forward<VC>(v_cache), std::forward<P>(position_start), seq_len); }
+// fmha_decode_gqa_split(q, k, v, att_out: [1,GROUP,D], lse_out: [1,GROUP], qk_scale, position_start: [1] u32)   cutile-kernels/src/attention.rs:737-755
+template <class Q, class K, class V, class A, class L, class P> auto fmha_decode_gqa_split(Q&& q, K&& k, V&& v, A&& att_out, L&& lse_out, float qk_scale, P&& position_start) { return make_launcher<kernels::FmhaDecodeGqaSplitFn>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<A>(att_out), std::forward<L>(lse_out), qk_scale, std::forward<P>(position_start)); }
+// splitk_reduce_merge(att_partial, lse_partial, out: [1,GROUP,CHUNK_D])          attention.rs:917-930
+template <class A, class L, class O> auto splitk_reduce_merge(A&& att_partial, L&& lse_partial, O&& out) { return make_launcher<kernels::SplitkReduceMergeFn>(std::forward<A>(att_partial), std::forward<L>(lse_partial), std::forward<O>(out)); }
 
 namespace api {
 template <class T> struct is_graph_node_memcpy : std::true_type {};

@@ -357,6 +357,29 @@ cutile_status_t cutile_launch_rope_f16(cutile_stream_t stream, const cutile_tens
                                        const cutile_tensor_arg_t* position_start_dev, int32_t position_start,
                                        const cutile_partition_arg_t* out, int32_t num_q_heads,
                                        const cutile_launch_opts_t* opts);
+/* KV cache update: cache[h, position_start + s, :] = new[s, h, :] for s < seq_len, K and V together; caches
+ * partitioned [1, rows, BLOCK_SIZE].  One entry point for kv_cache_update_seq_f16 (position_start_dev NULL; the
+ * by-value position must be 0 as the reference's call sites assert) and kv_cache_update_seq_dynpos_f16
+ * (position_start_dev: one u32) — cutile-kernels/src/kv_cache.rs:15-49, 58-97 */
+cutile_status_t cutile_launch_kv_cache_update_f16(cutile_stream_t stream, const cutile_tensor_arg_t* new_k,
+                                                  const cutile_tensor_arg_t* new_v, const cutile_partition_arg_t* k_cache,
+                                                  const cutile_partition_arg_t* v_cache,
+                                                  const cutile_tensor_arg_t* position_start_dev, int32_t position_start,
+                                                  int32_t seq_len, const cutile_launch_opts_t* opts);
+/* fmha_decode_gqa_split<GROUP, BN, D, NUM_KV_SPLITS>(q [kv_heads,GROUP,D], k, v [kv_heads,max_seq,D],
+ * att_out: [1,GROUP,D] tiles of [kv_heads, NUM_KV_SPLITS*GROUP, D], lse_out: [1,GROUP] tiles, qk_scale,
+ * position_start: [1] u32): keys 0..position_start, split over grid.y — cutile-kernels/src/attention.rs:737-902 */
+cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                                    const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                                    const cutile_partition_arg_t* att_out,
+                                                    const cutile_partition_arg_t* lse_out, float qk_scale,
+                                                    const cutile_tensor_arg_t* position_start,
+                                                    const cutile_launch_opts_t* opts);
+/* splitk_reduce_merge<GROUP, D, CHUNK_D, NUM_KV_SPLITS>(att_partial, lse_partial, out: [1,GROUP,CHUNK_D] tiles):
+ * softmax-weighted sum of the splits — cutile-kernels/src/attention.rs:917-1013 */
+cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const cutile_tensor_arg_t* att_partial,
+                                                  const cutile_tensor_arg_t* lse_partial, const cutile_partition_arg_t* out,
+                                                  const cutile_launch_opts_t* opts);
 /* gemm<T, BM, BN, BK>(z: [BM,BN] tiles, x, y, k): z <- z + x·y with f32
  * accumulation (z is read as the initial accumulator, like the reference bench;
  * `accumulate` = 0 starts from zero like the example) —

@@ -59,6 +59,9 @@ def lib() -> C.CDLL:
             "orc_add_f16": (None, [sz, vp, vp, vp]),
             "orc_silu_mul_f16": (None, [sz, vp, vp, vp]),
             "orc_rope_seq_f16": (None, [vp, vp, vp, i64, i64, i64, C.c_int32]),
+            "orc_kv_cache_update_f16": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64]),
+            "orc_fmha_decode_gqa_split": (None, [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, f32, i64]),
+            "orc_splitk_reduce_merge": (None, [vp, vp, vp, i64, i64, i64, i64]),
             "orc_softmax_f32": (None, [vp, vp, i64, i64, i64, i64]),
             "orc_softmax_f16": (None, [vp, vp, i64, i64, i64, i64]),
             "orc_cpu_gemm_f32": (None, [vp, vp, vp, i64, i64, i64]),
@@ -218,6 +221,35 @@ def rope_seq_f16(x_bits, inv_freq, position_start: int) -> np.ndarray:
     assert f.size == d // 2
     out = np.empty_like(x)
     lib().orc_rope_seq_f16(_p(x), _p(f), _p(out), seq, heads, d, position_start)
+    return out
+
+
+def kv_cache_update_f16(new_k_bits, new_v_bits, k_cache_bits, v_cache_bits, position_start: int, seq_len: int):
+    """-> (k_cache, v_cache) copies with cache[h, position_start + s] = new[s, h] for s < seq_len"""
+    nk, nv = _c(new_k_bits, np.uint16), _c(new_v_bits, np.uint16)
+    kc, vc = _c(k_cache_bits, np.uint16).copy(), _c(v_cache_bits, np.uint16).copy()
+    heads, max_seq, d = kc.shape
+    lib().orc_kv_cache_update_f16(_p(nk), _p(nv), _p(kc), _p(vc), heads, d, max_seq, position_start, seq_len)
+    return kc, vc
+
+
+def fmha_decode_gqa_split(q_bits, k_bits, v_bits, qk_scale: float, input_pos: int, bn: int, splits: int):
+    """-> (att_partial [kv_heads, splits*group, d] f16 bits, lse_partial [kv_heads, splits*group] f32)"""
+    q, k, v = _c(q_bits, np.uint16), _c(k_bits, np.uint16), _c(v_bits, np.uint16)
+    kv_heads, group, d = q.shape
+    max_seq = k.shape[1]
+    att = np.empty((kv_heads, splits * group, d), np.uint16)
+    lse = np.empty((kv_heads, splits * group), np.float32)
+    lib().orc_fmha_decode_gqa_split(_p(q), _p(k), _p(v), _p(att), _p(lse), kv_heads, group, d, max_seq, bn, splits,
+                                    qk_scale, input_pos)
+    return att, lse
+
+
+def splitk_reduce_merge(att_bits, lse, group: int) -> np.ndarray:
+    att, lse = _c(att_bits, np.uint16), _c(lse, np.float32)
+    kv_heads, ns_group, d = att.shape
+    out = np.empty((kv_heads, group, d), np.uint16)
+    lib().orc_splitk_reduce_merge(_p(att), _p(lse), _p(out), kv_heads, group, d, ns_group // group)
     return out
 
 

@@ -348,6 +348,112 @@ void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, i
 }
 
 /* ------------------------------------------------------------------------ */
+/* KV cache update and decode attention (cutile-kernels/src/{kv_cache,attention}.rs) */
+/* ------------------------------------------------------------------------ */
+/* kv_cache.rs:15-49 and :58-97: cache[h, position_start + s, :] = new[s, h, :] for s < seq_len.
+ * new_* are [seq, heads, d]; caches are [heads, max_seq, d]. */
+void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
+                             uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
+                             int64_t position_start, int64_t seq_len) {
+  for (int64_t s = 0; s < seq_len; s++)
+    for (int64_t h = 0; h < heads; h++) {
+      const int64_t src = (s * heads + h) * d, dst = (h * max_seq + position_start + s) * d;
+      memcpy(k_cache + dst, new_k + src, (size_t)d * 2);
+      memcpy(v_cache + dst, new_v + src, (size_t)d * 2);
+    }
+}
+
+/* attention.rs:737-902 fmha_decode_gqa_split, restated tile by tile.
+ * q [kv_heads, group, d]; k, v [kv_heads, max_seq, d]; s_kv = input_pos + 1 keys are visible.
+ * att_out [kv_heads, splits * group, d] (f16), lse_out [kv_heads, splits * group] (f32, log2 domain).
+ * Per split: KV tiles [start_tile, end_tile) of bn rows; running max m (init -1e30), per-lane
+ * sums l[bn][group] (init 1), acc[d][group]; only the last tile of the sequence is masked
+ * (+ -1e30 before scaling); p is rounded to f16 for the P·V product; att = acc / max(sum l, 1e-8);
+ * lse = m + log2(max(sum l, 1e-8)). */
+void orc_fmha_decode_gqa_split(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                               uint16_t* att_out, float* lse_out, int64_t kv_heads, int64_t group,
+                               int64_t d, int64_t max_seq, int64_t bn, int64_t splits,
+                               float qk_scale, int64_t input_pos) {
+  const int64_t s_kv = input_pos + 1;
+  const int64_t tiles = (s_kv + bn - 1) / bn;
+  const int64_t per_split = (tiles + splits - 1) / splits;
+  const float scale_log2 = qk_scale / logf(2.0f);
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t h = 0; h < kv_heads; h++)
+    for (int64_t sp = 0; sp < splits; sp++) {
+      int64_t start = sp * per_split, end = start + per_split;
+      if (end > tiles) end = tiles;
+      float* m = (float*)malloc(sizeof(float) * (size_t)group);
+      float* l = (float*)malloc(sizeof(float) * (size_t)(bn * group));
+      float* acc = (float*)calloc((size_t)(d * group), sizeof(float));
+      float* qk = (float*)malloc(sizeof(float) * (size_t)(bn * group));
+      for (int64_t g = 0; g < group; g++) m[g] = -1.0e30f;
+      for (int64_t i = 0; i < bn * group; i++) l[i] = 1.0f;
+      for (int64_t j = start; j < end; j++) {
+        for (int64_t n = 0; n < bn; n++) {
+          const int64_t row = j * bn + n;
+          for (int64_t g = 0; g < group; g++) {
+            float a = 0.0f;
+            if (row < max_seq)
+              for (int64_t c = 0; c < d; c++)
+                a += orc_f16_to_f32(k[(h * max_seq + row) * d + c]) * orc_f16_to_f32(q[(h * group + g) * d + c]);
+            if (j == tiles - 1) a = a + (row < s_kv ? 0.0f : -1.0e30f);
+            qk[n * group + g] = a * scale_log2;
+          }
+        }
+        for (int64_t g = 0; g < group; g++) {
+          float mx = -INFINITY;
+          for (int64_t n = 0; n < bn; n++) mx = fmaxf(mx, qk[n * group + g]);
+          const float m_new = fmaxf(m[g], mx);
+          const float alpha = exp2f(m[g] - m_new);
+          for (int64_t c = 0; c < d; c++) acc[c * group + g] *= alpha;
+          for (int64_t n = 0; n < bn; n++) {
+            const float p = exp2f(qk[n * group + g] - m_new);
+            l[n * group + g] = l[n * group + g] * alpha + p;
+            const float ph = orc_f16_to_f32(orc_f32_to_f16(p));
+            const int64_t row = j * bn + n;
+            if (row < max_seq && ph != 0.0f)
+              for (int64_t c = 0; c < d; c++)
+                acc[c * group + g] += orc_f16_to_f32(v[(h * max_seq + row) * d + c]) * ph;
+          }
+          m[g] = m_new;
+        }
+      }
+      for (int64_t g = 0; g < group; g++) {
+        float ls = 0.0f;
+        for (int64_t n = 0; n < bn; n++) ls += l[n * group + g];
+        const float safe = fmaxf(ls, 1.0e-8f);
+        for (int64_t c = 0; c < d; c++)
+          att_out[((h * splits + sp) * group + g) * d + c] = orc_f32_to_f16(acc[c * group + g] / safe);
+        lse_out[(h * splits + sp) * group + g] = m[g] + log2f(safe);
+      }
+      free(m); free(l); free(acc); free(qk);
+    }
+}
+
+/* attention.rs:917-1013 splitk_reduce_merge: weights = exp2(lse - max) / max(sum, 1e-8) over
+ * the splits; out[h, g, :] = sum_s weights[g, s] * att[h, s, g, :], f16. */
+void orc_splitk_reduce_merge(const uint16_t* att, const float* lse, uint16_t* out, int64_t kv_heads,
+                             int64_t group, int64_t d, int64_t splits) {
+#pragma omp parallel for schedule(static)
+  for (int64_t h = 0; h < kv_heads; h++)
+    for (int64_t g = 0; g < group; g++) {
+      float mx = -INFINITY, sum = 0.0f;
+      for (int64_t s = 0; s < splits; s++) mx = fmaxf(mx, lse[(h * splits + s) * group + g]);
+      for (int64_t s = 0; s < splits; s++) sum += exp2f(lse[(h * splits + s) * group + g] - mx);
+      const float safe = fmaxf(sum, 1.0e-8f);
+      for (int64_t c = 0; c < d; c++) {
+        float o = 0.0f;
+        for (int64_t s = 0; s < splits; s++) {
+          const float w = exp2f(lse[(h * splits + s) * group + g] - mx) / safe;
+          o += orc_f16_to_f32(att[((h * splits + s) * group + g) * d + c]) * w;
+        }
+        out[(h * group + g) * d + c] = orc_f32_to_f16(o);
+      }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* K3                                                                        */
 /* ------------------------------------------------------------------------ */
 static void softmax_tile_row(const float* xin, float* yout, int64_t valid, int64_t bn) {

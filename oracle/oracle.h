@@ -90,6 +90,18 @@ void orc_silu_mul_f16(size_t n, const uint16_t* gate, const uint16_t* up, uint16
 void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, int64_t seq,
                       int64_t heads, int64_t d, int32_t position_start);
 
+/* kv_cache_update_seq(_dynpos)_f16: cutile-kernels/src/kv_cache.rs:15-49, 58-97 */
+void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
+                             uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
+                             int64_t position_start, int64_t seq_len);
+/* fmha_decode_gqa_split / splitk_reduce_merge: cutile-kernels/src/attention.rs:737-902, 917-1013 */
+void orc_fmha_decode_gqa_split(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                               uint16_t* att_out, float* lse_out, int64_t kv_heads, int64_t group,
+                               int64_t d, int64_t max_seq, int64_t bn, int64_t splits,
+                               float qk_scale, int64_t input_pos);
+void orc_splitk_reduce_merge(const uint16_t* att, const float* lse, uint16_t* out, int64_t kv_heads,
+                             int64_t group, int64_t d, int64_t splits);
+
 /* ---- K3: softmax over tiles [bm, bn] ---------------------------------- */
 /* f32 IO.  Tile (i, j) covers rows i*bm.., cols j*bn..; every tile row is
  * normalised on its own (row softmax iff bn == n).  Columns beyond n read as 0

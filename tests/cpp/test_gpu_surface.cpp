@@ -104,6 +104,49 @@ TEST(transformer_block_kernels_closed_forms) {
   for (int i = 0; i < 16; ++i) CHECK(f32_from_f16(rot_host[16 + i]) == (float)i);   // head 1 of out = head 0 of k
 }
 
+TEST(decode_kernels_closed_forms) {
+  auto stream = new_stream();
+  const int heads = 4, group = 4, d = 128, max_seq = 256, splits = 4;
+  // cache update: three new rows of 3.0 land at positions 9..11 of a cache of 1.0
+  auto new_k = api::full<f16>(3.0, {3, heads, d}).sync_on(stream).unwrap();
+  auto new_v = api::full<f16>(-3.0, {3, heads, d}).sync_on(stream).unwrap();
+  auto k_cache = api::full<f16>(1.0, {heads, max_seq, d}).sync_on(stream).unwrap();
+  auto v_cache = api::full<f16>(1.0, {heads, max_seq, d}).sync_on(stream).unwrap();
+  auto pos = api::full<uint32_t>(9, {1}).sync_on(stream).unwrap();
+  CHECK(kv_cache_update_seq_dynpos_f16(&new_k, &new_v, k_cache.partition_mut({1, max_seq, d}), v_cache.partition_mut({1, max_seq, d}), &pos, 3)
+            .generics({"128", "128", "256"}).sync_on(stream).is_ok());
+  auto kh = api::to_host_vec(k_cache).sync_on(stream).unwrap();
+  auto vh = api::to_host_vec(v_cache).sync_on(stream).unwrap();
+  for (int h = 0; h < heads; ++h)
+    for (int r = 0; r < max_seq; ++r) {
+      const bool fresh = r >= 9 && r < 12;
+      CHECK(f32_from_f16(kh[((size_t)h * max_seq + r) * d + 5]) == (fresh ? 3.0f : 1.0f));
+      CHECK(f32_from_f16(vh[((size_t)h * max_seq + r) * d + 77]) == (fresh ? -3.0f : 1.0f));
+    }
+  // the prefill form writes rows 0..seq_len and refuses another offset
+  CHECK(kv_cache_update_seq_f16(&new_k, &new_v, k_cache.partition_mut({1, 16, 64}), v_cache.partition_mut({1, 16, 64}), 0, 2).sync_on(stream).is_ok());
+  CHECK(!kv_cache_update_seq_f16(&new_k, &new_v, k_cache.partition_mut({1, 16, 64}), v_cache.partition_mut({1, 16, 64}), 5, 2).sync_on(stream).is_ok());
+  kh = api::to_host_vec(k_cache).sync_on(stream).unwrap();
+  CHECK(f32_from_f16(kh[0]) == 3.0f && f32_from_f16(kh[d]) == 3.0f && f32_from_f16(kh[2 * d]) == 1.0f);
+  // decode: every value row is 2.0 -> softmax weights sum to one -> every output is 2.0, whatever the scores
+  auto q = api::full<f16>(0.5, {heads, group, d}).sync_on(stream).unwrap();
+  auto vals = api::full<f16>(2.0, {heads, max_seq, d}).sync_on(stream).unwrap();
+  auto att = api::zeros<f16>({heads, splits * group, d}).sync_on(stream).unwrap();
+  auto lse = api::zeros<float>({heads, splits * group}).sync_on(stream).unwrap();
+  auto out = api::zeros<f16>({heads, group, d}).sync_on(stream).unwrap();
+  auto at = api::full<uint32_t>(199, {1}).sync_on(stream).unwrap();
+  CHECK(fmha_decode_gqa_split(&q, &k_cache, &vals, att.partition_mut({1, group, d}), lse.partition_mut({1, group}), 0.0884f, &at)
+            .generics({"4", "64", "128", "4"}).sync_on(stream).is_ok());
+  CHECK(splitk_reduce_merge(&att, &lse, out.partition_mut({1, group, d})).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 2.0f);
+  // GROUP = 3 has no precompiled variant: an error that names what exists, not a wrong answer
+  auto q3 = api::zeros<f16>({heads, 3, d}).sync_on(stream).unwrap();
+  auto att3 = api::zeros<f16>({heads, 3, d}).sync_on(stream).unwrap();
+  auto lse3 = api::zeros<float>({heads, 3}).sync_on(stream).unwrap();
+  auto r = fmha_decode_gqa_split(&q3, &k_cache, &vals, att3.partition_mut({1, 3, d}), lse3.partition_mut({1, 3}), 0.1f, &at).sync_on(stream);
+  CHECK(!r.is_ok());
+}
+
 TEST(gemm_ones_non_divisible) {
   auto stream = new_stream();
   const int m = 200, n = 264, k = 128;
