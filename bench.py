@@ -280,8 +280,208 @@ class MxGemm(Workload):
                {"rel_l2_sampled_rows": rel, "tolerance": 3e-2, "ok": rel <= 3e-2}
 
 
+def _td_f16(torch, np, bits, dev):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.float16)).to(dev)
+
+
+def _f16_close(oracle, np, got_bits, ref_bits):
+    """every element within one f16 ulp of the oracle (relative 2^-10, absolute 1e-7 near zero)"""
+    g, r = oracle.f16_bits_to_f32(got_bits), oracle.f16_bits_to_f32(ref_bits)
+    return bool(np.all(np.abs(g - r) <= np.abs(r) * 2 ** -10 + 1e-7))
+
+
+class AddRmsNorm(Workload):
+    name, unit, dtype = "add_rms_norm_f16_16384x8192", "GB/s", "f16 io / f32 math"
+    m, n = 16384, 8192
+    work = float(4 * m * n * 2 + n * 2)
+    config = {"workload": "add_rms_norm fp16: residual + x [16384, 8192] -> normalised rows and the new residual, eps 1e-6"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.rb = oracle.f32_to_f16_bits(oracle.normal_f32((self.m, self.n), 21))
+        self.xb = oracle.f32_to_f16_bits(oracle.normal_f32((self.m, self.n), 22))
+        self.wb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.n, 23, 0.5, 1.5))
+        self.r, self.x, self.w = (_td_f16(torch, np, t, dev) for t in (self.rb, self.xb, self.wb))
+        self.o, self.ro = torch.empty_like(self.x), torch.empty_like(self.x)
+        self.op, self.rop = ct.partition(self.o, [1, self.n]), ct.partition(self.ro, [1, self.n])
+
+    def launch(self):
+        self.ct.add_rms_norm_f16(self.r, self.x, self.w, self.op, self.rop, 1e-6)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 1024
+        t0 = time.perf_counter()
+        ref, res = oracle.add_rms_norm_f16(self.rb[:rows], self.xb[:rows], self.wb, 1e-6)
+        dt = time.perf_counter() - t0
+        ok = _f16_close(oracle, np, self.o[:rows].cpu().numpy().view(np.uint16), ref)
+        exact = bool(np.array_equal(self.ro[:rows].cpu().numpy().view(np.uint16), res))
+        return {"value": (4 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"first {rows} of {self.m} rows"}, {"within_1_f16_ulp": ok, "residual_bit_exact": exact}
+
+
+class SiluMul(Workload):
+    name, unit, dtype = "silu_mul_f16_16384x8192", "GB/s", "f16 io / f32 math"
+    m, n = 16384, 8192
+    work = float(3 * m * n * 2)
+    config = {"workload": "silu_mul_2d fp16: silu(gate) * up, [16384, 8192], tiles [1, 1024]"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.gb = oracle.f32_to_f16_bits(oracle.normal_f32((self.m, self.n), 24))
+        self.ub = oracle.f32_to_f16_bits(oracle.normal_f32((self.m, self.n), 25))
+        self.g, self.u = _td_f16(torch, np, self.gb, dev), _td_f16(torch, np, self.ub, dev)
+        self.o = torch.empty_like(self.g)
+        self.op = ct.partition(self.o, [1, 1024])
+
+    def launch(self):
+        self.ct.silu_mul_2d_f16(self.op, self.g, self.u)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 2048
+        t0 = time.perf_counter()
+        ref = oracle.silu_mul_f16(self.gb[:rows], self.ub[:rows])
+        dt = time.perf_counter() - t0
+        ok = _f16_close(oracle, np, self.o[:rows].cpu().numpy().view(np.uint16), ref)
+        return {"value": (3 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"first {rows} of {self.m} rows"}, {"within_1_f16_ulp": ok}
+
+
+class QkNorm(Workload):
+    name, unit, dtype = "qk_norm_f16_655360x128", "GB/s", "f16 io / f32 math"
+    tokens, qh, kh, d = 16384, 32, 8, 128
+    work = float(2 * tokens * (qh + kh) * d * 2)
+    config = {"workload": "qk_norm fp16: 16384 tokens x (32 q + 8 k) heads of 128, per-head RMSNorm with q/k weights, eps 1e-6"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.qb = oracle.f32_to_f16_bits(oracle.normal_f32((self.tokens * self.qh, self.d), 26))
+        self.kb = oracle.f32_to_f16_bits(oracle.normal_f32((self.tokens * self.kh, self.d), 27))
+        self.qwb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.d, 28, 0.5, 1.5))
+        self.kwb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.d, 29, 0.5, 1.5))
+        self.q, self.k, self.qw, self.kw = (_td_f16(torch, np, t, dev) for t in (self.qb, self.kb, self.qwb, self.kwb))
+        self.o = torch.empty(self.tokens * (self.qh + self.kh), self.d, dtype=torch.float16, device=dev)
+        self.op = ct.partition(self.o, [1, self.d])
+
+    def launch(self):
+        self.ct.qk_norm_f16(self.q, self.k, self.qw, self.kw, self.op, 1e-6, self.tokens * self.qh)
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        ref = oracle.qk_norm_f16(self.qb, self.kb, self.qwb, self.kwb, 1e-6)
+        dt = time.perf_counter() - t0
+        ok = _f16_close(oracle, np, self.o.cpu().numpy().view(np.uint16), ref)
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": "full size"}, {"within_1_f16_ulp": ok}
+
+
+class Rope(Workload):
+    name, unit, dtype = "rope_f16_32768x32x128", "GB/s", "f16 io / f32 math"
+    seq, heads, d = 32768, 32, 128
+    work = float(2 * seq * heads * d * 2)
+    config = {"workload": "rope_seq fp16: x [32768, 32, 128], inv_freq [64] (base 10000), start position 7"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.xb = oracle.f32_to_f16_bits(oracle.normal_f32((self.seq, self.heads, self.d), 30))
+        self.inv = (1.0 / 10000.0 ** (np.arange(self.d // 2) / (self.d // 2))).astype(np.float32)
+        self.x, self.fr = _td_f16(torch, np, self.xb, dev), torch.from_numpy(self.inv).to(dev)
+        self.o = torch.empty_like(self.x)
+        self.op = ct.partition(self.o, [1, 1, self.d // 2])
+
+    def launch(self):
+        self.ct.rope_f16(self.op, self.x, self.fr, 7)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 1024
+        t0 = time.perf_counter()
+        ref = oracle.rope_seq_f16(self.xb[:rows], self.inv, 7)
+        dt = time.perf_counter() - t0
+        ok = _f16_close(oracle, np, self.o[:rows].cpu().numpy().view(np.uint16), ref)
+        return {"value": (2 * rows * self.heads * self.d * 2) / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                "kind": "port", "sample": f"first {rows} of {self.seq} positions"}, {"within_1_f16_ulp": ok}
+
+
+class KvCacheUpdate(Workload):
+    name, unit, dtype = "kv_cache_update_f16_32768x8x128", "GB/s", "f16 (copy)"
+    seq, heads, d, max_seq = 32768, 8, 128, 32768
+    work = float(4 * seq * heads * d * 2)
+    config = {"workload": "kv_cache_update_seq fp16 (prefill form): new K,V [32768, 8, 128] into caches [8, 32768, 128] at row 0"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.nkb = oracle.f32_to_f16_bits(oracle.normal_f32((self.seq, self.heads, self.d), 31))
+        self.nvb = oracle.f32_to_f16_bits(oracle.normal_f32((self.seq, self.heads, self.d), 32))
+        self.nk, self.nv = _td_f16(torch, np, self.nkb, dev), _td_f16(torch, np, self.nvb, dev)
+        self.kc = torch.zeros(self.heads, self.max_seq, self.d, dtype=torch.float16, device=dev)
+        self.vc = torch.zeros_like(self.kc)
+        self.kp, self.vp = ct.partition(self.kc, [1, 16, self.d]), ct.partition(self.vc, [1, 16, self.d])
+
+    def launch(self):
+        self.ct.kv_cache_update_f16(self.nk, self.nv, self.kp, self.vp, 0, self.seq)
+
+    def cpu_baseline(self, oracle, np, torch):
+        zero = np.zeros((self.heads, self.max_seq, self.d), np.uint16)
+        t0 = time.perf_counter()
+        k_ref, v_ref = oracle.kv_cache_update_f16(self.nkb, self.nvb, zero, zero, 0, self.seq)
+        dt = time.perf_counter() - t0
+        exact = bool(np.array_equal(self.kc.cpu().numpy().view(np.uint16), k_ref) and
+                     np.array_equal(self.vc.cpu().numpy().view(np.uint16), v_ref))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "full size"}, \
+               {"bit_exact": exact}
+
+
+class DecodeAttention(Workload):
+    name, unit, dtype = "decode_gqa_f16_h8g4d128_s131072", "GB/s", "f16 io / f32 softmax+acc"
+    heads, group, d, s, splits, bn = 8, 4, 128, 131072, 128, 64
+    work = float(2 * heads * s * d * 2)          # every K and V byte once; q, partials and out are < 0.2 %
+    config = {"workload": "decode attention fp16: fmha_decode_gqa_split + splitk_reduce_merge, 8 KV heads x GROUP 4, D 128, "
+                          "131072 cached keys, 128 KV splits, BN 64 (two launches per step)"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.qb = oracle.f32_to_f16_bits(oracle.normal_f32((self.heads, self.group, self.d), 33))
+        self.kb = oracle.f32_to_f16_bits(oracle.normal_f32((self.heads, self.s, self.d), 34))
+        self.vb = oracle.f32_to_f16_bits(oracle.normal_f32((self.heads, self.s, self.d), 35))
+        self.q, self.k, self.v = (_td_f16(torch, np, t, dev) for t in (self.qb, self.kb, self.vb))
+        self.att = torch.empty(self.heads, self.splits * self.group, self.d, dtype=torch.float16, device=dev)
+        self.lse = torch.empty(self.heads, self.splits * self.group, dtype=torch.float32, device=dev)
+        self.o = torch.empty(self.heads, self.group, self.d, dtype=torch.float16, device=dev)
+        self.pos = torch.tensor([self.s - 1], dtype=torch.int32, device=dev)
+        self.ap, self.lp = ct.partition(self.att, [1, self.group, self.d]), ct.partition(self.lse, [1, self.group])
+        self.op = ct.partition(self.o, [1, self.group, self.d])
+        self.scale = float(np.float16(self.d ** -0.5))
+
+    def launch(self):
+        self.ct.fmha_decode_gqa_split(self.q, self.k, self.v, self.ap, self.lp, self.scale, self.pos,
+                                      generics=[self.group, self.bn, self.d, self.splits])
+        self.ct.splitk_reduce_merge(self.att, self.lse, self.op)
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        att, lse = oracle.fmha_decode_gqa_split(self.qb, self.kb, self.vb, self.scale, self.s - 1, self.bn, self.splits)
+        ref = oracle.splitk_reduce_merge(att, lse, self.group)
+        dt = time.perf_counter() - t0
+        got = oracle.f16_bits_to_f32(self.o.cpu().numpy().view(np.uint16))
+        err = float(np.max(np.abs(got - oracle.f16_bits_to_f32(ref))))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": "full size"}, {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
+
+
 def make_workloads():
-    return [Gemm(8192), Gemm(4096), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm()]
+    return [Gemm(8192), Gemm(4096), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(),
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

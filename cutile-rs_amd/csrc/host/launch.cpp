@@ -975,7 +975,8 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
   args.push_tensor(*lse_partial);
   args.push_partition(*out);
   args.push_tile_grid(tg);
-  uint32_t grid[3] = {std::min<uint32_t>(tg[0], (uint32_t)ot.shape[0]), 1, 1};
+  // one workgroup per (KV head, query head of the group)
+  uint32_t grid[3] = {std::min<uint32_t>(tg[0], (uint32_t)ot.shape[0]) * (uint32_t)group, 1, 1};
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "kernel_args.h"
 
@@ -40,6 +41,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define LDS_PTR(T) __attribute__((address_space(3))) T*
@@ -665,26 +667,129 @@ struct FmhaPingPong {
 // fmha_decode_gqa_split / splitk_reduce_merge (cutile-kernels/src/attention.rs:737-902, 917-1013).
 // One new token: the GROUP query heads that share KV head h attend to keys
 // 0..input_pos of that head's cache.  A workgroup takes one (KV head, split) and
-// streams its share of the cache once; this is bandwidth work (every K and V
-// byte is used for GROUP dot products), so it runs on the vector ALUs:
-//  * a cache row of D halves is spread over D/8 lanes (16-byte loads), so a
-//    wavefront takes 512/D rows at a time and the four wavefronts interleave;
-//  * every row slot keeps its own online-softmax state (m, l, acc) in the log2
-//    domain; slots are merged by shuffles, wavefronts through LDS;
-//  * the partial result is normalised and stored with its log-sum-exp,
-//    lse = m + log2(l), as the merge kernel expects.  p is rounded to f16
-//    before it multiplies V, as in the tile program; a split with no keys
-//    stores att = 0 and lse = -1e30 + log2(BN) (the tile program's initial state).
+// streams its share of the cache once.  This is bandwidth work (every K and V
+// byte feeds only GROUP dot products), so it runs on the vector ALUs, arranged
+// to spend few instructions per byte:
+//  * a cache row of D halves is spread over the 16 lanes of one DPP row (D/16
+//    halves each); a wavefront holds four such rows side by side ("slots") and
+//    each lane works on R rows per pass, so a pass of the workgroup covers 16 R keys;
+//  * q.k partial sums use the packed-half dot instruction; the R*GROUP partial
+//    sums of a lane are reduced over the 16 lanes by a reduce-scatter butterfly
+//    (N-1 cross-lane adds instead of 4 N).  To make the butterfly free of
+//    selects every lane computes its partial sums in a lane-dependent order:
+//    register j holds the sum with index j ^ p(lane), which only changes the
+//    addresses of the K rows and q rows the lane loads;
+//  * after the butterfly one lane owns one (row, head) score; the online
+//    softmax (log2 domain, p rounded to f16 as in the tile program) runs on that
+//    single value, and the probabilities return to all lanes as f16 pairs by
+//    row broadcasts;
+//  * p.V uses the packed-half dot again on (row 2i, row 2i+1) pairs, f32 accumulators;
+//    the accumulators are rescaled only in passes where some running maximum moved.
+// The partial result is normalised and stored with lse = m + log2(l), as the merge
+// kernel expects; a split with no keys stores att = 0 and lse = -1e30 + log2(BN)
+// (the tile program's untouched initial state).
+namespace decode {
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+  return __builtin_bit_cast(float, dpp_u<CTRL>(__builtin_bit_cast(uint32_t, x)));
+}
+// The four pairings of the butterfly inside a row of 16 lanes: i^8, 7-i within
+// each group of 8, i^2, i^1.  Pairing 1 flips bits 2, 1 and 0 of the lane number together,
+// which is why the index a lane ends up owning is lane ^ (bit 2 ? 3 : 0) (see owner()).
+template <int STEP>
+__device__ __forceinline__ uint32_t partner_u(uint32_t x) {
+  static_assert(STEP >= 0 && STEP < 4, "butterfly step");
+  if constexpr (STEP == 0) return dpp_u<0x128>(x);        // row_ror:8
+  else if constexpr (STEP == 1) return dpp_u<0x141>(x);   // row_half_mirror
+  else if constexpr (STEP == 2) return dpp_u<0x4E>(x);    // quad_perm:[2,3,0,1]
+  else return dpp_u<0xB1>(x);                             // quad_perm:[1,0,3,2]
+}
+template <int STEP>
+__device__ __forceinline__ float partner_f(float x) {
+  return __builtin_bit_cast(float, partner_u<STEP>(__builtin_bit_cast(uint32_t, x)));
+}
+__host__ __device__ constexpr int owner(int index4) { return index4 ^ (((index4 >> 2) & 1) * 3); }   // an involution
+template <int LANE>
+__device__ __forceinline__ uint32_t row_bcast_u(uint32_t x) { return dpp_u<0x150 + LANE>(x); }        // row_newbcast
+template <int LANE>
+__device__ __forceinline__ float row_bcast_f(float x) { return dpp_f<0x150 + LANE>(x); }
+
+// x[0..N): reduce over the 16 lanes of the row.  While more than one value is left each step halves
+// them (a lane keeps the lower half and adds its partner's upper half); then plain all-reduce steps.
+template <int N, int STEP = 0>
+__device__ __forceinline__ void reduce_scatter(float* x) {
+  if constexpr (STEP < 4) {
+    if constexpr (N > 1) {
+#pragma unroll
+      for (int i = 0; i < N / 2; ++i) x[i] += partner_f<STEP>(x[i + N / 2]);
+      reduce_scatter<N / 2, STEP + 1>(x);
+    } else {
+      x[0] += partner_f<STEP>(x[0]);
+      reduce_scatter<1, STEP + 1>(x);
+    }
+  }
+}
+// all-reduce over the first STEPS pairings (the lanes that own the same head but different rows)
+template <int STEPS, bool MAX, int STEP = 0>
+__device__ __forceinline__ float reduce_rows(float x) {
+  if constexpr (STEP < STEPS) {
+    const float o = partner_f<STEP>(x);
+    return reduce_rows<STEPS, MAX, STEP + 1>(MAX ? fmaxf(x, o) : x + o);
+  } else {
+    return x;
+  }
+}
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+template <int W>
+__device__ __forceinline__ void load_row(const _Float16* p, uint32_t (&dst)[W]) {
+  if constexpr (W == 2) {
+    const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+    dst[0] = t[0], dst[1] = t[1];
+  } else {
+#pragma unroll
+    for (int i = 0; i < W / 4; ++i) {
+      const u32x4 t = *reinterpret_cast<const u32x4*>(p + i * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[i * 4 + e] = t[e];
+    }
+  }
+}
+constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v / 2); }
+}  // namespace decode
+
 template <int G, int D>
 __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const TensorArg<3>& k, const TensorArg<3>& v,
                                              const PartitionArg<3>& att_out, const PartitionArg<2>& lse_out,
                                              float qk_scale, const uint32_t* pos_dev, int32_t bn, const TileGrid& g) {
-  constexpr int LPR = D / 8, RPW = 64 / LPR, kWaves = 4;
-  static_assert(D % 8 == 0 && 64 % LPR == 0 && LPR <= 64, "head dimension");
+  using namespace decode;
+  constexpr int E = D / 16, W = E / 2;           // halves / dwords of a row held by one lane
+  constexpr int R = G * E > 64 ? 2 : 4;          // rows per lane and pass
+  constexpr int N = R * G;                       // partial sums per lane and pass
+  constexpr int NF = N > 16 ? N / 16 : 1;        // scores a lane owns after the butterfly
+  constexpr int LOGR = ilog2(R), LOGG = ilog2(G), LOGN = LOGR + LOGG;
+  constexpr int kWaves = 4, kSlots = 4, kRowsPerWave = kSlots * R;
+  static_assert(D % 32 == 0 && (G & (G - 1)) == 0 && N <= 32 && NF <= G, "decode tile");
   __shared__ float sm[kWaves][G], sl[kWaves][G];
   __shared__ __attribute__((aligned(16))) float sacc[kWaves][G][D];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int slot = lane / LPR, dl = lane % LPR;
+  const int slot = lane >> 4, dl = lane & 15;
+  // index bits this lane ends up owning: the top LOGN bits of owner(dl) (all four and one in-lane bit when N = 32)
+  const int own = owner(dl);
+  const int p = N <= 16 ? own >> (4 - (LOGN > 4 ? 4 : LOGN)) : own << 1;
+  const int pr = p >> LOGG, pg = p & (G - 1);
   const int32_t head = blockIdx.x, split = blockIdx.y, splits = (int32_t)g.y;
   const int32_t max_seq = min(k.shape[1], v.shape[1]);
   const int32_t s_kv = min((int32_t)pos_dev[0] + 1, max_seq);
@@ -693,61 +798,108 @@ __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const Tensor
   const int32_t r1 = min(min((split + 1) * per_split, tiles) * bn, s_kv);
   const float c = qk_scale * kLog2e;
 
-  float qv[G][8];
+  uint32_t qh[G][W];                             // register g' holds head g' ^ pg
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) {
-    const _Float16* qr = (const _Float16*)q.ptr + (int64_t)head * q.strides[0] + (int64_t)gi * q.strides[1] + dl * 8;
-    f16x8 t = *reinterpret_cast<const f16x8*>(qr);
+  for (int gi = 0; gi < G; ++gi)
+    load_row<W>((const _Float16*)q.ptr + (int64_t)head * q.strides[0] + (int64_t)(gi ^ pg) * q.strides[1] + dl * E, qh[gi]);
+  float m[NF], l[NF], acc[G][E];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qv[gi][e] = (float)t[e] * c;   // scale folded into q: s is in the log2 domain
-  }
-  float m[G], l[G], acc[G][8];
+  for (int i = 0; i < NF; ++i) m[i] = -1.0e30f, l[i] = 0.0f;
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) {
-    m[gi] = -1.0e30f;
-    l[gi] = 0.0f;
+  for (int gi = 0; gi < G; ++gi)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[gi][e] = 0.0f;
-  }
-  const _Float16* kb = (const _Float16*)k.ptr + (int64_t)head * k.strides[0] + dl * 8;
-  const _Float16* vb = (const _Float16*)v.ptr + (int64_t)head * v.strides[0] + dl * 8;
-  for (int32_t base = r0 + wave * RPW; base < r1; base += kWaves * RPW) {   // wavefront-uniform trip count
-    const int32_t row = base + slot;
-    const bool valid = row < r1;
-    f16x8 kr = {}, vr = {};
-    if (valid) {
-      kr = *reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1]);
-      vr = *reinterpret_cast<const f16x8*>(vb + (int64_t)row * v.strides[1]);
+    for (int e = 0; e < E; ++e) acc[gi][e] = 0.0f;
+  const _Float16* kb = (const _Float16*)k.ptr + (int64_t)head * k.strides[0] + dl * E;
+  const _Float16* vb = (const _Float16*)v.ptr + (int64_t)head * v.strides[0] + dl * E;
+  // which half of an f16 pair this lane's probability is: rows 2i (low) and 2i+1 (high)
+  const uint32_t pair_sel = (pr & 1) ? 0x05040100u : 0x01000504u;
+
+  for (int32_t base = r0 + wave * kRowsPerWave; base < r1; base += kWaves * kRowsPerWave) {   // wavefront-uniform
+    uint32_t kr[R][W], vr[R][W];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // rows past the end of the split re-read its last row: their scores are masked below, so p = 0
+      const int32_t krow = min(base + (r ^ pr) * kSlots + slot, r1 - 1), vrow = min(base + r * kSlots + slot, r1 - 1);
+      load_row<W>(kb + (int64_t)krow * k.strides[1], kr[r]);
+      load_row<W>(vb + (int64_t)vrow * v.strides[1], vr[r]);
     }
+    float x[N];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int gi = 0; gi < G; ++gi) {
+        float d = 0.0f;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+          d = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, kr[r][w]), __builtin_bit_cast(h2, qh[gi][w]), d, false);
+        x[r * G + gi] = d;
+      }
+    reduce_scatter<N>(x);
+    // this lane now owns the scores of row pr, heads pg .. pg + NF - 1
+    const bool valid = base + pr * kSlots + slot < r1;
+    uint32_t pair[NF];
+    float alpha[NF];
+    bool moved = false;
+#pragma unroll
+    for (int i = 0; i < NF; ++i) {
+      const float sc = valid ? x[i] * c : -INFINITY;
+      const float m_new = fmaxf(m[i], reduce_rows<LOGR, true>(sc));
+      alpha[i] = __builtin_amdgcn_exp2f(m[i] - m_new);
+      const float pv = __builtin_amdgcn_exp2f(sc - m_new);
+      l[i] = l[i] * alpha[i] + reduce_rows<LOGR, false>(pv);
+      moved |= m_new != m[i];
+      m[i] = m_new;
+      const uint32_t mine = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pv);
+      pair[i] = __builtin_amdgcn_perm(mine, partner_u<LOGR - 1>(mine), pair_sel);
+    }
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+      static_for<G>([&](auto gi) {
+        constexpr int t = gi.value;                                          // row 0, head gi
+        constexpr int src = owner(N <= 16 ? t << (4 - (LOGN > 4 ? 4 : LOGN)) : t >> 1);
+        const float a = row_bcast_f<src>(alpha[N <= 16 ? 0 : t & 1]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[gi.value][e] *= a;
+      });
+    }
+    static_for<R / 2>([&](auto rp) {
+      uint32_t lo[W], hi[W];
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        lo[w] = __builtin_amdgcn_perm(vr[2 * rp.value + 1][w], vr[2 * rp.value][w], 0x05040100u);
+        hi[w] = __builtin_amdgcn_perm(vr[2 * rp.value + 1][w], vr[2 * rp.value][w], 0x07060302u);
+      }
+      static_for<G>([&](auto gi) {
+        constexpr int t = 2 * rp.value * G + gi.value;                       // row 2 rp, head gi
+        constexpr int src = owner(N <= 16 ? t << (4 - (LOGN > 4 ? 4 : LOGN)) : t >> 1);
+        const h2 pp = __builtin_bit_cast(h2, row_bcast_u<src>(pair[N <= 16 ? 0 : t & 1]));
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          acc[gi.value][2 * w] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, lo[w]), pp, acc[gi.value][2 * w], false);
+          acc[gi.value][2 * w + 1] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, hi[w]), pp, acc[gi.value][2 * w + 1], false);
+        }
+      });
+    });
+  }
+  // running maximum and sum of every head, back in all lanes of the slot
+  float mg[G], lg[G];
+  static_for<G>([&](auto gi) {
+    constexpr int t = gi.value;
+    constexpr int src = owner(N <= 16 ? t << (4 - (LOGN > 4 ? 4 : LOGN)) : t >> 1);
+    mg[gi.value] = row_bcast_f<src>(m[N <= 16 ? 0 : t & 1]);
+    lg[gi.value] = row_bcast_f<src>(l[N <= 16 ? 0 : t & 1]);
+  });
+  // merge the four slots of this wavefront ...
+#pragma unroll
+  for (int o = 16; o < 64; o <<= 1) {
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
-      float sdot = 0.0f;
+      const float mo = __shfl_xor(mg[gi], o, 64), lo = __shfl_xor(lg[gi], o, 64);
+      const float m_new = fmaxf(mg[gi], mo);
+      const float fs = __builtin_amdgcn_exp2f(mg[gi] - m_new), fo = __builtin_amdgcn_exp2f(mo - m_new);
+      lg[gi] = lg[gi] * fs + lo * fo;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sdot = __builtin_fmaf((float)kr[e], qv[gi][e], sdot);
-#pragma unroll
-      for (int o = LPR / 2; o > 0; o >>= 1) sdot += __shfl_xor(sdot, o, 64);
-      const float m_new = valid ? fmaxf(m[gi], sdot) : m[gi];
-      const float alpha = __builtin_amdgcn_exp2f(m[gi] - m_new);
-      const float p = valid ? __builtin_amdgcn_exp2f(sdot - m_new) : 0.0f;
-      l[gi] = l[gi] * alpha + p;
-      const float ph = (float)(_Float16)p;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[gi][e] = __builtin_fmaf((float)vr[e], ph, acc[gi][e] * alpha);
-      m[gi] = m_new;
-    }
-  }
-  // merge the row slots of this wavefront ...
-#pragma unroll
-  for (int o = LPR; o < 64; o <<= 1) {
-#pragma unroll
-    for (int gi = 0; gi < G; ++gi) {
-      const float mo = __shfl_xor(m[gi], o, 64), lo = __shfl_xor(l[gi], o, 64);
-      const float m_new = fmaxf(m[gi], mo);
-      const float fs = __builtin_amdgcn_exp2f(m[gi] - m_new), fo = __builtin_amdgcn_exp2f(mo - m_new);
-      l[gi] = l[gi] * fs + lo * fo;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[gi][e] = acc[gi][e] * fs + __shfl_xor(acc[gi][e], o, 64) * fo;
-      m[gi] = m_new;
+      for (int e = 0; e < E; ++e) acc[gi][e] = acc[gi][e] * fs + __shfl_xor(acc[gi][e], o, 64) * fo;
+      mg[gi] = m_new;
     }
   }
   // ... and the wavefronts through LDS
@@ -755,62 +907,126 @@ __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const Tensor
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
       if (dl == 0) {
-        sm[wave][gi] = m[gi];
-        sl[wave][gi] = l[gi];
+        sm[wave][gi] = mg[gi];
+        sl[wave][gi] = lg[gi];
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sacc[wave][gi][dl * 8 + e] = acc[gi][e];
+      for (int e = 0; e < E; ++e) sacc[wave][gi][dl * E + e] = acc[gi][e];
     }
   }
   __syncthreads();
   if (wave == 0 && slot == 0) {
-    _Float16* ab = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + dl * 8;
+    _Float16* ab = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + dl * E;
     float* lb = (float*)lse_out.ptr + (int64_t)head * lse_out.strides[0];
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
       float mt = sm[0][gi];
 #pragma unroll
       for (int w = 1; w < kWaves; ++w) mt = fmaxf(mt, sm[w][gi]);
-      float lt = 0.0f, at[8] = {};
+      float lt = 0.0f, at[E] = {};
 #pragma unroll
       for (int w = 0; w < kWaves; ++w) {
         const float f = __builtin_amdgcn_exp2f(sm[w][gi] - mt);
         lt += sl[w][gi] * f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) at[e] += sacc[w][gi][dl * 8 + e] * f;
+        for (int e = 0; e < E; ++e) at[e] += sacc[w][gi][dl * E + e] * f;
       }
       if (r0 >= r1) lt = (float)bn;   // no keys in this split: the tile program's untouched l = 1 per lane
       const float safe = fmaxf(lt, 1.0e-8f);
       const int64_t orow = (int64_t)split * G + gi;
-      f16x8 o;
+      _Float16* dst = ab + orow * att_out.strides[1];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = (_Float16)(at[e] / safe);
-      *reinterpret_cast<f16x8*>(ab + orow * att_out.strides[1]) = o;
+      for (int e = 0; e < E; e += 4) {
+        f16x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = (_Float16)(at[e + j] / safe);
+        *reinterpret_cast<f16x4*>(dst + e) = o;
+      }
       if (dl == 0) lb[orow * lse_out.strides[1]] = mt + __builtin_log2f(safe);
     }
   }
 }
 
 // out[h, g, :] = sum_s w[g, s] att[h, s*GROUP + g, :], w = exp2(lse - max_s lse) / max(sum, 1e-8).
+// One workgroup per (KV head, query head of the group).  The weights come from two
+// workgroup-wide reductions over the splits; then the rows of the partial results are
+// streamed 256 / lanes-per-row at a time (16 bytes per lane when the layout allows it)
+// and the row groups are summed through LDS.
+__device__ __forceinline__ float block_reduce(float x, bool take_max, float* scratch) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float y = __shfl_xor(x, o, 64);
+    x = take_max ? fmaxf(x, y) : x + y;
+  }
+  __syncthreads();                       // scratch may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = x;
+  __syncthreads();
+  float r = scratch[0];
+  for (int w = 1; w < (int)(blockDim.x >> 6); ++w) r = take_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+  return r;
+}
+
 __device__ __forceinline__ void splitk_merge(const TensorArg<3>& att, const TensorArg<2>& lse, const PartitionArg<3>& out) {
-  const int32_t head = blockIdx.x, group = out.shape[1], d = out.shape[2];
+  constexpr int kThreads = 256;
+  __shared__ float red[4];
+  __shared__ __attribute__((aligned(16))) float part[kThreads * 8];
+  const int32_t group = out.shape[1], d = out.shape[2];
+  const int32_t head = blockIdx.x / group, gi = blockIdx.x % group;
   const int32_t splits = att.shape[1] / group;
-  const _Float16* ab = (const _Float16*)att.ptr + (int64_t)head * att.strides[0];
-  const float* lb = (const float*)lse.ptr + (int64_t)head * lse.strides[0];
-  _Float16* ob = (_Float16*)out.ptr + (int64_t)head * out.strides[0];
-  for (int32_t idx = threadIdx.x; idx < group * d; idx += blockDim.x) {
-    const int32_t gi = idx / d, cidx = idx % d;
-    float mx = -INFINITY, sum = 0.0f;
-    for (int32_t sidx = 0; sidx < splits; ++sidx) mx = fmaxf(mx, lb[(int64_t)(sidx * group + gi) * lse.strides[1]]);
-    for (int32_t sidx = 0; sidx < splits; ++sidx)
-      sum += __builtin_amdgcn_exp2f(lb[(int64_t)(sidx * group + gi) * lse.strides[1]] - mx);
-    const float safe = fmaxf(sum, 1.0e-8f);
-    float o = 0.0f;
-    for (int32_t sidx = 0; sidx < splits; ++sidx) {
-      const float w = __builtin_amdgcn_exp2f(lb[(int64_t)(sidx * group + gi) * lse.strides[1]] - mx) / safe;
-      o += (float)ab[(int64_t)(sidx * group + gi) * att.strides[1] + (int64_t)cidx * att.strides[2]] * w;
+  const int tid = threadIdx.x;
+  const _Float16* ab = (const _Float16*)att.ptr + (int64_t)head * att.strides[0] + (int64_t)gi * att.strides[1];
+  const float* lb = (const float*)lse.ptr + (int64_t)head * lse.strides[0] + (int64_t)gi * lse.strides[1];
+  _Float16* ob = (_Float16*)out.ptr + (int64_t)head * out.strides[0] + (int64_t)gi * out.strides[1];
+  const int64_t att_step = (int64_t)group * att.strides[1], lse_step = (int64_t)group * lse.strides[1];
+
+  float mx = -INFINITY;
+  for (int32_t sidx = tid; sidx < splits; sidx += kThreads) mx = fmaxf(mx, lb[sidx * lse_step]);
+  mx = block_reduce(mx, true, red);
+  float sum = 0.0f;
+  for (int32_t sidx = tid; sidx < splits; sidx += kThreads) sum += __builtin_amdgcn_exp2f(lb[sidx * lse_step] - mx);
+  sum = block_reduce(sum, false, red);
+  const float inv = 1.0f / fmaxf(sum, 1.0e-8f);
+
+  const bool vec = d % 8 == 0 && att.strides[2] == 1 && out.strides[2] == 1 && att.strides[1] % 8 == 0 && att.strides[0] % 8 == 0 &&
+                   out.strides[1] % 8 == 0 && out.strides[0] % 8 == 0 && ((uintptr_t)att.ptr & 15) == 0 && ((uintptr_t)out.ptr & 15) == 0;
+  const int epl = vec ? 8 : 1;                               // elements per lane
+  const int32_t chunks = d / epl;
+  int lpr = 1;
+  while (lpr < chunks && lpr < kThreads) lpr <<= 1;          // lanes per row (a power of two)
+  const int rows_par = kThreads / lpr, my_row = tid / lpr, my_c = tid % lpr;
+  for (int32_t c0 = 0; c0 < chunks; c0 += lpr) {             // one trip unless D > 2048 (256 without 16-byte accesses)
+    const int32_t cidx = c0 + my_c;
+    float a[8] = {};
+    if (cidx < chunks) {
+      for (int32_t sidx = my_row; sidx < splits; sidx += rows_par) {
+        const float w = __builtin_amdgcn_exp2f(lb[sidx * lse_step] - mx) * inv;
+        const _Float16* src = ab + sidx * att_step;
+        if (vec) {
+          const f16x8 t = *reinterpret_cast<const f16x8*>(src + cidx * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) a[e] = __builtin_fmaf((float)t[e], w, a[e]);
+        } else {
+          a[0] = __builtin_fmaf((float)src[(int64_t)cidx * att.strides[2]], w, a[0]);
+        }
+      }
     }
-    ob[(int64_t)gi * out.strides[1] + (int64_t)cidx * out.strides[2]] = (_Float16)o;
+    __syncthreads();                                         // part[] of the previous trip has been consumed
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[(my_row * lpr + my_c) * 8 + e] = a[e];
+    __syncthreads();
+    if (my_row == 0 && cidx < chunks) {
+      for (int r = 1; r < rows_par; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] += part[(r * lpr + my_c) * 8 + e];
+      if (vec) {
+        f16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (_Float16)a[e];
+        *reinterpret_cast<f16x8*>(ob + cidx * 8) = o;
+      } else {
+        ob[(int64_t)cidx * out.strides[2]] = (_Float16)a[0];
+      }
+    }
   }
 }
 
