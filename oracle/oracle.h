@@ -29,6 +29,19 @@
  *                        codecs pinned against torch.float8_e4m3fn /
  *                        float8_e8m0fnu over all 256 codes.  The quantiser is not
  *                        in the reference (OCP MX v1.0 rule): parity unpinned.
+ *   orc_add_rms_norm_f16, orc_qk_norm_f16      cutile-kernels/src/norms.rs (kernel bodies);
+ *   orc_add_f16, orc_silu_mul_f16              cutile-kernels/src/pointwise.rs;
+ *   orc_rope_seq_f16                           cutile-kernels/src/positional.rs:13-64;
+ *   orc_kv_cache_update_f16                    cutile-kernels/src/kv_cache.rs:15-49, 58-97;
+ *   orc_fmha_decode_gqa_split, orc_splitk_reduce_merge
+ *                                              cutile-kernels/src/attention.rs:737-902, 917-1013.
+ *                        The reference only compiles these kernels in its tests
+ *                        (cutile-kernels/tests/smoke.rs), so they are pinned by the
+ *                        mathematics: reduction to orc_rms_norm_f16, float64
+ *                        definitions, scipy expit, complex rotation, float64 softmax
+ *                        attention for any number of splits, per-split log-sum-exp,
+ *                        merge closed forms, exact-copy checks: parity unpinned by
+ *                        reference tests.
  */
 #ifndef CUTILE_ORACLE_H
 #define CUTILE_ORACLE_H
