@@ -44,6 +44,11 @@ class PartitionArg(C.Structure):
                 ("partition_strides", C.c_int32 * MAX_RANK), ("prefix_coverage", C.c_int32)]
 
 
+class MappedPartitionArg(C.Structure):
+    _fields_ = [("partition", PartitionArg), ("map_rank", C.c_int32), ("map_shape", C.c_int32 * 3),
+                ("num_tile_blocks", C.c_uint32)]
+
+
 class LaunchOpts(C.Structure):
     _fields_ = [("grid", C.c_uint32 * 3), ("generics", C.POINTER(C.c_char_p)), ("n_generics", C.c_int32),
                 ("variant", C.c_char_p)]
@@ -126,6 +131,10 @@ def lib() -> C.CDLL:
             "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
                                                 P(TensorArg), f32, P(LaunchOpts)],
             "cutile_partition_grid": [P(PartitionArg), P(C.c_uint32 * 3)],
+            "cutile_mapped_partition_grid": [P(MappedPartitionArg), P(C.c_uint32 * 3)],
+            "cutile_mapped_partition_index": [P(MappedPartitionArg), C.c_uint32, P(C.c_uint32 * 3), P(C.c_uint32)],
+            "cutile_launch_gemm_persistent": [vp, P(MappedPartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
+            "cutile_launch_mapped_tile_index": [vp, P(MappedPartitionArg), P(LaunchOpts)],
             "cutile_infer_launch_grid": [P(C.c_uint32 * 3), P(P(PartitionArg)), i32, P(C.c_uint32 * 3)],
             "cutile_compute_spec": [P(TensorArg), P(SpecBits)],
             "cutile_kernel_lookup": [vp, C.c_char_p, P(C.c_char_p), i32, C.c_char_p, P(KernelInfo)],
@@ -227,6 +236,48 @@ class Partition:
 
 def partition(tensor, shape: Sequence[int], prefix: bool = False, dtype: Optional[int] = None) -> Partition:
     return Partition(tensor, list(shape), prefix, dtype)
+
+
+OWNED = 0     # map-shape sentinel of an owned (not streamed) axis, cutile/src/tensor.rs:331-337
+
+
+@dataclass
+class MappedPartition:
+    """``partition.map(map_shape, num_tile_blocks)`` of the reference (cutile/src/tensor.rs:314-350): the
+    logical tile grid is walked by ``num_tile_blocks`` tile blocks in the order the map shape fixes."""
+    partition: Partition
+    map_shape: Sequence[int]
+    num_tile_blocks: int
+
+    def arg(self) -> MappedPartitionArg:
+        m = MappedPartitionArg()
+        m.partition = self.partition.arg()
+        m.map_rank = len(self.map_shape)
+        for i, d in enumerate(self.map_shape[:3]):
+            m.map_shape[i] = d
+        m.num_tile_blocks = self.num_tile_blocks
+        return m
+
+    def grid(self):
+        """MappedLaunchPartition::validate (cutile/src/tensor.rs:352-400)"""
+        g = (C.c_uint32 * 3)()
+        check(lib().cutile_mapped_partition_grid(C.byref(self.arg()), C.byref(g)))
+        return tuple(g)
+
+    def num_items(self) -> int:
+        idx, n = (C.c_uint32 * 3)(), C.c_uint32()
+        check(lib().cutile_mapped_partition_index(C.byref(self.arg()), 0, C.byref(idx), C.byref(n)))
+        return n.value
+
+    def index(self, item: int):
+        """block id per partition axis (owned axes 0) of stream item ``item``"""
+        idx, n = (C.c_uint32 * 3)(), C.c_uint32()
+        check(lib().cutile_mapped_partition_index(C.byref(self.arg()), int(item), C.byref(idx), C.byref(n)))
+        return tuple(idx)[:self.partition.tensor.dim()]
+
+
+def mapped(part: Partition, map_shape: Sequence[int], num_tile_blocks: int) -> MappedPartition:
+    return MappedPartition(part, list(map_shape), int(num_tile_blocks))
 
 
 def _opts(grid=None, generics=None, variant=None):
@@ -394,6 +445,20 @@ def gemm(z: Partition, x, y, k: int, *, accumulate: bool = True, stream=None, gr
     xa, ya = tensor_arg(x), tensor_arg(y)
     check(lib().cutile_launch_gemm(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), int(k),
                                    int(accumulate), C.byref(o)))
+
+
+def gemm_persistent(z: MappedPartition, x, y, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """cutile-examples/examples/persistent_gemm.rs:35-59: z <- x . y, tiles walked by z.num_tile_blocks tile blocks."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x), tensor_arg(y)
+    check(lib().cutile_launch_gemm_persistent(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), C.byref(o)))
+
+
+def mapped_tile_index(z: MappedPartition, *, stream=None, grid=None) -> None:
+    """every tile of the i32 tensor receives its row-major index in the logical grid
+    (cutile/tests/gpu/mapped_partition_schedule_matrix.rs:30-76)"""
+    o, _k = _opts(grid, None, None)
+    check(lib().cutile_launch_mapped_tile_index(_stream(stream), C.byref(z.arg()), C.byref(o)))
 
 
 def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_group_size: int = 1, *,

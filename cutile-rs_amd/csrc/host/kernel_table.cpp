@@ -148,6 +148,19 @@ std::vector<KernelEntry> build_table() {
     add("gemm", keep(std::string(dt) + "_generic"), keep(std::string("gemm_entry__") + dt + "_generic"), IMG_GEMM, 256,
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
+  // ---- persistent GEMM over a mapped partition: the pipelined bodies in a stream-item loop ----
+  for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2}}) {
+    std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
+    add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
+        (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "bf16", 0, 2);
+  }
+  for (const char* dt : {"bf16", "f16", "f32"})
+    add("gemm_persistent", keep(std::string(dt) + "_generic"), keep(std::string("gemm_persistent_entry__") + dt + "_generic"),
+        IMG_GEMM, 256, (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
+  for (int r = 1; r <= 3; ++r)
+    add("mapped_tile_index", keep("i32_r" + std::to_string(r)), keep("mapped_tile_index_entry__i32_r" + std::to_string(r)),
+        IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "i32", 0, r);
+
   // ---- FMHA: LDS = 2 stages x (K tile + V tile) ----
   // "_pp": the two wavefronts of a SIMD run half a tile apart (BM = 256 only)
   auto fmha = [&](const char* dtype, int bm, int bn, int d, const char* suffix = "") {

@@ -18,6 +18,10 @@
 #include "common.h"
 #include "kernel_table.h"
 #include "runtime_state.h"
+#include "../kernels/mapped_partition.h"
+
+using cutile::MappedArg;
+using cutile::mapped_index;
 
 using namespace cutile;
 
@@ -1070,6 +1074,154 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
     grid[0] = std::max<uint32_t>(1, div_up(cover_m, 64));
     grid[1] = std::max<uint32_t>(1, div_up(cover_n, 64));
   }
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+// ---- mapped partitions (cutile/src/tensor.rs:314-401) ---------------------------------------------------------
+static cutile_status_t mapped_record(const cutile_mapped_partition_arg_t* p, MappedArg* m, uint32_t grid[3]) {
+  CUTILE_REQUIRE(p && grid, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  CUTILE_REQUIRE(!p->partition.prefix_coverage, CUTILE_ERR_TENSOR,
+                 "a partial-coverage (prefix) partition cannot be mapped: a mapped schedule covers its full index space by construction");
+  uint32_t pg[3];
+  if (cutile_status_t s = cutile_partition_grid(&p->partition, pg)) return s;
+  const int rank = p->map_rank;
+  CUTILE_REQUIRE(rank >= 1 && rank <= 3, CUTILE_ERR_TENSOR, "mapped partitions require a rank-1 through rank-3 map shape.");
+  bool all_owned = true;
+  for (int a = 0; a < rank; ++a) {
+    CUTILE_REQUIRE(p->map_shape[a] >= 0, CUTILE_ERR_TENSOR, "mapped partition map dimensions must be non-negative.");
+    all_owned &= p->map_shape[a] == CUTILE_MAP_OWNED;
+  }
+  CUTILE_REQUIRE(!all_owned, CUTILE_ERR_TENSOR, "mapped partition requires at least one streamed (non-OWNED) map axis.");
+  for (int a = 0; a < rank; ++a)
+    CUTILE_REQUIRE(pg[a] != 0, CUTILE_ERR_TENSOR, "mapped partition requires a non-empty logical partition grid.");
+  for (int a = rank; a < 3; ++a)
+    CUTILE_REQUIRE(pg[a] == 1, CUTILE_ERR_TENSOR, "mapped partition map rank must match the logical partition grid rank.");
+  uint64_t streamed = 1;
+  int n_streamed = 0;
+  for (int a = 0; a < rank; ++a)
+    if (p->map_shape[a] != CUTILE_MAP_OWNED) {
+      streamed *= pg[a];
+      ++n_streamed;
+      CUTILE_REQUIRE(streamed <= 0xFFFFFFFFull, CUTILE_ERR_TENSOR, "mapped partition logical grid is too large");
+    }
+  CUTILE_REQUIRE(p->num_tile_blocks > 0, CUTILE_ERR_TENSOR, "mapped partition requires num_tile_blocks > 0.");
+  CUTILE_REQUIRE(p->num_tile_blocks <= streamed, CUTILE_ERR_TENSOR,
+                 "mapped partition num_tile_blocks cannot exceed the streamed logical tile count.");
+  // what the schedule itself accepts (emit_mapped_partition_schedule): only the trailing two streamed axes group
+  int seen = 0;
+  for (int a = 0; a < rank; ++a)
+    if (p->map_shape[a] != CUTILE_MAP_OWNED) {
+      ++seen;
+      const bool leading = n_streamed - seen >= 2 || n_streamed == 1;
+      CUTILE_REQUIRE(!leading || p->map_shape[a] == 1, CUTILE_ERR_TENSOR,
+                     n_streamed == 1 ? "rank-1 mapped partition maps must be [1], got [%d]"
+                                     : "mapped partition schedules group only the trailing two axes: a leading map axis must be 1, got %d",
+                     p->map_shape[a]);
+    }
+  if (m) {
+    for (int a = 0; a < 3; ++a) {
+      m->map[a] = a < rank ? p->map_shape[a] : 1;
+      m->grid[a] = pg[a];
+    }
+    m->rank = rank;
+    m->total = (uint32_t)streamed;
+  }
+  grid[0] = p->num_tile_blocks;
+  grid[1] = grid[2] = 1;
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_mapped_partition_grid(const cutile_mapped_partition_arg_t* p, uint32_t grid[3]) {
+  return mapped_record(p, nullptr, grid);
+}
+
+cutile_status_t cutile_mapped_partition_index(const cutile_mapped_partition_arg_t* p, uint32_t item, uint32_t index[3],
+                                              uint32_t* n_items) {
+  CUTILE_REQUIRE(index, CUTILE_ERR_INVALID_ARGUMENT, "index is null");
+  MappedArg m;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_record(p, &m, grid)) return s;
+  if (n_items) *n_items = m.total;
+  CUTILE_REQUIRE(item < m.total, CUTILE_ERR_INVALID_ARGUMENT, "stream item %u is outside the %u items of the mapped partition", item, m.total);
+  mapped_index(m, item, index);
+  return CUTILE_SUCCESS;
+}
+
+// The launch grid of a mapped kernel: (num_tile_blocks, 1, 1); an explicit .grid() is a checked override.
+static cutile_status_t mapped_launch_grid(const cutile_mapped_partition_arg_t* z, const cutile_launch_opts_t* opts, MappedArg* m,
+                                          uint32_t grid[3]) {
+  if (cutile_status_t s = mapped_record(z, m, grid)) return s;
+  if (opts && (opts->grid[0] | opts->grid[1] | opts->grid[2]))
+    CUTILE_REQUIRE(opts->grid[0] == grid[0] && opts->grid[1] == 1 && opts->grid[2] == 1, CUTILE_ERR_KERNEL_LAUNCH,
+                   "launch grid (%u, %u, %u) does not match the inferred partition grid (%u, 1, 1)", opts->grid[0],
+                   opts->grid[1], opts->grid[2], grid[0]);
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cutile_mapped_partition_arg_t* zm,
+                                              const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                              const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(zm, CUTILE_ERR_INVALID_ARGUMENT, "z is null");
+  const cutile_partition_arg_t* z = &zm->partition;
+  if (cutile_status_t s = check_partition(z, "z", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(y, "y", 2, 2)) return s;
+  const cutile_tensor_arg_t& zt = z->tensor;
+  const bool in_bf16 = x->dtype == CUTILE_DTYPE_BF16, in_f16 = x->dtype == CUTILE_DTYPE_F16, in_f32 = x->dtype == CUTILE_DTYPE_F32;
+  CUTILE_REQUIRE(x->dtype == y->dtype && zt.dtype == x->dtype && (in_bf16 || in_f16 || in_f32), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "gemm_persistent: z, x and y must share one element type of bf16, f16, f32 (got %s, %s, %s)",
+                 cutile_dtype_name(zt.dtype), cutile_dtype_name(x->dtype), cutile_dtype_name(y->dtype));
+  CUTILE_REQUIRE(zm->map_rank == 2 && zm->map_shape[0] != CUTILE_MAP_OWNED && zm->map_shape[1] != CUTILE_MAP_OWNED,
+                 CUTILE_ERR_KERNEL_LAUNCH, "gemm_persistent: z needs a rank-2 map with both axes streamed");
+  const int32_t bm = z->partition_shape[0], bn = z->partition_shape[1];
+  const char* dt = in_f32 ? "f32" : in_f16 ? "f16" : "bf16";
+  if (cutile_status_t s = check_generic(opts, 0, dt, "T")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(bn), "BN")) return s;
+  if (cutile_status_t s = check_generic(opts, 4, std::to_string(zm->map_shape[0]), "MAP_SHAPE[0]")) return s;
+  if (cutile_status_t s = check_generic(opts, 5, std::to_string(zm->map_shape[1]), "MAP_SHAPE[1]")) return s;
+  const int bk_user = generic_int(opts, 3, 64);
+  CUTILE_REQUIRE(bk_user > 0, CUTILE_ERR_KERNEL_LAUNCH, "gemm_persistent: BK must be positive");
+  // launch checks the reference derives from the kernel body (persistent_gemm.rs:20-26): the K tiles of x must exist in y
+  CUTILE_REQUIRE(div_up((uint32_t)x->shape[1], (uint32_t)bk_user) <= div_up((uint32_t)y->shape[0], (uint32_t)bk_user),
+                 CUTILE_ERR_KERNEL_LAUNCH, "gemm_persistent: ceil(dim(x, 1)/BK) <= ceil(dim(y, 0)/BK) failed (%d, %d, BK = %d)",
+                 x->shape[1], y->shape[0], bk_user);
+  MappedArg m;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_launch_grid(zm, opts, &m, grid)) return s;
+  const bool fast_layout = in_bf16 && x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
+                           y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
+                           aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0;
+  std::vector<std::string> acceptable;
+  if (fast_layout)
+    for (const auto& e : kernel_table())
+      if (strcmp(e.function, "gemm_persistent") == 0 && e.tile[0] == bm && e.tile[1] == bn) acceptable.push_back(e.variant);
+  acceptable.push_back(std::string(dt) + "_generic");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("gemm_persistent", opts, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_tensor(*x);
+  args.push_tensor(*y);
+  args.push_val<MappedArg>(m);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_mapped_tile_index(cutile_stream_t stream, const cutile_mapped_partition_arg_t* zm,
+                                                const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(zm, CUTILE_ERR_INVALID_ARGUMENT, "z is null");
+  const cutile_partition_arg_t* z = &zm->partition;
+  if (cutile_status_t s = check_partition(z, "z", 1, 3)) return s;
+  CUTILE_REQUIRE(z->tensor.dtype == CUTILE_DTYPE_I32, CUTILE_ERR_KERNEL_NOT_FOUND, "mapped_tile_index: z must be i32");
+  MappedArg m;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_launch_grid(zm, opts, &m, grid)) return s;
+  const std::string want = "i32_r" + std::to_string(z->tensor.rank);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("mapped_tile_index", opts, want, {want}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_val<MappedArg>(m);
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

@@ -19,6 +19,7 @@
 #include <hip/hip_bf16.h>
 
 #include "kernel_args.h"
+#include "mapped_partition.h"
 
 using namespace cutile;
 
@@ -437,3 +438,55 @@ CONVERT_FROM(_Float16, f16)
 CONVERT_FROM(__bf16, bf16)
 CONVERT_FROM(int32_t, i32)
 CONVERT_FROM(int64_t, i64)
+
+// ---- mapped partitions: every tile receives its own logical index ----------------------------
+// The reference checks its mapped schedules with kernels that store, into every tile a tile
+// block visits, that tile's row-major index in the logical grid
+// (cutile/tests/gpu/mapped_partition_schedule_matrix.rs:30-76): a dropped tile keeps
+// the caller's fill, a duplicated one overwrites a neighbour.  Same kernel here, for
+// i32 tensors of rank 1 to 3: workgroup b takes stream items b, b + gridDim.x, ...;
+// an OWNED axis is walked in full by the workgroup that owns the item.
+template <int R>
+__device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, const MappedArg& m) {
+  int32_t* zp = (int32_t*)z.ptr;
+  for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
+    uint32_t bid[3];
+    mapped_index(m, item, bid);
+    uint32_t lo[3] = {0, 0, 0}, hi[3] = {1, 1, 1};
+    for (int a = 0; a < R; ++a) {
+      lo[a] = m.map[a] == kOwnedAxis ? 0 : bid[a];
+      hi[a] = m.map[a] == kOwnedAxis ? m.grid[a] : bid[a] + 1;
+    }
+    for (uint32_t c0 = lo[0]; c0 < hi[0]; ++c0)
+      for (uint32_t c1 = lo[1]; c1 < hi[1]; ++c1)
+        for (uint32_t c2 = lo[2]; c2 < hi[2]; ++c2) {
+          const uint32_t c[3] = {c0, c1, c2};
+          int32_t flat = 0;
+          int64_t count = 1;
+          for (int a = 0; a < R; ++a) {
+            flat = flat * (int32_t)m.grid[a] + (int32_t)c[a];
+            count *= z.pshape[a];
+          }
+          for (int64_t e = threadIdx.x; e < count; e += kThreads) {
+            int64_t rest = e, off = 0;
+            bool inside = true;
+            for (int a = R - 1; a >= 0; --a) {
+              const int64_t idx = (int64_t)c[a] * z.pshape[a] + rest % z.pshape[a];
+              rest /= z.pshape[a];
+              inside &= idx < z.shape[a];
+              off += idx * z.strides[a];
+            }
+            if (inside) zp[off] = flat;
+          }
+        }
+  }
+}
+
+#define MAPPED_TILE_INDEX_KERNEL(R)                                                                \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      mapped_tile_index_entry__i32_r##R(PartitionArg<R> z, MappedArg m) {                          \
+    mapped_tile_index<R>(z, m);                                                                    \
+  }
+MAPPED_TILE_INDEX_KERNEL(1)
+MAPPED_TILE_INDEX_KERNEL(2)
+MAPPED_TILE_INDEX_KERNEL(3)

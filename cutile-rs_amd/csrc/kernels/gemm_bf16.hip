@@ -29,6 +29,7 @@
 #include <hip/hip_runtime.h>
 
 #include "gemm_common.h"
+#include "mapped_partition.h"
 #include "kernel_args.h"
 
 using namespace cutile;
@@ -259,6 +260,30 @@ struct GemmDirect {
 
   __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
                              int32_t k_total, const TileGrid& g, int32_t accumulate) {
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    run_tile(z, x, y, k_total, pm, pn, accumulate);
+  }
+
+  // gemm_persistent (cutile-examples/examples/persistent_gemm.rs:35-59): workgroup b computes the
+  // tiles of stream items b, b + gridDim.x, ... of the mapped output partition, from zero
+  // accumulators.  Workgroups are dealt round-robin to the XCDs, so item i is first sent to
+  // position (i % 8) * (total / 8) + i / 8 of the schedule (a bijection when 8 divides the
+  // total): each XCD then walks one contiguous eighth of the grouped order and its L2 sees
+  // neighbouring tiles, as in the one-tile-per-workgroup launch.
+  __device__ static void run_persistent(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                        const MappedArg& m) {
+    for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
+      const uint32_t pos = m.total % kNumXcd == 0 ? (item % kNumXcd) * (m.total / kNumXcd) + item / kNumXcd : item;
+      uint32_t bid[3];
+      mapped_index(m, pos, bid);
+      run_tile(z, x, y, x.shape[1], bid[0], bid[1], 0);
+      __syncthreads();   // the output bands live in the stages that the next tile refills
+    }
+  }
+
+  __device__ static __forceinline__ void run_tile(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                                  int32_t k_total, uint32_t pm, uint32_t pn, int32_t accumulate) {
     // Two separately named stages so that the compiler can tell a refill of one
     // from operand reads of the other.
     __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
@@ -266,8 +291,6 @@ struct GemmDirect {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    uint32_t pm, pn;
-    tile_coords(g.x, g.y, &pm, &pn);
     const int32_t M = x.shape[0], N = y.shape[1];
     const int32_t lda = x.strides[0], ldb = y.strides[0];
     const int32_t row0 = pm * BM, col0 = pn * BN;
@@ -726,17 +749,17 @@ struct GemmRing {
 template <typename T>
 __device__ __forceinline__ float elem_to_f32(T v) { return (float)v; }
 
+// One block of at most 64x64 outputs with its top-left corner at (row0, col0); stores
+// are limited to rows < row_end and columns < col_end.
 template <typename InT, typename OutT>
-__device__ void gemm_any_layout(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
-                                int32_t k_total, const TileGrid& g, int32_t accumulate) {
+__device__ __forceinline__ void any_layout_block(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                                 int32_t k_total, int64_t row0, int64_t col0, int64_t row_end,
+                                                 int64_t col_end, int32_t accumulate) {
   constexpr int TS = 64, KS = 16;
   __shared__ float xs[TS][KS + 1];
   __shared__ float ys[KS][TS + 1];
   const int tid = threadIdx.x;
   const int tr = tid / 16, tc = tid % 16;             // this lane's 4x4 block inside the 64x64 tile
-  const int64_t cover_m = min((int64_t)g.x * z.pshape[0], (int64_t)z.shape[0]);
-  const int64_t cover_n = min((int64_t)g.y * z.pshape[1], (int64_t)z.shape[1]);
-  const int64_t row0 = (int64_t)blockIdx.x * TS, col0 = (int64_t)blockIdx.y * TS;
   const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
   const InT* xp = (const InT*)x.ptr;
   const InT* yp = (const InT*)y.ptr;
@@ -775,13 +798,38 @@ __device__ void gemm_any_layout(const PartitionArg<2>& z, const TensorArg<2>& x,
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t gr = row0 + tr * 4 + i, gc = col0 + tc * 4 + j;
-      if (gr < cover_m && gc < cover_n) {
+      if (gr < row_end && gc < col_end) {
         OutT* dst = zp + gr * z.strides[0] + gc * z.strides[1];
         float v = acc[i][j];
         if (accumulate) v += elem_to_f32(*dst);
         *dst = (OutT)v;
       }
     }
+}
+
+template <typename InT, typename OutT>
+__device__ void gemm_any_layout(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                int32_t k_total, const TileGrid& g, int32_t accumulate) {
+  const int64_t cover_m = min((int64_t)g.x * z.pshape[0], (int64_t)z.shape[0]);
+  const int64_t cover_n = min((int64_t)g.y * z.pshape[1], (int64_t)z.shape[1]);
+  any_layout_block<InT, OutT>(z, x, y, k_total, (int64_t)blockIdx.x * 64, (int64_t)blockIdx.y * 64, cover_m, cover_n, accumulate);
+}
+
+// The persistent form for any tile shape: stream items in the reference's order, each
+// [BM, BN] tile of the partition covered by 64x64 blocks.
+template <typename InT, typename OutT>
+__device__ void gemm_any_layout_persistent(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                           const MappedArg& m) {
+  const int64_t bm = z.pshape[0], bn = z.pshape[1];
+  for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
+    uint32_t bid[3];
+    mapped_index(m, item, bid);
+    const int64_t r_end = min((int64_t)(bid[0] + 1) * bm, (int64_t)z.shape[0]);
+    const int64_t c_end = min((int64_t)(bid[1] + 1) * bn, (int64_t)z.shape[1]);
+    for (int64_t r = (int64_t)bid[0] * bm; r < r_end; r += 64)
+      for (int64_t c = (int64_t)bid[1] * bn; c < c_end; c += 64)
+        any_layout_block<InT, OutT>(z, x, y, x.shape[1], r, c, r_end, c_end, 0);
+  }
 }
 
 }  // namespace
@@ -837,3 +885,24 @@ GEMM_ANY_LAYOUT_KERNEL(bf16, __bf16, __bf16)
 GEMM_ANY_LAYOUT_KERNEL(bf16f32, __bf16, float)
 GEMM_ANY_LAYOUT_KERNEL(f16, _Float16, _Float16)
 GEMM_ANY_LAYOUT_KERNEL(f32, float, float)
+
+// gemm_persistent<T, BM, BN, BK, MAP_SHAPE>(z: mapped [BM,BN] tiles, x, y): grid (num_tile_blocks, 1, 1)
+#define GEMM_PERSISTENT_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                    \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_persistent_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
+    GemmDirect<BM, BN, WVM, WVN, OUT_T>::run_persistent(z, x, y, m);                            \
+  }
+
+GEMM_PERSISTENT_KERNEL(bf16_256x256x64_d4x2, 256, 256, 4, 2, __bf16)
+GEMM_PERSISTENT_KERNEL(bf16_256x256x64_d2x4, 256, 256, 2, 4, __bf16)
+GEMM_PERSISTENT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)
+
+#define GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                     \
+  extern "C" __global__ void __launch_bounds__(256)                                            \
+      gemm_persistent_entry__##NAME##_generic(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
+    gemm_any_layout_persistent<IN_T, OUT_T>(z, x, y, m);                                        \
+  }
+
+GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(bf16, __bf16, __bf16)
+GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(f16, _Float16, _Float16)
+GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(f32, float, float)

@@ -279,6 +279,35 @@ cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t 
 cutile_status_t cutile_infer_launch_grid(const uint32_t explicit_grid[3],
                                          const cutile_partition_arg_t* const* partitions,
                                          int32_t n_partitions, uint32_t grid[3]);
+/* Partition::map(map_shape, num_tile_blocks) -> MappedLaunchPartition — cutile/src/tensor.rs:314-350.
+ * The logical tile grid of `partition` is walked by `num_tile_blocks` tile blocks; a map dimension of
+ * CUTILE_MAP_OWNED marks an axis that is not streamed (each stream item owns its full extent). */
+#define CUTILE_MAP_OWNED 0
+typedef struct {
+  cutile_partition_arg_t partition;   /* must not be a prefix (partial-coverage) partition */
+  int32_t map_rank;                   /* 1..3, must equal the rank of the logical grid */
+  int32_t map_shape[3];
+  uint32_t num_tile_blocks;
+} cutile_mapped_partition_arg_t;
+/* MappedLaunchPartition::validate — cutile/src/tensor.rs:352-400: the launch grid (num_tile_blocks, 1, 1), or
+ * the reference's error ("rank-1 through rank-3 map shape", "at least one streamed (non-OWNED) map axis",
+ * "non-empty logical partition grid", "map rank must match the logical partition grid rank",
+ * "num_tile_blocks > 0", "num_tile_blocks cannot exceed the streamed logical tile count"). */
+cutile_status_t cutile_mapped_partition_grid(const cutile_mapped_partition_arg_t* p, uint32_t grid[3]);
+/* The schedule of `for index in z.iter_indices()` as a host-visible map: the block id per partition axis (owned
+ * axes 0) of stream item `item`, and the number of stream items.  Tile block b visits items b, b + num_tile_blocks, ...
+ * — cutile-compiler/src/compiler/compile_intrinsic.rs:2438-2900 (emit_swizzle_2d, emit_mapped_partition_schedule). */
+cutile_status_t cutile_mapped_partition_index(const cutile_mapped_partition_arg_t* p, uint32_t item, uint32_t index[3],
+                                              uint32_t* n_items);
+/* gemm_persistent<T, BM, BN, BK, MAP_SHAPE>(z: MappedPartitionMut [BM,BN], x, y): z <- x . y over all of x's K,
+ * zero initial accumulator — cutile-examples/examples/persistent_gemm.rs:35-59 */
+cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,
+                                              const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                              const cutile_launch_opts_t* opts);
+/* write_flat_index_rank{1,2,3}<.., MAP_SHAPE>(z: MappedPartitionMut<i32>): every tile a tile block visits is filled
+ * with its row-major index in the logical grid — cutile/tests/gpu/mapped_partition_schedule_matrix.rs:30-76 */
+cutile_status_t cutile_launch_mapped_tile_index(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,
+                                                const cutile_launch_opts_t* opts);
 /* SpecializationBits — cutile-compiler/src/specialization.rs:21-174 */
 typedef struct {
   int32_t shape_div[CUTILE_MAX_RANK];   /* largest power of two <= 16 dividing shape[i] */

@@ -253,6 +253,49 @@ def splitk_reduce_merge(att_bits, lse, group: int) -> np.ndarray:
     return out
 
 
+# ---- mapped partitions ----------------------------------------------------------------------
+def mapped_schedule(grid, map_shape):
+    """The order in which stream items visit the tiles of a mapped partition, as a list of block-id
+    tuples (one entry per partition axis, owned axes 0): item t of the stream is element t.
+
+    cutile-compiler/src/compiler/compile_intrinsic.rs:2438-2900 states the schedule as index arithmetic
+    (emit_swizzle_2d / emit_mapped_partition_schedule); here the same order is produced constructively,
+    by walking it: leading streamed axes row-major; the trailing two streamed axes (m, n) in bands of
+    GM tile rows, each band cut into groups of GN columns, each group column by column, rows fastest.
+    A map dimension of 0 (OWNED) takes the axis out of the stream.  Pure Python: small grids only."""
+    rank = len(map_shape)
+    streamed = [a for a in range(rank) if map_shape[a] != 0]
+    lens = [int(grid[a]) for a in streamed]
+    maps = [int(map_shape[a]) for a in streamed]
+
+    def place(coords):
+        out = [0] * rank
+        for a, c in zip(streamed, coords):
+            out[a] = c
+        return tuple(out)
+
+    def pairs(num_m, num_n, gm, gn):
+        for band in range(0, num_m, gm):
+            rows = min(gm, num_m - band)
+            for group in range(0, num_n, gn):
+                for n in range(group, min(group + gn, num_n)):
+                    for m in range(band, band + rows):
+                        yield m, n
+
+    order = []
+    if len(streamed) == 1:
+        order = [place((t,)) for t in range(lens[0])]
+    elif len(streamed) == 2:
+        gm, gn = maps
+        # (1, 1) is plain row-major in the reference (tile / num_n, tile % num_n), not bands of one row
+        # walked column by column -- which is the same thing: a band of one row IS a row.
+        order = [place(p) for p in pairs(lens[0], lens[1], gm, gn if (gm, gn) != (1, 1) else 1)]
+    elif len(streamed) == 3:
+        for lead in range(lens[0]):
+            order += [place((lead,) + p) for p in pairs(lens[1], lens[2], maps[1], maps[2])]
+    return order
+
+
 # ---- K3 -----------------------------------------------------------------------------------
 def softmax_f32(x, bm: int, bn: int) -> np.ndarray:
     x = _c(x, np.float32)

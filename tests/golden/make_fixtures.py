@@ -40,8 +40,50 @@ def persistent_gemm_case():
     }
 
 
+def mapped_partition_cases():
+    # cutile/src/tensor.rs:2203-2350: MappedLaunchPartition::validate(partition_grid, num_tile_blocks)
+    ok = lambda name, line, grid, mp, ntb: {"name": name, "cite": f"cutile/src/tensor.rs:{line}", "partition_grid": grid,
+                                            "map_shape": mp, "num_tile_blocks": ntb, "launch_grid": [ntb, 1, 1]}
+    err = lambda name, line, grid, mp, ntb, msg: {"name": name, "cite": f"cutile/src/tensor.rs:{line}", "partition_grid": grid,
+                                                  "map_shape": mp, "num_tile_blocks": ntb, "error_contains": msg}
+    validate = [
+        ok("swizzle_accepts_tile_block_count", "2203-2212", [2, 3, 1], [4, 1], 3),
+        err("swizzle_rejects_tile_block_count_larger_than_logical_grid", "2214-2226", [2, 3, 1], [4, 1], 7,
+            "num_tile_blocks cannot exceed the streamed logical tile count"),
+        ok("owned_axis_excluded_from_streamed_tile_count", "2228-2239", [2, 3, 1], [1, 0], 2),
+        err("owned_axis_excluded_from_streamed_tile_count_over", "2240-2249", [2, 3, 1], [1, 0], 3,
+            "num_tile_blocks cannot exceed the streamed logical tile count"),
+        err("owned_axis_rejects_all_owned_map", "2251-2262", [2, 3, 1], [0, 0], 1, "at least one streamed (non-OWNED) map axis"),
+        ok("owned_axis_accepts_leading_owned", "2264-2274", [2, 3, 1], [0, 1], 3),
+        err("swizzle_rejects_zero_tile_blocks", "2276-2285", [2, 3, 1], [4, 1], 0, "num_tile_blocks > 0"),
+        err("swizzle_rejects_grid_rank_above_map_rank", "2287-2298", [2, 3, 4], [4, 1], 3,
+            "map rank must match the logical partition grid rank"),
+        ok("swizzle_accepts_rank1_map", "2300-2309", [8, 1, 1], [1], 4),
+        ok("swizzle_accepts_rank3_map", "2311-2320", [2, 3, 4], [1, 4, 1], 6),
+        err("swizzle_rejects_rank1_map_with_2d_grid", "2322-2333", [2, 3, 1], [1], 2,
+            "map rank must match the logical partition grid rank"),
+        err("swizzle_rejects_map_rank_above_3", "2335-2345", [2, 3, 4], [1, 1, 1, 1], 2, "rank-1 through rank-3 map shape"),
+    ]
+    # cutile/tests/gpu/mapped_partition_schedule_matrix.rs:219-300: every (dims, tile, map, num_tile_blocks) of the
+    # coverage matrix; the expectation is that every element ends up holding its tile's row-major index.
+    matrix = [{"dims": [64], "tile": [16], "map_shape": [1], "num_tile_blocks": ntb} for ntb in (1, 3, 4)]
+    for rows, cols in ((4, 4), (3, 5)):
+        total = rows * cols
+        for mp in ([1, 1], [2, 1], [2, 2], [3, 2]):
+            for ntb in (1, min(5, total), total):
+                matrix.append({"dims": [rows * 8, cols * 8], "tile": [8, 8], "map_shape": mp, "num_tile_blocks": ntb})
+    for mp in ([1, 1, 1], [1, 2, 1], [1, 2, 2], [1, 3, 2]):
+        for ntb in (1, 5, 12):
+            matrix.append({"dims": [2, 12, 16], "tile": [1, 4, 8], "map_shape": mp, "num_tile_blocks": ntb})
+    return {"validate": validate, "schedule_matrix": {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:219-300",
+                                                      "poison": -0x5EAD, "cases": matrix},
+            "persistent_gemm_launch": {"cite": "cutile-examples/examples/persistent_gemm.rs:70-79",
+                                       "map_shape": [4, 1], "num_tile_blocks": 4}}
+
+
 def main():
     cases = {
+        "mapped_partition": mapped_partition_cases(),
         "saxpy_example": {
             "cite": "cutile-examples/examples/saxpy.rs:28-53",
             "a": 2.0, "shape": [4, 8], "partition": [2, 2],

@@ -1,0 +1,189 @@
+"""Mapped partitions (`partition.map(map_shape, num_tile_blocks)`, cutile/src/tensor.rs:314-401) and the
+persistent GEMM over them (cutile-examples/examples/persistent_gemm.rs).
+
+CPU: the host validation against the reference's own unit-test cases (golden fixtures), the oracle's
+constructive schedule pinned by what the definition fixes (a permutation of the tile grid; row-major and
+column-major special cases; band structure), and the library's host-visible schedule against the oracle.
+GPU: the reference's coverage matrix (every tile written exactly once, by the tile block the schedule
+names) and the persistent GEMM against the oracle.  The reference asserts coverage only, never the visiting
+order, so the ORDER is pinned by the mathematics alone; results do not depend on it."""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import normal_bf16_bits, to_dev_bf16, rel_l2
+
+CASES = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_cases.json")))["mapped_partition"]
+
+
+def _logical(grid, tile):
+    """a CPU tensor whose partition by `tile` has the logical grid `grid` (metadata only)"""
+    dims = [g * t for g, t in zip(grid, tile)]
+    return torch.zeros(dims, dtype=torch.int32), dims
+
+
+# ---- oracle (CPU) ---------------------------------------------------------------------------
+@pytest.mark.parametrize("grid,mp", [((4, 4), (1, 1)), ((3, 5), (2, 1)), ((3, 5), (2, 2)), ((3, 5), (3, 2)), ((7, 5), (4, 3)),
+                                     ((2, 3, 2), (1, 2, 2)), ((2, 3, 2), (1, 3, 2)), ((5,), (1,)), ((4, 6), (0, 1)), ((4, 6), (1, 0))])
+def test_oracle_schedule_is_a_permutation_of_the_streamed_grid(grid, mp):
+    order = oracle.mapped_schedule(grid, mp)
+    streamed = [range(g) if m != 0 else range(1) for g, m in zip(grid, mp)]
+    assert sorted(order) == sorted(itertools.product(*streamed)) and len(set(order)) == len(order)
+
+
+def test_oracle_schedule_special_cases():
+    # (1, 1): row-major
+    assert oracle.mapped_schedule((3, 4), (1, 1)) == [(m, n) for m in range(3) for n in range(4)]
+    # one band holding every row: column-major
+    assert oracle.mapped_schedule((3, 4), (3, 1)) == [(m, n) for n in range(4) for m in range(3)]
+    assert oracle.mapped_schedule((3, 4), (8, 1)) == [(m, n) for n in range(4) for m in range(3)]
+    # bands of GM rows: the first GM * num_n items stay inside rows 0..GM-1, and the short last band follows
+    order = oracle.mapped_schedule((5, 3), (2, 1))
+    assert [m for m, _ in order] == [0, 1] * 3 + [2, 3] * 3 + [4] * 3
+    assert [n for _, n in order] == [0, 0, 1, 1, 2, 2] * 2 + [0, 1, 2]
+    # groups of GN columns inside a band; a group is walked column by column
+    order = oracle.mapped_schedule((2, 5), (2, 2))
+    assert order == [(0, 0), (1, 0), (0, 1), (1, 1), (0, 2), (1, 2), (0, 3), (1, 3), (0, 4), (1, 4)]
+    order = oracle.mapped_schedule((4, 3), (2, 2))
+    assert order[:8] == [(0, 0), (1, 0), (0, 1), (1, 1), (0, 2), (1, 2), (2, 0), (3, 0)]
+    # rank 3: the leading axis is the slowest, the trailing pair is scheduled inside it
+    o3 = oracle.mapped_schedule((2, 3, 2), (1, 2, 1))
+    assert [c[0] for c in o3] == [0] * 6 + [1] * 6
+    assert [c[1:] for c in o3[:6]] == oracle.mapped_schedule((3, 2), (2, 1))
+    # an owned axis is not streamed: its coordinate stays 0
+    assert oracle.mapped_schedule((3, 4), (1, 0)) == [(0, 0), (1, 0), (2, 0)]
+
+
+# ---- host library (CPU) -----------------------------------------------------------------------
+@pytest.mark.parametrize("case", CASES["validate"], ids=lambda c: c["name"])
+def test_validate_matches_the_reference_unit_tests(ct, case):
+    grid = case["partition_grid"]
+    rank = 3 if grid[2] != 1 else 2 if grid[1] != 1 else 1
+    z, _ = _logical(grid[:rank], [4] * rank)
+    mp = ct.mapped(ct.partition(z, [4] * rank), case["map_shape"], case["num_tile_blocks"])
+    if "launch_grid" in case:
+        assert list(mp.grid()) == case["launch_grid"]
+    else:
+        with pytest.raises(ct.CutileError, match=case["error_contains"].replace("(", r"\(").replace(")", r"\)")):
+            mp.grid()
+
+
+def test_prefix_partitions_cannot_be_mapped(ct):
+    z = torch.zeros(8, 8, dtype=torch.int32)
+    with pytest.raises(ct.CutileError, match="partial-coverage .* cannot be mapped"):      # tensor.rs:319-323
+        ct.mapped(ct.partition(z, [4, 4], prefix=True), [1, 1], 2).grid()
+    with pytest.raises(ct.CutileError, match="leading map axis must be 1"):                 # compile_intrinsic.rs:2806-2815
+        ct.mapped(ct.partition(torch.zeros(2, 4, 4, dtype=torch.int32), [1, 2, 2]), [2, 1, 1], 2).grid()
+    with pytest.raises(ct.CutileError, match=r"rank-1 mapped partition maps must be \[1\]"):  # :2826-2835
+        ct.mapped(ct.partition(torch.zeros(8, dtype=torch.int32), [2]), [2], 2).grid()
+    with pytest.raises(ct.CutileError, match=r"rank-1 mapped partition maps must be \[1\]"):  # one streamed axis left
+        ct.mapped(ct.partition(torch.zeros(8, 12, dtype=torch.int32), [2, 2]), [2, 0], 2).grid()
+
+
+@pytest.mark.parametrize("grid,mp", [((4, 4), (1, 1)), ((3, 5), (2, 1)), ((3, 5), (2, 2)), ((3, 5), (3, 2)), ((7, 5), (4, 3)),
+                                     ((9, 2), (8, 1)), ((2, 3, 2), (1, 1, 1)), ((2, 3, 2), (1, 2, 2)), ((2, 3, 2), (1, 3, 2)),
+                                     ((5,), (1,)), ((4, 6), (0, 1)), ((4, 6), (1, 0)), ((3, 4, 5), (1, 0, 1)), ((3, 4, 5), (0, 2, 2))])
+def test_host_schedule_equals_the_oracle(ct, grid, mp):
+    z, _ = _logical(grid, [2] * len(grid))
+    m = ct.mapped(ct.partition(z, [2] * len(grid)), mp, 1)
+    order = oracle.mapped_schedule(grid, mp)
+    assert m.num_items() == len(order)
+    assert [m.index(t) for t in range(len(order))] == order
+    with pytest.raises(ct.CutileError, match="outside"):
+        m.index(len(order))
+
+
+# ---- HIP kernels (GPU) -----------------------------------------------------------------------
+def _expected_flat_index(dims, tile):
+    grid = [-(-d // t) for d, t in zip(dims, tile)]
+    idx = np.indices(dims)
+    flat = np.zeros(dims, np.int64)
+    for a in range(len(dims)):
+        flat = flat * grid[a] + idx[a] // tile[a]
+    return flat.astype(np.int32)
+
+
+@pytest.mark.gpu
+def test_gpu_schedule_matrix_covers_every_tile_exactly_once(ct, dev):
+    m = CASES["schedule_matrix"]
+    for c in m["cases"]:
+        z = torch.full(c["dims"], m["poison"], dtype=torch.int32, device=dev)
+        ct.mapped_tile_index(ct.mapped(ct.partition(z, c["tile"]), c["map_shape"], c["num_tile_blocks"]))
+        torch.cuda.synchronize()
+        assert np.array_equal(z.cpu().numpy(), _expected_flat_index(c["dims"], c["tile"])), c
+    # grids the tile shape does not divide, an owned axis, and a strided view
+    for dims, tile, mp, ntb in [([30, 21], [8, 8], [3, 2], 4), ([5, 70], [1, 16], [1, 0], 5), ([37], [8], [1], 2),
+                                ([3, 10, 9], [1, 4, 4], [1, 2, 2], 7), ([3, 10, 9], [1, 4, 4], [0, 1, 1], 9)]:
+        wide = torch.full(dims[:-1] + [dims[-1] + 3], m["poison"], dtype=torch.int32, device=dev)
+        z = wide[..., : dims[-1]]
+        ct.mapped_tile_index(ct.mapped(ct.partition(z, tile), mp, ntb))
+        torch.cuda.synchronize()
+        assert np.array_equal(z.cpu().numpy(), _expected_flat_index(dims, tile)), (dims, tile, mp, ntb)
+        assert torch.all(wide[..., dims[-1]:] == m["poison"])
+
+
+@pytest.mark.gpu
+def test_gpu_explicit_grid_is_a_checked_override(ct, dev):
+    # an explicit .grid() must equal (num_tile_blocks, 1, 1)
+    grid, mp = (5, 4), (2, 2)
+    z = torch.full((5 * 4, 4 * 4), -1, dtype=torch.int32, device=dev)
+    part = ct.mapped(ct.partition(z, [4, 4]), mp, 20)
+    ct.mapped_tile_index(part, grid=(20, 1, 1))
+    with pytest.raises(ct.CutileError, match="does not match the inferred partition grid"):
+        ct.mapped_tile_index(part, grid=(10, 1, 1))
+    torch.cuda.synchronize()
+    assert np.array_equal(z.cpu().numpy(), _expected_flat_index([20, 16], [4, 4]))
+
+
+def _persistent_inputs(case):
+    m, n, k = case["m"], case["n"], case["k"]
+    r, c = np.meshgrid(np.arange(m), np.arange(k), indexing="ij")
+    x = ((r % 7).astype(np.float32) - 3.0) * np.float32(0.25) + (c % 5).astype(np.float32) * np.float32(0.125)
+    r, c = np.meshgrid(np.arange(k), np.arange(n), indexing="ij")
+    y = ((r % 3).astype(np.float32) + 1.0) * np.float32(0.2) - (c % 11).astype(np.float32) * np.float32(0.05)
+    return x.astype(np.float32), y.astype(np.float32)
+
+
+@pytest.mark.gpu
+def test_gpu_persistent_gemm_reference_example(ct, dev):
+    """persistent_gemm.rs as written: f32, 16x16x8 tiles, M = N = 64, K = 32, map [4, 1], four tile blocks"""
+    all_cases = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_cases.json")))
+    p, launch = all_cases["persistent_gemm_patterned"], CASES["persistent_gemm_launch"]
+    x, y = _persistent_inputs(p)
+    z = torch.full((p["m"], p["n"]), float("nan"), dtype=torch.float32, device=dev)
+    bm, bn, bk = p["tile"]
+    ct.gemm_persistent(ct.mapped(ct.partition(z, [bm, bn]), launch["map_shape"], launch["num_tile_blocks"]),
+                       torch.from_numpy(x).to(dev), torch.from_numpy(y).to(dev),
+                       generics=["f32", bm, bn, bk, launch["map_shape"][0], launch["map_shape"][1]])
+    torch.cuda.synchronize()
+    got = z.cpu().numpy()
+    for s in p["samples"]:
+        assert abs(got[s["row"], s["col"]] - s["num"] / s["den"]) < p["abs_tol"]
+    assert np.max(np.abs(got - oracle.cpu_gemm_f32(x, y))) < p["abs_tol"]
+    with pytest.raises(ct.CutileError, match="MAP_SHAPE"):
+        ct.gemm_persistent(ct.mapped(ct.partition(z, [bm, bn]), [4, 1], 4), torch.from_numpy(x).to(dev),
+                           torch.from_numpy(y).to(dev), generics=["f32", bm, bn, bk, 2, 1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k,tile,mp,ntb,variant", [
+    (1024, 1024, 512, 256, (8, 1), 16, None),                   # full grid: one item per tile block
+    (1024, 768, 256, 256, (2, 1), 5, "bf16_256x256x64_d2x4"),   # a non-divisor number of tile blocks
+    (1000, 520, 200, 256, (3, 2), 1, None),                     # ragged edges, K tail, one tile block walks everything
+    (640, 384, 128, 128, (4, 1), 7, None),
+    (300, 200, 96, 64, (2, 2), 6, None),                        # no matrix-core variant for 64x64 tiles: any-layout kernel
+])
+def test_gpu_persistent_gemm_bf16(ct, dev, m, n, k, tile, mp, ntb, variant):
+    a, b = normal_bf16_bits((m, k), 801, k ** -0.5), normal_bf16_bits((k, n), 802)
+    z = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ct.gemm_persistent(ct.mapped(ct.partition(z, [tile, tile]), mp, ntb), to_dev_bf16(a, dev), to_dev_bf16(b, dev), variant=variant)
+    torch.cuda.synchronize()
+    ref = oracle.bf16_bits_to_f32(oracle.gemm_bf16(a, b))
+    got = z.float().cpu().numpy()
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, ref) <= 1e-2        # the bf16 GEMM tolerance
