@@ -203,6 +203,25 @@ class Gemm(Workload):
                {"rel_l2_sampled_rows": rel, "tolerance": 1e-2, "ok": rel <= 1e-2}
 
 
+class GemmPersistent(Gemm):
+    """The reference's persistent form (cutile-examples/examples/persistent_gemm.rs): one tile block per CU walks
+    the tiles of a mapped output partition in grouped order; zero initial accumulator (z is not read)."""
+
+    def __init__(self, s, tile_blocks=256, group_m=8):
+        super().__init__(s)
+        self.name = f"gemm_bf16_{s}_persistent"
+        self.tile_blocks, self.group_m = tile_blocks, group_m
+        self.config = {"workload": f"persistent GEMM bf16 M=N=K={s}, z = A·B over a mapped partition: map [{group_m}, 1], "
+                                   f"{tile_blocks} tile blocks, f32 accumulate, bf16 z", "tile": "256x256x64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        super().setup(ct, torch, oracle, dev)
+        self.zm = ct.mapped(self.zp, [self.group_m, 1], self.tile_blocks)
+
+    def launch(self):
+        self.ct.gemm_persistent(self.zm, self.a, self.b)
+
+
 class Fmha(Workload):
     unit, dtype, bound, peak_key = "TFLOP/s", "bf16 io / f32 softmax+acc", "mfma", "mfma_bf16"
     b, h, s, d = 4, 32, 4096, 128
@@ -483,7 +502,7 @@ class DecodeAttention(Workload):
 
 
 def make_workloads():
-    return [Gemm(8192), Gemm(4096), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(),
+    return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(),
             AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention()]
 
 

@@ -258,10 +258,24 @@ auto unpartition_op(Op op) {
 }
 
 // ---- kernel launchers ------------------------------------------------------------------------
+// What a launcher hands back for a stored argument (KernelOutput::recover, tensor.rs:1945-1969): the argument itself,
+// except that a mapped partition gives back its inner partition.
+template <class T>
+struct Recovered {
+  using type = T;
+  static T get(T&& v) { return std::move(v); }
+};
+template <class P>
+struct Recovered<MappedLaunchPartition<P>> {
+  using type = P;
+  static P get(MappedLaunchPartition<P>&& v) { return std::move(v).into_partition(); }
+};
+
 template <class Fn, class... ArgOps>
-class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple<typename ArgOps::Output...>> {
+class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple<typename Recovered<typename ArgOps::Output>::type...>> {
  public:
-  using Out = std::tuple<typename ArgOps::Output...>;
+  using Stored = std::tuple<typename ArgOps::Output...>;
+  using Out = std::tuple<typename Recovered<typename ArgOps::Output>::type...>;
   explicit KernelLauncher(ArgOps&&... ops) : ops_(std::move(ops)...) {}
   KernelLauncher(KernelLauncher&&) = default;
   // Builder methods of the generated launcher (cutile-macro/src/_module.rs:901-923).
@@ -273,7 +287,7 @@ class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple
     // 1. run the argument ops in signature order; 2. validate + launch; 3. hand the arguments back.
     auto args = std::move(ops_).execute(ctx);
     if (args.is_err()) return args.error();
-    Out vals = std::move(args).unwrap();
+    Stored vals = std::move(args).unwrap();
     std::vector<const char*> gptrs;
     for (auto& s : generics_) gptrs.push_back(s.c_str());
     cutile_launch_opts_t opts{};
@@ -283,7 +297,7 @@ class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple
     opts.variant = variant_.empty() ? nullptr : variant_.c_str();
     cutile_status_t s = std::apply([&](auto&... a) { return Fn::launch(ctx.stream()->raw(), &opts, a...); }, vals);
     if (s != CUTILE_SUCCESS) return DeviceError::from_status(s);
-    return vals;
+    return std::apply([](auto&... a) { return Out(Recovered<std::decay_t<decltype(a)>>::get(std::move(a))...); }, vals);
   }
 
  private:
@@ -451,6 +465,21 @@ struct SplitkReduceMergeFn {
     return cutile_launch_splitk_reduce_merge(s, &aa, &la, &op, o);
   }
 };
+struct GemmPersistentFn {
+  template <class Z, class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y) {
+    auto zm = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y);
+    return cutile_launch_gemm_persistent(s, &zm, &xa, &ya, o);
+  }
+};
+struct MappedTileIndexFn {
+  template <class Z>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z) {
+    auto zm = z.arg();
+    return cutile_launch_mapped_tile_index(s, &zm, o);
+  }
+};
 }  // namespace kernels
 
 // saxpy(y: partition, a, x) -> (y, a, x)        cutile-examples/examples/saxpy.rs:12-17
@@ -494,6 +523,10 @@ template <class NK, class NV, class KC, class VC, class P> auto kv_cache_update_
 template <class Q, class K, class V, class A, class L, class P> auto fmha_decode_gqa_split(Q&& q, K&& k, V&& v, A&& att_out, L&& lse_out, float qk_scale, P&& position_start) { return make_launcher<kernels::FmhaDecodeGqaSplitFn>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<A>(att_out), std::forward<L>(lse_out), qk_scale, std::forward<P>(position_start)); }
 // splitk_reduce_merge(att_partial, lse_partial, out: [1,GROUP,CHUNK_D])          attention.rs:917-930
 template <class A, class L, class O> auto splitk_reduce_merge(A&& att_partial, L&& lse_partial, O&& out) { return make_launcher<kernels::SplitkReduceMergeFn>(std::forward<A>(att_partial), std::forward<L>(lse_partial), std::forward<O>(out)); }
+// gemm_persistent(z: mapped partition [BM,BN], x, y) -> (z's partition, x, y)   cutile-examples/examples/persistent_gemm.rs:35-45
+template <class Z, class X, class Y> auto gemm_persistent(Z&& z, X&& x, Y&& y) { return make_launcher<kernels::GemmPersistentFn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y)); }
+// write_flat_index_rank{1,2,3}(z: mapped i32 partition) -> (z's partition)      cutile/tests/gpu/mapped_partition_schedule_matrix.rs:30-76
+template <class Z> auto mapped_tile_index(Z&& z) { return make_launcher<kernels::MappedTileIndexFn>(std::forward<Z>(z)); }
 
 namespace api {
 template <class T> struct is_graph_node_memcpy : std::true_type {};

@@ -192,6 +192,7 @@ size_t addressable_bytes(const std::vector<int32_t>& shape, const std::vector<in
 template <class T> class Tensor;
 template <class T> class TensorView;
 template <class X> class Partition;
+template <class P> class MappedLaunchPartition;
 
 // ---- Tensor ----------------------------------------------------------------------------------
 template <class T>
@@ -412,12 +413,72 @@ class Partition {
   }
   // unpartition(): recover the tensor (owned form), tensor.rs:1519-1541.
   X unpartition() && { return std::move(object_); }
+  // map(): attach a host-side partition map (tensor.rs:314-329); defined after MappedLaunchPartition.
+  MappedLaunchPartition<Partition<X>> map(std::vector<int32_t> map_shape, uint32_t num_tile_blocks) &&;
 
  private:
   X object_;
   std::vector<int32_t> tile_;
   bool prefix_;
 };
+
+// Map-shape sentinel of an owned axis (tensor.rs:331-337): the axis is not traversed by the stream of
+// work items; each item owns its full extent and the kernel walks it.
+constexpr int32_t OWNED = CUTILE_MAP_OWNED;
+
+// MappedLaunchPartition (tensor.rs:339-401): the logical tile grid of `partition` is walked by
+// `num_tile_blocks` tile blocks; the launch grid is (num_tile_blocks, 1, 1).  A kernel hands the inner
+// partition back (tensor.rs:1945-1969).
+template <class P>
+class MappedLaunchPartition {
+ public:
+  using Inner = P;
+  MappedLaunchPartition(P partition, std::vector<int32_t> map_shape, uint32_t num_tile_blocks)
+      : partition_(std::move(partition)), map_shape_(std::move(map_shape)), num_tile_blocks_(num_tile_blocks) {}
+  MappedLaunchPartition(MappedLaunchPartition&&) = default;
+  MappedLaunchPartition& operator=(MappedLaunchPartition&&) = default;
+
+  const P& partition() const { return partition_; }
+  const std::vector<int32_t>& map_shape() const { return map_shape_; }
+  uint32_t num_tile_blocks() const { return num_tile_blocks_; }
+
+  cutile_mapped_partition_arg_t arg() const {
+    cutile_mapped_partition_arg_t m{};
+    m.partition = partition_.arg();
+    m.map_rank = (int32_t)map_shape_.size();
+    for (size_t i = 0; i < map_shape_.size() && i < 3; ++i) m.map_shape[i] = map_shape_[i];
+    m.num_tile_blocks = num_tile_blocks_;
+    return m;
+  }
+  // validate (tensor.rs:352-400): the launch grid, or the reason the map cannot traverse the partition
+  Result<std::array<uint32_t, 3>> grid() const {
+    std::array<uint32_t, 3> g{};
+    cutile_mapped_partition_arg_t m = arg();
+    CUTILE_TRY_STATUS(cutile_mapped_partition_grid(&m, g.data()));
+    return g;
+  }
+  // the block id per partition axis that stream item `item` maps to (tile block b visits b, b + n, ...)
+  Result<std::array<uint32_t, 3>> index(uint32_t item) const {
+    std::array<uint32_t, 3> idx{};
+    cutile_mapped_partition_arg_t m = arg();
+    CUTILE_TRY_STATUS(cutile_mapped_partition_index(&m, item, idx.data(), nullptr));
+    return idx;
+  }
+  P into_partition() && { return std::move(partition_); }
+
+ private:
+  P partition_;
+  std::vector<int32_t> map_shape_;
+  uint32_t num_tile_blocks_;
+};
+
+template <class X>
+MappedLaunchPartition<Partition<X>> Partition<X>::map(std::vector<int32_t> map_shape, uint32_t num_tile_blocks) && {
+  if (prefix_)
+    throw std::logic_error("a partial-coverage (prefix) partition cannot be mapped: a mapped schedule covers its full "
+                           "index space by construction");
+  return MappedLaunchPartition<Partition<X>>(std::move(*this), std::move(map_shape), num_tile_blocks);
+}
 
 template <class T>
 Partition<Tensor<T>> Tensor<T>::partition(std::vector<int32_t> tile) && {

@@ -147,6 +147,36 @@ TEST(decode_kernels_closed_forms) {
   CHECK(!r.is_ok());
 }
 
+TEST(persistent_gemm_example) {
+  // cutile-examples/examples/persistent_gemm.rs:61-126 as written: f32, 16x16x8 tiles, M = N = 64, K = 32, map [4, 1], 4 tile blocks
+  auto stream = new_stream();
+  const int M = 64, N = 64, K = 32;
+  auto xh = std::make_shared<std::vector<float>>(M * K), yh = std::make_shared<std::vector<float>>(K * N);
+  for (int r = 0; r < M; ++r)
+    for (int c = 0; c < K; ++c) (*xh)[r * K + c] = ((float)(r % 7) - 3.0f) * 0.25f + (float)(c % 5) * 0.125f;
+  for (int r = 0; r < K; ++r)
+    for (int c = 0; c < N; ++c) (*yh)[r * N + c] = ((float)(r % 3) + 1.0f) * 0.2f - (float)(c % 11) * 0.05f;
+  auto z = api::full<float>(-333.25, {M, N}).sync_on(stream).unwrap().partition({16, 16}).map({4, 1}, 4);
+  auto x = std::make_shared<Tensor<float>>(reshape_op(api::copy_host_vec_to_device(xh), {M, K}).sync_on(stream).unwrap());
+  auto y = std::make_shared<Tensor<float>>(reshape_op(api::copy_host_vec_to_device(yh), {K, N}).sync_on(stream).unwrap());
+  auto [zp, x_, y_] = gemm_persistent(std::move(z), x, y).generics({"f32", "16", "16", "8", "4", "1"}).sync_on(stream).unwrap();
+  auto zh = api::to_host_vec(std::move(zp).unpartition()).sync_on(stream).unwrap();
+  float max_err = 0.0f;
+  for (int i = 0; i < M; ++i)
+    for (int j = 0; j < N; ++j) {
+      float ref = 0.0f;
+      for (int t = 0; t < K; ++t) ref += (*xh)[i * K + t] * (*yh)[t * N + j];   // cpu_gemm, persistent_gemm.rs:140-152
+      max_err = std::max(max_err, std::fabs(zh[i * N + j] - ref));
+    }
+  CHECK(max_err < 1e-3f);
+  // the coverage kernel of the reference's schedule tests: every tile holds its own index, none keeps the fill
+  auto idx = api::full<int32_t>(-0x5EAD, {24, 40}).sync_on(stream).unwrap().partition({8, 8}).map({3, 2}, 5);
+  auto [ip] = mapped_tile_index(std::move(idx)).sync_on(stream).unwrap();
+  auto ih = api::to_host_vec(std::move(ip).unpartition()).sync_on(stream).unwrap();
+  for (int r = 0; r < 24; ++r)
+    for (int c = 0; c < 40; ++c) CHECK(ih[r * 40 + c] == (r / 8) * 5 + c / 8);
+}
+
 TEST(gemm_ones_non_divisible) {
   auto stream = new_stream();
   const int m = 200, n = 264, k = 128;

@@ -260,6 +260,42 @@ TEST(launchers_hand_arguments_back_in_the_form_given) {
   CHECK(wrong.is_err() && wrong.error().message.find("does not match the inferred partition grid") != std::string::npos);
 }
 
+TEST(mapped_partitions_validate_and_hand_the_inner_partition_back) {
+  auto s = fresh_stream();
+  cutile_testing_clear_log();
+  // cutile/src/tensor.rs:2203-2345: the launch grid is (num_tile_blocks, 1, 1) when the map can traverse the partition
+  auto z = api::zeros<float>({8, 12}).sync_on(s).unwrap();     // logical grid (2, 3) with [4, 4] tiles
+  auto grid_of = [&](std::vector<int32_t> map, uint32_t n) { return z.partition_mut({4, 4}).map(std::move(map), n).grid(); };
+  CHECK(grid_of({4, 1}, 3).unwrap() == (std::array<uint32_t, 3>{3, 1, 1}));
+  CHECK(grid_of({4, 1}, 7).error().message.find("num_tile_blocks cannot exceed the streamed logical tile count") != std::string::npos);
+  CHECK(grid_of({1, OWNED}, 2).unwrap()[0] == 2 && grid_of({1, OWNED}, 3).is_err());
+  CHECK(grid_of({OWNED, OWNED}, 1).error().message.find("at least one streamed (non-OWNED) map axis") != std::string::npos);
+  CHECK(grid_of({OWNED, 1}, 3).unwrap()[0] == 3);
+  CHECK(grid_of({4, 1}, 0).error().message.find("num_tile_blocks > 0") != std::string::npos);
+  CHECK(grid_of({1}, 2).error().message.find("map rank must match the logical partition grid rank") != std::string::npos);
+  CHECK(grid_of({1, 1, 1, 1}, 2).error().message.find("rank-1 through rank-3 map shape") != std::string::npos);
+  CHECK_THROWS(z.partition_mut({4, 4}).prefix().map({1, 1}, 2), "cannot be mapped");   // tensor.rs:319-323
+  // the schedule as a host-visible map: bands of two tile rows, column by column
+  auto m = z.partition_mut({4, 4}).map({2, 1}, 2);
+  CHECK(m.index(0).unwrap() == (std::array<uint32_t, 3>{0, 0, 0}) && m.index(1).unwrap() == (std::array<uint32_t, 3>{1, 0, 0}) &&
+        m.index(2).unwrap() == (std::array<uint32_t, 3>{0, 1, 0}) && m.index(5).unwrap() == (std::array<uint32_t, 3>{1, 2, 0}));
+  CHECK(m.index(6).is_err());
+  // persistent_gemm.rs:96-108: the launcher takes the mapped partition and returns the partition
+  auto x = api::zeros<float>({64, 32}).sync_on(s).unwrap();
+  auto y = api::zeros<float>({32, 64}).sync_on(s).unwrap();
+  auto out = api::zeros<float>({64, 64}).sync_on(s).unwrap().partition({16, 16}).map({4, 1}, 4);
+  auto [zp, xb, yb] = gemm_persistent(std::move(out), &x, &y).generics({"f32", "16", "16", "8", "4", "1"}).sync_on(s).unwrap();
+  CHECK(last_symbol() == "gemm_persistent_entry__f32_generic");
+  CHECK(xb == &x && yb == &y);
+  Tensor<float> z_back = std::move(zp).unpartition();
+  CHECK(z_back.shape() == std::vector<int32_t>({64, 64}));
+  auto bad = gemm_persistent(z_back.partition_mut({16, 16}).map({4, 1}, 4), &x, &y).generics({"f32", "16", "16", "8", "2", "1"}).sync_on(s);
+  CHECK(bad.is_err() && bad.error().message.find("MAP_SHAPE") != std::string::npos);
+  auto short_y = api::zeros<float>({16, 64}).sync_on(s).unwrap();
+  auto ties = gemm_persistent(z_back.partition_mut({16, 16}).map({4, 1}, 4), &x, &short_y).generics({"f32", "16", "16", "8", "4", "1"}).sync_on(s);
+  CHECK(ties.is_err() && ties.error().message.find("ceil(dim(x, 1)/BK) <= ceil(dim(y, 0)/BK)") != std::string::npos);
+}
+
 TEST(graph_capture_replay_and_failure_matrix) {
   auto s = fresh_stream();
   Tensor<float> out = api::zeros<float>({1024}).sync_on(s).unwrap();
