@@ -87,8 +87,17 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
     if not os.path.exists(embed) or open(embed).read() != text:
         with open(embed, "w") as f:
             f.write(text)
+    # the device compiler's identity, for the provenance of tuning records
+    ver = subprocess.run([HIPCC, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True).stdout
+    keep = [l.strip() for l in ver.splitlines() if l.startswith(("HIP version", "AMD clang version", "clang version"))]
+    fingerprint = "; ".join(keep)[:200].replace("\\", "/").replace('"', "'") or "unknown"
+    toolchain = os.path.join(BUILD_DIR, "toolchain.h")
+    text_h = f'#define CUTILE_TOOLCHAIN_FINGERPRINT "{fingerprint}"\n'
+    if not os.path.exists(toolchain) or open(toolchain).read() != text_h:
+        with open(toolchain, "w") as f:
+            f.write(text_h)
     sources = [os.path.join(HOST_DIR, s) for s in HOST_SOURCES]
-    deps = sources + [embed] + list(images.values()) + [
+    deps = sources + [embed, toolchain] + list(images.values()) + [
         os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".h")
     ] + [os.path.join(ROOT, "..", "include", "cutile_hip.h")]
     if force or not _newer(LIB_PATH, deps):
@@ -98,7 +107,7 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
             o = os.path.join(BUILD_DIR, os.path.basename(s) + ".o")
             objs.append(o)
             if force or not _newer(o, deps):
-                jobs.append([CXX] + HOST_FLAGS + ["-c", s, "-o", o])
+                jobs.append([CXX] + HOST_FLAGS + ["-I", BUILD_DIR, "-c", s, "-o", o])
         with ThreadPoolExecutor(max_workers=6) as ex:
             list(ex.map(_run, jobs))
         _run([CXX, "-shared", "-o", LIB_PATH] + objs + ["-ldl", "-pthread", "-Wl,--no-undefined"])

@@ -1,5 +1,6 @@
 // Part B of the C ABI: the table of precompiled gfx950 kernels (see kernel_table.h).
 #include "kernel_table.h"
+#include "toolchain.h"   // written by the build: CUTILE_TOOLCHAIN_FINGERPRINT
 
 #include <atomic>
 #include <cstring>
@@ -306,6 +307,27 @@ cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const 
                  "no variant '%s' of kernel '%s'; available: %s", variant, function,
                  list_variants(function).c_str());
   g_preferred[function] = variant;
+  return CUTILE_SUCCESS;
+}
+
+const char* cutile_library_version(void) { return "0.1.0"; }
+const char* cutile_toolchain_fingerprint(void) { return CUTILE_TOOLCHAIN_FINGERPRINT; }
+const char* cutile_target_arch(void) { return "gfx950"; }
+
+cutile_status_t cutile_kernel_fingerprint(const char* function, const char* variant, char out[17]) {
+  CUTILE_REQUIRE(function && out, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  const KernelEntry* entry = nullptr;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, function) == 0 && (!variant || strcmp(e.variant, variant) == 0)) { entry = &e; break; }
+  CUTILE_REQUIRE(entry, CUTILE_ERR_KERNEL_NOT_FOUND, "no kernel '%s'%s%s; available: %s", function, variant ? " variant " : "",
+                 variant ? variant : "", list_variants(function).c_str());
+  uint64_t h = 0xcbf29ce484222325ull;   // FNV-1a
+  auto mix = [&](const unsigned char* p, size_t n) { for (size_t i = 0; i < n; ++i) { h ^= p[i]; h *= 0x100000001b3ull; } };
+  const ImageRef img = image_ref(entry->image);
+  mix(img.start, (size_t)(img.end - img.start));
+  mix((const unsigned char*)function, strlen(function) + 1);
+  if (variant) mix((const unsigned char*)entry->symbol, strlen(entry->symbol) + 1);
+  snprintf(out, 17, "%016llx", (unsigned long long)h);
   return CUTILE_SUCCESS;
 }
 

@@ -208,6 +208,16 @@ int32_t cutile_kernel_list(const char** names, int32_t cap);
  * several fit (the autotuner's output).  variant == NULL restores the default. */
 cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const char* variant);
 
+/* Provenance of the running library, for records of tuning winners (cutile/src/tune.rs:762-832 keeps
+ * source_hash, toolchain fingerprint, arch and crate version; here they come from the kernel table):
+ * the library version, the device compiler's version text captured at build time, the one target
+ * architecture, and a 16-hex-digit fingerprint of the code object that holds `function` (variant == NULL)
+ * or of that code object plus one variant's symbol. */
+const char* cutile_library_version(void);
+const char* cutile_toolchain_fingerprint(void);
+const char* cutile_target_arch(void);
+cutile_status_t cutile_kernel_fingerprint(const char* function, const char* variant, char out[17]);
+
 /* ======================================================================== */
 /* Part C — launch builder                                                   */
 /* ======================================================================== */

@@ -3,6 +3,7 @@
 // fake-backed tests: cuda-async/tests/{execute_once,error_handling,cuda_graph}.rs,
 // cutile/src/tensor.rs:2161-2202, cutile/src/bench.rs:266-291,
 // cutile/src/tune.rs (FakeOracle tests), cuda-async/src/device_future.rs:325-384.
+#include <unistd.h>
 #include <cutile/cutile.hpp>
 #include <cutile_hip_testing.h>
 
@@ -435,47 +436,226 @@ TEST(bench_quantiles) {
   CHECK(m.reps() == 3 && calls == 1 + 1 + 3);
 }
 
-struct FakeOracle : tune::Oracle {  // cutile/src/tune.rs:1045
+struct FakeOracle : tune::Oracle {  // cutile/src/tune.rs:1037-1069
   std::vector<tune::Config> cfgs;
   std::map<std::string, float> ms;
   std::vector<std::string> measured;
-  size_t budget = SIZE_MAX;
+  size_t budget = SIZE_MAX;    // measurements allowed before the budget reads zero
   const std::vector<tune::Config>& configs() const override { return cfgs; }
-  bool budget_exhausted() const override { return measured.size() >= budget; }
+  std::optional<std::chrono::nanoseconds> budget_remaining() const override {
+    if (budget == SIZE_MAX) return std::nullopt;
+    return std::chrono::nanoseconds(measured.size() >= budget ? 0 : 1000);
+  }
   tune::Trial measure(size_t i) override {
     measured.push_back(cfgs[i].id);
     auto it = ms.find(cfgs[i].id);
-    if (it == ms.end()) return tune::Trial::invalid(cfgs[i].id, "does not launch");
-    return tune::Trial::ok(cfgs[i].id, it->second, it->second, 5);
+    if (it == ms.end()) return tune::Trial::invalid(cfgs[i].id, "gate failed");
+    return tune::Trial::ok(cfgs[i].id, it->second, it->second, 3);
   }
 };
 
+static tune::Config bn_splits(int64_t bn, int64_t splits) { return tune::Config::make({{"BN", bn}, {"SPLITS", splits}}); }
+
 TEST(autotuner_search_semantics) {
   using tune::Config;
-  auto a = Config::make({{"bm", "128"}, {"bn", "128"}}), b = Config::make({{"bm", "256"}, {"bn", "256"}}), c = Config::make({{"bm", "64"}, {"bn", "64"}});
-  CHECK(a.id == "bm=128,bn=128" && *a.integer("bm") == 128 && !a.integer("zz") && *a.str("bn") == "128");
+  // tune.rs:1072-1080, 1424-1435, 1635-1644: ids are stable, sorted by key, and cannot alias
+  CHECK(Config::make({{"SPLITS", 8}, {"BN", 64}}).id == "BN=64,SPLITS=8" && bn_splits(64, 8).id == "BN=64,SPLITS=8");
+  CHECK(*bn_splits(64, 8).integer("BN") == 64 && !bn_splits(64, 8).integer("missing"));
+  CHECK(Config::make({{"A", 1}}).id != Config::make({{"A", "1"}}).id && Config::make({{"A", "1"}}).id == "A=\"1\"");
+  CHECK(Config::make({{"x", "1,y=2"}}).id != Config::make({{"x", "1"}, {"y", 2}}).id);
+  CHECK(Config::make({{"A=1,B", 2}}).id != Config::make({{"A", 1}, {"B", 2}}).id);
+  CHECK(Config::make({{"\"A\"", 1}}).id != Config::make({{"A", 1}}).id);
+  auto a = bn_splits(32, 2), b = bn_splits(64, 4), c = bn_splits(128, 8);
   CHECK(tune::space_hash({a, b, c}) == tune::space_hash({c, a, b}) && tune::space_hash({a, b}) != tune::space_hash({a, b, c}));
+  // FNV-1a over the sorted ids, each closed by a zero byte: no ids -> the offset basis; "a" -> two rounds by hand
+  CHECK(tune::space_hash({}) == "cbf29ce484222325");
+  {
+    uint64_t h = 0xcbf29ce484222325ull;
+    h = (h ^ 'x') * 0x100000001b3ull;
+    h = (h ^ '=') * 0x100000001b3ull;
+    h = (h ^ '1') * 0x100000001b3ull;
+    h = (h ^ 0) * 0x100000001b3ull;
+    char buf[17];
+    snprintf(buf, sizeof(buf), "%016llx", (unsigned long long)h);
+    CHECK(tune::space_hash({Config::make({{"x", 1}})}) == buf);
+  }
+  // tune.rs:1082-1112: every candidate once, the best median wins, an invalid one is data and never wins
   FakeOracle o;
   o.cfgs = {a, b, c};
-  o.ms = {{a.id, 2.0f}, {b.id, 1.0f}};  // c is invalid: data, not an error
+  o.ms = {{a.id, 32.0f}, {b.id, 64.0f}, {c.id, 128.0f}};
   auto trials = tune::GridSearch{}.search(o);
-  CHECK(trials.size() == 3 && !trials[2].measured && trials[2].invalid_reason == "does not launch");
-  CHECK(tune::best_config(o.cfgs, trials)->id == b.id);
-  // resume: measured known trials are kept, invalid ones retried, stale configs ignored
+  CHECK(o.measured.size() == 3 && trials.size() == 3 && *tune::best_config(o.cfgs, trials)->integer("BN") == 32);
+  FakeOracle inv;
+  inv.cfgs = {a, b};
+  inv.ms = {{b.id, 1.0f}};
+  auto ti = tune::GridSearch{}.search(inv);
+  CHECK(ti.size() == 2 && !ti[0].measured && ti[0].invalid_reason == "gate failed" && *tune::best_config(inv.cfgs, ti)->integer("BN") == 64);
+  // tune.rs:1114-1136, 1437-1479: resume keeps measured known trials, retries invalid ones, drops stale configs
   FakeOracle o2;
   o2.cfgs = {a, b, c};
-  o2.ms = {{a.id, 2.0f}, {b.id, 1.0f}, {c.id, 0.5f}};
-  std::vector<tune::Trial> known = {tune::Trial::ok(a.id, 2.0f, 2.0f, 5), tune::Trial::invalid(c.id, "transient"), tune::Trial::ok("gone=1", 0.1f, 0.1f, 5)};
-  auto t2 = tune::GridSearch{}.resume(known).search(o2);
-  CHECK(o2.measured == std::vector<std::string>({b.id, c.id}));
-  CHECK(tune::best_config(o2.cfgs, t2)->id == c.id);  // the stale 0.1 ms record neither wins nor shadows
-  // budget: stop measuring when exhausted
+  o2.ms = {{a.id, 9.0f}, {b.id, 9.0f}, {c.id, 9.0f}};
+  auto t2 = tune::GridSearch{}.resume({tune::Trial::ok(b.id, 0.5f, 0.5f, 3)}).search(o2);
+  CHECK(o2.measured.size() == 2 && t2.size() == 3 && *tune::best_config(o2.cfgs, t2)->integer("BN") == 64);
+  FakeOracle o4;
+  o4.cfgs = {b};
+  o4.ms = {{b.id, 1.0f}};
+  auto t4 = tune::GridSearch{}.resume({tune::Trial::ok("BN=16,SPLITS=2", 0.1f, 0.1f, 3)}).search(o4);
+  CHECK(t4.size() == 1 && *tune::best_config(o4.cfgs, t4)->integer("BN") == 64);
+  FakeOracle o5;
+  o5.cfgs = {b};
+  o5.ms = {{b.id, 1.0f}};
+  auto t5 = tune::GridSearch{}.resume({tune::Trial::invalid(b.id, "transient")}).search(o5);
+  CHECK(o5.measured.size() == 1 && t5.size() == 1 && *t5[0].median() == 1.0f);
+  // tune.rs:1138-1149: a zero budget measures nothing
   FakeOracle o3;
   o3.cfgs = {a, b, c};
   o3.ms = o2.ms;
-  o3.budget = 1;
-  CHECK(tune::GridSearch{}.search(o3).size() == 1);
-  // end to end on the recording runtime: candidates that fail to set up are recorded as invalid
+  o3.budget = 0;
+  CHECK(tune::GridSearch{}.search(o3).empty());
+  // tune.rs:1500-1522: NaN never wins
+  CHECK(*tune::best_config({b, c}, {tune::Trial::ok(b.id, NAN, NAN, 3), tune::Trial::ok(c.id, 2.0f, 2.0f, 3)})->integer("BN") == 128);
+  // tune.rs:1481-1498: prune composes with configs in either order
+  auto keep = [](const Config& cfg) { return *cfg.integer("BN") != 32; };
+  CHECK(tune::Autotuner("t").prune(keep).configs({a, b}).pruned_configs().size() == 1);
+  CHECK(tune::Autotuner("t").configs({a, b}).prune(keep).pruned_configs()[0].id == b.id);
+}
+
+TEST(autotuner_runoff_verdicts) {   // tune.rs:1533-1632
+  auto a = bn_splits(32, 2), b = bn_splits(64, 4);
+  auto silent = tune::TrialLog::open(std::nullopt, "t", "s").unwrap();
+  auto meas = [](std::vector<float> t) { return bench::Measurement(std::move(t)); };
+  for (bool b_failed : {false, true}) {
+    std::vector<tune::Trial> trials;
+    tune::RunoffError err{b_failed ? tune::RunoffError::Kind::SetupB : tune::RunoffError::Kind::SetupA, DeviceError::tensor("boom")};
+    auto winner = tune::runoff_verdict(a, b, err, &trials, &silent);
+    CHECK(winner.id == (b_failed ? a.id : b.id) && trials.size() == 1 && trials[0].config_id == (b_failed ? b.id : a.id));
+    CHECK(!trials[0].measured && trials[0].invalid_reason.find("runoff setup failed") != std::string::npos);
+  }
+  std::vector<tune::Trial> none;
+  CHECK(tune::runoff_verdict(a, b, tune::RunoffError{tune::RunoffError::Kind::Bench, DeviceError::tensor("stream died")}, &none, &silent).id == a.id && none.empty());
+  std::vector<tune::Trial> scratch;
+  CHECK(tune::runoff_verdict(a, b, std::make_pair(meas({2.0f, 2.0f, 2.0f}), meas({NAN, NAN})), &scratch, &silent).id == a.id);
+  CHECK(tune::runoff_verdict(a, b, std::make_pair(meas({NAN}), meas({3.0f})), &scratch, &silent).id == b.id);
+  std::vector<tune::Trial> real;
+  CHECK(tune::runoff_verdict(a, b, std::make_pair(meas({1.0f, 2.0f, 3.0f}), meas({4.0f, 5.0f, 6.0f})), &real, &silent).id == a.id);
+  CHECK(real.size() == 2 && real[0].measured && real[0].median_ms == 2.0f && real[0].min_ms == 1.0f && real[0].reps == 3);
+}
+
+TEST(trial_log_roundtrips_resumes_and_refuses_foreign_logs) {   // tune.rs:1364-1421, 1646-1663
+  std::string path = "/tmp/cutile_tune_log_" + std::to_string(getpid());
+  remove(path.c_str());
+  {
+    auto log = tune::TrialLog::open(path, "t", "s").unwrap();
+    log.append(tune::Trial::ok("BN=64", 1.5f, 1.4f, 5));
+    log.append(tune::Trial::invalid("BN=128", "launch check"));
+  }
+  {
+    std::ifstream in(path);
+    std::string l1, l2, l3;
+    std::getline(in, l1); std::getline(in, l2); std::getline(in, l3);
+    CHECK(l1 == "{\"log_schema\":1,\"tuner\":\"t\",\"space\":\"s\"}");
+    CHECK(l2 == "{\"config_id\":\"BN=64\",\"state\":{\"Measured\":{\"median_ms\":1.5,\"min_ms\":1.4,\"reps\":5}}}");
+    CHECK(l3 == "{\"config_id\":\"BN=128\",\"state\":{\"Invalid\":{\"reason\":\"launch check\"}}}");
+  }
+  auto again = tune::TrialLog::open(path, "t", "s").unwrap();
+  CHECK(again.existing_trials().size() == 2 && *again.existing_trials()[0].median() == 1.5f && !again.existing_trials()[1].median());
+  CHECK(tune::TrialLog::open(path, "other", "s").error().message.find("belongs to tuner") != std::string::npos);
+  CHECK(tune::TrialLog::open(path, "t", "different").error().message.find("belongs to tuner") != std::string::npos);
+  { std::ofstream torn(path, std::ios::app); torn << "{\"config_id\":\"torn"; }      // a crash mid-write
+  { auto log = tune::TrialLog::open(path, "t", "s").unwrap(); log.append(tune::Trial::ok("BN=256", 2.0f, 2.0f, 3)); }
+  CHECK(tune::TrialLog::open(path, "t", "s").unwrap().existing_trials().size() == 3);   // torn line dropped, new record intact
+  { std::ofstream junk(path, std::ios::trunc); junk << "not json\n"; }
+  CHECK(tune::TrialLog::open(path, "t", "s").error().message.find("no valid header") != std::string::npos);
+  { std::ofstream ws(path, std::ios::trunc); ws << "\n"; }                               // whitespace only: fresh
+  { auto log = tune::TrialLog::open(path, "t", "s").unwrap(); log.append(tune::Trial::invalid("BN=1,SPLITS=1", "x")); }
+  CHECK(tune::TrialLog::open(path, "t", "s").unwrap().existing_trials().size() == 1);
+  remove(path.c_str());
+}
+
+TEST(tuning_records_roundtrip_and_refuse_stale_provenance) {   // tune.rs:1151-1362
+  using tune::Record;
+  using tune::RecordEntry;
+  auto ws = [] { return tune::Workspace{"fmha_decode", "abc123", "sm_120", "release 13.3, V13.3.36", std::nullopt}; };
+  std::string path = "/tmp/cutile_record_" + std::to_string(getpid()) + ".json";
+  auto decline = [](const RecordEntry&) -> Result<std::optional<std::string>> { return std::optional<std::string>(); };
+  auto err_of = [&](const tune::Workspace& w, const Record::VerifyKey& v) { return Record::load_verified(path, w, v).error().message; };
+  {
+    Record a(ws());
+    a.cutile_version = cutile_library_version();
+    a.insert({"tg<=512", bn_splits(64, 8), 1.25f, 12, std::string(64, 'f')});
+    CHECK(a.save(path).is_ok());
+    auto [loaded, warnings] = Record::load_verified(path, ws(), [](const RecordEntry& e) -> Result<std::optional<std::string>> { return e.l2_key; }).unwrap();
+    CHECK(warnings.empty() && *loaded.get("tg<=512")->config.integer("BN") == 64 && loaded.get("tg<=512")->samples == 12 && loaded.get("tg<=512")->median_ms == 1.25f);
+    // recomputed key differs => refused; toolchain drift => the verifier is not even consulted, one warning
+    CHECK(err_of(ws(), [](const RecordEntry&) -> Result<std::optional<std::string>> { return std::optional<std::string>(std::string(64, 'b')); })
+              .find("l2 key for bucket") != std::string::npos);
+    auto drifted = ws();
+    drifted.tileiras_fingerprint = "release 13.4, V13.4.1";
+    bool called = false;
+    auto [rec2, warn2] = Record::load_verified(path, drifted, [&](const RecordEntry&) -> Result<std::optional<std::string>> {
+      called = true;
+      return std::optional<std::string>(std::string(64, 'b'));
+    }).unwrap();
+    CHECK(!called && warn2.size() == 1 && warn2[0].find("different tileiras") != std::string::npos && warn2[0].find("skipped") != std::string::npos);
+  }
+  {
+    CHECK(Record(ws()).save(path).is_ok());
+    auto other = ws(); other.source_hash = "different";
+    CHECK(err_of(other, decline).find("source_hash mismatch") != std::string::npos && err_of(other, decline).find("re-tune") != std::string::npos);
+    other = ws(); other.arch = "sm_100";
+    CHECK(err_of(other, decline).find("arch mismatch") != std::string::npos);
+    other = ws(); other.kernel = "other_kernel";
+    CHECK(err_of(other, decline).find("kernel mismatch") != std::string::npos);
+    // a record without space_hash where the workspace has one: a warning
+    auto expecting = ws(); expecting.space_hash = tune::space_hash({bn_splits(64, 8)});
+    auto [r3, w3] = Record::load_verified(path, expecting, decline).unwrap();
+    CHECK(w3.size() == 1 && w3[0].find("no space_hash") != std::string::npos);
+  }
+  {
+    auto with_space = ws(); with_space.space_hash = tune::space_hash({bn_splits(64, 8), bn_splits(128, 8)});
+    CHECK(Record(with_space).save(path).is_ok());
+    auto other = ws(); other.space_hash = tune::space_hash({bn_splits(64, 8)});
+    CHECK(err_of(other, decline).find("space_hash mismatch") != std::string::npos);
+    CHECK(Record::load_verified(path, ws(), decline).is_ok());       // loader without an expectation: accepted
+    Record dup(ws());
+    for (int i = 0; i < 2; ++i) dup.entries.push_back({"b", bn_splits(64, 8), 1.0f, 3, std::nullopt});
+    CHECK(dup.save(path).is_ok());
+    CHECK(err_of(ws(), decline).find("duplicate entries for bucket") != std::string::npos);
+  }
+  {
+    Record a(ws());
+    for (auto [bn, ms] : {std::make_pair(64, 2.0f), std::make_pair(128, 1.0f)}) a.insert({"b", bn_splits(bn, 4), ms, 3, std::nullopt});
+    CHECK(a.entries.size() == 1 && *a.get("b")->config.integer("BN") == 128);     // one winner per bucket
+    Record s(ws());
+    s.schema = tune::kRecordSchema + 1;
+    CHECK(s.save(path).is_ok());
+    CHECK(err_of(ws(), decline).find("schema mismatch") != std::string::npos);
+    Record edited(ws());
+    auto config = bn_splits(64, 8);
+    config.id = "BN=128,SPLITS=8";                                              // hand-edited: id and params disagree
+    edited.insert({"b", config, 1.0f, 3, std::nullopt});
+    CHECK(edited.save(path).is_ok());
+    CHECK(err_of(ws(), decline).find("config id for bucket") != std::string::npos);
+    Record old(ws());
+    old.cutile_version = "0.0.0-elsewhere";
+    CHECK(old.save(path).is_ok());
+    auto [r5, w5] = Record::load_verified(path, ws(), decline).unwrap();
+    CHECK(w5.size() == 1 && w5[0].find("produced by cutile 0.0.0-elsewhere") != std::string::npos);
+  }
+  // this build's provenance: fingerprints come from the kernel table
+  auto live = tune::Workspace::of_kernel("gemm").unwrap();
+  CHECK(live.arch == "gfx950" && live.source_hash.size() == 16 && !live.tileiras_fingerprint.empty());
+  auto k1 = tune::variant_key("gemm", "bf16_256x256x64_d4x2").unwrap(), k2 = tune::variant_key("gemm", "bf16_256x256x64_d2x4").unwrap();
+  CHECK(k1 && k2 && *k1 != *k2 && *k1 != live.source_hash);
+  CHECK(tune::variant_key("gemm", "no_such_variant").is_err() && tune::Workspace::of_kernel("no_such_kernel").is_err());
+  CHECK(tune::Workspace::of_kernel("rms_norm_f16").unwrap().source_hash != live.source_hash);   // another code object
+  remove(path.c_str());
+}
+
+TEST(autotuner_end_to_end_on_the_recording_runtime) {
+  using tune::Config;
+  auto a = Config::make({{"bm", 128}, {"bn", 128}}), b = Config::make({{"bm", 256}, {"bn", 256}}), c = Config::make({{"bm", 64}, {"bn", 64}});
+  // candidates that fail to set up are recorded as invalid; the log makes the second run resume
   auto s = fresh_stream();
   bench::BenchOptions bo;
   bo.warmup = std::chrono::milliseconds(0);
@@ -483,22 +663,29 @@ TEST(autotuner_search_semantics) {
   bo.min_reps = 2;
   bo.max_reps = 2;
   bo.clear_l2 = false;
-  std::string log = "/tmp/cutile_tune_test.jsonl";
+  std::string log = "/tmp/cutile_tune_test_" + std::to_string(getpid()) + ".jsonl";
   remove(log.c_str());
+  int setups = 0;
   auto run = [&] {
     return tune::Autotuner("unit").configs({a, b, c}).bench_options(bo).log(log)
         .prune([](const Config& cfg) { return *cfg.integer("bm") >= 128; })
         .run(s, [&](const std::shared_ptr<Stream>&, const Config& cfg) -> Result<bench::BenchFn> {
+          ++setups;
           if (*cfg.integer("bm") == 256) return DeviceError::launch("tile too large");
           return bench::BenchFn([](const std::shared_ptr<Stream>&) { return ok(); });
         }).unwrap();
   };
   auto out = run();
-  CHECK(out.best && out.best->id == a.id && out.trials.size() == 2);
-  auto out2 = run();  // resumed from the log: the measured candidate is not measured again
-  CHECK(out2.best->id == a.id);
+  CHECK(out.best && out.best->id == a.id && out.trials.size() == 2 && setups == 2);   // one measurable candidate: no runoff
+  auto out2 = run();  // resumed from the log: the measured candidate is not measured again, the invalid one is retried
+  CHECK(out2.best->id == a.id && setups == 3);
+  // the same log under another candidate set is refused, not overwritten
+  auto foreign = tune::Autotuner("unit").configs({a}).bench_options(bo).log(log)
+                     .run(s, [&](const std::shared_ptr<Stream>&, const Config&) -> Result<bench::BenchFn> { return DeviceError::launch("unused"); });
+  CHECK(foreign.is_err() && foreign.error().message.find("belongs to tuner") != std::string::npos);
+  remove(log.c_str());
   auto variants = tune::variant_configs("gemm", "256x256");
-  CHECK(variants.size() >= 3);
+  CHECK(variants.size() >= 3 && variants[0].id.rfind("variant=\"", 0) == 0);
 }
 
 int main(int argc, char** argv) {
