@@ -299,6 +299,43 @@ class MxGemm(Workload):
                {"rel_l2_sampled_rows": rel, "tolerance": 3e-2, "ok": rel <= 3e-2}
 
 
+class Nvfp4Gemm(Workload):
+    name, unit, bound, peak_key = "nvfp4_gemm_8192", "TFLOP/s", "mfma", "mfma_bf16"
+    dtype = "fp4 e2m1 x e4m3 scale per 16 K, expanded exactly to f16 / f32 acc / f32 out"
+    s = 8192
+    work = 2.0 * s ** 3
+    tile = 256
+    config = {"workload": "NVFP4 block-scaled GEMM A[8192,8192] B[8192,8192] packed e2m1 + e4m3fn scale per 16 K, f32 out; "
+                          "matrix work runs on the f16 pipe (peak 2.5 PFLOP/s): CDNA4's fp4 pipe cannot take e4m3 scales per 16",
+              "tile": "256x256x64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        s = self.s
+        self.ct = ct
+        self.xq, self.xs = oracle.nvfp4_quantize(oracle.normal_f32((s, s), 14))
+        self.yq, self.ys = oracle.nvfp4_quantize(oracle.normal_f32((s, s), 15))
+        td = lambda t: torch.from_numpy(t).to(dev)
+        self.x, self.y, self.xsd, self.ysd = td(self.xq), td(self.yq), td(self.xs), td(self.ys)
+        self.z = torch.zeros(s, s, dtype=torch.float32, device=dev)
+        self.zp = ct.partition(self.z, [self.tile, self.tile])
+
+    def launch(self):
+        self.ct.linear_tile_nvfp4(self.zp, self.x, self.y, self.xsd, self.ysd, 1.0)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rng = np.random.default_rng(16)
+        rows = np.sort(rng.choice(self.s, size=128, replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        ref = oracle.nvfp4_gemm_f32(self.xq, self.yq, self.xs, self.ys, 1.0, rows=rows)
+        dt = time.perf_counter() - t0
+        got = self.z[torch.from_numpy(rows).to(self.z.device)].cpu().numpy()
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        flops = 2.0 * len(rows) * self.s * self.s
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"{len(rows)} of {self.s} output rows, f32 dequantised reference (includes dequantising B once)"}, \
+               {"rel_l2_sampled_rows": rel, "tolerance": 1e-5, "ok": rel <= 1e-5}
+
+
 def _td_f16(torch, np, bits, dev):
     return torch.from_numpy(np.ascontiguousarray(bits).view(np.float16)).to(dev)
 
@@ -502,7 +539,7 @@ class DecodeAttention(Workload):
 
 
 def make_workloads():
-    return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(),
+    return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
             AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention()]
 
 

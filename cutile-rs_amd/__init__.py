@@ -23,8 +23,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libcutile_hip.so")
 MAX_RANK = 4
 
 # cutile_dtype_t
-(F32, F64, F16, BF16, I8, I16, I32, I64, U8, U16, U32, U64, BOOL, F8E4M3FN, F8E5M2, F8E8M0FNU,
- DTYPE_COUNT) = range(17)
+(F32, F64, F16, BF16, I8, I16, I32, I64, U8, U16, U32, U64, BOOL, F8E4M3FN, F8E5M2, F8E8M0FNU, F4E2M1FNX2,
+ DTYPE_COUNT) = range(18)
 
 
 class CutileError(RuntimeError):
@@ -129,6 +129,8 @@ def lib() -> C.CDLL:
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
             "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
+                                                P(TensorArg), f32, P(LaunchOpts)],
+            "cutile_launch_linear_tile_nvfp4": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
                                                 P(TensorArg), f32, P(LaunchOpts)],
             "cutile_partition_grid": [P(PartitionArg), P(C.c_uint32 * 3)],
             "cutile_mapped_partition_grid": [P(MappedPartitionArg), P(C.c_uint32 * 3)],
@@ -478,6 +480,17 @@ def linear_tile_mxfp8(z: Partition, x, y, x_scales, y_scales, alpha: float = 1.0
     xa, ya = tensor_arg(x, F8E4M3FN), tensor_arg(y, F8E4M3FN)
     xsa, ysa = tensor_arg(x_scales, F8E8M0FNU), tensor_arg(y_scales, F8E8M0FNU)
     check(lib().cutile_launch_linear_tile_mxfp8(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya),
+                                                C.byref(xsa), C.byref(ysa), float(alpha), C.byref(o)))
+
+
+def linear_tile_nvfp4(z: Partition, x, y, x_scales, y_scales, alpha: float = 1.0, *, stream=None, grid=None,
+                      generics=None, variant=None) -> None:
+    """cutile-examples/examples/nvfp4.rs:24-78.  x [M, K/2], y [N, K/2]: uint8 tensors of packed e2m1 pairs (low
+    nibble first); scales [M, K/16], [N, K/16]: uint8 (or float8_e4m3fn) tensors of e4m3fn bytes; z f32 or bf16."""
+    o, _k = _opts(grid, generics, variant)
+    xa, ya = tensor_arg(x, F4E2M1FNX2), tensor_arg(y, F4E2M1FNX2)
+    xsa, ysa = tensor_arg(x_scales, F8E4M3FN), tensor_arg(y_scales, F8E4M3FN)
+    check(lib().cutile_launch_linear_tile_nvfp4(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya),
                                                 C.byref(xsa), C.byref(ysa), float(alpha), C.byref(o)))
 
 

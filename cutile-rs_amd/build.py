@@ -31,6 +31,7 @@ IMAGES = {
     "gemm": "gemm_bf16.hip",
     "fmha": "fmha.hip",
     "mxgemm": "mxfp8_gemm.hip",
+    "nvfp4": "nvfp4_gemm.hip",
 }
 HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp"]
 

@@ -15,6 +15,7 @@ extern const unsigned char cutile_img_rowwise_start[], cutile_img_rowwise_end[];
 extern const unsigned char cutile_img_gemm_start[], cutile_img_gemm_end[];
 extern const unsigned char cutile_img_fmha_start[], cutile_img_fmha_end[];
 extern const unsigned char cutile_img_mxgemm_start[], cutile_img_mxgemm_end[];
+extern const unsigned char cutile_img_nvfp4_start[], cutile_img_nvfp4_end[];
 }
 
 namespace cutile {
@@ -35,6 +36,7 @@ ImageRef image_ref(Image img) {
     case IMG_GEMM: return {cutile_img_gemm_start, cutile_img_gemm_end};
     case IMG_FMHA: return {cutile_img_fmha_start, cutile_img_fmha_end};
     case IMG_MXGEMM: return {cutile_img_mxgemm_start, cutile_img_mxgemm_end};
+    case IMG_NVFP4: return {cutile_img_nvfp4_start, cutile_img_nvfp4_end};
     default: return {nullptr, nullptr};
   }
 }
@@ -148,6 +150,16 @@ std::vector<KernelEntry> build_table() {
   for (const char* dt : {"bf16", "bf16f32", "f16", "f32"})
     add("gemm", keep(std::string(dt) + "_generic"), keep(std::string("gemm_entry__") + dt + "_generic"), IMG_GEMM, 256,
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
+
+  // ---- NVFP4 GEMM: operands expanded to f16 on the way into LDS; LDS = 2 stages x (BM + BN) rows of 128 bytes ----
+  for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2},
+                 std::array<int, 4>{64, 64, 1, 1}, std::array<int, 4>{32, 32, 1, 1}})
+    for (const char* dt : {"f32", "bf16"}) {
+      if (dt[0] == 'b' && t[0] < 128) continue;
+      std::string v = std::string(dt) + "_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_w" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
+      add("linear_tile_nvfp4", keep(v), keep("linear_tile_nvfp4_entry__" + v), IMG_NVFP4, (uint32_t)(t[2] * t[3] * 64),
+          (uint32_t)(2 * (t[0] + t[1]) * 128), t[0], t[1], 64, 0, dt, 0, 2);
+    }
 
   // ---- persistent GEMM over a mapped partition: the pipelined bodies in a stream-item loop ----
   for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2}}) {

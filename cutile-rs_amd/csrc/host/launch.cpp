@@ -56,7 +56,8 @@ struct DTypeInfo {
 };
 const DTypeInfo kDTypes[CUTILE_DTYPE_COUNT] = {
     {"f32", 4}, {"f64", 8}, {"f16", 2}, {"bf16", 2}, {"i8", 1},  {"i16", 2},      {"i32", 4},    {"i64", 8},
-    {"u8", 1},  {"u16", 2}, {"u32", 4}, {"u64", 8},  {"bool", 1}, {"f8e4m3fn", 1}, {"f8e5m2", 1}, {"f8e8m0fnu", 1}};
+    {"u8", 1},  {"u16", 2}, {"u32", 4}, {"u64", 8},  {"bool", 1}, {"f8e4m3fn", 1}, {"f8e5m2", 1}, {"f8e8m0fnu", 1},
+    {"f4e2m1fnx2", 1}};
 
 uint16_t f32_to_f16_bits(float f) {
   uint32_t x;
@@ -1348,6 +1349,88 @@ cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cu
                  bk_user / 32, dt.c_str(), list_variants("linear_tile").c_str());
   Resolved res;
   if (cutile_status_t s = resolve_entry("linear_tile", opts, acceptable[0], acceptable, &res)) return s;
+  uint32_t kg[3] = {tg[0], tg[1], 1};
+  if (res.entry->tile[0] != bm || res.entry->tile[1] != bn) {
+    kg[0] = div_up(M, res.entry->tile[0]);
+    kg[1] = div_up(N, res.entry->tile[1]);
+  }
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_tensor(*x);
+  args.push_tensor(*y);
+  args.push_tensor(*xs);
+  args.push_tensor(*ys);
+  args.push_val<float>(alpha);
+  args.push_tile_grid(kg);
+  uint32_t grid[3] = {kg[0] * kg[1], 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_linear_tile_nvfp4(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                                const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                                const cutile_tensor_arg_t* xs, const cutile_tensor_arg_t* ys, float alpha,
+                                                const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(z, "z", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(y, "y", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(xs, "x_scales", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(ys, "y_scales", 2, 2)) return s;
+  const cutile_tensor_arg_t& zt = z->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F4E2M1FNX2 && y->dtype == CUTILE_DTYPE_F4E2M1FNX2 &&
+                     xs->dtype == CUTILE_DTYPE_F8E4M3FN && ys->dtype == CUTILE_DTYPE_F8E4M3FN,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "linear_tile (nvfp4): precompiled variants take f4e2m1fnx2 data with f8e4m3fn scales");
+  CUTILE_REQUIRE(zt.dtype == CUTILE_DTYPE_F32 || zt.dtype == CUTILE_DTYPE_BF16, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile (nvfp4): z must be f32 or bf16");
+  const int32_t M = x->shape[0], KP = x->shape[1], N = y->shape[0];
+  const int64_t K = 2 * (int64_t)KP;
+  CUTILE_REQUIRE(y->shape[1] == KP, CUTILE_ERR_KERNEL_LAUNCH, "linear_tile (nvfp4): x is [%d, %d] but y is [%d, %d] (packed bytes)", M,
+                 KP, N, y->shape[1]);
+  CUTILE_REQUIRE(K % 16 == 0 && xs->shape[0] == M && xs->shape[1] == K / 16 && ys->shape[0] == N && ys->shape[1] == K / 16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "linear_tile (nvfp4): scales must be [M, K/16] and [N, K/16] with K = %lld a multiple of 16",
+                 (long long)K);
+  CUTILE_REQUIRE(zt.shape[0] == M && zt.shape[1] == N, CUTILE_ERR_KERNEL_LAUNCH,
+                 "linear_tile (nvfp4): z is [%d, %d], expected [%d, %d]", zt.shape[0], zt.shape[1], M, N);
+  const int32_t bm = z->partition_shape[0], bn = z->partition_shape[1];
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bn), "BN")) return s;
+  const int bk_user = generic_int(opts, 2, 64);
+  CUTILE_REQUIRE(bk_user > 0 && bk_user % 16 == 0 && generic_int(opts, 3, bk_user / 2) == bk_user / 2 &&
+                     generic_int(opts, 4, bk_user / 16) == bk_user / 16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "linear_tile (nvfp4): BK must be a multiple of 16, BK_PACKED = BK/2 and BK_SCALES = BK/16");
+  // the tile program runs K / BK whole K tiles
+  CUTILE_REQUIRE(K % bk_user == 0, CUTILE_ERR_KERNEL_LAUNCH, "linear_tile (nvfp4): K = %lld is not a multiple of BK = %d", (long long)K,
+                 bk_user);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(z, opts, tg)) return s;
+  uint32_t full[3];
+  cutile_partition_grid(z, full);
+  const bool full_cover = tg[0] == full[0] && tg[1] == full[1];
+  CUTILE_REQUIRE(K % 64 == 0 && x->strides[1] == 1 && y->strides[1] == 1 && xs->strides[1] == 1 && ys->strides[1] == 1 &&
+                     zt.strides[1] == 1 && x->strides[0] % 16 == 0 && y->strides[0] % 16 == 0 && xs->strides[0] % 2 == 0 &&
+                     ys->strides[0] % 2 == 0 && zt.strides[0] % 4 == 0 && zt.shape[1] % 4 == 0 && aligned16(x->ptr) &&
+                     aligned16(y->ptr) && aligned16(zt.ptr) && ((uintptr_t)xs->ptr & 1) == 0 && ((uintptr_t)ys->ptr & 1) == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile (nvfp4): precompiled variants need K a multiple of 64, unit inner strides and aligned rows");
+  const std::string dt = zt.dtype == CUTILE_DTYPE_F32 ? "f32" : "bf16";
+  // A kernel tile that is a whole multiple of the partition tile computes the same output when the
+  // launch covers the whole tensor (the reference example's 16x16 tiles run on the 32x32 kernel).
+  std::vector<const KernelEntry*> fit;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, "linear_tile_nvfp4") == 0 && dt == e.dtype &&
+        ((e.tile[0] == bm && e.tile[1] == bn) || (full_cover && e.tile[0] % bm == 0 && e.tile[1] % bn == 0)))
+      fit.push_back(&e);
+  std::stable_sort(fit.begin(), fit.end(), [&](const KernelEntry* a, const KernelEntry* b) {
+    bool ea = a->tile[0] == bm && a->tile[1] == bn, eb = b->tile[0] == bm && b->tile[1] == bn;
+    if (ea != eb) return ea;
+    return a->tile[0] * a->tile[1] < b->tile[0] * b->tile[1];
+  });
+  std::vector<std::string> acceptable;
+  for (auto* e : fit) acceptable.push_back(e->variant);
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of nvfp4 linear_tile<%d, %d, %d, %d, %d> -> %s; available: %s", bm, bn, bk_user, bk_user / 2,
+                 bk_user / 16, dt.c_str(), list_variants("linear_tile_nvfp4").c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("linear_tile_nvfp4", opts, acceptable[0], acceptable, &res)) return s;
   uint32_t kg[3] = {tg[0], tg[1], 1};
   if (res.entry->tile[0] != bm || res.entry->tile[1] != bn) {
     kg[0] = div_up(M, res.entry->tile[0]);

@@ -248,6 +248,7 @@ typedef enum {
   CUTILE_DTYPE_I8, CUTILE_DTYPE_I16, CUTILE_DTYPE_I32, CUTILE_DTYPE_I64,
   CUTILE_DTYPE_U8, CUTILE_DTYPE_U16, CUTILE_DTYPE_U32, CUTILE_DTYPE_U64,
   CUTILE_DTYPE_BOOL, CUTILE_DTYPE_F8E4M3FN, CUTILE_DTYPE_F8E5M2, CUTILE_DTYPE_F8E8M0FNU,
+  CUTILE_DTYPE_F4E2M1FNX2,          /* one byte = two e2m1 values, low nibble first (cuda-core/src/dtype.rs:60-99) */
   CUTILE_DTYPE_COUNT
 } cutile_dtype_t;
 const char* cutile_dtype_name(cutile_dtype_t dtype);
@@ -442,6 +443,13 @@ cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cu
                                                 const cutile_tensor_arg_t* x_scales,
                                                 const cutile_tensor_arg_t* y_scales, float alpha,
                                                 const cutile_launch_opts_t* opts);
+/* NVFP4 linear_tile<BM, BN, BK, BK_PACKED, BK_SCALES>(z: [BM,BN] tiles, x, y, x_scales, y_scales, alpha):
+ * z = alpha * (x . sx) @ (y . sy)^T with x [M, K/2], y [N, K/2] packed e2m1 pairs, scales [M, K/16], [N, K/16]
+ * e4m3fn, one per 16 K values; z f32 (as the reference) or bf16 — cutile-examples/examples/nvfp4.rs:24-78 */
+cutile_status_t cutile_launch_linear_tile_nvfp4(cutile_stream_t stream, const cutile_partition_arg_t* z,
+                                                const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
+                                                const cutile_tensor_arg_t* x_scales, const cutile_tensor_arg_t* y_scales,
+                                                float alpha, const cutile_launch_opts_t* opts);
 
 /* ======================================================================== */
 /* Part E — asynchronous runtime                                             */

@@ -20,8 +20,14 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 def build(force: bool = False) -> str:
     """Compile liboracle.so with gcc (seconds)."""
-    if force or not os.path.exists(_LIB_PATH):
-        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    sources = [os.path.join(_HERE, f) for f in ("oracle.c", "oracle.h", "Makefile")]
+    stale = os.path.exists(_LIB_PATH) and any(os.path.getmtime(f) > os.path.getmtime(_LIB_PATH) for f in sources if os.path.exists(f))
+    if force or stale or not os.path.exists(_LIB_PATH):
+        try:
+            subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+        except (OSError, subprocess.CalledProcessError):
+            if force or not os.path.exists(_LIB_PATH):
+                raise          # nothing usable; a merely stale library is still loaded
     return _LIB_PATH
 
 
@@ -71,6 +77,11 @@ def lib() -> C.CDLL:
             "orc_mx_quantize_e4m3": (None, [vp, vp, vp, i64, i64]),
             "orc_mx_dequantize_e4m3": (None, [vp, vp, vp, i64, i64]),
             "orc_mx_gemm_f32": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, vp, i64]),
+            "orc_e2m1_to_f32": (f32, [C.c_uint8]),
+            "orc_f32_to_e2m1": (C.c_uint8, [f32]),
+            "orc_nvfp4_quantize": (None, [vp, vp, vp, i64, i64]),
+            "orc_nvfp4_dequantize": (None, [vp, vp, vp, i64, i64]),
+            "orc_nvfp4_gemm_f32": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, vp, i64]),
         }
         for name, (res, args) in sigs.items():
             fn = getattr(L, name)
@@ -387,4 +398,43 @@ def mx_gemm_f32(x, y, xs, ys, alpha: float = 1.0, rows=None) -> np.ndarray:
     keep, rp, nr = _rows_arg(rows)
     z = np.empty((nr if rows is not None else m, n), np.float32)
     lib().orc_mx_gemm_f32(_p(x), _p(y), _p(xs), _p(ys), _p(z), m, n, k, alpha, rp, nr)
+    return z
+
+
+# ---- NVFP4 ----------------------------------------------------------------------------------
+def e2m1_to_f32(nibble: int) -> float:
+    return float(lib().orc_e2m1_to_f32(nibble))
+
+
+def f32_to_e2m1(v: float) -> int:
+    return int(lib().orc_f32_to_e2m1(v))
+
+
+def nvfp4_quantize(src):
+    """-> (packed e2m1 pairs [rows, k/2] uint8, e4m3fn scales [rows, k/16] uint8)"""
+    src = _c(src, np.float32)
+    rows, k = src.shape
+    assert k % 16 == 0
+    data = np.empty((rows, k // 2), np.uint8)
+    scales = np.empty((rows, k // 16), np.uint8)
+    lib().orc_nvfp4_quantize(_p(src), _p(data), _p(scales), rows, k)
+    return data, scales
+
+
+def nvfp4_dequantize(data, scales) -> np.ndarray:
+    data, scales = _c(data, np.uint8), _c(scales, np.uint8)
+    rows, kp = data.shape
+    dst = np.empty((rows, kp * 2), np.float32)
+    lib().orc_nvfp4_dequantize(_p(data), _p(scales), _p(dst), rows, kp * 2)
+    return dst
+
+
+def nvfp4_gemm_f32(x, y, xs, ys, alpha: float = 1.0, rows=None) -> np.ndarray:
+    x, y, xs, ys = _c(x, np.uint8), _c(y, np.uint8), _c(xs, np.uint8), _c(ys, np.uint8)
+    m, kp = x.shape
+    n, kp2 = y.shape
+    assert kp == kp2
+    keep, rp, nr = _rows_arg(rows)
+    z = np.empty((nr if rows is not None else m, n), np.float32)
+    lib().orc_nvfp4_gemm_f32(_p(x), _p(y), _p(xs), _p(ys), _p(z), m, n, kp * 2, alpha, rp, nr)
     return z

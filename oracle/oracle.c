@@ -664,3 +664,90 @@ void orc_mx_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, cons
     free(xrow);
   }
 }
+
+/* ------------------------------------------------------------------------ */
+/* NVFP4 block-scaled GEMM (cutile-examples/examples/nvfp4.rs:24-78)         */
+/* ------------------------------------------------------------------------ */
+/* e2m1: sign, two exponent bits (bias 1), one mantissa bit; no inf, no NaN.
+ * Magnitudes 0, 0.5, 1, 1.5, 2, 3, 4, 6 (OCP MX v1.0 table 5; dtype.rs:225-229 uses
+ * nibble 0x2 as one()). */
+float orc_e2m1_to_f32(uint8_t nibble) {
+  int e = (nibble >> 1) & 3, m = nibble & 1;
+  float v = e == 0 ? 0.5f * (float)m : ldexpf(1.0f + 0.5f * (float)m, e - 1);
+  return (nibble & 8) ? -v : v;
+}
+
+/* round to nearest representable magnitude, ties to the even mantissa, saturating at 6 */
+uint8_t orc_f32_to_e2m1(float f) {
+  uint8_t sign = signbit(f) ? 8 : 0;
+  float a = fabsf(f);
+  if (!(a == a)) return (uint8_t)(sign | 7); /* NaN has no encoding: saturate */
+  uint8_t best = 0;
+  float best_d = INFINITY;
+  for (uint8_t c = 0; c < 8; c++) {
+    float d = fabsf(a - orc_e2m1_to_f32(c));
+    if (d < best_d || (d == best_d && (c & 1) == 0)) {
+      best = c;
+      best_d = d;
+    }
+  }
+  return (uint8_t)(sign | best);
+}
+
+/* Quantise src[rows, k] (f32), one e4m3fn scale per 16 contiguous K values: scale =
+ * e4m3(amax / 6) (the largest magnitude maps to the largest e2m1 value), data = e2m1(src /
+ * scale), packed two per byte with the even element in the low nibble.  Not in the
+ * reference (its example fills ones): used to build test operands. */
+void orc_nvfp4_quantize(const float* src, uint8_t* data, uint8_t* scales, int64_t rows, int64_t k) {
+  int64_t kb = k / 16;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; r++)
+    for (int64_t blk = 0; blk < kb; blk++) {
+      const float* s = src + r * k + blk * 16;
+      float amax = 0.0f;
+      for (int j = 0; j < 16; j++) amax = fmaxf(amax, fabsf(s[j]));
+      uint8_t sc = orc_f32_to_e4m3fn(amax / 6.0f);
+      float sf = orc_e4m3fn_to_f32(sc);
+      scales[r * kb + blk] = sc;
+      for (int j = 0; j < 16; j += 2) {
+        uint8_t lo = sf > 0.0f ? orc_f32_to_e2m1(s[j] / sf) : 0, hi = sf > 0.0f ? orc_f32_to_e2m1(s[j + 1] / sf) : 0;
+        data[r * (k / 2) + blk * 8 + j / 2] = (uint8_t)(lo | (hi << 4));
+      }
+    }
+}
+
+void orc_nvfp4_dequantize(const uint8_t* data, const uint8_t* scales, float* dst, int64_t rows, int64_t k) {
+  int64_t kb = k / 16;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; r++)
+    for (int64_t j = 0; j < k; j++) {
+      uint8_t byte = data[r * (k / 2) + j / 2];
+      dst[r * k + j] = orc_e2m1_to_f32((j & 1) ? (uint8_t)(byte >> 4) : (uint8_t)(byte & 15)) * orc_e4m3fn_to_f32(scales[r * kb + j / 16]);
+    }
+}
+
+/* z[m,n] = alpha * sum_k (x[i,k] sx[i,k/16]) * (y[j,k] sy[j,k/16]); x [m,k/2], y [n,k/2] packed,
+ * f32 accumulate in k order.  Row subset as for orc_gemm_bf16. */
+void orc_nvfp4_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys, float* z, int64_t m,
+                        int64_t n, int64_t k, float alpha, const int64_t* rows, int64_t n_rows) {
+  int64_t count = rows ? n_rows : m;
+  float* yd = (float*)malloc(sizeof(float) * (size_t)n * (size_t)k);
+  orc_nvfp4_dequantize(y, ys, yd, n, k);
+#pragma omp parallel
+  {
+    float* xrow = (float*)malloc(sizeof(float) * (size_t)k);
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t ri = 0; ri < count; ri++) {
+      int64_t row = rows ? rows[ri] : ri;
+      orc_nvfp4_dequantize(x + row * (k / 2), xs + row * (k / 16), xrow, 1, k);
+      for (int64_t col = 0; col < n; col++) {
+        const float* yr = yd + col * k;
+        float acc = 0.0f;
+        for (int64_t j = 0; j < k; j++) acc += xrow[j] * yr[j];
+        z[ri * n + col] = alpha * acc;
+      }
+    }
+    free(xrow);
+  }
+  free(yd);
+}

@@ -42,6 +42,12 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_nvfp4_*          cutile-examples/examples/nvfp4.rs:24-78 (layout, formula),
+ *                        cuda-core/src/dtype.rs:60-99 (low nibble first), :228 (0x2 = 1.0).
+ *                        Pinned by the reference's all-ones known answer (z = K), the
+ *                        e2m1 value table, torch.float8_e4m3fn scales and a float64
+ *                        evaluation of the dequantised product.  The quantiser is not in
+ *                        the reference: parity unpinned.
  */
 #ifndef CUTILE_ORACLE_H
 #define CUTILE_ORACLE_H
@@ -155,6 +161,15 @@ void orc_mx_dequantize_e4m3(const uint8_t* data, const uint8_t* scales, float* d
 void orc_mx_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys,
                      float* z, int64_t m, int64_t n, int64_t k, float alpha, const int64_t* rows,
                      int64_t n_rows);
+
+/* ---- NVFP4 block-scaled GEMM (cutile-examples/examples/nvfp4.rs:24-78) -------------------- */
+float orc_e2m1_to_f32(uint8_t nibble);   /* magnitudes 0, 0.5, 1, 1.5, 2, 3, 4, 6; bit 3 = sign */
+uint8_t orc_f32_to_e2m1(float f);        /* nearest, ties to even mantissa, saturating */
+/* scale per 16 K values = e4m3fn(amax / 6); data packed two per byte, even element in the low nibble */
+void orc_nvfp4_quantize(const float* src, uint8_t* data, uint8_t* scales, int64_t rows, int64_t k);
+void orc_nvfp4_dequantize(const uint8_t* data, const uint8_t* scales, float* dst, int64_t rows, int64_t k);
+void orc_nvfp4_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys, float* z, int64_t m,
+                        int64_t n, int64_t k, float alpha, const int64_t* rows, int64_t n_rows);
 
 #ifdef __cplusplus
 }
