@@ -380,6 +380,8 @@ struct LinearTileMxfp8Fn {
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, XS& xs, YS& ys, float alpha) {
     auto zp = z.arg();
     auto xa = input_arg(x), ya = input_arg(y), xsa = input_arg(xs), ysa = input_arg(ys);
+    // the reference has one `linear_tile` per module (mxfp8.rs, nvfp4.rs); here the operand type picks the kernel
+    if (xa.dtype == CUTILE_DTYPE_F4E2M1FNX2) return cutile_launch_linear_tile_nvfp4(s, &zp, &xa, &ya, &xsa, &ysa, alpha, o);
     return cutile_launch_linear_tile_mxfp8(s, &zp, &xa, &ya, &xsa, &ysa, alpha, o);
   }
 };
@@ -499,7 +501,7 @@ template <class Z, class X, class Y> auto gemm_zero_init(Z&& z, X&& x, Y&& y, in
 // fmha(out: partition [1,BM,D], q, k, v, qk_scale, input_pos, query_group_size)   flash_attention_causal.rs:32-40
 template <class O, class Q, class K, class V> auto fmha(O&& out, Q&& q, K&& k, V&& v, float scale, int32_t input_pos, int32_t group) { return make_launcher<kernels::FmhaFn<false>>(std::forward<O>(out), std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), scale, input_pos, group); }
 template <class O, class Q, class K, class V> auto fmha_causal(O&& out, Q&& q, K&& k, V&& v, float scale, int32_t input_pos, int32_t group) { return make_launcher<kernels::FmhaFn<true>>(std::forward<O>(out), std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), scale, input_pos, group); }
-// linear_tile(z: partition [BM,BN], x, y, x_scales, y_scales, alpha)   cutile-examples/examples/mxfp8.rs:35-42
+// linear_tile(z: partition [BM,BN], x, y, x_scales, y_scales, alpha)   cutile-examples/examples/mxfp8.rs:35-42 (f8e4m3fn x, y) and nvfp4.rs:39-51 (f4e2m1fnx2 x, y)
 template <class Z, class X, class Y, class XS, class YS> auto linear_tile(Z&& z, X&& x, Y&& y, XS&& xs, YS&& ys, float alpha) { return make_launcher<kernels::LinearTileMxfp8Fn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), std::forward<XS>(xs), std::forward<YS>(ys), alpha); }
 // add_rms_norm_f16(residual, x, w, out: [1,N], residual_out: [1,N], eps)      cutile-kernels/src/norms.rs:76-83
 template <class R, class X, class W, class O, class RO> auto add_rms_norm_f16(R&& residual, X&& x, W&& w, O&& out, RO&& residual_out, float eps) { return make_launcher<kernels::AddRmsNormF16Fn>(std::forward<R>(residual), std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), std::forward<RO>(residual_out), eps); }

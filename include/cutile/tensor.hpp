@@ -29,6 +29,14 @@ struct f16 { uint16_t bits; };
 struct bf16 { uint16_t bits; };
 struct f8e4m3fn { uint8_t bits; };
 struct f8e8m0fnu { uint8_t bits; };
+// Packed pair of e2m1 values in one byte: the low nibble is the first logical value (dtype.rs:60-99).
+struct f4e2m1fnx2 {
+  uint8_t bits;
+  static constexpr f4e2m1fnx2 from_bits(uint8_t b) { return {b}; }
+  static constexpr f4e2m1fnx2 from_nibbles(uint8_t low, uint8_t high) { return {(uint8_t)((low & 0x0F) | ((high & 0x0F) << 4))}; }
+  constexpr uint8_t low() const { return bits & 0x0F; }
+  constexpr uint8_t high() const { return bits >> 4; }
+};
 
 template <class T> struct DType;
 #define CUTILE_DTYPE(T, CODE) \
@@ -48,6 +56,7 @@ CUTILE_DTYPE(uint64_t, CUTILE_DTYPE_U64)
 CUTILE_DTYPE(bool, CUTILE_DTYPE_BOOL)
 CUTILE_DTYPE(f8e4m3fn, CUTILE_DTYPE_F8E4M3FN)
 CUTILE_DTYPE(f8e8m0fnu, CUTILE_DTYPE_F8E8M0FNU)
+CUTILE_DTYPE(f4e2m1fnx2, CUTILE_DTYPE_F4E2M1FNX2)
 #undef CUTILE_DTYPE
 // Host-side conversions of the 16-bit float storage types (round to nearest even).
 inline bf16 bf16_from_f32(float f) {
@@ -97,6 +106,7 @@ inline float f32_from_f16(f16 h) {
 // one(): the value tests fill operands with (dtype.rs:225-227)
 inline f8e4m3fn f8e4m3fn_one() { return {0x38}; }
 inline f8e8m0fnu f8e8m0fnu_one() { return {0x7F}; }
+inline f4e2m1fnx2 f4e2m1fnx2_one() { return f4e2m1fnx2::from_nibbles(0x2, 0x2); }   // dtype.rs:228
 
 // ---- device allocations (device_buffer.rs:40-226) --------------------------------------------
 // An allocation owned by another runtime, lent to a tensor (DeviceAllocation trait).

@@ -220,6 +220,26 @@ TEST(mxfp8_example_all_ones) {
   for (float v : host) CHECK(std::fabs(v - (float)K) <= 1e-3f);
 }
 
+TEST(nvfp4_example_all_ones) {
+  // cutile-examples/examples/nvfp4.rs:96-160: packed ones (nibble 0x2), scales 1.0 (0x38), 16x16x64 tiles -> z = K
+  auto stream = new_stream();
+  const int M = 16, N = 16, K = 128;
+  auto bytes = [&](uint8_t v, int n, std::vector<int32_t> shape) {
+    auto host = std::make_shared<std::vector<uint8_t>>(n, v);
+    return std::make_shared<Tensor<uint8_t>>(std::move(api::copy_host_vec_to_device(host).sync_on(stream).unwrap()).reshape(std::move(shape)).unwrap());
+  };
+  const uint8_t one = f4e2m1fnx2_one().bits;
+  CHECK(one == 0x22 && f4e2m1fnx2::from_nibbles(0x7, 0x1).low() == 0x7 && f4e2m1fnx2::from_nibbles(0x7, 0x1).high() == 0x1);
+  auto x = Tensor<uint8_t>::reinterpret<f4e2m1fnx2>(bytes(one, M * K / 2, {M, K / 2}), {M, K / 2}).unwrap();
+  auto y = Tensor<uint8_t>::reinterpret<f4e2m1fnx2>(bytes(one, N * K / 2, {N, K / 2}), {N, K / 2}).unwrap();
+  auto xs = Tensor<uint8_t>::reinterpret<f8e4m3fn>(bytes(0x38, M * K / 16, {M, K / 16}), {M, K / 16}).unwrap();
+  auto ys = Tensor<uint8_t>::reinterpret<f8e4m3fn>(bytes(0x38, N * K / 16, {N, K / 16}), {N, K / 16}).unwrap();
+  auto z = partition_op(api::zeros<float>({M, N}), {16, 16});
+  auto res = linear_tile(std::move(z), x, y, xs, ys, 1.0f).generics({"16", "16", "64", "32", "4"}).sync_on(stream).unwrap();
+  auto host = api::to_host_vec(std::move(std::get<0>(res)).unpartition()).sync_on(stream).unwrap();
+  for (float v : host) CHECK(v == (float)K);
+}
+
 TEST(graph_replay_matches_eager) {
   auto stream = new_stream();
   const int n = 1 << 16;
