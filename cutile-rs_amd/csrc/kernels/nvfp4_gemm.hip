@@ -118,13 +118,20 @@ struct Nvfp4Gemm {
         b_sc[i] = __builtin_amdgcn_raw_buffer_load_b16(rsb, b_soff[i], kt * 4, 0);
       }
     };
+    // LDS takes a 16-byte write from 8 lanes per cycle (128 bytes): lanes 0-7 are 4 rows x 2 halves, and rows
+    // 2j, 2j+1 share their swizzle term, so writing unit d of every row in step d would put both on the same
+    // banks.  Odd rows therefore walk their four units in the order 2, 3, 0, 1.
     auto expand_piece = [&](unsigned char* tile, int row, int half, const u32x4& q, uint32_t sc) {
+      const bool odd = row & 1;
       const _Float16 s0 = (_Float16)__builtin_amdgcn_cvt_f32_fp8((int)sc, 0);   // e4m3fn -> f32 -> f16: exact
       const _Float16 s1 = (_Float16)__builtin_amdgcn_cvt_f32_fp8((int)sc, 1);
-      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + 0)) = expand_fp4x8(q.x, s0);
-      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + 1)) = expand_fp4x8(q.y, s0);
-      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + 2)) = expand_fp4x8(q.z, s1);
-      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + 3)) = expand_fp4x8(q.w, s1);
+      const _Float16 sa = odd ? s1 : s0, sb = odd ? s0 : s1;
+      const uint32_t q0 = odd ? q.z : q.x, q1 = odd ? q.w : q.y, q2 = odd ? q.x : q.z, q3 = odd ? q.y : q.w;
+      const int flip = odd ? 2 : 0;
+      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + (0 ^ flip))) = expand_fp4x8(q0, sa);
+      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + (1 ^ flip))) = expand_fp4x8(q1, sa);
+      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + (2 ^ flip))) = expand_fp4x8(q2, sb);
+      *reinterpret_cast<u32x4*>(tile + lds_off(row, half * 4 + (3 ^ flip))) = expand_fp4x8(q3, sb);
     };
     auto store_lds = [&](int stage) {
       unsigned char* sa = lds + stage * kStageBytes;

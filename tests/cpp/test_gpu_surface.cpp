@@ -3,6 +3,7 @@
 // the known answers those examples assert (cutile-examples/examples/saxpy.rs:47-53,
 // softmax.rs:55-60, mxfp8.rs:129-135, cuda_graphs.rs:333-344,
 // cutile/tests/gpu/add_basic.rs:29-43, cutile/tests/slice_non_divisible.rs:459-500).
+#include <unistd.h>
 #include <cutile/cutile.hpp>
 
 #include <atomic>
@@ -342,6 +343,25 @@ TEST(do_bench_and_autotune_pick_a_variant) {
   CHECK(invalid >= 4);  // w1v1..w1v8 cannot hold the row
   std::string best = *tuned.best->str("variant");
   CHECK(best != "generic");
+  // the winner goes into a provenance-checked record and comes back verified (tune.rs:762-1016)
+  auto space = tune::space_hash(tune::variant_configs("rms_norm_f16"));
+  auto ws = tune::Workspace::of_kernel("rms_norm_f16", space).unwrap();
+  tune::Record record(ws);
+  float best_ms = INFINITY;
+  size_t best_reps = 0;
+  for (auto& t : tuned.trials)
+    if (t.measured && t.config_id == tuned.best->id && t.median_ms < best_ms) { best_ms = t.median_ms; best_reps = t.reps; }
+  record.insert({"n<=8192", *tuned.best, best_ms, best_reps, tune::variant_key("rms_norm_f16", best).unwrap()});
+  std::string record_path = "/tmp/cutile_rms_norm_record_" + std::to_string(getpid()) + ".json";
+  CHECK(record.save(record_path).is_ok());
+  auto [loaded, warnings] = tune::Record::load_verified(record_path, ws, [](const tune::RecordEntry& e) {
+    return tune::variant_key("rms_norm_f16", *e.config.str("variant"));
+  }).unwrap();
+  CHECK(warnings.empty() && *loaded.get("n<=8192")->config.str("variant") == best);
+  auto other = tune::Workspace::of_kernel("softmax", space).unwrap();       // another kernel's workspace refuses it
+  CHECK(tune::Record::load_verified(record_path, other, [](const tune::RecordEntry&) -> Result<std::optional<std::string>> { return std::optional<std::string>(); }).is_err());
+  remove(record_path.c_str());
+  best = *loaded.get("n<=8192")->config.str("variant");
   CHECK(cutile_kernel_set_preferred_variant("rms_norm_f16", best.c_str()) == CUTILE_SUCCESS);
   CHECK(rms_norm_f16(&x, &w, out.partition_mut({1, n}), 1e-6f).sync_on(stream).is_ok());
   CHECK(cutile_kernel_set_preferred_variant("rms_norm_f16", nullptr) == CUTILE_SUCCESS);
