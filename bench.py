@@ -5,7 +5,7 @@
 
 A step is one launch of the hot-path kernel over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the bf16 GEMM at M = N = K = 8192
-(the configuration the target fractions are quoted on); every other BASELINE
+(the configuration the target fractions are quoted on); every other benchmark
 configuration is measured the same way and reported under "also" in the same JSON line.
 
 Timing: W untimed launches, then exactly K launches between two device synchronisations
