@@ -152,7 +152,7 @@ std::vector<KernelEntry> build_table() {
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
   // ---- NVFP4 GEMM: operands expanded to f16 on the way into LDS; LDS = 2 stages x (BM + BN) rows of 128 bytes ----
-  for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2},
+  for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2},
                  std::array<int, 4>{64, 64, 1, 1}, std::array<int, 4>{32, 32, 1, 1}})
     for (const char* dt : {"f32", "bf16"}) {
       if (dt[0] == 'b' && t[0] < 128) continue;

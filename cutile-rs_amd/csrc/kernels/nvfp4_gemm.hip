@@ -22,6 +22,10 @@
 // scale) and written to the other stage as four 16-byte units.  Rows are 128 bytes of f16
 // with 16-byte unit u stored at unit u ^ ((row >> 1) & 7), so the operand reads of 32 rows
 // fall on distinct banks.
+//
+// A fully dealt-out schedule (fragments read one K step ahead, expansion units and fetches placed
+// between individual MFMAs, hand-over before the last K step, fetches two tiles ahead) was built
+// and measured equal to this form (1138 vs 1127-1140 TFLOP/s at 8192^3), so the simple form stays.
 #include <hip/hip_runtime.h>
 
 #include "gemm_common.h"
@@ -220,8 +224,8 @@ struct Nvfp4Gemm {
     Nvfp4Gemm<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, xs, ys, alpha, g);                            \
   }
 
-NVFP4_KERNEL(f32_256x256x64_w2x4, 256, 256, 2, 4, float)
 NVFP4_KERNEL(f32_256x256x64_w4x2, 256, 256, 4, 2, float)
+NVFP4_KERNEL(f32_256x256x64_w2x4, 256, 256, 2, 4, float)
 NVFP4_KERNEL(f32_128x128x64_w2x2, 128, 128, 2, 2, float)
 NVFP4_KERNEL(f32_64x64x64_w1x1, 64, 64, 1, 1, float)
 NVFP4_KERNEL(f32_32x32x64_w1x1, 32, 32, 1, 1, float)

@@ -96,6 +96,12 @@ def test_gpu_nvfp4_reference_example(ct, dev):
 @pytest.mark.parametrize("m,n,k,tile,variant,out", [
     (256, 256, 256, 256, None, "f32"),
     (512, 768, 1024, 256, "f32_256x256x64_w4x2", "f32"),
+    (512, 768, 1024, 256, "f32_256x256x64_w2x4", "f32"),
+    (300, 520, 64, 256, "f32_256x256x64_w4x2", "f32"),       # one K tile
+    (256, 256, 128, 256, "f32_256x256x64_w2x4", "f32"),      # two
+    (1000, 264, 192, 256, "f32_256x256x64_w4x2", "f32"),     # three, ragged edges
+    (256, 512, 256, 256, "f32_256x256x64_w2x4", "f32"),      # four
+    (520, 264, 320, 256, "bf16_256x256x64_w4x2", "bf16"),    # five
     (300, 200, 192, 128, None, "f32"),                    # ragged edges
     (96, 160, 64, 32, None, "f32"),                       # one K tile, smallest kernel tile
     (128, 128, 128, 64, None, "f32"),
