@@ -285,3 +285,72 @@ def test_driver_layer_on_the_recording_runtime(fake_hip):
     ct.check(L.cutile_testing_inject_failure(b"hipMallocAsync", 2, 1))
     st = L.cutile_malloc_async(64, s2, C.byref(p))
     assert st == 2 and b"DriverError(2)" in L.cutile_last_error_message()
+
+
+def test_decode_mapped_and_fp4_launchers_on_the_recording_runtime(fake_hip):
+    """grid translation, argument records and validation of the launchers added for the decode path,
+    mapped partitions and NVFP4 — no GPU involved"""
+    ct = fake_hip
+    L = ct.lib()
+    h = torch.half
+    # decode split: one workgroup per (KV head, split); the variant follows (GROUP, D)
+    q, kv = torch.zeros(8, 4, 128, dtype=h), torch.zeros(8, 1024, 128, dtype=h)
+    att, lse = torch.zeros(8, 16 * 4, 128, dtype=h), torch.zeros(8, 16 * 4)
+    pos = torch.zeros(1, dtype=torch.int32)
+    ct.fmha_decode_gqa_split(q, kv, kv, ct.partition(att, [1, 4, 128]), ct.partition(lse, [1, 4]), 0.088, pos, generics=[4, 64, 128, 16])
+    rec, args = _last(ct)
+    assert rec.symbol == b"fmha_decode_gqa_split_entry__f16_g4_d128" and tuple(rec.grid) == (8, 16, 1) and tuple(rec.block) == (256, 1, 1)
+    # q (32) + k (32) + v (32) + att partition (56) + lse partition (40) = 192, then scale, pad, position pointer, bn, tile grid
+    scale, = struct.unpack_from("<f", args, 192)
+    ptr, bn = struct.unpack_from("<Qi", args, 200)
+    assert abs(scale - 0.088) < 1e-7 and ptr == pos.data_ptr() and bn == 64
+    assert struct.unpack_from("<4I", args, 212)[:3] == (8, 16, 1)
+    out = torch.zeros(8, 4, 128, dtype=h)
+    ct.splitk_reduce_merge(att, lse, ct.partition(out, [1, 4, 64]))
+    rec, _ = _last(ct)
+    assert rec.symbol == b"splitk_reduce_merge_entry__f16" and tuple(rec.grid) == (8 * 4, 1, 1)
+    # kv cache update: a grid-stride copy sized by the rows written
+    nk = torch.zeros(33, 8, 128, dtype=h)
+    kc = torch.zeros(8, 96, 128, dtype=h)
+    ct.kv_cache_update_f16(nk, nk, ct.partition(kc, [1, 16, 64]), ct.partition(kc.clone(), [1, 16, 64]), 0, 33)
+    rec, _ = _last(ct)
+    assert rec.symbol == b"kv_cache_update_entry__f16" and tuple(rec.grid) == (-(-33 * 8 * 16 // 256), 1, 1)
+    # persistent GEMM: (num_tile_blocks, 1, 1) workgroups and the mapped record after the three tensors
+    z = torch.zeros(1024, 768, dtype=torch.bfloat16)
+    a, b = torch.zeros(1024, 256, dtype=torch.bfloat16), torch.zeros(256, 768, dtype=torch.bfloat16)
+    ct.gemm_persistent(ct.mapped(ct.partition(z, [256, 256]), [2, 1], 5), a, b)
+    rec, args = _last(ct)
+    assert rec.symbol == b"gemm_persistent_entry__bf16_256x256x64_d4x2" and tuple(rec.grid) == (5, 1, 1) and tuple(rec.block) == (512, 1, 1)
+    assert struct.unpack_from("<4i4I", args, 88) == (2, 1, 1, 2, 4, 3, 1, 12)      # map, rank, logical grid, stream items
+    # NVFP4: the reference example's 16x16 tiles run on the 32x32 kernel when the launch covers the tensor
+    x4, s4 = torch.zeros(16, 64, dtype=torch.uint8), torch.zeros(16, 8, dtype=torch.uint8)
+    z4 = torch.zeros(16, 16)
+    ct.linear_tile_nvfp4(ct.partition(z4, [16, 16]), x4, x4, s4, s4, 1.0, generics=[16, 16, 64, 32, 4])
+    rec, _ = _last(ct)
+    assert rec.symbol == b"linear_tile_nvfp4_entry__f32_32x32x64_w1x1" and tuple(rec.grid) == (1, 1, 1) and tuple(rec.block) == (64, 1, 1)
+    zb = torch.zeros(512, 512)
+    xb, sb = torch.zeros(512, 128, dtype=torch.uint8), torch.zeros(512, 16, dtype=torch.uint8)
+    ct.linear_tile_nvfp4(ct.partition(zb, [256, 256]), xb, xb, sb, sb, 1.0)
+    assert _last(ct)[0].symbol == b"linear_tile_nvfp4_entry__f32_256x256x64_w4x2" and tuple(_last(ct)[0].grid) == (4, 1, 1)
+
+    n0 = L.cutile_testing_launch_count()
+    q3 = torch.zeros(8, 3, 128, dtype=h)
+    att3, lse3 = torch.zeros(8, 6, 128, dtype=h), torch.zeros(8, 6)
+    cases = [
+        (lambda: ct.fmha_decode_gqa_split(q3, kv, kv, ct.partition(att3, [1, 3, 128]), ct.partition(lse3, [1, 3]), 0.1, pos), "no precompiled variant"),
+        (lambda: ct.fmha_decode_gqa_split(q, kv, kv, ct.partition(att, [1, 4, 128]), ct.partition(lse, [1, 4]), 0.1, pos, generics=[4, 64, 128, 8]), "NUM_KV_SPLITS"),
+        (lambda: ct.fmha_decode_gqa_split(q, kv, kv, ct.partition(att, [1, 4, 128]), ct.partition(lse[:, :32], [1, 4]), 0.1, pos), "do not agree"),
+        (lambda: ct.splitk_reduce_merge(att, lse, ct.partition(out, [1, 4, 48])), "CHUNK_D dividing D"),
+        (lambda: ct.kv_cache_update_f16(nk, nk, ct.partition(kc, [1, 16, 64]), ct.partition(kc.clone(), [1, 16, 64]), 4, 33), "position_start must be 0"),
+        (lambda: ct.kv_cache_update_f16(nk, nk, ct.partition(kc, [1, 16, 64]), ct.partition(kc.clone(), [1, 16, 64]), 0, 34), "seq_len = 34"),
+        (lambda: ct.gemm_persistent(ct.mapped(ct.partition(z, [256, 256]), [2, 1], 13), a, b), "cannot exceed the streamed logical tile count"),
+        (lambda: ct.gemm_persistent(ct.mapped(ct.partition(z, [256, 256]), [2, 0], 2), a, b), "both axes streamed"),
+        (lambda: ct.gemm_persistent(ct.mapped(ct.partition(z, [256, 256]), [2, 1], 5), a, b, grid=(4, 1, 1)), "does not match the inferred partition grid"),
+        (lambda: ct.linear_tile_nvfp4(ct.partition(z4, [16, 16]), x4, x4, s4[:, :4], s4, 1.0), "scales must be"),
+        (lambda: ct.linear_tile_nvfp4(ct.partition(z4, [16, 16]), x4, x4, s4, s4, 1.0, generics=[16, 16, 64, 32, 2]), "BK_SCALES"),
+        (lambda: ct.linear_tile_nvfp4(ct.partition(torch.zeros(16, 16, dtype=h), [16, 16]), x4, x4, s4, s4, 1.0), "z must be f32 or bf16"),
+    ]
+    for fn, msg in cases:
+        with pytest.raises(ct.CutileError, match=msg):
+            fn()
+    assert L.cutile_testing_launch_count() == n0
