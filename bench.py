@@ -538,9 +538,17 @@ class DecodeAttention(Workload):
                 "sample": "full size"}, {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
 
 
+class DecodeAttentionWide(DecodeAttention):
+    """GROUP 8: the split kernel runs on the matrix cores (heads are the N dimension of a 16x16x32 MFMA)."""
+    name = "decode_gqa_f16_h8g8d128_s131072"
+    group, splits = 8, 64
+    config = {"workload": "decode attention fp16: fmha_decode_gqa_split + splitk_reduce_merge, 8 KV heads x GROUP 8, D 128, "
+                          "131072 cached keys, 64 KV splits, BN 64 (two launches per step)"}
+
+
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

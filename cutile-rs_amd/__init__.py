@@ -425,10 +425,10 @@ def kv_cache_update_f16(new_k, new_v, k_cache: Partition, v_cache: Partition, po
 
 
 def fmha_decode_gqa_split(q, k, v, att_out: Partition, lse_out: Partition, qk_scale: float, position_start, *, stream=None,
-                          grid=None, generics=None) -> None:
+                          grid=None, generics=None, variant=None) -> None:
     """split-KV decode attention (attention.rs:737-902); position_start: one-element device tensor"""
     qa, ka, va, pa = tensor_arg(q), tensor_arg(k), tensor_arg(v), tensor_arg(position_start, dtype=U32)
-    o, keep = _opts(grid, generics, None)
+    o, keep = _opts(grid, generics, variant)
     check(lib().cutile_launch_fmha_decode_gqa_split(_stream(stream), C.byref(qa), C.byref(ka), C.byref(va),
                                                     C.byref(att_out.arg()), C.byref(lse_out.arg()), C.c_float(qk_scale),
                                                     C.byref(pa), C.byref(o)))

@@ -928,12 +928,16 @@ cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, cons
   CUTILE_REQUIRE(decode_vec_layout(*q) && decode_vec_layout(*k) && decode_vec_layout(*v) && decode_vec_layout(at) &&
                      ((uintptr_t)position_start->ptr & 3) == 0 && ((uintptr_t)lt.ptr & 3) == 0,
                  CUTILE_ERR_KERNEL_NOT_FOUND, "fmha_decode_gqa_split: precompiled variants need unit head-dim stride and 16-byte aligned rows");
-  const std::string want = "f16_g" + std::to_string(group) + "_d" + std::to_string(d);
-  CUTILE_REQUIRE(find_entry("fmha_decode_gqa_split", want), CUTILE_ERR_KERNEL_NOT_FOUND,
+  // GROUP >= 8: the matrix-core variant first (the vector-ALU one no longer keeps up with HBM there)
+  const std::string plain = "f16_g" + std::to_string(group) + "_d" + std::to_string(d);
+  std::vector<std::string> acceptable;
+  for (const std::string& name : {plain + "_mfma", plain})
+    if (find_entry("fmha_decode_gqa_split", name)) acceptable.push_back(name);
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
                  "no precompiled variant of fmha_decode_gqa_split<GROUP=%d, D=%d>; available: %s", group, d,
                  list_variants("fmha_decode_gqa_split").c_str());
   Resolved res;
-  if (cutile_status_t s = resolve_entry("fmha_decode_gqa_split", opts, want, {want}, &res)) return s;
+  if (cutile_status_t s = resolve_entry("fmha_decode_gqa_split", opts, acceptable[0], acceptable, &res)) return s;
   ArgPacker args;
   args.push_tensor(*q);
   args.push_tensor(*k);

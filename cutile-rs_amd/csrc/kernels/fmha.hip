@@ -947,6 +947,201 @@ __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const Tensor
   }
 }
 
+// ---- decode attention on the matrix cores, for wide groups ---------------------------------------
+// With GROUP >= 8 the vector ALUs no longer keep up with HBM (two dot products per cached value
+// and head).  Here a wavefront takes 32 keys at a time and uses v_mfma_f32_16x16x32_f16 with
+// the query heads as the 16-wide N dimension (heads beyond GROUP are zero):
+//   S^T [16 keys x 16 heads]  = K [16 keys x D]   . Q^T [D x 16 heads]     (two blocks of 16 keys)
+//   O^T [D x 16 heads]       += V^T [D x 32 keys]  . P^T [32 keys x 16 heads]
+// so that every lane owns ONE head (column) in both products: running maximum, sum and the
+// rescale factor are per-lane scalars, and the f32 scores a lane holds after the first product
+// (4 keys of each block) ARE, converted to f16, its 8 values of the second product's B operand —
+// the 32 keys of the slab are simply taken in the order in which the lanes already hold them.
+// K rows are MFMA A operands straight from global memory (a lane loads 16 bytes of one key).
+// V must be read transposed (8 keys of one column per lane): each wavefront streams its V rows
+// into a private LDS stage with 16-byte direct loads (chunk c of row r at chunk c ^ 2(r & 3),
+// so the transposing reads of 4 rows x 2 chunks are conflict-free) and reads them back with
+// ds_read_b64_tr_b16.  Two stages, one 32-key slab ahead; wavefront-private, so the loop has no
+// barrier.  Slabs past the end of the split re-read its last row and are masked (p = 0).
+template <int G, int D>
+__device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const TensorArg<3>& k, const TensorArg<3>& v,
+                                                  const PartitionArg<3>& att_out, const PartitionArg<2>& lse_out,
+                                                  float qk_scale, const uint32_t* pos_dev, int32_t bn, const TileGrid& g) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int kWaves = 4, kSlab = 32;
+  constexpr int QS = D / 32;                 // K slices of the first product
+  constexpr int OS = D / 16;                 // 16-row slices of O^T
+  constexpr int CP = D / 8;                  // 16-byte chunks per V row
+  constexpr int kRowsPerInstr = 64 / CP;     // V rows one direct load covers
+  constexpr int kVInstr = kSlab / kRowsPerInstr;
+  constexpr int kStageBytes = kSlab * D * 2;
+  static_assert(G <= 16 && D % 32 == 0 && CP <= 64 && 64 % CP == 0, "decode tile");
+  __shared__ __attribute__((aligned(1024))) unsigned char vst[kWaves][2][kStageBytes];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, quad = lane >> 4;           // head (column) and key group of this lane
+  const int32_t head = blockIdx.x, split = blockIdx.y, splits = (int32_t)g.y;
+  const int32_t max_seq = min(k.shape[1], v.shape[1]);
+  const int32_t s_kv = min((int32_t)pos_dev[0] + 1, max_seq);
+  const int32_t tiles = (s_kv + bn - 1) / bn, per_split = (tiles + splits - 1) / splits;
+  const int32_t r0 = split * per_split * bn;
+  const int32_t r1 = min(min((split + 1) * per_split, tiles) * bn, s_kv);
+  const float c = qk_scale * kLog2e;
+
+  // Q^T operands: column = head, 8 consecutive d per lane and slice
+  f16x8 qf[QS];
+#pragma unroll
+  for (int sidx = 0; sidx < QS; ++sidx) {
+    f16x8 t = {};
+    if (col < G) t = *reinterpret_cast<const f16x8*>((const _Float16*)q.ptr + (int64_t)head * q.strides[0] + (int64_t)col * q.strides[1] + sidx * 32 + quad * 8);
+    qf[sidx] = t;
+  }
+  const _Float16* kb = (const _Float16*)k.ptr + (int64_t)head * k.strides[0];
+  const _Float16* vbase = (const _Float16*)v.ptr + (int64_t)head * v.strides[0];
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(vbase, (uint32_t)(((int64_t)(max_seq - 1) * v.strides[1] + D) * 2));
+  unsigned char* my_stage[2] = {vst[wave][0], vst[wave][1]};
+
+  // LDS side of the transposing reads: lane i of a 16-lane group supplies row (i >> 2), columns 4 (i & 3) .. + 3
+  int tr_off[2];
+  {
+    const int i16 = lane & 15;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int row = blk * 16 + quad * 4 + (i16 >> 2);
+      const int cc = (i16 & 3) * 4;                    // column inside the 16-column slice
+      tr_off[blk] = row * (D * 2) + ((((cc >> 3)) ^ ((row & 3) << 1)) << 4) + (cc & 7) * 2;
+    }
+  }
+  auto request_slab = [&](int32_t base, f16x8 (&kreg)[2][QS], unsigned char* stage) {
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int32_t row = min(base + blk * 16 + col, r1 - 1);
+#pragma unroll
+      for (int sidx = 0; sidx < QS; ++sidx)
+        kreg[blk][sidx] = *reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1] + sidx * 32 + quad * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < kVInstr; ++i) {
+      const int lrow = i * kRowsPerInstr + lane / CP;
+      const int chunk = (lane % CP) ^ ((lrow & 3) << 1);
+      const int32_t row = min(base + lrow, r1 - 1);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (LDS_PTR(void))(stage + i * 1024), 16,
+                                               (uint32_t)(((int64_t)row * v.strides[1] + chunk * 8) * 2), 0, 0, 0);
+    }
+  };
+
+  float m = -1.0e30f, l = 0.0f;
+  f32x4 oacc[OS];
+#pragma unroll
+  for (int i = 0; i < OS; ++i) oacc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  auto slab = [&](int32_t base, const f16x8 (&kreg)[2][QS], const unsigned char* stage) {
+    f32x4 sc[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      sc[blk] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int sidx = 0; sidx < QS; ++sidx) sc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[blk][sidx], qf[sidx], sc[blk], 0, 0, 0);
+    }
+    // this lane: head `col`, keys base + 16 blk + 4 quad + i
+    float sv[8], mx = -INFINITY;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool valid = base + blk * 16 + quad * 4 + i < r1;
+        sv[blk * 4 + i] = valid ? sc[blk][i] * c : -INFINITY;
+        mx = fmaxf(mx, sv[blk * 4 + i]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    float rs = 0.0f;
+    f16x8 pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pv = __builtin_amdgcn_exp2f(sv[e] - m_new);
+      rs += pv;
+      pf[e] = (_Float16)pv;
+    }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * alpha + rs;
+    if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+#pragma unroll
+      for (int i = 0; i < OS; ++i) oacc[i] *= alpha;
+    }
+    m = m_new;
+    // this slab's V rows (requested one slab ago) have landed once at most the 2 QS + kVInstr loads
+    // of the slab requested after them are outstanding
+    __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * QS + kVInstr) & 15) | ((((2 * QS + kVInstr) >> 4) & 3) << 14));
+#pragma unroll
+    for (int i = 0; i < OS; ++i) {
+      // slice i lies 2 i chunks further; chunk numbers are XOR-swizzled, so the offset is an XOR too
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(stage + (tr_off[0] ^ (i << 5))));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(stage + (tr_off[1] ^ (i << 5))));
+      const f16x8 vt = __builtin_bit_cast(f16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      oacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pf, oacc[i], 0, 0, 0);
+    }
+  };
+
+  f16x8 ka[2][QS], kbuf[2][QS];
+  const int32_t first = r0 + wave * kSlab, stride = kWaves * kSlab;
+  if (first < r1) {
+    request_slab(first, ka, my_stage[0]);
+    for (int32_t base = first; base < r1; base += 2 * stride) {      // wavefront-uniform; slabs past r1 are masked
+      request_slab(base + stride, kbuf, my_stage[1]);
+      slab(base, ka, my_stage[0]);
+      request_slab(base + 2 * stride, ka, my_stage[0]);
+      slab(base + stride, kbuf, my_stage[1]);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();     // every wavefront is done with its stages: they now carry the partial results
+
+  float* sm = reinterpret_cast<float*>(&vst[0][0][0]);            // [kWaves][16]
+  float* sl = sm + kWaves * 16;                                   // [kWaves][16]
+  float* sacc = sl + kWaves * 16;                                 // [kWaves][G][D]
+  static_assert((2 * kWaves * 16 + kWaves * G * D) * 4 <= kWaves * 2 * kStageBytes, "partials fit the stages");
+  if (col < G) {
+    if (quad == 0) {
+      sm[wave * 16 + col] = m;
+      sl[wave * 16 + col] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < OS; ++i)
+      *reinterpret_cast<f32x4*>(sacc + ((wave * G + col) * D + i * 16 + quad * 4)) = oacc[i];
+  }
+  __syncthreads();
+  if (wave == 0 && col < G) {
+    float mt = sm[col];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mt = fmaxf(mt, sm[w * 16 + col]);
+    float lt = 0.0f, f[kWaves];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      f[w] = __builtin_amdgcn_exp2f(sm[w * 16 + col] - mt);
+      lt += sl[w * 16 + col] * f[w];
+    }
+    if (r0 >= r1) lt = (float)bn;   // no keys in this split: the tile program's untouched l = 1 per lane
+    const float safe = fmaxf(lt, 1.0e-8f);
+    const int64_t orow = (int64_t)split * G + col;
+    _Float16* dst = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + orow * att_out.strides[1];
+#pragma unroll
+    for (int i = 0; i < OS; ++i) {
+      f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) a += *reinterpret_cast<const f32x4*>(sacc + ((w * G + col) * D + i * 16 + quad * 4)) * f[w];
+      f16x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = (_Float16)(a[j] / safe);
+      *reinterpret_cast<f16x4*>(dst + i * 16 + quad * 4) = o;
+    }
+    if (quad == 0) ((float*)lse_out.ptr)[(int64_t)head * lse_out.strides[0] + orow * lse_out.strides[1]] = mt + __builtin_log2f(safe);
+  }
+}
+
 // out[h, g, :] = sum_s w[g, s] att[h, s*GROUP + g, :], w = exp2(lse - max_s lse) / max(sum, 1e-8).
 // One workgroup per (KV head, query head of the group).  The weights come from two
 // workgroup-wide reductions over the splits; then the rows of the partial results are
@@ -1076,6 +1271,21 @@ FMHA_PINGPONG_KERNEL(f16, _Float16, 64, 128)
 DECODE_SPLIT_GROUPS(64)
 DECODE_SPLIT_GROUPS(128)
 DECODE_SPLIT_GROUPS(256)
+
+#define DECODE_SPLIT_MFMA_KERNEL(G, D)                                                             \
+  extern "C" __global__ void __launch_bounds__(256)                                               \
+      fmha_decode_gqa_split_entry__f16_g##G##_d##D##_mfma(TensorArg<3> q, TensorArg<3> k, TensorArg<3> v, \
+                                                          PartitionArg<3> att_out, PartitionArg<2> lse_out, \
+                                                          float qk_scale, const uint32_t* position_start, \
+                                                          int32_t bn, TileGrid g) {                \
+    decode_split_mfma<G, D>(q, k, v, att_out, lse_out, qk_scale, position_start, bn, g);          \
+  }
+DECODE_SPLIT_MFMA_KERNEL(8, 64)
+DECODE_SPLIT_MFMA_KERNEL(8, 128)
+DECODE_SPLIT_MFMA_KERNEL(8, 256)
+DECODE_SPLIT_MFMA_KERNEL(16, 64)
+DECODE_SPLIT_MFMA_KERNEL(16, 128)
+DECODE_SPLIT_MFMA_KERNEL(16, 256)
 
 // splitk_reduce_merge<GROUP, D, CHUNK_D, NUM_KV_SPLITS, ..>(att_partial, lse_partial, out: [1,GROUP,CHUNK_D] tiles)
 extern "C" __global__ void __launch_bounds__(256)

@@ -147,14 +147,14 @@ def test_gpu_kv_cache_update_both_forms(ct, dev):
     assert torch.all(wide_k[..., d2:] == 0) and torch.all(wide_v[..., d2:] == 0)
 
 
-def _run_decode(ct, dev, q, k, v, scale, pos, bn, splits):
+def _run_decode(ct, dev, q, k, v, scale, pos, bn, splits, variant=None):
     heads, group, d = q.shape
     att = torch.full((heads, splits * group, d), float("nan"), dtype=torch.float16, device=dev)
     lse = torch.full((heads, splits * group), float("nan"), dtype=torch.float32, device=dev)
     out = torch.full((heads, group, d), float("nan"), dtype=torch.float16, device=dev)
     p = torch.tensor([pos], dtype=torch.int32, device=dev)
     ct.fmha_decode_gqa_split(_dev(q, dev), _dev(k, dev), _dev(v, dev), ct.partition(att, [1, group, d]),
-                             ct.partition(lse, [1, group]), scale, p, generics=[group, bn, d, splits])
+                             ct.partition(lse, [1, group]), scale, p, generics=[group, bn, d, splits], variant=variant)
     ct.splitk_reduce_merge(att, lse, ct.partition(out, [1, group, d]), generics=[group, d, d, splits])
     torch.cuda.synchronize()
     return _bits(att), lse.cpu().numpy(), _bits(out)
@@ -167,11 +167,17 @@ def _run_decode(ct, dev, q, k, v, scale, pos, bn, splits):
     (4, 1, 256, 200, 0, 64, 4),           # one key: three of four splits are empty
     (3, 2, 128, 520, 130, 64, 16),        # more splits than tiles
     (1, 8, 256, 4100, 4099, 128, 5),
+    (4, 16, 128, 1500, 1403, 64, 6),      # GROUP 16 exists on the matrix cores only
+    (2, 16, 64, 90, 70, 16, 2),
 ])
 def test_gpu_decode_split_and_merge(ct, dev, heads, group, d, max_seq, pos, bn, splits):
     q, k, v = normal_f16_bits((heads, group, d), 751), normal_f16_bits((heads, max_seq, d), 752), normal_f16_bits((heads, max_seq, d), 753)
     scale = float(np.float16(1.0 / np.sqrt(d)))
     att, lse, out = _run_decode(ct, dev, q, k, v, scale, pos, bn, splits)
+    if group == 8:      # GROUP 8 has two variants: the matrix-core one is the default, the vector-ALU one must agree too
+        att_v, lse_v, out_v = _run_decode(ct, dev, q, k, v, scale, pos, bn, splits, variant=f"f16_g8_d{d}")
+        assert np.max(np.abs(f32(att_v) - f32(att))) <= 2e-2 and np.max(np.abs(f32(out_v) - f32(out))) <= 2e-2
+        assert np.allclose(lse_v, lse, atol=2e-3)
     att_ref, lse_ref = oracle.fmha_decode_gqa_split(q, k, v, scale, pos, bn, splits)
     out_ref = oracle.splitk_reduce_merge(att_ref, lse_ref, group)
     # tolerance: max-abs 2e-2 as for the prefill attention kernel; observed differences are a few f16 ulps
