@@ -83,17 +83,26 @@ struct Elem<_Float16> {
 // the 8 XCDs in dispatch order; every query tile of one head is given to the same
 // XCD, consecutively, so that the head's K and V (read by each of its query
 // tiles) stay in that XCD's L2 instead of being fetched from HBM once per tile.
-// Causal launches keep the plain order instead, heaviest tiles (largest query
-// index) of all heads first: their tiles differ 16-fold in length and measured
-// faster balanced across the whole chip than cached per XCD.
+// Causal launches do the same with a few heads side by side per XCD, heaviest tiles
+// first (see below); one head at a time measured slower than the plain order because the
+// last head's long tiles start late.
 __device__ __forceinline__ void head_and_tile(uint32_t n_bh, uint32_t n_qt, int32_t causal, int32_t* bh, int32_t* q_tile) {
   constexpr uint32_t kNumXcd = 8;
   const uint32_t id = blockIdx.x + gridDim.x * blockIdx.y;
   uint32_t b, t;
+  constexpr uint32_t kCusPerXcd = 32;
+  const uint32_t side = n_qt >= kCusPerXcd ? 1 : kCusPerXcd / n_qt;     // heads an XCD works on side by side
   if (n_bh % kNumXcd == 0 && !causal) {
     const uint32_t xcd = id % kNumXcd, slot = id / kNumXcd;
     b = (slot / n_qt) * kNumXcd + xcd;
     t = slot % n_qt;
+  } else if (n_bh % (kNumXcd * side) == 0 && causal) {
+    // Causal tiles differ n_qt-fold in length.  An XCD takes `side` heads at a time (their K/V fit its L2) and
+    // walks their tiles heaviest first, heads interleaved: the compute units that drew the short tiles of one
+    // group free up first and draw the long tiles of the next, so lengths pair up (n_qt + 1 per two tiles).
+    const uint32_t xcd = id % kNumXcd, slot = id / kNumXcd, per_group = side * n_qt;
+    b = xcd * (n_bh / kNumXcd) + (slot / per_group) * side + (slot % per_group) % side;
+    t = (slot % per_group) / side;
   } else {   // plain order: every (head, tile) still covered exactly once
     b = id % n_bh;
     t = id / n_bh;
