@@ -498,10 +498,10 @@ class KvCacheUpdate(Workload):
 
 class DecodeAttention(Workload):
     name, unit, dtype = "decode_gqa_f16_h8g4d128_s131072", "GB/s", "f16 io / f32 softmax+acc"
-    heads, group, d, s, splits, bn = 8, 4, 128, 131072, 128, 64
+    heads, group, d, s, splits, bn = 8, 4, 128, 131072, 32, 64
     work = float(2 * heads * s * d * 2)          # every K and V byte once; q, partials and out are < 0.2 %
     config = {"workload": "decode attention fp16: fmha_decode_gqa_split + splitk_reduce_merge, 8 KV heads x GROUP 4, D 128, "
-                          "131072 cached keys, 128 KV splits, BN 64 (two launches per step)"}
+                          "131072 cached keys, 32 KV splits (one workgroup per CU), BN 64 (two launches per step)"}
 
     def setup(self, ct, torch, oracle, dev):
         import numpy as np
@@ -541,9 +541,9 @@ class DecodeAttention(Workload):
 class DecodeAttentionWide(DecodeAttention):
     """GROUP 8: the split kernel runs on the matrix cores (heads are the N dimension of a 16x16x32 MFMA)."""
     name = "decode_gqa_f16_h8g8d128_s131072"
-    group, splits = 8, 64
+    group, splits = 8, 32
     config = {"workload": "decode attention fp16: fmha_decode_gqa_split + splitk_reduce_merge, 8 KV heads x GROUP 8, D 128, "
-                          "131072 cached keys, 64 KV splits, BN 64 (two launches per step)"}
+                          "131072 cached keys, 32 KV splits (one workgroup per CU), BN 64 (two launches per step)"}
 
 
 def make_workloads():

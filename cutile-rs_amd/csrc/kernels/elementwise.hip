@@ -338,8 +338,8 @@ extern "C" __global__ void __launch_bounds__(kThreads)
       };
       if (vec) {
         Vec16<_Float16> lo, hi, ylo, yhi;
-        lo.raw = *reinterpret_cast<const u32x4*>(xr + i0);
-        hi.raw = *reinterpret_cast<const u32x4*>(xr + half + i0);
+        lo.raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr + i0));
+        hi.raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr + half + i0));
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           float sn, cs;
@@ -348,8 +348,8 @@ extern "C" __global__ void __launch_bounds__(kThreads)
           ylo.v[e] = (_Float16)(l * cs - hv * sn);
           yhi.v[e] = (_Float16)(hv * cs + l * sn);
         }
-        *reinterpret_cast<u32x4*>(orow + i0) = ylo.raw;
-        *reinterpret_cast<u32x4*>(orow + half + i0) = yhi.raw;
+        __builtin_nontemporal_store(ylo.raw, reinterpret_cast<u32x4*>(orow + i0));
+        __builtin_nontemporal_store(yhi.raw, reinterpret_cast<u32x4*>(orow + half + i0));
       } else {
         for (int32_t i = i0; i < min(i0 + 8, half); ++i) {
           float sn, cs;

@@ -762,21 +762,23 @@ template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
+// K and V rows are read once per launch by one workgroup: streamed past the caches (nontemporal).
 template <int W>
 __device__ __forceinline__ void load_row(const _Float16* p, uint32_t (&dst)[W]) {
   if constexpr (W == 2) {
-    const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+    const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
     dst[0] = t[0], dst[1] = t[1];
   } else {
 #pragma unroll
     for (int i = 0; i < W / 4; ++i) {
-      const u32x4 t = *reinterpret_cast<const u32x4*>(p + i * 8);
+      const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + i * 8));
 #pragma unroll
       for (int e = 0; e < 4; ++e) dst[i * 4 + e] = t[e];
     }
   }
 }
 constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v / 2); }
+constexpr int kNontemporal = 2;     // cache-policy operand of buffer loads: the nt bit
 }  // namespace decode
 
 template <int G, int D>
@@ -1027,7 +1029,7 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       const int32_t row = min(base + blk * 16 + col, r1 - 1);
 #pragma unroll
       for (int sidx = 0; sidx < QS; ++sidx)
-        kreg[blk][sidx] = *reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1] + sidx * 32 + quad * 8);
+        kreg[blk][sidx] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1] + sidx * 32 + quad * 8));
     }
 #pragma unroll
     for (int i = 0; i < kVInstr; ++i) {
@@ -1035,7 +1037,7 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       const int chunk = (lane % CP) ^ ((lrow & 3) << 1);
       const int32_t row = min(base + lrow, r1 - 1);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (LDS_PTR(void))(stage + i * 1024), 16,
-                                               (uint32_t)(((int64_t)row * v.strides[1] + chunk * 8) * 2), 0, 0, 0);
+                                               (uint32_t)(((int64_t)row * v.strides[1] + chunk * 8) * 2), 0, 0, decode::kNontemporal);
     }
   };
 
