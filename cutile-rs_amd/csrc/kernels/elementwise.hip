@@ -129,6 +129,70 @@ __device__ __forceinline__ void for_each_tile_elem(const P& out, F body) {
   }
 }
 
+// out[i * stride] = f(i) for i < count: 16 bytes per lane where the layout allows it
+// (unit stride, 16-byte aligned base), element by element otherwise and for the tail.
+template <typename T, typename F>
+__device__ __forceinline__ void flat_generate(T* out, int64_t stride, size_t count, F f) {
+  const size_t step = (size_t)gridDim.x * kThreads, gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (stride == 1 && ((uintptr_t)out & 15) == 0) {
+    using V = Vec16<T>;
+    const size_t nvec = count / V::N;
+    for (size_t j = gid; j < nvec; j += step) {
+      V r;
+#pragma unroll
+      for (int e = 0; e < V::N; ++e) r.v[e] = f(j * V::N + e);
+      reinterpret_cast<u32x4*>(out)[j] = r.raw;
+    }
+    done = nvec * V::N;
+  }
+  for (size_t i = done + gid; i < count; i += step) out[(int64_t)i * stride] = f(i);
+}
+
+template <typename D, typename S>
+__device__ __forceinline__ D convert_elem(S v) {
+  return (D)v;
+}
+// The two 16-bit float formats convert through f32 (exact in that direction).
+template <>
+__device__ __forceinline__ __bf16 convert_elem<__bf16, _Float16>(_Float16 v) {
+  return (__bf16)(float)v;
+}
+template <>
+__device__ __forceinline__ _Float16 convert_elem<_Float16, __bf16>(__bf16 v) {
+  return (_Float16)(float)v;
+}
+
+// dst[i] = convert(src[i]) for i < count, zero where src has no element i.  Streams of
+// unit stride and 16-byte aligned bases move kElems elements per lane and pass (16 bytes of the
+// narrower type, 16 to 64 of the wider), nontemporally; the rest goes element by element.
+template <typename D, typename S>
+__device__ __forceinline__ void flat_convert(const S* src, int64_t src_stride, size_t src_count, D* dst,
+                                             int64_t dst_stride, size_t count) {
+  constexpr int kElems = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));
+  constexpr int kSrcVecs = kElems * sizeof(S) / 16, kDstVecs = kElems * sizeof(D) / 16;
+  const size_t step = (size_t)gridDim.x * kThreads, gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (src_stride == 1 && dst_stride == 1 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    const size_t nvec = (count < src_count ? count : src_count) / kElems;
+    for (size_t j = gid; j < nvec; j += step) {
+      union { u32x4 raw[kSrcVecs]; S v[kElems]; } in;
+      union { u32x4 raw[kDstVecs]; D v[kElems]; } out;
+#pragma unroll
+      for (int q = 0; q < kSrcVecs; ++q) in.raw[q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + j * kSrcVecs + q);
+#pragma unroll
+      for (int e = 0; e < kElems; ++e) out.v[e] = convert_elem<D, S>(in.v[e]);
+#pragma unroll
+      for (int q = 0; q < kDstVecs; ++q) __builtin_nontemporal_store(out.raw[q], reinterpret_cast<u32x4*>(dst) + j * kDstVecs + q);
+    }
+    done = nvec * kElems;
+  }
+  for (size_t i = done + gid; i < count; i += step) {
+    const S v = i < src_count ? src[(int64_t)i * src_stride] : S(0);
+    dst[(int64_t)i * dst_stride] = convert_elem<D, S>(v);
+  }
+}
+
 }  // namespace
 
 // ---- saxpy: y <- a*x + y -------------------------------------------------------------------
@@ -367,17 +431,13 @@ extern "C" __global__ void __launch_bounds__(kThreads)
 #define CREATION_KERNELS(T, NAME)                                                                   \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \
       full_entry__##NAME(T value, PartitionArg<1> t, TileGrid g) {                                  \
-    size_t count = covered_1d(t.shape[0], t.pshape[0], g);                                         \
-    size_t stride = (size_t)gridDim.x * kThreads;                                                  \
-    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < count; i += stride)          \
-      ((T*)t.ptr)[i * t.strides[0]] = value;                                                       \
+    flat_generate<T>((T*)t.ptr, t.strides[0], covered_1d(t.shape[0], t.pshape[0], g),             \
+                     [&](size_t) { return value; });                                               \
   }                                                                                                 \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \
       arange_entry__##NAME(PartitionArg<1> t, TileGrid g) {                                         \
-    size_t count = covered_1d(t.shape[0], t.pshape[0], g);                                         \
-    size_t stride = (size_t)gridDim.x * kThreads;                                                  \
-    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < count; i += stride)          \
-      ((T*)t.ptr)[i * t.strides[0]] = (T)(int32_t)i;                                               \
+    flat_generate<T>((T*)t.ptr, t.strides[0], covered_1d(t.shape[0], t.pshape[0], g),             \
+                     [&](size_t i) { return (T)(int32_t)i; });                                     \
   }
 
 CREATION_KERNELS(float, f32)
@@ -392,36 +452,16 @@ CREATION_KERNELS(uint32_t, u32)
 
 extern "C" __global__ void __launch_bounds__(kThreads)
     linspace_entry__f32(PartitionArg<1> t, float start, float step, TileGrid g) {
-  size_t count = covered_1d(t.shape[0], t.pshape[0], g);
-  size_t stride = (size_t)gridDim.x * kThreads;
-  for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < count; i += stride)
-    ((float*)t.ptr)[i * t.strides[0]] = start + (float)(int32_t)i * step;
+  flat_generate<float>((float*)t.ptr, t.strides[0], covered_1d(t.shape[0], t.pshape[0], g),
+                       [&](size_t i) { return start + (float)(int32_t)i * step; });
 }
 
 // ---- convert -------------------------------------------------------------------------------
-template <typename D, typename S>
-__device__ __forceinline__ D convert_elem(S v) {
-  return (D)v;
-}
-// The two 16-bit float formats convert through f32 (exact in that direction).
-template <>
-__device__ __forceinline__ __bf16 convert_elem<__bf16, _Float16>(_Float16 v) {
-  return (__bf16)(float)v;
-}
-template <>
-__device__ __forceinline__ _Float16 convert_elem<_Float16, __bf16>(__bf16 v) {
-  return (_Float16)(float)v;
-}
-
 #define CONVERT_KERNEL(S, SN, D, DN)                                                                \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \
       convert_entry__##SN##_##DN(TensorArg<1> src, PartitionArg<1> dst, TileGrid g) {               \
-    size_t count = covered_1d(dst.shape[0], dst.pshape[0], g);                                     \
-    size_t stride = (size_t)gridDim.x * kThreads;                                                  \
-    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < count; i += stride) {        \
-      S v = i < (size_t)src.shape[0] ? ((const S*)src.ptr)[i * src.strides[0]] : S(0);            \
-      ((D*)dst.ptr)[i * dst.strides[0]] = convert_elem<D, S>(v);                                   \
-    }                                                                                               \
+    flat_convert<D, S>((const S*)src.ptr, src.strides[0], (size_t)src.shape[0], (D*)dst.ptr,       \
+                       dst.strides[0], covered_1d(dst.shape[0], dst.pshape[0], g));                \
   }
 
 #define CONVERT_FROM(S, SN)            \

@@ -143,6 +143,40 @@ def test_convert(ct, dev, src, dst):
     assert torch.equal(d, s.to(dst))
 
 
+def test_creation_and_convert_vector_paths_tails_and_layouts(ct, dev):
+    """16-byte paths with a ragged tail, a base that is not 16-byte aligned, a source shorter than the
+    destination (zero padding, cutile/src/_core.rs:651-657) and a strided destination"""
+    n = 100003
+    t = torch.full((n + 1,), 5.0, dtype=torch.float16, device=dev)
+    ct.full(-2.25, ct.partition(t[1:], [128]))                     # base 2 bytes past an aligned address
+    sync()
+    assert t[0] == 5.0 and torch.all(t[1:] == -2.25)
+    for dtype in (torch.int64, torch.float16, torch.uint8 if hasattr(ct, "U8") else torch.int32):
+        a = torch.zeros(n, dtype=dtype, device=dev)
+        ct.arange(ct.partition(a, [128]))
+        sync()
+        assert torch.equal(a, torch.arange(n, device=dev).to(dtype))
+    lin = torch.zeros(n, device=dev)
+    ct.linspace(ct.partition(lin, [128]), -3.0, 0.25)
+    sync()
+    assert torch.equal(lin, -3.0 + torch.arange(n, device=dev).float() * 0.25)
+    src = torch.from_numpy(oracle.uniform_f32(70001, 73, -100, 100)).to(dev)
+    for dst_dtype in (torch.float16, torch.bfloat16, torch.float64, torch.int32):
+        d = torch.full((n,), 7, dtype=dst_dtype, device=dev)
+        ct.convert(src, ct.partition(d, [128]))
+        sync()
+        assert torch.equal(d[:70001], src.to(dst_dtype)) and torch.all(d[70001:] == 0)
+    h = src.to(torch.float16)
+    wide = torch.zeros(2 * 70001, dtype=torch.float32, device=dev)
+    ct.convert(h, ct.partition(wide[::2], [128]))                  # strided destination: element by element
+    sync()
+    assert torch.equal(wide[::2], h.float()) and torch.all(wide[1::2] == 0)
+    d = torch.zeros(70000, dtype=torch.float32, device=dev)
+    ct.convert(h[1:], ct.partition(d, [128]))                      # source base not 16-byte aligned
+    sync()
+    assert torch.equal(d, h[1:].float())
+
+
 # ---- K2: RMSNorm ----------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,n,variant", [
     (64, 512, None), (33, 1024, None), (16, 2048, None), (16, 4096, None), (32, 8192, None),
