@@ -102,11 +102,11 @@ std::vector<KernelEntry> build_table() {
     add("softmax", keep("f32_" + v), keep("softmax_entry__f32_" + v), IMG_ROWWISE, 256, 0, 0, 0, rv.vpl, rv.wpr, "f32",
         (int64_t)rv.wpr * 64 * rv.vpl * 4, 2);
   }
-  // short rows: LPR lanes per row, 256 / LPR rows per workgroup (tile[1]); capacity LPR * 8
+  // short rows: LPR lanes per row, 4 passes of 256 / LPR rows per workgroup (tile[1] rows in all); capacity LPR * 8
   for (const char* fn : {"rms_norm_f16", "qk_norm_f16"})
     for (int lpr : {8, 16, 32}) {
       std::string v = "s" + std::to_string(lpr);
-      add(fn, keep(v), keep(std::string(fn) + "_entry__" + v), IMG_ROWWISE, 256, 0, 0, 256 / lpr, 1, 1, "f16", (int64_t)lpr * 8, 2);
+      add(fn, keep(v), keep(std::string(fn) + "_entry__" + v), IMG_ROWWISE, 256, 0, 0, 4 * 256 / lpr, 1, 1, "f16", (int64_t)lpr * 8, 2);
     }
   // the fused row norms of the transformer block share the register-resident row machinery
   static const RowVariant kFusedRow[] = {{1, 1}, {1, 2}, {1, 4}, {1, 8}, {2, 2}, {2, 4}, {2, 8}, {4, 1}, {4, 2}, {4, 4}, {4, 8}};

@@ -27,6 +27,8 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "kernel_args.h"
 
 using namespace cutile;
@@ -143,8 +145,25 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
 }
 
 // Short rows (head-dimension norms: N = 64 .. 256): LPR lanes per row, one
-// 16-byte vector per lane, 64 / LPR rows per wavefront; the reduction stays
-// inside the LPR-lane group.  With a wavefront per row most lanes would idle.
+// 16-byte vector per lane, 64 / LPR rows per wavefront and pass, kShortRowPasses passes per
+// wavefront with all their loads issued first (64 bytes in flight per lane, as in the long-row
+// kernels); the reduction stays inside the LPR-lane group, on the cross-lane data path (sums of
+// quad neighbours, then mirrored halves: every step pairs groups that already agree).
+// With a wavefront per row most lanes would idle.
+constexpr int kShortRowPasses = 4;
+template <int LPR>
+__device__ __forceinline__ float lane_group_sum(float v) {
+  auto add_dpp = [](float a, auto ctrl) {
+    constexpr int kCtrl = decltype(ctrl)::value;
+    return a + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), kCtrl, 0xf, 0xf, false));
+  };
+  v = add_dpp(v, std::integral_constant<int, 0xB1>{});                          // quad_perm [1,0,3,2]
+  v = add_dpp(v, std::integral_constant<int, 0x4E>{});                          // quad_perm [2,3,0,1]
+  if constexpr (LPR >= 8) v = add_dpp(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
+  if constexpr (LPR >= 16) v = add_dpp(v, std::integral_constant<int, 0x140>{}); // row_mirror
+  if constexpr (LPR >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
 template <int LPR>
 __device__ __forceinline__ void rms_norm_rows_short(const _Float16* __restrict__ x, int64_t x_row_stride,
                                                     const _Float16* __restrict__ w,
@@ -153,32 +172,46 @@ __device__ __forceinline__ void rms_norm_rows_short(const _Float16* __restrict__
                                                     const _Float16* __restrict__ x2 = nullptr, int64_t x2_row_stride = 0,
                                                     const _Float16* __restrict__ w2 = nullptr, int64_t split = INT64_MAX) {
   using V = Vec16<_Float16>;
-  constexpr int RPW = 64 / LPR;
+  constexpr int RPW = 64 / LPR, U = kShortRowPasses;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int64_t row = ((int64_t)blockIdx.x * kWaves + wave) * RPW + lane / LPR;
+  const int64_t row0 = ((int64_t)blockIdx.x * kWaves + wave) * (RPW * U) + lane / LPR;
   const int32_t vi = lane % LPR;
-  const bool live = row < rows && vi < (n >> 3);
-  const bool second = row >= split;
-  V xv;
-  float ss = 0.0f;
-  if (live) {
-    const u32x4* xr = reinterpret_cast<const u32x4*>(second ? x2 + (row - split) * x2_row_stride : x + row * x_row_stride);
-    xv.raw = __builtin_nontemporal_load(xr + vi);
+  V xv[U];
+  bool live[U];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float f = (float)xv.v[e];
-      ss = __builtin_fmaf(f, f, ss);
+  for (int u = 0; u < U; ++u) {
+    const int64_t row = row0 + u * RPW;
+    live[u] = row < rows && vi < (n >> 3);
+    if (live[u]) {
+      const u32x4* xr = reinterpret_cast<const u32x4*>(row >= split ? x2 + (row - split) * x2_row_stride : x + row * x_row_stride);
+      xv[u].raw = __builtin_nontemporal_load(xr + vi);
     }
   }
+  V wq, wk;
+  if (vi < (n >> 3)) {
+    wq.raw = reinterpret_cast<const u32x4*>(w)[vi];
+    if (w2) wk.raw = reinterpret_cast<const u32x4*>(w2)[vi];
+  }
 #pragma unroll
-  for (int o = LPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-  if (!live) return;
-  const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
-  V wv, ov;
-  wv.raw = reinterpret_cast<const u32x4*>(second ? w2 : w)[vi];
+  for (int u = 0; u < U; ++u) {
+    float ss = 0.0f;
+    if (live[u]) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) ov.v[e] = (_Float16)(((float)xv.v[e] * inv) * (float)wv.v[e]);
-  __builtin_nontemporal_store(ov.raw, reinterpret_cast<u32x4*>(out + row * out_row_stride) + vi);
+      for (int e = 0; e < 8; ++e) {
+        float f = (float)xv[u].v[e];
+        ss = __builtin_fmaf(f, f, ss);
+      }
+    }
+    ss = lane_group_sum<LPR>(ss);
+    if (!live[u]) continue;
+    const int64_t row = row0 + u * RPW;
+    const float inv = __builtin_amdgcn_rsqf(ss / (float)n + eps);
+    const V& wv = row >= split ? wk : wq;
+    V ov;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ov.v[e] = (_Float16)(((float)xv[u].v[e] * inv) * (float)wv.v[e]);
+    __builtin_nontemporal_store(ov.raw, reinterpret_cast<u32x4*>(out + row * out_row_stride) + vi);
+  }
 }
 
 // add_rms_norm_f16: combined = residual + x stays in f32 registers (it is both

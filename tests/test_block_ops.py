@@ -94,12 +94,16 @@ def test_gpu_add_rms_norm(ct, dev, rows, n, variant):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n,variant", [(128, None), (64, None), (256, "w1v1"), (120, None)])
-def test_gpu_qk_norm(ct, dev, n, variant):
-    q, k = normal_f16_bits((40, n), 651), normal_f16_bits((8, n), 652)
+@pytest.mark.parametrize("n,variant,q_rows,k_rows", [
+    (128, None, 40, 8), (64, None, 40, 8), (256, "w1v1", 40, 8), (120, None, 40, 8),
+    # many workgroups, a ragged last one, the q/k boundary inside one pass of one wavefront
+    (128, None, 1003, 251), (64, None, 1001, 77), (256, None, 2050, 513), (128, "s32", 333, 90),
+])
+def test_gpu_qk_norm(ct, dev, n, variant, q_rows, k_rows):
+    q, k = normal_f16_bits((q_rows, n), 651), normal_f16_bits((k_rows, n), 652)
     qw, kw = f16(oracle.uniform_f32((n,), 653, 0.5, 1.5)), f16(oracle.uniform_f32((n,), 654, 0.5, 1.5))
-    out = torch.zeros(48, n, dtype=torch.float16, device=dev)
-    ct.qk_norm_f16(_dev(q, dev), _dev(k, dev), _dev(qw, dev), _dev(kw, dev), ct.partition(out, [1, n]), 1e-6, 40, variant=variant)
+    out = torch.zeros(q_rows + k_rows, n, dtype=torch.float16, device=dev)
+    ct.qk_norm_f16(_dev(q, dev), _dev(k, dev), _dev(qw, dev), _dev(kw, dev), ct.partition(out, [1, n]), 1e-6, q_rows, variant=variant)
     torch.cuda.synchronize()
     assert np.max(f16_ulp_diff(_bits(out), oracle.qk_norm_f16(q, k, qw, kw, 1e-6))) <= 1
 

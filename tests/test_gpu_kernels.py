@@ -182,6 +182,7 @@ def test_creation_and_convert_vector_paths_tails_and_layouts(ct, dev):
     (64, 512, None), (33, 1024, None), (16, 2048, None), (16, 4096, None), (32, 8192, None),
     (32, 8192, "w4v4"), (32, 8192, "w2v8"), (32, 8192, "w4v8"), (8, 16384, None), (8, 32768, None),
     (16, 8192, "generic"), (7, 1000, None), (5, 24, None), (4, 8, None),
+    (777, 128, None), (1500, 64, None), (515, 256, None), (300, 128, "s32"),        # short rows, ragged last workgroup
 ])
 def test_rms_norm_f16(ct, dev, rows, n, variant):
     xb = normal_f16_bits((rows, n), 101)
