@@ -63,6 +63,33 @@ __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, 
 template <int WN>
 constexpr int kEpilogueBytesPerWave = 32 * WN * 4;
 
+// An output too large to still be cached when its consumer runs is read and stored past the caches
+// (nontemporal), which leaves them to the operand panels: measured +1.8 % at 8192^3 (128 MiB of bf16),
+// -3 % at 4096^3 (32 MiB, which a following launch finds in the memory-side cache).
+constexpr int64_t kStreamedOutputBytes = 64ll << 20;
+template <typename V>
+__device__ __forceinline__ V load_z(const V* p, bool stream) {
+  V v;
+  if (stream) {
+    asm volatile("");   // as in store_z
+    v = __builtin_nontemporal_load(p);
+    asm volatile("");
+  } else {
+    v = *p;
+  }
+  return v;
+}
+template <typename V>
+__device__ __forceinline__ void store_z(V v, V* p, bool stream) {
+  if (stream) {
+    asm volatile("");   // empty statements on both sides keep the optimiser from merging the two
+    __builtin_nontemporal_store(v, p);   // stores of this branch and the next into one plain store
+    asm volatile("");
+  } else {
+    *p = v;
+  }
+}
+
 template <int TM, int TN, typename OutT>
 __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
                                                   int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
@@ -77,6 +104,7 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
   const int rd_row = lane / LANES_PER_ROW, rd_col = (lane % LANES_PER_ROW) * COLS_PER_LANE;
   const int32_t gc = wave_col0 + rd_col;
   const bool col_ok = gc < zN;
+  const bool stream = (int64_t)zM * zN * (int64_t)sizeof(OutT) >= kStreamedOutputBytes;
   const bool full = gc + COLS_PER_LANE <= zN;  // zN is a multiple of 4: otherwise exactly the first 4 columns are inside
   // Old z, all of it requested before anything is waited for.
   u32x4 old[TM][PASSES];
@@ -90,9 +118,9 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
         if (gr < zM && col_ok) {
           const OutT* src = zp + (int64_t)gr * ldz + gc;
           if (full) {
-            old[tm][pass] = *reinterpret_cast<const u32x4*>(src);
+            old[tm][pass] = load_z(reinterpret_cast<const u32x4*>(src), stream);
           } else {
-            u32x2 h = *reinterpret_cast<const u32x2*>(src);
+            u32x2 h = load_z(reinterpret_cast<const u32x2*>(src), stream);
             old[tm][pass].x = h.x;
             old[tm][pass].y = h.y;
           }
@@ -134,15 +162,15 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
           if (full) {
             u32x4 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
                        pack_bf16x2(hi[2], hi[3])};
-            *reinterpret_cast<u32x4*>(dst) = w;
+            store_z(w, reinterpret_cast<u32x4*>(dst), stream);
           } else {
             u32x2 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
-            *reinterpret_cast<u32x2*>(dst) = w;
+            store_z(w, reinterpret_cast<u32x2*>(dst), stream);
           }
         }
       } else {
         if (accumulate) lo += __builtin_bit_cast(f32x4, o);
-        if (gr < zM && col_ok) *reinterpret_cast<f32x4*>(zp + (int64_t)gr * ldz + gc) = lo;
+        if (gr < zM && col_ok) store_z(lo, reinterpret_cast<f32x4*>(zp + (int64_t)gr * ldz + gc), stream);
       }
     }
   }
