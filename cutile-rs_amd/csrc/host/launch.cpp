@@ -135,6 +135,10 @@ cutile_status_t launch_packed(hipFunction_t fn, const uint32_t grid[3], const ui
   CUTILE_API_OR_RETURN(api);
   CUTILE_REQUIRE(grid[0] > 0 && grid[1] > 0 && grid[2] > 0, CUTILE_ERR_KERNEL_LAUNCH,
                  "launch grid (%u, %u, %u) has a zero axis", grid[0], grid[1], grid[2]);
+  // what one dispatch can express: 2^31 - 1 workgroups on x, 65535 on y and z, fewer than 2^32 lanes per axis
+  CUTILE_REQUIRE(grid[0] <= 0x7fffffffu && grid[1] <= 65535u && grid[2] <= 65535u &&
+                     (uint64_t)grid[0] * block[0] <= 0xffffffffull,
+                 CUTILE_ERR_KERNEL_LAUNCH, "launch grid (%u, %u, %u) exceeds what one dispatch can hold", grid[0], grid[1], grid[2]);
   size_t size = args.buf.size();
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.buf.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                    HIP_LAUNCH_PARAM_END};
@@ -261,9 +265,9 @@ cutile_dtype_t cutile_dtype_from_name(const char* name) {
 cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t grid[3]) {
   CUTILE_REQUIRE(p && grid, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
   const cutile_tensor_arg_t& t = p->tensor;
+  CUTILE_REQUIRE(t.rank >= 1 && t.rank <= 3, CUTILE_ERR_TENSOR, "Mutable tensor must be at most rank 3.");
   for (int i = 0; i < t.rank; ++i)
     CUTILE_REQUIRE(t.shape[i] > 0, CUTILE_ERR_TENSOR, "Shape dimensions must be positive.");
-  CUTILE_REQUIRE(t.rank >= 1 && t.rank <= 3, CUTILE_ERR_TENSOR, "Mutable tensor must be at most rank 3.");
   grid[0] = grid[1] = grid[2] = 1;
   for (int i = 0; i < t.rank; ++i) {
     CUTILE_REQUIRE(p->partition_shape[i] > 0, CUTILE_ERR_TENSOR, "partition shape must be positive");
@@ -274,7 +278,7 @@ cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t 
 
 cutile_status_t cutile_infer_launch_grid(const uint32_t explicit_grid[3], const cutile_partition_arg_t* const* partitions,
                                          int32_t n_partitions, uint32_t grid[3]) {
-  CUTILE_REQUIRE(grid, CUTILE_ERR_INVALID_ARGUMENT, "grid is null");
+  CUTILE_REQUIRE(grid && (partitions || n_partitions <= 0), CUTILE_ERR_INVALID_ARGUMENT, "null argument");
   struct Bound { uint32_t g[3]; bool exact; };
   std::vector<Bound> bounds;
   for (int i = 0; i < n_partitions; ++i) {
