@@ -546,9 +546,48 @@ class DecodeAttentionWide(DecodeAttention):
                           "131072 cached keys, 32 KV splits (one workgroup per CU), BN 64 (two launches per step)"}
 
 
+class PrefillAttention(Workload):
+    """fmha_prefill_causal (cutile-kernels/src/attention.rs:242-391): f16, [seq, heads, D] queries against a
+    [kv_heads, seq, D] cache, grouped heads; flops counted like the causal FMHA bench (half of 4 s^2 d per head)."""
+    name, unit, bound, peak_key = "prefill_attention_f16_s8192_h32g4_d128", "TFLOP/s", "mfma", "mfma_bf16"
+    dtype = "f16 io / f32 softmax+acc"
+    s, heads, group, d = 8192, 32, 4, 128
+    work = 2.0 * s * s * d * heads
+    config = {"workload": "fmha_prefill_causal fp16: q [8192, 32, 128], k/v [8, 8192, 128] (GROUP 4), causal, query_start 0, "
+                          "scale 1/sqrt(128)", "tile": "BM=256"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        kvh = self.heads // self.group
+        f16 = lambda a: a.astype(np.float16)
+        self.qh = f16(oracle.normal_f32((self.s, self.heads, self.d), 41))
+        self.kh, self.vh = f16(oracle.normal_f32((kvh, self.s, self.d), 42)), f16(oracle.normal_f32((kvh, self.s, self.d), 43))
+        self.q, self.k, self.v = (torch.from_numpy(t).to(dev) for t in (self.qh, self.kh, self.vh))
+        self.o = torch.zeros(self.s, self.heads, self.d, dtype=torch.float16, device=dev)
+        self.op = ct.partition(self.o, [128, 1, self.d])
+
+    def launch(self):
+        self.ct.fmha_seq_f16(self.q, self.k, self.v, self.op, self.d ** -0.5, self.group, kv_len=self.s, query_start=0, causal=True)
+
+    def cpu_baseline(self, oracle, np, torch):
+        # the first 1024 queries of the same problem see the first 1024 keys only: a self-contained sub-problem
+        n = 1024
+        q, k, v = self.qh[:n].astype(np.float32), self.kh[:, :n].astype(np.float32), self.vh[:, :n].astype(np.float32)
+        t0 = time.perf_counter()
+        ref = oracle.attention_seq_ref(q, k, v, self.d ** -0.5, self.group, n, 0, True)
+        dt = time.perf_counter() - t0
+        err = float(np.max(np.abs(self.o[:n].float().cpu().numpy() - ref)))
+        flops = 2.0 * n * n * self.d * self.heads
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"the first {n} of {self.s} queries (they see the first {n} keys only)"}, \
+               {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
+
+
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

@@ -128,6 +128,8 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_fmha_seq_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), f32, i32, i32, i32,
+                                           P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
                                                 P(TensorArg), f32, P(LaunchOpts)],
             "cutile_launch_linear_tile_nvfp4": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
@@ -470,6 +472,24 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def fmha_seq_f16(q, k, v, out: Partition, qk_scale: float, query_group_size: int, *, kv_len: int = 0, query_start: int = 0,
+                 position_start=None, kv_len_from_position: bool = False, causal: bool = True, stream=None, grid=None,
+                 generics=None, variant=None) -> None:
+    """The sequence-layout attention kernels of cutile-kernels/src/attention.rs (q, out [q_len, q_heads, D]; k, v
+    [kv_heads, max_seq, D]; out tiles [BM, G, D]):
+      flash_attn_causal_seq_f16 (:21-116)         kv_len, query_start by value, causal
+      flash_attn_causal_seq_dynpos_f16 (:128-231) position_start (one u32 on the device), kv_len_from_position
+      fmha_prefill_causal (:242-391), fmha_prefill_gqa (:408-587)   kv_len, query_start by value, causal or not
+      fmha_causal (:598-726)                      position_start, every key of k"""
+    o, _k = _opts(grid, generics, variant)
+    qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
+    pa = tensor_arg(position_start, dtype=U32) if position_start is not None else None
+    check(lib().cutile_launch_fmha_seq_f16(_stream(stream), C.byref(qa), C.byref(ka), C.byref(va), C.byref(out.arg()),
+                                           C.c_float(qk_scale), int(query_group_size), int(kv_len), int(query_start),
+                                           C.byref(pa) if pa is not None else None, int(kv_len_from_position), int(causal),
+                                           C.byref(o)))
 
 
 def linear_tile_mxfp8(z: Partition, x, y, x_scales, y_scales, alpha: float = 1.0, *, stream=None, grid=None,

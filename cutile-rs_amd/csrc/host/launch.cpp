@@ -1298,6 +1298,118 @@ cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partitio
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// Sequence-layout attention: q / out [q_len, q_heads, D] and k / v [kv_heads, max_seq, D] are handed to the
+// (batch, head, row, d) kernels as permuted views (batch 1, head stride D, row stride q_heads * D); the
+// kernel tile is chosen here, whatever BM the caller's partition names, because the output does not depend on it.
+cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                           const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                           const cutile_partition_arg_t* out, float qk_scale,
+                                           int32_t query_group_size, int32_t kv_len, int32_t query_start,
+                                           const cutile_tensor_arg_t* position_start, int32_t kv_len_from_position,
+                                           int32_t causal, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(q, "q", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(k, "k", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(v, "v", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 3, 3)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE(q->dtype == CUTILE_DTYPE_F16 && k->dtype == CUTILE_DTYPE_F16 && v->dtype == CUTILE_DTYPE_F16 &&
+                     ot.dtype == CUTILE_DTYPE_F16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "sequence attention: q, k, v and out must be f16");
+  const int32_t q_len = q->shape[0], q_heads = q->shape[1], d = q->shape[2], kv_heads = k->shape[0];
+  const int32_t max_seq = std::min(k->shape[1], v->shape[1]);
+  CUTILE_REQUIRE(k->shape[2] == d && v->shape[2] == d && v->shape[0] == kv_heads && ot.shape[2] == d &&
+                     ot.shape[0] <= q_len && ot.shape[1] <= q_heads,
+                 CUTILE_ERR_KERNEL_LAUNCH, "sequence attention: q/out [q_len, q_heads, D] and k/v [kv_heads, kv_len, D] do not agree");
+  CUTILE_REQUIRE(query_group_size > 0 && (int64_t)kv_heads * query_group_size == q_heads, CUTILE_ERR_KERNEL_LAUNCH,
+                 "sequence attention: %d query heads, %d kv heads, query_group_size %d do not agree", q_heads, kv_heads,
+                 query_group_size);
+  const int32_t bm = out->partition_shape[0], pack = out->partition_shape[1];
+  CUTILE_REQUIRE(out->partition_shape[2] == d && pack > 0 && query_group_size % pack == 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "sequence attention: out must be partitioned [BM, G, %d] with G dividing query_group_size = %d, got [%d, %d, %d]",
+                 d, query_group_size, bm, pack, out->partition_shape[2]);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(d), "D")) return s;
+  if (position_start) {
+    if (cutile_status_t s = check_tensor(position_start, "position_start", 1, 1)) return s;
+    CUTILE_REQUIRE(position_start->dtype == CUTILE_DTYPE_U32 && position_start->shape[0] == 1 &&
+                       ((uintptr_t)position_start->ptr & 3) == 0,
+                   CUTILE_ERR_KERNEL_LAUNCH, "sequence attention: position_start must be one aligned u32");
+    if (!kv_len_from_position) kv_len = max_seq;
+  } else {
+    CUTILE_REQUIRE(query_start >= 0 && kv_len >= 0 && kv_len <= max_seq, CUTILE_ERR_KERNEL_LAUNCH,
+                   "sequence attention: query_start = %d and kv_len = %d must be non-negative and kv_len within the %d rows of k and v",
+                   query_start, kv_len, max_seq);
+  }
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  auto rows_ok = [&](const cutile_tensor_arg_t& t) {
+    return t.strides[2] == 1 && t.strides[0] % 8 == 0 && t.strides[1] % 8 == 0 && aligned16(t.ptr);
+  };
+  CUTILE_REQUIRE(rows_ok(*q) && rows_ok(*k) && rows_ok(*v) && rows_ok(ot), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "sequence attention: precompiled variants need unit head-dim stride and 16-byte aligned rows");
+  // what the launch covers: rows 0 .. rows_cov and heads 0 .. heads_cov of out
+  const int32_t rows_cov = (int32_t)std::min<int64_t>((int64_t)tg[0] * bm, ot.shape[0]);
+  const int32_t heads_cov = (int32_t)std::min<int64_t>((int64_t)tg[1] * pack, ot.shape[1]);
+  // views in the kernels' (batch, head, row, d) order
+  cutile_tensor_arg_t qv{}, kv{}, vv{};
+  qv.ptr = q->ptr; qv.dtype = q->dtype; qv.rank = 4;
+  qv.shape[0] = 1; qv.shape[1] = q_heads; qv.shape[2] = rows_cov; qv.shape[3] = d;
+  qv.strides[0] = 0; qv.strides[1] = q->strides[1]; qv.strides[2] = q->strides[0]; qv.strides[3] = 1;
+  auto kv_view = [&](const cutile_tensor_arg_t& t, cutile_tensor_arg_t* o) {
+    o->ptr = t.ptr; o->dtype = t.dtype; o->rank = 4;
+    o->shape[0] = 1; o->shape[1] = kv_heads; o->shape[2] = position_start ? max_seq : kv_len; o->shape[3] = d;
+    o->strides[0] = 0; o->strides[1] = t.strides[0]; o->strides[2] = t.strides[1]; o->strides[3] = 1;
+  };
+  kv_view(*k, &kv);
+  kv_view(*v, &vv);
+  cutile_partition_arg_t ov{};
+  ov.tensor.ptr = ot.ptr; ov.tensor.dtype = ot.dtype; ov.tensor.rank = 3;
+  ov.tensor.shape[0] = heads_cov; ov.tensor.shape[1] = rows_cov; ov.tensor.shape[2] = d;
+  ov.tensor.strides[0] = ot.strides[1]; ov.tensor.strides[1] = ot.strides[0]; ov.tensor.strides[2] = 1;
+  // kernel tile: the ping-pong kernel for long D = 128 prefills, else the largest tile of that D
+  const char* function = position_start ? "fmha_seq" : "fmha";
+  std::vector<const KernelEntry*> fit;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, function) == 0 && strcmp(e.dtype, "f16") == 0 && e.tile[2] == d) fit.push_back(&e);
+  CUTILE_REQUIRE(!fit.empty(), CUTILE_ERR_KERNEL_NOT_FOUND, "no precompiled sequence attention for f16, D = %d; available: %s", d,
+                 list_variants(function).c_str());
+  const bool long_prefill = rows_cov >= 256 && kv_len > 0;
+  std::stable_sort(fit.begin(), fit.end(), [&](const KernelEntry* a, const KernelEntry* b) {
+    const bool pa = strstr(a->variant, "_pp") != nullptr, pb = strstr(b->variant, "_pp") != nullptr;
+    if (pa != pb) return long_prefill ? pa : pb;
+    return a->tile[0] > b->tile[0];
+  });
+  std::vector<std::string> acceptable;
+  for (auto* e : fit)
+    if (kv_len > 0 || strstr(e->variant, "_pp") == nullptr) acceptable.push_back(e->variant);   // an empty key range: the plain kernels only
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry(function, &o, acceptable[0], acceptable, &res)) return s;
+  const int32_t kbm = res.entry->tile[0];
+  ov.partition_shape[0] = 1; ov.partition_shape[1] = kbm; ov.partition_shape[2] = d;
+  for (int i = 0; i < 3; ++i) ov.partition_strides[i] = ov.tensor.strides[i];
+  const uint32_t kg[3] = {(uint32_t)heads_cov, div_up((uint64_t)rows_cov, (uint64_t)kbm), 1};
+  ArgPacker args;
+  args.push_partition(ov);
+  args.push_tensor(qv);
+  args.push_tensor(kv);
+  args.push_tensor(vv);
+  args.push_val<float>(qk_scale);
+  if (position_start) {
+    args.push_val<const void*>(position_start->ptr);
+    args.push_val<int32_t>(kv_len_from_position ? 1 : 0);
+  } else {
+    args.push_val<int32_t>(query_start);
+  }
+  args.push_val<int32_t>(query_group_size);
+  args.push_val<int32_t>(causal ? 1 : 0);
+  args.push_tile_grid(kg);
+  uint32_t grid[3] = {kg[0], kg[1], 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                                 const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                                 const cutile_tensor_arg_t* xs, const cutile_tensor_arg_t* ys, float alpha,

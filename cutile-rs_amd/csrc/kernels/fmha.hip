@@ -48,6 +48,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// Bytes from the first element of row 0 to the last of row rows - 1 (16-bit elements, `row_stride`
+// elements apart, `d` per row); nothing for an empty range, so that every access is out of range.
+__device__ __forceinline__ uint32_t rows_extent_bytes(int32_t rows, int32_t row_stride, int32_t d) {
+  return rows > 0 ? (uint32_t)(((int64_t)(rows - 1) * row_stride + d) * 2) : 0u;
+}
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
@@ -158,9 +163,9 @@ struct Fmha {
     const T* kb = (const T*)k.ptr + (int64_t)batch * k.strides[0] + (int64_t)kv_head * k.strides[1];
     const T* vb = (const T*)v.ptr + (int64_t)batch * v.strides[0] + (int64_t)kv_head * v.strides[1];
     const int32_t q_ld = q.strides[2], k_ld = k.strides[2], v_ld = v.strides[2];
-    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qb, (uint32_t)(((int64_t)(q_len - 1) * q_ld + D) * 2));
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kb, (uint32_t)(((int64_t)(k_len - 1) * k_ld + D) * 2));
-    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vb, (uint32_t)(((int64_t)(k_len - 1) * v_ld + D) * 2));
+    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qb, rows_extent_bytes(q_len, q_ld, D));
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kb, rows_extent_bytes(k_len, k_ld, D));
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vb, rows_extent_bytes(k_len, v_ld, D));
     constexpr uint32_t kOob = 0x80000000u;
 
     // Qᵀ operand: lane holds query row q0 + l32, d = ks*16 + half*8 .. +7.
@@ -325,6 +330,9 @@ struct Fmha {
     }
 
     // out[bh, q, d] = acc / l.  o_acc[db][e]: d = db*32 + (e/4)*8 + half*4 + e%4.
+    // A row that saw no key at all (an empty key range) has l = 0 and becomes 0, as in the
+    // production kernels (l_safe = max(l, 1e-8), cutile-kernels/src/attention.rs:383-386); any other row has l >= 1.
+    l_i = fmaxf(l_i, 1.0e-8f);
     const int32_t qr = q0 + l32;
     if (qr < out.shape[1] && qr < q_len) {
       T* orow = (T*)out.ptr + (int64_t)bh * out.strides[0] + (int64_t)qr * out.strides[1];
@@ -406,9 +414,9 @@ struct FmhaPingPong {
     const T* kb = (const T*)k.ptr + (int64_t)batch * k.strides[0] + (int64_t)kv_head * k.strides[1];
     const T* vb = (const T*)v.ptr + (int64_t)batch * v.strides[0] + (int64_t)kv_head * v.strides[1];
     const int32_t q_ld = q.strides[2], k_ld = k.strides[2], v_ld = v.strides[2];
-    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qb, (uint32_t)(((int64_t)(q_len - 1) * q_ld + D) * 2));
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kb, (uint32_t)(((int64_t)(k_len - 1) * k_ld + D) * 2));
-    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vb, (uint32_t)(((int64_t)(k_len - 1) * v_ld + D) * 2));
+    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qb, rows_extent_bytes(q_len, q_ld, D));
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kb, rows_extent_bytes(k_len, k_ld, D));
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vb, rows_extent_bytes(k_len, v_ld, D));
     constexpr uint32_t kOob = 0x80000000u;
 
     vec8 qf[KS];
@@ -648,7 +656,7 @@ struct FmhaPingPong {
     // out[bh, q, d] = acc / l through LDS: this wavefront's 32 rows x D as T, 16-byte
     // chunk c of row r at chunk c ^ (r & 15); then whole rows leave as 16-byte stores.
     unsigned char* band = (wave < 2 ? kb0 : wave < 4 ? kb1 : wave < 6 ? vb0 : vb1) + (wave & 1) * (32 * D * 2);
-    const float inv_l = 1.0f / l_i;
+    const float inv_l = 1.0f / fmaxf(l_i, 1.0e-8f);   // l = 0 only for an empty key range: the row becomes 0
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -1256,6 +1264,27 @@ FMHA_KERNEL(bf16, __bf16, 32, 32, 32)
 FMHA_KERNEL(f16, _Float16, 128, 64, 128)
 FMHA_KERNEL(f16, _Float16, 128, 64, 64)
 FMHA_KERNEL(f16, _Float16, 32, 32, 32)
+
+// The sequence-layout attention kernels of cutile-kernels whose position lives in device memory
+// (flash_attn_causal_seq_dynpos_f16 attention.rs:128-231, fmha_causal :598-726): q and out
+// [q_len, q_heads, D], k and v [kv_heads, max_seq, D], handed over as permuted views of the layout
+// above.  query_start = *position_start; with `kv_len_from_position` only keys 0 .. position are read
+// (the dynpos form), otherwise every key of the view.
+#define FMHA_SEQ_KERNEL(NAME, T, BM, BN, D)                                                       \
+  extern "C" __global__ void __launch_bounds__((BM / 32) * 64)                                   \
+      fmha_seq_entry__##NAME##_##BM##x##BN##x##D(PartitionArg<3> out, TensorArg<4> q, TensorArg<4> k, \
+                                                 TensorArg<4> v, float qk_scale,                  \
+                                                 const uint32_t* position_start,                  \
+                                                 int32_t kv_len_from_position,                    \
+                                                 int32_t query_group_size, int32_t causal, TileGrid g) { \
+    const int32_t pos = (int32_t)min(position_start[0], 0x3fffffffu);                             \
+    TensorArg<4> kk = k, vv = v;                                                                  \
+    if (kv_len_from_position) kk.shape[2] = vv.shape[2] = min(min(k.shape[2], v.shape[2]), pos + 1); \
+    Fmha<T, BM, BN, D>::run(out, q, kk, vv, qk_scale, pos, query_group_size, causal, g);         \
+  }
+FMHA_SEQ_KERNEL(f16, _Float16, 128, 64, 128)
+FMHA_SEQ_KERNEL(f16, _Float16, 128, 64, 64)
+FMHA_SEQ_KERNEL(f16, _Float16, 32, 32, 32)
 
 #define FMHA_PINGPONG_KERNEL(NAME, T, BN, D)                                                       \
   extern "C" __global__ void __launch_bounds__(512)                                               \

@@ -467,6 +467,27 @@ struct SplitkReduceMergeFn {
     return cutile_launch_splitk_reduce_merge(s, &aa, &la, &op, o);
   }
 };
+// The five sequence-layout attention kernels share one C entry point (cutile_launch_fmha_seq_f16).
+template <bool Causal>
+struct SeqAttentionFn {          // kv_len and query_start by value
+  template <class Q, class K, class V, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, O& out, float qk_scale,
+                                int32_t query_group_size, int32_t kv_len, int32_t query_start) {
+    auto qa = input_arg(q), ka = input_arg(k), va = input_arg(v);
+    auto op = out.arg();
+    return cutile_launch_fmha_seq_f16(s, &qa, &ka, &va, &op, qk_scale, query_group_size, kv_len, query_start, nullptr, 0, Causal, o);
+  }
+};
+template <bool Causal, bool KvLenFromPosition>
+struct SeqAttentionDynposFn {    // the position in device memory
+  template <class Q, class K, class V, class O, class P>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, O& out, float qk_scale,
+                                int32_t query_group_size, P& position_start) {
+    auto qa = input_arg(q), ka = input_arg(k), va = input_arg(v), pa = input_arg(position_start);
+    auto op = out.arg();
+    return cutile_launch_fmha_seq_f16(s, &qa, &ka, &va, &op, qk_scale, query_group_size, 0, 0, &pa, KvLenFromPosition, Causal, o);
+  }
+};
 struct GemmPersistentFn {
   template <class Z, class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y) {
@@ -525,6 +546,16 @@ template <class NK, class NV, class KC, class VC, class P> auto kv_cache_update_
 template <class Q, class K, class V, class A, class L, class P> auto fmha_decode_gqa_split(Q&& q, K&& k, V&& v, A&& att_out, L&& lse_out, float qk_scale, P&& position_start) { return make_launcher<kernels::FmhaDecodeGqaSplitFn>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<A>(att_out), std::forward<L>(lse_out), qk_scale, std::forward<P>(position_start)); }
 // splitk_reduce_merge(att_partial, lse_partial, out: [1,GROUP,CHUNK_D])          attention.rs:917-930
 template <class A, class L, class O> auto splitk_reduce_merge(A&& att_partial, L&& lse_partial, O&& out) { return make_launcher<kernels::SplitkReduceMergeFn>(std::forward<A>(att_partial), std::forward<L>(lse_partial), std::forward<O>(out)); }
+// flash_attn_causal_seq_f16(q, k, v, out: [BM,1,D], qk_scale, query_group_size, kv_len, query_start)   attention.rs:21-30
+template <class Q, class K, class V, class O> auto flash_attn_causal_seq_f16(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, int32_t kv_len, int32_t query_start) { return make_launcher<kernels::SeqAttentionFn<true>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, kv_len, query_start); }
+// flash_attn_causal_seq_dynpos_f16(q, k, v, out: [BM,1,D], qk_scale, query_group_size, position_start: [1] u32)   attention.rs:128-136
+template <class Q, class K, class V, class O, class P> auto flash_attn_causal_seq_dynpos_f16(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, P&& position_start) { return make_launcher<kernels::SeqAttentionDynposFn<true, true>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, std::forward<P>(position_start)); }
+// fmha_prefill_causal<.., CAUSAL, ..>(q, k, v, out: [BM,1,D], qk_scale, query_group_size, kv_len, query_start)   attention.rs:242-263
+template <bool CAUSAL = true, class Q, class K, class V, class O> auto fmha_prefill_causal(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, int32_t kv_len, int32_t query_start) { return make_launcher<kernels::SeqAttentionFn<CAUSAL>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, kv_len, query_start); }
+// fmha_prefill_gqa<.., GROUP, M_EFF, CAUSAL, ..>(q, k, v, out: [BM,GROUP,D], qk_scale, query_group_size, kv_len, query_start)   attention.rs:408-432
+template <bool CAUSAL = true, class Q, class K, class V, class O> auto fmha_prefill_gqa(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, int32_t kv_len, int32_t query_start) { return make_launcher<kernels::SeqAttentionFn<CAUSAL>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, kv_len, query_start); }
+// fmha_causal<.., CAUSAL, ..>(q, k, v, out: [BM,1,D], qk_scale (the f16 value, widened), query_group_size, position_start: [1] u32)   attention.rs:598-612
+template <bool CAUSAL = true, class Q, class K, class V, class O, class P> auto fmha_causal(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, P&& position_start) { return make_launcher<kernels::SeqAttentionDynposFn<CAUSAL, false>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, std::forward<P>(position_start)); }
 // gemm_persistent(z: mapped partition [BM,BN], x, y) -> (z's partition, x, y)   cutile-examples/examples/persistent_gemm.rs:35-45
 template <class Z, class X, class Y> auto gemm_persistent(Z&& z, X&& x, Y&& y) { return make_launcher<kernels::GemmPersistentFn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y)); }
 // write_flat_index_rank{1,2,3}(z: mapped i32 partition) -> (z's partition)      cutile/tests/gpu/mapped_partition_schedule_matrix.rs:30-76

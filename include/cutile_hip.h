@@ -427,6 +427,28 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* The sequence-layout attention kernels of cutile-kernels, one entry point for the five of them:
+ *   flash_attn_causal_seq_f16<BM,BN,D>(q, k, v, out, qk_scale, query_group_size, kv_len, query_start)
+ *       cutile-kernels/src/attention.rs:21-116   -> position_start = NULL, causal = 1
+ *   flash_attn_causal_seq_dynpos_f16<BM,BN,D>(.., query_group_size, position_start)
+ *       attention.rs:128-231  -> position_start given, kv_len_from_position = 1, causal = 1
+ *   fmha_prefill_causal<BM,BN,D,CAUSAL,EVEN_K,LATENCY>(.., kv_len, query_start)
+ *       attention.rs:242-391  -> position_start = NULL
+ *   fmha_prefill_gqa<BM,BN,D,GROUP,M_EFF,CAUSAL,EVEN_K,LATENCY>(..)   (out tiles [BM, GROUP, D])
+ *       attention.rs:408-587  -> position_start = NULL
+ *   fmha_causal<BM,BN,D,CAUSAL,EVEN_K>(.., qk_scale: f16, query_group_size, position_start)
+ *       attention.rs:598-726  -> position_start given, kv_len_from_position = 0, kv_len = dim(k, 1)
+ * q and out are [q_len, q_heads, D], k and v [kv_heads, max_seq, D], all f16; out is partitioned
+ * [BM, G, D] with G = 1 or the packing factor of the gqa form.  Query i of the launch stands at position
+ * query_start + i (by value, or *position_start: one u32 in device memory); it attends to keys j < kv_len
+ * and, when causal, j <= its position.  Rows without any key are written as zeros (l_safe = max(l, 1e-8)).
+ * Generics, when given, are checked at index 0 (BM) and 2 (D). */
+cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                           const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                           const cutile_partition_arg_t* out, float qk_scale,
+                                           int32_t query_group_size, int32_t kv_len, int32_t query_start,
+                                           const cutile_tensor_arg_t* position_start, int32_t kv_len_from_position,
+                                           int32_t causal, const cutile_launch_opts_t* opts);
 /* fmha<BM, BN, D, H, CAUSAL, EVEN_K>(out: [1,BM,D] tiles, q, k, v, qk_scale,
  * input_pos, query_group_size) — cutile-examples/examples/flash_attention_causal.rs:19-134,
  * cutile-benchmarks/benches/fmha.rs:20-145 (non-causal: causal = 0, input_pos = 0) */

@@ -74,6 +74,7 @@ def lib() -> C.CDLL:
             "orc_gemm_bf16": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_gemm_bf16_f32out": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_fmha_ref_cpu": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp, i64]),
+            "orc_attention_seq_ref": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, i64, C.c_int]),
             "orc_mx_quantize_e4m3": (None, [vp, vp, vp, i64, i64]),
             "orc_mx_dequantize_e4m3": (None, [vp, vp, vp, i64, i64]),
             "orc_mx_gemm_f32": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, vp, i64]),
@@ -368,6 +369,19 @@ def fmha_ref_cpu(q, k, v, qk_scale: float, input_pos: int = 0, query_group_size:
     out = np.empty((nr, d) if rows is not None else (b, h, m, d), np.float32)
     lib().orc_fmha_ref_cpu(_p(q), _p(k), _p(v), _p(out), b, h, hkv, m, d, qk_scale, input_pos,
                            query_group_size, int(causal), rp, nr)
+    return out
+
+
+def attention_seq_ref(q, k, v, qk_scale: float, query_group_size: int, kv_len: int, query_start: int = 0,
+                      causal: bool = True) -> np.ndarray:
+    """q [q_len, q_heads, D], k and v [kv_heads, max_seq, D] -> out [q_len, q_heads, D] (f32)"""
+    q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
+    q_len, q_heads, d = q.shape
+    kv_heads, max_seq, _ = k.shape
+    assert v.shape == k.shape and kv_heads * query_group_size == q_heads
+    out = np.empty((q_len, q_heads, d), np.float32)
+    lib().orc_attention_seq_ref(_p(q), _p(k), _p(v), _p(out), q_len, q_heads, kv_heads, max_seq, d, qk_scale,
+                                query_group_size, int(kv_len), int(query_start), int(causal))
     return out
 
 

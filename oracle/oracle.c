@@ -598,6 +598,54 @@ void orc_fmha_ref_cpu(const float* q, const float* k, const float* v, float* out
   }
 }
 
+/* The sequence-layout attention kernels of cutile-kernels/src/attention.rs: flash_attn_causal_seq_f16 (:21-116) and
+ * its dynpos form (:128-231), fmha_prefill_causal (:242-391), fmha_prefill_gqa (:408-587), fmha_causal (:598-726).
+ * q, out [q_len, q_heads, d]; k, v [kv_heads, max_seq, d].  Query i stands at position query_start + i (:44-49) and
+ * key j counts iff j < kv_len and (not causal or position >= j) (:83-88); kv head = q head / query_group_size (:34);
+ * scores are q.k * qk_scale, weights exp(score - max) / max(sum, 1e-8) (:90-110), so a query without any key gets zeros.
+ * The kernels stream the keys in tiles with a running maximum; evaluated here over the whole row at once, which is
+ * the same function. */
+void orc_attention_seq_ref(const float* q, const float* k, const float* v, float* out, int64_t q_len,
+                           int64_t q_heads, int64_t kv_heads, int64_t max_seq, int64_t dsz, float qk_scale,
+                           int64_t query_group_size, int64_t kv_len, int64_t query_start, int causal) {
+  (void)kv_heads;
+  if (kv_len > max_seq) kv_len = max_seq;
+#pragma omp parallel
+  {
+    float* scores = (float*)malloc(sizeof(float) * (size_t)(kv_len > 0 ? kv_len : 1));
+#pragma omp for schedule(dynamic, 16)
+    for (int64_t g = 0; g < q_len * q_heads; g++) {
+      int64_t i = g / q_heads, h = g % q_heads;
+      int64_t kv_h = h / query_group_size;
+      const float* qrow = q + (i * q_heads + h) * dsz;
+      const float* kb = k + kv_h * max_seq * dsz;
+      const float* vb = v + kv_h * max_seq * dsz;
+      float* o = out + (i * q_heads + h) * dsz;
+      int64_t n = kv_len;
+      if (causal && query_start + i + 1 < n) n = query_start + i + 1;   /* keys 0 .. position */
+      float max_logit = -INFINITY;
+      for (int64_t j = 0; j < n; j++) {
+        float dot = 0.0f;
+        for (int64_t dd = 0; dd < dsz; dd++) dot += qrow[dd] * kb[j * dsz + dd];
+        scores[j] = dot * qk_scale;
+        max_logit = fmaxf(max_logit, scores[j]);
+      }
+      float denom = 0.0f;
+      for (int64_t j = 0; j < n; j++) {
+        scores[j] = expf(scores[j] - max_logit);
+        denom += scores[j];
+      }
+      denom = fmaxf(denom, 1.0e-8f);
+      for (int64_t dd = 0; dd < dsz; dd++) {
+        float val = 0.0f;
+        for (int64_t j = 0; j < n; j++) val += scores[j] * vb[j * dsz + dd];
+        o[dd] = val / denom;
+      }
+    }
+    free(scores);
+  }
+}
+
 /* ------------------------------------------------------------------------ */
 /* K6                                                                        */
 /* ------------------------------------------------------------------------ */

@@ -42,6 +42,15 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_attention_seq_ref
+ *                        the five sequence-layout attention kernels of
+ *                        cutile-kernels/src/attention.rs:21-726 (kernel bodies).  Pinned by
+ *                        orc_fmha_ref_cpu (pinned above) where the two coincide (kv_len =
+ *                        q_len, permuted layout), a float64 evaluation with an explicit mask,
+ *                        row 0 = V[0], zero queries = mean of the visible V rows, empty key
+ *                        range = 0.
+ *                        The reference only compiles these kernels: parity unpinned by
+ *                        reference tests.
  *   orc_nvfp4_*          cutile-examples/examples/nvfp4.rs:24-78 (layout, formula),
  *                        cuda-core/src/dtype.rs:60-99 (low nibble first), :228 (0x2 = 1.0).
  *                        Pinned by the reference's all-ones known answer (z = K), the
@@ -113,6 +122,10 @@ void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, i
 void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
                              uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
                              int64_t position_start, int64_t seq_len);
+/* the five sequence-layout attention kernels: cutile-kernels/src/attention.rs:21-726 */
+void orc_attention_seq_ref(const float* q, const float* k, const float* v, float* out, int64_t q_len,
+                           int64_t q_heads, int64_t kv_heads, int64_t max_seq, int64_t dsz, float qk_scale,
+                           int64_t query_group_size, int64_t kv_len, int64_t query_start, int causal);
 /* fmha_decode_gqa_split / splitk_reduce_merge: cutile-kernels/src/attention.rs:737-902, 917-1013 */
 void orc_fmha_decode_gqa_split(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                uint16_t* att_out, float* lse_out, int64_t kv_heads, int64_t group,

@@ -148,6 +148,42 @@ TEST(decode_kernels_closed_forms) {
   CHECK(!r.is_ok());
 }
 
+TEST(sequence_attention_launchers_closed_forms) {
+  // every value row is 2.0: the weights sum to one, so each of the five kernels returns 2.0 whatever the scores;
+  // with no key in range (kv_len = 0) the production kernels return zeros
+  auto stream = new_stream();
+  const int q_len = 40, q_heads = 8, kv_heads = 2, d = 128, max_seq = 96, group = q_heads / kv_heads;
+  auto q = api::full<f16>(0.25, {q_len, q_heads, d}).sync_on(stream).unwrap();
+  auto k = api::full<f16>(0.5, {kv_heads, max_seq, d}).sync_on(stream).unwrap();
+  auto v = api::full<f16>(2.0, {kv_heads, max_seq, d}).sync_on(stream).unwrap();
+  auto pos = api::full<uint32_t>(50, {1}).sync_on(stream).unwrap();
+  auto all_equal = [&](Tensor<f16>& t, float want) {
+    for (f16 x : api::to_host_vec(t).sync_on(stream).unwrap())
+      if (f32_from_f16(x) != want) return false;
+    return true;
+  };
+  auto out = api::zeros<f16>({q_len, q_heads, d}).sync_on(stream).unwrap();
+  {
+    auto [q_, k_, v_, o_, scale, g, kv_len, start] =
+        flash_attn_causal_seq_f16(&q, &k, &v, out.partition_mut({16, 1, d}), 0.0884f, group, 90, 50).generics({"16", "32", "128"}).sync_on(stream).unwrap();
+    CHECK(g == group && kv_len == 90 && start == 50 && scale == 0.0884f);      // arguments come back in signature order
+  }
+  CHECK(all_equal(out, 2.0f));
+  CHECK(fmha_prefill_causal<false>(&q, &k, &v, out.partition_mut({16, 1, d}), 0.0884f, group, 0, 0).sync_on(stream).is_ok());
+  CHECK(all_equal(out, 0.0f));
+  CHECK(fmha_prefill_gqa(&q, &k, &v, out.partition_mut({8, group, d}), 0.0884f, group, 96, 56).sync_on(stream).is_ok());
+  CHECK(all_equal(out, 2.0f));
+  auto q1 = api::full<f16>(0.25, {1, q_heads, d}).sync_on(stream).unwrap();
+  auto o1 = api::zeros<f16>({1, q_heads, d}).sync_on(stream).unwrap();
+  CHECK(flash_attn_causal_seq_dynpos_f16(&q1, &k, &v, o1.partition_mut({1, 1, d}), 0.0884f, group, &pos).sync_on(stream).is_ok());
+  CHECK(all_equal(o1, 2.0f));
+  CHECK(api::full<f16>(0.0, {1, q_heads, d}).sync_on(stream).is_ok());
+  CHECK(fmha_causal(&q1, &k, &v, o1.partition_mut({1, 1, d}), 0.0884f, group, &pos).sync_on(stream).is_ok());
+  CHECK(all_equal(o1, 2.0f));
+  // the heads must group as the tensors say; nothing is launched otherwise
+  CHECK(!fmha_prefill_causal(&q, &k, &v, out.partition_mut({16, 1, d}), 0.0884f, 2, 96, 0).sync_on(stream).is_ok());
+}
+
 TEST(persistent_gemm_example) {
   // cutile-examples/examples/persistent_gemm.rs:61-126 as written: f32, 16x16x8 tiles, M = N = 64, K = 32, map [4, 1], 4 tile blocks
   auto stream = new_stream();
