@@ -585,9 +585,80 @@ class PrefillAttention(Workload):
                {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
 
 
+class LmHeadArgmax(Workload):
+    """lm_head_argmax_blocks_f16 + argmax_reduce_blocks_to_u32 (cutile-kernels/src/argmax.rs:88-158, 173-213): the greedy
+    token of one decode step; the weights stream through once, the logits are never stored."""
+    name, unit, dtype = "lm_head_argmax_f16_128256x4096", "GB/s", "f16 io / f32 accumulate"
+    vocab, k = 128256, 4096
+    work = 2.0 * vocab * k + 2.0 * k + 8.0 * (vocab // 64)
+    config = {"workload": "lm_head_argmax_blocks fp16: weights [128256, 4096], hidden [1, 4096], 2004 blocks of 64 rows, then "
+                          "argmax_reduce_blocks_to_u32 (two launches per step)"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.wb = oracle.f32_to_f16_bits(oracle.normal_f32((self.vocab, self.k), 51))
+        self.hb = oracle.f32_to_f16_bits(oracle.normal_f32(self.k, 52))
+        td = lambda bits: torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.float16)
+        self.w, self.h = td(self.wb), td(self.hb.reshape(1, self.k))
+        self.nb = self.vocab // 64
+        self.bm = torch.zeros(self.nb, device=dev)
+        self.bi = torch.zeros(self.nb, dtype=torch.int32, device=dev)
+        self.out = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.bmp, self.bip, self.outp = ct.partition(self.bm, [1]), ct.partition(self.bi, [1]), ct.partition(self.out, [1])
+
+    def launch_dominant(self):
+        self.ct.lm_head_argmax_blocks_f16(self.w, self.h, self.bmp, self.bip, self.vocab)
+
+    def launch(self):
+        self.launch_dominant()
+        self.ct.argmax_reduce_blocks_to_u32(self.bm, self.bi, self.outp, self.nb)
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        rm, ri = oracle.lm_head_argmax_blocks_f16(self.wb, self.hb, self.vocab)
+        want = oracle.argmax_reduce_blocks_to_u32(rm, ri, self.nb)
+        dt = time.perf_counter() - t0
+        got = int(self.out.item())
+        same_blocks = float(np.mean(self.bi.cpu().numpy().view(np.uint32) == ri))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port", "sample": "full size"}, \
+               {"token": got, "oracle_token": want, "ok": got == want, "blocks_with_the_same_index": same_blocks,
+                "max_abs_block_max": float(np.max(np.abs(self.bm.cpu().numpy() - rm)))}
+
+
+class EmbeddingBatch(Workload):
+    """embedding_batch_f16 (cutile-kernels/src/embeddings.rs:21-41): one table row per token."""
+    name, unit, dtype = "embedding_batch_f16_32768x4096", "GB/s", "f16 (gather)"
+    tokens, vocab, d = 32768, 128256, 4096
+    work = 4.0 * tokens * d + 4.0 * tokens
+    config = {"workload": "embedding_batch fp16: 32768 token ids into a [128256, 4096] table, out [32768, 4096] tiles [1, 1024]"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.tb = oracle.f32_to_f16_bits(oracle.normal_f32((self.vocab, self.d), 53))
+        self.ids = (np.random.default_rng(54).integers(0, self.vocab, self.tokens)).astype(np.uint32)
+        self.table = torch.from_numpy(self.tb.view(np.int16)).to(dev).view(torch.float16)
+        self.idd = torch.from_numpy(self.ids.view(np.int32)).to(dev)
+        self.out = torch.zeros(self.tokens, self.d, dtype=torch.float16, device=dev)
+        self.op = ct.partition(self.out, [1, 1024])
+
+    def launch(self):
+        self.ct.embedding_batch_f16(self.idd, self.table, self.op)
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        ref = oracle.embedding_batch_f16(self.ids, self.tb)
+        dt = time.perf_counter() - t0
+        exact = bool(np.array_equal(self.out.cpu().numpy().view(np.uint16), ref))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "full size"}, {"bit_exact": exact}
+
+
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

@@ -128,6 +128,12 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_argmax_blocks_f16": [vp, P(TensorArg), P(PartitionArg), P(PartitionArg), i32, P(LaunchOpts)],
+            "cutile_launch_lm_head_argmax_blocks_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(PartitionArg), i32,
+                                                        P(LaunchOpts)],
+            "cutile_launch_argmax_reduce_blocks_to_u32": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), i32, P(LaunchOpts)],
+            "cutile_launch_embedding_batch_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_gather_row_f16": [vp, P(TensorArg), P(PartitionArg), i32, P(LaunchOpts)],
             "cutile_launch_fmha_seq_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), f32, i32, i32, i32,
                                            P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
@@ -472,6 +478,50 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def _u32_partition(p: Partition) -> PartitionArg:
+    """the argument record of a partition of u32 values held in an int32 / uint32 tensor"""
+    return (p if p.dtype is not None else Partition(p.tensor, p.shape, p.prefix, U32)).arg()
+
+
+def argmax_blocks_f16(logits, block_max: Partition, block_idx: Partition, length: int, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-kernels/src/argmax.rs:21-71; block_idx: an int32 / uint32 tensor of u32 indices"""
+    o, _k = _opts(grid, generics, None)
+    la = tensor_arg(logits)
+    check(lib().cutile_launch_argmax_blocks_f16(_stream(stream), C.byref(la), C.byref(block_max.arg()), C.byref(_u32_partition(block_idx)),
+                                                int(length), C.byref(o)))
+
+
+def lm_head_argmax_blocks_f16(weights, hidden, block_max: Partition, block_idx: Partition, vocab_size: int, *, stream=None,
+                              grid=None, generics=None) -> None:
+    """cutile-kernels/src/argmax.rs:88-158"""
+    o, _k = _opts(grid, generics, None)
+    wa, ha = tensor_arg(weights), tensor_arg(hidden)
+    check(lib().cutile_launch_lm_head_argmax_blocks_f16(_stream(stream), C.byref(wa), C.byref(ha), C.byref(block_max.arg()),
+                                                        C.byref(_u32_partition(block_idx)), int(vocab_size), C.byref(o)))
+
+
+def argmax_reduce_blocks_to_u32(block_max, block_idx, out: Partition, num_blocks: int, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-kernels/src/argmax.rs:173-213"""
+    o, _k = _opts(grid, generics, None)
+    ma, ia = tensor_arg(block_max), tensor_arg(block_idx, dtype=U32)
+    check(lib().cutile_launch_argmax_reduce_blocks_to_u32(_stream(stream), C.byref(ma), C.byref(ia), C.byref(_u32_partition(out)),
+                                                          int(num_blocks), C.byref(o)))
+
+
+def embedding_batch_f16(token_ids, table, out: Partition, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-kernels/src/embeddings.rs:21-41; token_ids: an int32 / uint32 tensor of u32 ids"""
+    o, _k = _opts(grid, generics, None)
+    ia, ta = tensor_arg(token_ids, dtype=U32), tensor_arg(table)
+    check(lib().cutile_launch_embedding_batch_f16(_stream(stream), C.byref(ia), C.byref(ta), C.byref(out.arg()), C.byref(o)))
+
+
+def gather_row_f16(src, out: Partition, row_idx: int, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-kernels/src/pointwise.rs:86-99"""
+    o, _k = _opts(grid, generics, None)
+    sa = tensor_arg(src)
+    check(lib().cutile_launch_gather_row_f16(_stream(stream), C.byref(sa), C.byref(out.arg()), int(row_idx), C.byref(o)))
 
 
 def fmha_seq_f16(q, k, v, out: Partition, qk_scale: float, query_group_size: int, *, kv_len: int = 0, query_start: int = 0,

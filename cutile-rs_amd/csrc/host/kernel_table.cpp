@@ -71,6 +71,12 @@ std::vector<KernelEntry> build_table() {
   }
   add("rope", "f16", "rope_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
   add("kv_cache_update", "f16", "kv_cache_update_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
+  // greedy sampling and row gathers (cutile-kernels/src/argmax.rs, embeddings.rs, pointwise.rs:86-99)
+  add("argmax_blocks", "f16", "argmax_blocks_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 1);
+  add("lm_head_argmax_blocks", "f16", "lm_head_argmax_blocks_entry__f16", IMG_ELEMENTWISE, 256, 0, 64, 0, 0, 0, "f16", 0, 2);
+  add("argmax_reduce_blocks", "u32", "argmax_reduce_blocks_entry__u32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "u32", 0, 1);
+  add("embedding_batch", "f16", "embedding_batch_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
+  add("gather_row", "f16", "gather_row_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
 #undef EW
   static const char* kCreationTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64", "u8", "u16", "u32"};
   static std::deque<std::string> names;  // keeps generated strings alive at stable addresses

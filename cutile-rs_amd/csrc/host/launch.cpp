@@ -889,6 +889,159 @@ cutile_status_t cutile_launch_kv_cache_update_f16(cutile_stream_t stream, const 
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// ---- greedy sampling and row gathers (cutile-kernels/src/argmax.rs, embeddings.rs, pointwise.rs:86-99) ----
+// block_max / block_idx: rank-1 f32 / u32 outputs with tiles [1], one tile block per block.
+static cutile_status_t argmax_outputs_grid(const char* fn, const cutile_partition_arg_t* block_max,
+                                           const cutile_partition_arg_t* block_idx, const cutile_launch_opts_t* opts,
+                                           uint32_t tg[3]) {
+  if (cutile_status_t s = check_partition(block_max, "block_max", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(block_idx, "block_idx", 1, 1)) return s;
+  CUTILE_REQUIRE(block_max->tensor.dtype == CUTILE_DTYPE_F32 && block_idx->tensor.dtype == CUTILE_DTYPE_U32 &&
+                     block_max->partition_shape[0] == 1 && block_idx->partition_shape[0] == 1,
+                 CUTILE_ERR_KERNEL_LAUNCH, "%s: block_max must be f32 and block_idx u32, both partitioned [1]", fn);
+  uint32_t explicit_grid[3] = {0, 0, 0};
+  if (opts) memcpy(explicit_grid, opts->grid, sizeof(explicit_grid));
+  const cutile_partition_arg_t* parts[2] = {block_max, block_idx};
+  return cutile_infer_launch_grid(explicit_grid, parts, 2, tg);
+}
+
+cutile_status_t cutile_launch_argmax_blocks_f16(cutile_stream_t stream, const cutile_tensor_arg_t* logits,
+                                                const cutile_partition_arg_t* block_max,
+                                                const cutile_partition_arg_t* block_idx, int32_t len,
+                                                const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(logits, "logits", 1, 1)) return s;
+  CUTILE_REQUIRE(logits->dtype == CUTILE_DTYPE_F16, CUTILE_ERR_KERNEL_LAUNCH, "argmax_blocks_f16: logits must be f16");
+  uint32_t tg[3];
+  if (cutile_status_t s = argmax_outputs_grid("argmax_blocks_f16", block_max, block_idx, opts, tg)) return s;
+  const int block_size = generic_int(opts, 0, 1024);
+  CUTILE_REQUIRE(block_size > 0 && len >= 0, CUTILE_ERR_KERNEL_LAUNCH, "argmax_blocks_f16: BLOCK_SIZE must be positive and len non-negative");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("argmax_blocks", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*logits);
+  args.push_partition(*block_max);
+  args.push_partition(*block_idx);
+  args.push_val<int32_t>(len);
+  args.push_val<int32_t>(block_size);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {tg[0], 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_lm_head_argmax_blocks_f16(cutile_stream_t stream, const cutile_tensor_arg_t* weights,
+                                                        const cutile_tensor_arg_t* hidden,
+                                                        const cutile_partition_arg_t* block_max,
+                                                        const cutile_partition_arg_t* block_idx, int32_t vocab_size,
+                                                        const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(weights, "weights", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(hidden, "hidden", 2, 2)) return s;
+  const int32_t k = weights->shape[1];
+  CUTILE_REQUIRE(weights->dtype == CUTILE_DTYPE_F16 && hidden->dtype == CUTILE_DTYPE_F16, CUTILE_ERR_KERNEL_LAUNCH,
+                 "lm_head_argmax_blocks_f16: weights and hidden must be f16");
+  CUTILE_REQUIRE(hidden->shape[0] == 1 && hidden->shape[1] == k, CUTILE_ERR_KERNEL_LAUNCH,
+                 "lm_head_argmax_blocks_f16: weights are [%d, %d] but hidden is [%d, %d], expected [1, %d]", weights->shape[0], k,
+                 hidden->shape[0], hidden->shape[1], k);
+  // the tile program runs K / 32 whole tiles (argmax.rs:109-110)
+  CUTILE_REQUIRE(k % 32 == 0, CUTILE_ERR_KERNEL_LAUNCH, "lm_head_argmax_blocks_f16: K = %d must be a multiple of 32", k);
+  CUTILE_REQUIRE(k <= 30720, CUTILE_ERR_KERNEL_NOT_FOUND, "lm_head_argmax_blocks_f16: K = %d exceeds the 30720 the precompiled kernel keeps in LDS", k);
+  CUTILE_REQUIRE(vocab_size >= 0, CUTILE_ERR_KERNEL_LAUNCH, "lm_head_argmax_blocks_f16: vocab_size must be non-negative");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(k), "K")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = argmax_outputs_grid("lm_head_argmax_blocks_f16", block_max, block_idx, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("lm_head_argmax_blocks", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*weights);
+  args.push_tensor(*hidden);
+  args.push_partition(*block_max);
+  args.push_partition(*block_idx);
+  args.push_val<int32_t>(vocab_size);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {tg[0], 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, (uint32_t)k * 2, stream, args);
+}
+
+cutile_status_t cutile_launch_argmax_reduce_blocks_to_u32(cutile_stream_t stream, const cutile_tensor_arg_t* block_max,
+                                                          const cutile_tensor_arg_t* block_idx,
+                                                          const cutile_partition_arg_t* out, int32_t num_blocks,
+                                                          const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(block_max, "block_max", 1, 1)) return s;
+  if (cutile_status_t s = check_tensor(block_idx, "block_idx", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 1, 1)) return s;
+  CUTILE_REQUIRE(block_max->dtype == CUTILE_DTYPE_F32 && block_idx->dtype == CUTILE_DTYPE_U32 && out->tensor.dtype == CUTILE_DTYPE_U32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "argmax_reduce_blocks_to_u32: block_max is f32, block_idx and out are u32");
+  CUTILE_REQUIRE(out->tensor.shape[0] == 1 && out->partition_shape[0] == 1 && ((uintptr_t)out->tensor.ptr & 3) == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "argmax_reduce_blocks_to_u32: out must be one u32 partitioned [1]");
+  CUTILE_REQUIRE(num_blocks >= 0, CUTILE_ERR_KERNEL_LAUNCH, "argmax_reduce_blocks_to_u32: num_blocks must be non-negative");
+  const int block_size = generic_int(opts, 0, std::max(256, (num_blocks + 255) / 256 * 256));
+  CUTILE_REQUIRE(block_size > 0, CUTILE_ERR_KERNEL_LAUNCH, "argmax_reduce_blocks_to_u32: BLOCK_SIZE must be positive");
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("argmax_reduce_blocks", opts, "u32", {"u32"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*block_max);
+  args.push_tensor(*block_idx);
+  args.push_partition(*out);
+  args.push_val<int32_t>(num_blocks);
+  args.push_val<int32_t>(block_size);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {1, 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_embedding_batch_f16(cutile_stream_t stream, const cutile_tensor_arg_t* token_ids,
+                                                  const cutile_tensor_arg_t* table, const cutile_partition_arg_t* out,
+                                                  const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(token_ids, "token_ids", 1, 1)) return s;
+  if (cutile_status_t s = check_tensor(table, "table", 2, 2)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 2, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE(token_ids->dtype == CUTILE_DTYPE_U32 && table->dtype == CUTILE_DTYPE_F16 && ot.dtype == CUTILE_DTYPE_F16 &&
+                     ((uintptr_t)token_ids->ptr & 3) == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "embedding_batch_f16: token_ids must be u32, table and out f16");
+  const int32_t d = table->shape[1], block = out->partition_shape[1];
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && ot.shape[1] == d && ot.shape[0] <= token_ids->shape[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "embedding_batch_f16: out [%d, %d] tiles [%d, %d] must be [tokens <= %d, D = %d] partitioned [1, BLOCK_SIZE]",
+                 ot.shape[0], ot.shape[1], out->partition_shape[0], block, token_ids->shape[0], d);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(block), "BLOCK_SIZE")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("embedding_batch", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*token_ids);
+  args.push_tensor(*table);
+  args.push_partition(*out);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(std::min<uint32_t>(tg[0], (uint32_t)ot.shape[0]), 1u << 20)), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_gather_row_f16(cutile_stream_t stream, const cutile_tensor_arg_t* src,
+                                             const cutile_partition_arg_t* out, int32_t row_idx,
+                                             const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(src, "src", 2, 2)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 1, 1)) return s;
+  CUTILE_REQUIRE(src->dtype == CUTILE_DTYPE_F16 && out->tensor.dtype == CUTILE_DTYPE_F16, CUTILE_ERR_KERNEL_LAUNCH,
+                 "gather_row_f16: src and out must be f16");
+  CUTILE_REQUIRE(row_idx >= 0, CUTILE_ERR_KERNEL_LAUNCH, "gather_row_f16: row_idx must be non-negative");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(out->partition_shape[0]), "BLOCK_SIZE")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("gather_row", opts, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*src);
+  args.push_partition(*out);
+  args.push_val<int32_t>(row_idx);
+  args.push_tile_grid(tg);
+  const uint64_t width = std::min<uint64_t>((uint64_t)tg[0] * out->partition_shape[0], out->tensor.shape[0]);
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(width, 256), 4096)), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 static bool decode_vec_layout(const cutile_tensor_arg_t& t) {
   return t.strides[2] == 1 && t.strides[1] % 8 == 0 && t.strides[0] % 8 == 0 && aligned16(t.ptr);
 }

@@ -530,3 +530,198 @@ __device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, cons
 MAPPED_TILE_INDEX_KERNEL(1)
 MAPPED_TILE_INDEX_KERNEL(2)
 MAPPED_TILE_INDEX_KERNEL(3)
+
+// ---- greedy sampling and row gathers ---------------------------------------------------------
+// argmax_blocks_f16 / lm_head_argmax_blocks_f16 / argmax_reduce_blocks_to_u32
+// (cutile-kernels/src/argmax.rs:21-71, 88-158, 173-213), embedding_batch_f16
+// (embeddings.rs:21-41), gather_row_f16 (pointwise.rs:86-99).
+// A block's winner is its largest value and, among equal values, the smallest index; positions at or
+// beyond `len` count as -1e30 at their own index, exactly as the tile programs mask them (argmax.rs:42-55).
+namespace {
+
+struct Best {
+  float v;
+  int32_t i;
+};
+__device__ __forceinline__ Best better(Best a, Best b) {
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+// Winner of the workgroup, valid in every lane.  `scratch`: kThreads / 64 entries of LDS.
+__device__ __forceinline__ Best block_best(Best mine, Best* scratch) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    Best other = {__shfl_xor(mine.v, o, 64), __shfl_xor(mine.i, o, 64)};
+    mine = better(mine, other);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) scratch[wave] = mine;
+  __syncthreads();
+  Best r = scratch[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) r = better(r, scratch[w]);
+  return r;
+}
+constexpr float kMaskedLogit = -1.0e30f;
+
+}  // namespace
+
+// One workgroup per block of BLOCK_SIZE logits: block_max[b], block_idx[b].
+extern "C" __global__ void __launch_bounds__(kThreads)
+    argmax_blocks_entry__f16(TensorArg<1> logits, PartitionArg<1> block_max, PartitionArg<1> block_idx, int32_t len,
+                             int32_t block_size, TileGrid g) {
+  __shared__ Best scratch[kThreads / 64];
+  const int32_t b = blockIdx.x;
+  if (b >= (int32_t)g.x || b >= block_max.shape[0] || b >= block_idx.shape[0]) return;
+  const int64_t base = (int64_t)b * block_size;
+  const _Float16* lp = (const _Float16*)logits.ptr;
+  Best mine = {-INFINITY, INT32_MAX};
+  for (int32_t o = threadIdx.x; o < block_size; o += kThreads) {
+    const int64_t idx = base + o;
+    // beyond the tensor a tile load reads zero (cutile/src/_core.rs:651-657); beyond len the value is masked
+    float v = idx < logits.shape[0] ? (float)lp[idx * logits.strides[0]] : 0.0f;
+    if (idx >= len) v = kMaskedLogit;
+    mine = better(mine, Best{v, (int32_t)idx});
+  }
+  const Best r = block_best(mine, scratch);
+  if (threadIdx.x == 0) {
+    ((float*)block_max.ptr)[(int64_t)b * block_max.strides[0]] = r.v;
+    ((uint32_t*)block_idx.ptr)[(int64_t)b * block_idx.strides[0]] = (uint32_t)r.i;
+  }
+}
+
+// logits[r] = sum_k f32(weights[r, k]) * f32(hidden[0, k]) for the 64 rows of block b, then the block's winner.
+// The weights are read once, 16 bytes per lane and nontemporally (a [vocab, K] matrix streams through once per
+// token); the hidden vector sits in LDS.  A wavefront takes 16 of the 64 rows, two at a time.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    lm_head_argmax_blocks_entry__f16(TensorArg<2> weights, TensorArg<2> hidden, PartitionArg<1> block_max,
+                                     PartitionArg<1> block_idx, int32_t vocab_size, TileGrid g) {
+  constexpr int kRows = 64, kRowsPerWave = kRows / (kThreads / 64);
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  __shared__ float row_logit[kRows];
+  __shared__ Best scratch[kThreads / 64];
+  const int32_t b = blockIdx.x;
+  if (b >= (int32_t)g.x || b >= block_max.shape[0] || b >= block_idx.shape[0]) return;
+  const int32_t k_len = min(weights.shape[1], hidden.shape[1]);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const _Float16* wp = (const _Float16*)weights.ptr;
+  const _Float16* hp = (const _Float16*)hidden.ptr;
+  _Float16* hs = (_Float16*)lds_raw;
+  const bool vec = k_len % 8 == 0 && weights.strides[1] == 1 && weights.strides[0] % 8 == 0 && hidden.strides[1] == 1 &&
+                   (((uintptr_t)wp | (uintptr_t)hp) & 15) == 0;
+  for (int32_t k = threadIdx.x; k < k_len; k += kThreads) hs[k] = hp[(int64_t)k * hidden.strides[1]];
+  __syncthreads();
+  const int64_t row0 = (int64_t)b * kRows + wave * kRowsPerWave;
+  for (int rr = 0; rr < kRowsPerWave; rr += 2) {
+    float acc[2] = {0.0f, 0.0f};
+    if (vec) {
+      const int32_t chunks = k_len / 8;
+      for (int32_t c0 = 0; c0 < chunks; c0 += 64 * 4) {
+        Vec16<_Float16> w[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const int64_t r = row0 + rr + t;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int32_t c = c0 + u * 64 + lane;
+            if (r < weights.shape[0] && c < chunks)
+              w[t][u].raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + r * weights.strides[0]) + c);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int32_t c = c0 + u * 64 + lane;
+          if (c < chunks) {
+            Vec16<_Float16> h;
+            h.raw = *reinterpret_cast<const u32x4*>(hs + (int64_t)c * 8);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) acc[t] = __builtin_fmaf((float)w[t][u].v[e], (float)h.v[e], acc[t]);
+          }
+        }
+      }
+    } else {
+      for (int t = 0; t < 2; ++t) {
+        const int64_t r = row0 + rr + t;
+        if (r < weights.shape[0])
+          for (int32_t k = lane; k < k_len; k += 64)
+            acc[t] = __builtin_fmaf((float)wp[r * weights.strides[0] + (int64_t)k * weights.strides[1]], (float)hs[k], acc[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) acc[t] += __shfl_xor(acc[t], o, 64);
+      if (lane == 0) row_logit[wave * kRowsPerWave + rr + t] = acc[t];
+    }
+  }
+  __syncthreads();
+  Best mine = {-INFINITY, INT32_MAX};
+  if (threadIdx.x < kRows) {
+    const int64_t idx = (int64_t)b * kRows + threadIdx.x;
+    mine = Best{idx < vocab_size ? row_logit[threadIdx.x] : kMaskedLogit, (int32_t)idx};
+  }
+  const Best r = block_best(mine, scratch);
+  if (threadIdx.x == 0) {
+    ((float*)block_max.ptr)[(int64_t)b * block_max.strides[0]] = r.v;
+    ((uint32_t*)block_idx.ptr)[(int64_t)b * block_idx.strides[0]] = (uint32_t)r.i;
+  }
+}
+
+// One workgroup: the winner among the first `block_size` (value, index) pairs, of which `num_blocks` count.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    argmax_reduce_blocks_entry__u32(TensorArg<1> block_max, TensorArg<1> block_idx, PartitionArg<1> out,
+                                    int32_t num_blocks, int32_t block_size, TileGrid g) {
+  __shared__ Best scratch[kThreads / 64];
+  if (blockIdx.x != 0 || g.x == 0) return;
+  Best mine = {-INFINITY, INT32_MAX};
+  for (int32_t o = threadIdx.x; o < block_size; o += kThreads) {
+    float v = o < block_max.shape[0] ? ((const float*)block_max.ptr)[(int64_t)o * block_max.strides[0]] : 0.0f;
+    const int32_t i = o < block_idx.shape[0] ? (int32_t)((const uint32_t*)block_idx.ptr)[(int64_t)o * block_idx.strides[0]] : 0;
+    if (o >= num_blocks) v = kMaskedLogit;
+    mine = better(mine, Best{v, i});
+  }
+  const Best r = block_best(mine, scratch);
+  if (threadIdx.x == 0) ((uint32_t*)out.ptr)[0] = (uint32_t)r.i;
+}
+
+// out[row, :] = table[token_ids[row], :] (zeros for a token beyond the table, as a padded tile load gives);
+// a workgroup copies whole rows, 16 bytes per lane when the layout allows it.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    embedding_batch_entry__f16(TensorArg<1> token_ids, TensorArg<2> table, PartitionArg<2> out, TileGrid g) {
+  const int32_t rows = min(min((int32_t)g.x, out.shape[0]), token_ids.shape[0]);
+  const int64_t cover = (int64_t)g.y * out.pshape[1];
+  const int32_t width = (int32_t)(cover < out.shape[1] ? cover : out.shape[1]);
+  const _Float16* tp = (const _Float16*)table.ptr;
+  _Float16* op = (_Float16*)out.ptr;
+  const bool vec = width % 8 == 0 && table.strides[1] == 1 && out.strides[1] == 1 && table.strides[0] % 8 == 0 &&
+                   out.strides[0] % 8 == 0 && (((uintptr_t)tp | (uintptr_t)op) & 15) == 0;
+  for (int32_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const uint32_t token = ((const uint32_t*)token_ids.ptr)[(int64_t)row * token_ids.strides[0]];
+    const bool known = token < (uint32_t)table.shape[0];
+    const _Float16* src = tp + (int64_t)token * table.strides[0];
+    _Float16* dst = op + (int64_t)row * out.strides[0];
+    if (vec) {
+      for (int32_t c = threadIdx.x; c < width / 8; c += kThreads) {
+        u32x4 v = {0, 0, 0, 0};
+        if (known && c * 8 < table.shape[1]) v = *(reinterpret_cast<const u32x4*>(src) + c);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst) + c);
+      }
+    } else {
+      for (int32_t c = threadIdx.x; c < width; c += kThreads)
+        dst[(int64_t)c * out.strides[1]] = known && c < table.shape[1] ? src[(int64_t)c * table.strides[1]] : (_Float16)0;
+    }
+  }
+}
+
+// out[c] = src[row_idx, c]; zeros where the source has no such element.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    gather_row_entry__f16(TensorArg<2> src, PartitionArg<1> out, int32_t row_idx, TileGrid g) {
+  const int64_t cover = (int64_t)g.x * out.pshape[0];
+  const int32_t width = (int32_t)(cover < out.shape[0] ? cover : out.shape[0]);
+  const bool known = row_idx >= 0 && row_idx < src.shape[0];
+  const _Float16* sp = (const _Float16*)src.ptr + (int64_t)row_idx * src.strides[0];
+  _Float16* op = (_Float16*)out.ptr;
+  for (int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x; c < width; c += (int64_t)gridDim.x * kThreads)
+    op[c * out.strides[0]] = known && c < src.shape[1] ? sp[c * src.strides[1]] : (_Float16)0;
+}

@@ -467,6 +467,46 @@ struct SplitkReduceMergeFn {
     return cutile_launch_splitk_reduce_merge(s, &aa, &la, &op, o);
   }
 };
+struct ArgmaxBlocksF16Fn {
+  template <class L, class M, class I>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, L& logits, M& block_max, I& block_idx, int32_t len) {
+    auto la = input_arg(logits);
+    auto mp = block_max.arg(), ip = block_idx.arg();
+    return cutile_launch_argmax_blocks_f16(s, &la, &mp, &ip, len, o);
+  }
+};
+struct LmHeadArgmaxBlocksF16Fn {
+  template <class W, class H, class M, class I>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, W& weights, H& hidden, M& block_max, I& block_idx, int32_t vocab_size) {
+    auto wa = input_arg(weights), ha = input_arg(hidden);
+    auto mp = block_max.arg(), ip = block_idx.arg();
+    return cutile_launch_lm_head_argmax_blocks_f16(s, &wa, &ha, &mp, &ip, vocab_size, o);
+  }
+};
+struct ArgmaxReduceBlocksToU32Fn {
+  template <class M, class I, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, M& block_max, I& block_idx, O& out, int32_t num_blocks) {
+    auto ma = input_arg(block_max), ia = input_arg(block_idx);
+    auto op = out.arg();
+    return cutile_launch_argmax_reduce_blocks_to_u32(s, &ma, &ia, &op, num_blocks, o);
+  }
+};
+struct EmbeddingBatchF16Fn {
+  template <class I, class T, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, I& token_ids, T& table, O& out) {
+    auto ia = input_arg(token_ids), ta = input_arg(table);
+    auto op = out.arg();
+    return cutile_launch_embedding_batch_f16(s, &ia, &ta, &op, o);
+  }
+};
+struct GatherRowF16Fn {
+  template <class S, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, S& src, O& out, int32_t row_idx) {
+    auto sa = input_arg(src);
+    auto op = out.arg();
+    return cutile_launch_gather_row_f16(s, &sa, &op, row_idx, o);
+  }
+};
 // The five sequence-layout attention kernels share one C entry point (cutile_launch_fmha_seq_f16).
 template <bool Causal>
 struct SeqAttentionFn {          // kv_len and query_start by value
@@ -546,6 +586,16 @@ template <class NK, class NV, class KC, class VC, class P> auto kv_cache_update_
 template <class Q, class K, class V, class A, class L, class P> auto fmha_decode_gqa_split(Q&& q, K&& k, V&& v, A&& att_out, L&& lse_out, float qk_scale, P&& position_start) { return make_launcher<kernels::FmhaDecodeGqaSplitFn>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<A>(att_out), std::forward<L>(lse_out), qk_scale, std::forward<P>(position_start)); }
 // splitk_reduce_merge(att_partial, lse_partial, out: [1,GROUP,CHUNK_D])          attention.rs:917-930
 template <class A, class L, class O> auto splitk_reduce_merge(A&& att_partial, L&& lse_partial, O&& out) { return make_launcher<kernels::SplitkReduceMergeFn>(std::forward<A>(att_partial), std::forward<L>(lse_partial), std::forward<O>(out)); }
+// argmax_blocks_f16(logits, block_max: [1], block_idx: [1], len)                  cutile-kernels/src/argmax.rs:21-26
+template <class L, class M, class I> auto argmax_blocks_f16(L&& logits, M&& block_max, I&& block_idx, int32_t len) { return make_launcher<kernels::ArgmaxBlocksF16Fn>(std::forward<L>(logits), std::forward<M>(block_max), std::forward<I>(block_idx), len); }
+// lm_head_argmax_blocks_f16(weights, hidden, block_max: [1], block_idx: [1], vocab_size)   argmax.rs:88-94
+template <class W, class H, class M, class I> auto lm_head_argmax_blocks_f16(W&& weights, H&& hidden, M&& block_max, I&& block_idx, int32_t vocab_size) { return make_launcher<kernels::LmHeadArgmaxBlocksF16Fn>(std::forward<W>(weights), std::forward<H>(hidden), std::forward<M>(block_max), std::forward<I>(block_idx), vocab_size); }
+// argmax_reduce_blocks_to_u32(block_max, block_idx, out: [1], num_blocks)          argmax.rs:173-178
+template <class M, class I, class O> auto argmax_reduce_blocks_to_u32(M&& block_max, I&& block_idx, O&& out, int32_t num_blocks) { return make_launcher<kernels::ArgmaxReduceBlocksToU32Fn>(std::forward<M>(block_max), std::forward<I>(block_idx), std::forward<O>(out), num_blocks); }
+// embedding_batch_f16(token_ids, table, out: [1,BLOCK_SIZE])                       cutile-kernels/src/embeddings.rs:21-25
+template <class I, class T, class O> auto embedding_batch_f16(I&& token_ids, T&& table, O&& out) { return make_launcher<kernels::EmbeddingBatchF16Fn>(std::forward<I>(token_ids), std::forward<T>(table), std::forward<O>(out)); }
+// gather_row_f16(src, out: [BLOCK_SIZE], row_idx)                                  cutile-kernels/src/pointwise.rs:86-90
+template <class S, class O> auto gather_row_f16(S&& src, O&& out, int32_t row_idx) { return make_launcher<kernels::GatherRowF16Fn>(std::forward<S>(src), std::forward<O>(out), row_idx); }
 // flash_attn_causal_seq_f16(q, k, v, out: [BM,1,D], qk_scale, query_group_size, kv_len, query_start)   attention.rs:21-30
 template <class Q, class K, class V, class O> auto flash_attn_causal_seq_f16(Q&& q, K&& k, V&& v, O&& out, float qk_scale, int32_t query_group_size, int32_t kv_len, int32_t query_start) { return make_launcher<kernels::SeqAttentionFn<true>>(std::forward<Q>(q), std::forward<K>(k), std::forward<V>(v), std::forward<O>(out), qk_scale, query_group_size, kv_len, query_start); }
 // flash_attn_causal_seq_dynpos_f16(q, k, v, out: [BM,1,D], qk_scale, query_group_size, position_start: [1] u32)   attention.rs:128-136

@@ -427,6 +427,37 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* argmax_blocks_f16<BLOCK_SIZE>(logits: [n] f16, block_max: [blocks] f32 tiles [1], block_idx: [blocks] u32 tiles [1],
+ * len) — cutile-kernels/src/argmax.rs:21-71.  Block b holds the largest of logits[b*BLOCK_SIZE ..] (positions >= len
+ * count as -1e30) and the smallest index that attains it.  BLOCK_SIZE is generic 0 (default 1024). */
+cutile_status_t cutile_launch_argmax_blocks_f16(cutile_stream_t stream, const cutile_tensor_arg_t* logits,
+                                                const cutile_partition_arg_t* block_max,
+                                                const cutile_partition_arg_t* block_idx, int32_t len,
+                                                const cutile_launch_opts_t* opts);
+/* lm_head_argmax_blocks_f16<K>(weights: [vocab, K] f16, hidden: [1, K] f16, block_max, block_idx, vocab_size) —
+ * argmax.rs:88-158: logits = weights . hidden in f32, never stored; one block per 64 rows of weights. */
+cutile_status_t cutile_launch_lm_head_argmax_blocks_f16(cutile_stream_t stream, const cutile_tensor_arg_t* weights,
+                                                        const cutile_tensor_arg_t* hidden,
+                                                        const cutile_partition_arg_t* block_max,
+                                                        const cutile_partition_arg_t* block_idx, int32_t vocab_size,
+                                                        const cutile_launch_opts_t* opts);
+/* argmax_reduce_blocks_to_u32<BLOCK_SIZE>(block_max: [n] f32, block_idx: [n] u32, out: [1] u32 tile [1], num_blocks) —
+ * argmax.rs:173-213: the index of the largest of the first num_blocks block maxima (ties: smallest index).
+ * One tile of BLOCK_SIZE entries is read, as in the reference (generic 0, default: num_blocks rounded up to 256). */
+cutile_status_t cutile_launch_argmax_reduce_blocks_to_u32(cutile_stream_t stream, const cutile_tensor_arg_t* block_max,
+                                                          const cutile_tensor_arg_t* block_idx,
+                                                          const cutile_partition_arg_t* out, int32_t num_blocks,
+                                                          const cutile_launch_opts_t* opts);
+/* embedding_batch_f16<D, BLOCK_SIZE>(token_ids: [n] u32, table: [vocab, D] f16, out: [n, D] tiles [1, BLOCK_SIZE]) —
+ * cutile-kernels/src/embeddings.rs:21-41: out[r, :] = table[token_ids[r], :]. */
+cutile_status_t cutile_launch_embedding_batch_f16(cutile_stream_t stream, const cutile_tensor_arg_t* token_ids,
+                                                  const cutile_tensor_arg_t* table, const cutile_partition_arg_t* out,
+                                                  const cutile_launch_opts_t* opts);
+/* gather_row_f16<BLOCK_SIZE>(src: [rows, width] f16, out: [width] tiles [BLOCK_SIZE], row_idx) —
+ * cutile-kernels/src/pointwise.rs:86-99: out = src[row_idx, :]. */
+cutile_status_t cutile_launch_gather_row_f16(cutile_stream_t stream, const cutile_tensor_arg_t* src,
+                                             const cutile_partition_arg_t* out, int32_t row_idx,
+                                             const cutile_launch_opts_t* opts);
 /* The sequence-layout attention kernels of cutile-kernels, one entry point for the five of them:
  *   flash_attn_causal_seq_f16<BM,BN,D>(q, k, v, out, qk_scale, query_group_size, kv_len, query_start)
  *       cutile-kernels/src/attention.rs:21-116   -> position_start = NULL, causal = 1

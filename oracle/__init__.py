@@ -74,6 +74,9 @@ def lib() -> C.CDLL:
             "orc_gemm_bf16": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_gemm_bf16_f32out": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_fmha_ref_cpu": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp, i64]),
+            "orc_argmax_blocks_f16": (None, [vp, i64, i64, i64, vp, vp, i64]),
+            "orc_lm_head_argmax_blocks_f16": (None, [vp, vp, i64, i64, i64, vp, vp, i64]),
+            "orc_argmax_reduce_blocks_to_u32": (C.c_uint32, [vp, vp, i64, i64, i64]),
             "orc_attention_seq_ref": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, i64, C.c_int]),
             "orc_mx_quantize_e4m3": (None, [vp, vp, vp, i64, i64]),
             "orc_mx_dequantize_e4m3": (None, [vp, vp, vp, i64, i64]),
@@ -382,6 +385,54 @@ def attention_seq_ref(q, k, v, qk_scale: float, query_group_size: int, kv_len: i
     out = np.empty((q_len, q_heads, d), np.float32)
     lib().orc_attention_seq_ref(_p(q), _p(k), _p(v), _p(out), q_len, q_heads, kv_heads, max_seq, d, qk_scale,
                                 query_group_size, int(kv_len), int(query_start), int(causal))
+    return out
+
+
+# ---- greedy sampling and row gathers (cutile-kernels/src/argmax.rs, embeddings.rs, pointwise.rs) ----
+def argmax_blocks_f16(logits_bits, block_size: int, length: int, num_blocks: int = None):
+    """-> (block_max f32 [blocks], block_idx u32 [blocks])"""
+    logits_bits = _c(logits_bits, np.uint16)
+    n = logits_bits.shape[0]
+    nb = num_blocks if num_blocks is not None else -(-n // block_size)
+    bm, bi = np.empty(nb, np.float32), np.empty(nb, np.uint32)
+    lib().orc_argmax_blocks_f16(_p(logits_bits), n, block_size, length, _p(bm), _p(bi), nb)
+    return bm, bi
+
+
+def lm_head_argmax_blocks_f16(weight_bits, hidden_bits, vocab_size: int, num_blocks: int = None):
+    weight_bits, hidden_bits = _c(weight_bits, np.uint16), _c(hidden_bits, np.uint16)
+    rows, k = weight_bits.shape
+    assert hidden_bits.size == k
+    nb = num_blocks if num_blocks is not None else -(-rows // 64)
+    bm, bi = np.empty(nb, np.float32), np.empty(nb, np.uint32)
+    lib().orc_lm_head_argmax_blocks_f16(_p(weight_bits), _p(hidden_bits), rows, k, vocab_size, _p(bm), _p(bi), nb)
+    return bm, bi
+
+
+def argmax_reduce_blocks_to_u32(block_max, block_idx, num_blocks: int, block_size: int = None) -> int:
+    block_max, block_idx = _c(block_max, np.float32), _c(block_idx, np.uint32)
+    n = block_max.shape[0]
+    bs = block_size if block_size is not None else max(256, -(-num_blocks // 256) * 256)
+    return int(lib().orc_argmax_reduce_blocks_to_u32(_p(block_max), _p(block_idx), n, bs, num_blocks))
+
+
+def embedding_batch_f16(token_ids, table_bits) -> np.ndarray:
+    """embeddings.rs:21-41: out[r, :] = table[token_ids[r], :], zeros for a token beyond the table (padded tile load)"""
+    token_ids, table_bits = np.asarray(token_ids, np.int64), _c(table_bits, np.uint16)
+    out = np.zeros((token_ids.shape[0], table_bits.shape[1]), np.uint16)
+    ok = (token_ids >= 0) & (token_ids < table_bits.shape[0])
+    out[ok] = table_bits[token_ids[ok]]
+    return out
+
+
+def gather_row_f16(src_bits, row_idx: int, width: int = None) -> np.ndarray:
+    """pointwise.rs:86-99: out[c] = src[row_idx, c], zeros where src has no such element"""
+    src_bits = _c(src_bits, np.uint16)
+    width = src_bits.shape[1] if width is None else width
+    out = np.zeros(width, np.uint16)
+    if 0 <= row_idx < src_bits.shape[0]:
+        m = min(width, src_bits.shape[1])
+        out[:m] = src_bits[row_idx, :m]
     return out
 
 

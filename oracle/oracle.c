@@ -799,3 +799,85 @@ void orc_nvfp4_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, c
   }
   free(yd);
 }
+
+/* ---- greedy sampling (cutile-kernels/src/argmax.rs) ------------------------------------------------------ */
+static void block_winner(const float* vals, const int64_t* idx, int64_t n, float* out_max, uint32_t* out_idx,
+                         int64_t no_candidate) {
+  /* reduce_max, then reduce_min over the indices of the positions that attain it (argmax.rs:45-55) */
+  float mx = vals[0];
+  for (int64_t i = 1; i < n; i++) mx = fmaxf(mx, vals[i]);
+  int64_t best = INT64_MAX;
+  for (int64_t i = 0; i < n; i++) {
+    int64_t candidate = vals[i] == mx ? idx[i] : no_candidate;   /* select(is_max, indices, invalid_idx) */
+    if (candidate < best) best = candidate;
+  }
+  *out_max = mx;
+  *out_idx = (uint32_t)(int32_t)best;
+}
+
+/* argmax_blocks_f16<BLOCK_SIZE> (argmax.rs:21-71): block b covers logits[b*BLOCK_SIZE ..]; positions beyond the
+ * tensor load as zero (padded tile load), positions >= len count as -1e30 (:36-43); the index is the smallest one
+ * attaining the maximum, len + 1 if none (:47-55). */
+void orc_argmax_blocks_f16(const uint16_t* logits, int64_t n, int64_t block_size, int64_t len, float* block_max,
+                           uint32_t* block_idx, int64_t num_blocks) {
+  float* vals = (float*)malloc(sizeof(float) * (size_t)block_size);
+  int64_t* idx = (int64_t*)malloc(sizeof(int64_t) * (size_t)block_size);
+  for (int64_t b = 0; b < num_blocks; b++) {
+    for (int64_t o = 0; o < block_size; o++) {
+      int64_t i = b * block_size + o;
+      float v = i < n ? orc_f16_to_f32(logits[i]) : 0.0f;
+      vals[o] = i < len ? v : -1.0e30f;
+      idx[o] = i;
+    }
+    block_winner(vals, idx, block_size, &block_max[b], &block_idx[b], len + 1);
+  }
+  free(vals);
+  free(idx);
+}
+
+/* lm_head_argmax_blocks_f16<K> (argmax.rs:88-158): logits of 64 rows per block, accumulated in f32 over K / 32 tiles
+ * of 32 columns (each tile's 32 products summed, then added to the accumulator, :108-120), rows >= vocab_size masked
+ * to -1e30 (:127-132), then the block winner as above with vocab_size + 1 for "none" (:139-143). */
+void orc_lm_head_argmax_blocks_f16(const uint16_t* weights, const uint16_t* hidden, int64_t rows, int64_t k,
+                                   int64_t vocab_size, float* block_max, uint32_t* block_idx, int64_t num_blocks) {
+  float* h = (float*)malloc(sizeof(float) * (size_t)k);
+  for (int64_t i = 0; i < k; i++) h[i] = orc_f16_to_f32(hidden[i]);
+#pragma omp parallel for schedule(dynamic, 4)
+  for (int64_t b = 0; b < num_blocks; b++) {
+    float vals[64];
+    int64_t idx[64];
+    for (int64_t o = 0; o < 64; o++) {
+      int64_t r = b * 64 + o;
+      float acc = 0.0f;
+      if (r < rows)
+        for (int64_t kb = 0; kb + 32 <= k; kb += 32) {
+          float partial = 0.0f;
+          for (int64_t j = 0; j < 32; j++) partial += orc_f16_to_f32(weights[r * k + kb + j]) * h[kb + j];
+          acc += partial;
+        }
+      vals[o] = r < vocab_size ? acc : -1.0e30f;
+      idx[o] = r;
+    }
+    block_winner(vals, idx, 64, &block_max[b], &block_idx[b], vocab_size + 1);
+  }
+  free(h);
+}
+
+/* argmax_reduce_blocks_to_u32<BLOCK_SIZE> (argmax.rs:173-213): one tile of BLOCK_SIZE (value, index) pairs, entries
+ * beyond the tensors read as zero, entries >= num_blocks masked to -1e30; the result is the smallest index among the
+ * entries attaining the maximum (2147483647 if none). */
+uint32_t orc_argmax_reduce_blocks_to_u32(const float* block_max, const uint32_t* block_idx, int64_t n,
+                                         int64_t block_size, int64_t num_blocks) {
+  float* vals = (float*)malloc(sizeof(float) * (size_t)block_size);
+  int64_t* idx = (int64_t*)malloc(sizeof(int64_t) * (size_t)block_size);
+  for (int64_t o = 0; o < block_size; o++) {
+    vals[o] = o < num_blocks ? (o < n ? block_max[o] : 0.0f) : -1.0e30f;
+    idx[o] = o < n ? (int64_t)(int32_t)block_idx[o] : 0;
+  }
+  float mx;
+  uint32_t out;
+  block_winner(vals, idx, block_size, &mx, &out, 2147483647);
+  free(vals);
+  free(idx);
+  return out;
+}

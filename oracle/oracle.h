@@ -42,6 +42,14 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_argmax_blocks_f16, orc_lm_head_argmax_blocks_f16, orc_argmax_reduce_blocks_to_u32
+ *                        cutile-kernels/src/argmax.rs (kernel bodies).  Pinned by numpy.argmax
+ *                        (first index of the maximum) block by block and through the
+ *                        composition blocks -> reduce = argmax of the whole vector, and by a
+ *                        float64 matrix-vector product; the reference only compiles these
+ *                        kernels: parity unpinned by reference tests.  embedding_batch_f16
+ *                        and gather_row_f16 (embeddings.rs:21-41, pointwise.rs:86-99) are
+ *                        numpy indexing in the Python wrapper.
  *   orc_attention_seq_ref
  *                        the five sequence-layout attention kernels of
  *                        cutile-kernels/src/attention.rs:21-726 (kernel bodies).  Pinned by
@@ -122,6 +130,13 @@ void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, i
 void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
                              uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
                              int64_t position_start, int64_t seq_len);
+/* greedy sampling: cutile-kernels/src/argmax.rs:21-71, 88-158, 173-213 */
+void orc_argmax_blocks_f16(const uint16_t* logits, int64_t n, int64_t block_size, int64_t len, float* block_max,
+                           uint32_t* block_idx, int64_t num_blocks);
+void orc_lm_head_argmax_blocks_f16(const uint16_t* weights, const uint16_t* hidden, int64_t rows, int64_t k,
+                                   int64_t vocab_size, float* block_max, uint32_t* block_idx, int64_t num_blocks);
+uint32_t orc_argmax_reduce_blocks_to_u32(const float* block_max, const uint32_t* block_idx, int64_t n,
+                                         int64_t block_size, int64_t num_blocks);
 /* the five sequence-layout attention kernels: cutile-kernels/src/attention.rs:21-726 */
 void orc_attention_seq_ref(const float* q, const float* k, const float* v, float* out, int64_t q_len,
                            int64_t q_heads, int64_t kv_heads, int64_t max_seq, int64_t dsz, float qk_scale,

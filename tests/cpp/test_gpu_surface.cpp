@@ -184,6 +184,41 @@ TEST(sequence_attention_launchers_closed_forms) {
   CHECK(!fmha_prefill_causal(&q, &k, &v, out.partition_mut({16, 1, d}), 0.0884f, 2, 96, 0).sync_on(stream).is_ok());
 }
 
+TEST(greedy_sampling_and_gathers_closed_forms) {
+  // logits = arange: the largest valid index wins; constant weights and hidden: every logit is K / 2, the first row wins
+  auto stream = new_stream();
+  const int n = 2000, nb = 2;                          // f16 holds every integer up to 2048
+  auto logits = api::arange<f16>(n).sync_on(stream).unwrap();
+  auto bm = api::zeros<float>({nb}).sync_on(stream).unwrap();
+  auto bi = api::zeros<uint32_t>({nb}).sync_on(stream).unwrap();
+  auto tok = api::zeros<uint32_t>({1}).sync_on(stream).unwrap();
+  CHECK(argmax_blocks_f16(&logits, bm.partition_mut({1}), bi.partition_mut({1}), 1500).generics({"1024"}).sync_on(stream).is_ok());
+  CHECK(argmax_reduce_blocks_to_u32(&bm, &bi, tok.partition_mut({1}), nb).sync_on(stream).is_ok());
+  auto bih = api::to_host_vec(bi).sync_on(stream).unwrap();
+  auto bmh = api::to_host_vec(bm).sync_on(stream).unwrap();
+  CHECK(bih[0] == 1023 && bih[1] == 1499 && bmh[0] == 1023.0f && bmh[1] == 1499.0f);
+  CHECK(api::to_host_vec(tok).sync_on(stream).unwrap()[0] == 1499);
+  const int vocab = 256, k = 64;
+  auto table = api::full<f16>(0.5, {vocab, k}).sync_on(stream).unwrap();
+  auto hidden = api::full<f16>(1.0, {1, k}).sync_on(stream).unwrap();
+  auto bm2 = api::zeros<float>({4}).sync_on(stream).unwrap();
+  auto bi2 = api::zeros<uint32_t>({4}).sync_on(stream).unwrap();
+  CHECK(lm_head_argmax_blocks_f16(&table, &hidden, bm2.partition_mut({1}), bi2.partition_mut({1}), 200).generics({"64"}).sync_on(stream).is_ok());
+  auto bm2h = api::to_host_vec(bm2).sync_on(stream).unwrap();
+  auto bi2h = api::to_host_vec(bi2).sync_on(stream).unwrap();
+  for (int b = 0; b < 3; ++b) CHECK(bm2h[b] == 32.0f && bi2h[b] == (uint32_t)(b * 64));     // all equal: the first row of the block
+  CHECK(bm2h[3] == 32.0f && bi2h[3] == 192);                                              // rows 192 .. 199 are valid
+  // embedding rows and a gathered row are copies
+  auto ids = api::full<uint32_t>(7, {5}).sync_on(stream).unwrap();
+  auto emb = api::zeros<f16>({5, k}).sync_on(stream).unwrap();
+  CHECK(embedding_batch_f16(&ids, &table, emb.partition_mut({1, 32})).generics({"64", "32"}).sync_on(stream).is_ok());
+  for (f16 x : api::to_host_vec(emb).sync_on(stream).unwrap()) CHECK(f32_from_f16(x) == 0.5f);
+  auto row = api::zeros<f16>({k}).sync_on(stream).unwrap();
+  CHECK(gather_row_f16(&table, row.partition_mut({16}), 3).sync_on(stream).is_ok());
+  for (f16 x : api::to_host_vec(row).sync_on(stream).unwrap()) CHECK(f32_from_f16(x) == 0.5f);
+  CHECK(!gather_row_f16(&table, row.partition_mut({16}), -1).sync_on(stream).is_ok());
+}
+
 TEST(persistent_gemm_example) {
   // cutile-examples/examples/persistent_gemm.rs:61-126 as written: f32, 16x16x8 tiles, M = N = 64, K = 32, map [4, 1], 4 tile blocks
   auto stream = new_stream();
