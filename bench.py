@@ -585,6 +585,52 @@ class PrefillAttention(Workload):
                {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
 
 
+class GroupGemm(Workload):
+    """group_gemm_f16_nt_desc (cutile-kernels/src/experimental/moe.rs:67-128): expert batches of unequal size, one launch."""
+    name, unit, bound, peak_key = "group_gemm_f16_32x4096x4096", "TFLOP/s", "mfma", "mfma_bf16"
+    dtype = "f16 in / f32 acc / f16 out"
+    groups, n, k = 32, 4096, 4096
+    rows = [256 + 96 * ((7 * g) % 17) for g in range(32)]                 # 256 .. 1792 tokens per expert, multiples of 16
+    work = 2.0 * sum(rows) * n * k
+    config = {"workload": f"group_gemm_f16_nt_desc fp16: 32 groups, A_g [256..1792 rows ({sum(rows)} in all), 4096] x B_g [4096, 4096], "
+                          "descriptor tables in device memory, 256 persistent tile blocks", "tile": "256x256x64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        self.ab = [oracle.f32_to_f16_bits(oracle.normal_f32((m, self.k), 60 + g, 0, self.k ** -0.5)) for g, m in enumerate(self.rows)]
+        self.bb = oracle.f32_to_f16_bits(oracle.normal_f32((self.k, self.n), 59, 0, self.k ** -0.5))
+        td = lambda bits: torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.float16)
+        self.a = [td(b) for b in self.ab]
+        self.b = [td(self.bb) if g == 0 else td(self.bb).clone() for g in range(self.groups)]   # one weight matrix per expert
+        self.c = [torch.zeros(m, self.n, dtype=torch.float16, device=dev) for m in self.rows]
+
+        def tables(ts):
+            ptrs = torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+            metas = torch.zeros(len(ts), 8, dtype=torch.int32)
+            for i, t in enumerate(ts):
+                metas[i, 0], metas[i, 1], metas[i, 2] = t.shape[0], t.shape[1], t.stride(0)
+            return ptrs, metas.to(dev)
+        self.tabs = tables(self.a) + tables(self.b) + tables(self.c)
+
+    def launch(self):
+        ap, am, bp, bm, cp, cm = self.tabs
+        self.ct.group_gemm_f16_nt_desc(ap, bp, cp, am, bm, cm, self.groups, generics=[256, 256, 64, 256])
+
+    def cpu_baseline(self, oracle, np, torch):
+        g, rows = 5, 128
+        x = oracle.f16_bits_to_f32(self.ab[g][:rows])
+        t0 = time.perf_counter()
+        ref = oracle.cpu_gemm_f32(x, oracle.f16_bits_to_f32(self.bb))
+        dt = time.perf_counter() - t0
+        got = self.c[g][:rows].float().cpu().numpy()
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        return {"value": 2.0 * rows * self.n * self.k / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"the first {rows} rows of group {g} (naive f32 loop)"}, \
+               {"rel_l2_sampled_rows": rel, "tolerance": 1e-2, "ok": rel <= 1e-2}
+
+
 class LmHeadArgmax(Workload):
     """lm_head_argmax_blocks_f16 + argmax_reduce_blocks_to_u32 (cutile-kernels/src/argmax.rs:88-158, 173-213): the greedy
     token of one decode step; the weights stream through once, the logits are never stored."""
@@ -658,7 +704,7 @@ class EmbeddingBatch(Workload):
 
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

@@ -128,6 +128,8 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_group_gemm_f16_nt_desc": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg),
+                                                     P(TensorArg), i32, P(LaunchOpts)],
             "cutile_launch_argmax_blocks_f16": [vp, P(TensorArg), P(PartitionArg), P(PartitionArg), i32, P(LaunchOpts)],
             "cutile_launch_lm_head_argmax_blocks_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(PartitionArg), i32,
                                                         P(LaunchOpts)],
@@ -478,6 +480,15 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def group_gemm_f16_nt_desc(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups: int, *, stream=None, grid=None,
+                           generics=None, variant=None) -> None:
+    """cutile-kernels/src/experimental/moe.rs:67-128: pointer tables (int64) and descriptor tables (int32 [groups, 8]:
+    rows, cols, row stride) in device memory; generics [BM, BN, BK, NUM_SM]"""
+    o, _k = _opts(grid, generics, variant)
+    t = [tensor_arg(x) for x in (a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas)]
+    check(lib().cutile_launch_group_gemm_f16_nt_desc(_stream(stream), *[C.byref(x) for x in t], int(num_groups), C.byref(o)))
 
 
 def _u32_partition(p: Partition) -> PartitionArg:

@@ -151,6 +151,8 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 128, 256, 64, 2, 2);
   gemm("bf16", 128, 128, 64, 2, 2);
   gemm("bf16", 64, 128, 64, 2, 2);
+  gemm("f16", 256, 256, 64, 4, 2, "d");
+  gemm("f16", 128, 128, 64, 2, 2, "d");
   gemm("bf16f32", 128, 128, 64, 2, 2);
   gemm("bf16f32", 256, 256, 64, 2, 2);
   // any tile shape, strides and extents (tile = 0: not tied to a partition shape); 64x64 outputs per workgroup
@@ -173,6 +175,16 @@ std::vector<KernelEntry> build_table() {
     std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
     add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
         (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "bf16", 0, 2);
+  }
+  // f16: persistent and grouped (descriptor-table) forms of the pipelined bodies
+  for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2}}) {
+    std::string v = "f16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
+    add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
+        (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "f16", 0, 2);
+    // the grouped form keeps the group descriptors live across the tile loop: 2 x 4 wavefronts at 256 x 256 (no spills)
+    std::string gv = t[0] == 256 ? std::string("f16_256x256x64_d2x4") : v;
+    add("group_gemm_nt_desc", keep(gv), keep("group_gemm_nt_desc_entry__" + gv), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
+        (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "f16", 0, 2);
   }
   for (const char* dt : {"bf16", "f16", "f32"})
     add("gemm_persistent", keep(std::string(dt) + "_generic"), keep(std::string("gemm_persistent_entry__") + dt + "_generic"),

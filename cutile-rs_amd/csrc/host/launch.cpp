@@ -1351,13 +1351,14 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
   MappedArg m;
   uint32_t grid[3];
   if (cutile_status_t s = mapped_launch_grid(zm, opts, &m, grid)) return s;
-  const bool fast_layout = in_bf16 && x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
+  const bool fast_layout = (in_bf16 || in_f16) && x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
                            y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
                            aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0;
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
-      if (strcmp(e.function, "gemm_persistent") == 0 && e.tile[0] == bm && e.tile[1] == bn) acceptable.push_back(e.variant);
+      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn)
+        acceptable.push_back(e.variant);
   acceptable.push_back(std::string(dt) + "_generic");
   Resolved res;
   if (cutile_status_t s = resolve_entry("gemm_persistent", opts, acceptable[0], acceptable, &res)) return s;
@@ -1366,6 +1367,60 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
   args.push_tensor(*x);
   args.push_tensor(*y);
   args.push_val<MappedArg>(m);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+// group_gemm_f16_nt_desc (cutile-kernels/src/experimental/moe.rs:67-128): no partition argument, so the launch grid
+// (NUM_SM workgroups) comes from .grid() or the NUM_SM generic, and the tile shape from the BM / BN generics.
+cutile_status_t cutile_launch_group_gemm_f16_nt_desc(cutile_stream_t stream, const cutile_tensor_arg_t* a_ptrs,
+                                                     const cutile_tensor_arg_t* b_ptrs, const cutile_tensor_arg_t* c_ptrs,
+                                                     const cutile_tensor_arg_t* a_metas, const cutile_tensor_arg_t* b_metas,
+                                                     const cutile_tensor_arg_t* c_metas, int32_t num_groups,
+                                                     const cutile_launch_opts_t* opts) {
+  const cutile_tensor_arg_t* ptrs[3] = {a_ptrs, b_ptrs, c_ptrs};
+  const cutile_tensor_arg_t* metas[3] = {a_metas, b_metas, c_metas};
+  const char* names[3] = {"a", "b", "c"};
+  CUTILE_REQUIRE(num_groups >= 0, CUTILE_ERR_KERNEL_LAUNCH, "group_gemm_f16_nt_desc: num_groups must be non-negative");
+  for (int i = 0; i < 3; ++i) {
+    if (cutile_status_t s = check_tensor(ptrs[i], "pointer table", 1, 1)) return s;
+    if (cutile_status_t s = check_tensor(metas[i], "descriptor table", 2, 2)) return s;
+    CUTILE_REQUIRE(ptrs[i]->dtype == CUTILE_DTYPE_I64 && ((uintptr_t)ptrs[i]->ptr & 7) == 0 && ptrs[i]->shape[0] >= num_groups,
+                   CUTILE_ERR_KERNEL_LAUNCH, "group_gemm_f16_nt_desc: %s_ptrs must be an aligned i64 tensor of at least %d entries",
+                   names[i], num_groups);
+    CUTILE_REQUIRE(metas[i]->dtype == CUTILE_DTYPE_I32 && metas[i]->shape[1] == 8 && metas[i]->shape[0] >= num_groups &&
+                       ((uintptr_t)metas[i]->ptr & 3) == 0,
+                   CUTILE_ERR_KERNEL_LAUNCH, "group_gemm_f16_nt_desc: %s_metas must be an i32 tensor [>= %d, 8]", names[i], num_groups);
+  }
+  const int bm = generic_int(opts, 0, 128), bn = generic_int(opts, 1, 128), bk = generic_int(opts, 2, 64);
+  const int num_sm_generic = generic_int(opts, 3, 0);
+  CUTILE_REQUIRE(bk > 0, CUTILE_ERR_KERNEL_LAUNCH, "group_gemm_f16_nt_desc: BK must be positive");
+  uint32_t grid[3] = {0, 1, 1};
+  if (opts && (opts->grid[0] | opts->grid[1] | opts->grid[2])) {
+    CUTILE_REQUIRE(opts->grid[0] > 0 && opts->grid[1] == 1 && opts->grid[2] == 1, CUTILE_ERR_KERNEL_LAUNCH,
+                   "group_gemm_f16_nt_desc: the launch grid must be (NUM_SM, 1, 1), got (%u, %u, %u)", opts->grid[0], opts->grid[1],
+                   opts->grid[2]);
+    grid[0] = opts->grid[0];
+  }
+  CUTILE_REQUIRE(grid[0] || num_sm_generic > 0, CUTILE_ERR_KERNEL_LAUNCH, "Launch grid required.");
+  // tiles advance by NUM_SM (moe.rs:121): a grid of another size would skip or repeat tiles
+  CUTILE_REQUIRE(!grid[0] || num_sm_generic <= 0 || (uint32_t)num_sm_generic == grid[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "group_gemm_f16_nt_desc: the launch grid (%u) must equal NUM_SM = %d", grid[0], num_sm_generic);
+  if (!grid[0]) grid[0] = (uint32_t)num_sm_generic;
+  std::vector<std::string> acceptable;
+  for (const auto& e : kernel_table())
+    if (strcmp(e.function, "group_gemm_nt_desc") == 0 && e.tile[0] == bm && e.tile[1] == bn) acceptable.push_back(e.variant);
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of group_gemm_f16_nt_desc<BM=%d, BN=%d>; available: %s", bm, bn,
+                 list_variants("group_gemm_nt_desc").c_str());
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("group_gemm_nt_desc", &o, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  for (int i = 0; i < 3; ++i) args.push_tensor(*ptrs[i]);
+  for (int i = 0; i < 3; ++i) args.push_tensor(*metas[i]);
+  args.push_val<int32_t>(num_groups);
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

@@ -234,7 +234,7 @@ struct Gemm {
 //  * operands are read one MFMA block ahead (register double buffering);
 //  * the K advance of the global addresses rides in the scalar offset of the
 //    buffer instruction: no per-iteration address arithmetic in vector registers.
-template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT, typename InT = __bf16>
 struct GemmDirect {
   static constexpr int BK = 64;
   static constexpr int kWaves = WAVES_M * WAVES_N;
@@ -378,7 +378,7 @@ struct GemmDirect {
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
-          acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[tn], f.a[tm], acc[tn][tm], 0, 0, 0);
+          acc[tn][tm] = mfma_32x32x16<InT>(f.b[tn], f.a[tm], acc[tn][tm]);
     };
 
     const int k_tiles = (k_total + BK - 1) / BK;
@@ -438,7 +438,7 @@ struct GemmDirect {
         for (int r = 0; r < NR; ++r)
           if (r * READ_SLOTS / NR == j) read_operand(rd_stage, rd_ks, into, r);
         acc[j / TM][j % TM] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM], 0, 0, 0);
+            mfma_32x32x16<InT>(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM]);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
@@ -862,6 +862,74 @@ GEMM_KERNEL(bf16f32_256x256x64_w2x2, 256, 256, 64, 2, 2, float)
 GEMM_DIRECT_KERNEL(bf16_256x256x64_d4x2, 256, 256, 4, 2, __bf16)
 GEMM_DIRECT_KERNEL(bf16_256x256x64_d2x4, 256, 256, 2, 4, __bf16)
 GEMM_DIRECT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)
+
+// the same pipelines on f16 operands (v_mfma_f32_32x32x16_f16), f16 z
+#define GEMM_DIRECT_F16_KERNEL(NAME, BM, BN, WVM, WVN)                                            \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmDirect<BM, BN, WVM, WVN, _Float16, _Float16>::run(z, x, y, k, g, accumulate);           \
+  }                                                                                             \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_persistent_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
+    GemmDirect<BM, BN, WVM, WVN, _Float16, _Float16>::run_persistent(z, x, y, m);               \
+  }
+GEMM_DIRECT_F16_KERNEL(f16_256x256x64_d4x2, 256, 256, 4, 2)
+GEMM_DIRECT_F16_KERNEL(f16_128x128x64_d2x2, 128, 128, 2, 2)
+
+// group_gemm_f16_nt_desc<BM, BN, BK, NUM_SM>(a_ptrs, b_ptrs, c_ptrs: [groups] i64; a_metas, b_metas, c_metas:
+// [groups, 8] i32 = (rows, cols, row stride, ...); num_groups) — cutile-kernels/src/experimental/moe.rs:67-128.
+// Group g multiplies A_g [m, k] by B_g [k, n] into C_g [m, n] (f16, f32 accumulation); the tiles of all groups form
+// one sequence, group after group and row-major inside a group, and workgroup w computes tiles w, w + grid, ...
+// (:82-83, 106-124).  The descriptors are read from device memory by every workgroup; as in the reference they are
+// trusted: pointers 16-byte aligned, rows and columns multiples of 16, row strides multiples of 8 (:24, 47-55).
+template <int BM, int BN, int WVM, int WVN>
+__device__ __forceinline__ void group_gemm_desc(const TensorArg<1>& a_ptrs, const TensorArg<1>& b_ptrs, const TensorArg<1>& c_ptrs,
+                                                const TensorArg<2>& a_metas, const TensorArg<2>& b_metas,
+                                                const TensorArg<2>& c_metas, int32_t num_groups) {
+  using G = GemmDirect<BM, BN, WVM, WVN, _Float16, _Float16>;
+  auto uniform = [](int32_t v) { return __builtin_amdgcn_readfirstlane(v); };
+  auto describe = [&](const TensorArg<1>& ptrs, const TensorArg<2>& metas, int32_t g, TensorArg<2>* t) {
+    const uint32_t* pp = reinterpret_cast<const uint32_t*>((const int64_t*)ptrs.ptr + (int64_t)g * ptrs.strides[0]);
+    const int32_t* mp = (const int32_t*)metas.ptr + (int64_t)g * metas.strides[0];
+    const uint64_t addr = (uint64_t)(uint32_t)uniform((int32_t)pp[0]) | ((uint64_t)(uint32_t)uniform((int32_t)pp[1]) << 32);
+    t->ptr = (void*)addr;
+    t->shape[0] = uniform(mp[0]);
+    t->shape[1] = uniform(mp[metas.strides[1]]);
+    t->strides[0] = uniform(mp[2 * metas.strides[1]]);
+    t->strides[1] = 1;
+  };
+  uint32_t tile_idx = blockIdx.x, group_start = 0;
+  for (int32_t g = 0; g < num_groups; ++g) {
+    TensorArg<2> a, b, c;
+    describe(a_ptrs, a_metas, g, &a);
+    describe(b_ptrs, b_metas, g, &b);
+    describe(c_ptrs, c_metas, g, &c);
+    const int32_t m = a.shape[0], k = a.shape[1], n = b.shape[1];
+    const uint32_t tiles_n = (uint32_t)((n + BN - 1) / BN);
+    const uint32_t tiles = (uint32_t)((m + BM - 1) / BM) * tiles_n;
+    PartitionArg<2> z;
+    z.ptr = c.ptr;
+    z.shape[0] = c.shape[0], z.shape[1] = c.shape[1];
+    z.strides[0] = z.pstrides[0] = c.strides[0], z.strides[1] = z.pstrides[1] = 1;
+    z.pshape[0] = BM, z.pshape[1] = BN;
+    while (tile_idx >= group_start && tile_idx < group_start + tiles) {
+      const uint32_t in_group = tile_idx - group_start;
+      G::run_tile(z, a, b, k, in_group / tiles_n, in_group % tiles_n, 0);
+      __syncthreads();   // the output bands live in the stages that the next tile refills
+      tile_idx += gridDim.x;
+    }
+    group_start += tiles;
+  }
+}
+#define GROUP_GEMM_KERNEL(NAME, BM, BN, WVM, WVN)                                                 \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      group_gemm_nt_desc_entry__##NAME(TensorArg<1> a_ptrs, TensorArg<1> b_ptrs, TensorArg<1> c_ptrs, TensorArg<2> a_metas, \
+                                       TensorArg<2> b_metas, TensorArg<2> c_metas, int32_t num_groups) { \
+    group_gemm_desc<BM, BN, WVM, WVN>(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups); \
+  }
+GROUP_GEMM_KERNEL(f16_256x256x64_d2x4, 256, 256, 2, 4)
+GROUP_GEMM_KERNEL(f16_128x128x64_d2x2, 128, 128, 2, 2)
 
 #define GEMM_RING_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                          \
   extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \

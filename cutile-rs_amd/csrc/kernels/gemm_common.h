@@ -31,6 +31,46 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo, hi}, b2));  // v_cvt_pk_bf16_f32, round to nearest even
 }
 
+// 16-bit outputs: two f32 rounded to nearest even into one register, and a stored pair widened again.
+template <typename OutT>
+__device__ __forceinline__ uint32_t pack_out2(float lo, float hi) {
+  if constexpr (__is_same(OutT, _Float16)) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo, hi}, h2));   // v_cvt_pk_f16_f32
+  } else {
+    return pack_bf16x2(lo, hi);
+  }
+}
+template <typename OutT>
+__device__ __forceinline__ float stored_lo(uint32_t bits) {
+  if constexpr (__is_same(OutT, _Float16)) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return (float)__builtin_bit_cast(h2, bits)[0];
+  } else {
+    return __builtin_bit_cast(float, bits << 16);
+  }
+}
+template <typename OutT>
+__device__ __forceinline__ float stored_hi(uint32_t bits) {
+  if constexpr (__is_same(OutT, _Float16)) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return (float)__builtin_bit_cast(h2, bits)[1];
+  } else {
+    return __builtin_bit_cast(float, bits & 0xffff0000u);
+  }
+}
+// v_mfma_f32_32x32x16 on 16-byte operand fragments of bf16 or f16 (the fragments travel as raw bits).
+template <typename InT>
+__device__ __forceinline__ f32x16 mfma_32x32x16(bf16x8 a, bf16x8 b, f32x16 c) {
+  if constexpr (__is_same(InT, _Float16)) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+}
+
 // Tile index for this workgroup: XCD-contiguous, then grouped along M.
 __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t* pm,
                                             uint32_t* pn) {
@@ -148,23 +188,23 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
       if constexpr (sizeof(OutT) == 2) {
         f32x4 hi = *reinterpret_cast<const f32x4*>(src + ((((rd_col >> 2) + 1) ^ (r & 15)) << 4));
         if (accumulate) {
-          lo[0] += __builtin_bit_cast(float, o.x << 16);
-          lo[1] += __builtin_bit_cast(float, o.x & 0xffff0000u);
-          lo[2] += __builtin_bit_cast(float, o.y << 16);
-          lo[3] += __builtin_bit_cast(float, o.y & 0xffff0000u);
-          hi[0] += __builtin_bit_cast(float, o.z << 16);
-          hi[1] += __builtin_bit_cast(float, o.z & 0xffff0000u);
-          hi[2] += __builtin_bit_cast(float, o.w << 16);
-          hi[3] += __builtin_bit_cast(float, o.w & 0xffff0000u);
+          lo[0] += stored_lo<OutT>(o.x);
+          lo[1] += stored_hi<OutT>(o.x);
+          lo[2] += stored_lo<OutT>(o.y);
+          lo[3] += stored_hi<OutT>(o.y);
+          hi[0] += stored_lo<OutT>(o.z);
+          hi[1] += stored_hi<OutT>(o.z);
+          hi[2] += stored_lo<OutT>(o.w);
+          hi[3] += stored_hi<OutT>(o.w);
         }
         if (gr < zM && col_ok) {
           OutT* dst = zp + (int64_t)gr * ldz + gc;
           if (full) {
-            u32x4 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]),
-                       pack_bf16x2(hi[2], hi[3])};
+            u32x4 w = {pack_out2<OutT>(lo[0], lo[1]), pack_out2<OutT>(lo[2], lo[3]), pack_out2<OutT>(hi[0], hi[1]),
+                       pack_out2<OutT>(hi[2], hi[3])};
             store_z(w, reinterpret_cast<u32x4*>(dst), stream);
           } else {
-            u32x2 w = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+            u32x2 w = {pack_out2<OutT>(lo[0], lo[1]), pack_out2<OutT>(lo[2], lo[3])};
             store_z(w, reinterpret_cast<u32x2*>(dst), stream);
           }
         }

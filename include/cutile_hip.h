@@ -427,6 +427,18 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* group_gemm_f16_nt_desc<BM, BN, BK, NUM_SM>(a_ptrs, b_ptrs, c_ptrs: [groups] i64 device addresses; a_metas, b_metas,
+ * c_metas: [groups, 8] i32 rows = (rows, cols, row stride in elements, ...); num_groups) —
+ * cutile-kernels/src/experimental/moe.rs:67-128: C_g [m, n] = A_g [m, k] . B_g [k, n] per group, f16 with f32
+ * accumulation, NUM_SM persistent tile blocks over the tiles of all groups.  The descriptors live in device memory and
+ * are trusted as in the reference (16-byte aligned pointers, rows / cols multiples of 16, row strides multiples of 8).
+ * There is no partition to infer from: the grid comes from opts->grid or generic 3 (NUM_SM), the tile from generics
+ * 0 and 1 (BM, BN; default 128 x 128). */
+cutile_status_t cutile_launch_group_gemm_f16_nt_desc(cutile_stream_t stream, const cutile_tensor_arg_t* a_ptrs,
+                                                     const cutile_tensor_arg_t* b_ptrs, const cutile_tensor_arg_t* c_ptrs,
+                                                     const cutile_tensor_arg_t* a_metas, const cutile_tensor_arg_t* b_metas,
+                                                     const cutile_tensor_arg_t* c_metas, int32_t num_groups,
+                                                     const cutile_launch_opts_t* opts);
 /* argmax_blocks_f16<BLOCK_SIZE>(logits: [n] f16, block_max: [blocks] f32 tiles [1], block_idx: [blocks] u32 tiles [1],
  * len) — cutile-kernels/src/argmax.rs:21-71.  Block b holds the largest of logits[b*BLOCK_SIZE ..] (positions >= len
  * count as -1e30) and the smallest index that attains it.  BLOCK_SIZE is generic 0 (default 1024). */
