@@ -915,6 +915,8 @@ __device__ __forceinline__ void group_gemm_desc(const TensorArg<1>& a_ptrs, cons
     z.pshape[0] = BM, z.pshape[1] = BN;
     while (tile_idx >= group_start && tile_idx < group_start + tiles) {
       const uint32_t in_group = tile_idx - group_start;
+      // (consecutive positions run on different XCDs; with a tile row of 8 or 16 tiles every XCD keeps meeting the same
+      // one or two B panels, which measured better than handing each XCD a contiguous eighth of the group: 3.8 against 5.8 GB)
       G::run_tile(z, a, b, k, in_group / tiles_n, in_group % tiles_n, 0);
       __syncthreads();   // the output bands live in the stages that the next tile refills
       tile_idx += gridDim.x;
