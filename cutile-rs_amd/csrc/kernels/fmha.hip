@@ -91,17 +91,20 @@ struct Elem<_Float16> {
 // Causal launches do the same with a few heads side by side per XCD, heaviest tiles
 // first (see below); one head at a time measured slower than the plain order because the
 // last head's long tiles start late.
-__device__ __forceinline__ void head_and_tile(uint32_t n_bh, uint32_t n_qt, int32_t causal, int32_t* bh, int32_t* q_tile) {
+__device__ __forceinline__ void head_and_tile(uint32_t n_bh, uint32_t n_qt, int32_t causal, uint32_t group, int32_t* bh, int32_t* q_tile) {
   constexpr uint32_t kNumXcd = 8;
   const uint32_t id = blockIdx.x + gridDim.x * blockIdx.y;
   uint32_t b, t;
   constexpr uint32_t kCusPerXcd = 32;
-  const uint32_t side = n_qt >= kCusPerXcd ? 1 : kCusPerXcd / n_qt;     // heads an XCD works on side by side
-  if (n_bh % kNumXcd == 0 && !causal) {
+  uint32_t side = n_qt >= kCusPerXcd ? 1 : kCusPerXcd / n_qt;     // heads an XCD works on side by side
+  // Query heads that share a KV head (consecutive, `group` of them) run side by side on one XCD, tile for tile, so
+  // that the K/V rows one of them fetches serve all of them.
+  if (group > 1) side = (side + group - 1) / group * group;
+  if (n_bh % kNumXcd == 0 && !causal && group <= 1) {
     const uint32_t xcd = id % kNumXcd, slot = id / kNumXcd;
     b = (slot / n_qt) * kNumXcd + xcd;
     t = slot % n_qt;
-  } else if (n_bh % (kNumXcd * side) == 0 && causal) {
+  } else if (n_bh % (kNumXcd * side) == 0 && (causal || group > 1)) {
     // Causal tiles differ n_qt-fold in length.  An XCD takes `side` heads at a time (their K/V fit its L2) and
     // walks their tiles heaviest first, heads interleaved: the compute units that drew the short tiles of one
     // group free up first and draw the long tiles of the next, so lengths pair up (n_qt + 1 per two tiles).
@@ -154,7 +157,7 @@ struct Fmha {
 
     const int32_t H = q.shape[1];
     int32_t bh, q_tile;
-    head_and_tile(g.x, g.y, causal, &bh, &q_tile);
+    head_and_tile(g.x, g.y, causal, (uint32_t)group_size, &bh, &q_tile);
     const int32_t batch = bh / H, head = bh % H, kv_head = head / group_size;
     const int32_t q_len = q.shape[2], k_len = k.shape[2];
     const int32_t q0 = q_tile * BM + wave * 32;   // first query row of this wavefront
@@ -405,7 +408,7 @@ struct FmhaPingPong {
 
     const int32_t H = q.shape[1];
     int32_t bh, q_tile;
-    head_and_tile(g.x, g.y, causal, &bh, &q_tile);
+    head_and_tile(g.x, g.y, causal, (uint32_t)group_size, &bh, &q_tile);
     const int32_t batch = bh / H, head = bh % H, kv_head = head / group_size;
     const int32_t q_len = q.shape[2], k_len = k.shape[2];
     const int32_t q0 = q_tile * BM + wave * 32;
