@@ -585,6 +585,47 @@ class PrefillAttention(Workload):
                {"max_abs": err, "tolerance": 2e-2, "ok": err <= 2e-2}
 
 
+class FusedQkNormRopeKv(Workload):
+    """qk_norm_rope_kv_prefill_raw_f16 (cutile-kernels/src/experimental/fused_transformer.rs:22-345): Q/K norm, rotary
+    embedding and KV-cache update in one pass; every q, k, v element is read once and written once."""
+    name, unit, dtype = "qk_norm_rope_kv_f16_32768x48x128", "GB/s", "f16 io / f32 math"
+    seq, nq, nkv, d = 32768, 32, 8, 128
+    work = 4.0 * seq * (nq + 2 * nkv) * d
+    config = {"workload": "qk_norm_rope_kv_prefill_raw fp16: 32768 positions x (32 q + 8 k + 8 v heads) x 128, caches [8, 32768, 128]"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        f16 = lambda shape, seed: oracle.f32_to_f16_bits(oracle.normal_f32(shape, seed))
+        self.qb, self.kb, self.vb = f16((self.seq, self.nq, self.d), 71), f16((self.seq, self.nkv, self.d), 72), f16((self.seq, self.nkv, self.d), 73)
+        self.qwb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.d, 74, 0.5, 1.5))
+        self.kwb = oracle.f32_to_f16_bits(oracle.uniform_f32(self.d, 75, 0.5, 1.5))
+        self.inv = (1.0 / 10000.0 ** (np.arange(self.d // 2) / (self.d // 2))).astype(np.float32)
+        td = lambda bits: torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.float16)
+        self.q, self.k, self.v, self.qw, self.kw = td(self.qb), td(self.kb), td(self.vb), td(self.qwb), td(self.kwb)
+        self.invd = torch.from_numpy(self.inv).to(dev)
+        self.qo = torch.zeros_like(self.q)
+        self.kc = torch.zeros(self.nkv, self.seq, self.d, dtype=torch.float16, device=dev)
+        self.vc = torch.zeros_like(self.kc)
+
+    def launch(self):
+        self.ct.qk_norm_rope_kv_prefill_raw_f16(self.q, self.k, self.v, self.qw, self.kw, self.invd, self.qo, self.kc, self.vc, 1e-6, 0, self.seq)
+
+    def cpu_baseline(self, oracle, np, torch):
+        n = 2048
+        kc0 = np.zeros((self.nkv, n, self.d), np.uint16)
+        t0 = time.perf_counter()
+        rq, rk, rv = oracle.qk_norm_rope_kv_f16(self.qb[:n], self.kb[:n], self.vb[:n], self.qwb, self.kwb, self.inv, kc0, kc0, 1e-6, 0)
+        dt = time.perf_counter() - t0
+        bits = lambda t: t.cpu().numpy().view(np.uint16)
+        f = oracle.f16_bits_to_f32
+        err = max(float(np.max(np.abs(f(bits(self.qo[:n])) - f(rq)))), float(np.max(np.abs(f(bits(self.kc[:, :n])) - f(rk)))))
+        exact = bool(np.array_equal(bits(self.vc[:, :n]), rv))
+        return {"value": 4.0 * n * (self.nq + 2 * self.nkv) * self.d / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {n} of {self.seq} positions"}, {"max_abs": err, "tolerance": 4e-3, "ok": err <= 4e-3 and exact, "v_bit_exact": exact}
+
+
 class GroupGemm(Workload):
     """group_gemm_f16_nt_desc (cutile-kernels/src/experimental/moe.rs:67-128): expert batches of unequal size, one launch."""
     name, unit, bound, peak_key = "group_gemm_f16_32x4096x4096", "TFLOP/s", "mfma", "mfma_bf16"
@@ -704,7 +745,7 @@ class EmbeddingBatch(Workload):
 
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

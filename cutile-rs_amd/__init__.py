@@ -128,6 +128,8 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_qk_norm_rope_kv_prefill_raw_f16": [vp] + [vp] * 9 + [f32, i32, i32, i32, i32, i32, i32, P(LaunchOpts)],
+            "cutile_launch_qk_norm_rope_kv_decode_raw_f16": [vp] + [vp] * 7 + [P(TensorArg), f32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_group_gemm_f16_nt_desc": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg),
                                                      P(TensorArg), i32, P(LaunchOpts)],
             "cutile_launch_argmax_blocks_f16": [vp, P(TensorArg), P(PartitionArg), P(PartitionArg), i32, P(LaunchOpts)],
@@ -480,6 +482,31 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def qk_norm_rope_kv_prefill_raw_f16(q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache, eps: float, position_start: int,
+                                    seq_len: int, *, stream=None, generics=None) -> None:
+    """cutile-kernels/src/experimental/fused_transformer.rs:22-345; the reference takes raw pointers, this wrapper takes the
+    contiguous tensors q [seq, q_heads, D], k / v [seq, kv_heads, D], caches [kv_heads, MAX_SEQ, D] and passes their addresses"""
+    o, _k = _opts(None, generics, None)
+    for t in (q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache):
+        if not t.is_contiguous():
+            raise CutileError(-5, "qk_norm_rope_kv_prefill_raw_f16: raw-pointer kernel, every tensor must be contiguous")
+    check(lib().cutile_launch_qk_norm_rope_kv_prefill_raw_f16(
+        _stream(stream), *[C.c_void_p(t.data_ptr()) for t in (q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache)],
+        C.c_float(eps), int(position_start), int(seq_len), int(q.shape[1]), int(k.shape[1]), int(q.shape[2]), int(k_cache.shape[1]),
+        C.byref(o)))
+
+
+def qk_norm_rope_kv_decode_raw_f16(qkv, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache, position_start, eps: float,
+                                   num_q_heads: int, num_kv_heads: int, *, stream=None, generics=None) -> None:
+    """cutile-kernels/src/experimental/fused_transformer.rs:356-625; qkv: one token's q, k and v heads back to back"""
+    o, _k = _opts(None, generics, None)
+    pa = tensor_arg(position_start, dtype=U32)
+    d = int(k_cache.shape[2])
+    check(lib().cutile_launch_qk_norm_rope_kv_decode_raw_f16(
+        _stream(stream), *[C.c_void_p(t.data_ptr()) for t in (qkv, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache)],
+        C.byref(pa), C.c_float(eps), int(num_q_heads), int(num_kv_heads), d, int(k_cache.shape[1]), C.byref(o)))
 
 
 def group_gemm_f16_nt_desc(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups: int, *, stream=None, grid=None,

@@ -1042,6 +1042,91 @@ cutile_status_t cutile_launch_gather_row_f16(cutile_stream_t stream, const cutil
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// ---- fused Q/K norm + RoPE + KV-cache update (cutile-kernels/src/experimental/fused_transformer.rs) ----
+static cutile_status_t launch_qk_norm_rope_kv(const char* name, cutile_stream_t stream, const void* q, const void* k, const void* v,
+                                              const void* q_weight, const void* k_weight, const void* inv_freq, void* q_out,
+                                              void* k_cache, void* v_cache, const void* pos_dev, float eps, int32_t position_start,
+                                              int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t d,
+                                              int32_t max_seq, int64_t q_row_stride, int64_t kv_row_stride,
+                                              const cutile_launch_opts_t* opts) {
+  const void* ptrs[9] = {q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache};
+  for (const void* p : ptrs) {
+    CUTILE_REQUIRE(p, CUTILE_ERR_INVALID_ARGUMENT, "%s: null device pointer", name);
+    CUTILE_REQUIRE(p == inv_freq ? ((uintptr_t)p & 3) == 0 : aligned16(p), CUTILE_ERR_KERNEL_LAUNCH,
+                   "%s: device pointers must be 16-byte aligned (inv_freq: 4)", name);
+  }
+  CUTILE_REQUIRE(d > 0 && d % 16 == 0 && d <= 2048, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "%s: D = %d must be a multiple of 16, at most 2048, with D/16 a power of two", name, d);
+  CUTILE_REQUIRE(((d / 16) & (d / 16 - 1)) == 0 && d / 16 <= 64, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "%s: D = %d must be a multiple of 16, at most 2048, with D/16 a power of two", name, d);
+  CUTILE_REQUIRE(seq_len >= 0 && num_q_heads >= 0 && num_kv_heads >= 0 && max_seq > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: seq_len, head counts must be non-negative and MAX_SEQ positive", name);
+  if (!pos_dev)
+    CUTILE_REQUIRE(position_start >= 0 && (int64_t)position_start + seq_len <= max_seq, CUTILE_ERR_KERNEL_LAUNCH,
+                   "%s: positions %d .. %lld do not fit the %d rows of the caches", name, position_start,
+                   (long long)position_start + seq_len, max_seq);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(d / 2), "HALF_D")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(max_seq), "MAX_SEQ")) return s;
+  if (seq_len == 0 || num_q_heads + num_kv_heads == 0) return CUTILE_SUCCESS;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("qk_norm_rope_kv", &o, "f16", {"f16"}, &res)) return s;
+  ArgPacker args;
+  for (const void* p : ptrs) args.push_val<const void*>(p);
+  args.push_val<const void*>(pos_dev);
+  args.push_val<float>(eps);
+  args.push_val<int32_t>(position_start);
+  args.push_val<int32_t>(seq_len);
+  args.push_val<int32_t>(num_q_heads);
+  args.push_val<int32_t>(num_kv_heads);
+  args.push_val<int32_t>(d);
+  args.push_val<int32_t>(max_seq);
+  args.push_val<int64_t>(q_row_stride);
+  args.push_val<int64_t>(kv_row_stride);
+  uint32_t grid[3] = {std::min<uint32_t>((uint32_t)seq_len, 1u << 20), 1, 1};   // one workgroup per position
+  // lanes per workgroup: rows * D/16 lane slots per position; the size that idles the fewest lanes in the last pass
+  const uint32_t lane_slots = (uint32_t)(num_q_heads + 2 * num_kv_heads) * (uint32_t)(d / 16);
+  uint32_t block[3] = {256, 1, 1}, best_idle = UINT32_MAX;
+  for (uint32_t b : {256u, 192u, 128u, 64u}) {
+    const uint32_t idle = (lane_slots + b - 1) / b * b - lane_slots;
+    if (idle < best_idle) best_idle = idle, block[0] = b;
+  }
+  return launch_packed(res.fn, grid, block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_qk_norm_rope_kv_prefill_raw_f16(cutile_stream_t stream, const void* q, const void* k,
+                                                              const void* v, const void* q_weight, const void* k_weight,
+                                                              const void* inv_freq, void* q_out, void* k_cache,
+                                                              void* v_cache, float eps, int32_t position_start,
+                                                              int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                                                              int32_t d, int32_t max_seq, const cutile_launch_opts_t* opts) {
+  return launch_qk_norm_rope_kv("qk_norm_rope_kv_prefill_raw_f16", stream, q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache,
+                                v_cache, nullptr, eps, position_start, seq_len, num_q_heads, num_kv_heads, d, max_seq,
+                                (int64_t)num_q_heads * d, (int64_t)num_kv_heads * d, opts);
+}
+
+cutile_status_t cutile_launch_qk_norm_rope_kv_decode_raw_f16(cutile_stream_t stream, const void* qkv, const void* q_weight,
+                                                             const void* k_weight, const void* inv_freq, void* q_out,
+                                                             void* k_cache, void* v_cache,
+                                                             const cutile_tensor_arg_t* position_start, float eps,
+                                                             int32_t num_q_heads, int32_t num_kv_heads, int32_t d,
+                                                             int32_t max_seq, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(position_start, "position_start", 1, 1)) return s;
+  CUTILE_REQUIRE(position_start->dtype == CUTILE_DTYPE_U32 && position_start->shape[0] == 1 && ((uintptr_t)position_start->ptr & 3) == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "qk_norm_rope_kv_decode_raw_f16: position_start must be one aligned u32");
+  CUTILE_REQUIRE(qkv && num_q_heads >= 0 && num_kv_heads >= 0 && d > 0, CUTILE_ERR_INVALID_ARGUMENT,
+                 "qk_norm_rope_kv_decode_raw_f16: null qkv or negative head count");
+  const char* bytes = (const char*)qkv;
+  const void* k = bytes + (size_t)num_q_heads * d * 2;
+  const void* v = bytes + (size_t)(num_q_heads + num_kv_heads) * d * 2;
+  return launch_qk_norm_rope_kv("qk_norm_rope_kv_decode_raw_f16", stream, qkv, k, v, q_weight, k_weight, inv_freq, q_out, k_cache,
+                                v_cache, position_start->ptr, eps, 0, 1, num_q_heads, num_kv_heads, d, max_seq,
+                                (int64_t)num_q_heads * d, (int64_t)num_kv_heads * d, opts);
+}
+
 static bool decode_vec_layout(const cutile_tensor_arg_t& t) {
   return t.strides[2] == 1 && t.strides[1] % 8 == 0 && t.strides[0] % 8 == 0 && aligned16(t.ptr);
 }

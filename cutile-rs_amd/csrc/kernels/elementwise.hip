@@ -725,3 +725,112 @@ extern "C" __global__ void __launch_bounds__(kThreads)
   for (int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x; c < width; c += (int64_t)gridDim.x * kThreads)
     op[c * out.strides[0]] = known && c < src.shape[1] ? sp[c * src.strides[1]] : (_Float16)0;
 }
+
+// ---- fused Q/K norm + rotary embedding + KV-cache update -------------------------------------
+// qk_norm_rope_kv_prefill_raw_f16 / qk_norm_rope_kv_decode_raw_f16
+// (cutile-kernels/src/experimental/fused_transformer.rs:22-345, 356-625), raw device pointers as there.
+// For position s of the launch and head h: a q or k row [D] is RMS-normalised with its weight in f32
+// (x * rsqrt(mean(x^2) + eps) * w, :182-240) and rotated, still in f32, by the angles
+// (position_start + s) * inv_freq (:242-258); q rows go to q_out[s, h], k rows to
+// k_cache[h, position_start + s], and the v row is copied to v_cache[h, position_start + s] (:263-341).
+// q, q_out: rows of num_q_heads * D every q_row_stride elements; k, v: num_kv_heads * D every kv_row_stride;
+// the caches are [num_kv_heads, max_seq, D].  The decode form is the same work for one position whose q, k
+// and v rows sit back to back and whose position is read from device memory.
+// One workgroup per position: the D/2 (cos, sin) pairs are computed once into LDS; a lane holds 8 rotation
+// pairs of one row (two 16-byte accesses), D/16 neighbouring lanes hold a row and sum its squares.  The workgroup
+// size (64 .. 256 lanes) is the launcher's: the one that leaves the fewest lanes idle in the last pass over the rows.
+namespace {
+struct FusedRowsArgs {
+  const _Float16 *q, *k, *v, *q_weight, *k_weight;
+  _Float16 *q_out, *k_cache, *v_cache;
+  float eps;
+  int32_t num_q_heads, num_kv_heads, d, half, chunks, chunk_shift, max_seq, rows;
+  int64_t q_row_stride, kv_row_stride;
+};
+// where row r of position s_idx comes from
+__device__ __forceinline__ const _Float16* fused_source(const FusedRowsArgs& a, int64_t s_idx, int32_t r) {
+  if (r < a.num_q_heads) return a.q + s_idx * a.q_row_stride + (int64_t)r * a.d;
+  if (r < a.num_q_heads + a.num_kv_heads) return a.k + s_idx * a.kv_row_stride + (int64_t)(r - a.num_q_heads) * a.d;
+  return a.v + s_idx * a.kv_row_stride + (int64_t)(r - a.num_q_heads - a.num_kv_heads) * a.d;
+}
+// norm + rotation (q, k rows) or copy (v rows) of the 16 elements this lane holds of lane slot t
+__device__ __forceinline__ void fused_finish(const FusedRowsArgs& a, int64_t s_idx, int32_t pos_i, int32_t t, u32x4 lo_raw,
+                                             u32x4 hi_raw, const float* cs_tab, const float* sn_tab) {
+  Vec16<_Float16> lo, hi;
+  lo.raw = lo_raw;
+  hi.raw = hi_raw;
+  const int32_t r = t >> a.chunk_shift, c = t & (a.chunks - 1);
+  const bool is_q = r < a.num_q_heads, is_k = !is_q && r < a.num_q_heads + a.num_kv_heads;
+  float ss = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float l = (float)lo.v[e], h = (float)hi.v[e];
+    ss += l * l + h * h;
+  }
+  for (int32_t o = a.chunks >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  if (r >= a.rows || (!is_q && (pos_i < 0 || pos_i >= a.max_seq))) return;
+  _Float16* dst;
+  if (is_q) {
+    dst = a.q_out + s_idx * a.q_row_stride + (int64_t)r * a.d;
+  } else {
+    const int32_t kv_head = is_k ? r - a.num_q_heads : r - a.num_q_heads - a.num_kv_heads;
+    dst = (is_k ? a.k_cache : a.v_cache) + ((int64_t)kv_head * a.max_seq + pos_i) * a.d;
+  }
+  if (is_q || is_k) {
+    const float inv = __builtin_amdgcn_rsqf(ss / (float)a.d + a.eps);
+    const _Float16* w = is_q ? a.q_weight : a.k_weight;
+    Vec16<_Float16> wlo, whi, ylo, yhi;
+    wlo.raw = reinterpret_cast<const u32x4*>(w)[c];
+    whi.raw = reinterpret_cast<const u32x4*>(w + a.half)[c];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float nl = ((float)lo.v[e] * inv) * (float)wlo.v[e], nh = ((float)hi.v[e] * inv) * (float)whi.v[e];
+      const float cs = cs_tab[c * 8 + e], sn = sn_tab[c * 8 + e];
+      ylo.v[e] = (_Float16)(nl * cs - nh * sn);
+      yhi.v[e] = (_Float16)(nh * cs + nl * sn);
+    }
+    lo.raw = ylo.raw;
+    hi.raw = yhi.raw;
+  }
+  reinterpret_cast<u32x4*>(dst)[c] = lo.raw;
+  reinterpret_cast<u32x4*>(dst + a.half)[c] = hi.raw;
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(kThreads)
+    qk_norm_rope_kv_entry__f16(const _Float16* q, const _Float16* k, const _Float16* v, const _Float16* q_weight,
+                               const _Float16* k_weight, const float* inv_freq, _Float16* q_out, _Float16* k_cache,
+                               _Float16* v_cache, const uint32_t* pos_dev, float eps, int32_t position_start,
+                               int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t d, int32_t max_seq,
+                               int64_t q_row_stride, int64_t kv_row_stride) {
+  constexpr int kTable = 1024;                           // (cos, sin) pairs kept in LDS
+  __shared__ float cs_tab[kTable], sn_tab[kTable];
+  FusedRowsArgs a;
+  a.q = q, a.k = k, a.v = v, a.q_weight = q_weight, a.k_weight = k_weight;
+  a.q_out = q_out, a.k_cache = k_cache, a.v_cache = v_cache;
+  a.eps = eps, a.num_q_heads = num_q_heads, a.num_kv_heads = num_kv_heads, a.d = d, a.max_seq = max_seq;
+  a.half = d >> 1, a.chunks = d >> 4;                    // a lane: elements [8c, 8c+8) of both halves
+  a.chunk_shift = 31 - __builtin_clz((uint32_t)a.chunks);   // D/16 is a power of two
+  a.rows = num_q_heads + 2 * num_kv_heads;
+  a.q_row_stride = q_row_stride, a.kv_row_stride = kv_row_stride;
+  const int32_t base = pos_dev ? (int32_t)pos_dev[0] : position_start;
+  const int32_t threads = (int32_t)blockDim.x;          // chosen by the launcher so that the lane slots fill whole passes
+  const int32_t slots = (a.rows * a.chunks + threads - 1) / threads * threads;   // whole lane groups stay together
+  for (int64_t s_idx = blockIdx.x; s_idx < seq_len; s_idx += gridDim.x) {
+    const int32_t pos_i = base + (int32_t)s_idx;
+    __syncthreads();                                   // the previous position's table is no longer read
+    for (int32_t i = threadIdx.x; i < a.half; i += threads) sincosf((float)pos_i * inv_freq[i], &sn_tab[i], &cs_tab[i]);
+    __syncthreads();
+    // (requesting rows before the table is computed costs registers, hence residency: measured 4.9 - 5.3 against 5.4 TB/s)
+    for (int32_t t = (int32_t)threadIdx.x; t < slots; t += threads) {
+      const int32_t r = t >> a.chunk_shift, c = t & (a.chunks - 1);
+      u32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      if (r < a.rows) {
+        const _Float16* src = fused_source(a, s_idx, r);
+        lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + c);
+        hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + a.half) + c);
+      }
+      fused_finish(a, s_idx, pos_i, t, lo, hi, cs_tab, sn_tab);
+    }
+  }
+}

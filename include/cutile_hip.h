@@ -427,6 +427,28 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* qk_norm_rope_kv_prefill_raw_f16<D, HALF_D, MAX_SEQ>(q_ptr, k_ptr, v_ptr, q_weight_ptr, k_weight_ptr, inv_freq_ptr,
+ * q_out_ptr, k_cache_ptr, v_cache_ptr, eps, position_start, seq_len, num_q_heads, num_kv_heads) —
+ * cutile-kernels/src/experimental/fused_transformer.rs:22-345.  Raw device pointers as in the reference: q, q_out
+ * [seq_len, num_q_heads, D], k, v [seq_len, num_kv_heads, D], weights [D] (all f16, contiguous, 16-byte aligned),
+ * inv_freq [D/2] f32, caches [num_kv_heads, MAX_SEQ, D].  One launch does Q/K RMS norm, rotary embedding at positions
+ * position_start + s and the cache update.  D and MAX_SEQ are arguments here (generics 0 and 2 are checked). */
+cutile_status_t cutile_launch_qk_norm_rope_kv_prefill_raw_f16(cutile_stream_t stream, const void* q, const void* k,
+                                                              const void* v, const void* q_weight, const void* k_weight,
+                                                              const void* inv_freq, void* q_out, void* k_cache,
+                                                              void* v_cache, float eps, int32_t position_start,
+                                                              int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
+                                                              int32_t d, int32_t max_seq, const cutile_launch_opts_t* opts);
+/* qk_norm_rope_kv_decode_raw_f16<D, HALF_D, MAX_SEQ>(qkv_ptr, q_weight_ptr, k_weight_ptr, inv_freq_ptr, q_out_ptr,
+ * k_cache_ptr, v_cache_ptr, position_start: [1] u32, eps, num_q_heads, num_kv_heads) — fused_transformer.rs:356-625:
+ * the same for one token whose q, k and v heads sit back to back in qkv [(num_q_heads + 2 num_kv_heads) * D] and whose
+ * position is read from device memory. */
+cutile_status_t cutile_launch_qk_norm_rope_kv_decode_raw_f16(cutile_stream_t stream, const void* qkv, const void* q_weight,
+                                                             const void* k_weight, const void* inv_freq, void* q_out,
+                                                             void* k_cache, void* v_cache,
+                                                             const cutile_tensor_arg_t* position_start, float eps,
+                                                             int32_t num_q_heads, int32_t num_kv_heads, int32_t d,
+                                                             int32_t max_seq, const cutile_launch_opts_t* opts);
 /* group_gemm_f16_nt_desc<BM, BN, BK, NUM_SM>(a_ptrs, b_ptrs, c_ptrs: [groups] i64 device addresses; a_metas, b_metas,
  * c_metas: [groups, 8] i32 rows = (rows, cols, row stride in elements, ...); num_groups) —
  * cutile-kernels/src/experimental/moe.rs:67-128: C_g [m, n] = A_g [m, k] . B_g [k, n] per group, f16 with f32

@@ -74,6 +74,7 @@ def lib() -> C.CDLL:
             "orc_gemm_bf16": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_gemm_bf16_f32out": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_fmha_ref_cpu": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp, i64]),
+            "orc_qk_norm_rope_kv_f16": (None, [vp] * 9 + [f32, i64, i64, i64, i64, i64, i64]),
             "orc_argmax_blocks_f16": (None, [vp, i64, i64, i64, vp, vp, i64]),
             "orc_lm_head_argmax_blocks_f16": (None, [vp, vp, i64, i64, i64, vp, vp, i64]),
             "orc_argmax_reduce_blocks_to_u32": (C.c_uint32, [vp, vp, i64, i64, i64]),
@@ -386,6 +387,20 @@ def attention_seq_ref(q, k, v, qk_scale: float, query_group_size: int, kv_len: i
     lib().orc_attention_seq_ref(_p(q), _p(k), _p(v), _p(out), q_len, q_heads, kv_heads, max_seq, d, qk_scale,
                                 query_group_size, int(kv_len), int(query_start), int(causal))
     return out
+
+
+def qk_norm_rope_kv_f16(q_bits, k_bits, v_bits, qw_bits, kw_bits, inv_freq, k_cache_bits, v_cache_bits, eps: float,
+                        position_start: int):
+    """fused_transformer.rs:22-345 -> (q_out bits [seq, nq, d], k_cache bits, v_cache bits); the caches are copied first"""
+    q_bits, k_bits, v_bits = _c(q_bits, np.uint16), _c(k_bits, np.uint16), _c(v_bits, np.uint16)
+    qw_bits, kw_bits, inv_freq = _c(qw_bits, np.uint16), _c(kw_bits, np.uint16), _c(inv_freq, np.float32)
+    seq, nq, d = q_bits.shape
+    nkv = k_bits.shape[1]
+    kc, vc = _c(k_cache_bits, np.uint16).copy(), _c(v_cache_bits, np.uint16).copy()
+    q_out = np.empty_like(q_bits)
+    lib().orc_qk_norm_rope_kv_f16(_p(q_bits), _p(k_bits), _p(v_bits), _p(qw_bits), _p(kw_bits), _p(inv_freq), _p(q_out), _p(kc),
+                                  _p(vc), eps, int(position_start), seq, nq, nkv, d, kc.shape[1])
+    return q_out, kc, vc
 
 
 # ---- greedy sampling and row gathers (cutile-kernels/src/argmax.rs, embeddings.rs, pointwise.rs) ----

@@ -881,3 +881,43 @@ uint32_t orc_argmax_reduce_blocks_to_u32(const float* block_max, const uint32_t*
   free(idx);
   return out;
 }
+
+/* qk_norm_rope_kv_prefill_raw_f16 (cutile-kernels/src/experimental/fused_transformer.rs:22-345; the decode form
+ * :356-625 is the same for seq_len = 1).  q [seq, nq, d], k and v [seq, nkv, d], caches [nkv, max_seq, d].  Per row:
+ * ss = sum(x_lo^2 + x_hi^2) (:182-184), inv = rsqrt(ss / D + eps) (:185-189), norm = x * inv * w in f32 (:239-240),
+ * theta = f32(position_start + s) * inv_freq (:249-254), y_lo = n_lo cos - n_hi sin, y_hi = n_hi cos + n_lo sin
+ * (:257-258), one rounding to f16 (:259-260); q rows to q_out, k rows to k_cache[h, position], v copied (:263-341). */
+void orc_qk_norm_rope_kv_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* qw,
+                             const uint16_t* kw, const float* inv_freq, uint16_t* q_out, uint16_t* k_cache,
+                             uint16_t* v_cache, float eps, int64_t position_start, int64_t seq_len, int64_t nq,
+                             int64_t nkv, int64_t d, int64_t max_seq) {
+  const int64_t half = d / 2;
+  for (int64_t s = 0; s < seq_len; s++) {
+    const int64_t pos_i = position_start + s;
+    const float pos = (float)pos_i;
+    for (int64_t r = 0; r < nq + nkv; r++) {
+      const int is_q = r < nq;
+      const uint16_t* x = is_q ? q + (s * nq + r) * d : k + (s * nkv + (r - nq)) * d;
+      const uint16_t* w = is_q ? qw : kw;
+      uint16_t* dst = is_q ? q_out + (s * nq + r) * d : k_cache + ((r - nq) * max_seq + pos_i) * d;
+      if (!is_q && (pos_i < 0 || pos_i >= max_seq)) continue;
+      float ss = 0.0f;
+      for (int64_t i = 0; i < half; i++) {
+        float lo = orc_f16_to_f32(x[i]), hi = orc_f16_to_f32(x[half + i]);
+        ss += lo * lo + hi * hi;
+      }
+      const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+      for (int64_t i = 0; i < half; i++) {
+        const float nl = orc_f16_to_f32(x[i]) * inv * orc_f16_to_f32(w[i]);
+        const float nh = orc_f16_to_f32(x[half + i]) * inv * orc_f16_to_f32(w[half + i]);
+        const float theta = pos * inv_freq[i];
+        const float cs = cosf(theta), sn = sinf(theta);
+        dst[i] = orc_f32_to_f16(nl * cs - nh * sn);
+        dst[half + i] = orc_f32_to_f16(nh * cs + nl * sn);
+      }
+    }
+    if (pos_i >= 0 && pos_i < max_seq)
+      for (int64_t h = 0; h < nkv; h++)
+        memcpy(v_cache + (h * max_seq + pos_i) * d, v + (s * nkv + h) * d, sizeof(uint16_t) * (size_t)d);
+  }
+}

@@ -42,6 +42,14 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_qk_norm_rope_kv_f16
+ *                        cutile-kernels/src/experimental/fused_transformer.rs (kernel bodies).
+ *                        Pinned by orc_rms_norm_f16 at position 0 (no rotation), by
+ *                        orc_qk_norm_f16 -> orc_rope_seq_f16 -> orc_kv_cache_update_f16 (equal
+ *                        up to the f16 rounding between the separate kernels), by a float64
+ *                        evaluation, the norm-preserving rotation and exact copies of v;
+ *                        the reference only compiles these kernels: parity unpinned by
+ *                        reference tests.
  *   orc_argmax_blocks_f16, orc_lm_head_argmax_blocks_f16, orc_argmax_reduce_blocks_to_u32
  *                        cutile-kernels/src/argmax.rs (kernel bodies).  Pinned by numpy.argmax
  *                        (first index of the maximum) block by block and through the
@@ -130,6 +138,11 @@ void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, i
 void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
                              uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
                              int64_t position_start, int64_t seq_len);
+/* fused Q/K norm + RoPE + KV-cache update: cutile-kernels/src/experimental/fused_transformer.rs:22-345, 356-625 */
+void orc_qk_norm_rope_kv_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* qw,
+                             const uint16_t* kw, const float* inv_freq, uint16_t* q_out, uint16_t* k_cache,
+                             uint16_t* v_cache, float eps, int64_t position_start, int64_t seq_len, int64_t nq,
+                             int64_t nkv, int64_t d, int64_t max_seq);
 /* greedy sampling: cutile-kernels/src/argmax.rs:21-71, 88-158, 173-213 */
 void orc_argmax_blocks_f16(const uint16_t* logits, int64_t n, int64_t block_size, int64_t len, float* block_max,
                            uint32_t* block_idx, int64_t num_blocks);
