@@ -165,6 +165,13 @@ def lib() -> C.CDLL:
             "cutile_stream_release": [vp, vp],
             "cutile_stream_synchronize": [vp],
             "cutile_stream_query": [vp, P(i32)],
+            "cutile_stream_begin_capture": [vp],
+            "cutile_stream_end_capture": [vp, P(vp)],
+            "cutile_graph_instantiate": [vp, P(vp)],
+            "cutile_graph_upload": [vp, vp],
+            "cutile_graph_launch": [vp, vp],
+            "cutile_graph_exec_destroy": [vp],
+            "cutile_graph_destroy": [vp],
             "cutile_event_create": [P(vp)],
             "cutile_event_record": [vp, vp],
             "cutile_event_synchronize": [vp],
@@ -639,6 +646,48 @@ def kernel_lookup(function: str, generics: Sequence[str] = (), variant: Optional
     check(lib().cutile_kernel_lookup(device(ordinal), function.encode(), arr, len(generics),
                                      variant.encode() if variant else None, C.byref(info)))
     return info
+
+
+class CapturedGraph:
+    """Stream capture and replay through the C ABI (cuda-async/src/cuda_graph.rs:61-244): the launches `record` issues on
+    this object's stream are captured once and replayed with one call per step.
+
+        g = CapturedGraph().capture(lambda stream: (ct.saxpy(..., stream=stream), ct.add(..., stream=stream)))
+        g.launch(); g.synchronize()
+    """
+
+    def __init__(self, device: int = 0):
+        self.device, self.stream, self.graph, self.exec_ = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+        check(lib().cutile_device_get(int(device), C.byref(self.device)))
+        check(lib().cutile_stream_create(self.device, C.byref(self.stream)))
+
+    def capture(self, record) -> "CapturedGraph":
+        check(lib().cutile_stream_begin_capture(self.stream))
+        try:
+            record(self.stream.value)
+        finally:
+            status = lib().cutile_stream_end_capture(self.stream, C.byref(self.graph))
+        check(status)
+        check(lib().cutile_graph_instantiate(self.graph, C.byref(self.exec_)))
+        check(lib().cutile_graph_upload(self.exec_, self.stream))
+        return self
+
+    def launch(self) -> None:
+        check(lib().cutile_graph_launch(self.exec_, self.stream))
+
+    def synchronize(self) -> None:
+        check(lib().cutile_stream_synchronize(self.stream))
+
+    def close(self) -> None:
+        if self.exec_:
+            lib().cutile_graph_exec_destroy(self.exec_)
+            self.exec_ = C.c_void_p()
+        if self.graph:
+            lib().cutile_graph_destroy(self.graph)
+            self.graph = C.c_void_p()
+        if self.stream:
+            lib().cutile_stream_release(self.device, self.stream)
+            self.stream = C.c_void_p()
 
 
 class EventTimer:

@@ -211,3 +211,43 @@ def test_gpu_decode_rejects_what_no_variant_covers(ct, dev):
     with pytest.raises(ct.CutileError, match="NUM_KV_SPLITS"):
         ct.fmha_decode_gqa_split(q4, kv, kv, ct.partition(att4, [1, 4, 128]), ct.partition(lse4, [1, 4]), 0.1, p,
                                  generics=[4, 64, 128, 3])
+
+
+@pytest.mark.gpu
+def test_gpu_decode_step_replayed_from_a_captured_graph(ct, dev):
+    """one decode step (cache update at the device position, split attention, merge) captured once and replayed with the
+    program's own eager work between the replays: every replay must equal the eager step on the same inputs"""
+    heads, group, d, max_seq, splits = 4, 4, 128, 512, 4
+    rng = np.random.default_rng(77)
+    half = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float16)).to(dev)
+    q, new_k, new_v = half(heads, group, d), half(1, heads, d), half(1, heads, d)
+    k_cache, v_cache = half(heads, max_seq, d), half(heads, max_seq, d)
+    pos = torch.tensor([100], dtype=torch.int32, device=dev)
+    att = torch.zeros(heads, splits * group, d, dtype=torch.float16, device=dev)
+    lse = torch.zeros(heads, splits * group, device=dev)
+    out = torch.zeros(heads, group, d, dtype=torch.float16, device=dev)
+
+    def step(stream=None):
+        ct.kv_cache_update_f16(new_k, new_v, ct.partition(k_cache, [1, max_seq, d]), ct.partition(v_cache, [1, max_seq, d]), pos, 1, stream=stream)
+        ct.fmha_decode_gqa_split(q, k_cache, v_cache, ct.partition(att, [1, group, d]), ct.partition(lse, [1, group]), d ** -0.5, pos, stream=stream)
+        ct.splitk_reduce_merge(att, lse, ct.partition(out, [1, group, d]), stream=stream)
+
+    torch.cuda.synchronize()
+    graph = ct.CapturedGraph().capture(step)
+    try:
+        for it in range(4):
+            # new inputs through the same buffers, written by eager work on torch's stream
+            q.copy_(half(heads, group, d)); new_k.copy_(half(1, heads, d)); new_v.copy_(half(1, heads, d))
+            pos.fill_(100 + 37 * it)
+            saved_k, saved_v = k_cache.clone(), v_cache.clone()
+            torch.cuda.synchronize()
+            graph.launch()
+            graph.synchronize()
+            got, got_k = out.clone(), k_cache.clone()
+            k_cache.copy_(saved_k); v_cache.copy_(saved_v); out.zero_()
+            step()
+            torch.cuda.synchronize()
+            assert torch.equal(got, out) and torch.equal(got_k, k_cache)
+            assert torch.equal(k_cache[:, 100 + 37 * it], new_k[0])
+    finally:
+        graph.close()
