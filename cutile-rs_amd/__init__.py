@@ -111,6 +111,7 @@ def lib() -> C.CDLL:
             "cutile_launch_linspace": [vp, P(PartitionArg), f32, f32, P(LaunchOpts)],
             "cutile_launch_convert": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
+            "cutile_launch_rms_norm_f32": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
             "cutile_launch_softmax": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_add_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
                                                P(PartitionArg), f32, P(LaunchOpts)],
@@ -373,6 +374,14 @@ def rms_norm_f16(x, w, out: Partition, eps: float, *, stream=None, grid=None, ge
     o, _k = _opts(grid, generics, variant)
     xa, wa = tensor_arg(x), tensor_arg(w)
     check(lib().cutile_launch_rms_norm_f16(_stream(stream), C.byref(xa), C.byref(wa), C.byref(out.arg()), float(eps),
+                                           C.byref(o)))
+
+
+def rms_norm_f32(x, w, out: Partition, eps: float, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """the f32 example form, cutile-examples/examples/rms_norm.rs:17-61 (square root rounded toward minus infinity)"""
+    o, _k = _opts(grid, generics, variant)
+    xa, wa = tensor_arg(x), tensor_arg(w)
+    check(lib().cutile_launch_rms_norm_f32(_stream(stream), C.byref(xa), C.byref(wa), C.byref(out.arg()), float(eps),
                                            C.byref(o)))
 
 

@@ -127,6 +127,7 @@ std::vector<KernelEntry> build_table() {
     add(fn, "generic", keep(std::string(fn) + "_entry__generic"), IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   }
   add("rms_norm_f16", "generic", "rms_norm_f16_entry__generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
+  add("rms_norm", "f32", "rms_norm_entry__f32", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);   // the f32 example form
   add("softmax", "f16_generic", "softmax_entry__f16_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   add("softmax", "f32_generic", "softmax_entry__f32_generic", IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
 

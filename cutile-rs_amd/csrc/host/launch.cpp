@@ -686,6 +686,43 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
   return launch_packed(res.fn, grid, res.entry->block, rms_norm_residency_lds(res.entry, n), stream, args);
 }
 
+// rms_norm<N, BLOCK_SIZE> of cutile-examples/examples/rms_norm.rs:17-61: f32 throughout, square root rounded down.
+cutile_status_t cutile_launch_rms_norm_f32(cutile_stream_t stream, const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* w,
+                                           const cutile_partition_arg_t* out, float eps, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(w, "w", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 2, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F32 && w->dtype == CUTILE_DTYPE_F32 && ot.dtype == CUTILE_DTYPE_F32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "rms_norm: x, w and out must be f32");
+  const int32_t n = x->shape[1];
+  CUTILE_REQUIRE(w->shape[0] == n, CUTILE_ERR_KERNEL_LAUNCH, "rms_norm: w has %d elements, expected N = %d", w->shape[0], n);
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == n, CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm: out must be partitioned [1, %d], got [%d, %d]", n, out->partition_shape[0], out->partition_shape[1]);
+  CUTILE_REQUIRE(ot.shape[1] == n && ot.shape[0] <= x->shape[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm: out is [%d, %d] but x is [%d, %d]", ot.shape[0], ot.shape[1], x->shape[0], n);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(n), "N")) return s;
+  const int block = generic_int(opts, 1, 0);
+  CUTILE_REQUIRE(block >= 0 && (block == 0 || n % block == 0), CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm: N = %d is not a multiple of BLOCK_SIZE = %d", n, block);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("rms_norm", &o, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*x);
+  args.push_tensor(*w);
+  args.push_partition(*out);
+  args.push_val<float>(eps);
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>(tg[0], ot.shape[0]);
+  uint32_t grid[3] = {(uint32_t)std::min<uint64_t>(std::max<uint64_t>(rows, 1), 1u << 20), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 // The two fused row norms: same shape rules and variant choice as rms_norm_f16.
 static cutile_status_t launch_fused_norm(const char* fn, cutile_stream_t stream, const cutile_tensor_arg_t* a,
                                          const cutile_tensor_arg_t* b, const cutile_tensor_arg_t* w,

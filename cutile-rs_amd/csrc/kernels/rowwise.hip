@@ -558,6 +558,66 @@ extern "C" __global__ void __launch_bounds__(kThreads)
   rms_norm_row_generic(x, w, out, eps, rows);
 }
 
+// rms_norm<N, BLOCK_SIZE>(x: [-1, N] f32, w: [N] f32, out: [1, N] tiles f32, eps) — the f32 example form
+// (cutile-examples/examples/rms_norm.rs:17-61): scale = sqrt(1 / (sum(x^2) / N + eps)) with the square root rounded
+// toward minus infinity (:44-46), out = x * scale * w (:56).  One workgroup per row, 16-byte accesses where the
+// layout allows it; the row is re-read for the second pass (it is still in L2).
+__device__ __forceinline__ float sqrt_toward_minus_infinity(float v) {
+  float r = __builtin_sqrtf(v);                        // correctly rounded to nearest
+  if (__builtin_fmaf(r, r, -v) > 0.0f) r = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, r) - 1u);   // r^2 > v: one ulp down
+  return r;
+}
+extern "C" __global__ void __launch_bounds__(kThreads)
+    rms_norm_entry__f32(TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out, float eps, TileGrid g) {
+  __shared__ float lds[kWaves];
+  const int wave = threadIdx.x >> 6;
+  const int64_t rows = min((int64_t)g.x, (int64_t)out.shape[0]);
+  const int32_t n = x.shape[1];
+  const int32_t n_out = out.shape[1] < n ? out.shape[1] : n;
+  const bool vec = n % 4 == 0 && n_out % 4 == 0 && x.strides[1] == 1 && out.strides[1] == 1 && w.strides[0] == 1 &&
+                   x.strides[0] % 4 == 0 && out.strides[0] % 4 == 0 && w.shape[0] >= n_out &&
+                   (((uintptr_t)x.ptr | (uintptr_t)out.ptr | (uintptr_t)w.ptr) & 15) == 0;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float* xr = (const float*)x.ptr + row * x.strides[0];
+    float* orow = (float*)out.ptr + row * out.strides[0];
+    float ss = 0.0f;
+    if (vec) {
+      for (int32_t j = threadIdx.x; j < n / 4; j += kThreads) {
+        const f32x4 v = reinterpret_cast<const f32x4*>(xr)[j];
+        ss = __builtin_fmaf(v[0], v[0], ss);
+        ss = __builtin_fmaf(v[1], v[1], ss);
+        ss = __builtin_fmaf(v[2], v[2], ss);
+        ss = __builtin_fmaf(v[3], v[3], ss);
+      }
+    } else {
+      for (int32_t j = threadIdx.x; j < n; j += kThreads) {
+        const float f = xr[(int64_t)j * x.strides[1]];
+        ss = __builtin_fmaf(f, f, ss);
+      }
+    }
+    ss = group_reduce<kWaves, false>(ss, lds, 0, wave);
+    const float scale = sqrt_toward_minus_infinity(1.0f / (ss / (float)n + eps));
+    if (vec) {
+      for (int32_t j = threadIdx.x; j < n_out / 4; j += kThreads) {
+        const f32x4 v = reinterpret_cast<const f32x4*>(xr)[j];
+        const f32x4 wv = reinterpret_cast<const f32x4*>(w.ptr)[j];
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (v[e] * scale) * wv[e];
+        __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(orow) + j);
+      }
+    } else {
+      for (int32_t j = threadIdx.x; j < n_out; j += kThreads) {
+        const float f = xr[(int64_t)j * x.strides[1]];
+        const float wv = j < w.shape[0] ? ((const float*)w.ptr)[(int64_t)j * w.strides[0]] : 0.0f;
+        orow[(int64_t)j * out.strides[1]] = (f * scale) * wv;
+      }
+    }
+    __syncthreads();  // lds is reused by the next row
+  }
+}
+
 // softmax(x, y: [BM, BN] tiles).  g.x / g.y = tiles covered along rows / columns.
 #define SOFTMAX_KERNEL(T, NAME, WPR, VPL)                                                           \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \

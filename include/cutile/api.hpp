@@ -347,6 +347,14 @@ struct RmsNormF16Fn {
     return cutile_launch_rms_norm_f16(s, &xa, &wa, &op, eps, o);
   }
 };
+struct RmsNormF32Fn {
+  template <class X, class W, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, W& w, O& out, float eps) {
+    auto xa = input_arg(x), wa = input_arg(w);
+    auto op = out.arg();
+    return cutile_launch_rms_norm_f32(s, &xa, &wa, &op, eps, o);
+  }
+};
 struct SoftmaxFn {
   template <class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, Yv& y) {
@@ -562,6 +570,8 @@ template <class Z, class A, class X, class Y> auto axpy(Z&& z, A&& a, X&& x, Y&&
 template <class Z, class X, class Y> auto add(Z&& z, X&& x, Y&& y) { return make_launcher<kernels::AddFn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y)); }
 // rms_norm_f16(x, w, out: partition [1,N], eps) -> (x, w, out, eps)   cutile-kernels/src/norms.rs:22-27
 template <class X, class W, class O> auto rms_norm_f16(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormF16Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
+// rms_norm(x, w, out: partition [1,N], eps) -> (x, w, out, eps), f32   cutile-examples/examples/rms_norm.rs:17-23
+template <class X, class W, class O> auto rms_norm(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormF32Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
 // softmax(x, y: partition [BM,BN]) -> (x, y)    cutile-benchmarks/benches/softmax.rs:23-26
 template <class X, class Y> auto softmax(X&& x, Y&& y) { return make_launcher<kernels::SoftmaxFn>(std::forward<X>(x), std::forward<Y>(y)); }
 // gemm(z: partition [BM,BN], x, y, k) -> (z, x, y, k): z <- z + x·y   cutile-benchmarks/benches/gemm.rs:25-30

@@ -359,6 +359,12 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
                                            const cutile_tensor_arg_t* w,
                                            const cutile_partition_arg_t* out, float eps,
                                            const cutile_launch_opts_t* opts);
+/* rms_norm<N, BLOCK_SIZE>(x: [-1, N] f32, w: [N] f32, out: [1, N] tiles f32, eps) — the f32 example form,
+ * cutile-examples/examples/rms_norm.rs:17-61: out = x * sqrt_rd(1 / (mean(x^2) + eps)) * w with the square root
+ * rounded toward minus infinity (:44-46). */
+cutile_status_t cutile_launch_rms_norm_f32(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                           const cutile_tensor_arg_t* w, const cutile_partition_arg_t* out, float eps,
+                                           const cutile_launch_opts_t* opts);
 /* softmax<BM, BN>(x, y: [BM,BN] tiles), f16 or f32 — cutile-benchmarks/benches/softmax.rs:19-35,
  * cutile-examples/examples/softmax.rs:11-24 */
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,

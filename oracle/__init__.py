@@ -74,6 +74,7 @@ def lib() -> C.CDLL:
             "orc_gemm_bf16": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_gemm_bf16_f32out": (None, [vp, vp, vp, i64, i64, i64, vp, i64]),
             "orc_fmha_ref_cpu": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64, f32, i64, i64, C.c_int, vp, i64]),
+            "orc_rms_norm_f32_example": (None, [vp, vp, vp, i64, i64, f32, i64]),
             "orc_qk_norm_rope_kv_f16": (None, [vp] * 9 + [f32, i64, i64, i64, i64, i64, i64]),
             "orc_argmax_blocks_f16": (None, [vp, i64, i64, i64, vp, vp, i64]),
             "orc_lm_head_argmax_blocks_f16": (None, [vp, vp, i64, i64, i64, vp, vp, i64]),
@@ -187,6 +188,15 @@ def rms_norm_f16(x_bits, w_bits, eps: float, block: int = 0) -> np.ndarray:
     rows, n = x.shape
     out = np.empty_like(x)
     lib().orc_rms_norm_f16(_p(x), _p(w), _p(out), rows, n, eps, block or n)
+    return out
+
+
+def rms_norm_f32_example(x, w, eps: float, block: int = 0) -> np.ndarray:
+    """cutile-examples/examples/rms_norm.rs:17-61 (f32, square root rounded toward minus infinity)"""
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    lib().orc_rms_norm_f32_example(_p(x), _p(w), _p(out), rows, n, eps, block)
     return out
 
 

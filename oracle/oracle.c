@@ -921,3 +921,27 @@ void orc_qk_norm_rope_kv_f16(const uint16_t* q, const uint16_t* k, const uint16_
         memcpy(v_cache + (h * max_seq + pos_i) * d, v + (s * nkv + h) * d, sizeof(uint16_t) * (size_t)d);
   }
 }
+
+/* rms_norm<N, BLOCK_SIZE> f32 (cutile-examples/examples/rms_norm.rs:17-61): a [1, BLOCK] vector accumulates x*x over
+ * the N / BLOCK chunks of the row and is then summed (:33-41); scale = sqrt(1 / (sum / N + eps)) with the square root
+ * rounded toward minus infinity (:42-46); out = x * scale * w (:56).  block = 0 means one chunk (BLOCK = N). */
+void orc_rms_norm_f32_example(const float* x, const float* w, float* out, int64_t rows, int64_t n, float eps,
+                              int64_t block) {
+  if (block <= 0 || block > n) block = n;
+  float* acc = (float*)malloc(sizeof(float) * (size_t)block);
+  for (int64_t r = 0; r < rows; r++) {
+    const float* xr = x + r * n;
+    for (int64_t i = 0; i < block; i++) acc[i] = 0.0f;
+    for (int64_t j = 0; j + block <= n; j += block)
+      for (int64_t i = 0; i < block; i++) acc[i] = acc[i] + xr[j + i] * xr[j + i];
+    /* reduce_sum over the BLOCK lanes: pairwise (a tile reduction is a tree; the order is not part of the contract) */
+    for (int64_t width = block; width > 1; width = (width + 1) / 2)
+      for (int64_t i = 0; i < width / 2; i++) acc[i] = acc[i] + acc[i + (width + 1) / 2];
+    const float sum = acc[0];
+    const float v = 1.0f / (sum / (float)n + eps);
+    float scale = sqrtf(v);                                   /* correctly rounded to nearest */
+    if (fmaf(scale, scale, -v) > 0.0f) scale = nextafterf(scale, 0.0f);   /* toward minus infinity */
+    for (int64_t j = 0; j < n; j++) out[r * n + j] = xr[j] * scale * w[j];
+  }
+  free(acc);
+}

@@ -42,6 +42,12 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_rms_norm_f32_example
+ *                        cutile-examples/examples/rms_norm.rs:17-61 (the example only prints).
+ *                        Pinned by float64 (the scale is the largest f32 not above the exact
+ *                        square root), x = c -> out = sign(c) w, and agreement with
+ *                        orc_rms_norm_f16 on f16-representable inputs up to the rounding mode:
+ *                        parity unpinned by reference tests.
  *   orc_qk_norm_rope_kv_f16
  *                        cutile-kernels/src/experimental/fused_transformer.rs (kernel bodies).
  *                        Pinned by orc_rms_norm_f16 at position 0 (no rotation), by
@@ -138,6 +144,9 @@ void orc_rope_seq_f16(const uint16_t* x, const float* inv_freq, uint16_t* out, i
 void orc_kv_cache_update_f16(const uint16_t* new_k, const uint16_t* new_v, uint16_t* k_cache,
                              uint16_t* v_cache, int64_t heads, int64_t d, int64_t max_seq,
                              int64_t position_start, int64_t seq_len);
+/* the f32 example form of RMSNorm: cutile-examples/examples/rms_norm.rs:17-61 */
+void orc_rms_norm_f32_example(const float* x, const float* w, float* out, int64_t rows, int64_t n, float eps,
+                              int64_t block);
 /* fused Q/K norm + RoPE + KV-cache update: cutile-kernels/src/experimental/fused_transformer.rs:22-345, 356-625 */
 void orc_qk_norm_rope_kv_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* qw,
                              const uint16_t* kw, const float* inv_freq, uint16_t* q_out, uint16_t* k_cache,

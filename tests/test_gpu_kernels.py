@@ -194,6 +194,21 @@ def test_rms_norm_f16(ct, dev, rows, n, variant):
     assert f16_ulp_diff(from_dev_f16_bits(out), ref).max() <= 1
 
 
+@pytest.mark.parametrize("rows,n", [(64, 512), (33, 8192), (7, 1000), (5, 13)])
+def test_rms_norm_f32_example_form(ct, dev, rows, n):
+    """cutile-examples/examples/rms_norm.rs:17-61; the kernel adds the squares in another order than the oracle and the
+    downward rounding turns a last-bit difference into a whole ulp of the scale: 2e-6 relative on the outputs (f32 sums of
+    up to 8192 squares in two different tree orders)"""
+    x, w = oracle.normal_f32((rows, n), 121), oracle.uniform_f32(n, 122, 0.5, 1.5)
+    out = torch.zeros(rows, n, device=dev)
+    ct.rms_norm_f32(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev), ct.partition(out, [1, n]), 1e-6, generics=[n])
+    sync()
+    ref = oracle.rms_norm_f32_example(x, w, 1e-6)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=2e-6, atol=0)
+    with pytest.raises(ct.CutileError, match="must be f32"):
+        ct.rms_norm_f32(torch.from_numpy(x).to(dev).half(), torch.from_numpy(w).to(dev), ct.partition(out, [1, n]), 1e-6)
+
+
 def test_rms_norm_f16_strided_rows_and_prefix(ct, dev):
     rows, n = 24, 1024
     xb = normal_f16_bits((rows, 2 * n), 111)

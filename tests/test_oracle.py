@@ -274,3 +274,34 @@ def test_mx_quantiser_follows_ocp_rule():
     assert (np.abs(deq)[~unsat] == (448 * scale)[~unsat]).all()
     z, zs = oracle.mx_quantize_e4m3(np.zeros((1, 32), np.float32))
     assert not z.any() and zs[0, 0] == 127
+
+
+def test_rms_norm_f32_example_rounds_its_square_root_down():
+    """cutile-examples/examples/rms_norm.rs:17-61: scale = sqrt_rd(1 / (mean(x^2) + eps)); float64 fixes the scale as the
+    largest f32 that does not exceed the exact square root of the f32 argument"""
+    x, w = oracle.normal_f32((64, 512), 991), oracle.uniform_f32(512, 992, 0.5, 1.5)
+    out = oracle.rms_norm_f32_example(x, w, 1e-6, 128)
+    for r in range(64):
+        acc = np.zeros(128, np.float32)
+        for j in range(0, 512, 128):
+            acc = acc + x[r, j:j + 128] * x[r, j:j + 128]
+        width = 128                                        # the tile reduction: pairwise halves
+        while width > 1:
+            half = (width + 1) // 2
+            acc[:width // 2] = acc[:width // 2] + acc[half:half + width // 2]
+            width = half
+        s = acc[0]
+        arg = np.float32(np.float32(1.0) / np.float32(np.float32(s / np.float32(512)) + np.float32(1e-6)))
+        exact = np.sqrt(np.float64(arg))
+        scale = np.float32(exact)
+        if np.float64(scale) > exact:
+            scale = np.nextafter(scale, np.float32(0))
+        assert np.float64(scale) <= exact < np.float64(np.nextafter(scale, np.float32(np.inf)))
+        assert np.array_equal(out[r], x[r] * scale * w)
+    # a constant row: mean(x^2) = c^2, so out = sign(c) w up to the eps and the downward rounding
+    c = np.full((2, 256), -3.0, np.float32)
+    got = oracle.rms_norm_f32_example(c, w[:256], 0.0)
+    assert np.allclose(got, -w[:256], rtol=3e-7, atol=0) and np.all(np.abs(got) <= w[:256])
+    # against float64 as a whole
+    ref = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + 1e-6) * w
+    assert np.max(np.abs(out - ref) / np.abs(ref).max()) < 1e-6
