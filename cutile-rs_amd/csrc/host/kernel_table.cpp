@@ -215,8 +215,11 @@ std::vector<KernelEntry> build_table() {
   fmha("f16", 128, 64, 128);
   fmha("f16", 128, 64, 64);
   fmha("f16", 32, 32, 32);
+  fmha("bf16", 128, 32, 256);
+  fmha("f16", 128, 32, 256);
   // the same kernels with the query position read from device memory (sequence-layout callers)
-  for (auto t : {std::array<int, 3>{128, 64, 128}, std::array<int, 3>{128, 64, 64}, std::array<int, 3>{32, 32, 32}}) {
+  for (auto t : {std::array<int, 3>{128, 64, 128}, std::array<int, 3>{128, 64, 64}, std::array<int, 3>{32, 32, 32},
+                 std::array<int, 3>{128, 32, 256}}) {
     std::string v = "f16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x" + std::to_string(t[2]);
     add("fmha_seq", keep(v), keep("fmha_seq_entry__" + v), IMG_FMHA, (uint32_t)(t[0] / 32 * 64),
         (uint32_t)(2 * 2 * t[1] * t[2] * 2), t[0], t[1], t[2], 0, "f16", 0, 3);

@@ -1267,6 +1267,8 @@ FMHA_KERNEL(bf16, __bf16, 32, 32, 32)
 FMHA_KERNEL(f16, _Float16, 128, 64, 128)
 FMHA_KERNEL(f16, _Float16, 128, 64, 64)
 FMHA_KERNEL(f16, _Float16, 32, 32, 32)
+FMHA_KERNEL(bf16, __bf16, 128, 32, 256)
+FMHA_KERNEL(f16, _Float16, 128, 32, 256)
 
 // The sequence-layout attention kernels of cutile-kernels whose position lives in device memory
 // (flash_attn_causal_seq_dynpos_f16 attention.rs:128-231, fmha_causal :598-726): q and out
@@ -1288,6 +1290,7 @@ FMHA_KERNEL(f16, _Float16, 32, 32, 32)
 FMHA_SEQ_KERNEL(f16, _Float16, 128, 64, 128)
 FMHA_SEQ_KERNEL(f16, _Float16, 128, 64, 64)
 FMHA_SEQ_KERNEL(f16, _Float16, 32, 32, 32)
+FMHA_SEQ_KERNEL(f16, _Float16, 128, 32, 256)
 
 #define FMHA_PINGPONG_KERNEL(NAME, T, BN, D)                                                       \
   extern "C" __global__ void __launch_bounds__(512)                                               \

@@ -418,6 +418,13 @@ def test_fmha_gqa_and_ragged_lengths(ct, dev):
     assert _fmha_case(ct, dev, 1, 4, 2, 200, 64, 64, False, 0) <= 2e-2
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_fmha_d256(ct, dev, causal):
+    """head dimension 256 (128 x 32 tiles, accumulators in the second register file), grouped heads, ragged length"""
+    assert _fmha_case(ct, dev, 1, 4, 2, 300, 256, 128, causal, 0, seed=441) <= 2e-2
+    assert _fmha_case(ct, dev, 1, 2, 2, 256, 256, 128, causal, 7, dtype=torch.float16, seed=442) <= 2e-2
+
+
 def test_fmha_f16(ct, dev):
     assert _fmha_case(ct, dev, 1, 2, 2, 256, 128, 128, True, 0, dtype=torch.float16) <= 2e-2
 

@@ -142,6 +142,7 @@ def _check(out, ref):
     (64, 4, 4, 64, 64, 32, 64, 0),                # D 64, no grouping
     (70, 6, 2, 100, 32, 16, 100, 30),             # D 32
     (300, 8, 8, 300, 128, 64, 300, 0),            # long enough for the ping-pong kernel, ragged
+    (150, 4, 2, 256, 256, 32, 200, 50),           # D 256
 ])
 def test_gpu_flash_attn_causal_seq(ct, dev, q_len, q_heads, kv_heads, max_seq, d, bm, kv_len, start):
     q, k, v = _inputs(q_len, q_heads, kv_heads, max_seq, d, 721)
