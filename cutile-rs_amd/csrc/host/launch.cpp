@@ -1712,6 +1712,7 @@ cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_
   std::vector<std::string> acceptable;
   for (auto* e : fit)
     if (kv_len > 0 || strstr(e->variant, "_pp") == nullptr) acceptable.push_back(e->variant);   // an empty key range: the plain kernels only
+  CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND, "no precompiled sequence attention for f16, D = %d and an empty key range", d);
   cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
   o.generics = nullptr;
   o.n_generics = 0;
