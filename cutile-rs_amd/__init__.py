@@ -129,6 +129,7 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_add_rms_norm_decode_raw_f16": [vp, vp, vp, vp, vp, vp, f32, i32, P(LaunchOpts)],
             "cutile_launch_qk_norm_rope_kv_prefill_raw_f16": [vp] + [vp] * 9 + [f32, i32, i32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_qk_norm_rope_kv_decode_raw_f16": [vp] + [vp] * 7 + [P(TensorArg), f32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_group_gemm_f16_nt_desc": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg),
@@ -498,6 +499,13 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+def add_rms_norm_decode_raw_f16(residual, x, w, out, residual_out, eps: float, *, stream=None, generics=None) -> None:
+    """cutile-kernels/src/experimental/norms.rs:22-153: one row of N halves, the tensors' addresses passed as raw pointers"""
+    o, _k = _opts(None, generics, None)
+    check(lib().cutile_launch_add_rms_norm_decode_raw_f16(_stream(stream), *[C.c_void_p(t.data_ptr()) for t in (residual, x, w, out, residual_out)],
+                                                          C.c_float(eps), int(w.numel()), C.byref(o)))
 
 
 def qk_norm_rope_kv_prefill_raw_f16(q, k, v, q_weight, k_weight, inv_freq, q_out, k_cache, v_cache, eps: float, position_start: int,

@@ -802,6 +802,43 @@ cutile_status_t cutile_launch_add_rms_norm_f16(cutile_stream_t stream, const cut
   return launch_fused_norm("add_rms_norm_f16", stream, residual, x, w, nullptr, out, residual_out, eps, nullptr, opts);
 }
 
+// add_rms_norm_decode_raw_f16<N, BLOCK_SIZE> (cutile-kernels/src/experimental/norms.rs:22-153): add_rms_norm_f16 on one
+// row of N halves given as raw device pointers (the reference assumes them 16-byte aligned).
+cutile_status_t cutile_launch_add_rms_norm_decode_raw_f16(cutile_stream_t stream, const void* residual, const void* x,
+                                                          const void* w, void* out, void* residual_out, float eps,
+                                                          int32_t n, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(residual && x && w && out && residual_out, CUTILE_ERR_INVALID_ARGUMENT, "add_rms_norm_decode_raw_f16: null device pointer");
+  CUTILE_REQUIRE(n > 0, CUTILE_ERR_KERNEL_LAUNCH, "add_rms_norm_decode_raw_f16: N must be positive");
+  auto row = [&](const void* p) {
+    cutile_tensor_arg_t t{};
+    t.ptr = const_cast<void*>(p);
+    t.dtype = CUTILE_DTYPE_F16;
+    t.rank = 2;
+    t.shape[0] = 1, t.shape[1] = n;
+    t.strides[0] = n, t.strides[1] = 1;
+    return t;
+  };
+  cutile_tensor_arg_t rt = row(residual), xt = row(x), wt{};
+  wt.ptr = const_cast<void*>(w);
+  wt.dtype = CUTILE_DTYPE_F16;
+  wt.rank = 1;
+  wt.shape[0] = n;
+  wt.strides[0] = 1;
+  auto part = [&](void* p) {
+    cutile_partition_arg_t pa{};
+    pa.tensor = row(p);
+    pa.partition_shape[0] = 1, pa.partition_shape[1] = n;
+    pa.partition_strides[0] = n, pa.partition_strides[1] = 1;
+    return pa;
+  };
+  cutile_partition_arg_t op = part(out), rp = part(residual_out);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(n), "N")) return s;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  return cutile_launch_add_rms_norm_f16(stream, &rt, &xt, &wt, &op, &rp, eps, &o);
+}
+
 cutile_status_t cutile_launch_qk_norm_f16(cutile_stream_t stream, const cutile_tensor_arg_t* q,
                                           const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* q_weight,
                                           const cutile_tensor_arg_t* k_weight, const cutile_partition_arg_t* out,

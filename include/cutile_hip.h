@@ -433,6 +433,11 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* add_rms_norm_decode_raw_f16<N, BLOCK_SIZE>(residual_ptr, x_ptr, w_ptr, out_ptr, residual_out_ptr, eps) —
+ * cutile-kernels/src/experimental/norms.rs:22-153: add_rms_norm_f16 on one row of N halves, raw device pointers. */
+cutile_status_t cutile_launch_add_rms_norm_decode_raw_f16(cutile_stream_t stream, const void* residual, const void* x,
+                                                          const void* w, void* out, void* residual_out, float eps,
+                                                          int32_t n, const cutile_launch_opts_t* opts);
 /* qk_norm_rope_kv_prefill_raw_f16<D, HALF_D, MAX_SEQ>(q_ptr, k_ptr, v_ptr, q_weight_ptr, k_weight_ptr, inv_freq_ptr,
  * q_out_ptr, k_cache_ptr, v_cache_ptr, eps, position_start, seq_len, num_q_heads, num_kv_heads) —
  * cutile-kernels/src/experimental/fused_transformer.rs:22-345.  Raw device pointers as in the reference: q, q_out

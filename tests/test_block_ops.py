@@ -94,6 +94,19 @@ def test_gpu_add_rms_norm(ct, dev, rows, n, variant):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("n", [4096, 8192, 1000])
+def test_gpu_add_rms_norm_decode_raw(ct, dev, n):
+    """cutile-kernels/src/experimental/norms.rs:22-153: the one-row raw-pointer form is add_rms_norm_f16 on [1, N]"""
+    r, x = normal_f16_bits((1, n), 671), normal_f16_bits((1, n), 672)
+    w = f16(oracle.uniform_f32((n,), 673, 0.5, 1.5))
+    out, res = torch.zeros(n, dtype=torch.float16, device=dev), torch.zeros(n, dtype=torch.float16, device=dev)
+    ct.add_rms_norm_decode_raw_f16(_dev(r, dev), _dev(x, dev), _dev(w, dev), out, res, 1e-6, generics=[n])
+    torch.cuda.synchronize()
+    ref_out, ref_res = oracle.add_rms_norm_f16(r, x, w, 1e-6)
+    assert np.array_equal(_bits(res), ref_res[0]) and np.max(f16_ulp_diff(_bits(out), ref_out[0])) <= 1
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("n,variant,q_rows,k_rows", [
     (128, None, 40, 8), (64, None, 40, 8), (256, "w1v1", 40, 8), (120, None, 40, 8),
     # many workgroups, a ragged last one, the q/k boundary inside one pass of one wavefront
