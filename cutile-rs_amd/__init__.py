@@ -140,6 +140,7 @@ def lib() -> C.CDLL:
             "cutile_launch_argmax_reduce_blocks_to_u32": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), i32, P(LaunchOpts)],
             "cutile_launch_embedding_batch_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_gather_row_f16": [vp, P(TensorArg), P(PartitionArg), i32, P(LaunchOpts)],
+            "cutile_launch_fmha_prefill_gqa_lpt_raw_f16": [vp, vp, vp, vp, vp, f32, i32, i32, i32, i32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha_seq_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), f32, i32, i32, i32,
                                            P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_linear_tile_mxfp8": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg),
@@ -602,6 +603,16 @@ def fmha_seq_f16(q, k, v, out: Partition, qk_scale: float, query_group_size: int
                                            C.c_float(qk_scale), int(query_group_size), int(kv_len), int(query_start),
                                            C.byref(pa) if pa is not None else None, int(kv_len_from_position), int(causal),
                                            C.byref(o)))
+
+
+def fmha_prefill_gqa_lpt_raw_f16(q, k, v, out, qk_scale: float, query_group_size: int, kv_len: int, query_start: int, group: int, *,
+                                 causal: bool = True, stream=None, generics=None) -> None:
+    """cutile-kernels/src/experimental/attention.rs:22-377; contiguous q / out [q_len, q_heads, D] and k / v [kv_heads, kv_len, D]
+    passed as raw addresses"""
+    o, _k = _opts(None, generics, None)
+    check(lib().cutile_launch_fmha_prefill_gqa_lpt_raw_f16(
+        _stream(stream), *[C.c_void_p(t.data_ptr()) for t in (q, k, v, out)], C.c_float(qk_scale), int(query_group_size), int(q.shape[0]),
+        int(kv_len), int(query_start), int(q.shape[1]) // int(group), int(group), int(q.shape[2]), int(causal), C.byref(o)))
 
 
 def linear_tile_mxfp8(z: Partition, x, y, x_scales, y_scales, alpha: float = 1.0, *, stream=None, grid=None,

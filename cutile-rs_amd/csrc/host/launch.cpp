@@ -1778,6 +1778,44 @@ cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// fmha_prefill_gqa_lpt (cutile-kernels/src/experimental/attention.rs:22-377): fmha_prefill_gqa on raw pointers, with the
+// caller choosing the order in which tile blocks take (query block, head group) pairs (longest first, swizzled).  The
+// order does not change the result; this library's kernels have their own (heaviest tiles first, heads that share a
+// KV head side by side on one XCD), so the scheduling arguments of the reference have no counterpart here.
+cutile_status_t cutile_launch_fmha_prefill_gqa_lpt_raw_f16(cutile_stream_t stream, const void* q, const void* k, const void* v,
+                                                           void* out, float qk_scale, int32_t query_group_size, int32_t q_len,
+                                                           int32_t kv_len, int32_t query_start, int32_t num_head_groups,
+                                                           int32_t group, int32_t d, int32_t causal,
+                                                           const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(q && k && v && out, CUTILE_ERR_INVALID_ARGUMENT, "fmha_prefill_gqa_lpt: null device pointer");
+  CUTILE_REQUIRE(q_len > 0 && kv_len >= 0 && num_head_groups > 0 && group > 0 && d > 0 && query_group_size > 0 &&
+                     ((int64_t)num_head_groups * group) % query_group_size == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha_prefill_gqa_lpt: q_len, head groups, GROUP and D must be positive and the heads a multiple of query_group_size");
+  const int32_t q_heads = num_head_groups * group, kv_heads = q_heads / query_group_size;
+  auto t3 = [&](const void* p, int32_t a, int32_t b) {
+    cutile_tensor_arg_t t{};
+    t.ptr = const_cast<void*>(p);
+    t.dtype = CUTILE_DTYPE_F16;
+    t.rank = 3;
+    t.shape[0] = a, t.shape[1] = b, t.shape[2] = d;
+    t.strides[0] = b * d, t.strides[1] = d, t.strides[2] = 1;
+    return t;
+  };
+  // the reference views k and v as [kv_heads, kv_len, D] with kv_len rows per head (:66-72)
+  cutile_tensor_arg_t qt = t3(q, q_len, q_heads), kt = t3(k, kv_heads, std::max(kv_len, 1)), vt = t3(v, kv_heads, std::max(kv_len, 1));
+  cutile_partition_arg_t op{};
+  op.tensor = t3(out, q_len, q_heads);
+  const int32_t bm = std::max(1, generic_int(opts, 0, 64));
+  op.partition_shape[0] = bm, op.partition_shape[1] = group, op.partition_shape[2] = d;
+  for (int i = 0; i < 3; ++i) op.partition_strides[i] = op.tensor.strides[i];
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(d), "D")) return s;
+  if (cutile_status_t s = check_generic(opts, 3, std::to_string(group), "GROUP")) return s;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  return cutile_launch_fmha_seq_f16(stream, &qt, &kt, &vt, &op, qk_scale, query_group_size, kv_len, query_start, nullptr, 0, causal, &o);
+}
+
 cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                                 const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                                 const cutile_tensor_arg_t* xs, const cutile_tensor_arg_t* ys, float alpha,

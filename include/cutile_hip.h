@@ -525,6 +525,17 @@ cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_
                                            int32_t query_group_size, int32_t kv_len, int32_t query_start,
                                            const cutile_tensor_arg_t* position_start, int32_t kv_len_from_position,
                                            int32_t causal, const cutile_launch_opts_t* opts);
+/* fmha_prefill_gqa_lpt<BM, BN, D, GROUP, M_EFF, CAUSAL, EVEN_K, LATENCY, SCHED, MASK_SPLIT>(q_ptr, k_ptr, v_ptr, out_ptr,
+ * qk_scale, query_group_size, q_len, kv_len, query_start, num_q_blocks, num_head_groups, swizzle, ...) —
+ * cutile-kernels/src/experimental/attention.rs:22-377: fmha_prefill_gqa on raw pointers (q, out [q_len, heads, D];
+ * k, v [kv_heads, kv_len, D], contiguous).  The reference's scheduling arguments (block order, swizzle) do not change
+ * the result and have no counterpart: the kernels order their tiles themselves.  GROUP, D and CAUSAL are arguments
+ * here; generics 0 (BM), 2 (D) and 3 (GROUP) are checked when given. */
+cutile_status_t cutile_launch_fmha_prefill_gqa_lpt_raw_f16(cutile_stream_t stream, const void* q, const void* k, const void* v,
+                                                           void* out, float qk_scale, int32_t query_group_size, int32_t q_len,
+                                                           int32_t kv_len, int32_t query_start, int32_t num_head_groups,
+                                                           int32_t group, int32_t d, int32_t causal,
+                                                           const cutile_launch_opts_t* opts);
 /* fmha<BM, BN, D, H, CAUSAL, EVEN_K>(out: [1,BM,D] tiles, q, k, v, qk_scale,
  * input_pos, query_group_size) — cutile-examples/examples/flash_attention_causal.rs:19-134,
  * cutile-benchmarks/benches/fmha.rs:20-145 (non-causal: causal = 0, input_pos = 0) */

@@ -206,3 +206,16 @@ def test_gpu_seq_attention_empty_key_range_and_prefix_coverage(ct, dev):
     got = out.float().cpu().numpy()
     assert np.max(np.abs(got[:64, :3] - ref[:64, :3])) <= 2e-2
     assert np.all(got[64:] == 7.0) and np.all(got[:, 3] == 7.0)     # rows and heads outside the launch stay untouched
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("causal", [True, False])
+def test_gpu_fmha_prefill_gqa_lpt_raw(ct, dev, causal):
+    """cutile-kernels/src/experimental/attention.rs:22-377: the raw-pointer form with caller-chosen block order computes
+    fmha_prefill_gqa; k and v hold exactly kv_len rows per head"""
+    q, k, v = _inputs(200, 8, 2, 320, 128, 761)
+    out = torch.full((200, 8, 128), float("nan"), dtype=torch.half, device=dev)
+    ct.fmha_prefill_gqa_lpt_raw_f16(_dev(q, dev), _dev(k, dev), _dev(v, dev), out, 128 ** -0.5, 4, 320, 120, 4, causal=causal,
+                                    generics=[64, 64, 128, 4])
+    torch.cuda.synchronize()
+    _check(out, oracle.attention_seq_ref(q, k, v, 128 ** -0.5, 4, 320, 120, causal))
