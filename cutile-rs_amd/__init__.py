@@ -129,6 +129,8 @@ def lib() -> C.CDLL:
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_launch_fmha": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(TensorArg), f32, i32, i32, i32,
                                    P(LaunchOpts)],
+            "cutile_launch_copy_stacked_to_contiguous_f16": [vp, i32, i32, i32, P(TensorArg), P(TensorArg), i32, i32, i32, i32, i32, P(LaunchOpts)],
+            "cutile_launch_copy_contiguous_to_stacked_f16": [vp, i32, i32, i32, P(TensorArg), P(TensorArg), i32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_add_rms_norm_decode_raw_f16": [vp, vp, vp, vp, vp, vp, f32, i32, P(LaunchOpts)],
             "cutile_launch_qk_norm_rope_kv_prefill_raw_f16": [vp] + [vp] * 9 + [f32, i32, i32, i32, i32, i32, i32, P(LaunchOpts)],
             "cutile_launch_qk_norm_rope_kv_decode_raw_f16": [vp] + [vp] * 7 + [P(TensorArg), f32, i32, i32, i32, i32, P(LaunchOpts)],
@@ -500,6 +502,21 @@ def fmha(out: Partition, q, k, v, qk_scale: float, input_pos: int = 0, query_gro
     qa, ka, va = tensor_arg(q), tensor_arg(k), tensor_arg(v)
     check(lib().cutile_launch_fmha(_stream(stream), C.byref(out.arg()), C.byref(qa), C.byref(ka), C.byref(va),
                                    float(qk_scale), int(input_pos), int(query_group_size), int(causal), C.byref(o)))
+
+
+KVBM_STACKED_NHD, KVBM_STACKED_HND = 0, 1
+KVBM_OPERATIONAL_NHD, KVBM_OPERATIONAL_HND, KVBM_UNIVERSAL = 0, 1, 2
+
+
+def kvbm_copy_f16(to_stacked: bool, stacked_layout: int, contiguous_layout: int, num_blocks: int, stacked_tensors, contiguous_tensors,
+                  nh: int, nl: int, no: int, nt: int, hd: int, *, stream=None) -> None:
+    """copy_stacked_to_contiguous_f16 / copy_contiguous_to_stacked_f16 (cutile-kernels/src/experimental/kvbm.rs:112-352);
+    the tables are int64 device tensors of tensor addresses"""
+    sa, ca = tensor_arg(stacked_tensors), tensor_arg(contiguous_tensors)
+    o, _k = _opts(None, None, None)
+    fn = lib().cutile_launch_copy_contiguous_to_stacked_f16 if to_stacked else lib().cutile_launch_copy_stacked_to_contiguous_f16
+    check(fn(_stream(stream), int(stacked_layout), int(contiguous_layout), int(num_blocks), C.byref(sa), C.byref(ca), int(nh), int(nl),
+             int(no), int(nt), int(hd), C.byref(o)))
 
 
 def add_rms_norm_decode_raw_f16(residual, x, w, out, residual_out, eps: float, *, stream=None, generics=None) -> None:

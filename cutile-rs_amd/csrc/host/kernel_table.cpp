@@ -78,6 +78,7 @@ std::vector<KernelEntry> build_table() {
   add("embedding_batch", "f16", "embedding_batch_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   add("gather_row", "f16", "gather_row_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   add("qk_norm_rope_kv", "f16", "qk_norm_rope_kv_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
+  add("kvbm_copy", "f16", "kvbm_copy_entry__f16", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 #undef EW
   static const char* kCreationTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64", "u8", "u16", "u32"};
   static std::deque<std::string> names;  // keeps generated strings alive at stable addresses

@@ -1201,6 +1201,62 @@ cutile_status_t cutile_launch_qk_norm_rope_kv_decode_raw_f16(cutile_stream_t str
                                 (int64_t)num_q_heads * d, (int64_t)num_kv_heads * d, opts);
 }
 
+// ---- KV block layout conversion (cutile-kernels/src/experimental/kvbm.rs) ----
+static cutile_status_t launch_kvbm_copy(const char* name, cutile_stream_t stream, int32_t to_stacked, int32_t stacked_layout,
+                                        int32_t contiguous_layout, int32_t num_blocks, const cutile_tensor_arg_t* stacked_tensors,
+                                        const cutile_tensor_arg_t* contiguous_tensors, int32_t nh, int32_t nl, int32_t no, int32_t nt,
+                                        int32_t hd, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(stacked_tensors, "stacked_tensors", 1, 1)) return s;
+  if (cutile_status_t s = check_tensor(contiguous_tensors, "contiguous_tensors", 1, 1)) return s;
+  CUTILE_REQUIRE(num_blocks >= 0 && nh > 0 && nl > 0 && no > 0 && nt > 0 && hd > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: num_blocks must be non-negative and the block extents positive", name);
+  CUTILE_REQUIRE((stacked_layout == CUTILE_KVBM_STACKED_NHD || stacked_layout == CUTILE_KVBM_STACKED_HND) &&
+                     (contiguous_layout == CUTILE_KVBM_UNIVERSAL ||
+                      (stacked_layout == CUTILE_KVBM_STACKED_NHD && contiguous_layout == CUTILE_KVBM_OPERATIONAL_NHD) ||
+                      (stacked_layout == CUTILE_KVBM_STACKED_HND && contiguous_layout == CUTILE_KVBM_OPERATIONAL_HND)),
+                 CUTILE_ERR_KERNEL_LAUNCH, "unsupported KVBM %s layout map", to_stacked ? "contiguous-to-stacked" : "stacked-to-contiguous");
+  const int64_t stacked_count = (int64_t)num_blocks * nl * no;
+  CUTILE_REQUIRE(stacked_tensors->dtype == CUTILE_DTYPE_I64 && contiguous_tensors->dtype == CUTILE_DTYPE_I64 &&
+                     stacked_tensors->strides[0] == 1 && contiguous_tensors->strides[0] == 1 &&
+                     stacked_tensors->shape[0] >= stacked_count && contiguous_tensors->shape[0] >= num_blocks &&
+                     (((uintptr_t)stacked_tensors->ptr | (uintptr_t)contiguous_tensors->ptr) & 7) == 0,
+                 CUTILE_ERR_KERNEL_LAUNCH, "%s: the pointer tables must be dense aligned i64 tensors of %lld (stacked) and %d (contiguous) entries",
+                 name, (long long)stacked_count, num_blocks);
+  if (num_blocks == 0) return CUTILE_SUCCESS;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("kvbm_copy", nullptr, "f16", {"f16"}, &res)) return s;
+  (void)opts;
+  ArgPacker args;
+  args.push_val<const void*>(stacked_tensors->ptr);
+  args.push_val<const void*>(contiguous_tensors->ptr);
+  args.push_val<int32_t>(to_stacked);
+  args.push_val<int32_t>(stacked_layout == CUTILE_KVBM_STACKED_HND ? 1 : 0);
+  args.push_val<int32_t>(contiguous_layout);
+  args.push_val<int32_t>(num_blocks);
+  args.push_val<int32_t>(nh);
+  args.push_val<int32_t>(nl);
+  args.push_val<int32_t>(no);
+  args.push_val<int32_t>(nt);
+  args.push_val<int32_t>(hd);
+  const uint64_t lanes = (uint64_t)num_blocks * nh * nl * no * nt * (uint64_t)(hd % 8 == 0 ? hd / 8 : hd);
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(lanes, 256 * 4), 1u << 16)), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+cutile_status_t cutile_launch_copy_stacked_to_contiguous_f16(cutile_stream_t stream, int32_t stacked_layout, int32_t contiguous_layout,
+                                                             int32_t num_blocks, const cutile_tensor_arg_t* stacked_tensors,
+                                                             const cutile_tensor_arg_t* contiguous_tensors, int32_t nh, int32_t nl,
+                                                             int32_t no, int32_t nt, int32_t hd, const cutile_launch_opts_t* opts) {
+  return launch_kvbm_copy("copy_stacked_to_contiguous_f16", stream, 0, stacked_layout, contiguous_layout, num_blocks, stacked_tensors,
+                          contiguous_tensors, nh, nl, no, nt, hd, opts);
+}
+cutile_status_t cutile_launch_copy_contiguous_to_stacked_f16(cutile_stream_t stream, int32_t stacked_layout, int32_t contiguous_layout,
+                                                             int32_t num_blocks, const cutile_tensor_arg_t* stacked_tensors,
+                                                             const cutile_tensor_arg_t* contiguous_tensors, int32_t nh, int32_t nl,
+                                                             int32_t no, int32_t nt, int32_t hd, const cutile_launch_opts_t* opts) {
+  return launch_kvbm_copy("copy_contiguous_to_stacked_f16", stream, 1, stacked_layout, contiguous_layout, num_blocks, stacked_tensors,
+                          contiguous_tensors, nh, nl, no, nt, hd, opts);
+}
+
 static bool decode_vec_layout(const cutile_tensor_arg_t& t) {
   return t.strides[2] == 1 && t.strides[1] % 8 == 0 && t.strides[0] % 8 == 0 && aligned16(t.ptr);
 }

@@ -834,3 +834,49 @@ extern "C" __global__ void __launch_bounds__(kThreads)
     }
   }
 }
+
+// ---- KV block layout conversion ---------------------------------------------------------------
+// copy_stacked_to_contiguous_f16 / copy_contiguous_to_stacked_f16
+// (cutile-kernels/src/experimental/kvbm.rs:112-187, 283-352; layouts :358-400).  A cache block is nh heads x nl
+// layers x no offsets (K, V) x nt tokens x hd values.  Stacked form: one tensor per (block, layer, offset) — table
+// entry (block * nl + layer) * no + offset — laid out [nt, nh, hd] (NHD) or [nh, nt, hd] (HND).  Contiguous form: one
+// tensor per block, [nl, no, nt, nh, hd] (operational NHD), [nl, no, nh, nt, hd] (operational HND) or
+// [nh, nl, no, nt, hd] (universal).  Every element is copied once; a lane moves 16 bytes along hd.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    kvbm_copy_entry__f16(const int64_t* stacked_tensors, const int64_t* contiguous_tensors, int32_t to_stacked,
+                         int32_t stacked_hnd, int32_t contiguous_layout, int32_t num_blocks, int32_t nh, int32_t nl,
+                         int32_t no, int32_t nt, int32_t hd) {
+  const int32_t per_row = hd % 8 == 0 ? hd / 8 : hd;      // 16-byte vectors per (head, token) row, else elements
+  const bool vec = hd % 8 == 0;
+  const int64_t rows_per_block = (int64_t)nh * nl * no * nt;
+  const int64_t total = (int64_t)num_blocks * rows_per_block * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int32_t c = (int32_t)(i % per_row);
+    int64_t r = i / per_row;
+    const int32_t b = (int32_t)(r / rows_per_block);
+    r %= rows_per_block;
+    // walk the rows in the order of the contiguous tensor, so that its side is one linear stream
+    int32_t h, l, o, t;
+    if (contiguous_layout == 2) {            // universal [nh, nl, no, nt]
+      t = (int32_t)(r % nt), r /= nt;
+      o = (int32_t)(r % no), r /= no;
+      l = (int32_t)(r % nl), h = (int32_t)(r / nl);
+    } else if (contiguous_layout == 1) {     // operational HND [nl, no, nh, nt]
+      t = (int32_t)(r % nt), r /= nt;
+      h = (int32_t)(r % nh), r /= nh;
+      o = (int32_t)(r % no), l = (int32_t)(r / no);
+    } else {                                 // operational NHD [nl, no, nt, nh]
+      h = (int32_t)(r % nh), r /= nh;
+      t = (int32_t)(r % nt), r /= nt;
+      o = (int32_t)(r % no), l = (int32_t)(r / no);
+    }
+    const int64_t cont_row = (i / per_row) % rows_per_block;
+    const int64_t stacked_row = stacked_hnd ? (int64_t)h * nt + t : (int64_t)t * nh + h;
+    _Float16* sp = reinterpret_cast<_Float16*>(stacked_tensors[((int64_t)b * nl + l) * no + o]) + stacked_row * hd;
+    _Float16* cp = reinterpret_cast<_Float16*>(contiguous_tensors[b]) + cont_row * hd;
+    const _Float16* src = to_stacked ? cp : sp;
+    _Float16* dst = to_stacked ? sp : cp;
+    if (vec) reinterpret_cast<u32x4*>(dst)[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + c);
+    else dst[c] = src[c];
+  }
+}

@@ -433,6 +433,22 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* copy_stacked_to_contiguous_f16 / copy_contiguous_to_stacked_f16(num_blocks, stacked_tensors, contiguous_tensors, nh, nl,
+ * no, nt, hd) — cutile-kernels/src/experimental/kvbm.rs:112-187, 283-352.  KV cache blocks of nh heads x nl layers x
+ * no offsets x nt tokens x hd values move between the stacked form (one f16 tensor per (block, layer, offset), table
+ * entry (block * nl + layer) * no + offset, laid out [nt, nh, hd] or [nh, nt, hd]) and the contiguous form (one tensor
+ * per block).  The reference passes the layouts as index maps in its generics (StackedLayout / ContiguousLayout,
+ * kvbm.rs:358-400); here they are the two enumerators, with the same four supported pairs. */
+enum { CUTILE_KVBM_STACKED_NHD = 0, CUTILE_KVBM_STACKED_HND = 1 };
+enum { CUTILE_KVBM_OPERATIONAL_NHD = 0, CUTILE_KVBM_OPERATIONAL_HND = 1, CUTILE_KVBM_UNIVERSAL = 2 };
+cutile_status_t cutile_launch_copy_stacked_to_contiguous_f16(cutile_stream_t stream, int32_t stacked_layout, int32_t contiguous_layout,
+                                                             int32_t num_blocks, const cutile_tensor_arg_t* stacked_tensors,
+                                                             const cutile_tensor_arg_t* contiguous_tensors, int32_t nh, int32_t nl,
+                                                             int32_t no, int32_t nt, int32_t hd, const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_copy_contiguous_to_stacked_f16(cutile_stream_t stream, int32_t stacked_layout, int32_t contiguous_layout,
+                                                             int32_t num_blocks, const cutile_tensor_arg_t* stacked_tensors,
+                                                             const cutile_tensor_arg_t* contiguous_tensors, int32_t nh, int32_t nl,
+                                                             int32_t no, int32_t nt, int32_t hd, const cutile_launch_opts_t* opts);
 /* add_rms_norm_decode_raw_f16<N, BLOCK_SIZE>(residual_ptr, x_ptr, w_ptr, out_ptr, residual_out_ptr, eps) —
  * cutile-kernels/src/experimental/norms.rs:22-153: add_rms_norm_f16 on one row of N halves, raw device pointers. */
 cutile_status_t cutile_launch_add_rms_norm_decode_raw_f16(cutile_stream_t stream, const void* residual, const void* x,

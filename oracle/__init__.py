@@ -413,6 +413,29 @@ def qk_norm_rope_kv_f16(q_bits, k_bits, v_bits, qw_bits, kw_bits, inv_freq, k_ca
     return q_out, kc, vc
 
 
+# ---- KV block layout conversion (cutile-kernels/src/experimental/kvbm.rs) ----
+KVBM_UNIVERSAL_TO_STACKED = {"nhd": (1, 2, 3, 0, 4), "hnd": (1, 2, 0, 3, 4)}                        # kvbm.rs:390-394
+KVBM_STACKED_TO_CONTIGUOUS = {("nhd", "universal"): (3, 0, 1, 2, 4), ("hnd", "universal"): (2, 0, 1, 3, 4),
+                              ("nhd", "operational_nhd"): (0, 1, 2, 3, 4), ("hnd", "operational_hnd"): (0, 1, 2, 3, 4)}   # :378-383
+
+
+def kvbm_stacked_to_contiguous(stacked, stacked_layout: str, contiguous_layout: str) -> np.ndarray:
+    """copy_stacked_to_contiguous_f16 (kvbm.rs:112-187).  stacked: [blocks, nl, no] + the per-(block, layer, offset) tensor
+    ([nt, nh, hd] for "nhd", [nh, nt, hd] for "hnd"); returns [blocks] + the contiguous shape.  The kernel permutes every
+    tile with STACKED_TO_CONTIGUOUS_MAP (:176), i.e. transposes the block by that map."""
+    stacked = np.asarray(stacked)
+    axes = KVBM_STACKED_TO_CONTIGUOUS[(stacked_layout, contiguous_layout)]
+    return np.ascontiguousarray(np.transpose(stacked, (0,) + tuple(a + 1 for a in axes)))
+
+
+def kvbm_contiguous_to_stacked(contiguous, stacked_layout: str, contiguous_layout: str) -> np.ndarray:
+    """copy_contiguous_to_stacked_f16 (kvbm.rs:283-352): the inverse permutation"""
+    contiguous = np.asarray(contiguous)
+    axes = KVBM_STACKED_TO_CONTIGUOUS[(stacked_layout, contiguous_layout)]
+    inverse = np.argsort(axes)
+    return np.ascontiguousarray(np.transpose(contiguous, (0,) + tuple(int(a) + 1 for a in inverse)))
+
+
 # ---- greedy sampling and row gathers (cutile-kernels/src/argmax.rs, embeddings.rs, pointwise.rs) ----
 def argmax_blocks_f16(logits_bits, block_size: int, length: int, num_blocks: int = None):
     """-> (block_max f32 [blocks], block_idx u32 [blocks])"""

@@ -42,6 +42,10 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   kvbm_stacked_to_contiguous / kvbm_contiguous_to_stacked (numpy, Python wrapper)
+ *                        cutile-kernels/src/experimental/kvbm.rs:112-400: a transpose by the
+ *                        reference's index maps; pinned element by element against the layouts'
+ *                        definitions ([tokens, heads, head_dim] etc.) and by the round trip.
  *   orc_rms_norm_f32_example
  *                        cutile-examples/examples/rms_norm.rs:17-61 (the example only prints).
  *                        Pinned by float64 (the scale is the largest f32 not above the exact
