@@ -1031,7 +1031,12 @@ cutile_status_t cutile_launch_lm_head_argmax_blocks_f16(cutile_stream_t stream, 
   args.push_partition(*block_idx);
   args.push_val<int32_t>(vocab_size);
   args.push_tile_grid(tg);
-  uint32_t grid[3] = {tg[0], 1, 1};
+  // two workgroups per compute unit, each walking a contiguous run of blocks
+  cutile_device_t device = nullptr;
+  if (cutile_status_t s = current_device(&device)) return s;
+  int cus = 0;
+  if (cutile_status_t s = compute_units(device, &cus)) return s;
+  uint32_t grid[3] = {std::min(tg[0], (uint32_t)std::max(cus, 1) * 2u), 1, 1};
   return launch_packed(res.fn, grid, res.entry->block, (uint32_t)k * 2, stream, args);
 }
 

@@ -591,16 +591,92 @@ extern "C" __global__ void __launch_bounds__(kThreads)
 
 // logits[r] = sum_k f32(weights[r, k]) * f32(hidden[0, k]) for the 64 rows of block b, then the block's winner.
 // The weights are read once, 16 bytes per lane and nontemporally (a [vocab, K] matrix streams through once per
-// token); the hidden vector sits in LDS.  A wavefront takes 16 of the 64 rows, two at a time.
+// token); the hidden vector sits in LDS.  The launch holds two workgroups per compute unit, each taking a
+// contiguous run of blocks (a stream of this kind reads fastest from few resident wavefronts); a wavefront takes
+// 16 of a block's 64 rows, two at a time, 1024 columns per step, and requests the next step's weights before it
+// multiplies the current ones.
+namespace {
+
+constexpr int kLmRows = 64, kLmRowsPerWave = kLmRows / (kThreads / 64), kLmChunksPerStep = 64 * 4;
+
+struct LmHeadArgs {
+  const _Float16* wp;
+  const _Float16* hs;      // hidden in LDS
+  float* row_logit;        // kLmRows entries of LDS
+  Best* scratch;
+  float* block_max;
+  uint32_t* block_idx;
+  int64_t w_stride0, max_stride, idx_stride;
+  int32_t w_rows, chunks, steps_per_pair, steps_per_block, b_begin, vocab_size;
+  int lane, wave;
+};
+
+typedef Vec16<_Float16> LmTile[2][4];
+
+__device__ __forceinline__ void lm_head_issue(LmTile& w, const LmHeadArgs& a, int32_t step) {
+  const int32_t b = a.b_begin + step / a.steps_per_block, in_block = step % a.steps_per_block;
+  const int64_t r0 = (int64_t)b * kLmRows + (in_block / a.steps_per_pair * (kThreads / 64) + a.wave) * 2;
+  const int32_t c0 = in_block % a.steps_per_pair * kLmChunksPerStep;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int32_t c = c0 + u * 64 + a.lane;
+      w[t][u].raw = u32x4{0, 0, 0, 0};   // a row beyond the matrix reads as zeros, like a padded tile load
+      if (r0 + t < a.w_rows && c < a.chunks)
+        w[t][u].raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.wp + (r0 + t) * a.w_stride0) + c);
+    }
+}
+
+__device__ __forceinline__ void lm_head_consume(const LmTile& w, float (&acc)[2], const LmHeadArgs& a, int32_t step) {
+  const int32_t b = a.b_begin + step / a.steps_per_block, in_block = step % a.steps_per_block;
+  const int32_t pair = in_block / a.steps_per_pair, part = in_block % a.steps_per_pair;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int32_t c = part * kLmChunksPerStep + u * 64 + a.lane;
+    if (c < a.chunks) {
+      Vec16<_Float16> h;
+      h.raw = *reinterpret_cast<const u32x4*>(a.hs + (int64_t)c * 8);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[t] = __builtin_fmaf((float)w[t][u].v[e], (float)h.v[e], acc[t]);
+    }
+  }
+  if (part + 1 < a.steps_per_pair) return;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc[t] += __shfl_xor(acc[t], o, 64);
+    if (a.lane == 0) a.row_logit[(pair * (kThreads / 64) + a.wave) * 2 + t] = acc[t];
+    acc[t] = 0.0f;
+  }
+  if (in_block + 1 < a.steps_per_block) return;
+  __syncthreads();
+  Best mine = {-INFINITY, INT32_MAX};
+  if (threadIdx.x < kLmRows) {
+    const int64_t idx = (int64_t)b * kLmRows + threadIdx.x;
+    mine = Best{idx < a.vocab_size ? a.row_logit[threadIdx.x] : kMaskedLogit, (int32_t)idx};
+  }
+  const Best r = block_best(mine, a.scratch);   // its barrier also orders these reads before the next block's writes
+  if (threadIdx.x == 0) {
+    a.block_max[(int64_t)b * a.max_stride] = r.v;
+    a.block_idx[(int64_t)b * a.idx_stride] = (uint32_t)r.i;
+  }
+}
+
+}  // namespace
+
 extern "C" __global__ void __launch_bounds__(kThreads)
     lm_head_argmax_blocks_entry__f16(TensorArg<2> weights, TensorArg<2> hidden, PartitionArg<1> block_max,
                                      PartitionArg<1> block_idx, int32_t vocab_size, TileGrid g) {
-  constexpr int kRows = 64, kRowsPerWave = kRows / (kThreads / 64);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  __shared__ float row_logit[kRows];
+  __shared__ float row_logit[kLmRows];
   __shared__ Best scratch[kThreads / 64];
-  const int32_t b = blockIdx.x;
-  if (b >= (int32_t)g.x || b >= block_max.shape[0] || b >= block_idx.shape[0]) return;
+  const int32_t n_blocks = min((int32_t)g.x, min(block_max.shape[0], block_idx.shape[0]));
+  const int32_t b_begin = (int32_t)((int64_t)blockIdx.x * n_blocks / gridDim.x);
+  const int32_t b_end = (int32_t)((int64_t)(blockIdx.x + 1) * n_blocks / gridDim.x);
+  if (b_begin >= b_end) return;
   const int32_t k_len = min(weights.shape[1], hidden.shape[1]);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const _Float16* wp = (const _Float16*)weights.ptr;
@@ -610,61 +686,50 @@ extern "C" __global__ void __launch_bounds__(kThreads)
                    (((uintptr_t)wp | (uintptr_t)hp) & 15) == 0;
   for (int32_t k = threadIdx.x; k < k_len; k += kThreads) hs[k] = hp[(int64_t)k * hidden.strides[1]];
   __syncthreads();
-  const int64_t row0 = (int64_t)b * kRows + wave * kRowsPerWave;
-  for (int rr = 0; rr < kRowsPerWave; rr += 2) {
+  if (vec) {
+    LmHeadArgs a;
+    a.wp = wp, a.hs = hs, a.row_logit = row_logit, a.scratch = scratch;
+    a.block_max = (float*)block_max.ptr, a.block_idx = (uint32_t*)block_idx.ptr;
+    a.w_stride0 = weights.strides[0], a.max_stride = block_max.strides[0], a.idx_stride = block_idx.strides[0];
+    a.w_rows = weights.shape[0], a.chunks = k_len / 8;
+    a.steps_per_pair = max((a.chunks + kLmChunksPerStep - 1) / kLmChunksPerStep, 1);
+    a.steps_per_block = a.steps_per_pair * (kLmRowsPerWave / 2);
+    a.b_begin = b_begin, a.vocab_size = vocab_size, a.lane = lane, a.wave = wave;
+    const int32_t steps = (b_end - b_begin) * a.steps_per_block;
     float acc[2] = {0.0f, 0.0f};
-    if (vec) {
-      const int32_t chunks = k_len / 8;
-      for (int32_t c0 = 0; c0 < chunks; c0 += 64 * 4) {
-        Vec16<_Float16> w[2][4];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int64_t r = row0 + rr + t;
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int32_t c = c0 + u * 64 + lane;
-            if (r < weights.shape[0] && c < chunks)
-              w[t][u].raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + r * weights.strides[0]) + c);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int32_t c = c0 + u * 64 + lane;
-          if (c < chunks) {
-            Vec16<_Float16> h;
-            h.raw = *reinterpret_cast<const u32x4*>(hs + (int64_t)c * 8);
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-              for (int e = 0; e < 8; ++e) acc[t] = __builtin_fmaf((float)w[t][u].v[e], (float)h.v[e], acc[t]);
-          }
-        }
-      }
-    } else {
-      for (int t = 0; t < 2; ++t) {
-        const int64_t r = row0 + rr + t;
-        if (r < weights.shape[0])
-          for (int32_t k = lane; k < k_len; k += 64)
-            acc[t] = __builtin_fmaf((float)wp[r * weights.strides[0] + (int64_t)k * weights.strides[1]], (float)hs[k], acc[t]);
-      }
+    LmTile even, odd;
+    lm_head_issue(even, a, 0);
+    for (int32_t s = 0; s < steps; s += 2) {
+      if (s + 1 < steps) lm_head_issue(odd, a, s + 1);
+      lm_head_consume(even, acc, a, s);
+      if (s + 2 < steps) lm_head_issue(even, a, s + 2);
+      if (s + 1 < steps) lm_head_consume(odd, acc, a, s + 1);
     }
+    return;
+  }
+  for (int32_t b = b_begin; b < b_end; ++b) {
+    const int64_t row0 = (int64_t)b * kLmRows + wave * kLmRowsPerWave;
+    for (int rr = 0; rr < kLmRowsPerWave; ++rr) {
+      const int64_t r = row0 + rr;
+      float acc = 0.0f;
+      if (r < weights.shape[0])
+        for (int32_t k = lane; k < k_len; k += 64)
+          acc = __builtin_fmaf((float)wp[r * weights.strides[0] + (int64_t)k * weights.strides[1]], (float)hs[k], acc);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) acc[t] += __shfl_xor(acc[t], o, 64);
-      if (lane == 0) row_logit[wave * kRowsPerWave + rr + t] = acc[t];
+      for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      if (lane == 0) row_logit[wave * kLmRowsPerWave + rr] = acc;
     }
-  }
-  __syncthreads();
-  Best mine = {-INFINITY, INT32_MAX};
-  if (threadIdx.x < kRows) {
-    const int64_t idx = (int64_t)b * kRows + threadIdx.x;
-    mine = Best{idx < vocab_size ? row_logit[threadIdx.x] : kMaskedLogit, (int32_t)idx};
-  }
-  const Best r = block_best(mine, scratch);
-  if (threadIdx.x == 0) {
-    ((float*)block_max.ptr)[(int64_t)b * block_max.strides[0]] = r.v;
-    ((uint32_t*)block_idx.ptr)[(int64_t)b * block_idx.strides[0]] = (uint32_t)r.i;
+    __syncthreads();
+    Best mine = {-INFINITY, INT32_MAX};
+    if (threadIdx.x < kLmRows) {
+      const int64_t idx = (int64_t)b * kLmRows + threadIdx.x;
+      mine = Best{idx < vocab_size ? row_logit[threadIdx.x] : kMaskedLogit, (int32_t)idx};
+    }
+    const Best r = block_best(mine, scratch);
+    if (threadIdx.x == 0) {
+      ((float*)block_max.ptr)[(int64_t)b * block_max.strides[0]] = r.v;
+      ((uint32_t*)block_idx.ptr)[(int64_t)b * block_idx.strides[0]] = (uint32_t)r.i;
+    }
   }
 }
 

@@ -130,7 +130,8 @@ def test_gpu_argmax_blocks_and_reduce(ct, dev, n, bs, length):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("rows,k,vocab", [(4096, 1024, 4096), (1000, 256, 990), (130, 4096, 130), (640, 96, 640), (200, 8192, 150)])
+@pytest.mark.parametrize("rows,k,vocab", [(4096, 1024, 4096), (1000, 256, 990), (130, 4096, 130), (640, 96, 640), (200, 8192, 150),
+                                            (40000, 2080, 39990), (70016, 64, 70016)])
 def test_gpu_lm_head_argmax(ct, dev, rows, k, vocab):
     w, h = f16b(oracle.normal_f32((rows, k), 841)), f16b(oracle.normal_f32(k, 842))
     nb = -(-rows // 64)
