@@ -233,9 +233,9 @@ std::vector<KernelEntry> build_table() {
       add("fmha_decode_gqa_split", keep(v), keep("fmha_decode_gqa_split_entry__" + v), IMG_FMHA, 256,
           (uint32_t)(4 * grp * (d + 2) * 4), grp, 0, d, 0, "f16", 0, 3);
     }
-  // wide groups on the matrix cores (heads are the N dimension of a 16x16x32 MFMA); LDS = 4 wavefronts x 2 stages x 32 V rows
+  // the same on the matrix cores (heads are the N dimension of a 16x16x32 MFMA, columns beyond GROUP are zero); LDS = 4 wavefronts x 2 stages x 32 V rows
   for (int d : {64, 128, 256})
-    for (int grp : {8, 16}) {
+    for (int grp : {1, 2, 4, 8, 16}) {
       std::string v = "f16_g" + std::to_string(grp) + "_d" + std::to_string(d) + "_mfma";
       add("fmha_decode_gqa_split", keep(v), keep("fmha_decode_gqa_split_entry__" + v), IMG_FMHA, 256, (uint32_t)(4 * 2 * 32 * d * 2), grp,
           0, d, 0, "f16", 0, 3);

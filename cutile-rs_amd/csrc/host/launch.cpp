@@ -1305,10 +1305,12 @@ cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, cons
   CUTILE_REQUIRE(decode_vec_layout(*q) && decode_vec_layout(*k) && decode_vec_layout(*v) && decode_vec_layout(at) &&
                      ((uintptr_t)position_start->ptr & 3) == 0 && ((uintptr_t)lt.ptr & 3) == 0,
                  CUTILE_ERR_KERNEL_NOT_FOUND, "fmha_decode_gqa_split: precompiled variants need unit head-dim stride and 16-byte aligned rows");
-  // GROUP >= 8: the matrix-core variant first (the vector-ALU one no longer keeps up with HBM there)
+  // The matrix-core variant first: from GROUP 4 on the vector-ALU one no longer keeps up with HBM, and at D = 64 and
+  // 256 it is the slower one for every group; only GROUP 1 and 2 at D = 128 measured (3 %) faster on the vector ALUs.
   const std::string plain = "f16_g" + std::to_string(group) + "_d" + std::to_string(d);
   std::vector<std::string> acceptable;
-  for (const std::string& name : {plain + "_mfma", plain})
+  const bool vector_first = group <= 2 && d == 128;
+  for (const std::string& name : {vector_first ? plain : plain + "_mfma", vector_first ? plain + "_mfma" : plain})
     if (find_entry("fmha_decode_gqa_split", name)) acceptable.push_back(name);
   CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND,
                  "no precompiled variant of fmha_decode_gqa_split<GROUP=%d, D=%d>; available: %s", group, d,

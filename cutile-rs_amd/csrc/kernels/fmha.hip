@@ -969,9 +969,9 @@ __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const Tensor
   }
 }
 
-// ---- decode attention on the matrix cores, for wide groups ---------------------------------------
-// With GROUP >= 8 the vector ALUs no longer keep up with HBM (two dot products per cached value
-// and head).  Here a wavefront takes 32 keys at a time and uses v_mfma_f32_16x16x32_f16 with
+// ---- decode attention on the matrix cores ----------------------------------------------------
+// With GROUP >= 4 the vector ALUs no longer keep up with HBM (two dot products per cached value
+// and head), and at D = 64 they do not for any group.  Here a wavefront takes 32 keys at a time and uses v_mfma_f32_16x16x32_f16 with
 // the query heads as the 16-wide N dimension (heads beyond GROUP are zero):
 //   S^T [16 keys x 16 heads]  = K [16 keys x D]   . Q^T [D x 16 heads]     (two blocks of 16 keys)
 //   O^T [D x 16 heads]       += V^T [D x 32 keys]  . P^T [32 keys x 16 heads]
@@ -1326,6 +1326,15 @@ DECODE_SPLIT_GROUPS(256)
                                                           int32_t bn, TileGrid g) {                \
     decode_split_mfma<G, D>(q, k, v, att_out, lse_out, qk_scale, position_start, bn, g);          \
   }
+DECODE_SPLIT_MFMA_KERNEL(1, 64)
+DECODE_SPLIT_MFMA_KERNEL(1, 128)
+DECODE_SPLIT_MFMA_KERNEL(1, 256)
+DECODE_SPLIT_MFMA_KERNEL(2, 64)
+DECODE_SPLIT_MFMA_KERNEL(2, 128)
+DECODE_SPLIT_MFMA_KERNEL(2, 256)
+DECODE_SPLIT_MFMA_KERNEL(4, 64)
+DECODE_SPLIT_MFMA_KERNEL(4, 128)
+DECODE_SPLIT_MFMA_KERNEL(4, 256)
 DECODE_SPLIT_MFMA_KERNEL(8, 64)
 DECODE_SPLIT_MFMA_KERNEL(8, 128)
 DECODE_SPLIT_MFMA_KERNEL(8, 256)

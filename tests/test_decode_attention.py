@@ -174,12 +174,13 @@ def test_gpu_decode_split_and_merge(ct, dev, heads, group, d, max_seq, pos, bn, 
     q, k, v = normal_f16_bits((heads, group, d), 751), normal_f16_bits((heads, max_seq, d), 752), normal_f16_bits((heads, max_seq, d), 753)
     scale = float(np.float16(1.0 / np.sqrt(d)))
     att, lse, out = _run_decode(ct, dev, q, k, v, scale, pos, bn, splits)
-    if group == 8:      # GROUP 8 has two variants: the matrix-core one is the default, the vector-ALU one must agree too
-        att_v, lse_v, out_v = _run_decode(ct, dev, q, k, v, scale, pos, bn, splits, variant=f"f16_g8_d{d}")
-        assert np.max(np.abs(f32(att_v) - f32(att))) <= 2e-2 and np.max(np.abs(f32(out_v) - f32(out))) <= 2e-2
-        assert np.allclose(lse_v, lse, atol=2e-3)
     att_ref, lse_ref = oracle.fmha_decode_gqa_split(q, k, v, scale, pos, bn, splits)
     out_ref = oracle.splitk_reduce_merge(att_ref, lse_ref, group)
+    if group <= 8:      # two variants up to GROUP 8 (vector ALUs, matrix cores): whichever is not the default must hold too
+        for variant in (f"f16_g{group}_d{d}", f"f16_g{group}_d{d}_mfma"):
+            att_v, lse_v, out_v = _run_decode(ct, dev, q, k, v, scale, pos, bn, splits, variant=variant)
+            assert np.max(np.abs(f32(att_v) - f32(att_ref))) <= 2e-2 and np.max(np.abs(f32(out_v) - f32(out_ref))) <= 2e-2
+            assert np.array_equal(lse_ref > -1e29, lse_v > -1e29) and np.allclose(lse_v, lse_ref, atol=2e-3)
     # tolerance: max-abs 2e-2 as for the prefill attention kernel; observed differences are a few f16 ulps
     # (the kernel sums each split's keys in a different order than the tile program does)
     assert np.max(np.abs(f32(att) - f32(att_ref))) <= 2e-2

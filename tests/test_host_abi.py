@@ -299,7 +299,7 @@ def test_decode_mapped_and_fp4_launchers_on_the_recording_runtime(fake_hip):
     pos = torch.zeros(1, dtype=torch.int32)
     ct.fmha_decode_gqa_split(q, kv, kv, ct.partition(att, [1, 4, 128]), ct.partition(lse, [1, 4]), 0.088, pos, generics=[4, 64, 128, 16])
     rec, args = _last(ct)
-    assert rec.symbol == b"fmha_decode_gqa_split_entry__f16_g4_d128" and tuple(rec.grid) == (8, 16, 1) and tuple(rec.block) == (256, 1, 1)
+    assert rec.symbol == b"fmha_decode_gqa_split_entry__f16_g4_d128_mfma" and tuple(rec.grid) == (8, 16, 1) and tuple(rec.block) == (256, 1, 1)
     # q (32) + k (32) + v (32) + att partition (56) + lse partition (40) = 192, then scale, pad, position pointer, bn, tile grid
     scale, = struct.unpack_from("<f", args, 192)
     ptr, bn = struct.unpack_from("<Qi", args, 200)
