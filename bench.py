@@ -546,6 +546,47 @@ class DecodeAttentionWide(DecodeAttention):
                           "131072 cached keys, 32 KV splits (one workgroup per CU), BN 64 (two launches per step)"}
 
 
+class DecodeAttentionGrouped(Workload):
+    """attention_decode_kernel_grouped (cutile-kernels/src/experimental/attention.rs:385-846): the split-KV decode partial
+    over a batch of sequences; every cached K and V byte is read once."""
+    name, unit, dtype = "decode_grouped_f16_b8h8g4d128_s16384", "GB/s", "f16 io / f32 softmax+acc"
+    batch, heads, group, d, s, splits, tile_n = 8, 8, 4, 128, 16384, 4, 64
+    work = float(2 * batch * heads * s * d * 2)
+    config = {"workload": "attention_decode_kernel_grouped fp16: batch 8 x 8 KV heads x GROUP 4, D 128, 16384 cached keys each, "
+                          "4 KV splits of 4096 keys (one workgroup per CU), TILE_N 64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        bits = lambda shape, seed: oracle.f32_to_f16_bits(oracle.normal_f32(shape, seed))
+        self.qb = bits((self.batch, self.heads, self.group, self.d), 91)
+        self.kb, self.vb = bits((self.batch, self.heads, self.s, self.d), 92), bits((self.batch, self.heads, self.s, self.d), 93)
+        self.q, self.k, self.v = (_td_f16(torch, np, t, dev) for t in (self.qb, self.kb, self.vb))
+        self.att = torch.empty(self.batch, self.heads, self.group, self.splits, self.d, dtype=torch.float16, device=dev)
+        self.lse = torch.empty(self.batch, self.heads, self.group, self.splits, dtype=torch.float32, device=dev)
+        self.count = torch.tensor([self.s], dtype=torch.int32, device=dev)
+        self.scale = float(np.float16(self.d ** -0.5))
+
+    def launch(self):
+        self.ct.attention_decode_kernel_grouped_f16(self.q, self.k, self.v, self.att, self.lse, self.scale, self.count,
+                                                    tile_n=self.tile_n, kv_len_per_split=self.s // self.splits,
+                                                    query_group_tile_size=16)
+
+    def cpu_baseline(self, oracle, np, torch):
+        nb = 2                                   # the first two sequences of the batch: independent sub-problems
+        t0 = time.perf_counter()
+        att, lse = oracle.attention_decode_grouped_f16(self.qb[:nb], self.kb[:nb], self.vb[:nb], self.scale, self.s, self.tile_n,
+                                                       self.s // self.splits, self.splits)
+        dt = time.perf_counter() - t0
+        got = oracle.f16_bits_to_f32(self.att[:nb].cpu().numpy().view(np.uint16))
+        err = float(np.max(np.abs(got - oracle.f16_bits_to_f32(att))))
+        err_lse = float(np.max(np.abs(self.lse[:nb].cpu().numpy() - lse)))
+        return {"value": self.work * nb / self.batch / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"the first {nb} of {self.batch} sequences"}, \
+               {"max_abs": err, "max_abs_lse": err_lse, "tolerance": 2e-2, "ok": err <= 2e-2 and err_lse <= 2e-3}
+
+
 class PrefillAttention(Workload):
     """fmha_prefill_causal (cutile-kernels/src/attention.rs:242-391): f16, [seq, heads, D] queries against a
     [kv_heads, seq, D] cache, grouped heads; flops counted like the causal FMHA bench (half of 4 s^2 d per head)."""
@@ -745,7 +786,7 @@ class EmbeddingBatch(Workload):
 
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run

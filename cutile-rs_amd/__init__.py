@@ -466,6 +466,22 @@ def fmha_decode_gqa_split(q, k, v, att_out: Partition, lse_out: Partition, qk_sc
                                                     C.byref(pa), C.byref(o)))
 
 
+def attention_decode_kernel_grouped_f16(q, k, v, att, lse, softmax_scale: float, s_kv, *, tile_n: int = 64,
+                                        kv_len_per_split: int, query_group_tile_size=None, stream=None, grid=None,
+                                        generics=None) -> None:
+    """experimental/attention.rs:385-846 on device tensors: q [B, H_kv, G, D], k and v [B, H_kv, S, D],
+    att [B, H_kv, G, splits, D], lse [B, H_kv, G, splits] (f32), s_kv one int32 in device memory."""
+    def group(t, rank):
+        if t.dim() != rank or t.stride(-1) != 1:
+            raise ValueError(f"attention_decode_kernel_grouped: expected rank {rank} with unit innermost stride")
+        return (C.c_void_p(t.data_ptr()), (C.c_int32 * rank)(*t.shape), (C.c_int32 * (rank - 1))(*t.stride()[:-1]))
+    o, keep = _opts(grid, generics, None)
+    qgts = int(query_group_tile_size) if query_group_tile_size is not None else max(int(q.shape[2]), 1)
+    check(lib().cutile_launch_attention_decode_kernel_grouped_f16(
+        _stream(stream), *group(q, 4), *group(k, 4), *group(v, 4), *group(att, 5), *group(lse, 4), C.c_float(softmax_scale),
+        C.c_void_p(s_kv.data_ptr()), int(tile_n), int(kv_len_per_split), qgts, C.byref(o)))
+
+
 def splitk_reduce_merge(att_partial, lse_partial, out: Partition, *, stream=None, grid=None, generics=None) -> None:
     aa, la = tensor_arg(att_partial), tensor_arg(lse_partial)
     o, keep = _opts(grid, generics, None)

@@ -240,6 +240,13 @@ std::vector<KernelEntry> build_table() {
       add("fmha_decode_gqa_split", keep(v), keep("fmha_decode_gqa_split_entry__" + v), IMG_FMHA, 256, (uint32_t)(4 * 2 * 32 * d * 2), grp,
           0, d, 0, "f16", 0, 3);
     }
+  // the batched-layout form of the matrix-core kernel: one workgroup per (batch, KV head, split)
+  for (int d : {64, 128, 256})
+    for (int grp : {1, 2, 4, 8, 16}) {
+      std::string v = "f16_g" + std::to_string(grp) + "_d" + std::to_string(d);
+      add("attention_decode_kernel_grouped", keep(v), keep("attention_decode_grouped_entry__" + v), IMG_FMHA, 256,
+          (uint32_t)(4 * 2 * 32 * d * 2), grp, 0, d, 0, "f16", 0, 3);
+    }
   add("splitk_reduce_merge", "f16", "splitk_reduce_merge_entry__f16", IMG_FMHA, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 
   // ---- MXFP8 GEMM: LDS = 2 stages x (BM + BN) x 128 bytes ----

@@ -1331,6 +1331,82 @@ cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, cons
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+cutile_status_t cutile_launch_attention_decode_kernel_grouped_f16(
+    cutile_stream_t stream, const void* q, const int32_t* q_shape, const int32_t* q_strides, const void* k,
+    const int32_t* k_shape, const int32_t* k_strides, const void* v, const int32_t* v_shape, const int32_t* v_strides,
+    void* att, const int32_t* att_shape, const int32_t* att_strides, void* lse, const int32_t* lse_shape,
+    const int32_t* lse_strides, float softmax_scale, const void* s_kv, int32_t tile_n, int32_t kv_len_per_split,
+    int32_t query_group_tile_size, const cutile_launch_opts_t* opts) {
+  const char* fn = "attention_decode_kernel_grouped";
+  CUTILE_REQUIRE(q && k && v && att && lse && s_kv && q_shape && q_strides && k_shape && k_strides && v_shape && v_strides &&
+                     att_shape && att_strides && lse_shape && lse_strides,
+                 CUTILE_ERR_INVALID_ARGUMENT, "%s: null argument", fn);
+  for (int i = 0; i < 4; ++i)
+    CUTILE_REQUIRE(q_shape[i] > 0 && k_shape[i] > 0 && v_shape[i] > 0 && lse_shape[i] > 0, CUTILE_ERR_TENSOR,
+                   "%s: Shape dimensions must be positive.", fn);
+  for (int i = 0; i < 5; ++i)
+    CUTILE_REQUIRE(att_shape[i] > 0, CUTILE_ERR_TENSOR, "%s: Shape dimensions must be positive.", fn);
+  const int32_t batch = q_shape[0], kv_heads = q_shape[1], group = q_shape[2], d = q_shape[3], splits = att_shape[3];
+  CUTILE_REQUIRE(k_shape[0] == batch && k_shape[1] == kv_heads && k_shape[3] == d && v_shape[0] == batch && v_shape[1] == kv_heads &&
+                     v_shape[3] == d && att_shape[0] == batch && att_shape[1] == kv_heads && att_shape[2] == group && att_shape[4] == d &&
+                     lse_shape[0] == batch && lse_shape[1] == kv_heads && lse_shape[2] == group && lse_shape[3] == splits,
+                 CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: q [B, H_kv, G, D], k/v [B, H_kv, S, D], att [B, H_kv, G, NUM_KV_SPLITS, D] and lse [B, H_kv, G, NUM_KV_SPLITS] do not agree", fn);
+  CUTILE_REQUIRE(tile_n > 0 && kv_len_per_split > 0 && query_group_tile_size >= group, CUTILE_ERR_KERNEL_LAUNCH,
+                 "%s: TILE_N and KV_LEN_PER_SPLIT must be positive and QUERY_GROUP_TILE_SIZE (%d) at least NUM_Q_HEAD_PER_KV (%d)", fn,
+                 query_group_tile_size, group);
+  // with a remainder the tile program's splits overlap (its first tile is start / TILE_N rounded down, attention.rs:640-641)
+  CUTILE_REQUIRE(kv_len_per_split % tile_n == 0, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "%s: the precompiled kernels need KV_LEN_PER_SPLIT (%d) to be a multiple of TILE_N (%d)", fn, kv_len_per_split, tile_n);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(d), "HEAD_DIM")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(tile_n), "TILE_N")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(kv_len_per_split), "KV_LEN_PER_SPLIT")) return s;
+  if (cutile_status_t s = check_generic(opts, 3, std::to_string(group), "NUM_Q_HEAD_PER_KV")) return s;
+  if (cutile_status_t s = check_generic(opts, 4, std::to_string(query_group_tile_size), "QUERY_GROUP_TILE_SIZE")) return s;
+  if (cutile_status_t s = check_generic(opts, 5, std::to_string(splits), "NUM_KV_SPLITS")) return s;
+  auto rows_ok = [&](const int32_t* strides, int n) {
+    for (int i = 0; i < n; ++i)
+      if (strides[i] < 0 || strides[i] % 8 != 0) return false;
+    return true;
+  };
+  const int64_t v_extent = ((int64_t)(v_shape[2] - 1) * v_strides[2] + d) * 2;
+  CUTILE_REQUIRE(rows_ok(q_strides, 3) && rows_ok(k_strides, 3) && rows_ok(v_strides, 3) && rows_ok(att_strides, 4) &&
+                     lse_strides[0] >= 0 && lse_strides[1] >= 0 && lse_strides[2] >= 0 && aligned16(q) && aligned16(k) &&
+                     aligned16(v) && aligned16(att) && ((uintptr_t)lse & 3) == 0 && ((uintptr_t)s_kv & 3) == 0 &&
+                     v_extent <= 0xffffffffll,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "%s: precompiled variants need 16-byte aligned pointers, strides that are multiples of 8 elements and less than 4 GiB of V per head", fn);
+  uint32_t tg[3] = {(uint32_t)batch, (uint32_t)kv_heads, (uint32_t)splits};
+  if (opts && (opts->grid[0] || opts->grid[1] || opts->grid[2])) {
+    CUTILE_REQUIRE(opts->grid[0] == tg[0] && opts->grid[1] == tg[1] && opts->grid[2] == tg[2], CUTILE_ERR_KERNEL_LAUNCH,
+                   "%s: launch grid (%u, %u, %u) is not (batch, kv heads, NUM_KV_SPLITS) = (%u, %u, %u)", fn, opts->grid[0],
+                   opts->grid[1], opts->grid[2], tg[0], tg[1], tg[2]);
+  }
+  const std::string name = "f16_g" + std::to_string(group) + "_d" + std::to_string(d);
+  CUTILE_REQUIRE(find_entry(fn, name), CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no precompiled variant of %s<NUM_Q_HEAD_PER_KV=%d, HEAD_DIM=%d>; available: %s", fn, group, d, list_variants(fn).c_str());
+  Resolved res;
+  if (cutile_status_t s = resolve_entry(fn, opts, name, {name}, &res)) return s;
+  ArgPacker args;
+  args.push_val<const void*>(q);
+  args.push_val<const void*>(k);
+  args.push_val<const void*>(v);
+  args.push_val<void*>(att);
+  args.push_val<void*>(lse);
+  args.push_val<const void*>(s_kv);
+  for (int i = 0; i < 3; ++i) args.push_val<int32_t>(q_strides[i]);
+  for (int i = 0; i < 3; ++i) args.push_val<int32_t>(k_strides[i]);
+  for (int i = 0; i < 3; ++i) args.push_val<int32_t>(v_strides[i]);
+  for (int i = 0; i < 4; ++i) args.push_val<int32_t>(att_strides[i]);
+  for (int i = 0; i < 3; ++i) args.push_val<int32_t>(lse_strides[i]);
+  args.push_val<int32_t>(k_shape[2]);
+  args.push_val<int32_t>(v_shape[2]);
+  args.push_val<int32_t>(kv_len_per_split);
+  args.push_val<float>(softmax_scale);
+  args.push_tile_grid(tg);
+  return launch_packed(res.fn, tg, res.entry->block, 0, stream, args);
+}
+
 cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const cutile_tensor_arg_t* att_partial,
                                                   const cutile_tensor_arg_t* lse_partial, const cutile_partition_arg_t* out,
                                                   const cutile_launch_opts_t* opts) {

@@ -985,10 +985,23 @@ __device__ __forceinline__ void decode_split(const TensorArg<3>& q, const Tensor
 // so the transposing reads of 4 rows x 2 chunks are conflict-free) and reads them back with
 // ds_read_b64_tr_b16.  Two stages, one 32-key slab ahead; wavefront-private, so the loop has no
 // barrier.  Slabs past the end of the split re-read its last row and are masked (p = 0).
+// What one workgroup works on: the queries of one KV head, keys [r0, r1) of its cache, and where the partial
+// result of query head c goes (att + c * att_row_stride, lse + c * lse_row_stride).
+struct DecodeSplitView {
+  const _Float16* q;
+  const _Float16* k;
+  const _Float16* v;
+  _Float16* att;
+  float* lse;
+  int64_t q_row_stride, k_row_stride, v_row_stride, att_row_stride, lse_row_stride;
+  int32_t v_rows;      // rows of v that exist (extent of its buffer descriptor)
+  int32_t r0, r1;
+  float empty_sum;     // what a split without keys reports: its sum (the output is 0 / sum) and its lse
+  float empty_lse;
+};
+
 template <int G, int D>
-__device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const TensorArg<3>& k, const TensorArg<3>& v,
-                                                  const PartitionArg<3>& att_out, const PartitionArg<2>& lse_out,
-                                                  float qk_scale, const uint32_t* pos_dev, int32_t bn, const TileGrid& g) {
+__device__ __forceinline__ void decode_split_mfma_view(const DecodeSplitView& w, float qk_scale) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   constexpr int kWaves = 4, kSlab = 32;
   constexpr int QS = D / 32;                 // K slices of the first product
@@ -1002,12 +1015,7 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, quad = lane >> 4;           // head (column) and key group of this lane
-  const int32_t head = blockIdx.x, split = blockIdx.y, splits = (int32_t)g.y;
-  const int32_t max_seq = min(k.shape[1], v.shape[1]);
-  const int32_t s_kv = min((int32_t)pos_dev[0] + 1, max_seq);
-  const int32_t tiles = (s_kv + bn - 1) / bn, per_split = (tiles + splits - 1) / splits;
-  const int32_t r0 = split * per_split * bn;
-  const int32_t r1 = min(min((split + 1) * per_split, tiles) * bn, s_kv);
+  const int32_t r0 = w.r0, r1 = w.r1;
   const float c = qk_scale * kLog2e;
 
   // Q^T operands: column = head, 8 consecutive d per lane and slice
@@ -1015,12 +1023,12 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
 #pragma unroll
   for (int sidx = 0; sidx < QS; ++sidx) {
     f16x8 t = {};
-    if (col < G) t = *reinterpret_cast<const f16x8*>((const _Float16*)q.ptr + (int64_t)head * q.strides[0] + (int64_t)col * q.strides[1] + sidx * 32 + quad * 8);
+    if (col < G) t = *reinterpret_cast<const f16x8*>(w.q + (int64_t)col * w.q_row_stride + sidx * 32 + quad * 8);
     qf[sidx] = t;
   }
-  const _Float16* kb = (const _Float16*)k.ptr + (int64_t)head * k.strides[0];
-  const _Float16* vbase = (const _Float16*)v.ptr + (int64_t)head * v.strides[0];
-  const __amdgpu_buffer_rsrc_t rv = make_rsrc(vbase, (uint32_t)(((int64_t)(max_seq - 1) * v.strides[1] + D) * 2));
+  const _Float16* kb = w.k;
+  const int64_t k_row_stride = w.k_row_stride, v_row_stride = w.v_row_stride;
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(w.v, (uint32_t)(((int64_t)(w.v_rows - 1) * v_row_stride + D) * 2));
   unsigned char* my_stage[2] = {vst[wave][0], vst[wave][1]};
 
   // LDS side of the transposing reads: lane i of a 16-lane group supplies row (i >> 2), columns 4 (i & 3) .. + 3
@@ -1040,7 +1048,7 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       const int32_t row = min(base + blk * 16 + col, r1 - 1);
 #pragma unroll
       for (int sidx = 0; sidx < QS; ++sidx)
-        kreg[blk][sidx] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (int64_t)row * k.strides[1] + sidx * 32 + quad * 8));
+        kreg[blk][sidx] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (int64_t)row * k_row_stride + sidx * 32 + quad * 8));
     }
 #pragma unroll
     for (int i = 0; i < kVInstr; ++i) {
@@ -1048,7 +1056,7 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       const int chunk = (lane % CP) ^ ((lrow & 3) << 1);
       const int32_t row = min(base + lrow, r1 - 1);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (LDS_PTR(void))(stage + i * 1024), 16,
-                                               (uint32_t)(((int64_t)row * v.strides[1] + chunk * 8) * 2), 0, 0, decode::kNontemporal);
+                                               (uint32_t)(((int64_t)row * v_row_stride + chunk * 8) * 2), 0, 0, decode::kNontemporal);
     }
   };
 
@@ -1146,10 +1154,9 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       f[w] = __builtin_amdgcn_exp2f(sm[w * 16 + col] - mt);
       lt += sl[w * 16 + col] * f[w];
     }
-    if (r0 >= r1) lt = (float)bn;   // no keys in this split: the tile program's untouched l = 1 per lane
+    if (r0 >= r1) lt = w.empty_sum;   // no keys in this split: the tile program's untouched l = 1 per lane
     const float safe = fmaxf(lt, 1.0e-8f);
-    const int64_t orow = (int64_t)split * G + col;
-    _Float16* dst = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + orow * att_out.strides[1];
+    _Float16* dst = w.att + (int64_t)col * w.att_row_stride;
 #pragma unroll
     for (int i = 0; i < OS; ++i) {
       f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1160,8 +1167,75 @@ __device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const T
       for (int j = 0; j < 4; ++j) o[j] = (_Float16)(a[j] / safe);
       *reinterpret_cast<f16x4*>(dst + i * 16 + quad * 4) = o;
     }
-    if (quad == 0) ((float*)lse_out.ptr)[(int64_t)head * lse_out.strides[0] + orow * lse_out.strides[1]] = mt + __builtin_log2f(safe);
+    if (quad == 0) w.lse[(int64_t)col * w.lse_row_stride] = r0 >= r1 ? w.empty_lse : mt + __builtin_log2f(safe);
   }
+}
+
+// fmha_decode_gqa_split: q [kv_heads, GROUP, D], k and v [kv_heads, max_seq, D], partial results at row
+// split * GROUP + c of att_out [kv_heads, splits * GROUP, D] and lse_out [kv_heads, splits * GROUP]; the tiles of
+// `bn` keys are dealt to the splits in equal runs.
+template <int G, int D>
+__device__ __forceinline__ void decode_split_mfma(const TensorArg<3>& q, const TensorArg<3>& k, const TensorArg<3>& v,
+                                                  const PartitionArg<3>& att_out, const PartitionArg<2>& lse_out,
+                                                  float qk_scale, const uint32_t* pos_dev, int32_t bn, const TileGrid& g) {
+  const int32_t head = blockIdx.x, split = blockIdx.y, splits = (int32_t)g.y;
+  const int32_t max_seq = min(k.shape[1], v.shape[1]);
+  const int32_t s_kv = min((int32_t)pos_dev[0] + 1, max_seq);
+  const int32_t tiles = (s_kv + bn - 1) / bn, per_split = (tiles + splits - 1) / splits;
+  DecodeSplitView w;
+  w.r0 = split * per_split * bn;
+  w.r1 = min(min((split + 1) * per_split, tiles) * bn, s_kv);
+  w.q = (const _Float16*)q.ptr + (int64_t)head * q.strides[0];
+  w.k = (const _Float16*)k.ptr + (int64_t)head * k.strides[0];
+  w.v = (const _Float16*)v.ptr + (int64_t)head * v.strides[0];
+  w.q_row_stride = q.strides[1], w.k_row_stride = k.strides[1], w.v_row_stride = v.strides[1];
+  w.v_rows = max_seq;
+  const int64_t orow = (int64_t)split * G;
+  w.att = (_Float16*)att_out.ptr + (int64_t)head * att_out.strides[0] + orow * att_out.strides[1];
+  w.lse = (float*)lse_out.ptr + (int64_t)head * lse_out.strides[0] + orow * lse_out.strides[1];
+  w.att_row_stride = att_out.strides[1], w.lse_row_stride = lse_out.strides[1];
+  w.empty_sum = (float)bn;
+  w.empty_lse = -1.0e30f + __builtin_log2f((float)bn);
+  decode_split_mfma_view<G, D>(w, qk_scale);
+}
+
+// attention_decode_kernel_grouped (cutile-kernels/src/experimental/attention.rs:385-846): the same partial attention in
+// batched layouts.  q [B, kv_heads, GROUP, D]; k, v [B, kv_heads, S, D]; att [B, kv_heads, GROUP, splits, D];
+// lse [B, kv_heads, GROUP, splits]; innermost strides 1, the others given in elements.  Split t takes keys
+// [t * kv_len_per_split, min((t + 1) * kv_len_per_split, *s_kv)) (attention.rs:629-633, with kv_len_per_split a
+// multiple of the key tile); a split without keys writes zeros and lse = -inf (attention.rs:775-780, 806-807).
+// Workgroup (batch, kv head, split) as in the reference's grid (attention.rs:597-601).
+struct GroupedDecodeArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* att;
+  void* lse;
+  const int32_t* s_kv;
+  int32_t q_strides[3], k_strides[3], v_strides[3], att_strides[4], lse_strides[3];
+  int32_t k_rows, v_rows, kv_len_per_split;
+  float softmax_scale;
+};
+
+template <int G, int D>
+__device__ __forceinline__ void decode_grouped(const GroupedDecodeArgs& a, const TileGrid& g) {
+  const int32_t batch = blockIdx.x, head = blockIdx.y, split = blockIdx.z;
+  if (batch >= (int32_t)g.x || head >= (int32_t)g.y || split >= (int32_t)g.z) return;
+  const int32_t s_kv = min(a.s_kv[0], min(a.k_rows, a.v_rows));
+  DecodeSplitView w;
+  w.r0 = split * a.kv_len_per_split;
+  w.r1 = min(w.r0 + a.kv_len_per_split, s_kv);
+  w.q = (const _Float16*)a.q + (int64_t)batch * a.q_strides[0] + (int64_t)head * a.q_strides[1];
+  w.k = (const _Float16*)a.k + (int64_t)batch * a.k_strides[0] + (int64_t)head * a.k_strides[1];
+  w.v = (const _Float16*)a.v + (int64_t)batch * a.v_strides[0] + (int64_t)head * a.v_strides[1];
+  w.q_row_stride = a.q_strides[2], w.k_row_stride = a.k_strides[2], w.v_row_stride = a.v_strides[2];
+  w.v_rows = a.v_rows;
+  w.att = (_Float16*)a.att + (int64_t)batch * a.att_strides[0] + (int64_t)head * a.att_strides[1] + (int64_t)split * a.att_strides[3];
+  w.lse = (float*)a.lse + (int64_t)batch * a.lse_strides[0] + (int64_t)head * a.lse_strides[1] + split;
+  w.att_row_stride = a.att_strides[2], w.lse_row_stride = a.lse_strides[2];
+  w.empty_sum = 1.0f;
+  w.empty_lse = -INFINITY;
+  decode_split_mfma_view<G, D>(w, a.softmax_scale);
 }
 
 // out[h, g, :] = sum_s w[g, s] att[h, s*GROUP + g, :], w = exp2(lse - max_s lse) / max(sum, 1e-8).
@@ -1341,6 +1415,17 @@ DECODE_SPLIT_MFMA_KERNEL(8, 256)
 DECODE_SPLIT_MFMA_KERNEL(16, 64)
 DECODE_SPLIT_MFMA_KERNEL(16, 128)
 DECODE_SPLIT_MFMA_KERNEL(16, 256)
+
+#define DECODE_GROUPED_KERNEL(G, D)                                                                \
+  extern "C" __global__ void __launch_bounds__(256)                                               \
+      attention_decode_grouped_entry__f16_g##G##_d##D(GroupedDecodeArgs a, TileGrid g) {           \
+    decode_grouped<G, D>(a, g);                                                                   \
+  }
+#define DECODE_GROUPED_GROUPS(D) \
+  DECODE_GROUPED_KERNEL(1, D) DECODE_GROUPED_KERNEL(2, D) DECODE_GROUPED_KERNEL(4, D) DECODE_GROUPED_KERNEL(8, D) DECODE_GROUPED_KERNEL(16, D)
+DECODE_GROUPED_GROUPS(64)
+DECODE_GROUPED_GROUPS(128)
+DECODE_GROUPED_GROUPS(256)
 
 // splitk_reduce_merge<GROUP, D, CHUNK_D, NUM_KV_SPLITS, ..>(att_partial, lse_partial, out: [1,GROUP,CHUNK_D] tiles)
 extern "C" __global__ void __launch_bounds__(256)

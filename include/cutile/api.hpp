@@ -608,6 +608,8 @@ template <class A, class L, class O> auto splitk_reduce_merge(A&& att_partial, L
 // qk_norm_rope_kv_prefill_raw_f16 / qk_norm_rope_kv_decode_raw_f16 take raw device pointers (fused_transformer.rs:22-47,
 // 356-372): call cutile_launch_qk_norm_rope_kv_prefill_raw_f16 / ..._decode_raw_f16 of the C ABI with
 // tensor.device_ptr() values; there is no tensor argument to hand back, so they have no launcher object here.
+// attention_decode_kernel_grouped (experimental/attention.rs:385-846) likewise: raw pointers with shape and stride
+// arrays, cutile_launch_attention_decode_kernel_grouped_f16 of the C ABI.
 // group_gemm_f16_nt_desc(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups); needs .grid({NUM_SM, 1, 1}) or the NUM_SM generic   cutile-kernels/src/experimental/moe.rs:73-81
 template <class AP, class BP, class CP, class AM, class BM_, class CM> auto group_gemm_f16_nt_desc(AP&& a_ptrs, BP&& b_ptrs, CP&& c_ptrs, AM&& a_metas, BM_&& b_metas, CM&& c_metas, int32_t num_groups) { return make_launcher<kernels::GroupGemmF16NtDescFn>(std::forward<AP>(a_ptrs), std::forward<BP>(b_ptrs), std::forward<CP>(c_ptrs), std::forward<AM>(a_metas), std::forward<BM_>(b_metas), std::forward<CM>(c_metas), num_groups); }
 // argmax_blocks_f16(logits, block_max: [1], block_idx: [1], len)                  cutile-kernels/src/argmax.rs:21-26

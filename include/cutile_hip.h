@@ -421,6 +421,24 @@ cutile_status_t cutile_launch_fmha_decode_gqa_split(cutile_stream_t stream, cons
                                                     const cutile_partition_arg_t* lse_out, float qk_scale,
                                                     const cutile_tensor_arg_t* position_start,
                                                     const cutile_launch_opts_t* opts);
+/* attention_decode_kernel_grouped<E, HEAD_DIM, TILE_N, KV_LEN_PER_SPLIT, NUM_Q_HEAD_PER_KV, QUERY_GROUP_TILE_SIZE,
+ * NUM_KV_SPLITS>(q_ptr, q_s0..3, q_str0..2, k_ptr, .., v_ptr, .., att_ptr, att_s0..4, att_str0..3, lse_ptr, lse_s0..3,
+ * lse_str0..2, softmax_scale, s_kv_ptr) — cutile-kernels/src/experimental/attention.rs:385-846: the split-KV decode
+ * partial on raw pointers, f16.  Each (pointer, shape scalars, stride scalars) group of the reference arrives as a
+ * pointer and two arrays; strides are in elements and the innermost one (always 1) is not passed.
+ *   q [B, H_kv, G, D]   k, v [B, H_kv, S, D]   att [B, H_kv, G, NUM_KV_SPLITS, D]   lse [B, H_kv, G, NUM_KV_SPLITS] f32
+ * Split t covers keys [t * KV_LEN_PER_SPLIT, min((t + 1) * KV_LEN_PER_SPLIT, *s_kv)); *s_kv is one i32 in device memory
+ * (keys in the cache, at most S).  A split without keys writes zeros and lse = -inf.  lse is in the log2 domain:
+ * max + log2(sum) of softmax_scale * log2(e) * scores.  Launch grid (B, H_kv, NUM_KV_SPLITS) as in the reference.
+ * KV_LEN_PER_SPLIT must be a multiple of TILE_N (otherwise the reference's splits overlap: no variant is built for
+ * that).  Generics, when given, are checked in the order HEAD_DIM, TILE_N, KV_LEN_PER_SPLIT, NUM_Q_HEAD_PER_KV,
+ * QUERY_GROUP_TILE_SIZE, NUM_KV_SPLITS. */
+cutile_status_t cutile_launch_attention_decode_kernel_grouped_f16(
+    cutile_stream_t stream, const void* q, const int32_t* q_shape /*4*/, const int32_t* q_strides /*3*/, const void* k,
+    const int32_t* k_shape /*4*/, const int32_t* k_strides /*3*/, const void* v, const int32_t* v_shape /*4*/,
+    const int32_t* v_strides /*3*/, void* att, const int32_t* att_shape /*5*/, const int32_t* att_strides /*4*/, void* lse,
+    const int32_t* lse_shape /*4*/, const int32_t* lse_strides /*3*/, float softmax_scale, const void* s_kv, int32_t tile_n,
+    int32_t kv_len_per_split, int32_t query_group_tile_size, const cutile_launch_opts_t* opts);
 /* splitk_reduce_merge<GROUP, D, CHUNK_D, NUM_KV_SPLITS>(att_partial, lse_partial, out: [1,GROUP,CHUNK_D] tiles):
  * softmax-weighted sum of the splits — cutile-kernels/src/attention.rs:917-1013 */
 cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const cutile_tensor_arg_t* att_partial,

@@ -67,6 +67,7 @@ def lib() -> C.CDLL:
             "orc_rope_seq_f16": (None, [vp, vp, vp, i64, i64, i64, C.c_int32]),
             "orc_kv_cache_update_f16": (None, [vp, vp, vp, vp, i64, i64, i64, i64, i64]),
             "orc_fmha_decode_gqa_split": (None, [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, f32, i64]),
+            "orc_attention_decode_grouped_f16": (None, [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, i64]),
             "orc_splitk_reduce_merge": (None, [vp, vp, vp, i64, i64, i64, i64]),
             "orc_softmax_f32": (None, [vp, vp, i64, i64, i64, i64]),
             "orc_softmax_f16": (None, [vp, vp, i64, i64, i64, i64]),
@@ -268,6 +269,19 @@ def fmha_decode_gqa_split(q_bits, k_bits, v_bits, qk_scale: float, input_pos: in
     lse = np.empty((kv_heads, splits * group), np.float32)
     lib().orc_fmha_decode_gqa_split(_p(q), _p(k), _p(v), _p(att), _p(lse), kv_heads, group, d, max_seq, bn, splits,
                                     qk_scale, input_pos)
+    return att, lse
+
+
+def attention_decode_grouped_f16(q_bits, k_bits, v_bits, softmax_scale: float, s_kv: int, tile_n: int, kv_len_per_split: int,
+                                 splits: int):
+    """experimental/attention.rs:385-846 -> (att [b, h, g, splits, d] f16 bits, lse [b, h, g, splits] f32)"""
+    q, k, v = _c(q_bits, np.uint16), _c(k_bits, np.uint16), _c(v_bits, np.uint16)
+    batch, heads, group, d = q.shape
+    s_max = k.shape[2]
+    att = np.empty((batch, heads, group, splits, d), np.uint16)
+    lse = np.empty((batch, heads, group, splits), np.float32)
+    lib().orc_attention_decode_grouped_f16(_p(q), _p(k), _p(v), _p(att), _p(lse), batch, heads, group, d, s_max, splits,
+                                           tile_n, kv_len_per_split, softmax_scale, s_kv)
     return att, lse
 
 

@@ -431,6 +431,77 @@ void orc_fmha_decode_gqa_split(const uint16_t* q, const uint16_t* k, const uint1
     }
 }
 
+/* cutile-kernels/src/experimental/attention.rs:385-846 attention_decode_kernel_grouped, contiguous tensors:
+ * q [b, h, g, d]; k, v [b, h, s_max, d]; att [b, h, g, splits, d]; lse [b, h, g, splits].
+ * Split t: start = t * kv_len_per_split, end = min(start + kv_len_per_split, s_kv) (629-633); without keys it
+ * yields acc = 0, l = 1 per lane, m = -inf (775-780).  Otherwise cdiv(kv_len_per_split, tile_n) tiles from tile
+ * start / tile_n on (638-641, 685-687): qk = K . Q^T (703), rows at or beyond s_kv replaced by -1e6 when the tile
+ * crosses s_kv (705-725), scaled by softmax_scale * 1.44269502 (603-606, 729-730), online softmax in base 2 with
+ * l kept per (row of the tile, head) (732-760), acc *= alpha, acc += V^T . f16(p) (762-769); then
+ * att = f16(acc / sum_rows l), lse = m + log2(sum l) (786-807).  Tile rows beyond s_max read as zeros. */
+void orc_attention_decode_grouped_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* att, float* lse,
+                                      int64_t batch, int64_t heads, int64_t group, int64_t d, int64_t s_max,
+                                      int64_t splits, int64_t tile_n, int64_t kv_len_per_split, float softmax_scale,
+                                      int64_t s_kv) {
+  const float qk_scale = softmax_scale * 1.44269502f;
+  const int64_t num_tiles = (kv_len_per_split + tile_n - 1) / tile_n;
+#pragma omp parallel for collapse(3) schedule(static)
+  for (int64_t b = 0; b < batch; b++)
+    for (int64_t h = 0; h < heads; h++)
+      for (int64_t sp = 0; sp < splits; sp++) {
+        const int64_t bh = b * heads + h;
+        const int64_t start = sp * kv_len_per_split;
+        const int64_t end = start + kv_len_per_split < s_kv ? start + kv_len_per_split : s_kv;
+        float* m = (float*)malloc(sizeof(float) * (size_t)group);
+        float* l = (float*)malloc(sizeof(float) * (size_t)(tile_n * group));
+        float* acc = (float*)calloc((size_t)(d * group), sizeof(float));
+        float* qk = (float*)malloc(sizeof(float) * (size_t)(tile_n * group));
+        for (int64_t g = 0; g < group; g++) m[g] = -INFINITY;
+        for (int64_t i = 0; i < tile_n * group; i++) l[i] = 1.0f;
+        if (end > start) {
+          const int64_t start_tile = start / tile_n;
+          for (int64_t idx = 0; idx < num_tiles; idx++) {
+            const int64_t curr_n = (start_tile + idx) * tile_n;
+            const int boundary = curr_n + tile_n > s_kv;
+            for (int64_t n = 0; n < tile_n; n++) {
+              const int64_t row = curr_n + n;
+              for (int64_t g = 0; g < group; g++) {
+                float a = 0.0f;
+                if (row < s_max)
+                  for (int64_t c = 0; c < d; c++)
+                    a += orc_f16_to_f32(k[(bh * s_max + row) * d + c]) * orc_f16_to_f32(q[(bh * group + g) * d + c]);
+                if (boundary && !(row < s_kv)) a = -1000000.0f;
+                qk[n * group + g] = a * qk_scale;
+              }
+            }
+            for (int64_t g = 0; g < group; g++) {
+              float mx = -INFINITY;
+              for (int64_t n = 0; n < tile_n; n++) mx = fmaxf(mx, qk[n * group + g]);
+              const float m_new = fmaxf(m[g], mx);
+              const float alpha = exp2f(m[g] - m_new);
+              for (int64_t c = 0; c < d; c++) acc[c * group + g] *= alpha;
+              for (int64_t n = 0; n < tile_n; n++) {
+                const float p = exp2f(qk[n * group + g] - m_new);
+                l[n * group + g] = fmaf(l[n * group + g], alpha, p);
+                const float ph = orc_f16_to_f32(orc_f32_to_f16(p));
+                const int64_t row = curr_n + n;
+                if (row < s_max && ph != 0.0f)
+                  for (int64_t c = 0; c < d; c++) acc[c * group + g] += orc_f16_to_f32(v[(bh * s_max + row) * d + c]) * ph;
+              }
+              m[g] = m_new;
+            }
+          }
+        }
+        for (int64_t g = 0; g < group; g++) {
+          float ls = 0.0f;
+          for (int64_t n = 0; n < tile_n; n++) ls += l[n * group + g];
+          for (int64_t c = 0; c < d; c++) att[(((bh * group) + g) * splits + sp) * d + c] = orc_f32_to_f16(acc[c * group + g] / ls);
+          lse[(bh * group + g) * splits + sp] = m[g] + log2f(ls);
+        }
+        free(m); free(l); free(acc); free(qk);
+      }
+}
+
 /* attention.rs:917-1013 splitk_reduce_merge: weights = exp2(lse - max) / max(sum, 1e-8) over
  * the splits; out[h, g, :] = sum_s weights[g, s] * att[h, s, g, :], f16. */
 void orc_splitk_reduce_merge(const uint16_t* att, const float* lse, uint16_t* out, int64_t kv_heads,

@@ -42,6 +42,12 @@
  *                        attention for any number of splits, per-split log-sum-exp,
  *                        merge closed forms, exact-copy checks: parity unpinned by
  *                        reference tests.
+ *   orc_attention_decode_grouped_f16          cutile-kernels/src/experimental/attention.rs:385-846.
+ *                        Only compiled by the reference's tests; pinned per split against
+ *                        float64 softmax attention and log-sum-exp over the split's keys, by the
+ *                        lse-weighted merge against attention over all keys, by poisoned keys
+ *                        beyond s_kv, empty splits and a one-key split: parity unpinned by
+ *                        reference tests.
  *   kvbm_stacked_to_contiguous / kvbm_contiguous_to_stacked (numpy, Python wrapper)
  *                        cutile-kernels/src/experimental/kvbm.rs:112-400: a transpose by the
  *                        reference's index maps; pinned element by element against the layouts'
@@ -172,6 +178,10 @@ void orc_fmha_decode_gqa_split(const uint16_t* q, const uint16_t* k, const uint1
                                uint16_t* att_out, float* lse_out, int64_t kv_heads, int64_t group,
                                int64_t d, int64_t max_seq, int64_t bn, int64_t splits,
                                float qk_scale, int64_t input_pos);
+void orc_attention_decode_grouped_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* att, float* lse,
+                                      int64_t batch, int64_t heads, int64_t group, int64_t d, int64_t s_max,
+                                      int64_t splits, int64_t tile_n, int64_t kv_len_per_split, float softmax_scale,
+                                      int64_t s_kv);
 void orc_splitk_reduce_merge(const uint16_t* att, const float* lse, uint16_t* out, int64_t kv_heads,
                              int64_t group, int64_t d, int64_t splits);
 
