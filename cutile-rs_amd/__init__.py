@@ -154,6 +154,9 @@ def lib() -> C.CDLL:
             "cutile_mapped_partition_index": [P(MappedPartitionArg), C.c_uint32, P(C.c_uint32 * 3), P(C.c_uint32)],
             "cutile_launch_gemm_persistent": [vp, P(MappedPartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
             "cutile_launch_mapped_tile_index": [vp, P(MappedPartitionArg), P(LaunchOpts)],
+            "cutile_mapped_partition_index_within": [P(MappedPartitionArg), P(C.c_int32), C.c_uint32, P(C.c_uint32 * 3),
+                                                     P(C.c_uint32)],
+            "cutile_launch_mapped_tile_index_within": [vp, P(MappedPartitionArg), P(C.c_int32), P(LaunchOpts)],
             "cutile_infer_launch_grid": [P(C.c_uint32 * 3), P(P(PartitionArg)), i32, P(C.c_uint32 * 3)],
             "cutile_compute_spec": [P(TensorArg), P(SpecBits)],
             "cutile_kernel_lookup": [vp, C.c_char_p, P(C.c_char_p), i32, C.c_char_p, P(KernelInfo)],
@@ -502,6 +505,31 @@ def gemm_persistent(z: MappedPartition, x, y, *, stream=None, grid=None, generic
     o, _k = _opts(grid, generics, variant)
     xa, ya = tensor_arg(x), tensor_arg(y)
     check(lib().cutile_launch_gemm_persistent(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), C.byref(o)))
+
+
+def _ranges(z: MappedPartition, ranges):
+    flat = [int(v) for pair in ranges for v in pair]
+    if len(flat) != 2 * len(z.map_shape):
+        raise ValueError(f"sub-range iteration expects {len(z.map_shape)} (start_tile, num_tiles) pairs, got {len(ranges)}")
+    return (C.c_int32 * len(flat))(*flat)
+
+
+def mapped_indices_within(z: MappedPartition, ranges):
+    """the block ids of ``for index in z.iter_indices_within(ranges)`` in stream order (cutile/src/_core.rs:912-930)"""
+    r, n, idx = _ranges(z, ranges), C.c_uint32(0), (C.c_uint32 * 3)()
+    check(lib().cutile_mapped_partition_index_within(C.byref(z.arg()), r, 0, None, C.byref(n)))
+    out = []
+    for t in range(n.value):
+        check(lib().cutile_mapped_partition_index_within(C.byref(z.arg()), r, t, idx, None))
+        out.append(tuple(idx)[:len(z.map_shape)])
+    return out
+
+
+def mapped_tile_index_within(z: MappedPartition, ranges, *, stream=None, grid=None) -> None:
+    """only the tiles inside ``ranges`` receive their row-major index in the whole logical grid
+    (cutile/tests/gpu/mapped_partition_schedule_matrix.rs:75-106)"""
+    o, _k = _opts(grid, None, None)
+    check(lib().cutile_launch_mapped_tile_index_within(_stream(stream), C.byref(z.arg()), _ranges(z, ranges), C.byref(o)))
 
 
 def mapped_tile_index(z: MappedPartition, *, stream=None, grid=None) -> None:

@@ -196,6 +196,9 @@ std::vector<KernelEntry> build_table() {
   for (int r = 1; r <= 3; ++r)
     add("mapped_tile_index", keep("i32_r" + std::to_string(r)), keep("mapped_tile_index_entry__i32_r" + std::to_string(r)),
         IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "i32", 0, r);
+  for (int r = 1; r <= 3; ++r)
+    add("mapped_tile_index_within", keep("i32_r" + std::to_string(r)),
+        keep("mapped_tile_index_within_entry__i32_r" + std::to_string(r)), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "i32", 0, r);
 
   // ---- FMHA: LDS = 2 stages x (K tile + V tile) ----
   // "_pp": the two wavefronts of a SIMD run half a tile apart (BM = 256 only)

@@ -21,6 +21,7 @@
 #include "../kernels/mapped_partition.h"
 
 using cutile::MappedArg;
+using cutile::MappedRangeArg;
 using cutile::mapped_index;
 
 using namespace cutile;
@@ -1607,6 +1608,51 @@ cutile_status_t cutile_mapped_partition_index(const cutile_mapped_partition_arg_
   return CUTILE_SUCCESS;
 }
 
+// iter_indices_within: the (start_tile, num_tiles) pair of every axis checked against the grid as the reference's
+// compile-time and run-time asserts do (cutile-compiler/src/compiler/compile_expression.rs:1403-1560), then the
+// record of the narrowed schedule: lengths in m->grid, starts and the whole grid in *range.
+static cutile_status_t mapped_subrange(const cutile_mapped_partition_arg_t* p, const int32_t* ranges, MappedArg* m,
+                                       MappedRangeArg* range, uint32_t grid[3]) {
+  CUTILE_REQUIRE(ranges, CUTILE_ERR_INVALID_ARGUMENT, "ranges is null");
+  if (cutile_status_t s = mapped_record(p, m, grid)) return s;
+  uint64_t total = 1;
+  for (int a = 0; a < 3; ++a) {
+    range->start[a] = 0;
+    range->full_grid[a] = m->grid[a];
+  }
+  for (int a = 0; a < m->rank; ++a) {
+    CUTILE_REQUIRE(m->map[a] != CUTILE_MAP_OWNED, CUTILE_ERR_TENSOR,
+                   "sub-range iteration over a map with OWNED axes is not supported yet");
+    const int32_t start = ranges[2 * a], len = ranges[2 * a + 1];
+    CUTILE_REQUIRE(start >= 0, CUTILE_ERR_TENSOR, "sub-range axis %d start %d is negative", a, start);
+    CUTILE_REQUIRE(len >= -1, CUTILE_ERR_TENSOR, "sub-range axis %d length %d is negative (-1 means the rest of the axis)", a, len);
+    CUTILE_REQUIRE((uint32_t)start <= m->grid[a], CUTILE_ERR_TENSOR, "sub-range axis %d start %d exceeds the %u tiles of the axis", a,
+                   start, m->grid[a]);
+    const uint32_t n = len == -1 ? m->grid[a] - (uint32_t)start : (uint32_t)len;
+    CUTILE_REQUIRE((uint64_t)start + n <= m->grid[a], CUTILE_ERR_TENSOR,
+                   "sub-range axis %d (start %d, %u tiles) exceeds the %u tiles of the axis", a, start, n, m->grid[a]);
+    range->start[a] = start;
+    m->grid[a] = n;
+    total *= n;
+  }
+  m->total = (uint32_t)total;
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_mapped_partition_index_within(const cutile_mapped_partition_arg_t* p, const int32_t* ranges, uint32_t item,
+                                                     uint32_t index[3], uint32_t* n_items) {
+  MappedArg m;
+  MappedRangeArg range;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_subrange(p, ranges, &m, &range, grid)) return s;
+  if (n_items) *n_items = m.total;
+  if (!index) return CUTILE_SUCCESS;                     // the count alone (an empty range has no item to ask for)
+  CUTILE_REQUIRE(item < m.total, CUTILE_ERR_INVALID_ARGUMENT, "stream item %u is outside the %u items of the sub-range", item, m.total);
+  mapped_index(m, item, index);
+  for (int a = 0; a < 3; ++a) index[a] += (uint32_t)range.start[a];
+  return CUTILE_SUCCESS;
+}
+
 // The launch grid of a mapped kernel: (num_tile_blocks, 1, 1); an explicit .grid() is a checked override.
 static cutile_status_t mapped_launch_grid(const cutile_mapped_partition_arg_t* z, const cutile_launch_opts_t* opts, MappedArg* m,
                                           uint32_t grid[3]) {
@@ -1737,6 +1783,27 @@ cutile_status_t cutile_launch_mapped_tile_index(cutile_stream_t stream, const cu
   ArgPacker args;
   args.push_partition(*z);
   args.push_val<MappedArg>(m);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+cutile_status_t cutile_launch_mapped_tile_index_within(cutile_stream_t stream, const cutile_mapped_partition_arg_t* zm,
+                                                       const int32_t* ranges, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(zm, CUTILE_ERR_INVALID_ARGUMENT, "z is null");
+  const cutile_partition_arg_t* z = &zm->partition;
+  if (cutile_status_t s = check_partition(z, "z", 1, 3)) return s;
+  CUTILE_REQUIRE(z->tensor.dtype == CUTILE_DTYPE_I32, CUTILE_ERR_KERNEL_NOT_FOUND, "mapped_tile_index_within: z must be i32");
+  MappedArg full, m;
+  MappedRangeArg range;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_launch_grid(zm, opts, &full, grid)) return s;
+  if (cutile_status_t s = mapped_subrange(zm, ranges, &m, &range, grid)) return s;
+  const std::string want = "i32_r" + std::to_string(z->tensor.rank);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("mapped_tile_index_within", opts, want, {want}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_val<MappedArg>(m);
+  args.push_val<MappedRangeArg>(range);
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 

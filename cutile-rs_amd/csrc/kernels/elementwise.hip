@@ -486,16 +486,18 @@ CONVERT_FROM(int64_t, i64)
 // the caller's fill, a duplicated one overwrites a neighbour.  Same kernel here, for
 // i32 tensors of rank 1 to 3: workgroup b takes stream items b, b + gridDim.x, ...;
 // an OWNED axis is walked in full by the workgroup that owns the item.
+// With a sub-range (write_flat_index_subrange, the same file :75-106) the schedule runs over the range's lengths,
+// the starts are added, and the index stored is the one in the whole grid.
 template <int R>
-__device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, const MappedArg& m) {
+__device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, const MappedArg& m, const MappedRangeArg& range) {
   int32_t* zp = (int32_t*)z.ptr;
   for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
     uint32_t bid[3];
     mapped_index(m, item, bid);
     uint32_t lo[3] = {0, 0, 0}, hi[3] = {1, 1, 1};
     for (int a = 0; a < R; ++a) {
-      lo[a] = m.map[a] == kOwnedAxis ? 0 : bid[a];
-      hi[a] = m.map[a] == kOwnedAxis ? m.grid[a] : bid[a] + 1;
+      lo[a] = m.map[a] == kOwnedAxis ? 0 : bid[a] + (uint32_t)range.start[a];
+      hi[a] = m.map[a] == kOwnedAxis ? m.grid[a] : lo[a] + 1;
     }
     for (uint32_t c0 = lo[0]; c0 < hi[0]; ++c0)
       for (uint32_t c1 = lo[1]; c1 < hi[1]; ++c1)
@@ -504,7 +506,7 @@ __device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, cons
           int32_t flat = 0;
           int64_t count = 1;
           for (int a = 0; a < R; ++a) {
-            flat = flat * (int32_t)m.grid[a] + (int32_t)c[a];
+            flat = flat * (int32_t)range.full_grid[a] + (int32_t)c[a];
             count *= z.pshape[a];
           }
           for (int64_t e = threadIdx.x; e < count; e += kThreads) {
@@ -525,7 +527,12 @@ __device__ __forceinline__ void mapped_tile_index(const PartitionArg<R>& z, cons
 #define MAPPED_TILE_INDEX_KERNEL(R)                                                                \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \
       mapped_tile_index_entry__i32_r##R(PartitionArg<R> z, MappedArg m) {                          \
-    mapped_tile_index<R>(z, m);                                                                    \
+    const MappedRangeArg whole = {{0, 0, 0}, {m.grid[0], m.grid[1], m.grid[2]}};                   \
+    mapped_tile_index<R>(z, m, whole);                                                             \
+  }                                                                                                \
+  extern "C" __global__ void __launch_bounds__(kThreads)                                           \
+      mapped_tile_index_within_entry__i32_r##R(PartitionArg<R> z, MappedArg m, MappedRangeArg range) { \
+    mapped_tile_index<R>(z, m, range);                                                             \
   }
 MAPPED_TILE_INDEX_KERNEL(1)
 MAPPED_TILE_INDEX_KERNEL(2)

@@ -41,6 +41,14 @@ struct MappedArg {
 };
 static_assert(sizeof(MappedArg) == 32, "mapped records must stay a flat i32 sequence");
 
+// A sub-range of the logical grid (`iter_indices_within`, cutile/src/_core.rs:912-930; lowering in
+// cutile-compiler/src/compiler/compile_expression.rs:1403-1420): the schedule runs over the per-axis lengths
+// (MappedArg::grid holds them) and the axis starts are added to the block ids it yields.
+struct MappedRangeArg {
+  int32_t start[3];        // first tile per axis
+  uint32_t full_grid[3];   // the partition's whole logical grid
+};
+
 CUTILE_SCHED_FN void swizzle_2d(uint32_t t, uint32_t num_m, uint32_t num_n, uint32_t gm, uint32_t gn, uint32_t* bid_m,
                                 uint32_t* bid_n) {
   if (gm == 1 && gn == 1) {

@@ -474,6 +474,24 @@ class MappedLaunchPartition {
     CUTILE_TRY_STATUS(cutile_mapped_partition_index(&m, item, idx.data(), nullptr));
     return idx;
   }
+  // the block ids of `for index in z.iter_indices_within(ranges)` in stream order (cutile/src/_core.rs:912-930):
+  // one (start_tile, num_tiles) pair per map axis, num_tiles -1 = the rest of the axis
+  Result<std::vector<std::array<uint32_t, 3>>> indices_within(const std::vector<std::pair<int32_t, int32_t>>& ranges) const {
+    if (ranges.size() != map_shape_.size())
+      return DeviceError::tensor("sub-range iteration expects " + std::to_string(map_shape_.size()) +
+                                 " (start_tile, num_tiles) pairs, got " + std::to_string(ranges.size()));
+    std::vector<int32_t> flat;
+    for (auto& r : ranges) {
+      flat.push_back(r.first);
+      flat.push_back(r.second);
+    }
+    cutile_mapped_partition_arg_t m = arg();
+    uint32_t n = 0;
+    CUTILE_TRY_STATUS(cutile_mapped_partition_index_within(&m, flat.data(), 0, nullptr, &n));
+    std::vector<std::array<uint32_t, 3>> out(n);
+    for (uint32_t t = 0; t < n; ++t) CUTILE_TRY_STATUS(cutile_mapped_partition_index_within(&m, flat.data(), t, out[t].data(), nullptr));
+    return out;
+  }
   P into_partition() && { return std::move(partition_); }
 
  private:

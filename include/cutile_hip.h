@@ -310,6 +310,19 @@ cutile_status_t cutile_mapped_partition_grid(const cutile_mapped_partition_arg_t
  * — cutile-compiler/src/compiler/compile_intrinsic.rs:2438-2900 (emit_swizzle_2d, emit_mapped_partition_schedule). */
 cutile_status_t cutile_mapped_partition_index(const cutile_mapped_partition_arg_t* p, uint32_t item, uint32_t index[3],
                                               uint32_t* n_items);
+/* `for index in z.iter_indices_within(ranges)` — cutile/src/_core.rs:912-930: the same schedule over a sub-range of
+ * the logical grid.  `ranges` holds one (start_tile, num_tiles) pair per map axis (2 * map_rank values); num_tiles
+ * -1 is the rest of the axis.  The schedule runs over the lengths and the starts are added to the block ids
+ * (cutile-compiler/src/compiler/compile_expression.rs:1403-1420).  Errors as the reference's checks: negative
+ * start or length, a range beyond the grid, OWNED axes (:1279-1284, :1447-1470).  `index` may be NULL to ask for
+ * the item count alone (an empty range has none). */
+cutile_status_t cutile_mapped_partition_index_within(const cutile_mapped_partition_arg_t* p, const int32_t* ranges,
+                                                     uint32_t item, uint32_t index[3], uint32_t* n_items);
+/* write_flat_index_subrange / write_flat_index_subrange_rest<BM, BN, MAP_SHAPE>(z: MappedPartitionMut<i32>, start_tile,
+ * n_tiles): only the tiles inside the ranges receive their row-major index in the whole logical grid —
+ * cutile/tests/gpu/mapped_partition_schedule_matrix.rs:75-106 (any rank 1..3, a pair per axis as above) */
+cutile_status_t cutile_launch_mapped_tile_index_within(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,
+                                                       const int32_t* ranges, const cutile_launch_opts_t* opts);
 /* gemm_persistent<T, BM, BN, BK, MAP_SHAPE>(z: MappedPartitionMut [BM,BN], x, y): z <- x . y over all of x's K,
  * zero initial accumulator — cutile-examples/examples/persistent_gemm.rs:35-59 */
 cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,

@@ -281,6 +281,13 @@ TEST(mapped_partitions_validate_and_hand_the_inner_partition_back) {
   CHECK(m.index(0).unwrap() == (std::array<uint32_t, 3>{0, 0, 0}) && m.index(1).unwrap() == (std::array<uint32_t, 3>{1, 0, 0}) &&
         m.index(2).unwrap() == (std::array<uint32_t, 3>{0, 1, 0}) && m.index(5).unwrap() == (std::array<uint32_t, 3>{1, 2, 0}));
   CHECK(m.index(6).is_err());
+  // iter_indices_within (cutile/src/_core.rs:912-930): the schedule over the range's lengths, shifted by its starts
+  auto sub = m.indices_within({{0, -1}, {1, 2}}).unwrap();
+  CHECK(sub.size() == 4 && sub[0] == (std::array<uint32_t, 3>{0, 1, 0}) && sub[1] == (std::array<uint32_t, 3>{1, 1, 0}) &&
+        sub[2] == (std::array<uint32_t, 3>{0, 2, 0}) && sub[3] == (std::array<uint32_t, 3>{1, 2, 0}));
+  CHECK(m.indices_within({{1, 0}, {0, -1}}).unwrap().empty());
+  CHECK(m.indices_within({{-1, 2}, {0, -1}}).error().message.find("is negative") != std::string::npos);   // partition_index_schedules.rs:553
+  CHECK(m.indices_within({{0, -1}}).is_err());
   // persistent_gemm.rs:96-108: the launcher takes the mapped partition and returns the partition
   auto x = api::zeros<float>({64, 32}).sync_on(s).unwrap();
   auto y = api::zeros<float>({32, 64}).sync_on(s).unwrap();

@@ -75,7 +75,16 @@ def mapped_partition_cases():
     for mp in ([1, 1, 1], [1, 2, 1], [1, 2, 2], [1, 3, 2]):
         for ntb in (1, 5, 12):
             matrix.append({"dims": [2, 12, 16], "tile": [1, 4, 8], "map_shape": mp, "num_tile_blocks": ntb})
-    return {"validate": validate, "schedule_matrix": {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:219-300",
+    # cutile/tests/gpu/mapped_partition_schedule_matrix.rs:320-369: iter_indices_within([(start, len), (0, -1)]) on a
+    # 64 x 64 tensor in 16 x 16 tiles, 4 tile blocks; rows of tiles [lo, hi) receive their flat index, the rest keep
+    # the poison.
+    sub = lambda mp, start, length, lo, hi: {"map_shape": mp, "start": start, "len": length, "expect_lo": lo, "expect_hi": hi}
+    subrange = {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:320-369", "dims": [64, 64], "tile": [16, 16],
+                "num_tile_blocks": 4, "poison": -0x5EAD,
+                "cases": [sub([1, 1], 1, 0, 0, 0), sub([1, 1], 3, 1, 3, 4), sub([1, 1], 2, -1, 2, 4), sub([1, 1], 0, -1, 0, 4),
+                          sub([2, 1], 1, 2, 1, 3), sub([2, 2], 0, 3, 0, 3)]}
+    return {"validate": validate, "subrange": subrange,
+            "schedule_matrix": {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:219-300",
                                                       "poison": -0x5EAD, "cases": matrix},
             "persistent_gemm_launch": {"cite": "cutile-examples/examples/persistent_gemm.rs:70-79",
                                        "map_shape": [4, 1], "num_tile_blocks": 4}}

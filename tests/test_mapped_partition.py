@@ -98,6 +98,47 @@ def test_host_schedule_equals_the_oracle(ct, grid, mp):
         m.index(len(order))
 
 
+@pytest.mark.parametrize("grid,mp,ranges", [((4, 4), (1, 1), [(1, 2), (0, -1)]), ((4, 4), (2, 1), [(1, 2), (0, -1)]),
+                                            ((4, 4), (2, 2), [(0, 3), (0, -1)]), ((7, 5), (4, 3), [(2, -1), (1, 3)]),
+                                            ((5,), (1,), [(2, 2)]), ((2, 6, 5), (1, 2, 2), [(1, 1), (1, 4), (0, -1)]),
+                                            ((4, 4), (1, 1), [(1, 0), (0, -1)]), ((4, 4), (1, 1), [(4, -1), (0, -1)])])
+def test_subrange_schedule_is_the_schedule_of_the_lengths_shifted_by_the_starts(ct, grid, mp, ranges):
+    """iter_indices_within (cutile/src/_core.rs:912-930): 'the schedule runs over the effective lengths and the axis
+    starts are added to the minted coordinates' (cutile-compiler/src/compiler/compile_expression.rs:1403-1405)"""
+    z, _ = _logical(grid, [2] * len(grid))
+    m = ct.mapped(ct.partition(z, [2] * len(grid)), mp, 1)
+    starts = [s for s, _ in ranges]
+    lens = [g - s if n == -1 else n for g, (s, n) in zip(grid, ranges)]
+    want = [] if 0 in lens else [tuple(c + s for c, s in zip(idx, starts)) for idx in oracle.mapped_schedule(lens, mp)]
+    got = ct.mapped_indices_within(m, ranges)
+    assert got == want
+    assert len(set(got)) == len(got) and all(s <= c < s + n for idx in got for c, s, n in zip(idx, starts, lens))
+    if all(s == 0 for s in starts) and lens == list(grid):
+        assert got == [m.index(t) for t in range(m.num_items())]
+
+
+def test_subrange_over_the_whole_grid_is_the_plain_schedule(ct):
+    z, _ = _logical((5, 3), [2, 2])
+    m = ct.mapped(ct.partition(z, [2, 2]), (2, 2), 3)
+    assert ct.mapped_indices_within(m, [(0, -1), (0, -1)]) == [m.index(t) for t in range(m.num_items())]
+    assert ct.mapped_indices_within(m, [(0, 5), (0, 3)]) == [m.index(t) for t in range(m.num_items())]
+
+
+def test_subrange_rejects_what_the_reference_rejects(ct):
+    z, _ = _logical((4, 4), [2, 2])
+    m = ct.mapped(ct.partition(z, [2, 2]), (1, 1), 2)
+    for ranges, msg in [([(-1, 2), (0, -1)], "start -1 is negative"),                # partition_index_schedules.rs:553
+                        ([(0, -2), (0, -1)], "length -2 is negative"),
+                        ([(3, 2), (0, -1)], "exceeds the 4 tiles"), ([(5, -1), (0, -1)], "exceeds the 4 tiles")]:
+        with pytest.raises(ct.CutileError, match=msg):
+            ct.mapped_indices_within(m, ranges)
+    owned = ct.mapped(ct.partition(z, [2, 2]), (1, 0), 2)
+    with pytest.raises(ct.CutileError, match="OWNED axes is not supported"):         # compile_expression.rs:1279-1284
+        ct.mapped_indices_within(owned, [(0, -1), (0, -1)])
+    with pytest.raises(ValueError, match="expects 2"):
+        ct.mapped_indices_within(m, [(0, -1)])
+
+
 # ---- HIP kernels (GPU) -----------------------------------------------------------------------
 def _expected_flat_index(dims, tile):
     grid = [-(-d // t) for d, t in zip(dims, tile)]
@@ -125,6 +166,33 @@ def test_gpu_schedule_matrix_covers_every_tile_exactly_once(ct, dev):
         torch.cuda.synchronize()
         assert np.array_equal(z.cpu().numpy(), _expected_flat_index(dims, tile)), (dims, tile, mp, ntb)
         assert torch.all(wide[..., dims[-1]:] == m["poison"])
+
+
+@pytest.mark.gpu
+def test_gpu_subrange_writes_exactly_the_range(ct, dev):
+    """the reference's subrange_edge_cases_write_exactly_the_range (mapped_partition_schedule_matrix.rs:354-369), then
+    ranges on both axes, rank 1 and 3 and ragged edges"""
+    sr = CASES["subrange"]
+    whole = _expected_flat_index(sr["dims"], sr["tile"])
+    for c in sr["cases"]:
+        z = torch.full(sr["dims"], sr["poison"], dtype=torch.int32, device=dev)
+        ct.mapped_tile_index_within(ct.mapped(ct.partition(z, sr["tile"]), c["map_shape"], sr["num_tile_blocks"]),
+                                    [(c["start"], c["len"]), (0, -1)])
+        torch.cuda.synchronize()
+        want = np.full(sr["dims"], sr["poison"], np.int32)
+        lo, hi = c["expect_lo"] * sr["tile"][0], c["expect_hi"] * sr["tile"][0]
+        want[lo:hi] = whole[lo:hi]
+        assert np.array_equal(z.cpu().numpy(), want), c
+    for dims, tile, mp, ntb, ranges in [([30, 21], [8, 8], [3, 2], 4, [(1, 2), (1, -1)]), ([37], [8], [1], 2, [(2, 3)]),
+                                        ([3, 10, 9], [1, 4, 4], [1, 2, 2], 7, [(1, -1), (0, 2), (2, 1)])]:
+        z = torch.full(dims, -7, dtype=torch.int32, device=dev)
+        ct.mapped_tile_index_within(ct.mapped(ct.partition(z, tile), mp, ntb), ranges)
+        torch.cuda.synchronize()
+        grid = [-(-d // t) for d, t in zip(dims, tile)]
+        want = np.full(dims, -7, np.int32)
+        box = tuple(slice(s * t, (g if n == -1 else s + n) * t) for (s, n), t, g in zip(ranges, tile, grid))
+        want[box] = _expected_flat_index(dims, tile)[box]
+        assert np.array_equal(z.cpu().numpy(), want), (dims, tile, mp, ranges)
 
 
 @pytest.mark.gpu
