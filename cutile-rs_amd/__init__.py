@@ -157,6 +157,9 @@ def lib() -> C.CDLL:
             "cutile_mapped_partition_index_within": [P(MappedPartitionArg), P(C.c_int32), C.c_uint32, P(C.c_uint32 * 3),
                                                      P(C.c_uint32)],
             "cutile_launch_mapped_tile_index_within": [vp, P(MappedPartitionArg), P(C.c_int32), P(LaunchOpts)],
+            "cutile_mapped_partitions_shared": [P(MappedPartitionArg), P(MappedPartitionArg)],
+            "cutile_launch_mapped_shared_cache_update_f32": [vp, P(MappedPartitionArg), P(MappedPartitionArg), P(TensorArg), i32,
+                                                             P(TensorArg), i32, i32, P(LaunchOpts)],
             "cutile_infer_launch_grid": [P(C.c_uint32 * 3), P(P(PartitionArg)), i32, P(C.c_uint32 * 3)],
             "cutile_compute_spec": [P(TensorArg), P(SpecBits)],
             "cutile_kernel_lookup": [vp, C.c_char_p, P(C.c_char_p), i32, C.c_char_p, P(KernelInfo)],
@@ -530,6 +533,22 @@ def mapped_tile_index_within(z: MappedPartition, ranges, *, stream=None, grid=No
     (cutile/tests/gpu/mapped_partition_schedule_matrix.rs:75-106)"""
     o, _k = _opts(grid, None, None)
     check(lib().cutile_launch_mapped_tile_index_within(_stream(stream), C.byref(z.arg()), _ranges(z, ranges), C.byref(o)))
+
+
+def mapped_partitions_shared(a: MappedPartition, b: MappedPartition) -> None:
+    """the checks of ``a.iter_indices_with(&b)`` (cutile/src/_core.rs:904-911); raises CutileError when they fail"""
+    check(lib().cutile_mapped_partitions_shared(C.byref(a.arg()), C.byref(b.arg())))
+
+
+def mapped_shared_cache_update_f32(k_cache: MappedPartition, v_cache: MappedPartition, new_k, n_tiles: int, *, start_tile: int = 0,
+                                   position=None, source_seq_major: bool = False, stream=None, grid=None) -> None:
+    """dynpos_shared_rank3 / prefill_shared_rank3 of cutile/tests/gpu/mapped_partition_schedule_matrix.rs:107-153"""
+    o, _k = _opts(grid, None, None)
+    na = tensor_arg(new_k)
+    pa = tensor_arg(position) if position is not None else None
+    check(lib().cutile_launch_mapped_shared_cache_update_f32(
+        _stream(stream), C.byref(k_cache.arg()), C.byref(v_cache.arg()), C.byref(na), int(source_seq_major),
+        C.byref(pa) if pa is not None else None, int(start_tile), int(n_tiles), C.byref(o)))
 
 
 def mapped_tile_index(z: MappedPartition, *, stream=None, grid=None) -> None:

@@ -196,6 +196,7 @@ std::vector<KernelEntry> build_table() {
   for (int r = 1; r <= 3; ++r)
     add("mapped_tile_index", keep("i32_r" + std::to_string(r)), keep("mapped_tile_index_entry__i32_r" + std::to_string(r)),
         IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "i32", 0, r);
+  add("mapped_shared_cache_update", "f32", "mapped_shared_cache_update_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 3);
   for (int r = 1; r <= 3; ++r)
     add("mapped_tile_index_within", keep("i32_r" + std::to_string(r)),
         keep("mapped_tile_index_within_entry__i32_r" + std::to_string(r)), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "i32", 0, r);

@@ -1807,6 +1807,66 @@ cutile_status_t cutile_launch_mapped_tile_index_within(cutile_stream_t stream, c
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// iter_indices_with: the type gives both partitions one tile and map shape; their logical grids must match too
+// (cutile-compiler/src/compiler/compile_expression.rs:1318-1397).
+cutile_status_t cutile_mapped_partitions_shared(const cutile_mapped_partition_arg_t* a, const cutile_mapped_partition_arg_t* b) {
+  CUTILE_REQUIRE(a && b, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  uint32_t ga[3], gb[3], launch[3];
+  if (cutile_status_t s = mapped_record(a, nullptr, launch)) return s;
+  if (cutile_status_t s = mapped_record(b, nullptr, launch)) return s;
+  bool same = a->map_rank == b->map_rank && a->partition.tensor.rank == b->partition.tensor.rank;
+  for (int i = 0; same && i < a->map_rank; ++i) same = a->map_shape[i] == b->map_shape[i];
+  for (int i = 0; same && i < a->partition.tensor.rank; ++i) same = a->partition.partition_shape[i] == b->partition.partition_shape[i];
+  CUTILE_REQUIRE(same, CUTILE_ERR_TENSOR, "iter_indices_with requires both mapped partitions to share tile and map shapes");
+  if (cutile_status_t s = cutile_partition_grid(&a->partition, ga)) return s;
+  if (cutile_status_t s = cutile_partition_grid(&b->partition, gb)) return s;
+  for (int i = 0; i < 3; ++i)
+    CUTILE_REQUIRE(ga[i] == gb[i], CUTILE_ERR_TENSOR,
+                   "shared mapped partitions require equal logical partition grids: axis %d has %u vs %u tiles", i, ga[i], gb[i]);
+  CUTILE_REQUIRE(a->num_tile_blocks == b->num_tile_blocks, CUTILE_ERR_TENSOR,
+                 "shared mapped partitions disagree on num_tile_blocks (%u vs %u)", a->num_tile_blocks, b->num_tile_blocks);
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_launch_mapped_shared_cache_update_f32(cutile_stream_t stream, const cutile_mapped_partition_arg_t* k_cache,
+                                                             const cutile_mapped_partition_arg_t* v_cache,
+                                                             const cutile_tensor_arg_t* new_k, int32_t source_seq_major,
+                                                             const cutile_tensor_arg_t* position, int32_t start_tile,
+                                                             int32_t n_tiles, const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(k_cache && v_cache, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  if (cutile_status_t s = check_partition(&k_cache->partition, "k_cache", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(&v_cache->partition, "v_cache", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(new_k, "new_k", 3, 3)) return s;
+  CUTILE_REQUIRE(k_cache->partition.tensor.dtype == CUTILE_DTYPE_F32 && v_cache->partition.tensor.dtype == CUTILE_DTYPE_F32 &&
+                     new_k->dtype == CUTILE_DTYPE_F32,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "mapped_shared_cache_update: k_cache, v_cache and new_k must be f32");
+  if (position) {
+    if (cutile_status_t s = check_tensor(position, "position", 1, 1)) return s;
+    CUTILE_REQUIRE(position->dtype == CUTILE_DTYPE_I32 && position->shape[0] == 1 && ((uintptr_t)position->ptr & 3) == 0,
+                   CUTILE_ERR_KERNEL_LAUNCH, "mapped_shared_cache_update: position must be one i32 in device memory");
+  }
+  if (cutile_status_t s = cutile_mapped_partitions_shared(k_cache, v_cache)) return s;
+  MappedArg full, m;
+  MappedRangeArg range;
+  uint32_t grid[3];
+  if (cutile_status_t s = mapped_launch_grid(k_cache, opts, &full, grid)) return s;
+  // a start read on the device is checked there; its length must fit the axis in any case
+  const int32_t ranges[6] = {0, -1, position ? 0 : start_tile, n_tiles, 0, -1};
+  CUTILE_REQUIRE(n_tiles >= 0, CUTILE_ERR_TENSOR, "sub-range axis 1 length %d is negative", n_tiles);
+  if (cutile_status_t s = mapped_subrange(k_cache, ranges, &m, &range, grid)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("mapped_shared_cache_update", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(k_cache->partition);
+  args.push_partition(v_cache->partition);
+  args.push_tensor(*new_k);
+  args.push_val<MappedArg>(m);
+  args.push_val<MappedRangeArg>(range);
+  args.push_val<const void*>(position ? position->ptr : nullptr);
+  args.push_val<int32_t>(source_seq_major ? 1 : 0);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partition_arg_t* out, const cutile_tensor_arg_t* q,
                                    const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v, float qk_scale,
                                    int32_t input_pos, int32_t query_group_size, int32_t causal,

@@ -538,6 +538,49 @@ MAPPED_TILE_INDEX_KERNEL(1)
 MAPPED_TILE_INDEX_KERNEL(2)
 MAPPED_TILE_INDEX_KERNEL(3)
 
+// Two mapped outputs sharing one index stream (`iter_indices_within_with`, cutile/src/_core.rs:932-941): the
+// reference's dynpos_shared_rank3 / prefill_shared_rank3 kernels
+// (cutile/tests/gpu/mapped_partition_schedule_matrix.rs:107-153).  k_cache and v_cache are [heads, max_seq, d] in
+// tiles [B0, B1, B2]; the stream covers ranges [(0, -1), (start, n_tiles), (0, -1)], start by value or read from
+// device memory; tile (h, s, c) of the source is taken at (h, s - start, c) for a [heads, seq, d] source and at
+// (s - start, h, c) for a [seq, heads, d] one (out of range reads as zero), stored to k_cache and doubled to v_cache.
+// A start that does not fit the grid writes nothing (the reference's range assert stops its kernel).
+extern "C" __global__ void __launch_bounds__(kThreads)
+    mapped_shared_cache_update_entry__f32(PartitionArg<3> k_cache, PartitionArg<3> v_cache, TensorArg<3> new_k, MappedArg m,
+                                          MappedRangeArg range, const int32_t* pos_dev, int32_t seq_major) {
+  const int32_t start = pos_dev ? pos_dev[0] : range.start[1];
+  if (start < 0 || (uint32_t)start + m.grid[1] > range.full_grid[1]) return;
+  float* kp = (float*)k_cache.ptr;
+  float* vp = (float*)v_cache.ptr;
+  const float* sp = (const float*)new_k.ptr;
+  const int64_t count = (int64_t)k_cache.pshape[0] * k_cache.pshape[1] * k_cache.pshape[2];
+  for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
+    uint32_t bid[3];
+    mapped_index(m, item, bid);
+    const int64_t dst_tile[3] = {(int64_t)bid[0] + range.start[0], (int64_t)bid[1] + start, (int64_t)bid[2] + range.start[2]};
+    const int64_t src_tile[3] = {seq_major ? (int64_t)bid[1] : dst_tile[0], seq_major ? dst_tile[0] : (int64_t)bid[1], dst_tile[2]};
+    for (int64_t e = threadIdx.x; e < count; e += kThreads) {
+      int64_t rest = e, k_off = 0, v_off = 0, s_off = 0;
+      bool dst_inside = true, src_inside = true;
+      for (int a = 2; a >= 0; --a) {
+        const int64_t in_tile = rest % k_cache.pshape[a];
+        rest /= k_cache.pshape[a];
+        const int64_t di = dst_tile[a] * k_cache.pshape[a] + in_tile, si = src_tile[a] * k_cache.pshape[a] + in_tile;
+        dst_inside &= di < k_cache.shape[a] && di < v_cache.shape[a];
+        src_inside &= si < new_k.shape[a];
+        k_off += di * k_cache.strides[a];
+        v_off += di * v_cache.strides[a];
+        s_off += si * new_k.strides[a];
+      }
+      if (dst_inside) {
+        const float x = src_inside ? sp[s_off] : 0.0f;
+        kp[k_off] = x;
+        vp[v_off] = x + x;
+      }
+    }
+  }
+}
+
 // ---- greedy sampling and row gathers ---------------------------------------------------------
 // argmax_blocks_f16 / lm_head_argmax_blocks_f16 / argmax_reduce_blocks_to_u32
 // (cutile-kernels/src/argmax.rs:21-71, 88-158, 173-213), embedding_batch_f16

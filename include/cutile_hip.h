@@ -323,6 +323,21 @@ cutile_status_t cutile_mapped_partition_index_within(const cutile_mapped_partiti
  * cutile/tests/gpu/mapped_partition_schedule_matrix.rs:75-106 (any rank 1..3, a pair per axis as above) */
 cutile_status_t cutile_launch_mapped_tile_index_within(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,
                                                        const int32_t* ranges, const cutile_launch_opts_t* opts);
+/* `a.iter_indices_with(&b)` — cutile/src/_core.rs:904-911: two mapped outputs written at the same indices must share
+ * tile shape, map shape and logical grid (cutile-compiler/src/compiler/compile_expression.rs:1318-1397: "iter_indices_with
+ * requires both mapped partitions to share tile and map shapes", "shared mapped partitions require equal logical
+ * partition grids: axis N"). */
+cutile_status_t cutile_mapped_partitions_shared(const cutile_mapped_partition_arg_t* a, const cutile_mapped_partition_arg_t* b);
+/* dynpos_shared_rank3 / prefill_shared_rank3<BS, BD, MAP_SHAPE>(k_cache, v_cache: MappedPartitionMut<f32, [1,BS,BD]>, new_k,
+ * pos | seq_len, n_tiles) — cutile/tests/gpu/mapped_partition_schedule_matrix.rs:107-153: one stream over
+ * [(0,-1), (start, n_tiles), (0,-1)] of two caches [heads, max_seq, d]; cache tile (h, s, c) <- source tile
+ * (h, s - start, c) of a [heads, seq, d] source (source_seq_major 0) or (s - start, h, c) of a [seq, heads, d] one (1);
+ * v_cache receives twice the value.  `position` (one i32 in device memory) replaces start_tile when given. */
+cutile_status_t cutile_launch_mapped_shared_cache_update_f32(cutile_stream_t stream, const cutile_mapped_partition_arg_t* k_cache,
+                                                             const cutile_mapped_partition_arg_t* v_cache,
+                                                             const cutile_tensor_arg_t* new_k, int32_t source_seq_major,
+                                                             const cutile_tensor_arg_t* position, int32_t start_tile,
+                                                             int32_t n_tiles, const cutile_launch_opts_t* opts);
 /* gemm_persistent<T, BM, BN, BK, MAP_SHAPE>(z: MappedPartitionMut [BM,BN], x, y): z <- x . y over all of x's K,
  * zero initial accumulator — cutile-examples/examples/persistent_gemm.rs:35-59 */
 cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cutile_mapped_partition_arg_t* z,

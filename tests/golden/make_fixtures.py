@@ -83,7 +83,12 @@ def mapped_partition_cases():
                 "num_tile_blocks": 4, "poison": -0x5EAD,
                 "cases": [sub([1, 1], 1, 0, 0, 0), sub([1, 1], 3, 1, 3, 4), sub([1, 1], 2, -1, 2, 4), sub([1, 1], 0, -1, 0, 4),
                           sub([2, 1], 1, 2, 1, 3), sub([2, 2], 0, 3, 0, 3)]}
-    return {"validate": validate, "subrange": subrange,
+    # the same file :372-476: two caches [heads, max_seq, d] written through one shared stream over the sequence sub-range
+    shared = {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:372-476", "heads": 2, "max_seq": 8, "d": 16,
+              "tile": [1, 1, 16], "map_shape": [1, 1, 1], "poison": -333.25,
+              "dynpos": {"source_shape": [2, 2, 16], "source_scale": 0.5, "position": 3, "n_tiles": 2, "num_tile_blocks": 4},
+              "prefill": {"source_shape": [2, 2, 16], "source_scale": 0.25, "seq_len": 2, "num_tile_blocks": 4}}
+    return {"validate": validate, "subrange": subrange, "shared_rank3": shared,
             "schedule_matrix": {"cite": "cutile/tests/gpu/mapped_partition_schedule_matrix.rs:219-300",
                                                       "poison": -0x5EAD, "cases": matrix},
             "persistent_gemm_launch": {"cite": "cutile-examples/examples/persistent_gemm.rs:70-79",

@@ -195,6 +195,77 @@ def test_gpu_subrange_writes_exactly_the_range(ct, dev):
         assert np.array_equal(z.cpu().numpy(), want), (dims, tile, mp, ranges)
 
 
+def test_shared_mapped_partitions_need_equal_shapes_and_grids(ct):
+    """iter_indices_with (cutile/src/_core.rs:904-911; cutile-compiler/src/compiler/compile_expression.rs:1318-1397)"""
+    a = torch.zeros(2, 8, 16)
+    part = lambda t, tile=(1, 1, 16), mp=(1, 1, 1), n=4: ct.mapped(ct.partition(t, list(tile)), list(mp), n)
+    ct.mapped_partitions_shared(part(a), part(torch.zeros(2, 8, 16)))
+    ct.mapped_partitions_shared(part(a), part(torch.zeros(2, 8, 9)))                 # the same (2, 8, 1) grid
+    with pytest.raises(ct.CutileError, match="equal logical partition grids: axis 1 has 8 vs 9 tiles"):
+        ct.mapped_partitions_shared(part(a), part(torch.zeros(2, 9, 16)))
+    with pytest.raises(ct.CutileError, match="share tile and map shapes"):
+        ct.mapped_partitions_shared(part(a), part(torch.zeros(2, 16, 16), tile=(1, 2, 16)))
+    with pytest.raises(ct.CutileError, match="share tile and map shapes"):
+        ct.mapped_partitions_shared(part(a), part(torch.zeros(2, 8, 16), mp=(1, 2, 1)))
+
+
+@pytest.mark.gpu
+def test_gpu_two_caches_through_one_shared_stream(ct, dev):
+    """dynpos_shared_rank3_updates_only_the_device_read_range and
+    prefill_shared_rank3_bounds_the_source_by_the_subrange_not_the_cache (mapped_partition_schedule_matrix.rs:372-476)"""
+    c = CASES["shared_rank3"]
+    h, max_seq, d, poison = c["heads"], c["max_seq"], c["d"], c["poison"]
+
+    def caches(n_blocks):
+        k, v = (torch.full((h, max_seq, d), poison, device=dev) for _ in range(2))
+        mk = lambda t: ct.mapped(ct.partition(t, c["tile"]), c["map_shape"], n_blocks)
+        return k, v, mk(k), mk(v)
+
+    # start read from device memory; source [heads, seq, d]
+    dp = c["dynpos"]
+    src = (np.arange(np.prod(dp["source_shape"]), dtype=np.float32) * dp["source_scale"] + 1.0).reshape(dp["source_shape"])
+    k, v, mk, mv = caches(dp["num_tile_blocks"])
+    pos = torch.tensor([dp["position"]], dtype=torch.int32, device=dev)
+    ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), dp["n_tiles"], position=pos)
+    torch.cuda.synchronize()
+    want = np.full((h, max_seq, d), poison, np.float32)
+    want[:, dp["position"]:dp["position"] + dp["n_tiles"]] = src
+    want_v = np.where(want == poison, want, 2 * want)
+    assert np.array_equal(k.cpu().numpy(), want) and np.array_equal(v.cpu().numpy(), want_v)
+    # the same start by value
+    k, v, mk, mv = caches(dp["num_tile_blocks"])
+    ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), dp["n_tiles"], start_tile=dp["position"])
+    torch.cuda.synchronize()
+    assert np.array_equal(k.cpu().numpy(), want) and np.array_equal(v.cpu().numpy(), want_v)
+    # a device start that does not fit the axis writes nothing; a host one is an error
+    k, v, mk, mv = caches(dp["num_tile_blocks"])
+    ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), dp["n_tiles"],
+                                      position=torch.tensor([max_seq - 1], dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    assert torch.all(k == poison) and torch.all(v == poison)
+    with pytest.raises(ct.CutileError, match="exceeds the 8 tiles"):
+        ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), dp["n_tiles"], start_tile=max_seq - 1)
+    # prefill: source [seq, heads, d], rows 0..seq_len of a longer cache
+    pf = c["prefill"]
+    src = (np.arange(np.prod(pf["source_shape"]), dtype=np.float32) * pf["source_scale"] + 1.0).reshape(pf["source_shape"])
+    k, v, mk, mv = caches(pf["num_tile_blocks"])
+    ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), pf["seq_len"], source_seq_major=True)
+    torch.cuda.synchronize()
+    want = np.full((h, max_seq, d), poison, np.float32)
+    want[:, :pf["seq_len"]] = src.transpose(1, 0, 2)
+    assert np.array_equal(k.cpu().numpy(), want) and np.array_equal(v.cpu().numpy(), np.where(want == poison, want, 2 * want))
+    # larger, ragged: tiles [1, 4, 8] over caches [3, 22, 20] (grid (3, 6, 3)), grouped trailing axes, 7 tile blocks
+    hh, ms, dd, start, n = 3, 22, 20, 2, 3
+    src = np.random.default_rng(5).standard_normal((hh, n * 4, dd)).astype(np.float32)
+    k, v = (torch.full((hh, ms, dd), poison, device=dev) for _ in range(2))
+    mk, mv = (ct.mapped(ct.partition(t, [1, 4, 8]), [1, 2, 2], 7) for t in (k, v))
+    ct.mapped_shared_cache_update_f32(mk, mv, torch.from_numpy(src).to(dev), n, start_tile=start)
+    torch.cuda.synchronize()
+    want = np.full((hh, ms, dd), poison, np.float32)
+    want[:, start * 4:(start + n) * 4] = src
+    assert np.array_equal(k.cpu().numpy(), want) and np.array_equal(v.cpu().numpy(), np.where(want == poison, want, 2 * want))
+
+
 @pytest.mark.gpu
 def test_gpu_explicit_grid_is_a_checked_override(ct, dev):
     # an explicit .grid() must equal (num_tile_blocks, 1, 1)
