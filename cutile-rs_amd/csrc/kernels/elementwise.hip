@@ -907,8 +907,15 @@ __device__ __forceinline__ void fused_finish(const FusedRowsArgs& a, int64_t s_i
     lo.raw = ylo.raw;
     hi.raw = yhi.raw;
   }
-  reinterpret_cast<u32x4*>(dst)[c] = lo.raw;
-  reinterpret_cast<u32x4*>(dst + a.half)[c] = hi.raw;
+  if (is_q) {   // the rotated queries go to the attention kernel of a later launch: past the caches
+    asm volatile("");
+    __builtin_nontemporal_store(lo.raw, reinterpret_cast<u32x4*>(dst) + c);
+    __builtin_nontemporal_store(hi.raw, reinterpret_cast<u32x4*>(dst + a.half) + c);
+    asm volatile("");
+  } else {
+    reinterpret_cast<u32x4*>(dst)[c] = lo.raw;
+    reinterpret_cast<u32x4*>(dst + a.half)[c] = hi.raw;
+  }
 }
 }  // namespace
 
