@@ -587,6 +587,45 @@ class DecodeAttentionGrouped(Workload):
                {"max_abs": err, "max_abs_lse": err_lse, "tolerance": 2e-2, "ok": err <= 2e-2 and err_lse <= 2e-3}
 
 
+class KvbmCopy(Workload):
+    """copy_stacked_to_contiguous_f16 (cutile-kernels/src/experimental/kvbm.rs:112-187): per-layer NHD chunks gathered into
+    universal blocks [nh, nl, no, nt, hd] through pointer tables; every element is read once and written once."""
+    name, unit, dtype = "kvbm_stacked_nhd_to_universal_f16_256x4MiB", "GB/s", "f16 (layout conversion)"
+    blocks, nh, nl, no, nt, hd = 256, 8, 32, 2, 32, 128
+    work = 2.0 * blocks * nh * nl * no * nt * hd * 2
+    config = {"workload": "copy_stacked_to_contiguous fp16: 256 blocks x (8 heads, 32 layers, K and V, 32 tokens, 128), 16384 stacked "
+                          "NHD chunks of 64 KiB -> 256 universal blocks of 4 MiB"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct, self.np = ct, np
+        per_chunk = self.nt * self.nh * self.hd
+        n_chunks = self.blocks * self.nl * self.no
+        rng = np.random.default_rng(97)
+        self.host = rng.integers(0, 65536, (n_chunks, per_chunk), dtype=np.uint16)
+        self.stacked = torch.from_numpy(self.host.view(np.int16)).to(dev).view(torch.float16)
+        self.out = torch.zeros(self.blocks, self.nh * self.nl * self.no * self.nt * self.hd, dtype=torch.float16, device=dev)
+        base, step = self.stacked.data_ptr(), per_chunk * 2
+        self.s_table = torch.tensor([base + c * step for c in range(n_chunks)], dtype=torch.int64, device=dev)
+        self.c_table = torch.tensor([self.out[b].data_ptr() for b in range(self.blocks)], dtype=torch.int64, device=dev)
+
+    def launch(self):
+        self.ct.kvbm_copy_f16(False, self.ct.KVBM_STACKED_NHD, self.ct.KVBM_UNIVERSAL, self.blocks, self.s_table, self.c_table,
+                              self.nh, self.nl, self.no, self.nt, self.hd)
+
+    def cpu_baseline(self, oracle, np, torch):
+        nb = 32
+        st = self.host[: nb * self.nl * self.no].reshape(nb, self.nl, self.no, self.nt, self.nh, self.hd)
+        t0 = time.perf_counter()
+        ref = oracle.kvbm_stacked_to_contiguous(st, "nhd", "universal")
+        dt = time.perf_counter() - t0
+        got = self.out[:nb].cpu().numpy().view(np.uint16).reshape(ref.shape)
+        same = bool(np.array_equal(got, ref))
+        return {"value": self.work * nb / self.blocks / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"the first {nb} of {self.blocks} blocks (numpy transpose)"}, {"bit_exact": same, "ok": same}
+
+
 class PrefillAttention(Workload):
     """fmha_prefill_causal (cutile-kernels/src/attention.rs:242-391): f16, [seq, heads, D] queries against a
     [kv_heads, seq, D] cache, grouped heads; flops counted like the causal FMHA bench (half of 4 s^2 d per head)."""
@@ -786,7 +825,7 @@ class EmbeddingBatch(Workload):
 
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
+            AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
 
 
 EXTRA_WORKLOADS = [Copy]  # only by name, never in the default run
