@@ -124,6 +124,9 @@ def lib() -> C.CDLL:
             "cutile_launch_fmha_decode_gqa_split": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
                                                     P(PartitionArg), f32, P(TensorArg), P(LaunchOpts)],
             "cutile_launch_splitk_reduce_merge": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_fmha_decode_gqa_noalloc": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), f32,
+                                                      P(TensorArg), i32, i32],
+            "cutile_scratch_capacity": [P(C.c_size_t)],
             "cutile_launch_rope_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), i32, P(PartitionArg),
                                        i32, P(LaunchOpts)],
             "cutile_launch_gemm": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, i32, P(LaunchOpts)],
@@ -492,6 +495,22 @@ def splitk_reduce_merge(att_partial, lse_partial, out: Partition, *, stream=None
     aa, la = tensor_arg(att_partial), tensor_arg(lse_partial)
     o, keep = _opts(grid, generics, None)
     check(lib().cutile_launch_splitk_reduce_merge(_stream(stream), C.byref(aa), C.byref(la), C.byref(out.arg()), C.byref(o)))
+
+
+def fmha_decode_gqa_noalloc(q, k, v, out: Partition, qk_scale: float, position_start, num_kv_splits: int, bn: int = 64, *,
+                            stream=None) -> None:
+    """split-KV decode attention and merge in one call that allocates nothing: the partial results live in the
+    library's device-resident scratch array (8 MiB per GPU); position_start: one-element device tensor"""
+    qa, ka, va, pa = tensor_arg(q), tensor_arg(k), tensor_arg(v), tensor_arg(position_start, dtype=U32)
+    check(lib().cutile_launch_fmha_decode_gqa_noalloc(_stream(stream), C.byref(qa), C.byref(ka), C.byref(va),
+                                                      C.byref(out.arg()), C.c_float(qk_scale), C.byref(pa),
+                                                      int(num_kv_splits), int(bn)))
+
+
+def scratch_capacity() -> int:
+    n = C.c_size_t(0)
+    check(lib().cutile_scratch_capacity(C.byref(n)))
+    return int(n.value)
 
 
 def gemm(z: Partition, x, y, k: int, *, accumulate: bool = True, stream=None, grid=None, generics=None,

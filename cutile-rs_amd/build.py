@@ -23,6 +23,7 @@ HOST_DIR = os.path.join(ROOT, "csrc", "host")
 LIB_DIR = os.path.join(ROOT, "lib")
 BUILD_DIR = os.path.join(ROOT, "build")
 LIB_PATH = os.path.join(LIB_DIR, "libcutile_hip.so")
+SCRATCH_LIB_PATH = os.path.join(LIB_DIR, "libcutile_hip_scratch.so")
 
 # image symbol -> kernel source
 IMAGES = {
@@ -115,6 +116,18 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
     return LIB_PATH
 
 
+def build_scratch_library(force: bool = False) -> str:
+    """The side library that holds the device-resident scratch array: the one file hipcc compiles for host and
+    device.  It links the HIP runtime by soname; libcutile_hip.so opens it only after it has bound a runtime."""
+    src = os.path.join(HOST_DIR, "scratch.hip")
+    deps = [src, os.path.join(HOST_DIR, "scratch.h")]
+    if force or not _newer(SCRATCH_LIB_PATH, deps):
+        _run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+              "-o", SCRATCH_LIB_PATH, src])
+    return SCRATCH_LIB_PATH
+
+
 CPP_TEST_DIR = os.path.join(ROOT, "..", "tests", "cpp")
 CPP_TESTS = {
     # binary -> (source, needs the library, extra flags)
@@ -151,6 +164,7 @@ def build_cpp_tests(force: bool = False) -> str:
 
 def build(force: bool = False) -> str:
     lib = build_host_library(build_code_objects(force), force)
+    build_scratch_library(force)
     build_cpp_tests(force)
     return lib
 

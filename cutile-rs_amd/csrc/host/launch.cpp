@@ -8,16 +8,20 @@
 // precompiled variant instead of compiling), push the arguments in signature
 // order (cutile/src/tensor.rs:1723-1739,2005-2016) and launch.  Every check runs
 // before any GPU work, as in the reference.
+#include <dlfcn.h>
+
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
 #include "common.h"
 #include "kernel_table.h"
 #include "runtime_state.h"
+#include "scratch.h"
 #include "../kernels/mapped_partition.h"
 
 using cutile::MappedArg;
@@ -1443,6 +1447,111 @@ cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const 
   // one workgroup per (KV head, query head of the group)
   uint32_t grid[3] = {std::min<uint32_t>(tg[0], (uint32_t)ot.shape[0]) * (uint32_t)group, 1, 1};
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+// ---- decode attention step that allocates nothing ----
+// The partial results of the split kernel (att [kv_heads, NUM_KV_SPLITS*GROUP, D] f16 and lse [kv_heads,
+// NUM_KV_SPLITS*GROUP] f32) live in the device-resident scratch array of scratch.hip instead of caller tensors.
+// The side library that holds the array is opened on first use, after the HIP runtime is bound, so it attaches to the
+// runtime this process already runs.
+typedef int (*scratch_lookup_fn)(void**, size_t*, int*);
+static std::mutex g_scratch_mutex;
+static scratch_lookup_fn g_scratch_lookup = nullptr;
+static std::string g_scratch_error;
+
+static cutile_status_t scratch_memory(void** ptr, size_t* bytes) {
+  if (cutile_status_t s = ensure_init()) return s;
+  CUTILE_API_OR_RETURN(api);
+  (void)api;
+  scratch_lookup_fn fn;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_lookup && g_scratch_error.empty()) {
+      std::string path = CUTILE_SCRATCH_LIBRARY;
+      Dl_info info;
+      if (dladdr((const void*)&cutile_launch_fmha_decode_gqa_noalloc, &info) && info.dli_fname) {
+        std::string self = info.dli_fname;
+        size_t slash = self.rfind('/');
+        if (slash != std::string::npos) path = self.substr(0, slash + 1) + CUTILE_SCRATCH_LIBRARY;
+      }
+      void* h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+      if (!h) {
+        const char* e = dlerror();
+        g_scratch_error = std::string("cannot load ") + path + ": " + (e ? e : "unknown");
+      } else {
+        g_scratch_lookup = (scratch_lookup_fn)dlsym(h, CUTILE_SCRATCH_LOOKUP_SYMBOL);
+        if (!g_scratch_lookup) g_scratch_error = path + " lacks " CUTILE_SCRATCH_LOOKUP_SYMBOL;
+      }
+    }
+    fn = g_scratch_lookup;
+    if (!fn) return fail(CUTILE_ERR_LIBRARY_INIT, "shared object init failed: %s", g_scratch_error.c_str());
+  }
+  int ordinal = -1;
+  const int err = fn(ptr, bytes, &ordinal);
+  if (err != 0) return from_hip((hipError_t)err, "hipGetSymbolAddress(scratch)");
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_scratch_capacity(size_t* bytes) {
+  CUTILE_REQUIRE(bytes, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  *bytes = CUTILE_SCRATCH_BYTES;
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_launch_fmha_decode_gqa_noalloc(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                                      const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                                      const cutile_partition_arg_t* out, float qk_scale,
+                                                      const cutile_tensor_arg_t* position_start, int32_t num_kv_splits,
+                                                      int32_t bn) {
+  if (cutile_status_t s = check_tensor(q, "q", 3, 3)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 3, 3)) return s;
+  const int32_t kv_heads = q->shape[0], group = q->shape[1], d = q->shape[2];
+  CUTILE_REQUIRE(num_kv_splits > 0 && bn > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "fmha_decode_gqa_noalloc: NUM_KV_SPLITS and BN must be positive");
+  CUTILE_REQUIRE(out->tensor.shape[0] == kv_heads && out->tensor.shape[1] == group && out->tensor.shape[2] == d,
+                 CUTILE_ERR_KERNEL_LAUNCH, "fmha_decode_gqa_noalloc: out must be [kv_heads, GROUP, D] like q");
+  // partials first, their log-sum-exp behind them on the next 256-byte boundary
+  const uint64_t rows = (uint64_t)kv_heads * (uint64_t)num_kv_splits * (uint64_t)group;
+  const uint64_t att_bytes = (rows * (uint64_t)d * 2 + 255) / 256 * 256;
+  const uint64_t need = att_bytes + rows * 4;
+  CUTILE_REQUIRE((uint64_t)num_kv_splits * (uint64_t)group <= 0x7fffffffull / (uint64_t)std::max(d, 1) && need <= CUTILE_SCRATCH_BYTES,
+                 CUTILE_ERR_KERNEL_LAUNCH,
+                 "fmha_decode_gqa_noalloc: %d KV heads x %d splits x GROUP %d x D %d needs %llu bytes of partial results, "
+                 "the device-resident scratch holds %u; use fewer splits or the split + merge entry points with caller memory",
+                 kv_heads, num_kv_splits, group, d, (unsigned long long)need, (unsigned)CUTILE_SCRATCH_BYTES);
+  void* base = nullptr;
+  size_t capacity = 0;
+  if (cutile_status_t s = scratch_memory(&base, &capacity)) return s;
+  CUTILE_REQUIRE(base && need <= capacity, CUTILE_ERR_STATE, "fmha_decode_gqa_noalloc: scratch lookup returned %zu bytes", capacity);
+  const int32_t sg = num_kv_splits * group;
+  cutile_partition_arg_t att;
+  memset(&att, 0, sizeof(att));
+  att.tensor.ptr = base;
+  att.tensor.dtype = CUTILE_DTYPE_F16;
+  att.tensor.rank = 3;
+  att.tensor.shape[0] = kv_heads; att.tensor.shape[1] = sg; att.tensor.shape[2] = d;
+  att.tensor.strides[0] = sg * d; att.tensor.strides[1] = d; att.tensor.strides[2] = 1;
+  att.partition_shape[0] = 1; att.partition_shape[1] = group; att.partition_shape[2] = d;
+  att.partition_strides[0] = att.partition_strides[1] = att.partition_strides[2] = 1;
+  cutile_partition_arg_t lse;
+  memset(&lse, 0, sizeof(lse));
+  lse.tensor.ptr = (char*)base + att_bytes;
+  lse.tensor.dtype = CUTILE_DTYPE_F32;
+  lse.tensor.rank = 2;
+  lse.tensor.shape[0] = kv_heads; lse.tensor.shape[1] = sg;
+  lse.tensor.strides[0] = sg; lse.tensor.strides[1] = 1;
+  lse.partition_shape[0] = 1; lse.partition_shape[1] = group;
+  lse.partition_strides[0] = lse.partition_strides[1] = 1;
+  const std::string g_s = std::to_string(group), bn_s = std::to_string(bn), d_s = std::to_string(d), n_s = std::to_string(num_kv_splits);
+  const char* generics[4] = {g_s.c_str(), bn_s.c_str(), d_s.c_str(), n_s.c_str()};
+  cutile_launch_opts_t split_opts;
+  memset(&split_opts, 0, sizeof(split_opts));
+  split_opts.generics = generics;
+  split_opts.n_generics = 4;
+  // Every (head, split) workgroup of the split kernel writes its GROUP rows and log-sum-exp values, an empty split
+  // included, so nothing in the scratch has to start at zero and what an earlier call left there is never read.
+  if (cutile_status_t s = cutile_launch_fmha_decode_gqa_split(stream, q, k, v, &att, &lse, qk_scale, position_start, &split_opts)) return s;
+  return cutile_launch_splitk_reduce_merge(stream, &att.tensor, &lse.tensor, out, nullptr);
 }
 
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,

@@ -472,6 +472,24 @@ cutile_status_t cutile_launch_attention_decode_kernel_grouped_f16(
 cutile_status_t cutile_launch_splitk_reduce_merge(cutile_stream_t stream, const cutile_tensor_arg_t* att_partial,
                                                   const cutile_tensor_arg_t* lse_partial, const cutile_partition_arg_t* out,
                                                   const cutile_launch_opts_t* opts);
+/* One decode-attention step that allocates nothing.  It has no counterpart in the reference: it is for callers
+ * that cannot allocate device memory (code under graph capture, tight serving loops, harnesses that forbid it).
+ * Computes what cutile_launch_fmha_decode_gqa_split followed by cutile_launch_splitk_reduce_merge compute — q
+ * [kv_heads, GROUP, D], k, v [kv_heads, max_seq, D], keys 0..*position_start dealt to `num_kv_splits` splits in tiles
+ * of `bn` keys, out [kv_heads, GROUP, D] partitioned [1, GROUP, CHUNK_D] — with the partial results
+ * (kv_heads * num_kv_splits * GROUP rows of D f16 values, rounded up to 256 bytes, plus 4 bytes of log-sum-exp per row)
+ * in a device-resident array of cutile_scratch_capacity() bytes (8 MiB) that each GPU holds from its first call until
+ * the process ends.  A call that needs more fails with CUTILE_ERR_KERNEL_LAUNCH before any GPU work.  No device memory
+ * is allocated or freed, here or in the kernels.  Every call on one GPU uses that GPU's one array: calls that overlap
+ * on one GPU (two streams, two threads) race; calls on one stream are ordered.  Nothing in the array has to start
+ * at zero — the split kernel writes every row a merge reads — so nothing is cleared between calls. */
+cutile_status_t cutile_launch_fmha_decode_gqa_noalloc(cutile_stream_t stream, const cutile_tensor_arg_t* q,
+                                                      const cutile_tensor_arg_t* k, const cutile_tensor_arg_t* v,
+                                                      const cutile_partition_arg_t* out, float qk_scale,
+                                                      const cutile_tensor_arg_t* position_start, int32_t num_kv_splits,
+                                                      int32_t bn);
+/* bytes of the device-resident scratch array behind cutile_launch_fmha_decode_gqa_noalloc (needs no GPU) */
+cutile_status_t cutile_scratch_capacity(size_t* bytes);
 /* gemm<T, BM, BN, BK>(z: [BM,BN] tiles, x, y, k): z <- z + x·y with f32
  * accumulation (z is read as the initial accumulator, like the reference bench;
  * `accumulate` = 0 starts from zero like the example) —
