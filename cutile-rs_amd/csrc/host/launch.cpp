@@ -187,6 +187,17 @@ bool same_shape(const cutile_tensor_arg_t& a, const cutile_tensor_arg_t& b) {
   return true;
 }
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// The pipelined matrix kernels address a whole operand through one buffer descriptor with 32-bit byte offsets, and
+// offset 0x80000000 stands for "outside": an operand must end below 2 GiB from its first element.  Bytes from the
+// first element of row 0 to the end of the last row of a rank-2 tensor (rank-2 view of the two innermost axes).
+int64_t extent_bytes_2d(int64_t rows, int64_t cols, int64_t row_stride, int64_t elem_size) {
+  return rows > 0 && cols > 0 ? ((rows - 1) * row_stride + cols) * elem_size : 0;
+}
+int64_t extent_bytes_2d(const cutile_tensor_arg_t& t) {
+  return extent_bytes_2d(t.shape[0], t.shape[1], t.strides[0], (int64_t)cutile_dtype_size(t.dtype));
+}
+constexpr int64_t kDescriptorLimit = 1ll << 31;
 int64_t numel(const cutile_tensor_arg_t& t) {
   int64_t n = 1;
   for (int i = 0; i < t.rank; ++i) n *= t.shape[i];
@@ -1617,7 +1628,8 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   const bool fast_layout = x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
                            y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
                            aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
-                           k_total % 8 == 0;
+                           k_total % 8 == 0 && extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit &&
+                           extent_bytes_2d(zt) < kDescriptorLimit;   // larger operands: the any-layout kernel (64-bit addresses)
   const std::string dt = in_f32 ? "f32" : in_f16 ? "f16" : zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
   // The ring-pipelined variants ("_r") fetch whole K tiles only.
   const int32_t k_valid = std::min(std::min(x->shape[1], y->shape[0]), k_total);
@@ -1806,7 +1818,9 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
   if (cutile_status_t s = mapped_launch_grid(zm, opts, &m, grid)) return s;
   const bool fast_layout = (in_bf16 || in_f16) && x->strides[1] == 1 && y->strides[1] == 1 && zt.strides[1] == 1 && x->strides[0] % 8 == 0 &&
                            y->strides[0] % 8 == 0 && zt.strides[0] % 4 == 0 && aligned16(x->ptr) && aligned16(y->ptr) &&
-                           aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0;
+                           aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
+                           extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit &&
+                           extent_bytes_2d(zt) < kDescriptorLimit;
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
@@ -2014,6 +2028,10 @@ cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partitio
                      aligned16(ot.ptr) && q->strides[0] % 8 == 0 && q->strides[1] % 8 == 0 && k->strides[0] % 8 == 0 &&
                      k->strides[1] % 8 == 0 && v->strides[0] % 8 == 0 && v->strides[1] % 8 == 0,
                  CUTILE_ERR_KERNEL_NOT_FOUND, "fmha: precompiled variants need unit head-dim stride and 16-byte aligned rows");
+  // one descriptor per (batch, head): its rows must end below 2 GiB
+  CUTILE_REQUIRE(extent_bytes_2d(m, d, q->strides[2], 2) < kDescriptorLimit && extent_bytes_2d(k->shape[2], d, k->strides[2], 2) < kDescriptorLimit &&
+                     extent_bytes_2d(v->shape[2], d, v->strides[2], 2) < kDescriptorLimit && extent_bytes_2d(m, d, ot.strides[1], 2) < kDescriptorLimit,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "fmha: the rows of one (batch, head) of q, k, v and out must each end below 2 GiB from the first");
   const std::string dt = cutile_dtype_name(q->dtype);
   std::vector<std::string> acceptable, same_bn;
   for (const auto& e : kernel_table())
@@ -2089,6 +2107,9 @@ cutile_status_t cutile_launch_fmha_seq_f16(cutile_stream_t stream, const cutile_
   };
   CUTILE_REQUIRE(rows_ok(*q) && rows_ok(*k) && rows_ok(*v) && rows_ok(ot), CUTILE_ERR_KERNEL_NOT_FOUND,
                  "sequence attention: precompiled variants need unit head-dim stride and 16-byte aligned rows");
+  CUTILE_REQUIRE(extent_bytes_2d(q->shape[0], d, q->strides[0], 2) < kDescriptorLimit && extent_bytes_2d(max_seq, d, k->strides[1], 2) < kDescriptorLimit &&
+                     extent_bytes_2d(max_seq, d, v->strides[1], 2) < kDescriptorLimit && extent_bytes_2d(ot.shape[0], d, ot.strides[0], 2) < kDescriptorLimit,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "sequence attention: the rows of one head of q, k, v and out must each end below 2 GiB from the first");
   // what the launch covers: rows 0 .. rows_cov and heads 0 .. heads_cov of out
   const int32_t rows_cov = (int32_t)std::min<int64_t>((int64_t)tg[0] * bm, ot.shape[0]);
   const int32_t heads_cov = (int32_t)std::min<int64_t>((int64_t)tg[1] * pack, ot.shape[1]);
@@ -2230,6 +2251,12 @@ cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cu
                      aligned16(y->ptr) && aligned16(zt.ptr) && ((uintptr_t)xs->ptr & 3) == 0 && ((uintptr_t)ys->ptr & 3) == 0,
                  CUTILE_ERR_KERNEL_NOT_FOUND,
                  "linear_tile: precompiled variants need K a multiple of 128, unit inner strides and aligned rows");
+  CUTILE_REQUIRE(extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit && extent_bytes_2d(*xs) < kDescriptorLimit &&
+                     extent_bytes_2d(*ys) < kDescriptorLimit && extent_bytes_2d(zt) < kDescriptorLimit,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile: precompiled variants address an operand with 32-bit byte offsets: x, y, the scales and z must each end "
+                 "below 2 GiB from their first element (x spans %lld bytes, y %lld, z %lld)",
+                 (long long)extent_bytes_2d(*x), (long long)extent_bytes_2d(*y), (long long)extent_bytes_2d(zt));
   const std::string dt = zt.dtype == CUTILE_DTYPE_F32 ? "f32" : "bf16";
   // A kernel tile that is a whole multiple of the partition tile computes the
   // same output when the launch covers the whole tensor.
@@ -2312,6 +2339,12 @@ cutile_status_t cutile_launch_linear_tile_nvfp4(cutile_stream_t stream, const cu
                      aligned16(y->ptr) && aligned16(zt.ptr) && ((uintptr_t)xs->ptr & 1) == 0 && ((uintptr_t)ys->ptr & 1) == 0,
                  CUTILE_ERR_KERNEL_NOT_FOUND,
                  "linear_tile (nvfp4): precompiled variants need K a multiple of 64, unit inner strides and aligned rows");
+  CUTILE_REQUIRE(extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit && extent_bytes_2d(*xs) < kDescriptorLimit &&
+                     extent_bytes_2d(*ys) < kDescriptorLimit && extent_bytes_2d(zt) < kDescriptorLimit,
+                 CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "linear_tile (nvfp4): precompiled variants address an operand with 32-bit byte offsets: x, y, the scales and z must each "
+                 "end below 2 GiB from their first element (x spans %lld bytes, y %lld, z %lld)",
+                 (long long)extent_bytes_2d(*x), (long long)extent_bytes_2d(*y), (long long)extent_bytes_2d(zt));
   const std::string dt = zt.dtype == CUTILE_DTYPE_F32 ? "f32" : "bf16";
   // A kernel tile that is a whole multiple of the partition tile computes the same output when the
   // launch covers the whole tensor (the reference example's 16x16 tiles run on the 32x32 kernel).

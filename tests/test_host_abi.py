@@ -354,3 +354,42 @@ def test_decode_mapped_and_fp4_launchers_on_the_recording_runtime(fake_hip):
         with pytest.raises(ct.CutileError, match=msg):
             fn()
     assert L.cutile_testing_launch_count() == n0
+
+
+def test_operands_of_2_gib_and_more_leave_the_32_bit_offset_kernels(fake_hip):
+    """The pipelined matrix kernels address an operand through one descriptor with 32-bit byte offsets (0x80000000 means
+    'outside'), so an operand that spans 2 GiB or more must not reach them: GEMM falls to the any-layout kernel
+    (64-bit addresses), the block-scaled GEMMs and attention refuse.  Untouched host memory stands in for the operands."""
+    ct = fake_hip
+    bf = torch.bfloat16
+    z = torch.empty(256, 256, dtype=bf)
+    small_a, small_b = torch.empty(256, 512, dtype=bf), torch.empty(512, 256, dtype=bf)
+    ct.gemm(ct.partition(z, [256, 256]), small_a, small_b, 512)
+    assert _last(ct)[0].symbol.startswith(b"gemm_entry__bf16_256x256x64_d")
+    # x spans (255 * (2^22 + 2^15) + 512) * 2 bytes = 2^31 + 8.2 MB through its row stride
+    wide = torch.empty(256 * ((1 << 22) + (1 << 15)), dtype=bf).as_strided((256, 512), ((1 << 22) + (1 << 15), 1))
+    ct.gemm(ct.partition(z, [256, 256]), wide, small_b, 512)
+    assert _last(ct)[0].symbol == b"gemm_entry__bf16_generic"
+    just_below = torch.empty(256 * (1 << 22), dtype=bf).as_strided((256, 512), (1 << 22, 1))          # 2^31 - 8.4 MB
+    ct.gemm(ct.partition(z, [256, 256]), just_below, small_b, 512)
+    assert _last(ct)[0].symbol.startswith(b"gemm_entry__bf16_256x256x64_d")
+    with pytest.raises(ct.CutileError, match="does not fit these arguments"):
+        ct.gemm(ct.partition(z, [256, 256]), wide, small_b, 512, variant="bf16_256x256x64_d4x2")
+    zm = ct.mapped(ct.partition(z, [256, 256]), [1, 1], 1)
+    ct.gemm_persistent(zm, wide, small_b)
+    assert _last(ct)[0].symbol == b"gemm_persistent_entry__bf16_generic"
+    # block-scaled GEMM: no any-layout kernel exists, so the launch is refused before any GPU work
+    n_before = ct.lib().cutile_testing_launch_count()
+    u8 = torch.uint8
+    xq = torch.empty(256 * ((1 << 23) + (1 << 16)), dtype=u8).as_strided((256, 256), ((1 << 23) + (1 << 16), 1))
+    yq, sc = torch.empty(256, 256, dtype=u8), torch.empty(256, 8, dtype=u8)
+    zf = torch.empty(256, 256)
+    with pytest.raises(ct.CutileError, match="below 2 GiB"):
+        ct.linear_tile_mxfp8(ct.partition(zf, [256, 256]), xq, yq, sc, sc, 1.0)
+    # attention: one (batch, head) of k spanning 2 GiB
+    q = torch.empty(1, 1, 256, 128, dtype=bf)
+    k = torch.empty(256 * ((1 << 22) + (1 << 15)), dtype=bf).as_strided((1, 1, 256, 128), (0, 0, (1 << 22) + (1 << 15), 1))
+    out = torch.empty(1, 256, 128, dtype=bf)
+    with pytest.raises(ct.CutileError, match="below 2 GiB"):
+        ct.fmha(ct.partition(out, [1, 256, 128]), q, k, k, 0.1, 0, 1)
+    assert ct.lib().cutile_testing_launch_count() == n_before
