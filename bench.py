@@ -929,6 +929,72 @@ def library_same_box(torch, flush, reps=20):
             "tflops": 2.0 * s ** 3 / (med * 1e-3) / 1e12, "frac_of_2500": 2.0 * s ** 3 / (med * 1e-3) / 1e12 / 2500.0}
 
 
+def _timed(ct, torch, flush, launch, reps=15, warm=3):
+    for _ in range(warm):
+        launch()
+    torch.cuda.synchronize()
+    timer = ct.EventTimer()
+    times = []
+    for _ in range(reps):
+        flush.zero_()
+        timer.start()
+        launch()
+        times.append(timer.stop())
+    timer.close()
+    times.sort()
+    return _quantile(times, 0.5), times[0]
+
+
+def probe_ceilings(ct, torch, flush):
+    """What this box sustains on the bare resources (cutile-rs_amd/csrc/probes/ceilings.hip, a code object of its own
+    launched through the C ABI's module calls), under the same flush + event protocol as the workloads:
+    nothing but bf16 MFMAs on register operands (ones: few bits toggle; random: the bit activity of real data), the
+    same loop with the GEMM kernel's LDS operand traffic, and nontemporal read / write / copy streams of 1 GiB."""
+    import ctypes as C
+
+    path = os.path.join(ROOT, "cutile-rs_amd", "lib", "probes.hsaco")
+    if not os.path.exists(path):
+        return {"error": "lib/probes.hsaco is not built"}
+    with open(path, "rb") as f:
+        mod = ct.Module(f.read())
+    out = {}
+    cus = 256
+    sink = torch.empty(2 * cus * 512, dtype=torch.float32, device="cuda")
+    iters = 20000
+    flops = 2.0 * cus * 8 * iters * 2 * 8 * (2 * 32 * 32 * 16)
+    for name, fn in (("mfma_bf16_registers", "probe_mfma_bf16"), ("mfma_bf16_lds_operands", "probe_mfma_bf16_lds")):
+        f = mod.function(fn)
+        for mode, label in ((0, "ones"), (1, "random")):
+            med, mn = _timed(ct, torch, flush, lambda: ct.Module.launch(
+                f, (2 * cus, 1, 1), (512, 1, 1), [C.c_void_p(sink.data_ptr()), C.c_int32(iters), C.c_int32(mode)]), reps=7, warm=1)
+            out[f"{name}_{label}"] = {"TFLOP/s": round(flops / (med * 1e-3) / 1e12, 1), "frac_of_2500": round(flops / (med * 1e-3) / 1e12 / 2500, 4),
+                                      "kernel_ms": round(med, 3)}
+    n_bytes = 1 << 30
+    n_vec = n_bytes // 16
+    src = torch.empty(n_bytes // 4, dtype=torch.int32, device="cuda").fill_(0x3c003c00)
+    dst = torch.empty(n_bytes // 4, dtype=torch.int32, device="cuda")
+    small = torch.empty(4096, dtype=torch.int32, device="cuda")
+    for name, fn, moved, grids in (("hbm_read", "probe_stream_read", n_bytes, (512, 1024, 2048)),
+                                   ("hbm_write", "probe_stream_write", n_bytes, (512, 2048, 32768)),
+                                   ("hbm_copy", "probe_stream_copy", 2 * n_bytes, (2048, 8192, 32768))):
+        f = mod.function(fn)
+        best = None
+        for g in grids:
+            if fn == "probe_stream_read":
+                params = [C.c_void_p(src.data_ptr()), C.c_void_p(small.data_ptr()), C.c_uint64(n_vec)]
+            elif fn == "probe_stream_write":
+                params = [C.c_void_p(dst.data_ptr()), C.c_uint64(n_vec)]
+            else:
+                params = [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_uint64(n_vec)]
+            med, mn = _timed(ct, torch, flush, lambda: ct.Module.launch(f, (g, 1, 1), (256, 1, 1), params))
+            rate = moved / (med * 1e-3) / 1e9
+            if best is None or rate > best["GB/s"]:
+                best = {"GB/s": round(rate, 1), "frac_of_8000": round(rate / 8000, 4), "workgroups": g, "kernel_ms": round(med, 4)}
+        out[name] = best
+    mod.close()
+    return out
+
+
 BASELINE_CONFIGS = ["gemm_bf16_8192", "gemm_bf16_4096", "fmha_bf16", "fmha_bf16_causal", "rms_norm_f16_16384x8192",
                     "softmax_f16_16384x8192", "saxpy_f32_16777216", "mxfp8_gemm_8192"]
 
@@ -941,6 +1007,7 @@ def main():
     ap.add_argument("--workload", default="gemm_bf16_8192")
     ap.add_argument("--only", action="store_true", help="measure only --workload (no 'also' list)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / sampled parity leg")
+    ap.add_argument("--ceilings", action="store_true", help="with --only: also run the ceiling probes and the vendor-library GEMM")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel here is a one-GPU tile kernel; "
@@ -1004,8 +1071,9 @@ def main():
         c = by_name["copy_f32_67108864"]["roofline"]
         ceilings["hbm_copy_stream"] = {"what": "plain copy of 2^26 f32 through the library's convert kernel (one read + one write)",
                                        "GB/s": round(c["achieved"], 1), "frac_of_8000": round(c["frac"], 4)}
-    if not args.only:
+    if not args.only or args.ceilings:
         ceilings["library_same_box"] = library_same_box(torch, flush)
+        ceilings["probes"] = probe_ceilings(ct, torch, flush)
     if ceilings:
         line["ceilings"] = ceilings
     print(json.dumps(line))

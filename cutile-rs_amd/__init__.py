@@ -775,6 +775,39 @@ def kernel_lookup(function: str, generics: Sequence[str] = (), variant: Optional
     return info
 
 
+class Module:
+    """A code object loaded through the driver layer of the C ABI (cuda-core/src/runtime.rs:309-328, 828-835) and
+    launched with a parameter array (cuda-core/src/api.rs:48-70)."""
+
+    def __init__(self, image: bytes, ordinal: int = 0):
+        self.handle = C.c_void_p()
+        self._image = image
+        L = lib()
+        L.cutile_module_load_data.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        L.cutile_module_get_function.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        L.cutile_launch_kernel.argtypes = [C.c_void_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32, C.c_void_p,
+                                           C.POINTER(C.c_void_p)]
+        L.cutile_module_unload.argtypes = [C.c_void_p]
+        check(L.cutile_module_load_data(device(ordinal), image, len(image), C.byref(self.handle)))
+
+    def function(self, name: str) -> int:
+        f = C.c_void_p()
+        check(lib().cutile_module_get_function(self.handle, name.encode(), C.byref(f)))
+        return f.value
+
+    @staticmethod
+    def launch(function: int, grid, block, params, *, shared_mem_bytes: int = 0, stream=None) -> None:
+        """params: ctypes values in the kernel's signature order"""
+        ptrs = (C.c_void_p * max(1, len(params)))(*[C.cast(C.pointer(p), C.c_void_p) for p in params])
+        check(lib().cutile_launch_kernel(function, (C.c_uint32 * 3)(*grid), (C.c_uint32 * 3)(*block), shared_mem_bytes,
+                                         _stream(stream), ptrs))
+
+    def close(self) -> None:
+        if self.handle:
+            lib().cutile_module_unload(self.handle)
+            self.handle = C.c_void_p()
+
+
 class CapturedGraph:
     """Stream capture and replay through the C ABI (cuda-async/src/cuda_graph.rs:61-244): the launches `record` issues on
     this object's stream are captured once and replayed with one call per step.

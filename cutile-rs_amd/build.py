@@ -116,6 +116,18 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
     return LIB_PATH
 
 
+PROBES_PATH = os.path.join(LIB_DIR, "probes.hsaco")
+
+
+def build_probes(force: bool = False) -> str:
+    """Ceiling probes for bench.py (bare MFMA loop, streaming reads / writes / copies): a code object of their own,
+    not embedded in the host library."""
+    src = os.path.join(ROOT, "csrc", "probes", "ceilings.hip")
+    if force or not _newer(PROBES_PATH, [src]):
+        _run([HIPCC] + DEVICE_FLAGS + ["-o", PROBES_PATH, src])
+    return PROBES_PATH
+
+
 def build_scratch_library(force: bool = False) -> str:
     """The side library that holds the device-resident scratch array: the one file hipcc compiles for host and
     device.  It links the HIP runtime by soname; libcutile_hip.so opens it only after it has bound a runtime."""
@@ -165,6 +177,7 @@ def build_cpp_tests(force: bool = False) -> str:
 def build(force: bool = False) -> str:
     lib = build_host_library(build_code_objects(force), force)
     build_scratch_library(force)
+    build_probes(force)
     build_cpp_tests(force)
     return lib
 
