@@ -43,6 +43,8 @@ DEVICE_FLAGS = [
     # packed FP32 instructions are kept off on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# extra device-compiler flags for one-off builds (e.g. -DNAME=1), space separated
+DEVICE_FLAGS += os.environ.get("CUTILE_EXTRA_DEVICE_FLAGS", "").split()
 HOST_FLAGS = ["-std=c++17", "-O2", "-g0", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
               "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-pthread"]
 

@@ -431,6 +431,18 @@ struct FmhaPingPong {
         qf[ks] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0));
       }
     }
+    // The scores are wanted in the log2 domain, c * (q . k) with c = qk_scale * log2(e).  Q is multiplied by c once,
+    // here (rounded back to T: a relative 2^-9 per element for bf16, below the rounding of P), and the reference
+    // point of the softmax rides in the accumulator the S^T products start from (see neg_ref), so that the
+    // MFMAs deliver c * s - m directly and the softmax spends no multiply-add per score.
+    const float c = qk_scale * kLog2e;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = E::pack2((float)qf[ks][2 * e] * c, (float)qf[ks][2 * e + 1] * c);
+      qf[ks] = __builtin_bit_cast(vec8, w);
+    }
 
     int32_t tc = (k_len + BN - 1) / BN;
     int32_t mask_start = k_len / BN;
@@ -496,7 +508,11 @@ struct FmhaPingPong {
 #pragma unroll
       for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
     float m_i = -INFINITY, l_i = 0.0f;
-    const float c = qk_scale * kLog2e;
+    // Every S^T block starts from -m_ref in all 16 accumulators of the lane (a lane owns one query), m_ref being the
+    // row's reference point (0 until the first tile has set one).
+    f32x16 neg_ref;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) neg_ref[e] = 0.0f;
     const int32_t q_pos = q0 + l32 + input_pos;
 
     // Matrix segments.  Fragments are read kAhead steps before the MFMA that uses
@@ -517,11 +533,7 @@ struct FmhaPingPong {
           o_acc[n % DB] = E::mfma(ring[n % kRing], pf[n / DB], o_acc[n % DB]);
         } else {
           const int m = n - NO;
-          if (m < SB) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s[m % SB][e] = 0.0f;
-          }
-          s[m % SB] = E::mfma(ring[n % kRing], qf[m / SB], s[m % SB]);
+          s[m % SB] = E::mfma(ring[n % kRing], qf[m / SB], m < SB ? neg_ref : s[m % SB]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -534,15 +546,13 @@ struct FmhaPingPong {
 #pragma unroll
       for (int m = 0; m < NS; ++m) {
         if (m + kAhead < NS) ring[(m + kAhead) % kRing] = read_k(kbuf, m + kAhead);
-        if (m < SB) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) s[m % SB][e] = 0.0f;
-        }
-        s[m % SB] = E::mfma(ring[m % kRing], qf[m / SB], s[m % SB]);
+        s[m % SB] = E::mfma(ring[m % kRing], qf[m / SB], m < SB ? neg_ref : s[m % SB]);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    // Softmax segment of tile j: s -> pf, running statistics, rescale when the reference point moves.
+    // Softmax segment of tile j: s -> pf, running statistics.  s holds c * score - m_ref (m_ref = m_i, or 0 before the
+    // first tile).  The reference point moves only when some row's maximum rises more than 2^kSlack above it; then
+    // (and on the first tile) the scores are shifted to the new reference and O, l are rescaled.  Otherwise p = 2^s.
     auto softmax_segment = [&](int32_t j) {
       if (j >= mask_start) {
 #pragma unroll
@@ -560,18 +570,34 @@ struct FmhaPingPong {
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[sb][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      constexpr float kSlack = 8.0f;   // see Fmha: the reference point moves only on a rise above 2^kSlack
-      const float m_cand = fmaxf(m_i, mx * c);
+      constexpr float kSlack = 8.0f;
+      const float m_ref = m_i == -INFINITY ? 0.0f : m_i;       // what the accumulators started from
+      const float m_cand = fmaxf(m_i, mx + m_ref);
       const bool moved = __builtin_amdgcn_ballot_w64(m_cand > m_i + kSlack) != 0;
-      const float m_new = moved ? m_cand : m_i;
-      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+      if (moved) {
+        const float m_use = m_cand == -INFINITY ? 0.0f : m_cand;
+        const float shift = m_use - m_ref;
+#pragma unroll
+        for (int sb = 0; sb < SB; ++sb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) s[sb][e] -= shift;
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);   // 0 on the first tile (m_i = -inf)
+        l_i *= alpha;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+        m_i = m_cand;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) neg_ref[e] = -m_use;
+      }
       float rs = 0.0f;
 #pragma unroll
       for (int sb = 0; sb < SB; ++sb) {
         float p[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[sb][e], c, -m_use));
+          p[e] = __builtin_amdgcn_exp2f(s[sb][e]);
           rs += p[e];
         }
 #pragma unroll
@@ -585,15 +611,6 @@ struct FmhaPingPong {
         }
       }
       rs += __shfl_xor(rs, 32, 64);
-      if (moved) {
-        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-        l_i *= alpha;
-#pragma unroll
-        for (int i = 0; i < DB; ++i)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
-        m_i = m_new;
-      }
       l_i += rs;
     };
     auto interval_end = [&]() {
