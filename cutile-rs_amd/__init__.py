@@ -775,6 +775,63 @@ def kernel_lookup(function: str, generics: Sequence[str] = (), variant: Optional
     return info
 
 
+class Rng:
+    """Device random fills through the C ABI (cuda-core/src/api.rs:214-293): Philox4x32-10; `seed=None` keeps seed 0."""
+
+    def __init__(self, seed: Optional[int] = None):
+        self.handle = C.c_void_p()
+        L = lib()
+        vp, sz, u64 = C.c_void_p, C.c_size_t, C.c_uint64
+        L.cutile_rng_create.argtypes = [C.POINTER(vp)]
+        L.cutile_rng_set_seed.argtypes = [vp, u64]
+        L.cutile_rng_set_offset.argtypes = [vp, u64]
+        L.cutile_rng_get_offset.argtypes = [vp, C.POINTER(u64)]
+        L.cutile_rng_normal_f32.argtypes = [vp, vp, sz, C.c_float, C.c_float, vp]
+        L.cutile_rng_normal_f64.argtypes = [vp, vp, sz, C.c_double, C.c_double, vp]
+        L.cutile_rng_uniform_f32.argtypes = [vp, vp, sz, vp]
+        L.cutile_rng_uniform_f64.argtypes = [vp, vp, sz, vp]
+        L.cutile_rng_destroy.argtypes = [vp]
+        check(L.cutile_rng_create(C.byref(self.handle)))
+        if seed is not None:
+            check(L.cutile_rng_set_seed(self.handle, seed))
+
+    def set_seed(self, seed: int) -> None:
+        check(lib().cutile_rng_set_seed(self.handle, seed))
+
+    @property
+    def offset(self) -> int:
+        v = C.c_uint64()
+        check(lib().cutile_rng_get_offset(self.handle, C.byref(v)))
+        return int(v.value)
+
+    @offset.setter
+    def offset(self, value: int) -> None:
+        check(lib().cutile_rng_set_offset(self.handle, value))
+
+    def _fill(self, t, kind, mean, std, stream):
+        import torch
+
+        if not t.is_contiguous() or t.dtype not in (torch.float32, torch.float64):
+            raise ValueError("Rng fills take contiguous f32 or f64 tensors")
+        L, f32 = lib(), t.dtype == torch.float32
+        ptr, n, st = C.c_void_p(t.data_ptr()), t.numel(), _stream(stream)
+        if kind == "normal":
+            check((L.cutile_rng_normal_f32 if f32 else L.cutile_rng_normal_f64)(self.handle, ptr, n, mean, std, st))
+        else:
+            check((L.cutile_rng_uniform_f32 if f32 else L.cutile_rng_uniform_f64)(self.handle, ptr, n, st))
+
+    def normal_(self, t, mean: float = 0.0, std: float = 1.0, *, stream=None) -> None:
+        self._fill(t, "normal", mean, std, stream)
+
+    def uniform_(self, t, *, stream=None) -> None:
+        self._fill(t, "uniform", 0.0, 1.0, stream)
+
+    def close(self) -> None:
+        if self.handle:
+            lib().cutile_rng_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+
 class Module:
     """A code object loaded through the driver layer of the C ABI (cuda-core/src/runtime.rs:309-328, 828-835) and
     launched with a parameter array (cuda-core/src/api.rs:48-70)."""

@@ -33,6 +33,7 @@ IMAGES = {
     "fmha": "fmha.hip",
     "mxgemm": "mxfp8_gemm.hip",
     "nvfp4": "nvfp4_gemm.hip",
+    "rng": "rng.hip",
 }
 HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp"]
 

@@ -17,6 +17,7 @@ extern const unsigned char cutile_img_gemm_start[], cutile_img_gemm_end[];
 extern const unsigned char cutile_img_fmha_start[], cutile_img_fmha_end[];
 extern const unsigned char cutile_img_mxgemm_start[], cutile_img_mxgemm_end[];
 extern const unsigned char cutile_img_nvfp4_start[], cutile_img_nvfp4_end[];
+extern const unsigned char cutile_img_rng_start[], cutile_img_rng_end[];
 }
 
 namespace cutile {
@@ -38,6 +39,7 @@ ImageRef image_ref(Image img) {
     case IMG_FMHA: return {cutile_img_fmha_start, cutile_img_fmha_end};
     case IMG_MXGEMM: return {cutile_img_mxgemm_start, cutile_img_mxgemm_end};
     case IMG_NVFP4: return {cutile_img_nvfp4_start, cutile_img_nvfp4_end};
+    case IMG_RNG: return {cutile_img_rng_start, cutile_img_rng_end};
     default: return {nullptr, nullptr};
   }
 }
@@ -90,6 +92,9 @@ std::vector<KernelEntry> build_table() {
     add("full", ty, keep(std::string("full_entry__") + ty), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, ty, 0, 1);
     add("arange", ty, keep(std::string("arange_entry__") + ty), IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, ty, 0, 1);
   }
+  // random fills behind cutile_rng_* (Philox4x32-10)
+  add("rng_fill", "f32", "rng_fill_entry__f32", IMG_RNG, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  add("rng_fill", "f64", "rng_fill_entry__f64", IMG_RNG, 256, 0, 0, 0, 0, 0, "f64", 0, 1);
   add("linspace", "f32", "linspace_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
   static const char* kConvertTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64"};
   for (const char* s : kConvertTypes)

@@ -11,7 +11,7 @@
 
 namespace cutile {
 
-enum Image : int { IMG_ELEMENTWISE = 0, IMG_ROWWISE, IMG_GEMM, IMG_FMHA, IMG_MXGEMM, IMG_NVFP4, IMG_COUNT };
+enum Image : int { IMG_ELEMENTWISE = 0, IMG_ROWWISE, IMG_GEMM, IMG_FMHA, IMG_MXGEMM, IMG_NVFP4, IMG_RNG, IMG_COUNT };
 
 struct KernelEntry {
   const char* function;  // entry name in the reference, e.g. "gemm"

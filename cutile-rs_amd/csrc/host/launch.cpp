@@ -2383,3 +2383,81 @@ cutile_status_t cutile_launch_linear_tile_nvfp4(cutile_stream_t stream, const cu
 }
 
 }  // extern "C"
+
+// ---- RNG (cuda-core/src/api.rs:214-293) --------------------------------------------------------------------------
+struct cutile_rng {
+  uint64_t seed = 0;
+  uint64_t offset = 0;   // next Philox block of the stream
+};
+
+static cutile_status_t rng_fill(cutile_rng_t rng, const char* dtype, void* ptr, size_t n, int32_t kind, double mean, double std,
+                                cutile_stream_t stream) {
+  CUTILE_REQUIRE(rng, CUTILE_ERR_INVALID_ARGUMENT, "rng is null");
+  CUTILE_REQUIRE(ptr || n == 0, CUTILE_ERR_INVALID_ARGUMENT, "rng fill: null device pointer");
+  const bool is_f32 = strcmp(dtype, "f32") == 0;
+  CUTILE_REQUIRE(((uintptr_t)ptr & (is_f32 ? 3u : 7u)) == 0, CUTILE_ERR_INVALID_ARGUMENT, "rng fill: misaligned device pointer");
+  if (n == 0) return CUTILE_SUCCESS;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("rng_fill", nullptr, dtype, {dtype}, &res)) return s;
+  const uint64_t per_block = is_f32 ? 4 : 2, blocks = ((uint64_t)n + per_block - 1) / per_block;
+  ArgPacker args;
+  args.push_val<void*>(ptr);
+  args.push_val<uint64_t>((uint64_t)n);
+  args.push_val<uint64_t>(rng->seed);
+  args.push_val<uint64_t>(rng->offset);
+  args.push_val<int32_t>(kind);
+  if (is_f32) {
+    args.push_val<float>((float)mean);
+    args.push_val<float>((float)std);
+  } else {
+    args.push_val<double>(mean);
+    args.push_val<double>(std);
+  }
+  // enough lanes to keep the stores streaming; each lane walks its blocks with the grid's stride
+  uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(blocks, 256), 8192)), 1, 1};
+  if (cutile_status_t s = launch_packed(res.fn, grid, res.entry->block, 0, stream, args)) return s;
+  rng->offset += blocks;
+  return CUTILE_SUCCESS;
+}
+
+extern "C" {
+cutile_status_t cutile_rng_create(cutile_rng_t* rng) {
+  CUTILE_REQUIRE(rng, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  *rng = new cutile_rng();
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_rng_set_seed(cutile_rng_t rng, uint64_t seed) {
+  CUTILE_REQUIRE(rng, CUTILE_ERR_INVALID_ARGUMENT, "rng is null");
+  rng->seed = seed;
+  rng->offset = 0;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_rng_set_offset(cutile_rng_t rng, uint64_t offset) {
+  CUTILE_REQUIRE(rng, CUTILE_ERR_INVALID_ARGUMENT, "rng is null");
+  rng->offset = offset;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_rng_get_offset(cutile_rng_t rng, uint64_t* offset) {
+  CUTILE_REQUIRE(rng && offset, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  *offset = rng->offset;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_rng_normal_f32(cutile_rng_t rng, void* device_ptr, size_t num_elements, float mean, float std,
+                                      cutile_stream_t stream) {
+  return rng_fill(rng, "f32", device_ptr, num_elements, 1, mean, std, stream);
+}
+cutile_status_t cutile_rng_normal_f64(cutile_rng_t rng, void* device_ptr, size_t num_elements, double mean, double std,
+                                      cutile_stream_t stream) {
+  return rng_fill(rng, "f64", device_ptr, num_elements, 1, mean, std, stream);
+}
+cutile_status_t cutile_rng_uniform_f32(cutile_rng_t rng, void* device_ptr, size_t num_elements, cutile_stream_t stream) {
+  return rng_fill(rng, "f32", device_ptr, num_elements, 0, 0.0, 1.0, stream);
+}
+cutile_status_t cutile_rng_uniform_f64(cutile_rng_t rng, void* device_ptr, size_t num_elements, cutile_stream_t stream) {
+  return rng_fill(rng, "f64", device_ptr, num_elements, 0, 0.0, 1.0, stream);
+}
+cutile_status_t cutile_rng_destroy(cutile_rng_t rng) {
+  delete rng;
+  return CUTILE_SUCCESS;
+}
+}  // extern "C"

@@ -14,6 +14,8 @@
 #pragma once
 #include <array>
 #include <cmath>
+#include <optional>
+#include <stdexcept>
 #include <string>
 
 #include "tensor.hpp"
@@ -210,29 +212,73 @@ class Convert : public DeviceOp<Convert<To, From>, Tensor<To>> {
 };
 template <class To, class From> Convert<To, From> convert(std::shared_ptr<Tensor<From>> src) { return Convert<To, From>(std::move(src)); }
 
-// randn / rand: seeded host generator (SplitMix64 counter stream + Box–Muller),
-// copied to the device.  The reference draws from cuRAND (api.rs:683-719); those
-// streams do not exist on this platform, so only the distribution is kept.
-inline uint64_t splitmix64_at(uint64_t seed, uint64_t i) {
-  uint64_t z = seed + (i + 1) * 0x9e3779b97f4a7c15ull;
-  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
-  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
-  return z ^ (z >> 31);
-}
-inline CopyHostVecToDevice<float> randn_flat(float mean, float std, size_t n, uint64_t seed) {
-  auto host = std::make_shared<std::vector<float>>(n);
-  for (size_t i = 0; i < n; ++i) {
-    double u1 = (double)(splitmix64_at(seed, 2 * i) >> 11) * (1.0 / 9007199254740992.0);
-    double u2 = (double)(splitmix64_at(seed, 2 * i + 1) >> 11) * (1.0 / 9007199254740992.0);
-    if (u1 < 1e-300) u1 = 1e-300;
-    (*host)[i] = (float)(mean + std * std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2));
+// randn / rand / randn_f16 (api.rs:683-735): the values are drawn on the device by the library's generator
+// (cutile_rng_*: Philox4x32-10, one generator per op, seeded when a seed is given, as the reference creates one RNG
+// per call).  The op is a stream-ordered fill of a freshly allocated tensor: nothing blocks and nothing crosses the
+// host.  The value stream is this library's own; cuRAND's does not exist on this platform.
+template <class T> struct RngFill;
+template <> struct RngFill<float> {
+  static cutile_status_t normal(cutile_rng_t g, void* p, size_t n, float mean, float std, cutile_stream_t s) { return cutile_rng_normal_f32(g, p, n, mean, std, s); }
+  static cutile_status_t uniform(cutile_rng_t g, void* p, size_t n, cutile_stream_t s) { return cutile_rng_uniform_f32(g, p, n, s); }
+};
+template <> struct RngFill<double> {
+  static cutile_status_t normal(cutile_rng_t g, void* p, size_t n, double mean, double std, cutile_stream_t s) { return cutile_rng_normal_f64(g, p, n, mean, std, s); }
+  static cutile_status_t uniform(cutile_rng_t g, void* p, size_t n, cutile_stream_t s) { return cutile_rng_uniform_f64(g, p, n, s); }
+};
+// RAII generator (cuda-core/src/api.rs:214-293 `RNG`)
+class Rng {
+ public:
+  explicit Rng(std::optional<uint64_t> seed = std::nullopt) {
+    if (cutile_rng_create(&g_) != CUTILE_SUCCESS) throw std::runtime_error("cutile_rng_create failed");
+    if (seed) cutile_rng_set_seed(g_, *seed);
   }
-  return copy_host_vec_to_device(std::move(host));
+  ~Rng() { cutile_rng_destroy(g_); }
+  Rng(const Rng&) = delete;
+  Rng& operator=(const Rng&) = delete;
+  cutile_rng_t raw() const { return g_; }
+
+ private:
+  cutile_rng_t g_ = nullptr;
+};
+
+template <class T>
+class RandomFill : public DeviceOp<RandomFill<T>, Tensor<T>> {
+ public:
+  RandomFill(bool normal, T mean, T std, std::vector<int32_t> shape, std::optional<uint64_t> seed)
+      : normal_(normal), mean_(mean), std_(std), shape_(std::move(shape)), seed_(seed) {}
+  Result<Tensor<T>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<T>(shape_).execute(ctx);
+    if (t.is_err()) return t.error();
+    Rng rng(seed_);
+    const size_t n = t.value().size();
+    if (normal_) CUTILE_TRY_STATUS(RngFill<T>::normal(rng.raw(), t.value().device_pointer(), n, mean_, std_, ctx.stream()->raw()));
+    else CUTILE_TRY_STATUS(RngFill<T>::uniform(rng.raw(), t.value().device_pointer(), n, ctx.stream()->raw()));
+    return t;
+  }
+
+ private:
+  bool normal_;
+  T mean_, std_;
+  std::vector<int32_t> shape_;
+  std::optional<uint64_t> seed_;
+};
+// randn<T>(mean, std, shape, seed): T = float | double (api.rs:683-696)
+template <class T = float>
+RandomFill<T> randn(T mean, T std, std::vector<int32_t> shape, std::optional<uint64_t> seed = std::nullopt) {
+  return RandomFill<T>(true, mean, std, std::move(shape), seed);
 }
-inline auto randn(float mean, float std, std::vector<int32_t> shape, uint64_t seed = 0) {
-  size_t n = checked_num_elements(shape).value_or(0);
-  return randn_flat(mean, std, n, seed).then([shape = std::move(shape)](Tensor<float> t) mutable {
-    return value(std::move(t).reshape(std::move(shape)).unwrap());
+// rand<T>(shape, seed): uniform in [0, 1) (api.rs:722-735)
+template <class T = float>
+RandomFill<T> rand(std::vector<int32_t> shape, std::optional<uint64_t> seed = std::nullopt) {
+  return RandomFill<T>(false, T(0), T(1), std::move(shape), seed);
+}
+// randn_f16: f32 values drawn, then converted (api.rs:698-719: the generator has no f16 form)
+inline auto randn_f16(float mean, float std, std::vector<int32_t> shape, std::optional<uint64_t> seed = std::nullopt) {
+  const size_t n = checked_num_elements(shape).value_or(0);
+  return randn<float>(mean, std, {(int32_t)n}, seed).then([shape = std::move(shape)](Tensor<float> src) mutable {
+    return convert<f16>(std::make_shared<Tensor<float>>(std::move(src))).then([shape = std::move(shape)](Tensor<f16> t) mutable {
+      return value(std::move(t).reshape(std::move(shape)).unwrap());
+    });
   });
 }
 

@@ -174,6 +174,26 @@ cutile_status_t cutile_graph_launch(cutile_graph_exec_t exec, cutile_stream_t st
 cutile_status_t cutile_graph_exec_destroy(cutile_graph_exec_t exec);
 cutile_status_t cutile_graph_destroy(cutile_graph_t graph);
 
+/* RNG: create / seed / normal(f32, f64) / uniform(f32, f64) / destroy — cuda-core/src/api.rs:214-293 (the reference
+ * binds cuRAND's default generator).  Here the generator is Philox4x32-10, counter based, evaluated by a fill kernel of
+ * this library: element e of a stream depends only on (seed, position), so a fill is reproducible whatever the launch
+ * shape, and consecutive fills continue the stream (each fill advances the position by the Philox blocks it used:
+ * 4 f32 or 2 f64 values per block).  The value stream is this library's own, not cuRAND's.  uniform: [0, 1);
+ * normal: Box-Muller.  Fills are enqueued on `stream` (the reference's generator runs on its own stream setting);
+ * a generator is not thread safe (one fill at a time), like a curandGenerator_t. */
+typedef struct cutile_rng* cutile_rng_t;
+cutile_status_t cutile_rng_create(cutile_rng_t* rng);
+cutile_status_t cutile_rng_set_seed(cutile_rng_t rng, uint64_t seed);      /* also rewinds the stream position to 0 */
+cutile_status_t cutile_rng_set_offset(cutile_rng_t rng, uint64_t offset);  /* stream position in Philox blocks */
+cutile_status_t cutile_rng_get_offset(cutile_rng_t rng, uint64_t* offset);
+cutile_status_t cutile_rng_normal_f32(cutile_rng_t rng, void* device_ptr, size_t num_elements, float mean, float std,
+                                      cutile_stream_t stream);
+cutile_status_t cutile_rng_normal_f64(cutile_rng_t rng, void* device_ptr, size_t num_elements, double mean, double std,
+                                      cutile_stream_t stream);
+cutile_status_t cutile_rng_uniform_f32(cutile_rng_t rng, void* device_ptr, size_t num_elements, cutile_stream_t stream);
+cutile_status_t cutile_rng_uniform_f64(cutile_rng_t rng, void* device_ptr, size_t num_elements, cutile_stream_t stream);
+cutile_status_t cutile_rng_destroy(cutile_rng_t rng);
+
 /* ======================================================================== */
 /* Part B — kernel table                                                     */
 /* ======================================================================== */

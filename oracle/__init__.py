@@ -89,6 +89,9 @@ def lib() -> C.CDLL:
             "orc_nvfp4_quantize": (None, [vp, vp, vp, i64, i64]),
             "orc_nvfp4_dequantize": (None, [vp, vp, vp, i64, i64]),
             "orc_nvfp4_gemm_f32": (None, [vp, vp, vp, vp, vp, i64, i64, i64, f32, vp, i64]),
+            "orc_philox4x32_10": (None, [vp, vp, vp]),
+            "orc_rng_fill_f32": (None, [vp, sz, u64, u64, C.c_int, f32, f32]),
+            "orc_rng_fill_f64": (None, [vp, sz, u64, u64, C.c_int, f64, f64]),
         }
         for name, (res, args) in sigs.items():
             fn = getattr(L, name)
@@ -565,3 +568,19 @@ def nvfp4_gemm_f32(x, y, xs, ys, alpha: float = 1.0, rows=None) -> np.ndarray:
     z = np.empty((nr if rows is not None else m, n), np.float32)
     lib().orc_nvfp4_gemm_f32(_p(x), _p(y), _p(xs), _p(ys), _p(z), m, n, kp * 2, alpha, rp, nr)
     return z
+
+
+def philox4x32_10(counter, key) -> np.ndarray:
+    """one Philox4x32-10 block: counter 4 x u32, key 2 x u32 -> 4 x u32"""
+    c, k = _c(counter, np.uint32), _c(key, np.uint32)
+    out = np.empty(4, np.uint32)
+    lib().orc_philox4x32_10(_p(c), _p(k), _p(out))
+    return out
+
+
+def rng_fill(n: int, seed: int, offset: int = 0, kind: str = "uniform", mean: float = 0.0, std: float = 1.0, dtype=np.float32) -> np.ndarray:
+    """what cutile_rng_{uniform,normal}_{f32,f64} write for (seed, stream offset in Philox blocks)"""
+    out = np.empty(n, dtype)
+    fn = lib().orc_rng_fill_f32 if dtype == np.float32 else lib().orc_rng_fill_f64
+    fn(_p(out), n, seed, offset, 0 if kind == "uniform" else 1, mean, std)
+    return out

@@ -1016,3 +1016,60 @@ void orc_rms_norm_f32_example(const float* x, const float* w, float* out, int64_
   }
   free(acc);
 }
+
+/* ---- Philox4x32-10 and the random fills ------------------------------------------------------------ */
+void orc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = counter[0], c1 = counter[1], c2 = counter[2], c3 = counter[3], k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c0 = n0; c1 = (uint32_t)p1; c2 = n2; c3 = (uint32_t)p0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+void orc_rng_fill_f32(float* out, size_t n, uint64_t seed, uint64_t offset, int kind, float mean, float std) {
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  const size_t blocks = (n + 3) / 4;
+  for (size_t b = 0; b < blocks; ++b) {
+    const uint64_t ctr = offset + b;
+    const uint32_t counter[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
+    uint32_t r[4];
+    orc_philox4x32_10(counter, key, r);
+    float v[4];
+    if (kind == 0) {
+      for (int i = 0; i < 4; ++i) v[i] = (float)(r[i] >> 8) * 5.9604644775390625e-8f;
+    } else {
+      for (int pair = 0; pair < 2; ++pair) {
+        const float u1 = (float)((r[2 * pair] >> 8) + 1u) * 5.9604644775390625e-8f;
+        const float u2 = (float)(r[2 * pair + 1] >> 8) * 5.9604644775390625e-8f;
+        const float rad = sqrtf(-2.0f * logf(u1)), t = 6.283185307179586f * u2;
+        v[2 * pair] = fmaf(std, rad * cosf(t), mean);
+        v[2 * pair + 1] = fmaf(std, rad * sinf(t), mean);
+      }
+    }
+    for (int i = 0; i < 4; ++i)
+      if (b * 4 + i < n) out[b * 4 + i] = v[i];
+  }
+}
+
+void orc_rng_fill_f64(double* out, size_t n, uint64_t seed, uint64_t offset, int kind, double mean, double std) {
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  const size_t blocks = (n + 1) / 2;
+  for (size_t b = 0; b < blocks; ++b) {
+    const uint64_t ctr = offset + b;
+    const uint32_t counter[4] = {(uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u};
+    uint32_t r[4];
+    orc_philox4x32_10(counter, key, r);
+    double v0 = (double)((((uint64_t)r[1]) << 21) ^ (uint64_t)(r[0] >> 11)) * 1.1102230246251565e-16;
+    double v1 = (double)((((uint64_t)r[3]) << 21) ^ (uint64_t)(r[2] >> 11)) * 1.1102230246251565e-16;
+    if (kind != 0) {
+      const double rad = sqrt(-2.0 * log(v0 + 1.1102230246251565e-16)), t = 6.283185307179586476925 * v1;
+      v0 = fma(std, rad * cos(t), mean);
+      v1 = fma(std, rad * sin(t), mean);
+    }
+    if (b * 2 < n) out[b * 2] = v0;
+    if (b * 2 + 1 < n) out[b * 2 + 1] = v1;
+  }
+}

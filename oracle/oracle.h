@@ -235,6 +235,17 @@ void orc_nvfp4_dequantize(const uint8_t* data, const uint8_t* scales, float* dst
 void orc_nvfp4_gemm_f32(const uint8_t* x, const uint8_t* y, const uint8_t* xs, const uint8_t* ys, float* z, int64_t m,
                         int64_t n, int64_t k, float alpha, const int64_t* rows, int64_t n_rows);
 
+/* ---- device random fills (cutile_rng_*; the reference binds cuRAND: cuda-core/src/api.rs:214-293) ----------
+ * Philox4x32-10 as published (Salmon et al., SC'11; multipliers 0xD2511F53 / 0xCD9E8D57, Weyl keys 0x9E3779B9 /
+ * 0xBB67AE85), pinned by the Random123 known-answer vectors; the fills restate the layout of the fill kernels:
+ * f32 element e = word e % 4 of block offset + e / 4, f64 element e = words 2(e % 2), 2(e % 2) + 1 of block
+ * offset + e / 2, counter (block, 0), key = seed; uniform in [0, 1); normal by Box-Muller per pair.  The value
+ * stream is this build's own (cuRAND's cannot be reproduced): parity against the reference's stream is unpinned,
+ * the distribution is what the tests check. */
+void orc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+void orc_rng_fill_f32(float* out, size_t n, uint64_t seed, uint64_t offset, int kind, float mean, float std);
+void orc_rng_fill_f64(double* out, size_t n, uint64_t seed, uint64_t offset, int kind, double mean, double std);
+
 #ifdef __cplusplus
 }
 #endif

@@ -312,6 +312,40 @@ TEST(nvfp4_example_all_ones) {
   for (float v : host) CHECK(v == (float)K);
 }
 
+TEST(random_constructors_draw_on_the_device) {
+  // api::randn / rand / randn_f16 (cutile/src/api.rs:683-735): distribution, seed determinism, shapes
+  auto stream = new_stream();
+  const int n = 1 << 20;
+  auto a = api::to_host_vec(api::randn(1.0f, 2.0f, {n}, 42).sync_on(stream).unwrap()).sync_on(stream).unwrap();
+  auto b = api::to_host_vec(api::randn(1.0f, 2.0f, {n}, 42).sync_on(stream).unwrap()).sync_on(stream).unwrap();
+  auto c = api::to_host_vec(api::randn(1.0f, 2.0f, {n}, 43).sync_on(stream).unwrap()).sync_on(stream).unwrap();
+  CHECK(a == b);
+  CHECK(a != c);
+  double mean = 0, var = 0;
+  for (float v : a) mean += v;
+  mean /= n;
+  for (float v : a) var += (v - mean) * (v - mean);
+  var /= n;
+  CHECK(std::fabs(mean - 1.0) < 1e-2 && std::fabs(std::sqrt(var) - 2.0) < 1e-2);
+  auto u_t = api::rand<double>({64, 32}, 5).sync_on(stream).unwrap();
+  CHECK((u_t.shape() == std::vector<int32_t>{64, 32}));
+  auto u = api::to_host_vec(u_t).sync_on(stream).unwrap();
+  double umean = 0;
+  for (double v : u) {
+    CHECK(v >= 0.0 && v < 1.0);
+    umean += v;
+  }
+  CHECK(std::fabs(umean / u.size() - 0.5) < 0.03);
+  auto h_t = api::randn_f16(0.0f, 1.0f, {128, 256}, 9).sync_on(stream).unwrap();
+  CHECK((h_t.shape() == std::vector<int32_t>{128, 256}));
+  auto h = api::to_host_vec(h_t).sync_on(stream).unwrap();
+  auto f = api::to_host_vec(api::randn(0.0f, 1.0f, {128 * 256}, 9).sync_on(stream).unwrap()).sync_on(stream).unwrap();
+  for (size_t i = 0; i < h.size(); ++i) CHECK(std::fabs(f32_from_f16(h[i]) - f[i]) <= std::fabs(f[i]) * 0.001f + 1e-7f);   // the f32 draw, rounded
+  // without a seed the generator's default seed is used: still a valid draw
+  auto d = api::to_host_vec(api::rand<float>({1000}).sync_on(stream).unwrap()).sync_on(stream).unwrap();
+  for (float v : d) CHECK(v >= 0.0f && v < 1.0f);
+}
+
 TEST(graph_replay_matches_eager) {
   auto stream = new_stream();
   const int n = 1 << 16;

@@ -393,3 +393,30 @@ def test_operands_of_2_gib_and_more_leave_the_32_bit_offset_kernels(fake_hip):
     with pytest.raises(ct.CutileError, match="below 2 GiB"):
         ct.fmha(ct.partition(out, [1, 256, 128]), q, k, k, 0.1, 0, 1)
     assert ct.lib().cutile_testing_launch_count() == n_before
+
+
+def test_rng_fills_on_the_recording_runtime(fake_hip):
+    """cutile_rng_*: the fill kernel, its arguments and the stream position (4 f32 or 2 f64 values per Philox block)"""
+    ct = fake_hip
+    rng = ct.Rng(0x1122334455667788)
+    t = torch.zeros(1001)
+    rng.normal_(t, 0.5, 2.0)
+    rec, args = _last(ct)
+    assert rec.symbol == b"rng_fill_entry__f32" and tuple(rec.block) == (256, 1, 1) and tuple(rec.grid) == (1, 1, 1)
+    ptr, n, seed, offset, kind, mean, std = struct.unpack("<QQQQiff", args[:44])
+    assert (ptr, n, seed, offset, kind, mean, std) == (t.data_ptr(), 1001, 0x1122334455667788, 0, 1, 0.5, 2.0)
+    assert rng.offset == 251
+    d = torch.zeros(7, dtype=torch.float64)
+    rng.uniform_(d)
+    rec, args = _last(ct)
+    assert rec.symbol == b"rng_fill_entry__f64"
+    ptr, n, seed, offset, kind = struct.unpack("<QQQQi", args[:36])
+    assert (n, offset, kind) == (7, 251, 0) and rng.offset == 255
+    rng.set_seed(3)
+    assert rng.offset == 0
+    before = ct.lib().cutile_testing_launch_count()
+    rng.uniform_(torch.zeros(0))                                   # nothing to fill: no launch
+    assert ct.lib().cutile_testing_launch_count() == before
+    with pytest.raises(ValueError):
+        rng.uniform_(torch.zeros(4, dtype=torch.float16))
+    rng.close()
