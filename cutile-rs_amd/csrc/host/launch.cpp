@@ -135,8 +135,19 @@ struct ArgPacker {
   }
 };
 
+// What the calling thread's next launcher calls do once their checks have passed (cutile_set_launch_mode), and the
+// table entry the thread's last launcher call resolved (cutile_last_resolved_kernel).
+thread_local int g_launch_mode = 0;
+thread_local const KernelEntry* g_last_entry = nullptr;
+thread_local hipFunction_t g_last_fn = nullptr;
+
 cutile_status_t launch_packed(hipFunction_t fn, const uint32_t grid[3], const uint32_t block[3],
                               uint32_t dyn_lds, cutile_stream_t stream, ArgPacker& args) {
+  if (g_launch_mode != 0) {   // compile-only / specialize-only: every check has run, nothing is enqueued
+    CUTILE_REQUIRE(grid[0] > 0 && grid[1] > 0 && grid[2] > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                   "launch grid (%u, %u, %u) has a zero axis", grid[0], grid[1], grid[2]);
+    return CUTILE_SUCCESS;
+  }
   CUTILE_API_OR_RETURN(api);
   CUTILE_REQUIRE(grid[0] > 0 && grid[1] > 0 && grid[2] > 0, CUTILE_ERR_KERNEL_LAUNCH,
                  "launch grid (%u, %u, %u) has a zero axis", grid[0], grid[1], grid[2]);
@@ -252,8 +263,13 @@ cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* 
   r->entry = find_entry(function, want);
   CUTILE_REQUIRE(r->entry, CUTILE_ERR_KERNEL_NOT_FOUND, "no variant '%s' of kernel '%s'; available: %s",
                  want.c_str(), function, list_variants(function).c_str());
+  g_last_entry = r->entry;
+  g_last_fn = nullptr;
+  if (g_launch_mode == 2) return CUTILE_SUCCESS;   // specialize-only: the identity is known, nothing is loaded
   if (cutile_status_t s = current_device(&r->device)) return s;
-  return load_entry(r->device, r->entry, &r->fn);
+  if (cutile_status_t s = load_entry(r->device, r->entry, &r->fn)) return s;
+  g_last_fn = r->fn;
+  return CUTILE_SUCCESS;
 }
 
 uint32_t div_up(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
@@ -2461,3 +2477,30 @@ cutile_status_t cutile_rng_destroy(cutile_rng_t rng) {
   return CUTILE_SUCCESS;
 }
 }  // extern "C"
+
+// ---- launch modes of the generated launcher (cutile-macro/src/_module.rs:852-900) -------------------------------
+extern "C" {
+cutile_status_t cutile_set_launch_mode(int32_t mode) {
+  CUTILE_REQUIRE(mode >= 0 && mode <= 2, CUTILE_ERR_INVALID_ARGUMENT, "launch mode must be 0 (launch), 1 (compile only) or 2 (specialize only)");
+  g_launch_mode = mode;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_get_launch_mode(int32_t* mode) {
+  CUTILE_REQUIRE(mode, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  *mode = g_launch_mode;
+  return CUTILE_SUCCESS;
+}
+cutile_status_t cutile_last_resolved_kernel(const char** function, cutile_kernel_info_t* info) {
+  CUTILE_REQUIRE(function && info, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
+  CUTILE_REQUIRE(g_last_entry, CUTILE_ERR_STATE, "no launcher call has resolved a kernel on this thread yet");
+  *function = g_last_entry->function;
+  info->function = (cutile_function_t)g_last_fn;
+  info->symbol = g_last_entry->symbol;
+  info->variant = g_last_entry->variant;
+  memcpy(info->block, g_last_entry->block, sizeof(info->block));
+  info->lds_bytes = g_last_entry->lds_bytes;
+  memcpy(info->tile, g_last_entry->tile, sizeof(info->tile));
+  return CUTILE_SUCCESS;
+}
+}  // extern "C"
+

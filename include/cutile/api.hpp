@@ -18,6 +18,8 @@
 #include <stdexcept>
 #include <string>
 
+#include "runtime.hpp"
+#include "specialization.hpp"
 #include "tensor.hpp"
 
 namespace cutile {
@@ -317,6 +319,39 @@ struct Recovered<MappedLaunchPartition<P>> {
   static P get(MappedLaunchPartition<P>&& v) { return std::move(v).into_partition(); }
 };
 
+// How one stored argument enters the specialization identity (kernel_launcher_generator.rs:600-700): a tensor-like
+// argument contributes its stride-one pattern and SpecializationBits, an integer scalar a divisibility hint, a
+// floating-point scalar nothing.
+namespace detail {
+template <class A, class = void> struct has_input_arg : std::false_type {};
+template <class A> struct has_input_arg<A, std::void_t<decltype(input_arg(std::declval<const A&>()))>> : std::true_type {};
+template <class A, class = void> struct has_arg_method : std::false_type {};
+template <class A> struct has_arg_method<A, std::void_t<decltype(std::declval<const A&>().arg())>> : std::true_type {};
+inline const cutile_tensor_arg_t& tensor_of(const cutile_tensor_arg_t& t) { return t; }
+inline const cutile_tensor_arg_t& tensor_of(const cutile_partition_arg_t& p) { return p.tensor; }
+inline const cutile_tensor_arg_t& tensor_of(const cutile_mapped_partition_arg_t& m) { return m.partition.tensor; }
+template <class A>
+void describe_arg(const A& a, size_t index, int32_t max_div, std::vector<std::pair<std::string, std::vector<int32_t>>>* strides,
+                  std::vector<std::pair<std::string, SpecializationBits>>* specs, std::vector<std::pair<std::string, DivHint>>* scalars) {
+  const std::string name = "arg" + std::to_string(index);
+  if constexpr (std::is_integral_v<A>) {
+    scalars->emplace_back(name, DivHint::from_value((int64_t)a).with_max(max_div));
+  } else if constexpr (std::is_floating_point_v<A>) {
+  } else {
+    cutile_tensor_arg_t t{};
+    if constexpr (has_input_arg<A>::value) t = input_arg(a);
+    else if constexpr (has_arg_method<A>::value) { auto rec = a.arg(); t = tensor_of(rec); }
+    else return;
+    std::vector<int32_t> one;
+    for (int i = 0; i < t.rank; ++i) one.push_back(t.strides[i] == 1 ? 1 : 0);
+    strides->emplace_back(name, std::move(one));
+    specs->emplace_back(name, SpecializationBits::from_tensor_arg(t, max_div));
+  }
+}
+template <class Fn, class = void> struct kernel_name { static constexpr const char* value = "kernel"; };
+template <class Fn> struct kernel_name<Fn, std::void_t<decltype(Fn::name)>> { static constexpr const char* value = Fn::name; };
+}  // namespace detail
+
 template <class Fn, class... ArgOps>
 class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple<typename Recovered<typename ArgOps::Output>::type...>> {
  public:
@@ -326,10 +361,69 @@ class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple
   KernelLauncher(KernelLauncher&&) = default;
   // Builder methods of the generated launcher (cutile-macro/src/_module.rs:901-923).
   KernelLauncher generics(std::vector<std::string> g) && { generics_ = std::move(g); return std::move(*this); }
-  KernelLauncher grid(uint32_t x, uint32_t y, uint32_t z) && { grid_ = {x, y, z}; return std::move(*this); }
+  KernelLauncher grid(uint32_t x, uint32_t y, uint32_t z) && { grid_ = {x, y, z}; const_grid_ = false; return std::move(*this); }
+  // const_grid: the same launch grid, and the grid becomes part of the specialization identity.
+  KernelLauncher const_grid(uint32_t x, uint32_t y, uint32_t z) && { grid_ = {x, y, z}; const_grid_ = true; return std::move(*this); }
+  std::array<uint32_t, 3> get_launch_grid() const { return grid_; }
+  KernelLauncher compile_options(CompileOptions o) && { compile_options_ = std::move(o); return std::move(*this); }
   KernelLauncher variant(std::string v) && { variant_ = std::move(v); return std::move(*this); }
 
-  Result<Out> execute(const ExecutionContext& ctx) && {
+  // compile / compile_on (_module.rs:852-866): everything a launch does except the launch block; afterwards the
+  // kernel's code object is loaded on the device, so the first real launch loads nothing.
+  Result<Unit> compile_on(const std::shared_ptr<Stream>& stream) && {
+    ExecutionContext ctx(stream);
+    auto r = std::move(*this).run(ctx, CUTILE_LAUNCH_MODE_COMPILE_ONLY, nullptr);
+    if (r.is_err()) return r.error();
+    return ok();
+  }
+  Result<Unit> compile() && {
+    auto stream = next_stream();
+    if (stream.is_err()) return stream.error();
+    return std::move(*this).compile_on(stream.value());
+  }
+  // specialize / specialize_on (_module.rs:868-878): the identity of this launch, nothing compiled or launched.
+  Result<Specialization> specialize_on(const std::shared_ptr<Stream>& stream) && {
+    ExecutionContext ctx(stream);
+    std::optional<Specialization> spec;
+    auto r = std::move(*this).run(ctx, CUTILE_LAUNCH_MODE_SPECIALIZE_ONLY, &spec);
+    if (r.is_err()) return r.error();
+    return std::move(*spec);
+  }
+  Result<Specialization> specialize() && {
+    auto stream = next_stream();
+    if (stream.is_err()) return stream.error();
+    return std::move(*this).specialize_on(stream.value());
+  }
+  Result<TileFunctionKey> l1_cache_key_on(const std::shared_ptr<Stream>& stream) && {
+    auto s = std::move(*this).specialize_on(stream);
+    if (s.is_err()) return s.error();
+    return std::move(s).unwrap().into_l1_cache_key();
+  }
+  Result<TileFunctionKey> l1_cache_key() && {
+    auto s = std::move(*this).specialize();
+    if (s.is_err()) return s.error();
+    return std::move(s).unwrap().into_l1_cache_key();
+  }
+  Result<std::string> l2_cache_key_on(const std::shared_ptr<Stream>& stream) && {
+    auto s = std::move(*this).specialize_on(stream);
+    if (s.is_err()) return s.error();
+    return s.value().l2_cache_key();
+  }
+  Result<std::string> l2_cache_key() && {
+    auto s = std::move(*this).specialize();
+    if (s.is_err()) return s.error();
+    return s.value().l2_cache_key();
+  }
+
+  Result<Out> execute(const ExecutionContext& ctx) && { return std::move(*this).run(ctx, CUTILE_LAUNCH_MODE_LAUNCH, nullptr); }
+
+ private:
+  enum : int32_t { CUTILE_LAUNCH_MODE_LAUNCH = 0, CUTILE_LAUNCH_MODE_COMPILE_ONLY = 1, CUTILE_LAUNCH_MODE_SPECIALIZE_ONLY = 2 };
+  struct ModeGuard {   // the mode is a property of the thread for the duration of one launcher call
+    explicit ModeGuard(int32_t m) { cutile_set_launch_mode(m); }
+    ~ModeGuard() { cutile_set_launch_mode(0); }
+  };
+  Result<Out> run(const ExecutionContext& ctx, int32_t mode, std::optional<Specialization>* spec) && {
     // 1. run the argument ops in signature order; 2. validate + launch; 3. hand the arguments back.
     auto args = std::move(ops_).execute(ctx);
     if (args.is_err()) return args.error();
@@ -341,15 +435,50 @@ class KernelLauncher : public DeviceOp<KernelLauncher<Fn, ArgOps...>, std::tuple
     opts.generics = gptrs.empty() ? nullptr : gptrs.data();
     opts.n_generics = (int32_t)gptrs.size();
     opts.variant = variant_.empty() ? nullptr : variant_.c_str();
-    cutile_status_t s = std::apply([&](auto&... a) { return Fn::launch(ctx.stream()->raw(), &opts, a...); }, vals);
+    cutile_status_t s;
+    {
+      ModeGuard guard(mode);
+      s = std::apply([&](auto&... a) { return Fn::launch(ctx.stream()->raw(), &opts, a...); }, vals);
+    }
     if (s != CUTILE_SUCCESS) return DeviceError::from_status(s);
+    if (spec) {
+      const char* fn_name = nullptr;
+      cutile_kernel_info_t info{};
+      CUTILE_TRY_STATUS(cutile_last_resolved_kernel(&fn_name, &info));
+      const int32_t max_div = compile_options_.max_divisibility_.value_or(16);
+      std::vector<std::pair<std::string, std::vector<int32_t>>> strides;
+      std::vector<std::pair<std::string, SpecializationBits>> specs;
+      std::vector<std::pair<std::string, DivHint>> scalars;
+      size_t index = 0;
+      std::apply([&](auto&... a) { (detail::describe_arg(a, index++, max_div, &strides, &specs, &scalars), ...); }, vals);
+      char fp[17] = {0};
+      CUTILE_TRY_STATUS(cutile_kernel_fingerprint(fn_name, info.variant, fp));
+      char arch[256] = {0};
+      cutile_device_t dev = nullptr;
+      CUTILE_TRY_STATUS(cutile_device_get(ctx.device_id(), &dev));
+      CUTILE_TRY_STATUS(cutile_device_arch(dev, arch, sizeof(arch)));
+      auto b = TileFunctionKey::builder("cutile_kernels", detail::kernel_name<Fn>::value)
+                   .generics(generics_)
+                   .stride_args(std::move(strides))
+                   .spec_args(std::move(specs))
+                   .scalar_hints(std::move(scalars))
+                   .compile_options(compile_options_)
+                   .source_hash(fp)
+                   .device_id((size_t)ctx.device_id())
+                   .gpu_name(arch)
+                   .compiler_version(cutile_version())
+                   .toolchain_fingerprint(cutile_toolchain_fingerprint());
+      if (const_grid_) b = std::move(b).grid(grid_[0], grid_[1], grid_[2]);
+      spec->emplace(std::move(b).build(), info.variant ? info.variant : "", info.symbol ? info.symbol : "");
+    }
     return std::apply([](auto&... a) { return Out(Recovered<std::decay_t<decltype(a)>>::get(std::move(a))...); }, vals);
   }
 
- private:
   Zip<ArgOps...> ops_;
   std::vector<std::string> generics_;
   std::array<uint32_t, 3> grid_{0, 0, 0};
+  bool const_grid_ = false;
+  CompileOptions compile_options_;
   std::string variant_;
 };
 template <class Fn, class... ArgOps>
@@ -360,8 +489,15 @@ auto make_launcher(Xs&&... xs) {
   return KernelLauncher<Fn, into_op_t<Xs>...>(into_op(std::forward<Xs>(xs))...);
 }
 
+// <kernel>_apply(tuple): the launcher over a tuple of materialised arguments (kernel_launcher_generator.rs:1036-1044).
+template <class Fn, class... Xs>
+auto apply_launcher(std::tuple<Xs...> args) {
+  return std::apply([](auto&&... xs) { return make_launcher<Fn>(std::move(xs)...); }, std::move(args));
+}
+
 namespace kernels {
 struct SaxpyFn {
+  static constexpr const char* name = "saxpy";
   template <class Y, class X>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Y& y, double a, X& x) {
     auto yp = y.arg();
@@ -370,6 +506,7 @@ struct SaxpyFn {
   }
 };
 struct AxpyFn {
+  static constexpr const char* name = "axpy";
   template <class Z, class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, double a, X& x, Yv& y) {
     auto zp = z.arg();
@@ -378,6 +515,7 @@ struct AxpyFn {
   }
 };
 struct AddFn {
+  static constexpr const char* name = "add";
   template <class Z, class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y) {
     auto zp = z.arg();
@@ -386,6 +524,7 @@ struct AddFn {
   }
 };
 struct RmsNormF16Fn {
+  static constexpr const char* name = "rms_norm_f16";
   template <class X, class W, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, W& w, O& out, float eps) {
     auto xa = input_arg(x), wa = input_arg(w);
@@ -394,6 +533,7 @@ struct RmsNormF16Fn {
   }
 };
 struct RmsNormF32Fn {
+  static constexpr const char* name = "rms_norm";
   template <class X, class W, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, W& w, O& out, float eps) {
     auto xa = input_arg(x), wa = input_arg(w);
@@ -402,6 +542,7 @@ struct RmsNormF32Fn {
   }
 };
 struct SoftmaxFn {
+  static constexpr const char* name = "softmax";
   template <class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, Yv& y) {
     auto xa = input_arg(x);
@@ -411,6 +552,7 @@ struct SoftmaxFn {
 };
 template <bool Accumulate>
 struct GemmFn {
+  static constexpr const char* name = "gemm";
   template <class Z, class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, int32_t k) {
     auto zp = z.arg();
@@ -420,6 +562,7 @@ struct GemmFn {
 };
 template <bool Causal>
 struct FmhaFn {
+  static constexpr const char* name = "fmha";
   // fmha(out, q, k, v, qk_scale, input_pos, query_group_size) — flash_attention_causal.rs:32-40
   template <class O, class Q, class K, class V>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, O& out, Q& q, K& k, V& v, float scale,
@@ -430,6 +573,7 @@ struct FmhaFn {
   }
 };
 struct LinearTileMxfp8Fn {
+  static constexpr const char* name = "linear_tile";
   template <class Z, class X, class Yv, class XS, class YS>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, XS& xs, YS& ys, float alpha) {
     auto zp = z.arg();
@@ -441,6 +585,7 @@ struct LinearTileMxfp8Fn {
 };
 // ---- transformer-block kernels (cutile-kernels/src/{norms,pointwise,positional}.rs) ----
 struct AddRmsNormF16Fn {
+  static constexpr const char* name = "add_rms_norm_f16";
   template <class R, class X, class W, class O, class RO>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, R& residual, X& x, W& w, O& out, RO& residual_out, float eps) {
     auto ra = input_arg(residual), xa = input_arg(x), wa = input_arg(w);
@@ -449,6 +594,7 @@ struct AddRmsNormF16Fn {
   }
 };
 struct QkNormF16Fn {
+  static constexpr const char* name = "qk_norm_f16";
   template <class Q, class K, class QW, class KW, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, QW& qw, KW& kw, O& out, float eps, int32_t num_q_rows) {
     auto qa = input_arg(q), ka = input_arg(k), qwa = input_arg(qw), kwa = input_arg(kw);
@@ -458,6 +604,7 @@ struct QkNormF16Fn {
 };
 template <bool Silu>
 struct Pointwise2dF16Fn {
+  static constexpr const char* name = Silu ? "silu_mul_2d_f16" : "add_2d_f16";
   template <class O, class A, class B>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, O& out, A& a, B& b) {
     auto op = out.arg();
@@ -466,6 +613,7 @@ struct Pointwise2dF16Fn {
   }
 };
 struct RopeSeqF16Fn {
+  static constexpr const char* name = "rope_seq_f16";
   template <class X, class F, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, F& inv_freq, O& out, int32_t position_start) {
     auto xa = input_arg(x), fa = input_arg(inv_freq);
@@ -474,6 +622,7 @@ struct RopeSeqF16Fn {
   }
 };
 struct RopeSeqDynposF16Fn {
+  static constexpr const char* name = "rope_seq_dynpos_f16";
   template <class X, class F, class P, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, F& inv_freq, P& position_start, O& out) {
     auto xa = input_arg(x), fa = input_arg(inv_freq), pa = input_arg(position_start);
@@ -482,6 +631,7 @@ struct RopeSeqDynposF16Fn {
   }
 };
 struct QkRopeDynposF16Fn {
+  static constexpr const char* name = "qk_rope_dynpos_f16";
   template <class Q, class K, class F, class P, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, F& inv_freq, P& position_start, O& out, int32_t num_q_heads) {
     auto qa = input_arg(q), ka = input_arg(k), fa = input_arg(inv_freq), pa = input_arg(position_start);
@@ -490,6 +640,7 @@ struct QkRopeDynposF16Fn {
   }
 };
 struct KvCacheUpdateSeqF16Fn {
+  static constexpr const char* name = "kv_cache_update_seq_f16";
   template <class NK, class NV, class KC, class VC>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, NK& new_k, NV& new_v, KC& k_cache, VC& v_cache, int32_t position_start, int32_t seq_len) {
     auto ka = input_arg(new_k), va = input_arg(new_v);
@@ -498,6 +649,7 @@ struct KvCacheUpdateSeqF16Fn {
   }
 };
 struct KvCacheUpdateSeqDynposF16Fn {
+  static constexpr const char* name = "kv_cache_update_seq_dynpos_f16";
   template <class NK, class NV, class KC, class VC, class P>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, NK& new_k, NV& new_v, KC& k_cache, VC& v_cache, P& position_start, int32_t seq_len) {
     auto ka = input_arg(new_k), va = input_arg(new_v), pa = input_arg(position_start);
@@ -506,6 +658,7 @@ struct KvCacheUpdateSeqDynposF16Fn {
   }
 };
 struct FmhaDecodeGqaSplitFn {
+  static constexpr const char* name = "fmha_decode_gqa_split";
   template <class Q, class K, class V, class A, class L, class P>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, A& att_out, L& lse_out, float qk_scale, P& position_start) {
     auto qa = input_arg(q), ka = input_arg(k), va = input_arg(v), pa = input_arg(position_start);
@@ -514,6 +667,7 @@ struct FmhaDecodeGqaSplitFn {
   }
 };
 struct SplitkReduceMergeFn {
+  static constexpr const char* name = "splitk_reduce_merge";
   template <class A, class L, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, A& att_partial, L& lse_partial, O& out) {
     auto aa = input_arg(att_partial), la = input_arg(lse_partial);
@@ -522,6 +676,7 @@ struct SplitkReduceMergeFn {
   }
 };
 struct GroupGemmF16NtDescFn {
+  static constexpr const char* name = "group_gemm_f16_nt_desc";
   template <class AP, class BP, class CP, class AM, class BM_, class CM>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, AP& a_ptrs, BP& b_ptrs, CP& c_ptrs, AM& a_metas,
                                 BM_& b_metas, CM& c_metas, int32_t num_groups) {
@@ -531,6 +686,7 @@ struct GroupGemmF16NtDescFn {
   }
 };
 struct ArgmaxBlocksF16Fn {
+  static constexpr const char* name = "argmax_blocks_f16";
   template <class L, class M, class I>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, L& logits, M& block_max, I& block_idx, int32_t len) {
     auto la = input_arg(logits);
@@ -539,6 +695,7 @@ struct ArgmaxBlocksF16Fn {
   }
 };
 struct LmHeadArgmaxBlocksF16Fn {
+  static constexpr const char* name = "lm_head_argmax_blocks_f16";
   template <class W, class H, class M, class I>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, W& weights, H& hidden, M& block_max, I& block_idx, int32_t vocab_size) {
     auto wa = input_arg(weights), ha = input_arg(hidden);
@@ -547,6 +704,7 @@ struct LmHeadArgmaxBlocksF16Fn {
   }
 };
 struct ArgmaxReduceBlocksToU32Fn {
+  static constexpr const char* name = "argmax_reduce_blocks_to_u32";
   template <class M, class I, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, M& block_max, I& block_idx, O& out, int32_t num_blocks) {
     auto ma = input_arg(block_max), ia = input_arg(block_idx);
@@ -555,6 +713,7 @@ struct ArgmaxReduceBlocksToU32Fn {
   }
 };
 struct EmbeddingBatchF16Fn {
+  static constexpr const char* name = "embedding_batch_f16";
   template <class I, class T, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, I& token_ids, T& table, O& out) {
     auto ia = input_arg(token_ids), ta = input_arg(table);
@@ -563,6 +722,7 @@ struct EmbeddingBatchF16Fn {
   }
 };
 struct GatherRowF16Fn {
+  static constexpr const char* name = "gather_row_f16";
   template <class S, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, S& src, O& out, int32_t row_idx) {
     auto sa = input_arg(src);
@@ -573,6 +733,7 @@ struct GatherRowF16Fn {
 // The five sequence-layout attention kernels share one C entry point (cutile_launch_fmha_seq_f16).
 template <bool Causal>
 struct SeqAttentionFn {          // kv_len and query_start by value
+  static constexpr const char* name = "fmha_prefill_causal";
   template <class Q, class K, class V, class O>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, O& out, float qk_scale,
                                 int32_t query_group_size, int32_t kv_len, int32_t query_start) {
@@ -583,6 +744,7 @@ struct SeqAttentionFn {          // kv_len and query_start by value
 };
 template <bool Causal, bool KvLenFromPosition>
 struct SeqAttentionDynposFn {    // the position in device memory
+  static constexpr const char* name = "fmha_causal";
   template <class Q, class K, class V, class O, class P>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Q& q, K& k, V& v, O& out, float qk_scale,
                                 int32_t query_group_size, P& position_start) {
@@ -592,6 +754,7 @@ struct SeqAttentionDynposFn {    // the position in device memory
   }
 };
 struct GemmPersistentFn {
+  static constexpr const char* name = "gemm_persistent";
   template <class Z, class X, class Yv>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y) {
     auto zm = z.arg();
@@ -600,6 +763,7 @@ struct GemmPersistentFn {
   }
 };
 struct MappedTileIndexFn {
+  static constexpr const char* name = "mapped_tile_index";
   template <class Z>
   static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z) {
     auto zm = z.arg();

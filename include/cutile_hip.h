@@ -303,6 +303,18 @@ typedef struct {
   const char* variant;              /* NULL = library's choice */
 } cutile_launch_opts_t;
 
+/* Launch modes of the generated launcher — cutile-macro/src/_module.rs:852-900.  `.compile()` / `.compile_on()` run a
+ * launcher with its launch block skipped (_compile_only): arguments are validated, the kernel is resolved and its code
+ * object loaded on the device, nothing is enqueued.  `.specialize()` resolves the launch's identity without compiling
+ * or launching.  Here a mode is a property of the calling thread: 0 = launch, 1 = compile only (validate, resolve,
+ * load), 2 = specialize only (validate, resolve; nothing is loaded).  The C++ surface sets it around one launcher call
+ * and restores 0. */
+cutile_status_t cutile_set_launch_mode(int32_t mode);
+cutile_status_t cutile_get_launch_mode(int32_t* mode);
+/* The kernel the calling thread's last launcher call resolved: its table name and the same record cutile_kernel_lookup
+ * fills (`function` is NULL after a specialize-only call: nothing was loaded). */
+cutile_status_t cutile_last_resolved_kernel(const char** function, cutile_kernel_info_t* info);
+
 /* Partition::grid — cutile/src/tensor.rs:447-468 */
 cutile_status_t cutile_partition_grid(const cutile_partition_arg_t* p, uint32_t grid[3]);
 /* infer_launch_grid over the bounds of all partition arguments —

@@ -261,6 +261,116 @@ TEST(launchers_hand_arguments_back_in_the_form_given) {
   CHECK(wrong.is_err() && wrong.error().message.find("does not match the inferred partition grid") != std::string::npos);
 }
 
+// ---- cache-key identity: cutile/tests/warmup.rs, case by case -------------------------------------------------
+static TileFunctionKeyBuilder default_key() {
+  return TileFunctionKey::builder("m", "f").source_hash("hash").gpu_name("gfx950").compiler_version("0.0.1").toolchain_fingerprint(
+      "AMD clang version 20.0.0");
+}
+TEST(tile_function_key_distinguishes_everything_that_selects_a_kernel) {
+  // cache_key_deterministic
+  auto k1 = TileFunctionKey::builder("mod", "fn").generics({"f32"}).source_hash("abc123").gpu_name("gfx950").compiler_version("0.0.1-alpha")
+                .toolchain_fingerprint("AMD clang version 20.0.0").build();
+  auto k2 = k1;
+  CHECK(k1 == k2 && k1.display_hash() == k2.display_hash());
+  // different source hash / gpu name / device id / compiler version / toolchain fingerprint / generics
+  CHECK(default_key().source_hash("hash_v1").build() != default_key().source_hash("hash_v2").build());
+  CHECK(default_key().gpu_name("gfx942").build() != default_key().gpu_name("gfx950").build());
+  CHECK(default_key().device_id(0).build() != default_key().device_id(1).build());
+  CHECK(default_key().compiler_version("0.0.1").build() != default_key().compiler_version("0.0.2").build());
+  CHECK(default_key().toolchain_fingerprint("AMD clang version 19.0.0").build() != default_key().toolchain_fingerprint("AMD clang version 20.0.0").build());
+  // the stat-style fallback fingerprint (embedded NULs) must not collide with a version string
+  CHECK(default_key().toolchain_fingerprint(std::string("stat\0/opt/rocm/bin/hipcc\094855128\0170000000", 44)).build() !=
+        default_key().toolchain_fingerprint("AMD clang version 20.0.0").build());
+  CHECK(default_key().generics({"f32"}).build() != default_key().generics({"f16"}).build());
+  // cache_key_different_spec_args
+  SpecializationBits aligned, misaligned;
+  aligned.shape_div = {DivHint::from_value(16), DivHint::from_value(16)};
+  aligned.stride_div = {DivHint::from_value(16), DivHint::from_value(16)};
+  aligned.stride_one = {false, true};
+  aligned.base_ptr_div = DivHint::from_ptr(16);
+  misaligned = aligned;
+  misaligned.shape_div = {DivHint::from_value(4), DivHint::from_value(4)};
+  misaligned.stride_div = {DivHint::from_value(4), DivHint::from_value(4)};
+  misaligned.base_ptr_div = DivHint::from_ptr(4);
+  CHECK(DivHint::from_value(16).divisor == 16 && DivHint::from_value(48).divisor == 16 && DivHint::from_value(12).divisor == 4 &&
+        DivHint::from_value(7).divisor == 1 && DivHint::from_ptr(0x7f0000001008ull).divisor == 8 && DivHint::from_value(64).with_max(8).divisor == 8);
+  CHECK(default_key().spec_args({{"x", aligned}}).build() != default_key().spec_args({{"x", misaligned}}).build());
+  // cache_key_different_compile_options
+  CHECK(default_key().compile_options(CompileOptions().max_divisibility(8)).build() != default_key().compile_options(CompileOptions().max_divisibility(16)).build());
+  CHECK(default_key().compile_options(CompileOptions().occupancy(2)).build() != default_key().compile_options(CompileOptions().occupancy(4)).build());
+  CHECK(default_key().compile_options(CompileOptions().num_worker_warps_per_cta(4)).build() !=
+        default_key().compile_options(CompileOptions().num_worker_warps_per_cta(8)).build());
+  CHECK(default_key().compile_options(CompileOptions().occupancy(2)).build() != default_key().build());
+  // cache_key_no_field_boundary_ambiguity: also in the digest's input
+  auto ka = default_key().gpu_name("sm_9").compiler_version("0").build(), kb = default_key().gpu_name("sm_90").compiler_version("").build();
+  CHECK(ka != kb && ka.canonical() != kb.canonical());
+  // a constant grid is part of the key, a plain grid is not there at all
+  CHECK(default_key().grid(4, 1, 1).build() != default_key().build() && default_key().grid(4, 1, 1).build() != default_key().grid(8, 1, 1).build());
+}
+
+TEST(launcher_compile_specialize_and_cache_keys) {
+  // .compile() / .compile_on() / .specialize() / .l1_cache_key() / .l2_cache_key() / .const_grid() / .compile_options() / _apply
+  // (cutile-macro/src/_module.rs:852-923, kernel_launcher_generator.rs:1036-1044)
+  auto s = fresh_stream();
+  auto z = [&] { return partition_op(api::zeros<bf16>({256, 256}), {128, 128}); };
+  auto x = api::zeros<bf16>({256, 64}).sync_on(s).unwrap();
+  auto y = api::zeros<bf16>({64, 256}).sync_on(s).unwrap();
+  // specialize: the identity, nothing loaded, nothing launched
+  uint64_t loads0 = cutile_module_load_count();
+  int n0 = launches();
+  auto spec = gemm(z(), &x, &y, 64).generics({"bf16", "128", "128", "64"}).specialize_on(s).unwrap();
+  CHECK(launches() == n0 + 1);                                   // the fill of z ran; the kernel did not
+  CHECK(spec.l1_cache_key().function_name() == "gemm" && spec.variant() == "bf16_128x128x64_d2x2" && spec.symbol() == "gemm_entry__bf16_128x128x64_d2x2");
+  CHECK(spec.l1_cache_key().function_generics == std::vector<std::string>({"bf16", "128", "128", "64"}));
+  CHECK(spec.l1_cache_key().spec_args.size() == 3 && spec.l1_cache_key().scalar_hints.size() == 1 && spec.l1_cache_key().scalar_hints[0].second.divisor == 16);
+  CHECK(spec.l1_cache_key().gpu_name().find("gfx") == 0 && !spec.l1_cache_key().source_hash().empty() && !spec.l1_cache_key().grid);
+  CHECK(spec.l2_cache_key().find("gemm:bf16_128x128x64_d2x2:") == 0);
+  // compile: the code object is loaded now ...
+  uint64_t loads1 = cutile_module_load_count();
+  int n1 = launches();
+  CHECK(gemm(z(), &x, &y, 64).compile_on(s).is_ok());
+  CHECK(launches() == n1 + 1 && cutile_module_load_count() >= loads1);
+  uint64_t loads2 = cutile_module_load_count();
+  // ... so the first launch after it loads nothing
+  CHECK(gemm(z(), &x, &y, 64).sync_on(s).is_ok() && last_symbol() == "gemm_entry__bf16_128x128x64_d2x2");
+  CHECK(cutile_module_load_count() == loads2 && launches() == n1 + 3);
+  (void)loads0;
+  // compile reports what a launch would: validation still runs
+  auto bad = gemm(z(), &x, &y, 64).generics({"bf16", "64", "128", "64"}).compile_on(s);
+  CHECK(bad.is_err() && bad.error().message.find("generic BM") != std::string::npos);
+  int32_t mode = -1;
+  CHECK(cutile_get_launch_mode(&mode) == CUTILE_SUCCESS && mode == 0);        // the mode never leaks out of a call
+  // keys: equal for equal launches whatever the extents, different for a misaligned view / options / const grid
+  auto key = [&](auto launcher) { return std::move(launcher).l1_cache_key_on(s).unwrap(); };
+  auto base = key(gemm(z(), &x, &y, 64));
+  CHECK(base == key(gemm(z(), &x, &y, 64)));
+  auto x_big = api::zeros<bf16>({512, 64}).sync_on(s).unwrap();
+  auto z_big = [&] { return partition_op(api::zeros<bf16>({512, 256}), {128, 128}); };
+  CHECK(base == key(gemm(z_big(), &x_big, &y, 64)));                          // extents are not part of the key
+  CHECK(base != key(gemm(z(), &x, &y, 64).compile_options(CompileOptions().occupancy(2))));
+  CHECK(base != key(gemm(z(), &x, &y, 64).const_grid(2, 2, 1)));
+  CHECK(base == key(gemm(z(), &x, &y, 64).grid(2, 2, 1)));                    // a plain grid is a launch parameter only
+  CHECK(key(gemm(z(), &x, &y, 64).const_grid(2, 2, 1)) == key(gemm(z(), &x, &y, 64).const_grid(2, 2, 1)));
+  auto wide = api::zeros<bf16>({256, 72}).sync_on(s).unwrap();
+  auto x_view = wide.slice({{0, 256}, {8, 72}}).unwrap();                    // same shape as x, row stride 72, base 16 bytes in
+  auto misaligned = key(gemm(z(), x_view, &y, 64));
+  CHECK(base != misaligned && misaligned.spec_args[1].second.stride_div[0].divisor == 8);
+  CHECK(key(gemm(z(), &x, &y, 64).compile_options(CompileOptions().max_divisibility(4))).spec_args[1].second.stride_div[0].divisor == 4);
+  // l2 key names the resolved kernel; a launch that resolves to another variant has another key
+  auto l2a = gemm(z(), &x, &y, 64).l2_cache_key_on(s).unwrap();
+  auto l2b = gemm(z(), &x, &y, 64).variant("bf16_128x128x64_w2x2").l2_cache_key_on(s).unwrap();
+  CHECK(l2a != l2b && l2b.find("gemm:bf16_128x128x64_w2x2:") == 0);
+  // default-stream forms
+  CHECK(gemm(z(), &x, &y, 64).compile().is_ok() && gemm(z(), &x, &y, 64).l1_cache_key().unwrap() == base);
+  CHECK(gemm(z(), &x, &y, 64).get_launch_grid() == (std::array<uint32_t, 3>{0, 0, 0}) &&
+        gemm(z(), &x, &y, 64).const_grid(2, 2, 1).get_launch_grid() == (std::array<uint32_t, 3>{2, 2, 1}));
+  // _apply: a launcher over a tuple of materialised arguments
+  auto yv = api::ones<float>({32}).sync_on(s).unwrap();
+  auto xv = std::make_shared<Tensor<float>>(api::ones<float>({32}).sync_on(s).unwrap());
+  auto out = apply_launcher<kernels::SaxpyFn>(std::make_tuple(std::move(yv).partition({8}), 2.0f, xv)).sync_on(s).unwrap();
+  CHECK(last_symbol() == "saxpy_entry__f32_r1_flat" && std::get<2>(out).get() == xv.get());
+}
+
 TEST(mapped_partitions_validate_and_hand_the_inner_partition_back) {
   auto s = fresh_stream();
   cutile_testing_clear_log();
