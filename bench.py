@@ -895,9 +895,11 @@ def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np, flush):
                      "protocol": "median of per-launch HIP-event times, 512 MiB cache flush before each",
                      "algorithmic_work": w.work},
     }
-    chosen = getattr(w, "variant_source", None)
-    if chosen:
-        rec["config"] = dict(rec["config"], **chosen)
+    try:      # which precompiled variant ran, and whether a tuning record, a pin or the table's order chose it
+        got = ct.last_resolved()
+        rec["kernel"] = {"variant": got["variant"], "chosen_by": got["source"], "shape_class": got["bucket"]}
+    except ct.CutileError:
+        pass
     if with_cpu:
         res = w.cpu_baseline(oracle, np, torch)
         if res:
@@ -1051,7 +1053,10 @@ def main():
         "vs_baseline": None, "dtype": h["dtype"], "data": "synthetic (seeded host PRNG, same bytes fed to the CPU oracle)",
         "config": h["config"], "roofline": h["roofline"],
         "device": ct.device_arch(0),
+        "tuning_records": ct.tuning_report().strip().splitlines(),
     }
+    if "kernel" in h:
+        line["kernel"] = h["kernel"]
     if "cpu_baseline" in h:
         line["cpu_baseline"] = h["cpu_baseline"]
         line["parity"] = h["parity"]

@@ -748,6 +748,40 @@ def set_preferred_variant(function: str, variant: Optional[str]) -> None:
     check(lib().cutile_kernel_set_preferred_variant(function.encode(), variant.encode() if variant else None))
 
 
+def set_preferred_variant_for(function: str, bucket: str, variant: Optional[str]) -> None:
+    check(lib().cutile_kernel_set_preferred_variant_for(function.encode(), bucket.encode(), variant.encode() if variant else None))
+
+
+def tuning_reload(directory: Optional[str] = None) -> str:
+    """drop the applied tuning records and load `directory` (None = the directory beside the library); returns the report"""
+    check(lib().cutile_tuning_reload(directory.encode() if directory is not None else None))
+    return tuning_report()
+
+
+def tuning_report() -> str:
+    L = lib()
+    L.cutile_tuning_report.restype = C.c_char_p
+    return L.cutile_tuning_report().decode()
+
+
+def last_resolved() -> dict:
+    """what the calling thread's last launcher call resolved: kernel, variant, where the choice came from, its shape class"""
+    L = lib()
+    L.cutile_last_resolved_source.restype = C.c_char_p
+    L.cutile_last_resolved_bucket.restype = C.c_char_p
+    fn = C.c_char_p()
+    info = KernelInfo()
+    check(L.cutile_last_resolved_kernel(C.byref(fn), C.byref(info)))
+    return {"function": fn.value.decode(), "variant": info.variant.decode(), "symbol": info.symbol.decode(),
+            "source": L.cutile_last_resolved_source().decode(), "bucket": L.cutile_last_resolved_bucket().decode()}
+
+
+def kernel_fingerprint(function: str, variant: Optional[str] = None) -> str:
+    buf = C.create_string_buffer(17)
+    check(lib().cutile_kernel_fingerprint(function.encode(), variant.encode() if variant else None, buf))
+    return buf.value.decode()
+
+
 def device(ordinal: int = 0) -> int:
     d = C.c_void_p()
     check(lib().cutile_device_get(ordinal, C.byref(d)))

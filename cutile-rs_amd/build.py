@@ -35,7 +35,7 @@ IMAGES = {
     "nvfp4": "nvfp4_gemm.hip",
     "rng": "rng.hip",
 }
-HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp"]
+HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp", "tuning.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")
@@ -148,6 +148,7 @@ CPP_TESTS = {
     # binary -> (source, needs the library, extra flags)
     "test_host_surface": ("test_host_surface.cpp", True, []),
     "test_gpu_surface": ("test_gpu_surface.cpp", True, []),
+    "write_record": ("write_record.cpp", True, []),
     "test_slot_table": ("test_slot_table.cpp", False, []),
     "test_slot_table_tsan": ("test_slot_table.cpp", False, ["-fsanitize=thread"]),
 }
@@ -177,8 +178,23 @@ def build_cpp_tests(force: bool = False) -> str:
     return out_dir
 
 
+def build_tuner(force: bool = False) -> str:
+    """The program that writes the tuning records (cutile-rs_amd/tune/tune_baseline.cpp -> cutile-rs_amd/bin/)."""
+    out_dir = os.path.join(ROOT, "bin")
+    os.makedirs(out_dir, exist_ok=True)
+    include = os.path.join(ROOT, "..", "include")
+    src = os.path.join(ROOT, "tune", "tune_baseline.cpp")
+    dst = os.path.join(out_dir, "tune_baseline")
+    deps = [src, LIB_PATH] + [os.path.join(include, "cutile", f) for f in os.listdir(os.path.join(include, "cutile"))]
+    if force or not _newer(dst, deps):
+        _run([CXX, "-std=c++17", "-O1", "-g0", "-I" + include, "-Wall", "-Wextra", "-Wno-unused-parameter", src, "-o", dst, "-pthread",
+              "-L" + LIB_DIR, "-lcutile_hip", "-Wl,-rpath,$ORIGIN/../lib"])
+    return dst
+
+
 def build(force: bool = False) -> str:
     lib = build_host_library(build_code_objects(force), force)
+    build_tuner(force)
     build_scratch_library(force)
     build_probes(force)
     build_cpp_tests(force)

@@ -26,6 +26,8 @@ namespace {
 std::atomic<uint64_t> g_module_loads{0};
 std::mutex g_pref_mutex;
 std::map<std::string, std::string> g_preferred;
+// winners of tuning records: "function|bucket" -> variant
+std::map<std::string, std::string> g_bucket_preferred;
 
 struct ImageRef {
   const unsigned char* start;
@@ -308,6 +310,18 @@ std::string preferred_variant(const char* function) {
   return it == g_preferred.end() ? std::string() : it->second;
 }
 
+std::string preferred_variant_for(const char* function, const std::string& bucket) {
+  if (bucket.empty()) return std::string();
+  std::lock_guard<std::mutex> lock(g_pref_mutex);
+  auto it = g_bucket_preferred.find(std::string(function) + "|" + bucket);
+  return it == g_bucket_preferred.end() ? std::string() : it->second;
+}
+
+void clear_bucket_preferences() {
+  std::lock_guard<std::mutex> lock(g_pref_mutex);
+  g_bucket_preferred.clear();
+}
+
 void count_module_load() { g_module_loads.fetch_add(1, std::memory_order_relaxed); }
 
 cutile_status_t load_entry(cutile_device_t device, const KernelEntry* entry, hipFunction_t* fn) {
@@ -374,6 +388,20 @@ cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const 
                  "no variant '%s' of kernel '%s'; available: %s", variant, function,
                  list_variants(function).c_str());
   g_preferred[function] = variant;
+  return CUTILE_SUCCESS;
+}
+
+cutile_status_t cutile_kernel_set_preferred_variant_for(const char* function, const char* bucket, const char* variant) {
+  CUTILE_REQUIRE(function && bucket && *bucket, CUTILE_ERR_INVALID_ARGUMENT, "function or bucket is null");
+  std::lock_guard<std::mutex> lock(g_pref_mutex);
+  const std::string key = std::string(function) + "|" + bucket;
+  if (!variant) {
+    g_bucket_preferred.erase(key);
+    return CUTILE_SUCCESS;
+  }
+  CUTILE_REQUIRE(find_entry(function, variant) != nullptr, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "no variant '%s' of kernel '%s'; available: %s", variant, function, list_variants(function).c_str());
+  g_bucket_preferred[key] = variant;
   return CUTILE_SUCCESS;
 }
 

@@ -35,6 +35,11 @@ const KernelEntry* find_entry(const char* function, const std::string& variant);
 cutile_status_t load_entry(cutile_device_t device, const KernelEntry* entry, hipFunction_t* fn);
 // Preferred variant set through cutile_kernel_set_preferred_variant, or "".
 std::string preferred_variant(const char* function);
+// Winner a tuning record names for (function, shape-class bucket), or "".
+std::string preferred_variant_for(const char* function, const std::string& bucket);
+void clear_bucket_preferences();
+// Loads the tuning records once per process (tuning.cpp); cheap afterwards.
+void ensure_tuning_records_loaded();
 // Human-readable list of variants of `function`, for error messages.
 std::string list_variants(const char* function);
 

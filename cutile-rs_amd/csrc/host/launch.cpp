@@ -138,6 +138,16 @@ struct ArgPacker {
 // What the calling thread's next launcher calls do once their checks have passed (cutile_set_launch_mode), and the
 // table entry the thread's last launcher call resolved (cutile_last_resolved_kernel).
 thread_local int g_launch_mode = 0;
+// Shape class of the launch being resolved (set by the launchers that tuning records cover) and where the last
+// resolved variant came from: "caller" (opts.variant), "record:<bucket>" (a verified tuning record), "pinned"
+// (cutile_kernel_set_preferred_variant) or "table" (the table's order).
+thread_local std::string g_bucket;
+thread_local std::string g_last_source;
+thread_local std::string g_last_bucket;
+struct BucketScope {
+  explicit BucketScope(std::string b) { g_bucket = std::move(b); }
+  ~BucketScope() { g_bucket.clear(); }
+};
 thread_local const KernelEntry* g_last_entry = nullptr;
 thread_local hipFunction_t g_last_fn = nullptr;
 
@@ -248,12 +258,28 @@ cutile_status_t resolve_grid(const cutile_partition_arg_t* out, const cutile_lau
 cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* opts, const std::string& fallback,
                               const std::vector<std::string>& acceptable, Resolved* r) {
   std::string want;
+  g_last_source = "caller";
+  g_last_bucket = g_bucket;
   if (opts && opts->variant) want = opts->variant;
+  if (want.empty() && !g_bucket.empty()) {
+    ensure_tuning_records_loaded();
+    std::string pref = preferred_variant_for(function, g_bucket);
+    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) {
+      want = pref;
+      g_last_source = "record:" + g_bucket;
+    }
+  }
   if (want.empty()) {
     std::string pref = preferred_variant(function);
-    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) want = pref;
+    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) {
+      want = pref;
+      g_last_source = "pinned";
+    }
   }
-  if (want.empty()) want = fallback;
+  if (want.empty()) {
+    want = fallback;
+    g_last_source = "table";
+  }
   if (!acceptable.empty() && std::find(acceptable.begin(), acceptable.end(), want) == acceptable.end()) {
     std::string list;
     for (auto& a : acceptable) list += (list.empty() ? "" : ", ") + a;
@@ -273,6 +299,13 @@ cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* 
 }
 
 uint32_t div_up(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
+
+// Shape classes of tuning records: row lengths by the next power of two (at least 256).
+std::string pow2_class(int64_t n) {
+  int64_t p = 256;
+  while (p < n) p *= 2;
+  return "<=" + std::to_string(p);
+}
 
 const char* float_dtype_name(cutile_dtype_t dt) { return kDTypes[dt].name; }
 
@@ -509,6 +542,7 @@ static cutile_status_t launch_elementwise3(const char* fn_name, cutile_stream_t 
   CUTILE_REQUIRE(!acceptable.empty(), CUTILE_ERR_KERNEL_NOT_FOUND, "no precompiled variant of %s<%s> for rank %d; available: %s",
                  fn_name, dt.c_str(), rank, list_variants(fn_name).c_str());
   Resolved res;
+  BucketScope bucket(dt + r);
   if (cutile_status_t s = resolve_entry(fn_name, opts, acceptable[0], acceptable, &res)) return s;
 
   ArgPacker args;
@@ -704,6 +738,7 @@ cutile_status_t cutile_launch_rms_norm_f16(cutile_stream_t stream, const cutile_
   if (vec_ok) acceptable = fitting_row_variants("rms_norm_f16", "", n);
   acceptable.push_back("generic");
   Resolved res;
+  BucketScope bucket("n" + pow2_class(n));
   if (cutile_status_t s = resolve_entry("rms_norm_f16", opts, acceptable[0], acceptable, &res)) return s;
 
   ArgPacker args;
@@ -1603,6 +1638,7 @@ cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tenso
   if (vec_ok) acceptable = fitting_row_variants("softmax", dt + "_w", bn);
   acceptable.push_back(dt + "_generic");
   Resolved res;
+  BucketScope bucket(dt + "|bn" + pow2_class(bn));
   if (cutile_status_t s = resolve_entry("softmax", opts, acceptable[0], acceptable, &res)) return s;
   ArgPacker args;
   args.push_tensor(*x);
@@ -1657,6 +1693,8 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
         acceptable.push_back(e.variant);
   acceptable.push_back(dt + "_generic");
   Resolved res;
+  // shape class for tuning records: the tile, and whether the tiles fit one wave of workgroups over the 256 CUs
+  BucketScope bucket(dt + "_" + std::to_string(bm) + "x" + std::to_string(bn) + ((uint64_t)tg[0] * tg[1] <= 256 ? "|tiles<=256" : "|tiles>256"));
   if (cutile_status_t s = resolve_entry("gemm", opts, acceptable[0], acceptable, &res)) return s;
   ArgPacker args;
   args.push_partition(*z);
@@ -2059,6 +2097,7 @@ cutile_status_t cutile_launch_fmha(cutile_stream_t stream, const cutile_partitio
                  "no precompiled variant of fmha<%s, BM=%d, D=%d>; available: %s", dt.c_str(), bm, d,
                  list_variants("fmha").c_str());
   Resolved res;
+  BucketScope bucket(dt + "_bm" + std::to_string(bm) + "_d" + std::to_string(d) + (causal ? "|causal" : "|full"));
   if (cutile_status_t s = resolve_entry("fmha", opts, same_bn.empty() ? acceptable[0] : same_bn[0], acceptable, &res)) return s;
   ArgPacker args;
   args.push_partition(*out);
@@ -2292,6 +2331,7 @@ cutile_status_t cutile_launch_linear_tile_mxfp8(cutile_stream_t stream, const cu
                  "no precompiled variant of linear_tile<%d, %d, %d, %d> -> %s; available: %s", bm, bn, bk_user,
                  bk_user / 32, dt.c_str(), list_variants("linear_tile").c_str());
   Resolved res;
+  BucketScope bucket("mxfp8_" + dt + "_" + std::to_string(bm) + "x" + std::to_string(bn));
   if (cutile_status_t s = resolve_entry("linear_tile", opts, acceptable[0], acceptable, &res)) return s;
   uint32_t kg[3] = {tg[0], tg[1], 1};
   if (res.entry->tile[0] != bm || res.entry->tile[1] != bn) {
@@ -2490,6 +2530,8 @@ cutile_status_t cutile_get_launch_mode(int32_t* mode) {
   *mode = g_launch_mode;
   return CUTILE_SUCCESS;
 }
+const char* cutile_last_resolved_source(void) { return g_last_source.c_str(); }
+const char* cutile_last_resolved_bucket(void) { return g_last_bucket.c_str(); }
 cutile_status_t cutile_last_resolved_kernel(const char** function, cutile_kernel_info_t* info) {
   CUTILE_REQUIRE(function && info, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
   CUTILE_REQUIRE(g_last_entry, CUTILE_ERR_STATE, "no launcher call has resolved a kernel on this thread yet");

@@ -228,6 +228,24 @@ int32_t cutile_kernel_list(const char** names, int32_t cap);
  * several fit (the autotuner's output).  variant == NULL restores the default. */
 cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const char* variant);
 
+/* The same per shape class: `bucket` names the class a launcher derives from its arguments (what
+ * cutile_last_resolved_bucket reports after a launch, e.g. "bf16_256x256|tiles>256" for gemm).  This is how the winners of
+ * verified tuning records reach the launchers; order of precedence at a launch: the caller's variant, the bucket's
+ * winner, the function-wide pin, the table's order. */
+cutile_status_t cutile_kernel_set_preferred_variant_for(const char* function, const char* bucket, const char* variant);
+/* Tuning records (cutile/src/tune.rs:762-1016): JSON records of autotuner winners, one file per kernel, in the directory
+ * `tuned` beside the library (or $CUTILE_TUNING_RECORDS; empty = none), loaded on the first launcher call.  A record is
+ * applied only if Record::load_verified accepts it against the running library (schema, kernel, architecture,
+ * code-object fingerprint, every winner's variant fingerprint, same device toolchain); anything else is refused as a
+ * whole and said so in the report.  cutile_tuning_reload(dir) drops what was applied and loads `dir` (NULL = default). */
+cutile_status_t cutile_tuning_reload(const char* directory);
+const char* cutile_tuning_report(void);           /* one line per file: applied / refused / warning; valid until the thread's next call */
+int32_t cutile_tuning_applied_count(void);        /* buckets with a winner from a record */
+/* Where the calling thread's last launcher call took its variant from: "caller", "record:<bucket>", "pinned" or "table";
+ * and the shape class that call was filed under ("" for launchers without classes). */
+const char* cutile_last_resolved_source(void);
+const char* cutile_last_resolved_bucket(void);
+
 /* Provenance of the running library, for records of tuning winners (cutile/src/tune.rs:762-832 keeps
  * source_hash, toolchain fingerprint, arch and crate version; here they come from the kernel table):
  * the library version, the device compiler's version text captured at build time, the one target

@@ -9,10 +9,13 @@ import pytest
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
 
 
-def _run(name, timeout=300):
+def _run(name, timeout=300, records=False):
     path = os.path.join(BIN, name)
     assert os.path.exists(path), f"{path} is missing: run python cutile-rs_amd/build.py"
-    res = subprocess.run([path], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+    env = dict(os.environ)
+    if not records:
+        env["CUTILE_TUNING_RECORDS"] = ""     # variant choices these programs assert are the table's own, not a tuning record's
+    res = subprocess.run([path], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout, env=env)
     tail = "\n".join(res.stdout.splitlines()[-25:])
     assert res.returncode == 0 and "TESTS PASSED" in res.stdout, tail
     return res.stdout

@@ -420,3 +420,63 @@ def test_rng_fills_on_the_recording_runtime(fake_hip):
     with pytest.raises(ValueError):
         rng.uniform_(torch.zeros(4, dtype=torch.float16))
     rng.close()
+
+
+def test_tuning_records_choose_variants_per_shape_class_and_stale_ones_are_refused(fake_hip, tmp_path):
+    """cutile/src/tune.rs:762-1016 applied at start-up: a verified record's winner is what a launch of its shape class
+    uses; without the record the table's order decides; a record whose provenance is stale is refused as a whole."""
+    import json, subprocess, os
+
+    ct = fake_hip
+    bf = torch.bfloat16
+    z, a, b = torch.empty(512, 512, dtype=bf), torch.empty(512, 256, dtype=bf), torch.empty(256, 512, dtype=bf)
+    launch = lambda: ct.gemm(ct.partition(z, [256, 256]), a, b, 256)
+    try:
+        assert "switched off" in ct.tuning_reload("")
+        launch()
+        base = ct.last_resolved()
+        assert base["source"] == "table" and base["bucket"] == "bf16_256x256|tiles<=256" and base["variant"] == "bf16_256x256x64_d4x2"
+        # records are written by the C++ surface (tune::Record::save); build one through it so the config ids are the library's own
+        helper = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tests", "cpp", "bin", "write_record")
+        def write(name, kernel, bucket, variant, **kw):
+            path = tmp_path / name
+            args = [helper, str(path), kernel, bucket, variant] + [f"{k}={v}" for k, v in kw.items()]
+            subprocess.check_call(args)
+            return path
+        write("gemm.json", "gemm", base["bucket"], "bf16_256x256x64_d2x4")
+        report = ct.tuning_reload(str(tmp_path))
+        assert "applied" in report and "1 bucket(s) of kernel gemm" in report
+        launch()
+        got = ct.last_resolved()
+        assert got["variant"] == "bf16_256x256x64_d2x4" and got["source"] == "record:" + base["bucket"]
+        assert _last(ct)[0].symbol == b"gemm_entry__bf16_256x256x64_d2x4"
+        # another shape class is not touched by that entry
+        zb = torch.empty(8192, 8192, dtype=bf)
+        ct.gemm(ct.partition(zb, [256, 256]), torch.empty(8192, 64, dtype=bf), torch.empty(64, 8192, dtype=bf), 64)
+        assert ct.last_resolved()["source"] == "table" and ct.last_resolved()["bucket"] == "bf16_256x256|tiles>256"
+        # the caller's variant still wins over the record
+        ct.gemm(ct.partition(z, [256, 256]), a, b, 256, variant="bf16_256x256x64_w2x2")
+        assert ct.last_resolved()["source"] == "caller"
+        # a record whose winner does not fit the arguments (another tile) is ignored for this launch
+        ct.set_preferred_variant_for("gemm", base["bucket"], "bf16_128x128x64_d2x2")
+        launch()
+        assert ct.last_resolved()["source"] == "table"
+        # stale provenance: each is refused and said so; the launch falls back to the table's order
+        for kw, why in (({"source_hash": "0123456789abcdef"}, "source_hash mismatch"), ({"arch": "gfx942"}, "arch mismatch"),
+                        ({"l2_key": "fedcba9876543210"}, "l2 key"), ({"tileiras_fingerprint": "another compiler"}, "another device toolchain"),
+                        ({"schema": 7}, "schema mismatch")):
+            for f in tmp_path.iterdir():
+                f.unlink()
+            write("gemm.json", "gemm", base["bucket"], "bf16_256x256x64_d2x4", **kw)
+            report = ct.tuning_reload(str(tmp_path))
+            assert "refused" in report and why in report, (kw, report)
+            assert ct.lib().cutile_tuning_applied_count() == 0
+            launch()
+            assert ct.last_resolved()["source"] == "table" and ct.last_resolved()["variant"] == base["variant"]
+        # a torn file is refused too, and does not stop the other files
+        (tmp_path / "aaa.json").write_text("{ not json")
+        write("rms.json", "rms_norm_f16", "n<=1024", "w1v2")
+        report = ct.tuning_reload(str(tmp_path))
+        assert "refused" in report and "1 bucket(s) of kernel rms_norm_f16" in report
+    finally:
+        ct.tuning_reload(None)
