@@ -997,6 +997,29 @@ def probe_ceilings(ct, torch, flush):
     return out
 
 
+def launch_modes():
+    """Host-visible latency of the execution modes of the C++ host surface (sync / chained / future / graph replay), one
+    small kernel and a 1000-kernel chain: cutile-rs_amd/bench/launch_overhead.cpp, the measurement of the reference's
+    cutile-benchmarks/paper/sec5_exp2_execution_mode_overhead.  A child process (it owns its own streams); microseconds
+    only, no roofline.  The reference's published medians (another vendor's desktop GPU, RTX 5090) are beside it."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "cutile-rs_amd", "bin", "launch_overhead")
+    if not os.path.exists(exe):
+        return {"error": "cutile-rs_amd/bin/launch_overhead is not built"}
+    try:
+        res = subprocess.run([exe, "--samples", "30"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=180)
+        out = json.loads([l for l in res.stdout.splitlines() if l.startswith("{")][-1])
+    except Exception as e:      # the measurement is informational: never fail the bench line over it
+        return {"error": f"{type(e).__name__}: {e}"}
+    ref = {"sync-individual/n=1": 7.282, "async/n=1": 22.024, "graph/n=1": 5.551, "sync-individual/n=1000": 7441.384,
+           "sync-chained/n=1000": 3364.874, "async/n=1000": 3398.144, "graph/n=1000": 810.009}
+    return {"kernel": out["kernel"], "unit": "us per pipeline, median",
+            "median_us": {k: round(v["median_us"], 2) for k, v in out["modes"].items()},
+            "reference_rtx5090_median_us": ref,
+            "reference_source": "cutile-benchmarks/paper/sec5_exp2_execution_mode_overhead/launch_overhead_rust/results_part_a.csv"}
+
+
 BASELINE_CONFIGS = ["gemm_bf16_8192", "gemm_bf16_4096", "fmha_bf16", "fmha_bf16_causal", "rms_norm_f16_16384x8192",
                     "softmax_f16_16384x8192", "saxpy_f32_16777216", "mxfp8_gemm_8192"]
 
@@ -1081,6 +1104,8 @@ def main():
         ceilings["probes"] = probe_ceilings(ct, torch, flush)
     if ceilings:
         line["ceilings"] = ceilings
+    if not args.only or args.ceilings:
+        line["launch_modes"] = launch_modes()
     print(json.dumps(line))
 
 

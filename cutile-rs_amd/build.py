@@ -178,18 +178,28 @@ def build_cpp_tests(force: bool = False) -> str:
     return out_dir
 
 
+PROGRAMS = {
+    # cutile-rs_amd/bin/<name>: programs on the C++ host surface
+    "tune_baseline": os.path.join("tune", "tune_baseline.cpp"),        # writes the tuning records
+    "launch_overhead": os.path.join("bench", "launch_overhead.cpp"),   # execution-mode latency, run by bench.py
+}
+
+
 def build_tuner(force: bool = False) -> str:
-    """The program that writes the tuning records (cutile-rs_amd/tune/tune_baseline.cpp -> cutile-rs_amd/bin/)."""
+    """The programs of the package that sit on the C++ host surface (cutile-rs_amd/bin/)."""
     out_dir = os.path.join(ROOT, "bin")
     os.makedirs(out_dir, exist_ok=True)
     include = os.path.join(ROOT, "..", "include")
-    src = os.path.join(ROOT, "tune", "tune_baseline.cpp")
-    dst = os.path.join(out_dir, "tune_baseline")
-    deps = [src, LIB_PATH] + [os.path.join(include, "cutile", f) for f in os.listdir(os.path.join(include, "cutile"))]
-    if force or not _newer(dst, deps):
-        _run([CXX, "-std=c++17", "-O1", "-g0", "-I" + include, "-Wall", "-Wextra", "-Wno-unused-parameter", src, "-o", dst, "-pthread",
-              "-L" + LIB_DIR, "-lcutile_hip", "-Wl,-rpath,$ORIGIN/../lib"])
-    return dst
+    headers = [os.path.join(include, "cutile", f) for f in os.listdir(os.path.join(include, "cutile"))]
+    jobs = []
+    for name, rel in PROGRAMS.items():
+        src, dst = os.path.join(ROOT, rel), os.path.join(out_dir, name)
+        if force or not _newer(dst, [src, LIB_PATH] + headers):
+            jobs.append([CXX, "-std=c++17", "-O2", "-g0", "-I" + include, "-Wall", "-Wextra", "-Wno-unused-parameter", src, "-o", dst, "-pthread",
+                         "-L" + LIB_DIR, "-lcutile_hip", "-Wl,-rpath,$ORIGIN/../lib"])
+    with ThreadPoolExecutor(max_workers=2) as ex:
+        list(ex.map(_run, jobs))
+    return out_dir
 
 
 def build(force: bool = False) -> str:
