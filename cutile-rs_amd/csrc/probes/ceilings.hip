@@ -102,6 +102,35 @@ extern "C" __global__ void __launch_bounds__(512) probe_mfma_bf16_lds(float* sin
 }
 
 // Each workgroup walks chunks of 256 lanes x VEC vectors, chunk c, c + gridDim.x, ...; n_vec is a multiple of 256 * VEC.
+// Store policies: 0 plain, 1 nontemporal, 2 sc1, 3 sc0 sc1 (the cache-scope bits of gfx950 stores).
+namespace {
+template <int POLICY>
+__device__ __forceinline__ void store_vec(u32x4* p, u32x4 v) {
+  if (POLICY == 0) *p = v;
+  else if (POLICY == 1) __builtin_nontemporal_store(v, p);
+  else if (POLICY == 2) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+  else asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+template <int POLICY, int VEC>
+__device__ __forceinline__ void write_stream(u32x4* dst, uint64_t n_vec) {
+  const u32x4 x = {threadIdx.x, blockIdx.x, 0x3c003c00u, 0xbc00bc00u};
+  for (uint64_t base = (uint64_t)blockIdx.x * 256 * VEC; base < n_vec; base += (uint64_t)gridDim.x * 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) store_vec<POLICY>(dst + base + i * 256 + threadIdx.x, x);
+  }
+}
+template <int POLICY, int VEC>
+__device__ __forceinline__ void copy_stream(const u32x4* src, u32x4* dst, uint64_t n_vec) {
+  for (uint64_t base = (uint64_t)blockIdx.x * 256 * VEC; base < n_vec; base += (uint64_t)gridDim.x * 256 * VEC) {
+    u32x4 v[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = __builtin_nontemporal_load(src + base + i * 256 + threadIdx.x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) store_vec<POLICY>(dst + base + i * 256 + threadIdx.x, v[i]);
+  }
+}
+}  // namespace
+
 constexpr int kVec = 8;
 extern "C" __global__ void __launch_bounds__(256) probe_stream_read(const u32x4* src, u32x4* sink, uint64_t n_vec) {
   u32x4 x = {0, 0, 0, 0};
@@ -114,19 +143,15 @@ extern "C" __global__ void __launch_bounds__(256) probe_stream_read(const u32x4*
   }
   if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[threadIdx.x] = x;   // keeps the loads alive; practically never taken
 }
-extern "C" __global__ void __launch_bounds__(256) probe_stream_write(u32x4* dst, uint64_t n_vec) {
-  const u32x4 x = {threadIdx.x, blockIdx.x, 0x3c003c00u, 0xbc00bc00u};
-  for (uint64_t base = (uint64_t)blockIdx.x * 256 * kVec; base < n_vec; base += (uint64_t)gridDim.x * 256 * kVec) {
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) __builtin_nontemporal_store(x, dst + base + i * 256 + threadIdx.x);
-  }
-}
-extern "C" __global__ void __launch_bounds__(256) probe_stream_copy(const u32x4* src, u32x4* dst, uint64_t n_vec) {
-  for (uint64_t base = (uint64_t)blockIdx.x * 256 * kVec; base < n_vec; base += (uint64_t)gridDim.x * 256 * kVec) {
-    u32x4 v[kVec];
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) v[i] = __builtin_nontemporal_load(src + base + i * 256 + threadIdx.x);
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) __builtin_nontemporal_store(v[i], dst + base + i * 256 + threadIdx.x);
-  }
-}
+#define WRITE_PROBE(NAME, POLICY) \
+  extern "C" __global__ void __launch_bounds__(256) probe_stream_write_##NAME(u32x4* dst, uint64_t n_vec) { write_stream<POLICY, 8>(dst, n_vec); }
+WRITE_PROBE(plain, 0)
+WRITE_PROBE(nt, 1)
+WRITE_PROBE(sc1, 2)
+WRITE_PROBE(sc0sc1, 3)
+#define COPY_PROBE(NAME, POLICY, VEC) \
+  extern "C" __global__ void __launch_bounds__(256) probe_stream_copy_##NAME(const u32x4* src, u32x4* dst, uint64_t n_vec) { copy_stream<POLICY, VEC>(src, dst, n_vec); }
+COPY_PROBE(plain_v8, 0, 8)
+COPY_PROBE(nt_v8, 1, 8)
+COPY_PROBE(nt_v4, 1, 4)
+COPY_PROBE(sc0sc1_v8, 3, 8)
