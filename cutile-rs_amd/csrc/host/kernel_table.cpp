@@ -163,6 +163,8 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 64, 128, 64, 2, 2);
   gemm("f16", 256, 256, 64, 4, 2, "d");
   gemm("f16", 128, 128, 64, 2, 2, "d");
+  gemm("f16", 256, 256, 64, 4, 2, "r");
+  gemm("f16", 256, 256, 64, 2, 4, "r");
   gemm("bf16f32", 128, 128, 64, 2, 2);
   gemm("bf16f32", 256, 256, 64, 2, 2);
   // any tile shape, strides and extents (tile = 0: not tied to a partition shape); 64x64 outputs per workgroup

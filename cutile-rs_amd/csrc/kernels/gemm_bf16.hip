@@ -517,7 +517,7 @@ struct GemmDirect {
 //  * fetches past the end of K read zeros through the descriptor's range check,
 //    so the loop has one shape for every tile, including a ragged last one.
 // LDS: 3 * BM*BK*2 + 2 * BK*BN*2 bytes (160 KiB for 256x256).
-template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT, typename InT = __bf16>
 struct GemmRing {
   static constexpr int BK = 64;
   static constexpr int kWaves = WAVES_M * WAVES_N;
@@ -659,7 +659,7 @@ struct GemmRing {
         for (int r = 0; r < NR; ++r)
           if (r * SLOTS / NR == j) read_operand(rd_x, rd_y, rd_ks, into, r);
         acc[j / TM][j % TM] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM], 0, 0, 0);
+            mfma_32x32x16<InT>(use.b[j / TM], use.a[j % TM], acc[j / TM][j % TM]);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
@@ -943,6 +943,14 @@ GROUP_GEMM_KERNEL(f16_128x128x64_d2x2, 128, 128, 2, 2)
 GEMM_RING_KERNEL(bf16_256x256x64_r2x4, 256, 256, 2, 4, __bf16)
 GEMM_RING_KERNEL(bf16_256x256x64_r4x2, 256, 256, 4, 2, __bf16)
 GEMM_RING_KERNEL(bf16_128x128x64_r2x2, 128, 128, 2, 2, __bf16)
+#define GEMM_RING_KERNEL_F16(NAME, BM, BN, WVM, WVN)                                            \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmRing<BM, BN, WVM, WVN, _Float16, _Float16>::run(z, x, y, k, g, accumulate);            \
+  }
+GEMM_RING_KERNEL_F16(f16_256x256x64_r2x4, 256, 256, 2, 4)
+GEMM_RING_KERNEL_F16(f16_256x256x64_r4x2, 256, 256, 4, 2)
 
 #define GEMM_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                                \
   extern "C" __global__ void __launch_bounds__(256)                                            \

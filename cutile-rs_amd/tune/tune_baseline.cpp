@@ -100,6 +100,15 @@ int main(int argc, char** argv) {
       return enqueue(gemm(z.partition_mut({256, 256}), x, y, s), v, st);
     });
   }
+  {   // GEMM f16 at 8192^3 (the operand type of the reference's own published GEMM figure)
+    const int s = 8192;
+    auto x = converted<f16>(api::randn(0.0f, 1.0f / std::sqrt((float)s), {s * s}, 5).sync_on(g_stream).unwrap(), {s, s});
+    auto y = converted<f16>(api::randn(0.0f, 1.0f / std::sqrt((float)s), {s * s}, 6).sync_on(g_stream).unwrap(), {s, s});
+    auto z = api::zeros<f16>({s, s}).sync_on(g_stream).unwrap();
+    all &= tune_one("gemm", "f16 M=N=K=8192", [&](const std::string& v, const std::shared_ptr<Stream>& st) {
+      return enqueue(gemm(z.partition_mut({256, 256}), x, y, s), v, st);
+    });
+  }
   {   // FMHA bf16 b4 h32 s4096 d128
     const int b = 4, h = 32, s = 4096, d = 128;
     auto mk = [&](uint64_t seed) { return converted<bf16>(api::randn(0.0f, 1.0f, {b * h * s * d}, seed).sync_on(g_stream).unwrap(), {b, h, s, d}); };

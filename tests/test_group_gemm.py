@@ -89,6 +89,26 @@ def test_gpu_gemm_f16(ct, dev, m, n, k, tile, accumulate):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("variant", ["f16_256x256x64_r4x2", "f16_256x256x64_r2x4", "f16_256x256x64_d4x2"])
+@pytest.mark.parametrize("m,n,k,accumulate", [(512, 768, 1024, False), (300, 264, 448, True), (256, 256, 64, False)])
+def test_gpu_gemm_f16_pipelined_variants(ct, dev, variant, m, n, k, accumulate):
+    """every f16 variant of the 256 x 256 tile, the ring-pipelined ones included (whole K tiles), against cpu_gemm"""
+    ab, bb = f16b(oracle.normal_f32((m, k), 864, 0, k ** -0.5)), f16b(oracle.normal_f32((k, n), 865, 0, k ** -0.5))
+    z0 = f16b(oracle.normal_f32((m, n), 866))
+    z = _dev16(z0, dev).clone()
+    ct.gemm(ct.partition(z, [256, 256]), _dev16(ab, dev), _dev16(bb, dev), k, accumulate=accumulate, variant=variant)
+    torch.cuda.synchronize()
+    ref = oracle.cpu_gemm_f32(f16v(ab), f16v(bb)) + (f16v(z0) if accumulate else 0.0)
+    assert rel_l2(z.float().cpu().numpy(), ref) <= 1e-2
+    eye = torch.eye(k, n, dtype=torch.half, device=dev)
+    zi = torch.zeros(m, n, dtype=torch.half, device=dev)
+    ct.gemm(ct.partition(zi, [256, 256]), _dev16(ab, dev), eye, k, accumulate=False, variant=variant)
+    torch.cuda.synchronize()
+    w = min(k, n)
+    assert torch.equal(zi[:, :w], _dev16(ab, dev)[:, :w]) and not zi[:, w:].any()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tile,num_sm", [(128, 8), (128, 256), (256, 3), (256, 64)])
 def test_gpu_group_gemm_desc(ct, dev, tile, num_sm):
     shapes = [(128, 256, 64), (48, 16, 32), (0, 64, 64), (400, 272, 192), (16, 528, 16), (256, 256, 256)]   # (m, n, k)
