@@ -20,6 +20,8 @@ from typing import Optional, Sequence
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libcutile_hip.so")
+# the same library plus the recording stand-in for the HIP runtime (include/cutile_hip_testing.h): what the CPU tests load
+TESTING_LIB_PATH = os.path.join(_HERE, "lib", "libcutile_hip_testing.so")
 MAX_RANK = 4
 
 # cutile_dtype_t
@@ -98,8 +100,9 @@ def lib() -> C.CDLL:
         L.cutile_dtype_from_name.restype = C.c_int
         L.cutile_dtype_from_name.argtypes = [C.c_char_p]
         L.cutile_module_load_count.restype = C.c_uint64
-        L.cutile_testing_streams_created.restype = C.c_uint64
-        L.cutile_testing_bytes_allocated.restype = C.c_uint64
+        if hasattr(L, "cutile_testing_use_fake_hip"):      # only the testing library carries the recording runtime
+            L.cutile_testing_streams_created.restype = C.c_uint64
+            L.cutile_testing_bytes_allocated.restype = C.c_uint64
         vp, f32, f64, i32, i64 = C.c_void_p, C.c_float, C.c_double, C.c_int32, C.c_int64
         P = C.POINTER
         sig = {
@@ -202,6 +205,8 @@ def lib() -> C.CDLL:
             "cutile_testing_inject_failure": [C.c_char_p, i32, i32],
         }
         for name, argtypes in sig.items():
+            if name.startswith("cutile_testing_") and not hasattr(L, name):
+                continue
             fn = getattr(L, name)
             fn.argtypes = argtypes
             fn.restype = C.c_int32

@@ -35,7 +35,11 @@ IMAGES = {
     "nvfp4": "nvfp4_gemm.hip",
     "rng": "rng.hip",
 }
-HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "fake_hip.cpp", "tuning.cpp"]
+HOST_SOURCES = ["hip_api.cpp", "driver.cpp", "kernel_table.cpp", "launch.cpp", "runtime.cpp", "tuning.cpp"]
+# The recording stand-in for the HIP runtime (include/cutile_hip_testing.h) is not part of the product library: the CPU
+# tests load a second library, the same objects plus this source.
+TESTING_SOURCES = ["fake_hip.cpp"]
+TESTING_LIB_PATH = os.path.join(LIB_DIR, "libcutile_hip_testing.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXX = os.environ.get("CXX", "g++")
@@ -102,20 +106,25 @@ def build_host_library(images: dict[str, str], force: bool = False) -> str:
         with open(toolchain, "w") as f:
             f.write(text_h)
     sources = [os.path.join(HOST_DIR, s) for s in HOST_SOURCES]
-    deps = sources + [embed, toolchain] + list(images.values()) + [
+    testing = [os.path.join(HOST_DIR, s) for s in TESTING_SOURCES]
+    include = os.path.join(ROOT, "..", "include")
+    deps = sources + testing + [embed, toolchain] + list(images.values()) + [
         os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".h")
-    ] + [os.path.join(ROOT, "..", "include", "cutile_hip.h")]
-    if force or not _newer(LIB_PATH, deps):
-        objs = []
+    ] + [os.path.join(include, "cutile_hip.h"), os.path.join(include, "cutile_hip_testing.h")] + [
+        os.path.join(include, "cutile", f) for f in ("tune.hpp", "json.hpp", "bench.hpp", "runtime.hpp", "error.hpp", "device_op.hpp")]
+    if force or not _newer(LIB_PATH, deps) or not _newer(TESTING_LIB_PATH, deps):
+        objs = {}
         jobs = []
-        for s in sources + [embed]:
+        for s in sources + testing + [embed]:
             o = os.path.join(BUILD_DIR, os.path.basename(s) + ".o")
-            objs.append(o)
+            objs[s] = o
             if force or not _newer(o, deps):
                 jobs.append([CXX] + HOST_FLAGS + ["-I", BUILD_DIR, "-c", s, "-o", o])
         with ThreadPoolExecutor(max_workers=6) as ex:
             list(ex.map(_run, jobs))
-        _run([CXX, "-shared", "-o", LIB_PATH] + objs + ["-ldl", "-pthread", "-Wl,--no-undefined"])
+        product = [objs[s] for s in sources + [embed]]
+        _run([CXX, "-shared", "-o", LIB_PATH] + product + ["-ldl", "-pthread", "-Wl,--no-undefined"])
+        _run([CXX, "-shared", "-o", TESTING_LIB_PATH] + product + [objs[s] for s in testing] + ["-ldl", "-pthread", "-Wl,--no-undefined"])
     return LIB_PATH
 
 
@@ -145,8 +154,8 @@ def build_scratch_library(force: bool = False) -> str:
 
 CPP_TEST_DIR = os.path.join(ROOT, "..", "tests", "cpp")
 CPP_TESTS = {
-    # binary -> (source, needs the library, extra flags)
-    "test_host_surface": ("test_host_surface.cpp", True, []),
+    # binary -> (source, library it links: True = the product library, "testing" = the one with the recording runtime, extra flags)
+    "test_host_surface": ("test_host_surface.cpp", "testing", []),
     "test_gpu_surface": ("test_gpu_surface.cpp", True, []),
     "write_record": ("write_record.cpp", True, []),
     "test_slot_table": ("test_slot_table.cpp", False, []),
@@ -166,12 +175,13 @@ def build_cpp_tests(force: bool = False) -> str:
     for name, (src, needs_lib, extra) in CPP_TESTS.items():
         dst = os.path.join(out_dir, name)
         src_path = os.path.join(CPP_TEST_DIR, src)
-        deps = [src_path] + headers + ([LIB_PATH] if needs_lib else [])
+        deps = [src_path] + headers + ([TESTING_LIB_PATH if needs_lib == "testing" else LIB_PATH] if needs_lib else [])
         if force or not _newer(dst, deps):
             cmd = [CXX, "-std=c++17", "-O1", "-g0", "-I" + include, "-Wall", "-Wextra", "-Wno-unused-parameter"] + extra
             cmd += [src_path, "-o", dst, "-pthread"]
             if needs_lib:
-                cmd += ["-L" + LIB_DIR, "-lcutile_hip", "-Wl,-rpath,$ORIGIN/../../../cutile-rs_amd/lib"]
+                cmd += ["-L" + LIB_DIR, "-lcutile_hip_testing" if needs_lib == "testing" else "-lcutile_hip",
+                        "-Wl,-rpath,$ORIGIN/../../../cutile-rs_amd/lib"]
             jobs.append(cmd)
     with ThreadPoolExecutor(max_workers=4) as ex:
         list(ex.map(_run, jobs))

@@ -1,6 +1,7 @@
 // A minimal JSON value, reader and writer: what the tuner's trial logs and records need
 // (objects keep insertion order so that saved records diff cleanly).
 #pragma once
+#include <cerrno>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -172,7 +173,17 @@ class Reader {
     }
     return false;   // unterminated: a torn line
   }
+  // Nesting deeper than any record or log line this library writes (they nest three levels) is refused: a corrupted
+  // or hostile file must not be able to overflow the stack through the recursion below.
+  static constexpr int kMaxDepth = 64;
+  struct DepthGuard {
+    int& d;
+    explicit DepthGuard(int& depth) : d(depth) { ++d; }
+    ~DepthGuard() { --d; }
+  };
   bool value(Value* out) {
+    DepthGuard guard(depth_);
+    if (depth_ > kMaxDepth) return false;
     space();
     if (p_ >= t_.size()) return false;
     char c = t_[p_];
@@ -225,12 +236,26 @@ class Reader {
       ++p_;
     }
     if (p_ == start) return false;
+    // The scan above takes any run of number characters; the conversion must consume all of it, or the token is
+    // not a number ("1-2", "--", "1e", "1.2.3") and the document is refused like any other torn text.
     std::string num = t_.substr(start, p_ - start);
-    *out = is_float ? Value::number(strtod(num.c_str(), nullptr)) : Value::integer(strtoll(num.c_str(), nullptr, 10));
+    if (!(num[0] == '-' || isdigit((unsigned char)num[0]))) return false;   // JSON numbers do not start with '+' or '.'
+    char* end = nullptr;
+    errno = 0;
+    if (is_float) {
+      const double v = strtod(num.c_str(), &end);
+      if (end != num.c_str() + num.size() || !isdigit((unsigned char)num.back())) return false;
+      *out = Value::number(v);
+    } else {
+      const long long v = strtoll(num.c_str(), &end, 10);
+      if (end != num.c_str() + num.size() || errno == ERANGE || !isdigit((unsigned char)num.back())) return false;
+      *out = Value::integer(v);
+    }
     return true;
   }
   const std::string& t_;
   size_t p_ = 0;
+  int depth_ = 0;
 };
 
 inline std::optional<Value> parse(const std::string& text) { return Reader(text).document(); }

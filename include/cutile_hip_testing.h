@@ -11,7 +11,9 @@
  * machine without a GPU.  "Device" memory is host memory, copies are memcpy,
  * streams complete immediately, host callbacks run inline.
  *
- * Never enabled implicitly; product code paths do not reference it.
+ * These entry points are exported by libcutile_hip_testing.so only (the product
+ * library's objects plus the stand-in); libcutile_hip.so, the library that ships,
+ * exports none of them.  Never enabled implicitly.
  */
 #ifndef CUTILE_HIP_TESTING_H
 #define CUTILE_HIP_TESTING_H

@@ -28,8 +28,12 @@ def oracle():
 
 
 @pytest.fixture()
-def fake_hip(ct):
-    """Routes the library to the recording stand-in for the HIP runtime for one test."""
+def fake_hip():
+    """A binding of the TESTING library (the product library's objects plus the recording stand-in for the HIP
+    runtime), routed to that stand-in for one test."""
+    import __graft_entry__ as entry
+
+    ct = entry.load_package(testing=True)
     ct.check(ct.lib().cutile_testing_use_fake_hip(1))
     ct.lib().cutile_testing_clear_log()
     ct.tuning_reload("")            # the variant choices asserted on this runtime are the table's own, not a record's

@@ -689,6 +689,19 @@ TEST(trial_log_roundtrips_resumes_and_refuses_foreign_logs) {   // tune.rs:1364-
   remove(path.c_str());
 }
 
+TEST(json_reader_refuses_deep_nesting_and_malformed_numbers) {
+  CHECK(json::parse("{\"a\": [1, 2.5, -3e2, {\"b\": null}]}").has_value());
+  CHECK(json::parse("[1, 2.5e-3, -0.5, 10]")->items[1].as_double() == 2.5e-3);
+  for (const char* bad : {"1-2", "--", "-", "1e", "1.2.3", "[1, 2-]", "{\"a\": +1}", "1e+", "12.", "99999999999999999999"})
+    CHECK(!json::parse(bad).has_value());
+  std::string deep(100000, '[');      // would recurse 100000 frames without the cap
+  CHECK(!json::parse(deep).has_value());
+  std::string ok_depth = std::string(60, '[') + "1" + std::string(60, ']');
+  CHECK(json::parse(ok_depth).has_value());
+  std::string too_deep = std::string(70, '[') + "1" + std::string(70, ']');
+  CHECK(!json::parse(too_deep).has_value());
+}
+
 TEST(tuning_records_roundtrip_and_refuse_stale_provenance) {   // tune.rs:1151-1362
   using tune::Record;
   using tune::RecordEntry;

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 import oracle
-from util import f16_ulp_diff, from_dev_f16_bits, normal_f16_bits, rel_l2, to_dev_bf16, to_dev_f16
+from util import assert_rounded_close, f16_ulp_diff, from_dev_f16_bits, normal_f16_bits, rel_l2, to_dev_bf16, to_dev_f16
 
 pytestmark = pytest.mark.gpu
 
@@ -78,6 +78,8 @@ def test_gemm_bf16_full_size(ct, dev, s):
     ref = oracle.gemm_bf16(ab, bb, rows=rows, f32out=True)
     idx = torch.from_numpy(rows).to(dev)
     assert rel_l2(z[idx].float().cpu().numpy(), ref) <= 1e-2
+    # element by element on the sampled rows: one bf16 rounding of the f32 sum (the sample spans every column tile)
+    assert_rounded_close(z[idx].float().cpu().numpy(), ref, (len(rows), 256), what=f"gemm {s}")
     ct.gemm(zp, a, b, s, accumulate=True)                             # a second pass adds the same product again
     torch.cuda.synchronize()
     assert rel_l2(z[idx].float().cpu().numpy(), 2.0 * ref) <= 1e-2
@@ -128,6 +130,7 @@ def test_mxfp8_8192(ct, dev):
     rows = _sample(s, 32, 17)
     ref = oracle.mx_gemm_f32(xq, yq, xs, ys, 1.0, rows=rows)
     assert rel_l2(z[torch.from_numpy(rows).to(dev)].float().cpu().numpy(), ref) <= 3e-2
+    assert_rounded_close(z[torch.from_numpy(rows).to(dev)].float().cpu().numpy(), ref, (len(rows), 256), what="mxfp8 8192")
     # cutile-examples/examples/mxfp8.rs:91-135 at full size: e4m3 1.0 (0x38) and e8m0 2^0 (0x7F) everywhere -> K
     one = torch.full((s, s), 0x38, dtype=torch.uint8, device=dev)
     unit = torch.full((s, s // 32), 0x7F, dtype=torch.uint8, device=dev)

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from util import (f16_ulp_diff, from_dev_bf16_bits, from_dev_f16_bits, normal_bf16_bits, normal_f16_bits, rel_l2,
+from util import (assert_rounded_close, f16_ulp_diff, from_dev_bf16_bits, from_dev_f16_bits, normal_bf16_bits, normal_f16_bits, rel_l2,
                   to_dev_bf16, to_dev_f16)
 
 pytestmark = pytest.mark.gpu
@@ -473,3 +473,6 @@ def test_mxfp8_random_blocks(ct, dev, m, n, k, tile, out_dtype, variant):
     assert rel_l2(got, ref) <= tol
     if out_dtype == torch.float32:      # exact products of fp8 values: only summation order differs
         assert rel_l2(got, ref) <= 1e-4
+        assert_rounded_close(got, ref, (tile, tile), rel_ulp=1e-5, what="mxfp8 f32")
+    else:                               # bf16 output: the f32 sum rounded once
+        assert_rounded_close(got, ref, (tile, tile), what="mxfp8 bf16")

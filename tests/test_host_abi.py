@@ -13,16 +13,25 @@ import torch
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(cutile_[a-z0-9_]+)\s*\(", text))
+
+
 def test_library_exports_every_declared_symbol(ct):
+    import __graft_entry__ as entry
+
     L = ct.lib()
-    declared = set()
-    for h in ("cutile_hip.h", "cutile_hip_testing.h"):
-        text = open(os.path.join(ROOT, "include", h)).read()
-        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        declared |= set(re.findall(r"\b(cutile_[a-z0-9_]+)\s*\(", text))
-    assert len(declared) > 80
+    declared = _declared("cutile_hip.h")
+    assert len(declared) > 100
     missing = [s for s in sorted(declared) if not hasattr(L, s)]
     assert not missing, missing
+    # the test hooks live in the testing library only: the product library carries none of them
+    hooks = _declared("cutile_hip_testing.h")
+    assert len(hooks) >= 8 and not [s for s in hooks if hasattr(L, s)]
+    T = entry.load_package(testing=True).lib()
+    assert not [s for s in sorted(declared | hooks) if not hasattr(T, s)]
 
 
 def test_status_names_and_dtypes(ct):

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle
-from util import rel_l2
+from util import assert_rounded_close, rel_l2
 
 E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
 
@@ -119,6 +119,8 @@ def test_gpu_nvfp4_gemm(ct, dev, m, n, k, tile, variant, out):
     got = z.float().cpu().numpy()
     assert np.all(np.isfinite(got))
     assert rel_l2(got, ref) <= (1e-5 if out == "f32" else 4e-3)     # f32: order of additions only; bf16: output rounding
+    # and element by element, the last (partial) tile's rows and columns on their own
+    assert_rounded_close(got, ref, (tile, tile), rel_ulp=1e-5 if out == "f32" else 2.0 ** -7, what=f"nvfp4 {out}")
 
 
 @pytest.mark.gpu

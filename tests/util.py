@@ -43,3 +43,17 @@ def f16_ulp_diff(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
 def rel_l2(got: np.ndarray, ref: np.ndarray) -> float:
     return float(np.linalg.norm(got.astype(np.float64) - ref.astype(np.float64)) /
                  max(np.linalg.norm(ref.astype(np.float64)), 1e-30))
+
+
+def assert_rounded_close(got: np.ndarray, ref: np.ndarray, tile, rel_ulp: float = 2.0 ** -7, atol_frac: float = 2e-5, what: str = "") -> None:
+    """Elementwise: every output within one unit in the last place of the 16-bit output type (relative `rel_ulp`:
+    2^-7 for bf16, 2^-10 for f16) of the f32 reference, plus a small absolute term for sums that cancel; asserted on the
+    whole matrix and, separately, on the rows and columns of the last (partial) tile, where a wrong tail would hide in
+    a whole-matrix norm."""
+    got64, ref64 = got.astype(np.float64), ref.astype(np.float64)
+    bound = np.abs(ref64) * rel_ulp + atol_frac * np.max(np.abs(ref64))
+    bad = np.abs(got64 - ref64) > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than one ulp, first at {np.argwhere(bad)[0]}"
+    bm, bn = tile
+    r0, c0 = (got.shape[0] - 1) // bm * bm, (got.shape[1] - 1) // bn * bn
+    assert not bad[r0:, :].any() and not bad[:, c0:].any(), f"{what}: last tile rows/columns"
