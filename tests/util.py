@@ -45,13 +45,16 @@ def rel_l2(got: np.ndarray, ref: np.ndarray) -> float:
                  max(np.linalg.norm(ref.astype(np.float64)), 1e-30))
 
 
-def assert_rounded_close(got: np.ndarray, ref: np.ndarray, tile, rel_ulp: float = 2.0 ** -7, atol_frac: float = 2e-5, what: str = "") -> None:
+def assert_rounded_close(got: np.ndarray, ref: np.ndarray, tile, rel_ulp: float = 2.0 ** -7, atol_frac: float = 2e-5, what: str = "",
+                         mag: np.ndarray | None = None) -> None:
     """Elementwise: every output within one unit in the last place of the 16-bit output type (relative `rel_ulp`:
     2^-7 for bf16, 2^-10 for f16) of the f32 reference, plus a small absolute term for sums that cancel; asserted on the
     whole matrix and, separately, on the rows and columns of the last (partial) tile, where a wrong tail would hide in
-    a whole-matrix norm."""
+    a whole-matrix norm.  The absolute term is `atol_frac` of `mag`, the element's own sum of |products| (what the
+    rounding of an f32 accumulation in another order scales with: one missing product of K is mag/K, far above it),
+    or of the largest |ref| where no `mag` is given."""
     got64, ref64 = got.astype(np.float64), ref.astype(np.float64)
-    bound = np.abs(ref64) * rel_ulp + atol_frac * np.max(np.abs(ref64))
+    bound = np.abs(ref64) * rel_ulp + atol_frac * (np.max(np.abs(ref64)) if mag is None else mag.astype(np.float64))
     bad = np.abs(got64 - ref64) > bound
     assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than one ulp, first at {np.argwhere(bad)[0]}"
     bm, bn = tile
