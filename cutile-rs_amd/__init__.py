@@ -111,6 +111,7 @@ def lib() -> C.CDLL:
             "cutile_launch_add": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), P(LaunchOpts)],
             "cutile_launch_full": [vp, f64, i64, P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_arange": [vp, P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_eye": [vp, P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_linspace": [vp, P(PartitionArg), f32, f32, P(LaunchOpts)],
             "cutile_launch_convert": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
@@ -374,6 +375,12 @@ def full(value, t: Partition, *, stream=None, grid=None, variant=None) -> None:
 def arange(t: Partition, *, stream=None, grid=None, variant=None) -> None:
     o, _k = _opts(grid, None, variant)
     check(lib().cutile_launch_arange(_stream(stream), C.byref(t.arg()), C.byref(o)))
+
+
+def eye(t: Partition, *, stream=None, grid=None, generics=None) -> None:
+    """creation::eye over [BR, BC] tiles of an f32 matrix (cutile/src/kernels/_creation.rs:110-138)"""
+    o, _k = _opts(grid, generics, None)
+    check(lib().cutile_launch_eye(_stream(stream), C.byref(t.arg()), C.byref(o)))
 
 
 def linspace(t: Partition, start: float, step: float, *, stream=None, grid=None) -> None:

@@ -98,6 +98,7 @@ std::vector<KernelEntry> build_table() {
   add("rng_fill", "f32", "rng_fill_entry__f32", IMG_RNG, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
   add("rng_fill", "f64", "rng_fill_entry__f64", IMG_RNG, 256, 0, 0, 0, 0, 0, "f64", 0, 1);
   add("linspace", "f32", "linspace_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  add("eye", "f32", "eye_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
   static const char* kConvertTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64"};
   for (const char* s : kConvertTypes)
     for (const char* d : kConvertTypes)

@@ -636,6 +636,23 @@ cutile_status_t cutile_launch_arange(cutile_stream_t stream, const cutile_partit
                                      const cutile_launch_opts_t* opts) {
   return launch_creation("arange", stream, t, nullptr, 0, false, nullptr, 0, opts);
 }
+cutile_status_t cutile_launch_eye(cutile_stream_t stream, const cutile_partition_arg_t* t, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(t, "tensor", 2, 2)) return s;
+  CUTILE_REQUIRE(t->tensor.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_LAUNCH, "eye: tensor must be f32");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(t->partition_shape[0]), "BR")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(t->partition_shape[1]), "BC")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(t, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("eye", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*t);
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>((uint64_t)tg[0] * t->partition_shape[0], t->tensor.shape[0]);
+  const uint64_t cols = std::min<uint64_t>((uint64_t)tg[1] * t->partition_shape[1], t->tensor.shape[1]);
+  uint32_t grid[3] = {std::min<uint32_t>(std::max<uint32_t>(1, div_up(rows * cols, 256 * 4)), 16384), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
 cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_partition_arg_t* t, float start, float step,
                                        const cutile_launch_opts_t* opts) {
   CUTILE_REQUIRE(t && t->tensor.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_LAUNCH, "linspace: tensor must be f32");

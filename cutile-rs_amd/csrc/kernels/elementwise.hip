@@ -1,5 +1,5 @@
 // Elementwise and creation kernels for gfx950: saxpy, axpy with a separate
-// output, add, full, arange, linspace, convert.
+// output, add, full, arange, linspace, eye, convert.
 //
 // Bodies follow the reference's tile programs:
 //   saxpy    cutile-examples/examples/saxpy.rs:12-17, async_saxpy.rs:21-30
@@ -454,6 +454,20 @@ extern "C" __global__ void __launch_bounds__(kThreads)
     linspace_entry__f32(PartitionArg<1> t, float start, float step, TileGrid g) {
   flat_generate<float>((float*)t.ptr, t.strides[0], covered_1d(t.shape[0], t.pshape[0], g),
                        [&](size_t i) { return start + (float)(int32_t)i * step; });
+}
+
+// eye<BR, BC>(tensor: [BR, BC] tiles of an f32 matrix): 1 where row == column, 0 elsewhere, over the
+// region the tile grid covers (cutile/src/kernels/_creation.rs:110-138).  Flat over that region: the
+// tile shape only decides how far the grid reaches, every element is written exactly once.
+extern "C" __global__ void __launch_bounds__(kThreads) eye_entry__f32(PartitionArg<2> t, TileGrid g) {
+  const int64_t rows = min((int64_t)t.shape[0], (int64_t)g.x * t.pshape[0]);
+  const int64_t cols = min((int64_t)t.shape[1], (int64_t)g.y * t.pshape[1]);
+  float* p = (float*)t.ptr;
+  const int64_t total = rows * cols;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int64_t r = i / cols, c = i - r * cols;
+    p[r * t.strides[0] + c * t.strides[1]] = r == c ? 1.0f : 0.0f;
+  }
 }
 
 // ---- convert -------------------------------------------------------------------------------

@@ -95,6 +95,31 @@ class Arange : public DeviceOp<Arange<T>, Tensor<T>> {
 };
 template <class T> Arange<T> arange(size_t n) { return Arange<T>(n); }
 
+// eye / eye_rect: allocate [rows, cols] f32, then creation::eye over tiles of 16 x 16
+// (api.rs:613-639; kernel cutile/src/kernels/_creation.rs:110-138).
+class Eye : public DeviceOp<Eye, Tensor<float>> {
+ public:
+  Eye(size_t rows, size_t cols) : rows_(rows), cols_(cols) {}
+  Result<Tensor<float>> execute(const ExecutionContext& ctx) && {
+    auto t = Uninitialized<float>({(int32_t)rows_, (int32_t)cols_}).execute(ctx);
+    if (t.is_err()) return t.error();
+    if (t.value().size() == 0) return t;
+    cutile_partition_arg_t p{};
+    p.tensor = t.value().arg();
+    for (int i = 0; i < 2; ++i) {
+      p.partition_shape[i] = 16;
+      p.partition_strides[i] = p.tensor.strides[i];
+    }
+    CUTILE_TRY_STATUS(cutile_launch_eye(ctx.stream()->raw(), &p, nullptr));
+    return t;
+  }
+
+ private:
+  size_t rows_, cols_;
+};
+inline Eye eye_rect(size_t rows, size_t cols) { return Eye(rows, cols); }
+inline Eye eye(size_t n) { return Eye(n, n); }
+
 class Linspace : public DeviceOp<Linspace, Tensor<float>> {
  public:
   Linspace(float start, float stop, size_t n) : start_(start), stop_(stop), n_(n) {}

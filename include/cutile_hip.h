@@ -429,6 +429,10 @@ cutile_status_t cutile_launch_arange(cutile_stream_t stream, const cutile_partit
                                      const cutile_launch_opts_t* opts);
 cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_partition_arg_t* t,
                                        float start, float step, const cutile_launch_opts_t* opts);
+/* creation::eye<BR, BC>(tensor: [BR, BC] tiles, f32, rank 2): 1 where row == column, 0 elsewhere —
+ * cutile/src/kernels/_creation.rs:110-138 (behind api::eye / eye_rect, cutile/src/api.rs:613-639). */
+cutile_status_t cutile_launch_eye(cutile_stream_t stream, const cutile_partition_arg_t* t,
+                                  const cutile_launch_opts_t* opts);
 /* conversion::convert — cutile/src/kernels/_conversion.rs:78-85 */
 cutile_status_t cutile_launch_convert(cutile_stream_t stream, const cutile_tensor_arg_t* src,
                                       const cutile_partition_arg_t* dst, const cutile_launch_opts_t* opts);

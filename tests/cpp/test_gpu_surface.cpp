@@ -312,6 +312,22 @@ TEST(nvfp4_example_all_ones) {
   for (float v : host) CHECK(v == (float)K);
 }
 
+TEST(eye_and_eye_rect) {
+  // cutile/tests/arange.rs:106-186: eye(4), eye(32), eye_rect(16, 32), eye_rect(32, 16), plus sizes off the 16 x 16 tiles
+  auto stream = new_stream();
+  const std::pair<size_t, size_t> cases[] = {{4, 4}, {32, 32}, {16, 32}, {32, 16}, {3, 5}, {100, 37}};
+  for (auto [rows, cols] : cases) {
+    auto m = (rows == cols ? api::eye(rows) : api::eye_rect(rows, cols)).sync_on(stream).unwrap();
+    CHECK(m.shape() == (std::vector<int32_t>{(int32_t)rows, (int32_t)cols}));
+    auto host = api::to_host_vec(m).sync_on(stream).unwrap();
+    CHECK(host.size() == rows * cols);
+    bool ok = true;
+    for (size_t r = 0; r < rows; ++r)
+      for (size_t c = 0; c < cols; ++c) ok = ok && host[r * cols + c] == (r == c ? 1.0f : 0.0f);
+    CHECK(ok);
+  }
+}
+
 TEST(random_constructors_draw_on_the_device) {
   // api::randn / rand / randn_f16 (cutile/src/api.rs:683-735): distribution, seed determinism, shapes
   auto stream = new_stream();

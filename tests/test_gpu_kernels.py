@@ -132,6 +132,33 @@ def test_linspace(ct, dev):
     assert torch.equal(t, 1.0 + torch.arange(257, device=dev).float() * 0.5)
 
 
+@pytest.mark.parametrize("rows,cols,tile", [(4, 4, 16), (32, 32, 16), (16, 32, 16), (32, 16, 16),      # cutile/tests/arange.rs:106-186
+                                            (100, 37, 16), (1, 1, 16), (513, 1025, 64), (48, 48, 8)])
+def test_eye(ct, dev, rows, cols, tile):
+    t = torch.full((rows, cols), float("nan"), device=dev)
+    ct.eye(ct.partition(t, [tile, tile]))
+    sync()
+    assert torch.equal(t, torch.eye(rows, cols, device=dev))
+
+
+def test_eye_on_a_strided_view_and_a_prefix_grid(ct, dev):
+    base = torch.full((40, 96), -1.0, device=dev)
+    view = base[:, 8:72:2]                                   # 40 x 32, row stride 96, column stride 2
+    ct.eye(ct.partition(view, [16, 16]))
+    sync()
+    assert torch.equal(view, torch.eye(40, 32, device=dev))
+    mask = torch.ones_like(base, dtype=torch.bool)
+    mask[:, 8:72:2] = False
+    assert torch.all(base[mask] == -1.0)                     # nothing beside the view was written
+    # a prefix partition launched over 2 x 1 tiles touches rows 0..31, columns 0..15 only
+    t = torch.full((40, 40), -1.0, device=dev)
+    ct.eye(ct.partition(t, [16, 16], prefix=True), grid=(2, 1, 1))
+    sync()
+    want = torch.full((40, 40), -1.0, device=dev)
+    want[:32, :16] = torch.eye(32, 16, device=dev)
+    assert torch.equal(t, want)
+
+
 @pytest.mark.parametrize("src,dst", [(torch.int32, torch.float32), (torch.float32, torch.float16),
                                      (torch.float32, torch.bfloat16), (torch.float16, torch.float32),
                                      (torch.float64, torch.int64), (torch.bfloat16, torch.float16)])

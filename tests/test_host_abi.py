@@ -229,6 +229,24 @@ def test_grid_translation_per_kernel_family(fake_hip):
     assert rec.symbol == b"linear_tile_entry__mxfp8_f32_32x32x128_w1x1" and tuple(rec.grid) == (1, 1, 1)
 
 
+def test_eye_launcher_on_the_recording_runtime(fake_hip):
+    ct = fake_hip
+    t = torch.zeros(40, 72)
+    ct.eye(ct.partition(t, [16, 16]), generics=[16, 16])
+    rec, args = _last(ct)
+    assert rec.symbol == b"eye_entry__f32" and tuple(rec.block) == (256, 1, 1) and tuple(rec.grid) == (3, 1, 1)   # ceil(40*72 / 1024)
+    ptr, s0, s1, st0, st1, p0, p1, _ps0, _ps1, gx, gy, gz, _ = struct.unpack("<Q8i4I", args)
+    assert ptr == t.data_ptr() and (s0, s1, st0, st1, p0, p1) == (40, 72, 72, 1, 16, 16) and (gx, gy, gz) == (3, 5, 1)
+    n = ct.lib().cutile_testing_launch_count()
+    with pytest.raises(ct.CutileError, match="must be f32"):
+        ct.eye(ct.partition(torch.zeros(16, 16, dtype=torch.half), [16, 16]))
+    with pytest.raises(ct.CutileError, match="generic BC"):
+        ct.eye(ct.partition(t, [16, 16]), generics=[16, 8])
+    with pytest.raises(ct.CutileError):
+        ct.eye(ct.partition(torch.zeros(64), [16]))                 # rank 1
+    assert ct.lib().cutile_testing_launch_count() == n
+
+
 def test_kernel_table_lookup_and_single_flight_module_load(fake_hip):
     ct = fake_hip
     L = ct.lib()
