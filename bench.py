@@ -162,6 +162,47 @@ class Softmax(RmsNorm):
                 "kind": "port", "sample": f"first {rows} of {self.m} rows"}, {"within_1_f16_ulp": ok}
 
 
+class RmsNormAllF16(RmsNorm):
+    """The benchmark program's own arithmetic (cutile-benchmarks/benches/rmsnorm.rs:20-66): every operation in f16,
+    BLOCK_SIZE = 512 as the benchmark sets it; the result must equal the oracle's bit for bit."""
+    name, dtype = "rms_norm_all_f16_16384x8192", "f16 throughout"
+    config = {"workload": "RMSNorm fp16 rows [16384, 8192], weight [8192], eps 1e-5, all-f16 arithmetic, BLOCK_SIZE 512"}
+
+    def launch(self):
+        self.ct.rms_norm_all_f16(self.x, self.w, self.op, 1e-5, generics=[self.n, 512])
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 1024
+        t0 = time.perf_counter()
+        ref = oracle.rms_norm_all_f16(self.xb[:rows], self.wb, 1e-5, 512)
+        dt = time.perf_counter() - t0
+        got = self.o[:rows].cpu().numpy().view(np.uint16)
+        return {"value": (2 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {rows} of {self.m} rows (numpy, one f16 rounding per operation)"}, {"bit_exact": bool(np.array_equal(got, ref))}
+
+
+class SoftmaxAllF16(Softmax):
+    """cutile-benchmarks/benches/softmax.rs:19-35 with its own arithmetic: every operation in f16."""
+    name, dtype = "softmax_all_f16_16384x8192", "f16 throughout"
+    config = {"workload": "row softmax fp16 [16384, 8192], tiles [1, 8192], all-f16 arithmetic"}
+
+    def launch(self):
+        self.ct.softmax_all_f16(self.x, self.op)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = 1024
+        t0 = time.perf_counter()
+        ref = oracle.softmax_all_f16(self.xb[:rows], 1, self.n)
+        dt = time.perf_counter() - t0
+        got = self.o[:rows].cpu().numpy().view(np.uint16)
+        def ordered(u):
+            u = u.astype(np.int32)
+            return np.where(u & 0x8000, -(u & 0x7FFF), u)
+        d = np.abs(ordered(got) - ordered(ref))
+        return {"value": (2 * rows * self.n * 2) / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {rows} of {self.m} rows (numpy, one f16 rounding per operation)"}, {"within_2_f16_steps": bool(d.max() <= 2)}
+
+
 class Gemm(Workload):
     unit, dtype, bound, peak_key = "TFLOP/s", "bf16 in / f32 acc / bf16 out", "mfma", "mfma_bf16"
     tile = (256, 256)
@@ -828,7 +869,7 @@ class EmbeddingBatch(Workload):
 
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            Copy(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
+            Copy(), RmsNormAllF16(), SoftmaxAllF16(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
 
 
 EXTRA_WORKLOADS = []  # only by name, never in the default run

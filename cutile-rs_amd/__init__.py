@@ -117,6 +117,8 @@ def lib() -> C.CDLL:
             "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
             "cutile_launch_rms_norm_f32": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
             "cutile_launch_softmax": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_rms_norm_all_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
+            "cutile_launch_softmax_all_f16": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_add_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
                                                P(PartitionArg), f32, P(LaunchOpts)],
             "cutile_launch_qk_norm_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg),
@@ -408,6 +410,21 @@ def rms_norm_f32(x, w, out: Partition, eps: float, *, stream=None, grid=None, ge
     xa, wa = tensor_arg(x), tensor_arg(w)
     check(lib().cutile_launch_rms_norm_f32(_stream(stream), C.byref(xa), C.byref(wa), C.byref(out.arg()), float(eps),
                                            C.byref(o)))
+
+
+def rms_norm_all_f16(x, w, out: Partition, eps: float, *, generics, stream=None, grid=None) -> None:
+    """cutile-benchmarks/benches/rmsnorm.rs:20-66: every operation in f16; generics = [N, BLOCK_SIZE]."""
+    o, _k = _opts(grid, generics, None)
+    xa, wa = tensor_arg(x), tensor_arg(w)
+    check(lib().cutile_launch_rms_norm_all_f16(_stream(stream), C.byref(xa), C.byref(wa), C.byref(out.arg()), float(eps),
+                                               C.byref(o)))
+
+
+def softmax_all_f16(x, y: Partition, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-benchmarks/benches/softmax.rs:19-35 with its own arithmetic: every operation in f16."""
+    o, _k = _opts(grid, generics, None)
+    xa = tensor_arg(x)
+    check(lib().cutile_launch_softmax_all_f16(_stream(stream), C.byref(xa), C.byref(y.arg()), C.byref(o)))
 
 
 def softmax(x, y: Partition, *, stream=None, grid=None, generics=None, variant=None) -> None:

@@ -99,6 +99,13 @@ std::vector<KernelEntry> build_table() {
   add("rng_fill", "f64", "rng_fill_entry__f64", IMG_RNG, 256, 0, 0, 0, 0, 0, "f64", 0, 1);
   add("linspace", "f32", "linspace_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
   add("eye", "f32", "eye_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
+  // the benchmark programs' all-f16 arithmetic (one wavefront per row; v = tile lanes per lane, c = 512-wide chunks)
+  for (int v : {1, 2, 4, 8, 16})
+    add("rms_norm_all_f16", keep("v" + std::to_string(v)), keep("rms_norm_all_f16_entry__v" + std::to_string(v)), IMG_ROWWISE, 256, 0, 0, 0, 0,
+        0, "f16", 0, 2);
+  for (auto cv : {std::pair<int, int>{1, 1}, {1, 2}, {1, 4}, {1, 8}, {2, 8}, {4, 8}, {8, 8}, {16, 8}, {32, 8}})
+    add("softmax_all_f16", keep("c" + std::to_string(cv.first) + "v" + std::to_string(cv.second)),
+        keep("softmax_all_f16_entry__c" + std::to_string(cv.first) + "v" + std::to_string(cv.second)), IMG_ROWWISE, 256, 0, 0, 0, 0, 0, "f16", 0, 2);
   static const char* kConvertTypes[] = {"f32", "f64", "f16", "bf16", "i32", "i64"};
   for (const char* s : kConvertTypes)
     for (const char* d : kConvertTypes)

@@ -807,6 +807,91 @@ cutile_status_t cutile_launch_rms_norm_f32(cutile_stream_t stream, const cutile_
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 
+// rms_norm<N, BLOCK_SIZE> of cutile-benchmarks/benches/rmsnorm.rs:20-66: every operation in f16.  One wavefront per
+// row, BLOCK_SIZE / 64 tile lanes per lane; the tile's reduce_sum is the stride-halving tree over BLOCK_SIZE lanes.
+static bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+cutile_status_t cutile_launch_rms_norm_all_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* w,
+                                               const cutile_partition_arg_t* out, float eps, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(w, "w", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 2, 2)) return s;
+  const cutile_tensor_arg_t& ot = out->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F16 && w->dtype == CUTILE_DTYPE_F16 && ot.dtype == CUTILE_DTYPE_F16,
+                 CUTILE_ERR_KERNEL_LAUNCH, "rms_norm_all_f16: x, w and out must be f16");
+  const int32_t n = x->shape[1];
+  CUTILE_REQUIRE(w->shape[0] == n, CUTILE_ERR_KERNEL_LAUNCH, "rms_norm_all_f16: w has %d elements, expected N = %d", w->shape[0], n);
+  CUTILE_REQUIRE(out->partition_shape[0] == 1 && out->partition_shape[1] == n, CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_all_f16: out must be partitioned [1, %d], got [%d, %d]", n, out->partition_shape[0],
+                 out->partition_shape[1]);
+  CUTILE_REQUIRE(ot.shape[1] == n && ot.shape[0] <= x->shape[0], CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_all_f16: out is [%d, %d] but x is [%d, %d]", ot.shape[0], ot.shape[1], x->shape[0], n);
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(n), "N")) return s;
+  const int block = generic_int(opts, 1, 0);
+  CUTILE_REQUIRE(block > 0, CUTILE_ERR_KERNEL_LAUNCH,
+                 "rms_norm_all_f16: the generics [N, BLOCK_SIZE] are required (BLOCK_SIZE is the width of the f16 accumulator tile)");
+  CUTILE_REQUIRE(is_pow2(block) && block <= 1024 && n >= block && n % block == 0, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "rms_norm_all_f16: BLOCK_SIZE = %d must be a power of two, at most 1024, that divides N = %d", block, n);
+  const int v = std::max(1, block / 64);
+  CUTILE_REQUIRE(x->strides[1] == 1 && ot.strides[1] == 1 && w->strides[0] == 1 && x->strides[0] % v == 0 && ot.strides[0] % v == 0 &&
+                     ((uintptr_t)x->ptr | (uintptr_t)ot.ptr | (uintptr_t)w->ptr) % (2 * (uintptr_t)std::min(v, 8)) == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "rms_norm_all_f16: rows must be contiguous and aligned to %d bytes", 2 * std::min(v, 8));
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  const std::string variant = "v" + std::to_string(v);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("rms_norm_all_f16", &o, variant, {variant}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*x);
+  args.push_tensor(*w);
+  args.push_partition(*out);
+  args.push_val<float>(eps);
+  args.push_val<int32_t>(block);
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>(tg[0], ot.shape[0]);
+  uint32_t grid[3] = {(uint32_t)std::min<uint64_t>(std::max<uint64_t>(div_up(rows, 4), 1), 1u << 20), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
+// softmax<BM, BN> of cutile-benchmarks/benches/softmax.rs:19-35: every operation in f16.  One wavefront per tile row.
+cutile_status_t cutile_launch_softmax_all_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x, const cutile_partition_arg_t* y,
+                                              const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_partition(y, "y", 2, 2)) return s;
+  const cutile_tensor_arg_t& yt = y->tensor;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F16 && yt.dtype == CUTILE_DTYPE_F16, CUTILE_ERR_KERNEL_LAUNCH,
+                 "softmax_all_f16: x and y must be f16");
+  const int32_t bm = y->partition_shape[0], bn = y->partition_shape[1];
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bn), "BN")) return s;
+  CUTILE_REQUIRE(is_pow2(bn) && bn <= 16384, CUTILE_ERR_KERNEL_NOT_FOUND,
+                 "softmax_all_f16: BN = %d must be a power of two, at most 16384 (the row is held in one wavefront's registers)", bn);
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(y, opts, tg)) return s;
+  const uint64_t rows = std::min<uint64_t>((uint64_t)tg[0] * bm, yt.shape[0]);
+  const int v = bn >= 512 ? 8 : std::max(1, bn / 64), ch = bn >= 512 ? bn / 512 : 1;
+  CUTILE_REQUIRE(x->shape[1] == yt.shape[1] && (uint64_t)x->shape[0] >= rows, CUTILE_ERR_KERNEL_LAUNCH,
+                 "softmax_all_f16: x is [%d, %d] but y is [%d, %d]", x->shape[0], x->shape[1], yt.shape[0], yt.shape[1]);
+  CUTILE_REQUIRE(x->strides[1] == 1 && yt.strides[1] == 1 && x->strides[0] % v == 0 && yt.strides[0] % v == 0 &&
+                     ((uintptr_t)x->ptr | (uintptr_t)yt.ptr) % (2 * (uintptr_t)v) == 0,
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "softmax_all_f16: rows must be contiguous and aligned to %d bytes", 2 * v);
+  cutile_launch_opts_t o = opts ? *opts : cutile_launch_opts_t{};
+  o.generics = nullptr;
+  o.n_generics = 0;
+  const std::string variant = "c" + std::to_string(ch) + "v" + std::to_string(v);
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("softmax_all_f16", &o, variant, {variant}, &res)) return s;
+  ArgPacker args;
+  args.push_tensor(*x);
+  args.push_partition(*y);
+  args.push_tile_grid(tg);
+  const uint64_t segments = rows * tg[1];
+  uint32_t grid[3] = {(uint32_t)std::min<uint64_t>(std::max<uint64_t>(div_up(segments, 4), 1), 1u << 20), 1, 1};
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 // The two fused row norms: same shape rules and variant choice as rms_norm_f16.
 static cutile_status_t launch_fused_norm(const char* fn, cutile_stream_t stream, const cutile_tensor_arg_t* a,
                                          const cutile_tensor_arg_t* b, const cutile_tensor_arg_t* w,

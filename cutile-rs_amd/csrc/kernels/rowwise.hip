@@ -618,6 +618,273 @@ extern "C" __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// ---- the benchmark programs' all-f16 arithmetic ------------------------------------------------
+namespace {
+// cutile-benchmarks/benches/rmsnorm.rs:20-66 and benches/softmax.rs:19-35 are written entirely in f16: every
+// product, sum, quotient and the square root are f16 operations.  The kernels above compute the statistics in
+// f32 (the arithmetic of cutile-kernels/src/norms.rs and of the examples); the two below reproduce the
+// benchmark programs' own arithmetic, one rounding to f16 per operation, no fused multiply-add.
+//
+// The tile programs leave one thing to their compiler: the order in which reduce_sum adds the lanes of a
+// tile.  The order here is the stride-halving tree: for step = L/2, L/4, .. 1: a[l] += a[l + step] (l < step)
+// over the L lanes of the tile.  A wavefront owns one row; lane t holds the V consecutive tile lanes
+// V*t .. V*t+V-1 (and, for a softmax row longer than 512, the same lanes of every 512-wide chunk), so the
+// tree's large steps are in-register adds across chunks, the middle steps cross-lane exchanges (both partners
+// compute the same IEEE sum, addition being commutative) and the last steps adds inside a lane.
+__device__ __forceinline__ _Float16 shfl_xor_f16(_Float16 v, int mask) {
+  const int bits = (int)__builtin_bit_cast(uint16_t, v);
+  return __builtin_bit_cast(_Float16, (uint16_t)__shfl_xor(bits, mask, 64));
+}
+// Cross-lane exchange of V halves, two per 32-bit exchange.
+template <int V>
+__device__ __forceinline__ auto shfl_xor_hv(_Float16 __attribute__((ext_vector_type(V))) v, int mask) {
+  typedef _Float16 hv __attribute__((ext_vector_type(V)));
+  if constexpr (V == 1) {
+    hv r;
+    r[0] = shfl_xor_f16(v[0], mask);
+    return r;
+  } else {
+    typedef int iv __attribute__((ext_vector_type(V / 2)));
+    iv bits = __builtin_bit_cast(iv, v);
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) bits[i] = __shfl_xor(bits[i], mask, 64);
+    return __builtin_bit_cast(hv, bits);
+  }
+}
+// a / b rounded once to f16: the correctly rounded f32 quotient of two f16 values rounds to the correctly rounded
+// f16 quotient (24 >= 2 * 11 + 2 bits).  The empty asm keeps the division an f32 division: folded into an f16
+// division the compiler may use the f16 reciprocal, which is accurate to one unit in the last place only.
+__device__ __forceinline__ _Float16 div_f16(_Float16 a, _Float16 b) {
+  float q = (float)a / (float)b;
+  asm volatile("" : "+v"(q));
+  return (_Float16)q;
+}
+// sqrt(v) rounded toward minus infinity in f16 (rounding::NegativeInf of the tile program): the f32 square
+// root of an f16 value, truncated to f16, is at most one f16 step above the exact floor, and exactly when its
+// square (exact in f32: 22 bits) exceeds v.
+__device__ __forceinline__ _Float16 sqrt_f16_toward_minus_infinity(_Float16 v) {
+  const float f = __builtin_sqrtf((float)v);
+  if (!(f <= 65504.0f) || f == 0.0f) return (_Float16)f;          // NaN (negative input), +inf, +-0
+  uint16_t bits = (uint16_t)((__builtin_bit_cast(uint32_t, f) >> 13) - (112u << 10));   // truncation; sqrt of an f16 is a normal f16
+  const float h = (float)__builtin_bit_cast(_Float16, bits);
+  if (h * h > (float)v) bits -= 1;
+  return __builtin_bit_cast(_Float16, bits);
+}
+
+// rms_norm<N, BLOCK_SIZE> of cutile-benchmarks/benches/rmsnorm.rs:20-66.  V = tile lanes per lane of the
+// wavefront: BLOCK_SIZE = 64 * V, or BLOCK_SIZE <= 64 with V = 1 (the lanes beyond it hold zeros).
+template <int V>
+__device__ __forceinline__ void rms_norm_all_f16_rows(const TensorArg<2>& x, const TensorArg<1>& w, const PartitionArg<2>& out,
+                                                      float eps_f32, int32_t block_size, int64_t rows) {
+#pragma clang fp contract(off)
+  typedef _Float16 hv __attribute__((ext_vector_type(V)));
+  constexpr int kCached = V >= 16 ? 8 : 16;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int32_t n = x.shape[1], tiles = n / block_size;
+  const bool active = lane * V < block_size;
+  const _Float16 eps = (_Float16)eps_f32;
+  for (int64_t row = (int64_t)blockIdx.x * kWaves + wave; row < rows; row += (int64_t)gridDim.x * kWaves) {
+    const _Float16* xr = (const _Float16*)x.ptr + row * x.strides[0];
+    _Float16* orow = (_Float16*)out.ptr + row * out.strides[0];
+    _Float16 acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = (_Float16)0.0f;
+    // The first kCached tiles of the row stay in registers for the second pass (all of a row of up to
+    // kCached * BLOCK_SIZE elements: read from memory once); their loads are issued together.
+    hv cached[kCached];
+    if (active) {
+#pragma unroll
+      for (int j = 0; j < kCached; ++j)     // tiles past the row's end repeat the last one (loaded, never used)
+        cached[j] = __builtin_nontemporal_load(reinterpret_cast<const hv*>(xr + (int64_t)min(j, tiles - 1) * block_size + lane * V));
+#pragma unroll
+      for (int j = 0; j < kCached; ++j)
+        if (j < tiles) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            const _Float16 sq = cached[j][e] * cached[j][e];
+            acc[e] = acc[e] + sq;
+          }
+        }
+      for (int32_t j = kCached; j < tiles; ++j) {
+        const hv t = *reinterpret_cast<const hv*>(xr + (int64_t)j * block_size + lane * V);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const _Float16 sq = t[e] * t[e];
+          acc[e] = acc[e] + sq;
+        }
+      }
+    }
+    {
+      hv av;
+#pragma unroll
+      for (int e = 0; e < V; ++e) av[e] = acc[e];
+#pragma unroll
+      for (int step = 32; step >= 1; step >>= 1) av = av + shfl_xor_hv<V>(av, step);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = av[e];
+    }
+#pragma unroll
+    for (int step = V / 2; step >= 1; step >>= 1)
+#pragma unroll
+      for (int e = 0; e < step; ++e) acc[e] = acc[e] + acc[e + step];
+    // rms = sqrt(1 / (sum / N + eps)), each step an f16 operation (:46-52)
+    const _Float16 mean = div_f16(acc[0], (_Float16)(float)n);
+    const _Float16 denom = mean + eps;
+    const _Float16 inv = div_f16((_Float16)1.0f, denom);
+    const _Float16 scale = sqrt_f16_toward_minus_infinity(inv);
+    if (active) {
+      auto emit = [&](int32_t j, const hv& t, const hv& tw) {
+        hv o;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const _Float16 scaled = t[e] * scale;
+          o[e] = scaled * tw[e];
+        }
+        __builtin_nontemporal_store(o, reinterpret_cast<hv*>(orow + (int64_t)j * block_size + lane * V));
+      };
+      const _Float16* wl = (const _Float16*)w.ptr + lane * V;
+      // The weights of the cached tiles come four tiles at a time, the next four on their way while these are used
+      // (tiles past the row's end repeat the last one: loaded, never used).
+      constexpr int kGroup = 4, kGroups = kCached / kGroup;
+      hv wc[2][kGroup];
+      auto fetch_w = [&](int g) {
+#pragma unroll
+        for (int i = 0; i < kGroup; ++i) wc[g & 1][i] = *reinterpret_cast<const hv*>(wl + (int64_t)min(g * kGroup + i, tiles - 1) * block_size);
+      };
+      fetch_w(0);
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) {
+        if (g + 1 < kGroups) fetch_w(g + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < kGroup; ++i)
+          if (g * kGroup + i < tiles) emit(g * kGroup + i, cached[g * kGroup + i], wc[g & 1][i]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      for (int32_t j = kCached; j < tiles; ++j)
+        emit(j, *reinterpret_cast<const hv*>(xr + (int64_t)j * block_size + lane * V), *reinterpret_cast<const hv*>(wl + (int64_t)j * block_size));
+    }
+  }
+}
+
+// softmax<BM, BN> of cutile-benchmarks/benches/softmax.rs:19-35 over one tile row (a "segment" of BN columns):
+// CH chunks of 64 * V columns.  Columns of the tile beyond the tensor read 0 and take part (padding::Zero).
+template <int CH, int V>
+__device__ __forceinline__ void softmax_all_f16_segments(const TensorArg<2>& x, const PartitionArg<2>& y, int32_t segs_per_row,
+                                                         int64_t n_segments) {
+#pragma clang fp contract(off)
+  typedef _Float16 hv __attribute__((ext_vector_type(V)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int32_t bn = y.pshape[1], n_cols = x.shape[1];
+  const bool active = lane * V < bn;
+  for (int64_t seg = (int64_t)blockIdx.x * kWaves + wave; seg < n_segments; seg += (int64_t)gridDim.x * kWaves) {
+    const int64_t row = seg / segs_per_row;
+    const int32_t col0 = (int32_t)(seg % segs_per_row) * bn;
+    const _Float16* xr = (const _Float16*)x.ptr + row * x.strides[0];
+    _Float16* yr = (_Float16*)y.ptr + row * y.strides[0];
+    hv a[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int32_t col = col0 + c * 64 * V + lane * V;
+      if (active && col + V <= n_cols) {
+        a[c] = __builtin_nontemporal_load(reinterpret_cast<const hv*>(xr + col));   // streamed: read once
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) a[c][e] = (active && col + e < n_cols) ? xr[col + e] : (_Float16)0.0f;
+      }
+    }
+    hv mv = a[0];
+#pragma unroll
+    for (int c = 1; c < CH; ++c) mv = __builtin_elementwise_max(mv, a[c]);
+    _Float16 mx = mv[0];
+#pragma unroll
+    for (int e = 1; e < V; ++e) mx = mv[e] > mx ? mv[e] : mx;
+    if (!active) mx = (_Float16)(-__builtin_inff());
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) {
+      const _Float16 o = shfl_xor_f16(mx, step);
+      mx = o > mx ? o : mx;
+    }
+    // num = exp(x - max): the difference is an f16 operation, the exponential is evaluated in f32 and rounded once
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const hv d = a[c] - mx;
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[c][e] = active ? (_Float16)__builtin_amdgcn_exp2f((float)d[e] * kLog2e) : (_Float16)0.0f;
+      __builtin_amdgcn_sched_barrier(0);      // chunk by chunk: the f32 intermediates of one chunk only are live
+    }
+    // denom = reduce_sum(num): chunks first (the tree's largest steps), then across lanes, then inside the lane
+    constexpr int H = CH > 1 ? CH / 2 : 1;
+    hv t[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) t[c] = CH > 1 ? a[c] + a[c + H] : a[c];
+#pragma unroll
+    for (int step = H / 2; step >= 1; step >>= 1)
+#pragma unroll
+      for (int c = 0; c < step; ++c) t[c] = t[c] + t[c + step];
+    hv tot = t[0];
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) tot = tot + shfl_xor_hv<V>(tot, step);
+#pragma unroll
+    for (int step = V / 2; step >= 1; step >>= 1)
+#pragma unroll
+      for (int e = 0; e < step; ++e) tot[e] = tot[e] + tot[e + step];
+    // num / denom, rounded once to f16: q0 = num * (1 / denom) corrected by its own residual is within 2^-24 (1 + 2^-20)
+    // of the quotient, and the quotient of two f16 values is either exactly on an f16 rounding boundary (then q is
+    // exact) or at least 2^-23 away from one, so q rounds to f16 as the exact quotient does.
+    const float denom = (float)tot[0];
+    const float recip = __builtin_amdgcn_rcpf(denom);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int32_t col = col0 + c * 64 * V + lane * V;
+      hv o;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float num = (float)a[c][e];
+        const float q0 = num * recip;
+        o[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(-q0, denom, num), recip, q0);
+      }
+      if (active && col + V <= n_cols) {
+        __builtin_nontemporal_store(o, reinterpret_cast<hv*>(yr + col));
+      } else if (active) {
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          if (col + e < n_cols) yr[col + e] = o[e];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+}  // namespace
+
+#define RMS_NORM_ALL_F16_KERNEL(V)                                                                                   \
+  extern "C" __global__ void __launch_bounds__(kThreads) rms_norm_all_f16_entry__v##V(                               \
+      TensorArg<2> x, TensorArg<1> w, PartitionArg<2> out, float eps, int32_t block_size, TileGrid g) {              \
+    rms_norm_all_f16_rows<V>(x, w, out, eps, block_size, min((int64_t)g.x, (int64_t)out.shape[0]));                  \
+  }
+RMS_NORM_ALL_F16_KERNEL(1)
+RMS_NORM_ALL_F16_KERNEL(2)
+RMS_NORM_ALL_F16_KERNEL(4)
+RMS_NORM_ALL_F16_KERNEL(8)
+RMS_NORM_ALL_F16_KERNEL(16)
+
+#define SOFTMAX_ALL_F16_KERNEL(CH, V)                                                                                \
+  extern "C" __global__ void __launch_bounds__(kThreads) softmax_all_f16_entry__c##CH##v##V(                         \
+      TensorArg<2> x, PartitionArg<2> y, TileGrid g) {                                                               \
+    const int64_t rows = min((int64_t)g.x * y.pshape[0], (int64_t)y.shape[0]);                                       \
+    softmax_all_f16_segments<CH, V>(x, y, (int32_t)g.y, rows * (int64_t)g.y);                                        \
+  }
+SOFTMAX_ALL_F16_KERNEL(1, 1)
+SOFTMAX_ALL_F16_KERNEL(1, 2)
+SOFTMAX_ALL_F16_KERNEL(1, 4)
+SOFTMAX_ALL_F16_KERNEL(1, 8)
+SOFTMAX_ALL_F16_KERNEL(2, 8)
+SOFTMAX_ALL_F16_KERNEL(4, 8)
+SOFTMAX_ALL_F16_KERNEL(8, 8)
+SOFTMAX_ALL_F16_KERNEL(16, 8)
+SOFTMAX_ALL_F16_KERNEL(32, 8)
+
 // softmax(x, y: [BM, BN] tiles).  g.x / g.y = tiles covered along rows / columns.
 #define SOFTMAX_KERNEL(T, NAME, WPR, VPL)                                                           \
   extern "C" __global__ void __launch_bounds__(kThreads)                                           \

@@ -451,6 +451,21 @@ cutile_status_t cutile_launch_rms_norm_f32(cutile_stream_t stream, const cutile_
  * cutile-examples/examples/softmax.rs:11-24 */
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
                                       const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts);
+/* The two benchmark programs with their own arithmetic: every product, sum, quotient and the square root an f16
+ * operation (one rounding each, no fused multiply-add), where the entries above keep the statistics in f32.
+ *   rms_norm<N, BLOCK_SIZE>(x, w, out: [1,N] tiles, eps: f16) — cutile-benchmarks/benches/rmsnorm.rs:20-66:
+ *     a BLOCK_SIZE-lane f16 accumulator of x^2 over the N / BLOCK_SIZE tiles, reduce_sum, 1 / (sum / N + eps),
+ *     square root rounded toward minus infinity, out = x * rms * w.  opts->generics = [N, BLOCK_SIZE] is required.
+ *   softmax<BM, BN>(x, y: [BM,BN] tiles) — cutile-benchmarks/benches/softmax.rs:19-35: exp(x - max) / sum, the
+ *     exponential evaluated in f32 and rounded once.
+ * The tile programs leave the order of reduce_sum over a tile's lanes to their compiler; here it is the
+ * stride-halving tree (a[l] += a[l + step], step = L/2 .. 1).  BLOCK_SIZE and BN must be powers of two
+ * (at most 1024 and 16384), rows contiguous. */
+cutile_status_t cutile_launch_rms_norm_all_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                               const cutile_tensor_arg_t* w, const cutile_partition_arg_t* out, float eps,
+                                               const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_softmax_all_f16(cutile_stream_t stream, const cutile_tensor_arg_t* x,
+                                              const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts);
 /* ---- transformer-block kernels of cutile-kernels (f16 IO, f32 math) ------ */
 /* add_rms_norm_f16<N, BLOCK_SIZE>(residual, x, w, out: [1,N] tiles, residual_out: [1,N] tiles, eps):
  * combined = residual + x; out = RMSNorm(combined) * w; residual_out = combined —

@@ -4,7 +4,11 @@ TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` an
 ``cpu_baseline`` leg of ``bench.py``; the shipped library never touches it.
 
 Every function follows the C declaration of the same name in ``oracle.h``, which cites
-the reference file:line it restates.
+the reference file:line it restates.  PARITY UNPINNED (the reference leaves the point to
+its compiler or to a vendor library, and holds no vector for it): the lane order of
+reduce_sum in ``rms_norm_all_f16`` / ``softmax_all_f16`` (stated above those functions), and
+the value stream of ``rng_fill`` against the vendor generator the reference calls (Philox
+itself is pinned by the Random123 known-answer vectors).
 """
 from __future__ import annotations
 
@@ -210,6 +214,74 @@ def rms_norm_f16_f64(x_bits, w_bits, eps: float) -> np.ndarray:
     out = np.empty_like(x)
     lib().orc_rms_norm_f16_f64(_p(x), _p(w), _p(out), rows, n, eps)
     return out
+
+
+# ---- the benchmark programs' all-f16 arithmetic (numpy; every operation rounded once to f16) -------------------
+# cutile-benchmarks/benches/rmsnorm.rs:20-66 and benches/softmax.rs:19-35 compute entirely in f16.  PARITY UNPINNED
+# against the reference for one choice both programs leave to their compiler: the order in which reduce_sum adds the
+# lanes of a tile.  The order restated here is the stride-halving tree (a[l] += a[l + step], step = L/2 .. 1).  The
+# softmax's f16 exp is evaluated in f32 and rounded once.  Everything else (the per-lane accumulation over tiles, the
+# scalar chain, the downward-rounded square root, the order of the two multiplications) is fixed by the programs.
+# An f32 operation on two f16 values, rounded to f16, is the correctly rounded f16 operation (24 >= 2 * 11 + 2 bits),
+# which is how every step below is computed.
+def _h(op, a, b):
+    with np.errstate(over="ignore", divide="ignore", invalid="ignore"):      # f16 overflow to inf is part of the arithmetic
+        return op(a.astype(np.float32), np.asarray(b, np.float16).astype(np.float32)).astype(np.float16)
+
+
+def _tree_sum_f16(a: np.ndarray) -> np.ndarray:
+    """stride-halving tree over the last axis (a power of two long), one f16 rounding per addition"""
+    step = a.shape[-1] // 2
+    while step >= 1:
+        a = _h(np.add, a[..., :step], a[..., step:2 * step])
+        step //= 2
+    return a[..., 0]
+
+
+def sqrt_f16_toward_minus_infinity(v: np.ndarray) -> np.ndarray:
+    """largest f16 whose square does not exceed v (rounding::NegativeInf): squares of f16 values are exact in f64"""
+    v = np.asarray(v, np.float16)
+    with np.errstate(invalid="ignore"):
+        r = np.sqrt(v.astype(np.float64)).astype(np.float16)                       # nearest: at most one step above the floor
+        above = np.isfinite(r) & (r.astype(np.float64) ** 2 > v.astype(np.float64))
+    return np.where(above, np.nextafter(r, np.float16(-np.inf)), r).astype(np.float16)
+
+
+def rms_norm_all_f16(x_bits, w_bits, eps: float, block: int) -> np.ndarray:
+    """cutile-benchmarks/benches/rmsnorm.rs:20-66 -> f16 bit patterns"""
+    x, w = _c(x_bits, np.uint16).view(np.float16), _c(w_bits, np.uint16).view(np.float16)
+    rows, n = x.shape
+    assert n % block == 0 and block & (block - 1) == 0
+    acc = np.zeros((rows, block), np.float16)
+    for j in range(n // block):                                  # rms = rms + tx * tx, lane by lane (:37-40)
+        t = x[:, j * block:(j + 1) * block]
+        acc = _h(np.add, acc, _h(np.multiply, t, t))
+    total = _tree_sum_f16(acc)                                   # reduce_sum (:43)
+    with np.errstate(divide="ignore", over="ignore", invalid="ignore"):
+        mean = _h(np.divide, total, np.float16(n))               # rms / n (:46-48)
+        inv = _h(np.divide, np.ones_like(mean), _h(np.add, mean, np.float16(eps)))
+        scale = sqrt_f16_toward_minus_infinity(inv)              # :49-50
+        out = _h(np.multiply, _h(np.multiply, x, scale[:, None]), w[None, :])   # tx * rms * tw (:62)
+    return out.view(np.uint16)
+
+
+def softmax_all_f16(x_bits, bm: int, bn: int) -> np.ndarray:
+    """cutile-benchmarks/benches/softmax.rs:19-35 over [bm, bn] tiles -> f16 bit patterns; columns of a tile beyond the
+    tensor read 0 and take part in max and sum"""
+    x = _c(x_bits, np.uint16).view(np.float16)
+    m, n = x.shape
+    assert bn & (bn - 1) == 0
+    tiles = -(-n // bn)
+    xp = np.zeros((m, tiles * bn), np.float16)
+    xp[:, :n] = x
+    seg = xp.reshape(m, tiles, bn)
+    mx = seg.max(axis=2, keepdims=True)
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore"):
+        d = _h(np.subtract, seg, mx)
+        num = np.exp(d.astype(np.float32)).astype(np.float16)
+        den = _tree_sum_f16(num)[..., None]
+        y = _h(np.divide, num, den)
+    return np.ascontiguousarray(y.reshape(m, tiles * bn)[:, :n]).view(np.uint16)
 
 
 # ---- transformer-block kernels ---------------------------------------------------------------

@@ -2,6 +2,9 @@
 the reference's own tests hold for this path, against library routines (numpy / torch /
 scipy) and against what the mathematics fixes.  Each check is chosen so that a plausible
 slip (dropped term, wrong sign or index, transposed operand, wrong rounding) fails it."""
+import math
+from fractions import Fraction
+
 import numpy as np
 import pytest
 import torch
@@ -305,3 +308,94 @@ def test_rms_norm_f32_example_rounds_its_square_root_down():
     # against float64 as a whole
     ref = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + 1e-6) * w
     assert np.max(np.abs(out - ref) / np.abs(ref).max()) < 1e-6
+
+
+# ---- the benchmark programs' all-f16 arithmetic ---------------------------------------------------------------
+def _rn_f16(q: Fraction) -> Fraction:
+    """round-to-nearest-even of a non-negative rational to the f16 grid (normal and subnormal range, no overflow)"""
+    if q == 0:
+        return Fraction(0)
+    e = max(math.floor(math.log2(q)), -14)
+    while Fraction(2) ** e > q and e > -14:
+        e -= 1
+    while Fraction(2) ** (e + 1) <= q:
+        e += 1
+    ulp = Fraction(2) ** (e - 10)
+    k = q / ulp
+    lo = math.floor(k)
+    k = lo + 1 if (k - lo > Fraction(1, 2) or (k - lo == Fraction(1, 2) and lo % 2 == 1)) else lo
+    return k * ulp
+
+
+def test_f16_square_root_rounded_down_over_every_positive_f16():
+    v = np.arange(0, 0x7C01, dtype=np.uint16).view(np.float16)          # +0 .. +inf
+    r = oracle.sqrt_f16_toward_minus_infinity(v)
+    fin = np.isfinite(v)
+    r64, v64 = r.astype(np.float64)[fin], v.astype(np.float64)[fin]     # squares of f16 values are exact in f64
+    up = np.nextafter(r, np.float16(np.inf)).astype(np.float64)[fin]
+    assert (r64 ** 2 <= v64).all() and (up ** 2 > v64).all()
+    assert np.isinf(r[-1]) and np.isnan(oracle.sqrt_f16_toward_minus_infinity(np.float16(-1.0)))
+
+
+def test_all_f16_rms_norm_against_exact_rational_arithmetic_rounded_step_by_step():
+    # A row of constants makes every step of cutile-benchmarks/benches/rmsnorm.rs:37-62 checkable with exact rationals:
+    # lane sums, the tree, sum / N, + eps, 1 / x, the downward square root, x * rms * w.
+    n, block = 2048, 512
+    for xv, wv, eps in [(1.0, 1.0, 1e-5), (3.0, 0.5, 1e-5), (0.3330078125, 1.5, 1e-3), (5.25, 0.0999755859375, 1e-5)]:
+        x = np.full((2, n), xv, np.float16)
+        w = np.full(n, wv, np.float16)
+        got = oracle.rms_norm_all_f16(x.view(np.uint16), w.view(np.uint16), eps, block).view(np.float16)
+        fx, fw = Fraction(float(x[0, 0])), Fraction(float(w[0]))
+        lane = Fraction(0)
+        for _ in range(n // block):
+            lane = _rn_f16(lane + _rn_f16(fx * fx))
+        total, lanes = lane, block
+        while lanes > 1:                       # equal lanes: every tree level doubles, rounded
+            total, lanes = _rn_f16(total + total), lanes // 2
+        mean = _rn_f16(total / _rn_f16(Fraction(n)))
+        inv = _rn_f16(1 / _rn_f16(mean + Fraction(float(np.float16(eps)))))
+        grid = [Fraction(float(h)) for h in np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16)]
+        scale = max(h for h in grid if h * h <= inv)
+        want = _rn_f16(_rn_f16(fx * scale) * fw)
+        assert Fraction(float(got[0, 0])) == want and (got == got[0, 0]).all(), (xv, wv, float(got[0, 0]), float(want))
+    # the f16 sum of squares overflows early (17.5^2 * 2048 > 65504): inf -> 1 / inf = 0 -> every output is 0
+    x = np.full((1, n), 17.5, np.float16)
+    assert (oracle.rms_norm_all_f16(x.view(np.uint16), np.ones(n, np.float16).view(np.uint16), 1e-5, block) == 0).all()
+
+
+def test_all_f16_reduce_sum_is_the_stride_halving_tree():
+    # brute force with scalar f16 additions in the stated order, on lanes chosen so that the order matters
+    rng = np.random.default_rng(11)
+    lanes = (rng.standard_normal(64) * np.exp2(rng.integers(-6, 7, 64))).astype(np.float16)
+    a = [np.float16(v) for v in np.abs(lanes)]
+    step = 32
+    while step >= 1:
+        for l in range(step):
+            a[l] = np.float16(np.float32(a[l]) + np.float32(a[l + step]))
+        step //= 2
+    assert oracle._tree_sum_f16(np.abs(lanes)[None, :])[0] == a[0]
+    # through rms_norm_all_f16: one tile, x = sqrt of the lanes would not be exact, so check the softmax denominator
+    # instead: exp(0) = 1 everywhere -> the tree of ones is exact: every output is 1 / BN
+    y = oracle.softmax_all_f16(np.zeros((3, 256), np.float16).view(np.uint16), 1, 256).view(np.float16)
+    assert (y == np.float16(1 / 256)).all()
+
+
+def test_all_f16_forms_stay_near_the_float64_functions():
+    x = oracle.f32_to_f16_bits(oracle.normal_f32((16, 4096), 3))
+    w = oracle.f32_to_f16_bits(oracle.normal_f32((4096,), 4))
+    xf, wf = x.view(np.float16).astype(np.float64), w.view(np.float16).astype(np.float64)
+    o = oracle.rms_norm_all_f16(x, w, 1e-5, 512).view(np.float16).astype(np.float64)
+    ref = xf / np.sqrt((xf ** 2).mean(1, keepdims=True) + 1e-5) * wf
+    assert np.abs(o - ref).max() <= 4e-3 * np.abs(ref).max()              # f16 accumulation of 4096 squares: ~2^-9 relative
+    for bm, bn in [(1, 4096), (4, 1024), (2, 64)]:
+        y = oracle.softmax_all_f16(x, bm, bn).view(np.float16).astype(np.float64)
+        seg = xf.reshape(16, 4096 // bn, bn)
+        e = np.exp(seg - seg.max(2, keepdims=True))
+        sref = (e / e.sum(2, keepdims=True)).reshape(16, 4096)
+        assert np.abs(y - sref).max() <= 3e-3 * sref.max()
+    # ragged width: the last tile's missing columns read 0 and take part (exp(0 - max) joins the denominator)
+    xr = x[:, :100]
+    y = oracle.softmax_all_f16(xr, 1, 64).view(np.float16).astype(np.float64)
+    seg = np.concatenate([xf[:, 64:100], np.zeros((16, 28))], axis=1)
+    e = np.exp(seg - seg.max(1, keepdims=True))
+    assert np.abs(y[:, 64:] - (e / e.sum(1, keepdims=True))[:, :36]).max() <= 2e-3
