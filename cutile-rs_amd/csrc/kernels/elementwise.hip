@@ -340,10 +340,13 @@ extern "C" __global__ void __launch_bounds__(kThreads)
     const int64_t dst_k = (int64_t)h * k_cache.strides[0] + pos * k_cache.strides[1];
     const int64_t dst_v = (int64_t)h * v_cache.strides[0] + pos * v_cache.strides[1];
     if (vec) {
-      *reinterpret_cast<u32x4*>((_Float16*)k_cache.ptr + dst_k + c * 8) =
-          *reinterpret_cast<const u32x4*>((const _Float16*)new_k.ptr + src_k + c * 8);
-      *reinterpret_cast<u32x4*>((_Float16*)v_cache.ptr + dst_v + c * 8) =
-          *reinterpret_cast<const u32x4*>((const _Float16*)new_v.ptr + src_v + c * 8);
+      // Streamed both ways: the new rows are read once, and a plain load or store would take a place in the
+      // memory-side cache, pushing out whatever dirty lines the previous kernel left there at the cost of their
+      // write-back.
+      const u32x4 kv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const _Float16*)new_k.ptr + src_k + c * 8));
+      const u32x4 vv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const _Float16*)new_v.ptr + src_v + c * 8));
+      __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>((_Float16*)k_cache.ptr + dst_k + c * 8));
+      __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>((_Float16*)v_cache.ptr + dst_v + c * 8));
     } else {
       ((_Float16*)k_cache.ptr)[dst_k + (int64_t)c * k_cache.strides[2]] = ((const _Float16*)new_k.ptr)[src_k + (int64_t)c * new_k.strides[2]];
       ((_Float16*)v_cache.ptr)[dst_v + (int64_t)c * v_cache.strides[2]] = ((const _Float16*)new_v.ptr)[src_v + (int64_t)c * new_v.strides[2]];
@@ -833,7 +836,7 @@ extern "C" __global__ void __launch_bounds__(kThreads)
     if (vec) {
       for (int32_t c = threadIdx.x; c < width / 8; c += kThreads) {
         u32x4 v = {0, 0, 0, 0};
-        if (known && c * 8 < table.shape[1]) v = *(reinterpret_cast<const u32x4*>(src) + c);
+        if (known && c * 8 < table.shape[1]) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + c);
         __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst) + c);
       }
     } else {
