@@ -227,6 +227,7 @@ struct Fmha {
     float m_i = -INFINITY, l_i = 0.0f;
     const float c = qk_scale * kLog2e;  // qk_scale / ln 2
     const int32_t q_pos = q0 + l32 + input_pos;  // this lane's query position for the causal rule
+    const int32_t last_visible = (causal ? min(q_pos, k_len - 1) : k_len - 1) - half * 4;   // last key the lane may see
 
     if (tc > 0) {
       load_global(0);
@@ -253,15 +254,12 @@ struct Fmha {
         }
       }
       // s[sb][e] belongs to kv = j*BN + sb*32 + (e/4)*8 + half*4 + e%4, query = this lane's.
-      if (j >= mask_start) {
+      if (j >= mask_start) {   // visible iff the key's lane-independent index in the tile is <= lim: a compare and a select
+        const int32_t lim = last_visible - j * BN;
 #pragma unroll
         for (int sb = 0; sb < SB; ++sb)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            int32_t kv = j * BN + sb * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-            bool visible = kv < k_len && (!causal || q_pos >= kv);
-            s[sb][e] = visible ? s[sb][e] : -INFINITY;
-          }
+          for (int e = 0; e < 16; ++e) s[sb][e] = (sb * 32 + (e >> 2) * 8 + (e & 3)) <= lim ? s[sb][e] : -INFINITY;
       }
       float mx = -INFINITY;
 #pragma unroll
@@ -514,6 +512,8 @@ struct FmhaPingPong {
 #pragma unroll
     for (int e = 0; e < 16; ++e) neg_ref[e] = 0.0f;
     const int32_t q_pos = q0 + l32 + input_pos;
+    // Last key this lane may see, less the part of a key's index inside a tile that depends on the lane (half * 4).
+    const int32_t last_visible = (causal ? min(q_pos, k_len - 1) : k_len - 1) - half * 4;
 
     // Matrix segments.  Fragments are read kAhead steps before the MFMA that uses
     // them; sched_barrier(0) after every step keeps reads and MFMAs in this order.
@@ -555,14 +555,13 @@ struct FmhaPingPong {
     // (and on the first tile) the scores are shifted to the new reference and O, l are rescaled.  Otherwise p = 2^s.
     auto softmax_segment = [&](int32_t j) {
       if (j >= mask_start) {
+        // Key sb*32 + (e>>2)*8 + half*4 + (e&3) of this tile is visible iff it is <= last_visible: one compare
+        // against a constant and one select per element.
+        const int32_t lim = last_visible - j * BN;
 #pragma unroll
         for (int sb = 0; sb < SB; ++sb)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            int32_t kv = j * BN + sb * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-            bool visible = kv < k_len && (!causal || q_pos >= kv);
-            s[sb][e] = visible ? s[sb][e] : -INFINITY;
-          }
+          for (int e = 0; e < 16; ++e) s[sb][e] = (sb * 32 + (e >> 2) * 8 + (e & 3)) <= lim ? s[sb][e] : -INFINITY;
       }
       float mx = -INFINITY;
 #pragma unroll
