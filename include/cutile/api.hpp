@@ -566,6 +566,26 @@ struct RmsNormF32Fn {
     return cutile_launch_rms_norm_f32(s, &xa, &wa, &op, eps, o);
   }
 };
+// The benchmark programs with their own all-f16 arithmetic (cutile-benchmarks/benches/rmsnorm.rs:20-66,
+// benches/softmax.rs:19-35); .generics({N, BLOCK_SIZE}) is required for the RMSNorm form.
+struct RmsNormAllF16Fn {
+  static constexpr const char* name = "rms_norm";
+  template <class X, class W, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, W& w, O& out, float eps) {
+    auto xa = input_arg(x), wa = input_arg(w);
+    auto op = out.arg();
+    return cutile_launch_rms_norm_all_f16(s, &xa, &wa, &op, eps, o);
+  }
+};
+struct SoftmaxAllF16Fn {
+  static constexpr const char* name = "softmax";
+  template <class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, X& x, Yv& y) {
+    auto xa = input_arg(x);
+    auto yp = y.arg();
+    return cutile_launch_softmax_all_f16(s, &xa, &yp, o);
+  }
+};
 struct SoftmaxFn {
   static constexpr const char* name = "softmax";
   template <class X, class Yv>
@@ -809,6 +829,9 @@ template <class X, class W, class O> auto rms_norm_f16(X&& x, W&& w, O&& out, fl
 template <class X, class W, class O> auto rms_norm(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormF32Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
 // softmax(x, y: partition [BM,BN]) -> (x, y)    cutile-benchmarks/benches/softmax.rs:23-26
 template <class X, class Y> auto softmax(X&& x, Y&& y) { return make_launcher<kernels::SoftmaxFn>(std::forward<X>(x), std::forward<Y>(y)); }
+// the benchmark programs' all-f16 forms: rms_norm(x, w, out: [1,N], eps) with .generics({N, BLOCK_SIZE}); softmax(x, y: [BM,BN])
+template <class X, class W, class O> auto rms_norm_all_f16(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormAllF16Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
+template <class X, class Y> auto softmax_all_f16(X&& x, Y&& y) { return make_launcher<kernels::SoftmaxAllF16Fn>(std::forward<X>(x), std::forward<Y>(y)); }
 // gemm(z: partition [BM,BN], x, y, k) -> (z, x, y, k): z <- z + x·y   cutile-benchmarks/benches/gemm.rs:25-30
 template <class Z, class X, class Y> auto gemm(Z&& z, X&& x, Y&& y, int32_t k) { return make_launcher<kernels::GemmFn<true>>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), k); }
 // gemm_zero_init: accumulator starts at 0                              cutile-examples/examples/gemm.rs:20-36

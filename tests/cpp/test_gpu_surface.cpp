@@ -62,6 +62,28 @@ TEST(rms_norm_constant_rows) {
   for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 0.5f);  // x == c -> out = w
 }
 
+TEST(all_f16_benchmark_forms_closed_forms) {
+  // Constant rows make the f16 chain checkable by hand (values from exact rational arithmetic rounded step by step,
+  // tests/test_oracle.py): x = 1.7 (f16 1.7002), w = 0.5, N = 2048, BLOCK_SIZE 512 gives 0x37FF (0.49976) with the
+  // square root rounded toward minus infinity and 0x3800 (0.5) with it rounded to nearest; x = 6 overflows the f16
+  // sum of squares (36 * 2048 > 65504): inf -> 1 / inf = 0 -> every output is 0.
+  auto stream = new_stream();
+  auto w = api::full<f16>(0.5, {2048}).sync_on(stream).unwrap();
+  auto out = api::zeros<f16>({16, 2048}).sync_on(stream).unwrap();
+  auto x = api::full<f16>(1.7, {16, 2048}).sync_on(stream).unwrap();
+  CHECK(rms_norm_all_f16(&x, &w, out.partition_mut({1, 2048}), 1e-5f).generics({"2048", "512"}).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(v.bits == 0x37FF);
+  auto big = api::full<f16>(6.0, {16, 2048}).sync_on(stream).unwrap();
+  CHECK(rms_norm_all_f16(&big, &w, out.partition_mut({1, 2048}), 1e-5f).generics({"2048", "512"}).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(out).sync_on(stream).unwrap()) CHECK(v.bits == 0);
+  // BLOCK_SIZE is part of the arithmetic: leaving it out is an error, not a default
+  CHECK(rms_norm_all_f16(&x, &w, out.partition_mut({1, 2048}), 1e-5f).sync_on(stream).is_err());
+  // softmax of a constant row: exp(0) = 1, the tree of ones is exact, every output is 1 / BN
+  auto y = api::zeros<f16>({16, 2048}).sync_on(stream).unwrap();
+  CHECK(softmax_all_f16(&x, y.partition_mut({1, 512})).sync_on(stream).is_ok());
+  for (f16 v : api::to_host_vec(y).sync_on(stream).unwrap()) CHECK(f32_from_f16(v) == 1.0f / 512.0f);
+}
+
 TEST(transformer_block_kernels_closed_forms) {
   auto stream = new_stream();
   // add_rms_norm: residual = 1, x = 2 -> combined = 3 everywhere; out = w, residual_out = 3
