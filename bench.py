@@ -1065,13 +1065,22 @@ def same_kernel_zero_operands(ct, torch, flush):
                 "back_to_back_frac_of_2500": round(tf(runs[len(runs) // 2]) / 2500, 4)}
 
     out = {}
-    s = 8192
-    a = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
-    b = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
+    for s in (8192, 4096):
+        a = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
+        b = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
+        z = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
+        zp = ct.partition(z, [256, 256])
+        out[f"gemm_bf16_{s}"] = both(lambda: ct.gemm(zp, a, b, s, accumulate=True), 2.0 * s ** 3)
+        del a, b, z, zp
+    s = 8192                        # MXFP8: e4m3 zeros with unit scales (e8m0 127), priced at the fp8 peak
+    x = torch.zeros(s, s, dtype=torch.uint8, device="cuda")
+    sc = torch.full((s, s // 32), 127, dtype=torch.uint8, device="cuda")
     z = torch.zeros(s, s, dtype=torch.bfloat16, device="cuda")
     zp = ct.partition(z, [256, 256])
-    out["gemm_bf16_8192"] = both(lambda: ct.gemm(zp, a, b, s, accumulate=True), 2.0 * s ** 3)
-    del a, b, z, zp
+    r = both(lambda: ct.linear_tile_mxfp8(zp, x, x, sc, sc, 1.0), 2.0 * s ** 3)
+    out["mxfp8_gemm_8192"] = {"TFLOP/s": r["TFLOP/s"], "frac_of_5000": round(r["TFLOP/s"] / 5000, 4), "back_to_back_TFLOP/s": r["back_to_back_TFLOP/s"],
+                              "back_to_back_frac_of_5000": round(r["back_to_back_TFLOP/s"] / 5000, 4)}
+    del x, sc, z, zp
     bb, h, sq, d = Fmha.b, Fmha.h, Fmha.s, Fmha.d
     q, k, v = (torch.zeros(bb, h, sq, d, dtype=torch.bfloat16, device="cuda") for _ in range(3))
     o = torch.zeros(bb * h, sq, d, dtype=torch.bfloat16, device="cuda")
