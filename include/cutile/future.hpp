@@ -39,9 +39,9 @@ struct StreamCallbackState {
   }
 };
 
-// Microseconds to spin on the stream before registering for a notification
-// (device_future.rs:233-262); CUTILE_ASYNC_SPIN_BUDGET_US=0 forces every future
-// through the notification path.
+// Microseconds the first poll spins on the completion flag before it reports
+// "pending" and the caller parks (device_future.rs:233-262);
+// CUTILE_ASYNC_SPIN_BUDGET_US=0 sends every future through the parked path.
 inline uint64_t inline_spin_budget_us() {
   static const uint64_t budget = [] {
     const char* v = std::getenv("CUTILE_ASYNC_SPIN_BUDGET_US");
@@ -98,20 +98,6 @@ class DeviceFuture {
           return Result<T>(r.error());
         }
         result_.emplace(std::move(r).unwrap());
-        // Inline fast path: bounded spin on the stream before any registration.
-        if (uint64_t budget = inline_spin_budget_us()) {
-          auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(budget);
-          for (;;) {
-            auto q = ctx_->stream()->query();
-            if (q.is_err()) break;
-            if (q.value()) {
-              ExecutionLock::release();
-              state_ = DeviceFutureState::Complete;
-              return Result<T>(std::move(*result_));
-            }
-            if (std::chrono::steady_clock::now() >= deadline) break;
-          }
-        }
         // Register the completion signal, once.  The callback owns a reference
         // to the shared state, so it may fire after this future is gone.
         auto* held = new std::shared_ptr<StreamCallbackState>(cb_);
@@ -123,6 +109,19 @@ class DeviceFuture {
           return Result<T>(DeviceError::from_status(s));
         }
         state_ = DeviceFutureState::Executing;
+        // Inline fast path (device_future.rs:233-262 spins on the stream before registering): here the
+        // registration comes first, it is one 32-bit stream write into pinned memory, and the bounded spin
+        // watches the completion flag it leads to.  A hipStreamQuery poll loop reported the completion of one small
+        // kernel about 10 us later than this flag (22.6 against 13.0 us from launch), past the default budget, so
+        // short operations always fell through to the parked path.
+        if (uint64_t budget = inline_spin_budget_us()) {
+          auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(budget);
+          while (!cb_->complete.load(std::memory_order_acquire) && std::chrono::steady_clock::now() < deadline) {}
+          if (cb_->complete.load(std::memory_order_acquire)) {
+            state_ = DeviceFutureState::Complete;
+            return Result<T>(std::move(*result_));
+          }
+        }
         return std::nullopt;
       }
       case DeviceFutureState::Executing: {
