@@ -8,6 +8,8 @@
 #include <deque>
 #include <map>
 #include <mutex>
+#include <string>
+#include <unordered_map>
 
 // Code objects, embedded by embed.S (one ELF image per kernel source file).
 extern "C" {
@@ -298,10 +300,20 @@ const std::vector<KernelEntry>& kernel_table() {
   return table;
 }
 
+// (function, variant) -> entry.  Every launch looks its kernel up at least once, so the table is indexed once
+// (the first entry of a key wins, as a scan in table order would find it).
 const KernelEntry* find_entry(const char* function, const std::string& variant) {
-  for (const auto& e : kernel_table())
-    if (strcmp(e.function, function) == 0 && variant == e.variant) return &e;
-  return nullptr;
+  static const std::unordered_map<std::string, const KernelEntry*> index = [] {
+    std::unordered_map<std::string, const KernelEntry*> m;
+    for (const auto& e : kernel_table()) m.emplace(std::string(e.function) + '|' + e.variant, &e);
+    return m;
+  }();
+  std::string key;
+  key.reserve(strlen(function) + 1 + variant.size());
+  key.append(function).push_back('|');
+  key.append(variant);
+  auto it = index.find(key);
+  return it == index.end() ? nullptr : it->second;
 }
 
 std::string list_variants(const char* function) {
