@@ -105,3 +105,37 @@ def test_mxfp8_random_shapes(ct, dev, m, n, k, out_dtype):
     got = z.float().cpu().numpy()
     assert np.isfinite(got).all() and rel_l2(got, ref) <= 3e-2
     assert_rounded_close(got, ref, (256, 256), rel_ulp=1e-5 if out_dtype == torch.float32 else 2.0 ** -7, atol_frac=1e-4, what="mxfp8", mag=mag)
+
+
+DECODE_CASES = _cases(9005, 10, lambda r: (int(r.integers(1, 9)), [1, 2, 4, 8, 16][int(r.integers(0, 5))], [64, 128, 256][int(r.integers(0, 3))],
+                                           int(r.integers(1, 3000)), [16, 32, 64, 128][int(r.integers(0, 4))], int(r.integers(1, 20))))
+
+
+@pytest.mark.parametrize("heads,group,d,pos,bn,splits", DECODE_CASES)
+def test_decode_attention_random_shapes(ct, dev, heads, group, d, pos, bn, splits):
+    max_seq = pos + 1 + (pos * 7) % 50           # the cache holds rows past the newest key; they must not matter
+    q, k, v = normal_f16_bits((heads, group, d), 7000 + pos), normal_f16_bits((heads, max_seq, d), 7001 + pos), normal_f16_bits((heads, max_seq, d), 7002 + pos)
+    scale = float(np.float16(1.0 / np.sqrt(d)))
+    dv = lambda bits: torch.from_numpy(np.ascontiguousarray(bits).view(np.float16)).to(dev)
+    att = torch.full((heads, splits * group, d), float("nan"), dtype=torch.float16, device=dev)
+    lse = torch.full((heads, splits * group), float("nan"), dtype=torch.float32, device=dev)
+    out = torch.full((heads, group, d), float("nan"), dtype=torch.float16, device=dev)
+    p = torch.tensor([pos], dtype=torch.int32, device=dev)
+    ct.fmha_decode_gqa_split(dv(q), dv(k), dv(v), ct.partition(att, [1, group, d]), ct.partition(lse, [1, group]), scale, p,
+                             generics=[group, bn, d, splits])
+    ct.splitk_reduce_merge(att, lse, ct.partition(out, [1, group, d]), generics=[group, d, d, splits])
+    torch.cuda.synchronize()
+    att_ref, lse_ref = oracle.fmha_decode_gqa_split(q, k, v, scale, pos, bn, splits)
+    out_ref = oracle.splitk_reduce_merge(att_ref, lse_ref, group)
+    f32 = oracle.f16_bits_to_f32
+    got = out.cpu().numpy().view(np.uint16)
+    assert np.isfinite(f32(got)).all() and np.max(np.abs(f32(got) - f32(out_ref))) <= 2e-2
+    live = lse_ref > -1e29
+    assert np.array_equal(live, lse.cpu().numpy() > -1e29)
+    assert np.max(np.abs(lse.cpu().numpy()[live] - lse_ref[live])) <= 2e-3
+    # float64 softmax attention over keys 0..pos of each KV head
+    qf, kf, vf = f32(q).astype(np.float64), f32(k).astype(np.float64)[:, :pos + 1], f32(v).astype(np.float64)[:, :pos + 1]
+    sc = np.einsum("hgd,hkd->hgk", qf, kf) * scale
+    w = np.exp(sc - sc.max(-1, keepdims=True))
+    ref64 = np.einsum("hgk,hkd->hgd", w / w.sum(-1, keepdims=True), vf)
+    assert np.max(np.abs(f32(got) - ref64)) <= 2e-2
