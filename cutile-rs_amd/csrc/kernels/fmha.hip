@@ -84,6 +84,28 @@ struct Elem<_Float16> {
   }
 };
 
+// The two lanes that own one query row are 32 apart.  v_permlane32_swap exchanges the upper 32 lanes of its first
+// operand with the lower 32 of its second inside the vector ALU, where a lane-indexed permute would go through the
+// LDS crossbar and back (a wait of its own in the middle of every softmax segment).  Given two copies of v it leaves
+// the lower half's values in every lane of one register and the upper half's in the other; max and sum take both.
+// The instruction needs two idle issue cycles after a vector write of its operands (the s_nop in front).
+__device__ __forceinline__ void split_halves(float v, float* lower, float* upper) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+  *lower = a;
+  *upper = b;
+}
+__device__ __forceinline__ float max_across_halves(float v) {
+  float lo, hi;
+  split_halves(v, &lo, &hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum_across_halves(float v) {
+  float lo, hi;
+  split_halves(v, &lo, &hi);
+  return lo + hi;
+}
+
 // (batch*head, query tile) of this workgroup.  Workgroups are dealt round-robin to
 // the 8 XCDs in dispatch order; every query tile of one head is given to the same
 // XCD, consecutively, so that the head's K and V (read by each of its query
@@ -266,7 +288,7 @@ struct Fmha {
       for (int sb = 0; sb < SB; ++sb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[sb][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_across_halves(mx);
       // Statistics are kept in the scaled log2 domain: m = c * rowmax(raw).  The
       // reference point m only has to bound the exponents, not equal the maximum:
       // it moves (and the accumulators are rescaled) only when some row's maximum
@@ -297,7 +319,7 @@ struct Fmha {
           pf[sb * 2 + hh] = __builtin_bit_cast(vec8, w);
         }
       }
-      rs += __shfl_xor(rs, 32, 64);
+      rs = sum_across_halves(rs);
       if (moved) {
         const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
         l_i *= alpha;
@@ -568,7 +590,7 @@ struct FmhaPingPong {
       for (int sb = 0; sb < SB; ++sb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[sb][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_across_halves(mx);
       constexpr float kSlack = 8.0f;
       const float m_ref = m_i == -INFINITY ? 0.0f : m_i;       // what the accumulators started from
       const float m_cand = fmaxf(m_i, mx + m_ref);
@@ -609,7 +631,7 @@ struct FmhaPingPong {
           pf[sb * 2 + hh] = __builtin_bit_cast(vec8, w);
         }
       }
-      rs += __shfl_xor(rs, 32, 64);
+      rs = sum_across_halves(rs);
       l_i += rs;
     };
     auto interval_end = [&]() {
