@@ -95,6 +95,27 @@ __device__ __forceinline__ void split_halves(float v, float* lower, float* upper
   *lower = a;
   *upper = b;
 }
+// The same one level down: v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand with the even
+// rows of its second, so two copies of v become (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).
+__device__ __forceinline__ void split_row_pairs(float v, float* even, float* odd) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+  *even = a;
+  *odd = b;
+}
+// max / sum over the four lanes l, l^16, l^32, l^48
+__device__ __forceinline__ float max_across_rows(float v) {
+  float e, o, lo, hi;
+  split_row_pairs(v, &e, &o);
+  split_halves(fmaxf(e, o), &lo, &hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum_across_rows(float v) {
+  float e, o, lo, hi;
+  split_row_pairs(v, &e, &o);
+  split_halves(e + o, &lo, &hi);
+  return lo + hi;
+}
 __device__ __forceinline__ float max_across_halves(float v) {
   float lo, hi;
   split_halves(v, &lo, &hi);
@@ -1121,8 +1142,7 @@ __device__ __forceinline__ void decode_split_mfma_view(const DecodeSplitView& w,
         sv[blk * 4 + i] = valid ? sc[blk][i] * c : -INFINITY;
         mx = fmaxf(mx, sv[blk * 4 + i]);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_across_rows(mx);
     const float m_new = fmaxf(m, mx);
     const float alpha = __builtin_amdgcn_exp2f(m - m_new);
     float rs = 0.0f;
@@ -1133,8 +1153,7 @@ __device__ __forceinline__ void decode_split_mfma_view(const DecodeSplitView& w,
       rs += pv;
       pf[e] = (_Float16)pv;
     }
-    rs += __shfl_xor(rs, 16, 64);
-    rs += __shfl_xor(rs, 32, 64);
+    rs = sum_across_rows(rs);
     l = l * alpha + rs;
     if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
 #pragma unroll
