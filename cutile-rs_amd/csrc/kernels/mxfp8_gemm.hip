@@ -364,24 +364,28 @@ struct MxGemmDirect {
         for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
 
     i32x8 af[TM], bfr[TN];               // the one set of operand fragments
-    uint32_t sa_cur[TM], sb_cur[TN];     // scale dwords (4 MX blocks) of the tile whose first K step is next
+    // A row's 16 scale bytes for the four K tiles of a scale block, read once per block as one 16-byte LDS read
+    // (rows are 16 bytes apart: a wavefront's read is one contiguous 512-byte run, free of bank conflicts, where a
+    // dword per row and tile puts rows r and r+16 on the same bank); component p belongs to tile 4q + p.
+    u32x4 sa_blk[TM], sb_blk[TN];
     int sas[TM], sbs[TN];                // scales of a tile's second K step, already moved to byte 0
     // K step ks covers MX blocks 2ks and 2ks+1 of the tile; lanes 0-31 supply the scale
     // of the first, lanes 32-63 of the second, in byte 0 of the scale operand.
     const int sh0 = 8 * khalf, sh1 = 8 * (2 + khalf);
-    auto read_scales = [&](int32_t tile) {
-      const unsigned char* blk = scale_block(tile) + (tile & 3) * 4;
+    auto read_scale_block = [&](int32_t tile) {      // tile: a multiple of 4
+      const unsigned char* blk = scale_block(tile);
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) sa_cur[tm] = *reinterpret_cast<const uint32_t*>(blk + sa_addr + tm * 32 * 16);
+      for (int tm = 0; tm < TM; ++tm) sa_blk[tm] = *reinterpret_cast<const u32x4*>(blk + sa_addr + tm * 32 * 16);
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) sb_cur[tn] = *reinterpret_cast<const uint32_t*>(blk + sb_addr + tn * 32 * 16);
+      for (int tn = 0; tn < TN; ++tn) sb_blk[tn] = *reinterpret_cast<const u32x4*>(blk + sb_addr + tn * 32 * 16);
     };
     // MFMA j of a K step (outer-major) and, after it, the reload of whatever fragment it used last.
-    auto mfma_step = [&](int j, int ks) {
+    auto mfma_step = [&](int j, int ks, auto phase) {
+      constexpr int PH = decltype(phase)::value;
       const int o = j / NI, i = j % NI;
       const int tn = kOuterIsN ? o : i, tm = kOuterIsN ? i : o;
-      const int sb = ks == 0 ? (int)(sb_cur[tn] >> sh0) : sbs[tn];
-      const int sa = ks == 0 ? (int)(sa_cur[tm] >> sh0) : sas[tm];
+      const int sb = ks == 0 ? (int)(sb_blk[tn][PH] >> sh0) : sbs[tn];
+      const int sa = ks == 0 ? (int)(sa_blk[tm][PH] >> sh0) : sas[tm];
       acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0, sb, 0, sa);
     };
     auto reload_after = [&](int j, const unsigned char* stage, int ks) {
@@ -406,16 +410,18 @@ struct MxGemmDirect {
       for (int tm = 0; tm < TM; ++tm) af[tm] = read_a(stage0, 0, tm);
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) bfr[tn] = read_b(stage0, 0, tn);
-      read_scales(0);
+      read_scale_block(0);
     }
     constexpr int kHandOverAt = 3;   // MFMAs of the second K step issued before the hand-over
     // `with_scales`: tile kt+2 opens a scale block (kt + 2 is a multiple of 4).
-    auto k_tile = [&](unsigned char* cur, const unsigned char* nxt, int kt, auto with_scales) {
+    // `phase` = kt % 4 (the tile's place in its scale block), known where the call is written.
+    auto k_tile = [&](unsigned char* cur, const unsigned char* nxt, int kt, auto with_scales, auto phase) {
+      constexpr int PH = decltype(phase)::value;
       constexpr int NFT = NF + (decltype(with_scales)::value ? kSInstr : 0);
       // K step 0; fragments of step 1 are reloaded from `cur` as they free up.
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
-        mfma_step(j, 0);
+        mfma_step(j, 0, phase);
         __builtin_amdgcn_sched_barrier(0);   // the reload must follow the last reader, or it needs registers of its own
         reload_after(j, cur, 1);
         __builtin_amdgcn_sched_barrier(0);
@@ -423,23 +429,23 @@ struct MxGemmDirect {
       // K step 1; after the hand-over, fragments and scales of tile kt+1 come from
       // `nxt` and tile kt+2 is fetched into `cur`.
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm) sas[tm] = (int)(sa_cur[tm] >> sh1);
+      for (int tm = 0; tm < TM; ++tm) sas[tm] = (int)(sa_blk[tm][PH] >> sh1);
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) sbs[tn] = (int)(sb_cur[tn] >> sh1);
+      for (int tn = 0; tn < TN; ++tn) sbs[tn] = (int)(sb_blk[tn][PH] >> sh1);
 #pragma unroll
       for (int j = 0; j < kHandOverAt; ++j) {
-        mfma_step(j, 1);
+        mfma_step(j, 1, phase);
         __builtin_amdgcn_sched_barrier(0);
       }
       __builtin_amdgcn_s_waitcnt(0);   // own reads of `cur` done, own share of tile kt+1 landed
       __syncthreads();
-      read_scales(kt + 1);
+      if constexpr (PH == 3) read_scale_block(kt + 1);   // the next tile opens a scale block; this tile's second K step has its scales in sas / sbs
 #pragma unroll
       for (int j = kHandOverAt; j < NB; ++j) {
 #pragma unroll
         for (int i = 0; i < NFT; ++i)
           if (i * (NB - kHandOverAt) / NFT == j - kHandOverAt) fetch_one(cur, kt + 2, i);
-        mfma_step(j, 1);
+        mfma_step(j, 1, phase);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jj = 0; jj < NB; ++jj)   // reloads that fell before the hand-over are issued with the first MFMA after it
@@ -451,15 +457,19 @@ struct MxGemmDirect {
     // under a condition inside the loop the compiler would have to assume, at the
     // top of the loop, a refill of stage0 in flight and wait for it before every read.
     int kt = 0;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
+    using P3 = std::integral_constant<int, 3>;
     for (; kt + 4 <= k_tiles; kt += 4) {
-      k_tile(stage0, stage1, kt, std::false_type{});
-      k_tile(stage1, stage0, kt + 1, std::false_type{});
-      k_tile(stage0, stage1, kt + 2, std::true_type{});
-      k_tile(stage1, stage0, kt + 3, std::false_type{});
+      k_tile(stage0, stage1, kt, std::false_type{}, P0{});
+      k_tile(stage1, stage0, kt + 1, std::false_type{}, P1{});
+      k_tile(stage0, stage1, kt + 2, std::true_type{}, P2{});
+      k_tile(stage1, stage0, kt + 3, std::false_type{}, P3{});
     }
-    if (kt < k_tiles) k_tile(stage0, stage1, kt, std::false_type{});
-    if (kt + 1 < k_tiles) k_tile(stage1, stage0, kt + 1, std::false_type{});
-    if (kt + 2 < k_tiles) k_tile(stage0, stage1, kt + 2, std::true_type{});
+    if (kt < k_tiles) k_tile(stage0, stage1, kt, std::false_type{}, P0{});
+    if (kt + 1 < k_tiles) k_tile(stage1, stage0, kt + 1, std::false_type{}, P1{});
+    if (kt + 2 < k_tiles) k_tile(stage0, stage1, kt + 2, std::true_type{}, P2{});
 
     // Every wavefront is past its operand reads and every fetch has landed: the
     // stages are free to carry the output.
