@@ -50,16 +50,32 @@ union Vec16 {
   __device__ Vec16() : raw{} {}
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+// Sum / maximum over the 64 lanes, delivered to every lane, without leaving the vector ALU: inside a row of 16 lanes
+// by DPP (quad neighbours, then mirrored halves: every step pairs groups that already agree), across rows by
+// v_permlane16_swap / v_permlane32_swap (two copies of v in; the even rows' values in every lane of one register, the
+// odd rows' in the other; the instructions need two idle issue cycles after a vector write of their operands).  A
+// lane-indexed permute per step would take six trips through the LDS crossbar, each with a wait of its own.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+template <bool IS_MAX>
+__device__ __forceinline__ float combine(float a, float b) { return IS_MAX ? fmaxf(a, b) : a + b; }
+template <bool IS_MAX>
+__device__ __forceinline__ float wave_reduce(float v) {
+  v = combine<IS_MAX>(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+  v = combine<IS_MAX>(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+  v = combine<IS_MAX>(v, dpp_move<0x141>(v));   // row_half_mirror
+  v = combine<IS_MAX>(v, dpp_move<0x140>(v));   // row_mirror
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+  v = combine<IS_MAX>(a, b);
+  a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+  return combine<IS_MAX>(a, b);
 }
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce<false>(v); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
 
 // Reduction across the WPR wavefronts that share a segment.  `slot` is the
 // segment's index inside the workgroup, `sub` the wavefront's index inside the
