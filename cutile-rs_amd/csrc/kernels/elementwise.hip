@@ -19,6 +19,7 @@
 #include <hip/hip_bf16.h>
 
 #include "kernel_args.h"
+#include "lane_exchange.h"
 #include "mapped_partition.h"
 
 using namespace cutile;
@@ -713,8 +714,7 @@ __device__ __forceinline__ void lm_head_consume(const LmTile& w, float (&acc)[2]
   if (part + 1 < a.steps_per_pair) return;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) acc[t] += __shfl_xor(acc[t], o, 64);
+    acc[t] = lanes::across_wave<lanes::Sum>(acc[t]);
     if (a.lane == 0) a.row_logit[(pair * (kThreads / 64) + a.wave) * 2 + t] = acc[t];
     acc[t] = 0.0f;
   }
@@ -782,8 +782,7 @@ extern "C" __global__ void __launch_bounds__(kThreads)
       if (r < weights.shape[0])
         for (int32_t k = lane; k < k_len; k += 64)
           acc = __builtin_fmaf((float)wp[r * weights.strides[0] + (int64_t)k * weights.strides[1]], (float)hs[k], acc);
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      acc = lanes::across_wave<lanes::Sum>(acc);
       if (lane == 0) row_logit[wave * kLmRowsPerWave + rr] = acc;
     }
     __syncthreads();
@@ -899,7 +898,18 @@ __device__ __forceinline__ void fused_finish(const FusedRowsArgs& a, int64_t s_i
     const float l = (float)lo.v[e], h = (float)hi.v[e];
     ss += l * l + h * h;
   }
-  for (int32_t o = a.chunks >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  // the row's lanes are `chunks` neighbours (D / 16, a power of two; the same for every lane): quad steps, the mirrored
+  // halves of a row of 16 lanes, then whole rows
+  if (a.chunks >= 2) ss += lanes::dpp<lanes::kQuadXor1>(ss);
+  if (a.chunks >= 4) ss += lanes::dpp<lanes::kQuadXor2>(ss);
+  if (a.chunks >= 8) ss += lanes::dpp<lanes::kHalfMirror>(ss);
+  if (a.chunks >= 16) ss += lanes::dpp<lanes::kRowMirror>(ss);
+  if (a.chunks >= 32) {
+    float e, o;
+    lanes::split_row_pairs(ss, &e, &o);
+    ss = e + o;
+  }
+  if (a.chunks >= 64) ss = lanes::across_halves<lanes::Sum>(ss);
   if (r >= a.rows || (!is_q && (pos_i < 0 || pos_i >= a.max_seq))) return;
   _Float16* dst;
   if (is_q) {

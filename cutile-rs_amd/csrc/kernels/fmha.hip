@@ -30,6 +30,7 @@
 #include <utility>
 
 #include "kernel_args.h"
+#include "lane_exchange.h"
 
 using namespace cutile;
 
@@ -84,48 +85,14 @@ struct Elem<_Float16> {
   }
 };
 
-// The two lanes that own one query row are 32 apart.  v_permlane32_swap exchanges the upper 32 lanes of its first
-// operand with the lower 32 of its second inside the vector ALU, where a lane-indexed permute would go through the
-// LDS crossbar and back (a wait of its own in the middle of every softmax segment).  Given two copies of v it leaves
-// the lower half's values in every lane of one register and the upper half's in the other; max and sum take both.
-// The instruction needs two idle issue cycles after a vector write of its operands (the s_nop in front).
-__device__ __forceinline__ void split_halves(float v, float* lower, float* upper) {
-  float a = v, b = v;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
-  *lower = a;
-  *upper = b;
-}
-// The same one level down: v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand with the even
-// rows of its second, so two copies of v become (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).
-__device__ __forceinline__ void split_row_pairs(float v, float* even, float* odd) {
-  float a = v, b = v;
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
-  *even = a;
-  *odd = b;
-}
-// max / sum over the four lanes l, l^16, l^32, l^48
-__device__ __forceinline__ float max_across_rows(float v) {
-  float e, o, lo, hi;
-  split_row_pairs(v, &e, &o);
-  split_halves(fmaxf(e, o), &lo, &hi);
-  return fmaxf(lo, hi);
-}
-__device__ __forceinline__ float sum_across_rows(float v) {
-  float e, o, lo, hi;
-  split_row_pairs(v, &e, &o);
-  split_halves(e + o, &lo, &hi);
-  return lo + hi;
-}
-__device__ __forceinline__ float max_across_halves(float v) {
-  float lo, hi;
-  split_halves(v, &lo, &hi);
-  return fmaxf(lo, hi);
-}
-__device__ __forceinline__ float sum_across_halves(float v) {
-  float lo, hi;
-  split_halves(v, &lo, &hi);
-  return lo + hi;
-}
+// The two lanes that own one query row are 32 apart: their maximum and sum go through v_permlane32_swap, and the
+// four lanes of a head in the matrix-core decode kernel through v_permlane16_swap first (lane_exchange.h), inside the
+// vector ALU, where a lane-indexed permute would cost a trip through the LDS crossbar and a wait of its own in the middle
+// of every softmax segment.
+__device__ __forceinline__ float max_across_halves(float v) { return lanes::across_halves<lanes::Max>(v); }
+__device__ __forceinline__ float sum_across_halves(float v) { return lanes::across_halves<lanes::Sum>(v); }
+__device__ __forceinline__ float max_across_rows(float v) { return lanes::across_rows<lanes::Max>(v); }
+__device__ __forceinline__ float sum_across_rows(float v) { return lanes::across_rows<lanes::Sum>(v); }
 
 // (batch*head, query tile) of this workgroup.  Workgroups are dealt round-robin to
 // the 8 XCDs in dispatch order; every query tile of one head is given to the same

@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "kernel_args.h"
+#include "lane_exchange.h"
 
 using namespace cutile;
 
@@ -50,32 +51,9 @@ union Vec16 {
   __device__ Vec16() : raw{} {}
 };
 
-// Sum / maximum over the 64 lanes, delivered to every lane, without leaving the vector ALU: inside a row of 16 lanes
-// by DPP (quad neighbours, then mirrored halves: every step pairs groups that already agree), across rows by
-// v_permlane16_swap / v_permlane32_swap (two copies of v in; the even rows' values in every lane of one register, the
-// odd rows' in the other; the instructions need two idle issue cycles after a vector write of their operands).  A
-// lane-indexed permute per step would take six trips through the LDS crossbar, each with a wait of its own.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
-}
-template <bool IS_MAX>
-__device__ __forceinline__ float combine(float a, float b) { return IS_MAX ? fmaxf(a, b) : a + b; }
-template <bool IS_MAX>
-__device__ __forceinline__ float wave_reduce(float v) {
-  v = combine<IS_MAX>(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
-  v = combine<IS_MAX>(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
-  v = combine<IS_MAX>(v, dpp_move<0x141>(v));   // row_half_mirror
-  v = combine<IS_MAX>(v, dpp_move<0x140>(v));   // row_mirror
-  float a = v, b = v;
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
-  v = combine<IS_MAX>(a, b);
-  a = v, b = v;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
-  return combine<IS_MAX>(a, b);
-}
-__device__ __forceinline__ float wave_sum(float v) { return wave_reduce<false>(v); }
-__device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
+// Sum / maximum over the 64 lanes, in every lane, without leaving the vector ALU (lane_exchange.h).
+__device__ __forceinline__ float wave_sum(float v) { return lanes::across_wave<lanes::Sum>(v); }
+__device__ __forceinline__ float wave_max(float v) { return lanes::across_wave<lanes::Max>(v); }
 
 // Reduction across the WPR wavefronts that share a segment.  `slot` is the
 // segment's index inside the workgroup, `sub` the wavefront's index inside the
@@ -169,16 +147,7 @@ __device__ __forceinline__ void rms_norm_rows(const _Float16* __restrict__ x, in
 constexpr int kShortRowPasses = 4;
 template <int LPR>
 __device__ __forceinline__ float lane_group_sum(float v) {
-  auto add_dpp = [](float a, auto ctrl) {
-    constexpr int kCtrl = decltype(ctrl)::value;
-    return a + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), kCtrl, 0xf, 0xf, false));
-  };
-  v = add_dpp(v, std::integral_constant<int, 0xB1>{});                          // quad_perm [1,0,3,2]
-  v = add_dpp(v, std::integral_constant<int, 0x4E>{});                          // quad_perm [2,3,0,1]
-  if constexpr (LPR >= 8) v = add_dpp(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
-  if constexpr (LPR >= 16) v = add_dpp(v, std::integral_constant<int, 0x140>{}); // row_mirror
-  if constexpr (LPR >= 32) v += __shfl_xor(v, 16, 64);
-  return v;
+  return lanes::across_group<lanes::Sum, LPR>(v);
 }
 template <int LPR>
 __device__ __forceinline__ void rms_norm_rows_short(const _Float16* __restrict__ x, int64_t x_row_stride,
