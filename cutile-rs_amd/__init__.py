@@ -112,6 +112,11 @@ def lib() -> C.CDLL:
             "cutile_launch_full": [vp, f64, i64, P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_arange": [vp, P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_eye": [vp, P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_relu": [vp, P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_dropout": [vp, f32, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
+            "cutile_launch_scale_ptr": [vp, vp, vp, f32, i32, P(LaunchOpts)],
+            "cutile_launch_matvec": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, P(LaunchOpts)],
+            "cutile_launch_batch_matmul": [vp, P(PartitionArg), P(TensorArg), P(TensorArg), i32, P(LaunchOpts)],
             "cutile_launch_linspace": [vp, P(PartitionArg), f32, f32, P(LaunchOpts)],
             "cutile_launch_convert": [vp, P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_rms_norm_f16": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), f32, P(LaunchOpts)],
@@ -383,6 +388,41 @@ def eye(t: Partition, *, stream=None, grid=None, generics=None) -> None:
     """creation::eye over [BR, BC] tiles of an f32 matrix (cutile/src/kernels/_creation.rs:110-138)"""
     o, _k = _opts(grid, generics, None)
     check(lib().cutile_launch_eye(_stream(stream), C.byref(t.arg()), C.byref(o)))
+
+
+def relu(input_output: Partition, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-examples/examples/async_mlp.rs:56-61: max(0, x) in place over [D] tiles of an f32 vector"""
+    o, _k = _opts(grid, generics, None)
+    check(lib().cutile_launch_relu(_stream(stream), C.byref(input_output.arg()), C.byref(o)))
+
+
+def dropout(p: float, x, x_keep, out: Partition, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-examples/examples/dropout.rs:17-32: out = select(x_keep > p, x_keep, 0) / (1 - p); x is never read"""
+    o, _k = _opts(grid, generics, None)
+    xa, ka = tensor_arg(x), tensor_arg(x_keep)
+    check(lib().cutile_launch_dropout(_stream(stream), float(p), C.byref(xa), C.byref(ka), C.byref(out.arg()), C.byref(o)))
+
+
+def scale_ptr(out_ptr: int, in_ptr: int, scale: float, length: int, *, stream=None, grid=None) -> None:
+    """cutile-examples/examples/scale_ptr.rs:26-80: out[i] = in[i] * scale for i < length on raw device pointers (f32);
+    the launch grid is required, as for every launcher without a partition argument"""
+    o, _k = _opts(grid, None, None)
+    check(lib().cutile_launch_scale_ptr(_stream(stream), C.c_void_p(out_ptr), C.c_void_p(in_ptr), float(scale), int(length),
+                                        C.byref(o)))
+
+
+def matvec(z: Partition, x, y, k: int, *, stream=None, grid=None, generics=None) -> None:
+    """cutile-examples/examples/async_mlp.rs:38-54: z[r] += sum_k x[r, k] * y[k] over [BM] tiles of z (f32)"""
+    o, _k = _opts(grid, generics, None)
+    xa, ya = tensor_arg(x), tensor_arg(y)
+    check(lib().cutile_launch_matvec(_stream(stream), C.byref(z.arg()), C.byref(xa), C.byref(ya), int(k), C.byref(o)))
+
+
+def batch_matmul(c: Partition, a, b, k: int, *, stream=None, grid=None, generics=None, variant=None) -> None:
+    """cutile-examples/examples/batch_matmul.rs:16-44: c[p] = a[p] . b[p] over [1, BM, BN] tiles of c"""
+    o, _k = _opts(grid, generics, variant)
+    aa, ba = tensor_arg(a), tensor_arg(b)
+    check(lib().cutile_launch_batch_matmul(_stream(stream), C.byref(c.arg()), C.byref(aa), C.byref(ba), int(k), C.byref(o)))
 
 
 def linspace(t: Partition, start: float, step: float, *, stream=None, grid=None) -> None:

@@ -101,6 +101,11 @@ std::vector<KernelEntry> build_table() {
   add("rng_fill", "f64", "rng_fill_entry__f64", IMG_RNG, 256, 0, 0, 0, 0, 0, "f64", 0, 1);
   add("linspace", "f32", "linspace_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
   add("eye", "f32", "eye_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
+  // the example programs' small kernels (cutile-examples/examples/async_mlp.rs, dropout.rs, scale_ptr.rs)
+  add("relu", "f32", "relu_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  add("dropout", "f32", "dropout_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  add("scale_ptr", "f32", "scale_ptr_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 1);
+  add("matvec", "f32", "matvec_entry__f32", IMG_ELEMENTWISE, 256, 0, 0, 0, 0, 0, "f32", 0, 2);
   // the benchmark programs' all-f16 arithmetic (one wavefront per row; v = tile lanes per lane, c = 512-wide chunks)
   for (int v : {1, 2, 4, 8, 16})
     add("rms_norm_all_f16", keep("v" + std::to_string(v)), keep("rms_norm_all_f16_entry__v" + std::to_string(v)), IMG_ROWWISE, 256, 0, 0, 0, 0,
@@ -181,6 +186,21 @@ std::vector<KernelEntry> build_table() {
   for (const char* dt : {"bf16", "bf16f32", "f16", "f32"})
     add("gemm", keep(std::string(dt) + "_generic"), keep(std::string("gemm_entry__") + dt + "_generic"), IMG_GEMM, 256,
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
+
+  // batched GEMM (cutile-examples/examples/batch_matmul.rs): the pipelined bodies with the batch on a grid axis
+  for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2}}) {
+    std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
+    add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
+        (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "bf16", 0, 3);
+  }
+  for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2}}) {
+    std::string v = "f16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
+    add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
+        (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "f16", 0, 3);
+  }
+  for (const char* dt : {"bf16", "f16", "f32"})
+    add("batch_matmul", keep(std::string(dt) + "_generic"), keep(std::string("batch_matmul_entry__") + dt + "_generic"), IMG_GEMM, 256,
+        (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 3);
 
   // ---- NVFP4 GEMM: operands expanded to f16 on the way into LDS; LDS = 2 stages x (BM + BN) rows of 128 bytes ----
   for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2},

@@ -653,6 +653,94 @@ cutile_status_t cutile_launch_eye(cutile_stream_t stream, const cutile_partition
   uint32_t grid[3] = {std::min<uint32_t>(std::max<uint32_t>(1, div_up(rows * cols, 256 * 4)), 16384), 1, 1};
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
+// ---- the example programs' small kernels ---------------------------------------------------
+// grid of a flat f32 stream over `count` elements: 16 bytes per lane, four passes per lane at most
+static void flat_f32_grid(uint64_t count, uint32_t grid[3]) {
+  grid[0] = std::min<uint32_t>(std::max<uint32_t>(1, div_up(count, 256 * 4 * 4)), 16384);
+  grid[1] = grid[2] = 1;
+}
+cutile_status_t cutile_launch_relu(cutile_stream_t stream, const cutile_partition_arg_t* input_output,
+                                   const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(input_output, "input_output", 1, 1)) return s;
+  CUTILE_REQUIRE(input_output->tensor.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_LAUNCH, "relu: tensor must be f32");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(input_output->partition_shape[0]), "D")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(input_output, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("relu", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*input_output);
+  args.push_tile_grid(tg);
+  uint32_t grid[3];
+  flat_f32_grid(std::min<uint64_t>((uint64_t)tg[0] * input_output->partition_shape[0], input_output->tensor.shape[0]), grid);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+cutile_status_t cutile_launch_dropout(cutile_stream_t stream, float p, const cutile_tensor_arg_t* x,
+                                      const cutile_tensor_arg_t* x_keep, const cutile_partition_arg_t* out,
+                                      const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_tensor(x, "x", 1, 1)) return s;
+  if (cutile_status_t s = check_tensor(x_keep, "x_keep", 1, 1)) return s;
+  if (cutile_status_t s = check_partition(out, "out", 1, 1)) return s;
+  CUTILE_REQUIRE(x->dtype == CUTILE_DTYPE_F32 && x_keep->dtype == CUTILE_DTYPE_F32 && out->tensor.dtype == CUTILE_DTYPE_F32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "dropout: x, x_keep and out must be f32");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(out->partition_shape[0]), "S")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(out, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("dropout", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_val<float>(p);
+  args.push_tensor(*x);
+  args.push_tensor(*x_keep);
+  args.push_partition(*out);
+  args.push_tile_grid(tg);
+  uint32_t grid[3];
+  flat_f32_grid(std::min<uint64_t>((uint64_t)tg[0] * out->partition_shape[0], out->tensor.shape[0]), grid);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+cutile_status_t cutile_launch_scale_ptr(cutile_stream_t stream, void* out_ptr, const void* in_ptr, float scale, int32_t len,
+                                        const cutile_launch_opts_t* opts) {
+  CUTILE_REQUIRE(out_ptr && in_ptr, CUTILE_ERR_INVALID_ARGUMENT, "scale_ptr: null device pointer");
+  // no partition argument to infer a grid from: the caller names it, as for every launcher of pointer arguments
+  CUTILE_REQUIRE(opts && opts->grid[0] > 0 && opts->grid[1] > 0 && opts->grid[2] > 0, CUTILE_ERR_KERNEL_LAUNCH, "Launch grid required.");
+  CUTILE_REQUIRE(len >= 0, CUTILE_ERR_KERNEL_LAUNCH, "scale_ptr: len must be non-negative");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("scale_ptr", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_val<void*>(out_ptr);
+  args.push_val<const void*>(in_ptr);
+  args.push_val<float>(scale);
+  args.push_val<int32_t>(len);
+  uint32_t grid[3];
+  flat_f32_grid((uint64_t)len, grid);
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+cutile_status_t cutile_launch_matvec(cutile_stream_t stream, const cutile_partition_arg_t* z, const cutile_tensor_arg_t* x,
+                                     const cutile_tensor_arg_t* y, int32_t k, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(z, "z", 1, 1)) return s;
+  if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
+  if (cutile_status_t s = check_tensor(y, "y", 1, 1)) return s;
+  CUTILE_REQUIRE(z->tensor.dtype == CUTILE_DTYPE_F32 && x->dtype == CUTILE_DTYPE_F32 && y->dtype == CUTILE_DTYPE_F32,
+                 CUTILE_ERR_KERNEL_LAUNCH, "matvec: z, x and y must be f32");
+  if (cutile_status_t s = check_generic(opts, 0, std::to_string(z->partition_shape[0]), "BM")) return s;
+  const int bk = generic_int(opts, 1, 1);
+  CUTILE_REQUIRE(bk > 0, CUTILE_ERR_KERNEL_LAUNCH, "matvec: BK must be positive");
+  CUTILE_REQUIRE(k >= 0, CUTILE_ERR_KERNEL_LAUNCH, "matvec: k must be non-negative");
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(k), "K")) return s;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(z, opts, tg)) return s;
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("matvec", opts, "f32", {"f32"}, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*z);
+  args.push_tensor(*x);
+  args.push_tensor(*y);
+  args.push_val<int32_t>((k / bk) * bk);   // the tile program runs k / BK whole K tiles
+  args.push_tile_grid(tg);
+  const uint64_t rows = std::min<uint64_t>((uint64_t)tg[0] * z->partition_shape[0], z->tensor.shape[0]);
+  uint32_t grid[3] = {std::min<uint32_t>(std::max<uint32_t>(1, div_up(rows, 4)), 65536), 1, 1};   // one wavefront per row
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
 cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_partition_arg_t* t, float start, float step,
                                        const cutile_launch_opts_t* opts) {
   CUTILE_REQUIRE(t && t->tensor.dtype == CUTILE_DTYPE_F32, CUTILE_ERR_KERNEL_LAUNCH, "linspace: tensor must be f32");
@@ -1816,6 +1904,64 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
 }
 
 // ---- mapped partitions (cutile/src/tensor.rs:314-401) ---------------------------------------------------------
+cutile_status_t cutile_launch_batch_matmul(cutile_stream_t stream, const cutile_partition_arg_t* c, const cutile_tensor_arg_t* a,
+                                           const cutile_tensor_arg_t* b, int32_t k, const cutile_launch_opts_t* opts) {
+  if (cutile_status_t s = check_partition(c, "c", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(a, "a", 3, 3)) return s;
+  if (cutile_status_t s = check_tensor(b, "b", 3, 3)) return s;
+  const cutile_tensor_arg_t& ct = c->tensor;
+  CUTILE_REQUIRE(a->dtype == b->dtype && a->dtype == ct.dtype &&
+                     (ct.dtype == CUTILE_DTYPE_F32 || ct.dtype == CUTILE_DTYPE_F16 || ct.dtype == CUTILE_DTYPE_BF16),
+                 CUTILE_ERR_KERNEL_NOT_FOUND, "batch_matmul: c, a and b must share one element type of f32, f16, bf16 (got %s, %s, %s)",
+                 cutile_dtype_name(ct.dtype), cutile_dtype_name(a->dtype), cutile_dtype_name(b->dtype));
+  CUTILE_REQUIRE(c->partition_shape[0] == 1, CUTILE_ERR_KERNEL_LAUNCH, "batch_matmul: c must be partitioned [1, BM, BN]");
+  const int32_t bm = c->partition_shape[1], bn = c->partition_shape[2];
+  const std::string dt = cutile_dtype_name(ct.dtype);
+  if (cutile_status_t s = check_generic(opts, 0, dt, "E")) return s;
+  if (cutile_status_t s = check_generic(opts, 1, std::to_string(bm), "BM")) return s;
+  if (cutile_status_t s = check_generic(opts, 2, std::to_string(bn), "BN")) return s;
+  const int bk_user = generic_int(opts, 3, 64);
+  CUTILE_REQUIRE(bk_user > 0, CUTILE_ERR_KERNEL_LAUNCH, "batch_matmul: BK must be positive");
+  CUTILE_REQUIRE(k >= 0, CUTILE_ERR_KERNEL_LAUNCH, "batch_matmul: k must be non-negative");
+  if (cutile_status_t s = check_generic(opts, 4, std::to_string(k), "K")) return s;
+  const int32_t k_total = (k / bk_user) * bk_user;
+  uint32_t tg[3];
+  if (cutile_status_t s = resolve_grid(c, opts, tg)) return s;
+  const uint32_t batches = std::min<uint32_t>(tg[0], (uint32_t)ct.shape[0]);
+  // The matrix-core variants need what the plain GEMM's need of every rank-2 slice, 16-byte aligned batch strides, and
+  // operands that have every batch the launch covers.
+  const size_t es = cutile_dtype_size(ct.dtype);
+  auto slice_ok = [&](const cutile_tensor_arg_t& t) {
+    return t.strides[2] == 1 && t.strides[1] % 8 == 0 && t.strides[0] % 8 == 0 && aligned16(t.ptr) && t.shape[2] % 8 == 0 &&
+           extent_bytes_2d(t.shape[1], t.shape[2], t.strides[1], (int64_t)es) < kDescriptorLimit;
+  };
+  const bool fast_layout = ct.dtype != CUTILE_DTYPE_F32 && slice_ok(*a) && slice_ok(*b) && slice_ok(ct) && k_total % 8 == 0 &&
+                           (uint32_t)a->shape[0] >= batches && (uint32_t)b->shape[0] >= batches;
+  std::vector<std::string> acceptable;
+  if (fast_layout)
+    for (const auto& e : kernel_table())
+      if (strcmp(e.function, "batch_matmul") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn)
+        acceptable.push_back(e.variant);
+  acceptable.push_back(dt + "_generic");
+  Resolved res;
+  if (cutile_status_t s = resolve_entry("batch_matmul", opts, acceptable[0], acceptable, &res)) return s;
+  ArgPacker args;
+  args.push_partition(*c);
+  args.push_tensor(*a);
+  args.push_tensor(*b);
+  args.push_val<int32_t>(k_total);
+  args.push_tile_grid(tg);
+  uint32_t grid[3] = {tg[1] * tg[2], batches, 1};
+  if (res.entry->tile[0] == 0) {   // any-layout kernel: 64x64 outputs per workgroup over the covered region of each batch
+    const uint64_t cover_m = std::min<uint64_t>((uint64_t)tg[1] * bm, ct.shape[1]);
+    const uint64_t cover_n = std::min<uint64_t>((uint64_t)tg[2] * bn, ct.shape[2]);
+    grid[0] = std::max<uint32_t>(1, div_up(cover_m, 64));
+    grid[1] = std::max<uint32_t>(1, div_up(cover_n, 64));
+    grid[2] = batches;
+  }
+  return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
+}
+
 static cutile_status_t mapped_record(const cutile_mapped_partition_arg_t* p, MappedArg* m, uint32_t grid[3]) {
   CUTILE_REQUIRE(p && grid, CUTILE_ERR_INVALID_ARGUMENT, "null argument");
   CUTILE_REQUIRE(!p->partition.prefix_coverage, CUTILE_ERR_TENSOR,

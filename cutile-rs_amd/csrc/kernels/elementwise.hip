@@ -1,5 +1,6 @@
 // Elementwise and creation kernels for gfx950: saxpy, axpy with a separate
-// output, add, full, arange, linspace, eye, convert.
+// output, add, full, arange, linspace, eye, convert, and the example programs'
+// relu, dropout, scale_ptr and matvec.
 //
 // Bodies follow the reference's tile programs:
 //   saxpy    cutile-examples/examples/saxpy.rs:12-17, async_saxpy.rs:21-30
@@ -191,6 +192,32 @@ __device__ __forceinline__ void flat_convert(const S* src, int64_t src_stride, s
   for (size_t i = done + gid; i < count; i += step) {
     const S v = i < src_count ? src[(int64_t)i * src_stride] : S(0);
     dst[(int64_t)i * dst_stride] = convert_elem<D, S>(v);
+  }
+}
+
+// dst[i] = f(src[i]) for i < count, with src read as 0 where it has no element i (a tile loaded "like" the output
+// is zero-padded).  src may be dst (an update in place: every lane reads what it then writes).  Unit strides and
+// 16-byte aligned bases move 16 bytes per lane and access; anything else goes element by element, like the tail.
+template <typename T, typename F>
+__device__ __forceinline__ void flat_map1(const T* src, int64_t src_stride, size_t src_count, T* dst, int64_t dst_stride,
+                                          size_t count, F f) {
+  using V = Vec16<T>;
+  const size_t step = (size_t)gridDim.x * kThreads, gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (src_stride == 1 && dst_stride == 1 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    const size_t nvec = (count < src_count ? count : src_count) / V::N;
+    for (size_t j = gid; j < nvec; j += step) {
+      V in, out;
+      in.raw = reinterpret_cast<const u32x4*>(src)[j];
+#pragma unroll
+      for (int e = 0; e < V::N; ++e) out.v[e] = f(in.v[e]);
+      reinterpret_cast<u32x4*>(dst)[j] = out.raw;
+    }
+    done = nvec * V::N;
+  }
+  for (size_t i = done + gid; i < count; i += step) {
+    const T v = i < src_count ? src[(int64_t)i * src_stride] : T(0);
+    dst[(int64_t)i * dst_stride] = f(v);
   }
 }
 
@@ -471,6 +498,75 @@ extern "C" __global__ void __launch_bounds__(kThreads) eye_entry__f32(PartitionA
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
     const int64_t r = i / cols, c = i - r * cols;
     p[r * t.strides[0] + c * t.strides[1]] = r == c ? 1.0f : 0.0f;
+  }
+}
+
+// ---- the example programs' small kernels --------------------------------------------------------
+// relu<D>(input_output: [D] tiles of an f32 vector, updated in place): max(0, x) —
+// cutile-examples/examples/async_mlp.rs:56-61.  A NaN becomes 0 (the maximum returns its other operand).
+extern "C" __global__ void __launch_bounds__(kThreads) relu_entry__f32(PartitionArg<1> io, TileGrid g) {
+  const size_t count = covered_1d(io.shape[0], io.pshape[0], g);
+  flat_map1<float>((const float*)io.ptr, io.strides[0], count, (float*)io.ptr, io.strides[0], count,
+                   [](float v) { return __builtin_fmaxf(0.0f, v); });
+}
+
+// dropout<S>(p, _x, x_keep, out: [S] tiles): out = select(x_keep > p, x_keep, 0) / (1 - p), x_keep loaded like the
+// output tile (0 beyond its extent) — cutile-examples/examples/dropout.rs:17-32.  The first tensor is an argument the
+// tile program never reads; it is marshalled and ignored here too.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    dropout_entry__f32(float p, TensorArg<1> x, TensorArg<1> x_keep, PartitionArg<1> out, TileGrid g) {
+  (void)x;
+  const float keep_scale = 1.0f - p;
+  flat_map1<float>((const float*)x_keep.ptr, x_keep.strides[0], (size_t)x_keep.shape[0], (float*)out.ptr, out.strides[0],
+                   covered_1d(out.shape[0], out.pshape[0], g), [=](float v) { return (v > p ? v : 0.0f) / keep_scale; });
+}
+
+// scale_ptr(out_ptr, in_ptr, scale, len): out[i] = in[i] * scale for i < len, on raw pointers —
+// cutile-examples/examples/scale_ptr.rs:26-80.  The tile program strides its 128-element blocks over the launch
+// grid until len is covered, so every launch grid gives the same result; the walk here is over 16-byte vectors.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    scale_ptr_entry__f32(float* out, const float* in, float scale, int32_t len) {
+  const size_t count = len > 0 ? (size_t)len : 0;
+  flat_map1<float>(in, 1, count, out, 1, count, [=](float v) { return v * scale; });
+}
+
+// matvec<BM, BK, K>(z: [BM] tiles, x: [M, K], y: [K]), all f32: z[r] <- z[r] + sum_k x[r, k] * y[k] over the
+// K / BK whole K tiles (k_total) — cutile-examples/examples/async_mlp.rs:38-54.  Rows and K positions that x or y do
+// not have read 0.  One wavefront per row: the row is the stream (x is read once, y stays in cache), lanes take
+// 16-byte pieces 1 KiB apart, four accumulators per lane, then the wavefront's sum.
+extern "C" __global__ void __launch_bounds__(kThreads)
+    matvec_entry__f32(PartitionArg<1> z, TensorArg<2> x, TensorArg<1> y, int32_t k_total, TileGrid g) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  constexpr int kWaves = kThreads / 64;
+  const int64_t rows = (int64_t)covered_1d(z.shape[0], z.pshape[0], g);
+  const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
+  const float* yp = (const float*)y.ptr;
+  const bool vectors = x.strides[1] == 1 && y.strides[0] == 1 && (x.strides[0] & 3) == 0 &&
+                       (((uintptr_t)x.ptr | (uintptr_t)y.ptr) & 15) == 0;
+  for (int64_t r = (int64_t)blockIdx.x * kWaves + wave; r < rows; r += (int64_t)gridDim.x * kWaves) {
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (r < x.shape[0]) {
+      const float* xr = (const float*)x.ptr + r * x.strides[0];
+      int32_t done = 0;
+      if (vectors) {
+        const int32_t nvec = k_valid / 4;
+        for (int32_t j = lane; j < nvec; j += 64) {
+          Vec16<float> a, b;
+          a.raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr) + j);
+          b.raw = reinterpret_cast<const u32x4*>(yp)[j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(a.v[e], b.v[e], acc[e]);
+        }
+        done = nvec * 4;
+      }
+      for (int32_t k = done + lane; k < k_valid; k += 64)
+        acc[0] = __builtin_fmaf(xr[(int64_t)k * x.strides[1]], yp[(int64_t)k * y.strides[0]], acc[0]);
+    }
+    const float sum = lanes::across_wave<lanes::Sum>((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    if (lane == 0) {
+      float* dst = (float*)z.ptr + r * z.strides[0];
+      *dst = *dst + sum;
+    }
   }
 }
 

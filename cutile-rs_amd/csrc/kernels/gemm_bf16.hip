@@ -984,3 +984,52 @@ GEMM_PERSISTENT_KERNEL(bf16_128x128x64_d2x2, 128, 128, 2, 2, __bf16)
 GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(bf16, __bf16, __bf16)
 GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(f16, _Float16, _Float16)
 GEMM_PERSISTENT_ANY_LAYOUT_KERNEL(f32, float, float)
+
+// batch_matmul<E, BM, BN, BK, K>(c: [1, BM, BN] tiles of [batches, M, N], a: [batches, M, K], b: [batches, K, N]) —
+// cutile-examples/examples/batch_matmul.rs:16-44: c[p] = a[p] · b[p] from zero accumulators over K / BK whole K tiles,
+// every batch in one launch.  A workgroup takes its batch from one grid axis, cuts the three rank-2 slices out of the
+// operands and runs the tile body of the plain GEMM on them; a batch that a or b does not have reads as zeros.
+template <typename T>
+__device__ __forceinline__ void batch_slices(const PartitionArg<3>& c, const TensorArg<3>& a, const TensorArg<3>& b,
+                                             uint32_t batch, PartitionArg<2>* z, TensorArg<2>* x, TensorArg<2>* y) {
+  z->ptr = (T*)c.ptr + (int64_t)batch * c.strides[0];
+  x->ptr = (T*)a.ptr + (int64_t)batch * a.strides[0];
+  y->ptr = (T*)b.ptr + (int64_t)batch * b.strides[0];
+  for (int d = 0; d < 2; ++d) {
+    z->shape[d] = c.shape[d + 1], z->strides[d] = c.strides[d + 1];
+    z->pshape[d] = c.pshape[d + 1], z->pstrides[d] = c.pstrides[d + 1];
+    x->shape[d] = a.shape[d + 1], x->strides[d] = a.strides[d + 1];
+    y->shape[d] = b.shape[d + 1], y->strides[d] = b.strides[d + 1];
+  }
+  if (batch >= (uint32_t)a.shape[0] || batch >= (uint32_t)b.shape[0]) {   // zero padding of the missing batch
+    x->ptr = a.ptr, y->ptr = b.ptr;
+    x->shape[1] = 0, y->shape[0] = 0;
+  }
+}
+// tile grid (batches, M tiles, N tiles); HIP grid (M tiles * N tiles, batches, 1)
+#define BATCH_MATMUL_KERNEL(NAME, T, BM, BN, WVM, WVN)                                           \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      batch_matmul_entry__##NAME(PartitionArg<3> c, TensorArg<3> a, TensorArg<3> b, int32_t k, TileGrid g) { \
+    PartitionArg<2> z;                                                                         \
+    TensorArg<2> x, y;                                                                         \
+    batch_slices<T>(c, a, b, blockIdx.y, &z, &x, &y);                                          \
+    const TileGrid tiles = {g.y, g.z, 1, 0};                                                   \
+    GemmDirect<BM, BN, WVM, WVN, T, T>::run(z, x, y, k, tiles, 0);                             \
+  }
+BATCH_MATMUL_KERNEL(bf16_256x256x64_d2x4, __bf16, 256, 256, 2, 4)
+BATCH_MATMUL_KERNEL(bf16_128x128x64_d2x2, __bf16, 128, 128, 2, 2)
+BATCH_MATMUL_KERNEL(f16_256x256x64_d4x2, _Float16, 256, 256, 4, 2)
+BATCH_MATMUL_KERNEL(f16_128x128x64_d2x2, _Float16, 128, 128, 2, 2)
+// any tile shape, strides and extents: HIP grid (64-row blocks, 64-column blocks, batches)
+#define BATCH_MATMUL_ANY_LAYOUT_KERNEL(NAME, T)                                                  \
+  extern "C" __global__ void __launch_bounds__(256)                                            \
+      batch_matmul_entry__##NAME##_generic(PartitionArg<3> c, TensorArg<3> a, TensorArg<3> b, int32_t k, TileGrid g) { \
+    PartitionArg<2> z;                                                                         \
+    TensorArg<2> x, y;                                                                         \
+    batch_slices<T>(c, a, b, blockIdx.z, &z, &x, &y);                                          \
+    const TileGrid tiles = {g.y, g.z, 1, 0};                                                   \
+    gemm_any_layout<T, T>(z, x, y, k, tiles, 0);                                               \
+  }
+BATCH_MATMUL_ANY_LAYOUT_KERNEL(bf16, __bf16)
+BATCH_MATMUL_ANY_LAYOUT_KERNEL(f16, _Float16)
+BATCH_MATMUL_ANY_LAYOUT_KERNEL(f32, float)

@@ -595,6 +595,48 @@ struct SoftmaxFn {
     return cutile_launch_softmax(s, &xa, &yp, o);
   }
 };
+// the example programs' small kernels
+struct ReluFn {
+  static constexpr const char* name = "relu";
+  template <class IO>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, IO& io) {
+    auto p = io.arg();
+    return cutile_launch_relu(s, &p, o);
+  }
+};
+struct DropoutFn {
+  static constexpr const char* name = "dropout";
+  template <class X, class XK, class O>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, float p, X& x, XK& x_keep, O& out) {
+    auto op = out.arg();
+    auto xa = input_arg(x), ka = input_arg(x_keep);
+    return cutile_launch_dropout(s, p, &xa, &ka, &op, o);
+  }
+};
+struct ScalePtrFn {
+  static constexpr const char* name = "scale_ptr";
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, void* out_ptr, void* in_ptr, float scale, int32_t len) {
+    return cutile_launch_scale_ptr(s, out_ptr, in_ptr, scale, len, o);
+  }
+};
+struct MatvecFn {
+  static constexpr const char* name = "matvec";
+  template <class Z, class X, class Yv>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Z& z, X& x, Yv& y, int32_t k) {
+    auto zp = z.arg();
+    auto xa = input_arg(x), ya = input_arg(y);
+    return cutile_launch_matvec(s, &zp, &xa, &ya, k, o);
+  }
+};
+struct BatchMatmulFn {
+  static constexpr const char* name = "batch_matmul";
+  template <class Cp, class A, class B>
+  static cutile_status_t launch(cutile_stream_t s, const cutile_launch_opts_t* o, Cp& c, A& a, B& b, int32_t k) {
+    auto cp = c.arg();
+    auto aa = input_arg(a), ba = input_arg(b);
+    return cutile_launch_batch_matmul(s, &cp, &aa, &ba, k, o);
+  }
+};
 template <bool Accumulate>
 struct GemmFn {
   static constexpr const char* name = "gemm";
@@ -832,6 +874,16 @@ template <class X, class Y> auto softmax(X&& x, Y&& y) { return make_launcher<ke
 // the benchmark programs' all-f16 forms: rms_norm(x, w, out: [1,N], eps) with .generics({N, BLOCK_SIZE}); softmax(x, y: [BM,BN])
 template <class X, class W, class O> auto rms_norm_all_f16(X&& x, W&& w, O&& out, float eps) { return make_launcher<kernels::RmsNormAllF16Fn>(std::forward<X>(x), std::forward<W>(w), std::forward<O>(out), eps); }
 template <class X, class Y> auto softmax_all_f16(X&& x, Y&& y) { return make_launcher<kernels::SoftmaxAllF16Fn>(std::forward<X>(x), std::forward<Y>(y)); }
+// relu(input_output: partition [D]) -> (input_output)                  cutile-examples/examples/async_mlp.rs:56-61
+template <class IO> auto relu(IO&& io) { return make_launcher<kernels::ReluFn>(std::forward<IO>(io)); }
+// dropout(p, _x, x_keep, out: partition [S]) -> (p, _x, x_keep, out)     cutile-examples/examples/dropout.rs:17-32
+template <class X, class XK, class O> auto dropout(float p, X&& x, XK&& x_keep, O&& out) { return make_launcher<kernels::DropoutFn>(p, std::forward<X>(x), std::forward<XK>(x_keep), std::forward<O>(out)); }
+// scale_ptr(out_ptr, in_ptr, scale, len) on raw device pointers; .grid(..) is required   cutile-examples/examples/scale_ptr.rs:26-80
+inline auto scale_ptr(void* out_ptr, void* in_ptr, float scale, int32_t len) { return make_launcher<kernels::ScalePtrFn>(out_ptr, in_ptr, scale, len); }
+// matvec(z: partition [BM], x, y, k) -> (z, x, y, k): z <- z + x·y       cutile-examples/examples/async_mlp.rs:38-54
+template <class Z, class X, class Y> auto matvec(Z&& z, X&& x, Y&& y, int32_t k) { return make_launcher<kernels::MatvecFn>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), k); }
+// batch_matmul(c: partition [1,BM,BN], a, b, k) -> (c, a, b, k)          cutile-examples/examples/batch_matmul.rs:16-44
+template <class Cp, class A, class B> auto batch_matmul(Cp&& c, A&& a, B&& b, int32_t k) { return make_launcher<kernels::BatchMatmulFn>(std::forward<Cp>(c), std::forward<A>(a), std::forward<B>(b), k); }
 // gemm(z: partition [BM,BN], x, y, k) -> (z, x, y, k): z <- z + x·y   cutile-benchmarks/benches/gemm.rs:25-30
 template <class Z, class X, class Y> auto gemm(Z&& z, X&& x, Y&& y, int32_t k) { return make_launcher<kernels::GemmFn<true>>(std::forward<Z>(z), std::forward<X>(x), std::forward<Y>(y), k); }
 // gemm_zero_init: accumulator starts at 0                              cutile-examples/examples/gemm.rs:20-36

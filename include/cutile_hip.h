@@ -433,6 +433,24 @@ cutile_status_t cutile_launch_linspace(cutile_stream_t stream, const cutile_part
  * cutile/src/kernels/_creation.rs:110-138 (behind api::eye / eye_rect, cutile/src/api.rs:613-639). */
 cutile_status_t cutile_launch_eye(cutile_stream_t stream, const cutile_partition_arg_t* t,
                                   const cutile_launch_opts_t* opts);
+/* The small kernels of the reference's example programs (all f32).
+ *   relu<D>(input_output: [D] tiles, updated in place): max(0, x)           cutile-examples/examples/async_mlp.rs:56-61
+ *   dropout<S>(p, _x, x_keep, out: [S] tiles): select(x_keep > p, x_keep, 0) / (1 - p), x_keep read as 0 beyond its
+ *     extent; _x is an argument the tile program never reads                 cutile-examples/examples/dropout.rs:17-32
+ *   scale_ptr(out_ptr, in_ptr, scale, len): out[i] = in[i] * scale, i < len, raw device pointers.  Like every launcher
+ *     without a partition argument it needs opts->grid ("Launch grid required."); the tile program strides its blocks
+ *     over whatever grid it gets, so the result does not depend on it        cutile-examples/examples/scale_ptr.rs:26-80
+ *   matvec<BM, BK, K>(z: [BM] tiles, x: [M, K], y: [K]): z[r] <- z[r] + sum_k x[r, k] * y[k] over k / BK whole K tiles,
+ *     rows and K positions that x or y lack reading 0                        cutile-examples/examples/async_mlp.rs:38-54 */
+cutile_status_t cutile_launch_relu(cutile_stream_t stream, const cutile_partition_arg_t* input_output,
+                                   const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_dropout(cutile_stream_t stream, float p, const cutile_tensor_arg_t* x,
+                                      const cutile_tensor_arg_t* x_keep, const cutile_partition_arg_t* out,
+                                      const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_scale_ptr(cutile_stream_t stream, void* out_ptr, const void* in_ptr, float scale, int32_t len,
+                                        const cutile_launch_opts_t* opts);
+cutile_status_t cutile_launch_matvec(cutile_stream_t stream, const cutile_partition_arg_t* z, const cutile_tensor_arg_t* x,
+                                     const cutile_tensor_arg_t* y, int32_t k, const cutile_launch_opts_t* opts);
 /* conversion::convert — cutile/src/kernels/_conversion.rs:78-85 */
 cutile_status_t cutile_launch_convert(cutile_stream_t stream, const cutile_tensor_arg_t* src,
                                       const cutile_partition_arg_t* dst, const cutile_launch_opts_t* opts);
@@ -566,6 +584,13 @@ cutile_status_t cutile_scratch_capacity(size_t* bytes);
 cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partition_arg_t* z,
                                    const cutile_tensor_arg_t* x, const cutile_tensor_arg_t* y,
                                    int32_t k, int32_t accumulate, const cutile_launch_opts_t* opts);
+/* batch_matmul<E, BM, BN, BK, K>(c: [1, BM, BN] tiles of [batches, M, N], a: [batches, M, K], b: [batches, K, N]):
+ * c[p] = a[p] · b[p] from zero accumulators over k / BK whole K tiles, all batches in one launch, tile grid
+ * (batches, M tiles, N tiles) — cutile-examples/examples/batch_matmul.rs:16-44.  E = f32 (the example), f16 or bf16
+ * (f32 accumulation, one rounding at the store). */
+cutile_status_t cutile_launch_batch_matmul(cutile_stream_t stream, const cutile_partition_arg_t* c,
+                                           const cutile_tensor_arg_t* a, const cutile_tensor_arg_t* b, int32_t k,
+                                           const cutile_launch_opts_t* opts);
 /* copy_stacked_to_contiguous_f16 / copy_contiguous_to_stacked_f16(num_blocks, stacked_tensors, contiguous_tensors, nh, nl,
  * no, nt, hd) — cutile-kernels/src/experimental/kvbm.rs:112-187, 283-352.  KV cache blocks of nh heads x nl layers x
  * no offsets x nt tokens x hd values move between the stacked form (one f16 tensor per (block, layer, offset), table

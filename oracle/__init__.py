@@ -411,6 +411,47 @@ def mapped_schedule(grid, map_shape):
     return order
 
 
+# ---- the example programs' small kernels (numpy, f32) ---------------------------------------
+def relu_f32(x) -> np.ndarray:
+    """cutile-examples/examples/async_mlp.rs:56-61: max_tile(0, x)"""
+    x = _c(x, np.float32)
+    return np.where(x > 0, x, np.float32(0)).astype(np.float32)
+
+
+def dropout_f32(p: float, x_keep, n_out: int = None) -> np.ndarray:
+    """cutile-examples/examples/dropout.rs:23-31: select(x_keep > p, x_keep, 0) / (1 - p), every step in f32;
+    x_keep is loaded like the output tile, so positions it does not have read 0"""
+    k = _c(x_keep, np.float32).reshape(-1)
+    n = k.size if n_out is None else n_out
+    padded = np.zeros(n, np.float32)
+    padded[:min(n, k.size)] = k[:n]
+    p32 = np.float32(p)
+    kept = np.where(padded > p32, padded, np.float32(0)).astype(np.float32)
+    return (kept / (np.float32(1) - p32)).astype(np.float32)
+
+
+def scale_f32(x, scale: float) -> np.ndarray:
+    """cutile-examples/examples/scale_ptr.rs:66 (tile * scale_tile), the check at :102-110"""
+    return (_c(x, np.float32) * np.float32(scale)).astype(np.float32)
+
+
+def matvec_f32(z, x, y, k: int = None, bk: int = 1) -> np.ndarray:
+    """cutile-examples/examples/async_mlp.rs:38-54: z + x . y over k / BK whole K tiles, as cpu_gemm_f32 with one
+    column (the order in which a tile's products are added is the assembler's)"""
+    x, y, z = _c(x, np.float32), _c(y, np.float32), _c(z, np.float32)
+    k = x.shape[1] if k is None else k
+    kt = min((k // bk) * bk, x.shape[1], y.shape[0])
+    return (z + cpu_gemm_f32(x[:, :kt], y[:kt].reshape(kt, 1)).reshape(-1)).astype(np.float32)
+
+
+def batch_matmul_f32(a, b, k: int = None, bk: int = 1) -> np.ndarray:
+    """cutile-examples/examples/batch_matmul.rs:31-43: cpu_gemm_f32 of every batch, from zero accumulators"""
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    k = a.shape[2] if k is None else k
+    kt = min((k // bk) * bk, a.shape[2], b.shape[1])
+    return np.stack([cpu_gemm_f32(a[i, :, :kt], b[i, :kt, :]) for i in range(a.shape[0])])
+
+
 # ---- K3 -----------------------------------------------------------------------------------
 def softmax_f32(x, bm: int, bn: int) -> np.ndarray:
     x = _c(x, np.float32)

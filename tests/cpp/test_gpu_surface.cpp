@@ -350,6 +350,61 @@ TEST(eye_and_eye_rect) {
   }
 }
 
+TEST(example_programs_batch_matmul_scale_ptr_dropout_mlp) {
+  auto stream = new_stream();
+  {  // cutile-examples/examples/batch_matmul.rs:49-76: ones [4,128,64] x ones [4,64,256], tiles (64, 64, 32) -> every output K
+    const int batch = 4, m = 128, n = 256, k = 64;
+    auto a = std::make_shared<Tensor<float>>(api::ones<float>({batch, m, k}).sync_on(stream).unwrap());
+    auto b = std::make_shared<Tensor<float>>(api::ones<float>({batch, k, n}).sync_on(stream).unwrap());
+    auto c = api::zeros<float>({batch, m, n}).sync_on(stream).unwrap().partition({1, 64, 64});
+    auto res = batch_matmul(std::move(c), a, b, k).generics({"f32", "64", "64", "32", "64"}).sync_on(stream).unwrap();
+    auto host = api::to_host_vec(std::move(std::get<0>(res)).unpartition()).sync_on(stream).unwrap();
+    CHECK(host.size() == (size_t)batch * m * n);
+    for (float v : host) CHECK(v == (float)k);
+  }
+  {  // cutile-examples/examples/scale_ptr.rs:86-110: arange(1024) * 3 through raw pointers, 4 tile blocks
+    const int len = 1024;
+    auto input = api::arange<float>(len).sync_on(stream).unwrap();
+    auto output = api::zeros<float>({len}).sync_on(stream).unwrap();
+    CHECK(scale_ptr(output.device_pointer(), input.device_pointer(), 3.0f, len).grid(4, 1, 1).sync_on(stream).is_ok());
+    auto in_host = api::to_host_vec(input).sync_on(stream).unwrap();
+    auto out_host = api::to_host_vec(output).sync_on(stream).unwrap();
+    for (int i = 0; i < len; ++i) CHECK(out_host[i] == in_host[i] * 3.0f);
+    // no partition to infer a grid from
+    auto err = scale_ptr(output.device_pointer(), input.device_pointer(), 3.0f, len).sync_on(stream);
+    CHECK(err.is_err() && err.error().message.find("Launch grid required.") != std::string::npos);
+  }
+  {  // cutile-examples/examples/dropout.rs:39-50: m = 16, tiles of 4, p = 0.4, seeded inputs; (p, x, x_keep, out) come back
+    const float p = 0.4f;
+    auto x = std::make_shared<Tensor<float>>(api::randn(0.0f, 1.0f, {16}, 123).sync_on(stream).unwrap());
+    auto x_keep = std::make_shared<Tensor<float>>(api::rand<float>({16}, 123).sync_on(stream).unwrap());
+    auto out = api::zeros<float>({16}).sync_on(stream).unwrap().partition({4});
+    auto res = dropout(p, x, x_keep, std::move(out)).sync_on(stream).unwrap();
+    auto host = api::to_host_vec(std::move(std::get<3>(res)).unpartition()).sync_on(stream).unwrap();
+    auto keep = api::to_host_vec(x_keep).sync_on(stream).unwrap();
+    for (int i = 0; i < 16; ++i) CHECK(host[i] == (keep[i] > p ? keep[i] : 0.0f) / (1.0f - p));
+  }
+  {  // cutile-examples/examples/async_mlp.rs:124-137: gemm(data, w0) -> matvec(., w1) -> relu, dim 16, tiles of 4, lazily chained
+    const int dim = 16, bd = 4;
+    auto data = std::make_shared<Tensor<float>>(api::randn(0.0f, 1.0f, {dim, dim}, 1).sync_on(stream).unwrap());
+    auto w0 = std::make_shared<Tensor<float>>(api::randn(0.0f, 1.0f, {dim, dim}, 2).sync_on(stream).unwrap());
+    auto w1 = std::make_shared<Tensor<float>>(api::randn(0.0f, 1.0f, {dim}, 3).sync_on(stream).unwrap());
+    auto out0 = gemm(partition_op(api::zeros<float>({dim, dim}), {bd, bd}), data, w0, dim).generics({"f32", "4", "4", "4"}).first();
+    auto out1 = matvec(partition_op(api::zeros<float>({dim}), {bd}), unpartition_op(std::move(out0)), w1, dim).generics({"4", "4", "16"}).first();
+    auto out = api::to_host_vec_op(unpartition_op(relu(std::move(out1)).first())).sync_on(stream).unwrap();
+    auto d = api::to_host_vec(data).sync_on(stream).unwrap(), a = api::to_host_vec(w0).sync_on(stream).unwrap(), v = api::to_host_vec(w1).sync_on(stream).unwrap();
+    for (int r = 0; r < dim; ++r) {
+      double acc = 0;
+      for (int c = 0; c < dim; ++c) {
+        double h = 0;
+        for (int kk = 0; kk < dim; ++kk) h += (double)d[r * dim + kk] * a[kk * dim + c];
+        acc += h * v[c];
+      }
+      CHECK(std::fabs(out[r] - std::max(acc, 0.0)) < 1e-3);
+    }
+  }
+}
+
 TEST(random_constructors_draw_on_the_device) {
   // api::randn / rand / randn_f16 (cutile/src/api.rs:683-735): distribution, seed determinism, shapes
   auto stream = new_stream();

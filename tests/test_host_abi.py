@@ -247,6 +247,54 @@ def test_eye_launcher_on_the_recording_runtime(fake_hip):
     assert ct.lib().cutile_testing_launch_count() == n
 
 
+def test_example_program_launchers_on_the_recording_runtime(fake_hip):
+    ct = fake_hip
+    # relu: (partition, tile grid); flat over the covered elements, 4096 per workgroup
+    t = torch.zeros(10000)
+    ct.relu(ct.partition(t, [100]), generics=[100])
+    rec, args = _last(ct)
+    assert rec.symbol == b"relu_entry__f32" and tuple(rec.grid) == (3, 1, 1) and tuple(rec.block) == (256, 1, 1)
+    ptr, n, st, p, _ps, gx, gy, gz, _ = struct.unpack("<Q4i4I", args)
+    assert ptr == t.data_ptr() and (n, st, p) == (10000, 1, 100) and (gx, gy, gz) == (100, 1, 1)
+    # dropout: p first, then the two tensors, the partition, the tile grid (signature order)
+    x, keep, out = torch.zeros(16), torch.zeros(16), torch.zeros(16)
+    ct.dropout(0.4, x, keep, ct.partition(out, [4]), generics=[4])
+    rec, args = _last(ct)
+    assert rec.symbol == b"dropout_entry__f32" and tuple(rec.grid) == (1, 1, 1)
+    pv, xp, xn, xs, kp, kn, ks, op = struct.unpack_from("<f4xQ2iQ2iQ", args, 0)
+    assert abs(pv - 0.4) < 1e-7 and (xp, xn, xs) == (x.data_ptr(), 16, 1) and (kp, kn, ks) == (keep.data_ptr(), 16, 1) and op == out.data_ptr()
+    # scale_ptr: raw pointers, scale, len; the caller's grid is required but does not shape the dispatch
+    ct.scale_ptr(out.data_ptr(), x.data_ptr(), 3.0, 16, grid=(4, 1, 1))
+    rec, args = _last(ct)
+    assert rec.symbol == b"scale_ptr_entry__f32" and tuple(rec.grid) == (1, 1, 1)
+    assert struct.unpack("<QQfi", args) == (out.data_ptr(), x.data_ptr(), 3.0, 16)
+    # matvec: one wavefront per row, four rows per workgroup; k is cut to whole K tiles
+    z, xm, y = torch.zeros(1000), torch.zeros(1000, 70), torch.zeros(70)
+    ct.matvec(ct.partition(z, [8]), xm, y, 70, generics=[8, 16, 70])
+    rec, args = _last(ct)
+    assert rec.symbol == b"matvec_entry__f32" and tuple(rec.grid) == (250, 1, 1)
+    assert struct.unpack_from("<i4I", args, 24 + 24 + 16) == (64, 125, 1, 1, 0)
+    # batch_matmul: tile grid (batches, M tiles, N tiles); pipelined variant on (M tiles * N tiles, batches), any-layout on 64 x 64 blocks
+    a, b, c = torch.zeros(3, 256, 64, dtype=torch.bfloat16), torch.zeros(3, 64, 384, dtype=torch.bfloat16), torch.zeros(3, 256, 384, dtype=torch.bfloat16)
+    ct.batch_matmul(ct.partition(c, [1, 128, 128]), a, b, 64, generics=["bf16", 128, 128, 64, 64])
+    rec, args = _last(ct)
+    assert rec.symbol == b"batch_matmul_entry__bf16_128x128x64_d2x2" and tuple(rec.grid) == (6, 3, 1) and tuple(rec.block) == (256, 1, 1)
+    assert struct.unpack_from("<i4I", args, 56 + 32 + 32) == (64, 3, 2, 3, 0)
+    ct.batch_matmul(ct.partition(torch.zeros(4, 128, 256), [1, 64, 64]), torch.zeros(4, 128, 64), torch.zeros(4, 64, 256), 64, generics=["f32", 64, 64, 32, 64])
+    rec, _ = _last(ct)
+    assert rec.symbol == b"batch_matmul_entry__f32_generic" and tuple(rec.grid) == (2, 4, 4)
+    n = ct.lib().cutile_testing_launch_count()
+    with pytest.raises(ct.CutileError, match="Launch grid required."):
+        ct.scale_ptr(out.data_ptr(), x.data_ptr(), 3.0, 16)
+    with pytest.raises(ct.CutileError, match="generic D"):
+        ct.relu(ct.partition(t, [100]), generics=[64])
+    with pytest.raises(ct.CutileError, match="must be f32"):
+        ct.matvec(ct.partition(z.half(), [8]), xm, y, 70)
+    with pytest.raises(ct.CutileError, match=r"partitioned \[1, BM, BN\]"):
+        ct.batch_matmul(ct.partition(c, [3, 128, 128]), a, b, 64)
+    assert ct.lib().cutile_testing_launch_count() == n
+
+
 def test_kernel_table_lookup_and_single_flight_module_load(fake_hip):
     ct = fake_hip
     L = ct.lib()

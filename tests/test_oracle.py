@@ -399,3 +399,42 @@ def test_all_f16_forms_stay_near_the_float64_functions():
     seg = np.concatenate([xf[:, 64:100], np.zeros((16, 28))], axis=1)
     e = np.exp(seg - seg.max(1, keepdims=True))
     assert np.abs(y[:, 64:] - (e / e.sum(1, keepdims=True))[:, :36]).max() <= 2e-3
+
+
+# ---- the example programs' small kernels: pinned by hand-worked cases, the reference programs' own checks and f64 sums ----
+def test_relu_and_dropout_hand_worked_cases():
+    assert oracle.relu_f32([-1.5, -0.0, 0.0, 2.25]).tolist() == [0.0, 0.0, 0.0, 2.25]
+    # p = 0.5: values at or below p go, the rest double (exact in binary)
+    assert oracle.dropout_f32(0.5, [0.25, 0.5, 0.75, 1.0]).tolist() == [0.0, 0.0, 1.5, 2.0]
+    # a shorter keep tensor reads 0 beyond its end; a longer one is cut
+    assert oracle.dropout_f32(0.5, [0.75], 3).tolist() == [1.5, 0.0, 0.0]
+    assert oracle.dropout_f32(0.5, [0.75, 1.0, 0.625], 2).tolist() == [1.5, 2.0]
+    # p = 0.4 as in cutile-examples/examples/dropout.rs:45: the quotient is the f32 division by the f32 value of 1 - p
+    got = oracle.dropout_f32(0.4, [0.9])[0]
+    assert got == np.float32(0.9) / (np.float32(1) - np.float32(0.4)) and abs(float(got) - 1.5) < 1e-6
+    # the keep fraction of uniform samples is 1 - p
+    keep = oracle.uniform_f32(100000, 5, 0.0, 1.0)
+    assert abs(np.count_nonzero(oracle.dropout_f32(0.4, keep)) / keep.size - 0.6) < 0.01
+
+
+def test_scale_is_the_reference_programs_own_check():
+    # cutile-examples/examples/scale_ptr.rs:102-110: output[i] == input[i] * scale for arange(1024), scale 3
+    x = np.arange(1024, dtype=np.float32)
+    assert np.array_equal(oracle.scale_f32(x, 3.0), np.arange(1024) * 3)
+
+
+def test_matvec_and_batch_matmul_against_f64_sums_and_closed_forms():
+    x, y, z = oracle.normal_f32((37, 300), 1), oracle.normal_f32(300, 2), oracle.normal_f32(37, 3)
+    want = z.astype(np.float64) + x.astype(np.float64) @ y.astype(np.float64)
+    assert np.allclose(oracle.matvec_f32(z, x, y), want, rtol=0, atol=1e-4)
+    # k / BK whole K tiles: the last 300 - 256 products are left out; a transposed operand or a dropped z would show
+    cut = z.astype(np.float64) + x[:, :256].astype(np.float64) @ y[:256].astype(np.float64)
+    assert np.allclose(oracle.matvec_f32(z, x, y, 300, 128), cut, rtol=0, atol=1e-4)
+    assert not np.allclose(cut, want, atol=1e-2)
+    # cutile-examples/examples/batch_matmul.rs:49-76: ones x ones = K everywhere
+    assert np.array_equal(oracle.batch_matmul_f32(np.ones((4, 128, 64), np.float32), np.ones((4, 64, 256), np.float32)), np.full((4, 128, 256), 64, np.float32))
+    a, b = oracle.normal_f32((3, 20, 40), 4), oracle.normal_f32((3, 40, 30), 5)
+    assert np.allclose(oracle.batch_matmul_f32(a, b), np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64)), rtol=0, atol=1e-4)
+    # batches stay apart: permuting the batches of both operands permutes the result
+    perm = [2, 0, 1]
+    assert np.array_equal(oracle.batch_matmul_f32(a[perm], b[perm]), oracle.batch_matmul_f32(a, b)[perm])
