@@ -867,9 +867,112 @@ class EmbeddingBatch(Workload):
         return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "full size"}, {"bit_exact": exact}
 
 
+class BatchMatmul(Workload):
+    """batch_matmul (cutile-examples/examples/batch_matmul.rs:16-44) at a size that fills the chip: 16 batches of 2048^3."""
+    name, unit, dtype, bound, peak_key = "batch_matmul_bf16_16x2048x2048x2048", "TFLOP/s", "bf16 in / f32 acc / bf16 out", "mfma", "mfma_bf16"
+    batch, s = 16, 2048
+    work = 2.0 * batch * s ** 3
+    config = {"workload": "batch_matmul bf16: 16 batches of M=N=K=2048, c[p] = a[p]·b[p], entries ~ N(0,1)/sqrt(K), tiles [1, 256, 256]",
+              "tile": "256x256x64"}
+
+    def setup(self, ct, torch, oracle, dev):
+        import numpy as np
+
+        self.ct = ct
+        b, s = self.batch, self.s
+        self.ab = oracle.f32_to_bf16_bits(oracle.normal_f32((b, s, s), 61, 0, s ** -0.5))
+        self.bb = oracle.f32_to_bf16_bits(oracle.normal_f32((b, s, s), 62, 0, s ** -0.5))
+        self.a, self.b = _td_bf16(torch, np, self.ab, dev), _td_bf16(torch, np, self.bb, dev)
+        self.c = torch.zeros(b, s, s, dtype=torch.bfloat16, device=dev)
+        self.cp = ct.partition(self.c, [1, 256, 256])
+
+    def launch(self):
+        self.ct.batch_matmul(self.cp, self.a, self.b, self.s)
+
+    def cpu_baseline(self, oracle, np, torch):
+        rows = np.arange(0, self.s, 16, dtype=np.int64)          # 128 rows of every batch
+        t0 = time.perf_counter()
+        ref = np.stack([oracle.gemm_bf16(self.ab[i], self.bb[i], rows=rows, f32out=True) for i in range(self.batch)])
+        dt = time.perf_counter() - t0
+        got = self.c[:, ::16].float().cpu().numpy()
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        flops = 2.0 * self.batch * len(rows) * self.s * self.s
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": f"{len(rows)} of {self.s} output rows of every batch (naive f32 loop)"}, \
+               {"rel_l2_sampled_rows": rel, "tolerance": 1e-2, "ok": rel <= 1e-2}
+
+
+class Matvec(Workload):
+    """matvec (cutile-examples/examples/async_mlp.rs:38-54): the matrix is the stream."""
+    name, unit, dtype = "matvec_f32_16384x16384", "GB/s", "f32"
+    m = k = 16384
+    work = 4.0 * m * k + 4.0 * k + 8.0 * m
+    config = {"workload": "matvec fp32: z[16384] += x[16384, 16384] · y[16384], tiles of 64 rows"}
+
+    def setup(self, ct, torch, oracle, dev):
+        self.ct = ct
+        self.xh, self.yh = oracle.normal_f32((self.m, self.k), 63), oracle.normal_f32(self.k, 64, 0, self.k ** -0.5)
+        self.x, self.y = torch.from_numpy(self.xh).to(dev), torch.from_numpy(self.yh).to(dev)
+        self.z = torch.zeros(self.m, device=dev)
+        self.zp = ct.partition(self.z, [64])
+
+    def launch(self):
+        self.ct.matvec(self.zp, self.x, self.y, self.k)
+
+    def cpu_baseline(self, oracle, np, torch):
+        self.z.zero_()          # the timed launches accumulated into z: one launch from zero for the comparison
+        self.launch()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ref = oracle.matvec_f32(np.zeros(self.m, np.float32), self.xh, self.yh)
+        dt = time.perf_counter() - t0
+        mag = np.abs(self.xh).astype(np.float64) @ np.abs(self.yh).astype(np.float64)
+        err = np.abs(self.z.cpu().numpy().astype(np.float64) - ref)
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port", "sample": "full size"}, \
+               {"max_err_over_sum_of_magnitudes": float((err / mag).max()), "tolerance": 1e-5, "ok": bool((err <= 1e-5 * mag).all())}
+
+
+class ExampleStream(Workload):
+    """relu / dropout / scale_ptr of the example programs on 2^26 f32: one read and one write per element."""
+    unit, dtype = "GB/s", "f32"
+    n = 1 << 26
+    work = 8.0 * n
+
+    def __init__(self, kind):
+        self.kind = kind
+        self.name = f"{kind}_f32_{self.n}"
+        what = {"relu": "relu in place (async_mlp.rs:56-61), tiles of 1024", "dropout": "dropout p = 0.4 (dropout.rs:17-32), tiles of 1024",
+                "scale_ptr": "scale_ptr on raw pointers, scale 3 (scale_ptr.rs:26-80), grid (1024, 1, 1)"}[kind]
+        self.config = {"workload": f"{what}, n = 2^26 f32"}
+
+    def setup(self, ct, torch, oracle, dev):
+        self.ct = ct
+        self.xh = oracle.uniform_f32(self.n, 65, 0.0, 1.0) if self.kind == "dropout" else oracle.normal_f32(self.n, 65)
+        self.x = torch.from_numpy(self.xh).to(dev)
+        self.out = self.x.clone() if self.kind == "relu" else torch.empty_like(self.x)
+        self.op = ct.partition(self.out, [1024])
+
+    def launch(self):
+        if self.kind == "relu":
+            self.ct.relu(self.op)
+        elif self.kind == "dropout":
+            self.ct.dropout(0.4, self.x, self.x, self.op)
+        else:
+            self.ct.scale_ptr(self.out.data_ptr(), self.x.data_ptr(), 3.0, self.n, grid=(1024, 1, 1))
+
+    def cpu_baseline(self, oracle, np, torch):
+        t0 = time.perf_counter()
+        ref = {"relu": lambda: oracle.relu_f32(self.xh), "dropout": lambda: oracle.dropout_f32(0.4, self.xh),
+               "scale_ptr": lambda: oracle.scale_f32(self.xh, 3.0)}[self.kind]()
+        dt = time.perf_counter() - t0
+        exact = bool(np.array_equal(self.out.cpu().numpy(), ref))
+        return {"value": self.work / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "full size (numpy)"}, {"bit_exact": exact}
+
+
 def make_workloads():
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            Copy(), RmsNormAllF16(), SoftmaxAllF16(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
+            Copy(), RmsNormAllF16(), SoftmaxAllF16(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv(),
+            BatchMatmul(), Matvec(), ExampleStream("relu"), ExampleStream("dropout"), ExampleStream("scale_ptr")]
 
 
 EXTRA_WORKLOADS = []  # only by name, never in the default run

@@ -188,6 +188,10 @@ std::vector<KernelEntry> build_table() {
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
   // batched GEMM (cutile-examples/examples/batch_matmul.rs): the pipelined bodies with the batch on a grid axis
+  for (const char* dt : {"bf16", "f16"}) {   // ring of three a stages and two b stages; whole K tiles only
+    std::string v = std::string(dt) + "_256x256x64_r2x4";
+    add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 3);
+  }
   for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2}}) {
     std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
     add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),

@@ -654,9 +654,9 @@ cutile_status_t cutile_launch_eye(cutile_stream_t stream, const cutile_partition
   return launch_packed(res.fn, grid, res.entry->block, 0, stream, args);
 }
 // ---- the example programs' small kernels ---------------------------------------------------
-// grid of a flat f32 stream over `count` elements: 16 bytes per lane, four passes per lane at most
+// grid of a flat f32 stream over `count` elements: a workgroup per 1024 vectors of 16 bytes (the kernels loop beyond 2^20 workgroups)
 static void flat_f32_grid(uint64_t count, uint32_t grid[3]) {
-  grid[0] = std::min<uint32_t>(std::max<uint32_t>(1, div_up(count, 256 * 4 * 4)), 16384);
+  grid[0] = std::min<uint32_t>(std::max<uint32_t>(1, div_up(count, 256 * 4 * 4)), 1u << 20);
   grid[1] = grid[2] = 1;
 }
 cutile_status_t cutile_launch_relu(cutile_stream_t stream, const cutile_partition_arg_t* input_output,
@@ -1937,10 +1937,12 @@ cutile_status_t cutile_launch_batch_matmul(cutile_stream_t stream, const cutile_
   };
   const bool fast_layout = ct.dtype != CUTILE_DTYPE_F32 && slice_ok(*a) && slice_ok(*b) && slice_ok(ct) && k_total % 8 == 0 &&
                            (uint32_t)a->shape[0] >= batches && (uint32_t)b->shape[0] >= batches;
+  const int32_t k_valid = std::min(std::min(a->shape[2], b->shape[1]), k_total);
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
-      if (strcmp(e.function, "batch_matmul") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn)
+      if (strcmp(e.function, "batch_matmul") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
+          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
         acceptable.push_back(e.variant);
   acceptable.push_back(dt + "_generic");
   Resolved res;

@@ -205,13 +205,22 @@ __device__ __forceinline__ void flat_map1(const T* src, int64_t src_stride, size
   const size_t step = (size_t)gridDim.x * kThreads, gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
   size_t done = 0;
   if (src_stride == 1 && dst_stride == 1 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    // a workgroup takes kThreads * kUnroll consecutive vectors at a time: kUnroll nontemporal loads in flight per
+    // lane, then the stores (a stream touched once should not push other data out of the caches)
     const size_t nvec = (count < src_count ? count : src_count) / V::N;
-    for (size_t j = gid; j < nvec; j += step) {
-      V in, out;
-      in.raw = reinterpret_cast<const u32x4*>(src)[j];
+    for (size_t j0 = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x; j0 < nvec; j0 += step * kUnroll) {
+      V in[kUnroll];
 #pragma unroll
-      for (int e = 0; e < V::N; ++e) out.v[e] = f(in.v[e]);
-      reinterpret_cast<u32x4*>(dst)[j] = out.raw;
+      for (int u = 0; u < kUnroll; ++u)
+        if (j0 + (size_t)u * kThreads < nvec) in[u].raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + j0 + (size_t)u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        if (j0 + (size_t)u * kThreads < nvec) {
+          V out;
+#pragma unroll
+          for (int e = 0; e < V::N; ++e) out.v[e] = f(in[u].v[e]);
+          __builtin_nontemporal_store(out.raw, reinterpret_cast<u32x4*>(dst) + j0 + (size_t)u * kThreads);
+        }
     }
     done = nvec * V::N;
   }

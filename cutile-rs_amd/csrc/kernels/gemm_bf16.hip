@@ -1007,15 +1007,19 @@ __device__ __forceinline__ void batch_slices(const PartitionArg<3>& c, const Ten
   }
 }
 // tile grid (batches, M tiles, N tiles); HIP grid (M tiles * N tiles, batches, 1)
-#define BATCH_MATMUL_KERNEL(NAME, T, BM, BN, WVM, WVN)                                           \
+#define BATCH_MATMUL_KERNEL(NAME, T, BM, BN, WVM, WVN) BATCH_MATMUL_KERNEL_OF(GemmDirect, NAME, T, BM, BN, WVM, WVN)
+#define BATCH_MATMUL_KERNEL_OF(BODY, NAME, T, BM, BN, WVM, WVN)                                  \
   extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
       batch_matmul_entry__##NAME(PartitionArg<3> c, TensorArg<3> a, TensorArg<3> b, int32_t k, TileGrid g) { \
     PartitionArg<2> z;                                                                         \
     TensorArg<2> x, y;                                                                         \
     batch_slices<T>(c, a, b, blockIdx.y, &z, &x, &y);                                          \
     const TileGrid tiles = {g.y, g.z, 1, 0};                                                   \
-    GemmDirect<BM, BN, WVM, WVN, T, T>::run(z, x, y, k, tiles, 0);                             \
+    BODY<BM, BN, WVM, WVN, T, T>::run(z, x, y, k, tiles, 0);                                   \
   }
+// the ring-pipelined bodies first (they fetch whole K tiles only: K % 64 == 0)
+BATCH_MATMUL_KERNEL_OF(GemmRing, bf16_256x256x64_r2x4, __bf16, 256, 256, 2, 4)
+BATCH_MATMUL_KERNEL_OF(GemmRing, f16_256x256x64_r2x4, _Float16, 256, 256, 2, 4)
 BATCH_MATMUL_KERNEL(bf16_256x256x64_d2x4, __bf16, 256, 256, 2, 4)
 BATCH_MATMUL_KERNEL(bf16_128x128x64_d2x2, __bf16, 128, 128, 2, 2)
 BATCH_MATMUL_KERNEL(f16_256x256x64_d4x2, _Float16, 256, 256, 4, 2)

@@ -174,7 +174,8 @@ def test_batch_matmul_f32_ragged(ct, dev, batch, m, n, k, bm, bn, bk):
     assert (err <= 1e-5 * mag + 1e-30).all(), err.max()
 
 
-@pytest.mark.parametrize("dtype,tile,variant", [("bf16", 256, "bf16_256x256x64_d2x4"), ("bf16", 128, "bf16_128x128x64_d2x2"),
+@pytest.mark.parametrize("dtype,tile,variant", [("bf16", 256, "bf16_256x256x64_r2x4"), ("bf16", 256, "bf16_256x256x64_d2x4"),
+                                                ("bf16", 128, "bf16_128x128x64_d2x2"), ("f16", 256, "f16_256x256x64_r2x4"),
                                                 ("f16", 256, "f16_256x256x64_d4x2"), ("f16", 128, "f16_128x128x64_d2x2"),
                                                 ("bf16", 128, "bf16_generic"), ("f16", 64, "f16_generic")])
 def test_batch_matmul_16_bit_against_the_gemm_oracle(ct, dev, dtype, tile, variant):
@@ -185,8 +186,7 @@ def test_batch_matmul_16_bit_against_the_gemm_oracle(ct, dev, dtype, tile, varia
     to_f32 = oracle.bf16_bits_to_f32 if dtype == "bf16" else oracle.f16_bits_to_f32
     a_bits, b_bits = mk((batch, m, k), 461, 1.0), mk((batch, k, n), 462, k ** -0.5)
     c = torch.full((batch, m, n), 5.0, device=dev).to(torch.bfloat16 if dtype == "bf16" else torch.half)
-    ct.batch_matmul(ct.partition(c, [1, tile, tile]), to_dev(a_bits, dev), to_dev(b_bits, dev), k, generics=[dtype, tile, tile, 64, k],
-                    variant=variant if "generic" in variant else None)
+    ct.batch_matmul(ct.partition(c, [1, tile, tile]), to_dev(a_bits, dev), to_dev(b_bits, dev), k, generics=[dtype, tile, tile, 64, k], variant=variant)
     sync()
     assert ct.last_resolved()["variant"] == variant
     a, b = to_f32(a_bits), to_f32(b_bits)
@@ -196,6 +196,18 @@ def test_batch_matmul_16_bit_against_the_gemm_oracle(ct, dev, dtype, tile, varia
     mag = np.einsum("bmk,bkn->bmn", np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
     for i in range(batch):
         assert_rounded_close(got[i], want[i], (tile, tile), rel_ulp=2.0 ** -7 if dtype == "bf16" else 2.0 ** -10, what=f"batch {i}", mag=mag[i])
+
+
+def test_batch_matmul_default_variants(ct, dev):
+    # whole K tiles of 64: the ring-pipelined body; a K that is not (the pipelined one that masks the K tail); f32: any-layout
+    for k, want in ((128, "bf16_256x256x64_r2x4"), (96, "bf16_256x256x64_d2x4")):
+        a_bits, b_bits = normal_bf16_bits((2, 256, k), 465), normal_bf16_bits((2, k, 256), 466, k ** -0.5)
+        c = torch.zeros(2, 256, 256, device=dev, dtype=torch.bfloat16)
+        ct.batch_matmul(ct.partition(c, [1, 256, 256]), to_dev_bf16(a_bits, dev), to_dev_bf16(b_bits, dev), k, generics=["bf16", 256, 256, 32, k])
+        sync()
+        assert ct.last_resolved()["variant"] == want
+        ref = oracle.batch_matmul_f32(oracle.bf16_bits_to_f32(a_bits), oracle.bf16_bits_to_f32(b_bits))
+        assert rel_l2(oracle.bf16_bits_to_f32(from_dev_bf16_bits(c)), ref) <= 1e-2
 
 
 def test_batch_matmul_batches_are_independent_and_strided(ct, dev):
