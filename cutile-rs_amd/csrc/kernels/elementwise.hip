@@ -176,16 +176,31 @@ __device__ __forceinline__ void flat_convert(const S* src, int64_t src_stride, s
   const size_t step = (size_t)gridDim.x * kThreads, gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
   size_t done = 0;
   if (src_stride == 1 && dst_stride == 1 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    // a workgroup takes kThreads * kGroups consecutive groups of kElems elements at a time and requests all of a
+    // lane's loads before it converts the first value (at least 64 bytes in flight per lane)
+    constexpr int kGroups = kSrcVecs >= 4 ? 1 : kSrcVecs == 2 ? 2 : 4;
     const size_t nvec = (count < src_count ? count : src_count) / kElems;
-    for (size_t j = gid; j < nvec; j += step) {
-      union { u32x4 raw[kSrcVecs]; S v[kElems]; } in;
-      union { u32x4 raw[kDstVecs]; D v[kElems]; } out;
+    for (size_t j0 = (size_t)blockIdx.x * (kThreads * kGroups) + threadIdx.x; j0 < nvec; j0 += step * kGroups) {
+      union { u32x4 raw[kSrcVecs]; S v[kElems]; } in[kGroups];
 #pragma unroll
-      for (int q = 0; q < kSrcVecs; ++q) in.raw[q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + j * kSrcVecs + q);
+      for (int u = 0; u < kGroups; ++u) {
+        const size_t j = j0 + (size_t)u * kThreads;
+        if (j < nvec) {
 #pragma unroll
-      for (int e = 0; e < kElems; ++e) out.v[e] = convert_elem<D, S>(in.v[e]);
+          for (int q = 0; q < kSrcVecs; ++q) in[u].raw[q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + j * kSrcVecs + q);
+        }
+      }
 #pragma unroll
-      for (int q = 0; q < kDstVecs; ++q) __builtin_nontemporal_store(out.raw[q], reinterpret_cast<u32x4*>(dst) + j * kDstVecs + q);
+      for (int u = 0; u < kGroups; ++u) {
+        const size_t j = j0 + (size_t)u * kThreads;
+        if (j < nvec) {
+          union { u32x4 raw[kDstVecs]; D v[kElems]; } out;
+#pragma unroll
+          for (int e = 0; e < kElems; ++e) out.v[e] = convert_elem<D, S>(in[u].v[e]);
+#pragma unroll
+          for (int q = 0; q < kDstVecs; ++q) __builtin_nontemporal_store(out.raw[q], reinterpret_cast<u32x4*>(dst) + j * kDstVecs + q);
+        }
+      }
     }
     done = nvec * kElems;
   }
@@ -365,6 +380,26 @@ extern "C" __global__ void __launch_bounds__(kThreads)
                    vec_ok(k_cache.ptr, k_cache.strides) && vec_ok(v_cache.ptr, v_cache.strides);
   const int32_t per_row = vec ? d / 8 : d;
   const int64_t total = (int64_t)seq_len * heads * per_row;
+  if (vec && (per_row & (per_row - 1)) == 0 && per_row <= kThreads && (int64_t)seq_len * heads < (1ll << 31)) {
+    // Head rows of 8, 16 or 32 vectors (D = 64, 128, 256): a lane keeps its place in the row and groups of lanes walk
+    // the (position, head) rows, so an item costs one 32-bit division.  The general walk below takes four 64-bit
+    // divisions per item, which is more vector work than the copy is memory work.
+    const uint32_t shift = (uint32_t)__builtin_ctz((uint32_t)per_row);
+    const uint32_t c = threadIdx.x & (uint32_t)(per_row - 1), rows_per_wg = (uint32_t)kThreads >> shift;
+    const uint32_t n_rows = (uint32_t)seq_len * (uint32_t)heads;
+    for (uint32_t r = blockIdx.x * rows_per_wg + (threadIdx.x >> shift); r < n_rows; r += gridDim.x * rows_per_wg) {
+      const uint32_t sidx = r / (uint32_t)heads, h = r - sidx * (uint32_t)heads;
+      const int64_t pos = (int64_t)base + sidx;
+      if (pos < 0 || pos >= max_seq) continue;
+      const u32x4 kv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+          (const _Float16*)new_k.ptr + (int64_t)sidx * new_k.strides[0] + (int64_t)h * new_k.strides[1]) + c);
+      const u32x4 vv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+          (const _Float16*)new_v.ptr + (int64_t)sidx * new_v.strides[0] + (int64_t)h * new_v.strides[1]) + c);
+      __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>((_Float16*)k_cache.ptr + (int64_t)h * k_cache.strides[0] + pos * k_cache.strides[1]) + c);
+      __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>((_Float16*)v_cache.ptr + (int64_t)h * v_cache.strides[0] + pos * v_cache.strides[1]) + c);
+    }
+    return;
+  }
   for (int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
     const int32_t c = (int32_t)(t % per_row);
     const int64_t sh = t / per_row;
@@ -938,10 +973,20 @@ extern "C" __global__ void __launch_bounds__(kThreads)
     const _Float16* src = tp + (int64_t)token * table.strides[0];
     _Float16* dst = op + (int64_t)row * out.strides[0];
     if (vec) {
-      for (int32_t c = threadIdx.x; c < width / 8; c += kThreads) {
-        u32x4 v = {0, 0, 0, 0};
-        if (known && c * 8 < table.shape[1]) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + c);
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst) + c);
+      // up to four vectors per lane requested before the first is stored (a row of 4096 halves is two per lane)
+      for (int32_t c0 = threadIdx.x; c0 < width / 8; c0 += kThreads * kUnroll) {
+        u32x4 v[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int32_t c = c0 + u * kThreads;
+          v[u] = u32x4{0, 0, 0, 0};
+          if (known && c < width / 8 && c * 8 < table.shape[1]) v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + c);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int32_t c = c0 + u * kThreads;
+          if (c < width / 8) __builtin_nontemporal_store(v[u], reinterpret_cast<u32x4*>(dst) + c);
+        }
       }
     } else {
       for (int32_t c = threadIdx.x; c < width; c += kThreads)

@@ -353,8 +353,9 @@ __device__ __forceinline__ void softmax_segments(const T* __restrict__ x, int64_
   const int slot = wave / WPR, sub = wave % WPR;
   const int64_t seg = (int64_t)blockIdx.x * SEGS_PER_WG + slot;
   const bool live = seg < n_segments;
-  const int64_t row = live ? seg / segs_per_row : 0;
-  const int32_t col0 = live ? (int32_t)(seg % segs_per_row) * seg_len : 0;
+  // whole rows (one segment per row) are the common case: no 64-bit division on the way to the first load
+  const int64_t row = !live ? 0 : segs_per_row == 1 ? seg : seg / segs_per_row;
+  const int32_t col0 = !live || segs_per_row == 1 ? 0 : (int32_t)(seg % segs_per_row) * seg_len;
   const int32_t seg_vec = seg_len / E;                 // vectors in a full segment
   const int32_t x_valid = live ? max(0, min(seg_len, x_cols - col0)) / E : 0;  // readable vectors
   const int32_t y_valid = live ? max(0, min(seg_len, y_cols - col0)) / E : 0;  // storable vectors
@@ -363,10 +364,16 @@ __device__ __forceinline__ void softmax_segments(const T* __restrict__ x, int64_
   V xv[VPL];
   float m = -INFINITY;
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * x_row_stride + col0);
+  // every load is requested before the first value is looked at: a use between two loads makes the second
+  // wait for the first, and the row would cost VPL memory latencies instead of one
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     int32_t vi = v0 + i * (64 * WPR);
     if (vi < x_valid) xv[i].raw = __builtin_nontemporal_load(xr + vi);  // else stays 0 (padding)
+  }
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int32_t vi = v0 + i * (64 * WPR);
     if (live && vi < seg_vec) {
 #pragma unroll
       for (int e = 0; e < E; ++e) m = fmaxf(m, to_f32(xv[i].v[e]));
@@ -768,14 +775,22 @@ __device__ __forceinline__ void softmax_all_f16_segments(const TensorArg<2>& x, 
     const _Float16* xr = (const _Float16*)x.ptr + row * x.strides[0];
     _Float16* yr = (_Float16*)y.ptr + row * y.strides[0];
     hv a[CH];
+    if (bn == CH * 64 * V && col0 + bn <= n_cols) {
+      // the whole tile row lies inside the tensor: nothing but vector loads, all requested before the first use
+      // (an element-wise path between them would make every chunk wait for the one before: CH memory latencies)
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int32_t col = col0 + c * 64 * V + lane * V;
-      if (active && col + V <= n_cols) {
-        a[c] = __builtin_nontemporal_load(reinterpret_cast<const hv*>(xr + col));   // streamed: read once
-      } else {
+      for (int c = 0; c < CH; ++c)
+        a[c] = __builtin_nontemporal_load(reinterpret_cast<const hv*>(xr + col0 + c * 64 * V + lane * V));   // streamed: read once
+    } else {
 #pragma unroll
-        for (int e = 0; e < V; ++e) a[c][e] = (active && col + e < n_cols) ? xr[col + e] : (_Float16)0.0f;
+      for (int c = 0; c < CH; ++c) {
+        const int32_t col = col0 + c * 64 * V + lane * V;
+        if (active && col + V <= n_cols) {
+          a[c] = __builtin_nontemporal_load(reinterpret_cast<const hv*>(xr + col));
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) a[c][e] = (active && col + e < n_cols) ? xr[col + e] : (_Float16)0.0f;
+        }
       }
     }
     hv mv = a[0];
