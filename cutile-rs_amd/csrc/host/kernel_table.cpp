@@ -159,7 +159,7 @@ std::vector<KernelEntry> build_table() {
     std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" +
                     std::to_string(bk) + "_" + kind + std::to_string(wvm) + "x" + std::to_string(wvn);
     // "r" = ring of three x stages and two y stages, the others hold two stages of each
-    const uint32_t lds = kind[0] == 'r' ? (uint32_t)((3 * bm * bk + 2 * bk * bn) * 2) : (uint32_t)(2 * (bm * bk + bk * bn) * 2);
+    const uint32_t lds = kind[0] == 'r' || kind[0] == 'q' ? (uint32_t)((3 * bm * bk + 2 * bk * bn) * 2) : (uint32_t)(2 * (bm * bk + bk * bn) * 2);
     add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64), lds, bm, bn, bk, 0, dtype, 0, 2);
   };
   // first entry of a tile shape = default variant; "d" = global->LDS direct, pipelined
@@ -169,6 +169,7 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 256, 256, 64, 4, 2, "r");
   gemm("bf16", 256, 256, 64, 2, 4, "r");
   gemm("bf16", 128, 128, 64, 2, 2, "r");
+  gemm("bf16", 256, 256, 64, 2, 4, "q");   // "q" = the ring on v_mfma_f32_16x16x32
   gemm("bf16", 256, 256, 64, 4, 2);
   gemm("bf16", 256, 256, 64, 2, 4);
   gemm("bf16", 256, 256, 64, 2, 2);
@@ -180,6 +181,7 @@ std::vector<KernelEntry> build_table() {
   gemm("f16", 128, 128, 64, 2, 2, "d");
   gemm("f16", 256, 256, 64, 4, 2, "r");
   gemm("f16", 256, 256, 64, 2, 4, "r");
+  gemm("f16", 256, 256, 64, 2, 4, "q");
   gemm("bf16f32", 128, 128, 64, 2, 2);
   gemm("bf16f32", 256, 256, 64, 2, 2);
   // any tile shape, strides and extents (tile = 0: not tied to a partition shape); 64x64 outputs per workgroup
@@ -188,10 +190,11 @@ std::vector<KernelEntry> build_table() {
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
   // batched GEMM (cutile-examples/examples/batch_matmul.rs): the pipelined bodies with the batch on a grid axis
-  for (const char* dt : {"bf16", "f16"}) {   // ring of three a stages and two b stages; whole K tiles only
-    std::string v = std::string(dt) + "_256x256x64_r2x4";
-    add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 3);
-  }
+  for (const char* kind : {"q", "r"})          // rings of three a stages and two b stages (q: on v_mfma_f32_16x16x32); whole K tiles only
+    for (const char* dt : {"bf16", "f16"}) {
+      std::string v = std::string(dt) + "_256x256x64_" + kind + "2x4";
+      add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 3);
+    }
   for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2}}) {
     std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);
     add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),

@@ -737,6 +737,242 @@ struct GemmRing {
   }
 };
 
+// ---- the ring variant on v_mfma_f32_16x16x32 -----------------------------------------------
+// Same stages, fetches, barriers and wait counts as GemmRing; the matrix instruction is the 16 x 16 x 32 form.
+// On this chip the matrix kernels run against the power limit, and per flop the 16 x 16 x 32 form writes half as
+// many accumulator values as 32 x 32 x 16: a loop of nothing but MFMAs on random bf16 operands sustains
+// 2093 TFLOP/s with it against 1854 (equal, 2463 - 2481, on constant operands).  A block is 16 MFMAs (half of the
+// sub-tile's rows by all of its columns, one 32-wide K step) and lasts as long as a block of GemmRing; the y
+// fragments of a K step serve two blocks, so LDS traffic is unchanged.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT, typename InT = __bf16>
+struct GemmRing16 {
+  static constexpr int BK = 64;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 16, TN = WN / 16;   // 16 x 16 accumulator blocks of the wavefront's sub-tile
+  static constexpr int TMH = TM / 2;                   // x fragments of one MFMA block (half the sub-tile's rows)
+  static_assert(TM % 2 == 0, "a block takes half of the sub-tile's rows");
+  static constexpr int UB = BN / 8;                         // 16-byte units per y-tile row
+  static constexpr int kAInstr = BM / 8 / kWaves;           // 1 KiB = 8 x-tile rows
+  static constexpr int kBRowsPerInstr = 64 / UB;
+  static constexpr int kBInstr = BK / kBRowsPerInstr / kWaves;
+  static constexpr int kABytes = BM * BK * 2, kBBytes = BK * BN * 2;
+  static constexpr int kLdsBytes = 3 * kABytes + 2 * kBBytes;
+  static_assert(BM % (8 * kWaves) == 0 && BK % (kBRowsPerInstr * kWaves) == 0, "tile must split evenly");
+  static_assert(UB >= 16 && UB <= 64, "y-tile row must be 16..64 units");
+  static_assert(kBInstr % 2 == 0, "each wavefront fetches the same share of both y halves");
+  static_assert(kAInstr + kBInstr <= 15, "the wait count must fit the low vmcnt field");
+
+  __device__ static __forceinline__ int a_lds_off(int r, int u) { return r * (BK * 2) + ((u ^ ((r >> 1) & 7)) << 4); }
+  // y rows 8 apart are read by neighbouring lane groups of one transposing read: bit 3 of the row moves them 32 bytes apart
+  __device__ static __forceinline__ int b_swizzle(int r) { return ((r & 3) << 2) | (((r >> 3) & 1) << 1); }
+  __device__ static __forceinline__ int b_lds_off(int r, int u) { return r * (BN * 2) + ((u ^ b_swizzle(r)) << 4); }
+
+
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                             int32_t k_total, const TileGrid& g, int32_t accumulate) {
+    // Separately named stages: the compiler can then tell a refill of one from
+    // operand reads of another and adds no waits of its own.
+    __shared__ __attribute__((aligned(1024))) unsigned char xs0[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs1[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs2[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char ys0a[kBBytes / 2];  // y stage 0, K rows 0..31
+    __shared__ __attribute__((aligned(1024))) unsigned char ys0b[kBBytes / 2];  //            K rows 32..63
+    __shared__ __attribute__((aligned(1024))) unsigned char ys1a[kBBytes / 2];
+    __shared__ __attribute__((aligned(1024))) unsigned char ys1b[kBBytes / 2];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    const int32_t M = x.shape[0], N = y.shape[1];
+    const int32_t lda = x.strides[0], ldb = y.strides[0];
+    const int32_t row0 = pm * BM, col0 = pn * BN;
+    const int32_t k_valid = min(min(x.shape[1], y.shape[0]), k_total);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)(((int64_t)(M - 1) * lda + x.shape[1]) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)(((int64_t)(y.shape[0] - 1) * ldb + N) * 2));
+    constexpr uint32_t kOob = 0x80000000u;
+
+    // Global side of the fetches (per lane, K tile 0; the K advance is scalar).
+    // y instruction i of this wavefront covers K rows of half i / (kBInstr/2).
+    uint32_t a_goff[kAInstr], b_goff[kBInstr];
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_goff[i] = (row0 + r < M) ? (uint32_t)(((int64_t)(row0 + r) * lda + u * 8) * 2) : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < kBInstr; ++i) {
+      const int r = (i * kWaves + wave) * kBRowsPerInstr + lane / UB;
+      const int u = (lane % UB) ^ b_swizzle(r);
+      b_goff[i] = (col0 + u * 8 < N) ? (uint32_t)(((int64_t)r * ldb + col0 + u * 8) * 2) : kOob;
+    }
+    // K is a whole number of tiles here (the launcher sends ragged K to the
+    // two-stage variant), so a tile is either wholly inside K or wholly beyond it;
+    // beyond it every lane's offset is out of range and the fetch reads zeros.
+    auto fetch_a = [&](unsigned char* stage, int32_t k0, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
+                                               k0 < k_valid ? a_goff[i] : kOob, k0 * 2, 0, 0);
+    };
+    // `half` = the y half-stage receiving K rows 32*h..32*h+31, h = i / (kBInstr/2)
+    auto fetch_b = [&](unsigned char* half, int32_t k0, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(half + ((i % (kBInstr / 2)) * kWaves + wave) * 1024),
+                                               16, k0 < k_valid ? b_goff[i] : kOob, k0 * ldb * 2, 0, 0);
+    };
+
+    // LDS side of the operand reads (byte offsets inside a stage).  v_mfma_f32_16x16x32: a lane holds 8 consecutive K
+    // values (group lane / 16 of the 32-wide K step) of row lane % 16 of its operand.
+    const int grp = lane >> 4, l16 = lane & 15;
+    const int tr_row = l16 >> 2, tr_col = (l16 & 3) * 4;
+    // x: the swizzle term of row r + 16 tm is that of row r, so one address per K step serves all row blocks
+    // (16 rows = 16 * BK * 2 bytes further on, an immediate offset of the read)
+    int a_addr[2], b_addr[TN];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) a_addr[ks] = a_lds_off(wm * WM + l16, ks * 4 + grp);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int n = wn * WN + tn * 16 + tr_col;
+      const int kr = grp * 8 + tr_row;         // row inside the y half-stage that holds this K step; the swizzle of kr + 4 is the same
+      b_addr[tn] = b_lds_off(kr, n >> 3) + (n & 7) * 2;
+    }
+    constexpr int NB = TMH * TN;  // MFMAs per block: half the sub-tile's rows, one 32-wide K step
+    // x fragments i of rows [mh * TMH * 16, ..) at K step ks of stage xs
+    auto read_a = [&](const unsigned char* xs, int ks, int mh, bf16x8 (&into)[TMH], int i) {
+      into[i] = *reinterpret_cast<const bf16x8*>(xs + a_addr[ks] + (mh * TMH + i) * (16 * BK * 2));
+    };
+    // y fragment tn of the K step held by the half-stage yh
+    auto read_b = [&](const unsigned char* yh, bf16x8 (&into)[TN], int tn) {
+      const unsigned char* p = yh + b_addr[tn];
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 4 * (BN * 2)));
+      into[tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+
+    f32x4 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[tn][tm][v] = 0.0f;
+
+    // One MFMA block: rows [mh * TMH * 16, ..) of the sub-tile times all its columns, on the x fragments `a` and the
+    // y fragments `ub`, row block by row block.  Dealt out between its MFMAs, at most two per MFMA and in this
+    // order: refill instructions first..last of the x stage `fill_x` (if any) and of the y stage `fill_y`
+    // (instructions fb0..fb1-1), then, if rd_y, the reads of the next K step's y fragments into `ib`.  The x
+    // fragments are one set: as soon as the last MFMA on a row block has issued, its fragment is read again for the
+    // next block (rd_x, rd_ks, rd_mh) — three row blocks of MFMAs before it is used.  A wavefront issues in order
+    // and an MFMA holds the issue slot until the matrix pipe takes it, so memory work placed after a run of MFMAs
+    // would start late; sched_barrier(0) after every step keeps the order written here.
+    constexpr int SLOTS = NB / 2 > 0 ? NB / 2 : 1;
+    // (what a block does besides its MFMAs is said by the flags with_y / with_fill_x and the range fb0..fb1: a null
+    // test of an LDS pointer is a run-time test, address 0 being a valid one)
+    auto block = [&](bf16x8 (&a)[TMH], const bf16x8 (&ub)[TN], int mh, const unsigned char* rd_x, int rd_ks, int rd_mh,
+                     bool with_y, const unsigned char* rd_y, bf16x8 (&ib)[TN], bool with_fill_x, unsigned char* fill_x,
+                     unsigned char* fill_y, int fb0, int fb1, int32_t k0_x, int32_t k0_y) {
+      const int n_fill = (with_fill_x ? kAInstr : 0) + (fb1 - fb0);
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int tm = j / TN, tn = j % TN;
+#pragma unroll
+        for (int i = 0; i < kAInstr + kBInstr; ++i) {
+          if (i < n_fill && i * SLOTS / n_fill == j) {
+            if (with_fill_x && i < kAInstr)
+              fetch_a(fill_x, k0_x, i);
+            else
+              fetch_b(fill_y, k0_y, fb0 + i - (with_fill_x ? kAInstr : 0));
+          }
+        }
+        if (with_y) {
+#pragma unroll
+          for (int q = 0; q < TN; ++q)
+            if (q * SLOTS / TN == j) read_b(rd_y, ib, q);
+        }
+        acc[tn][mh * TMH + tm] = mfma_16x16x32<InT>(ub[tn], a[tm], acc[tn][mh * TMH + tm]);
+        if (tn == TN - 1) read_a(rd_x, rd_ks, rd_mh, a, tm);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // s_waitcnt immediate of gfx9: vmcnt [3:0] (and [15:14]), expcnt [6:4], lgkmcnt [11:8].
+    constexpr int kWaitOlderLoads = (kAInstr + kBInstr) | (7 << 4) | (0 << 8);
+    constexpr int kWaitPrologue = ((2 * kAInstr + 3 * kBInstr / 2) & 15) | (7 << 4) | (0 << 8) | (((2 * kAInstr + 3 * kBInstr / 2) >> 4) << 14);
+
+    const int k_tiles = (k_total + BK - 1) / BK;
+    bf16x8 af[TMH], b0[TN], b1[TN];
+    // Prologue, in the issue order the steady state would have produced.
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs0, 0, i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys0a, 0, i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs1, BK, i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys0b, 0, i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys1a, BK, i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs2, 2 * BK, i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys1b, BK, i);
+    __builtin_amdgcn_s_waitcnt(kWaitPrologue);  // x tile 0 and the first y half of tile 0 have landed
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) read_b(ys0a, b0, tn);
+#pragma unroll
+    for (int i = 0; i < TMH; ++i) read_a(xs0, 0, 0, af, i);
+
+    // Tile kt lives in x_cur and the y halves (ya_cur, yb_cur); tile kt+1 in x_nxt, ya_nxt.
+    auto k_tile = [&](unsigned char* x_cur, unsigned char* ya_cur, unsigned char* yb_cur, const unsigned char* x_nxt,
+                      const unsigned char* ya_nxt, int kt) {
+      // blocks: (K step 0, upper rows) (K step 0, lower rows) (K step 1, upper) (K step 1, lower); every block reads
+      // the next block's x fragments, the second and the fourth also the next K step's y fragments
+      block(af, b0, 0, x_cur, 0, 1, false, x_cur, b1, false, x_cur, x_cur, 0, 0, 0, 0);
+      // First y half of tile kt is in registers everywhere; its second half has landed.
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(af, b0, 1, x_cur, 1, 0, true, yb_cur, b1, false, x_cur, ya_cur, 0, kBInstr / 2, 0, (kt + 2) * BK);
+      block(af, b1, 0, x_cur, 1, 1, false, x_cur, b0, false, x_cur, x_cur, 0, 0, 0, 0);
+      // Hand-over: all of tile kt is in registers; x tile kt+1 and its first y half have landed.
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(af, b1, 1, x_nxt, 0, 0, true, ya_nxt, b0, true, x_cur, yb_cur, kBInstr / 2, kBInstr, (kt + 3) * BK, (kt + 2) * BK);
+    };
+    // The stage names repeat every 6 tiles (3 x stages, 2 y stages).
+    int kt = 0;
+    for (; kt + 6 <= k_tiles; kt += 6) {
+      k_tile(xs0, ys0a, ys0b, xs1, ys1a, kt);
+      k_tile(xs1, ys1a, ys1b, xs2, ys0a, kt + 1);
+      k_tile(xs2, ys0a, ys0b, xs0, ys1a, kt + 2);
+      k_tile(xs0, ys1a, ys1b, xs1, ys0a, kt + 3);
+      k_tile(xs1, ys0a, ys0b, xs2, ys1a, kt + 4);
+      k_tile(xs2, ys1a, ys1b, xs0, ys0a, kt + 5);
+    }
+    const int rest = k_tiles - kt;
+    if (rest > 0) k_tile(xs0, ys0a, ys0b, xs1, ys1a, kt);
+    if (rest > 1) k_tile(xs1, ys1a, ys1b, xs2, ys0a, kt + 1);
+    if (rest > 2) k_tile(xs2, ys0a, ys0b, xs0, ys1a, kt + 2);
+    if (rest > 3) k_tile(xs0, ys1a, ys1b, xs1, ys0a, kt + 3);
+    if (rest > 4) k_tile(xs1, ys0a, ys0b, xs2, ys1a, kt + 4);
+    __builtin_amdgcn_s_waitcnt(0);  // trailing (zero-filling) fetches must not outlive the workgroup's LDS
+
+    // Every wavefront is past its operand reads and every fetch has landed: the
+    // stages are free to carry the output (two wavefronts share an x stage, the
+    // last two take the y stages).
+    __syncthreads();
+    static_assert(2 * kEpilogueBytesPerWave<WN> <= kABytes && kEpilogueBytesPerWave<WN> <= kBBytes / 2 && kWaves <= 10,
+                  "the output bands must fit the stages");
+    unsigned char* band = wave < 2 ? xs0 : wave < 4 ? xs1 : wave < 6 ? xs2 : wave == 6 ? ys0a : wave == 7 ? ys0b : wave == 8 ? ys1a : ys1b;
+    if (wave < 6) band += (wave & 1) * kEpilogueBytesPerWave<WN>;
+    store_tile_staged16<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0], z.shape[0], z.shape[1], row0 + wm * WM,
+                                    col0 + wn * WN, lane, accumulate);
+  }
+};
+
 // ---- any-layout variant ---------------------------------------------------------------------
 // The tile program for arbitrary tile shapes, element types (bf16, f16, f32),
 // strides and extents — what the pipelined variants cannot take (rows that are
@@ -952,6 +1188,16 @@ GEMM_RING_KERNEL(bf16_128x128x64_r2x2, 128, 128, 2, 2, __bf16)
 GEMM_RING_KERNEL_F16(f16_256x256x64_r2x4, 256, 256, 2, 4)
 GEMM_RING_KERNEL_F16(f16_256x256x64_r4x2, 256, 256, 4, 2)
 
+// the ring pipeline on v_mfma_f32_16x16x32 ("q")
+#define GEMM_RING16_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T, IN_T)                                  \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmRing16<BM, BN, WVM, WVN, OUT_T, IN_T>::run(z, x, y, k, g, accumulate);                  \
+  }
+GEMM_RING16_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16, __bf16)
+GEMM_RING16_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16, _Float16)
+
 #define GEMM_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                                \
   extern "C" __global__ void __launch_bounds__(256)                                            \
       gemm_entry__##NAME##_generic(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, \
@@ -1018,6 +1264,8 @@ __device__ __forceinline__ void batch_slices(const PartitionArg<3>& c, const Ten
     BODY<BM, BN, WVM, WVN, T, T>::run(z, x, y, k, tiles, 0);                                   \
   }
 // the ring-pipelined bodies first (they fetch whole K tiles only: K % 64 == 0)
+BATCH_MATMUL_KERNEL_OF(GemmRing16, bf16_256x256x64_q2x4, __bf16, 256, 256, 2, 4)
+BATCH_MATMUL_KERNEL_OF(GemmRing16, f16_256x256x64_q2x4, _Float16, 256, 256, 2, 4)
 BATCH_MATMUL_KERNEL_OF(GemmRing, bf16_256x256x64_r2x4, __bf16, 256, 256, 2, 4)
 BATCH_MATMUL_KERNEL_OF(GemmRing, f16_256x256x64_r2x4, _Float16, 256, 256, 2, 4)
 BATCH_MATMUL_KERNEL(bf16_256x256x64_d2x4, __bf16, 256, 256, 2, 4)

@@ -71,6 +71,18 @@ __device__ __forceinline__ f32x16 mfma_32x32x16(bf16x8 a, bf16x8 b, f32x16 c) {
   }
 }
 
+// v_mfma_f32_16x16x32 on the same fragments: half as many accumulator values written per flop.
+typedef float f32x4_acc __attribute__((ext_vector_type(4)));
+template <typename InT>
+__device__ __forceinline__ f32x4_acc mfma_16x16x32(bf16x8 a, bf16x8 b, f32x4_acc c) {
+  if constexpr (__is_same(InT, _Float16)) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+}
+
 // Tile index for this workgroup: XCD-contiguous, then grouped along M.
 __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, uint32_t* pm,
                                             uint32_t* pn) {
@@ -130,17 +142,17 @@ __device__ __forceinline__ void store_z(V v, V* p, bool stream) {
   }
 }
 
-template <int TM, int TN, typename OutT>
-__device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
-                                                  int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
-                                                  int lane, int32_t accumulate) {
-  constexpr int WN = TN * 32;
+// `write_band(tm)` puts rows [32 tm, 32 tm + 32) of the wavefront's sub-tile into `stage` (f32, row r at r * WN * 4,
+// 16-byte chunk c of row r at chunk c ^ (r & 15)); TM = 32-row bands, WN = columns of the sub-tile.
+template <int TM, int WN, typename OutT, typename BandWriter>
+__device__ __forceinline__ void store_bands_staged(BandWriter write_band, unsigned char* stage, OutT* zp, int32_t ldz,
+                                                   int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
+                                                   int lane, int32_t accumulate) {
   constexpr int PITCH = WN * 4;
   constexpr int COLS_PER_LANE = sizeof(OutT) == 2 ? 8 : 4;      // 16 bytes of output per lane
   constexpr int LANES_PER_ROW = WN / COLS_PER_LANE;
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
   constexpr int PASSES = 32 / ROWS_PER_PASS;
-  const int l32 = lane & 31, khalf = lane >> 5;
   const int rd_row = lane / LANES_PER_ROW, rd_col = (lane % LANES_PER_ROW) * COLS_PER_LANE;
   const int32_t gc = wave_col0 + rd_col;
   const bool col_ok = gc < zN;
@@ -170,13 +182,7 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) {
     // write this band in the MFMA layout
-#pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        f32x4 v = {acc[tn][tm][q * 4 + 0], acc[tn][tm][q * 4 + 1], acc[tn][tm][q * 4 + 2], acc[tn][tm][q * 4 + 3]};
-        *reinterpret_cast<f32x4*>(stage + l32 * PITCH + (((tn * 8 + q * 2 + khalf) ^ (l32 & 15)) << 4)) = v;
-      }
+    write_band(tm);
     // read it back row-contiguous and store
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
@@ -214,6 +220,49 @@ __device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigne
       }
     }
   }
+}
+
+// accumulators of v_mfma_f32_32x32x16: a lane holds row lane % 32 and, per 32-column block, the column quadruples
+// 2 q + lane / 32 (q = 0..3)
+template <int TM, int TN, typename OutT>
+__device__ __forceinline__ void store_tile_staged(f32x16 (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
+                                                  int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
+                                                  int lane, int32_t accumulate) {
+  constexpr int PITCH = TN * 32 * 4;
+  const int l32 = lane & 31, khalf = lane >> 5;
+  store_bands_staged<TM, TN * 32, OutT>(
+      [&](int tm) {
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            f32x4 v = {acc[tn][tm][q * 4 + 0], acc[tn][tm][q * 4 + 1], acc[tn][tm][q * 4 + 2], acc[tn][tm][q * 4 + 3]};
+            *reinterpret_cast<f32x4*>(stage + l32 * PITCH + (((tn * 8 + q * 2 + khalf) ^ (l32 & 15)) << 4)) = v;
+          }
+      },
+      stage, zp, ldz, zM, zN, wave_row0, wave_col0, lane, accumulate);
+}
+// accumulators of v_mfma_f32_16x16x32 (TM, TN count 16 x 16 blocks): a lane holds row lane % 16 and the column
+// quadruple lane / 16 of each block; two row blocks make one 32-row band
+template <int TM, int TN, typename OutT>
+__device__ __forceinline__ void store_tile_staged16(f32x4_acc (&acc)[TN][TM], unsigned char* stage, OutT* zp, int32_t ldz,
+                                                    int32_t zM, int32_t zN, int32_t wave_row0, int32_t wave_col0,
+                                                    int lane, int32_t accumulate) {
+  static_assert(TM % 2 == 0, "two 16-row blocks per band");
+  constexpr int PITCH = TN * 16 * 4;
+  const int l16 = lane & 15, grp = lane >> 4;
+  store_bands_staged<TM / 2, TN * 16, OutT>(
+      [&](int band) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) {
+            const int r = h * 16 + l16;
+            const f32x4 v = {acc[tn][band * 2 + h][0], acc[tn][band * 2 + h][1], acc[tn][band * 2 + h][2], acc[tn][band * 2 + h][3]};
+            *reinterpret_cast<f32x4*>(stage + r * PITCH + (((tn * 4 + grp) ^ (r & 15)) << 4)) = v;
+          }
+      },
+      stage, zp, ldz, zM, zN, wave_row0, wave_col0, lane, accumulate);
 }
 
 }  // namespace gemm

@@ -174,8 +174,8 @@ def test_batch_matmul_f32_ragged(ct, dev, batch, m, n, k, bm, bn, bk):
     assert (err <= 1e-5 * mag + 1e-30).all(), err.max()
 
 
-@pytest.mark.parametrize("dtype,tile,variant", [("bf16", 256, "bf16_256x256x64_r2x4"), ("bf16", 256, "bf16_256x256x64_d2x4"),
-                                                ("bf16", 128, "bf16_128x128x64_d2x2"), ("f16", 256, "f16_256x256x64_r2x4"),
+@pytest.mark.parametrize("dtype,tile,variant", [("bf16", 256, "bf16_256x256x64_q2x4"), ("bf16", 256, "bf16_256x256x64_r2x4"), ("bf16", 256, "bf16_256x256x64_d2x4"),
+                                                ("bf16", 128, "bf16_128x128x64_d2x2"), ("f16", 256, "f16_256x256x64_q2x4"), ("f16", 256, "f16_256x256x64_r2x4"),
                                                 ("f16", 256, "f16_256x256x64_d4x2"), ("f16", 128, "f16_128x128x64_d2x2"),
                                                 ("bf16", 128, "bf16_generic"), ("f16", 64, "f16_generic")])
 def test_batch_matmul_16_bit_against_the_gemm_oracle(ct, dev, dtype, tile, variant):
@@ -200,7 +200,7 @@ def test_batch_matmul_16_bit_against_the_gemm_oracle(ct, dev, dtype, tile, varia
 
 def test_batch_matmul_default_variants(ct, dev):
     # whole K tiles of 64: the ring-pipelined body; a K that is not (the pipelined one that masks the K tail); f32: any-layout
-    for k, want in ((128, "bf16_256x256x64_r2x4"), (96, "bf16_256x256x64_d2x4")):
+    for k, want in ((128, "bf16_256x256x64_q2x4"), (96, "bf16_256x256x64_d2x4")):
         a_bits, b_bits = normal_bf16_bits((2, 256, k), 465), normal_bf16_bits((2, k, 256), 466, k ** -0.5)
         c = torch.zeros(2, 256, 256, device=dev, dtype=torch.bfloat16)
         ct.batch_matmul(ct.partition(c, [1, 256, 256]), to_dev_bf16(a_bits, dev), to_dev_bf16(b_bits, dev), k, generics=["bf16", 256, 256, 32, k])

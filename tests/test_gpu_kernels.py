@@ -281,7 +281,7 @@ def test_softmax_f32(ct, dev, m, n, bm, bn):
 
 
 # ---- K4: bf16 GEMM --------------------------------------------------------------------------
-GEMM_VARIANTS = ["bf16_256x256x64_r2x4", "bf16_256x256x64_r4x2", "bf16_128x128x64_r2x2", "bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
+GEMM_VARIANTS = ["bf16_256x256x64_q2x4", "bf16_256x256x64_r2x4", "bf16_256x256x64_r4x2", "bf16_128x128x64_r2x2", "bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
                  "bf16_128x256x64_w2x2", "bf16_128x128x64_w2x2", "bf16_64x128x64_w2x2"]
 
 
@@ -300,7 +300,7 @@ def test_gemm_bf16_variants(ct, dev, variant):
     np.testing.assert_allclose(got, ref, rtol=1.6e-2, atol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["bf16_256x256x64_r2x4", "bf16_128x128x64_r2x2"])
+@pytest.mark.parametrize("variant", ["bf16_256x256x64_q2x4", "bf16_256x256x64_r2x4", "bf16_128x128x64_r2x2"])
 @pytest.mark.parametrize("k_tiles", [1, 2, 3, 6, 7, 13])
 def test_gemm_ring_pipeline_every_loop_shape(ct, dev, variant, k_tiles):
     # the ring pipeline repeats its stage names every 6 K tiles: cover the unrolled

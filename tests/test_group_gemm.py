@@ -89,7 +89,7 @@ def test_gpu_gemm_f16(ct, dev, m, n, k, tile, accumulate):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("variant", ["f16_256x256x64_r4x2", "f16_256x256x64_r2x4", "f16_256x256x64_d4x2"])
+@pytest.mark.parametrize("variant", ["f16_256x256x64_q2x4", "f16_256x256x64_r4x2", "f16_256x256x64_r2x4", "f16_256x256x64_d4x2"])
 @pytest.mark.parametrize("m,n,k,accumulate", [(512, 768, 1024, False), (300, 264, 448, True), (256, 256, 64, False)])
 def test_gpu_gemm_f16_pipelined_variants(ct, dev, variant, m, n, k, accumulate):
     """every f16 variant of the 256 x 256 tile, the ring-pipelined ones included (whole K tiles), against cpu_gemm"""
