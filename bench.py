@@ -1108,12 +1108,14 @@ def probe_ceilings(ct, torch, flush):
     sink = torch.empty(2 * cus * 512, dtype=torch.float32, device="cuda")
     iters = 20000
     flops = 2.0 * cus * 8 * iters * 2 * 8 * (2 * 32 * 32 * 16)
-    for name, fn in (("mfma_bf16_registers", "probe_mfma_bf16"), ("mfma_bf16_lds_operands", "probe_mfma_bf16_lds")):
+    for name, fn in (("mfma_bf16_registers", "probe_mfma_bf16"), ("mfma_bf16_lds_operands", "probe_mfma_bf16_lds"),
+                     ("mfma_16x16x32_bf16_registers", "probe_mfma16_bf16"), ("mfma_16x16x32_bf16_lds_operands", "probe_mfma16_bf16_lds")):
         f = mod.function(fn)
         for mode, label in ((0, "ones"), (1, "random")):
             med, mn = _timed(ct, torch, flush, lambda: ct.Module.launch(
                 f, (2 * cus, 1, 1), (512, 1, 1), [C.c_void_p(sink.data_ptr()), C.c_int32(iters), C.c_int32(mode)]), reps=7, warm=1)
-            out[f"{name}_{label}"] = {"TFLOP/s": round(flops / (med * 1e-3) / 1e12, 1), "frac_of_2500": round(flops / (med * 1e-3) / 1e12 / 2500, 4),
+            fl = flops * (2.0 if "16x16x32" in name else 1.0)     # 64 MFMAs of 16 x 16 x 32 per iteration: twice the flops of 16 of 32 x 32 x 16
+            out[f"{name}_{label}"] = {"TFLOP/s": round(fl / (med * 1e-3) / 1e12, 1), "frac_of_2500": round(fl / (med * 1e-3) / 1e12 / 2500, 4),
                                       "kernel_ms": round(med, 3)}
     n_bytes = 1 << 30
     n_vec = n_bytes // 16
@@ -1309,6 +1311,8 @@ def main():
         line["ceilings_summary"] = {
             "TFLOP/s": {"mfma_loop_ones": pr["mfma_bf16_registers_ones"]["TFLOP/s"], "mfma_loop_random": pr["mfma_bf16_registers_random"]["TFLOP/s"],
                         "mfma_loop_random_lds_operands": pr["mfma_bf16_lds_operands_random"]["TFLOP/s"],
+                        "mfma_16x16x32_loop_random": pr.get("mfma_16x16x32_bf16_registers_random", {}).get("TFLOP/s"),
+                        "mfma_16x16x32_loop_random_lds_operands": pr.get("mfma_16x16x32_bf16_lds_operands_random", {}).get("TFLOP/s"),
                         "vendor_library_gemm_8192": round(ceilings["library_same_box"]["tflops"], 1),
                         "own_kernels_zero_operands_flushed|back_to_back": {n: [v["TFLOP/s"], v["back_to_back_TFLOP/s"]] for n, v in ceilings["same_kernel_zero_operands"].items()}},
             "GB/s": {"read": pr["hbm_read"]["GB/s"], "write": pr["hbm_write"]["GB/s"], "copy": pr["hbm_copy"]["GB/s"]}}

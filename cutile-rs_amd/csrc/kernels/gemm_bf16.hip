@@ -859,14 +859,14 @@ struct GemmRing16 {
         for (int v = 0; v < 4; ++v) acc[tn][tm][v] = 0.0f;
 
     // One MFMA block: rows [mh * TMH * 16, ..) of the sub-tile times all its columns, on the x fragments `a` and the
-    // y fragments `ub`, row block by row block.  Dealt out between its MFMAs, at most two per MFMA and in this
+    // y fragments `ub`, row block by row block.  Dealt out between its MFMAs in this
     // order: refill instructions first..last of the x stage `fill_x` (if any) and of the y stage `fill_y`
     // (instructions fb0..fb1-1), then, if rd_y, the reads of the next K step's y fragments into `ib`.  The x
     // fragments are one set: as soon as the last MFMA on a row block has issued, its fragment is read again for the
     // next block (rd_x, rd_ks, rd_mh) — three row blocks of MFMAs before it is used.  A wavefront issues in order
     // and an MFMA holds the issue slot until the matrix pipe takes it, so memory work placed after a run of MFMAs
     // would start late; sched_barrier(0) after every step keeps the order written here.
-    constexpr int SLOTS = NB / 2 > 0 ? NB / 2 : 1;
+    constexpr int SLOTS = NB;   // memory instructions spread over all the block's MFMAs: one per MFMA at most (measured +3 % over the first half only)
     // (what a block does besides its MFMAs is said by the flags with_y / with_fill_x and the range fb0..fb1: a null
     // test of an LDS pointer is a run-time test, address 0 being a valid one)
     auto block = [&](bf16x8 (&a)[TMH], const bf16x8 (&ub)[TN], int mh, const unsigned char* rd_x, int rd_ks, int rd_mh,

@@ -12,6 +12,8 @@
 //                      The gap between the two is the power cap at work.
 //   probe_mfma_bf16_lds  the same loop with the GEMM kernel's operand traffic: six
 //                      16-byte LDS fragment reads per eight MFMAs.
+//   probe_mfma16_bf16 / probe_mfma16_bf16_lds   the two loops on v_mfma_f32_16x16x32_bf16
+//                      (64 MFMAs, twice the flops, per iteration).
 //   probe_stream_read / _write / _copy   16-byte nontemporal accesses over a
 //                      buffer, the access pattern of the row kernels.
 #include <hip/hip_runtime.h>
@@ -91,9 +93,79 @@ __device__ __forceinline__ void mfma_loop(float* sink, int32_t iters, int32_t mo
   sink[(size_t)blockIdx.x * blockDim.x + tid] = s;
 }
 
+// The same two loops on v_mfma_f32_16x16x32_bf16: per iteration 64 MFMAs on a 8 x 4 grid of 16 x 16 accumulator
+// blocks (two 32-wide K steps; twice the flops of an iteration of the loops above), with the GemmRing16 kernel's operand traffic in the LDS
+// form (eight 16-byte x fragment reads and four y fragment reads per 32 MFMAs).  Per flop this form writes half as
+// many accumulator values, and on random operands that shows at the power limit.
+template <bool USE_LDS>
+__device__ __forceinline__ void mfma16_loop(float* sink, int32_t iters, int32_t mode) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int TM = 8, TN = 4;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[USE_LDS ? 65536 : 16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (USE_LDS) {
+    for (int i = tid; i < 65536 / 4; i += blockDim.x)
+      ((uint32_t*)lds)[i] = mode ? random_bf16_pair(hash32(i + blockIdx.x * 7919u)) : 0x3f803f80u;
+    __syncthreads();
+  }
+  bf16x8 a[TM / 2], b[2][TN];
+  const int r = (wave & 3) * 32 + (lane & 15), u = (lane >> 4) ^ ((r >> 1) & 7);
+  const uint32_t addr = r * 128 + u * 16;
+#pragma unroll
+  for (int i = 0; i < TM / 2 + 2 * TN; ++i) {
+    u32x4 v;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      v[c] = mode ? random_bf16_pair(hash32((uint32_t)(blockIdx.x * blockDim.x + tid) * 64u + i * 4 + c)) : 0x3f803f80u;
+    if (i < TM / 2) a[i] = __builtin_bit_cast(bf16x8, v);
+    else b[(i - TM / 2) / TN][(i - TM / 2) % TN] = __builtin_bit_cast(bf16x8, v);
+  }
+  f32x4 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {       // one 32-wide K step: 32 MFMAs in two blocks of 16
+#pragma unroll
+      for (int mh = 0; mh < 2; ++mh) {
+        const uint32_t o = ((it * 4 + half * 2 + mh) & 3) * 512;
+        if (USE_LDS && mh == 1) {
+#pragma unroll
+          for (int i = 0; i < TN; ++i) b[half ^ 1][i] = *(const bf16x8*)(lds + addr + 32768 + i * 4096 + o);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int tm = 0; tm < TM / 2; ++tm) {
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[tn][mh * (TM / 2) + tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[half][tn], a[tm], acc[tn][mh * (TM / 2) + tm], 0, 0, 0);
+          if (USE_LDS) a[tm] = *(const bf16x8*)(lds + addr + tm * 4096 + o);   // the fragment of the next block
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) s += acc[i][j][v];
+  sink[(size_t)blockIdx.x * blockDim.x + tid] = s;
+}
 }  // namespace
-
-// flops per launch = gridDim.x * (blockDim.x / 64) * iters * 2 * 8 * (2 * 32 * 32 * 16)
+extern "C" __global__ void __launch_bounds__(512) probe_mfma16_bf16(float* sink, int32_t iters, int32_t mode) {
+  mfma16_loop<false>(sink, iters, mode);
+}
+extern "C" __global__ void __launch_bounds__(512) probe_mfma16_bf16_lds(float* sink, int32_t iters, int32_t mode) {
+  mfma16_loop<true>(sink, iters, mode);
+}
+// flops per launch = gridDim.x * (blockDim.x / 64) * iters * 2 * 8 * (2 * 32 * 32 * 16); twice that for the mfma16 probes
 extern "C" __global__ void __launch_bounds__(512) probe_mfma_bf16(float* sink, int32_t iters, int32_t mode) {
   mfma_loop<false>(sink, iters, mode);
 }
