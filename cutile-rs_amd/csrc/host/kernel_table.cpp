@@ -220,6 +220,11 @@ std::vector<KernelEntry> build_table() {
     }
 
   // ---- persistent GEMM over a mapped partition: the pipelined bodies in a stream-item loop ----
+  // first the ring on v_mfma_f32_16x16x32 (whole K tiles of 64 only; the launcher skips it otherwise)
+  for (const char* dt : {"bf16", "f16"}) {
+    std::string v = std::string(dt) + "_256x256x64_q2x4";
+    add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 2);
+  }
   // 2 x 4 wavefronts first at 256 x 256: the item loop around the tile body costs the 4 x 2 form ten spilled registers (-2 %)
   for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2}}) {
     std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);

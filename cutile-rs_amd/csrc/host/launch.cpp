@@ -2128,7 +2128,8 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
-      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn)
+      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn &&
+          (std::min(x->shape[1], y->shape[0]) % 64 == 0 || strstr(e.variant, "_q") == nullptr))   // the ring fetches whole K tiles
         acceptable.push_back(e.variant);
   acceptable.push_back(std::string(dt) + "_generic");
   Resolved res;

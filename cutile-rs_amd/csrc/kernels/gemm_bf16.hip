@@ -772,6 +772,26 @@ struct GemmRing16 {
 
   __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
                              int32_t k_total, const TileGrid& g, int32_t accumulate) {
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    run_tile(z, x, y, k_total, pm, pn, accumulate);
+  }
+
+  // gemm_persistent: workgroup b computes the tiles of stream items b, b + gridDim.x, ... of the mapped output
+  // partition from zero accumulators, in the XCD-contiguous order of GemmDirect::run_persistent.
+  __device__ static void run_persistent(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                        const MappedArg& m) {
+    for (uint32_t item = blockIdx.x; item < m.total; item += gridDim.x) {
+      const uint32_t pos = m.total % kNumXcd == 0 ? (item % kNumXcd) * (m.total / kNumXcd) + item / kNumXcd : item;
+      uint32_t bid[3];
+      mapped_index(m, pos, bid);
+      run_tile(z, x, y, x.shape[1], bid[0], bid[1], 0);
+      __syncthreads();   // the output bands live in the stages that the next tile refills
+    }
+  }
+
+  __device__ static __forceinline__ void run_tile(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                                  int32_t k_total, uint32_t pm, uint32_t pn, int32_t accumulate) {
     // Separately named stages: the compiler can then tell a refill of one from
     // operand reads of another and adds no waits of its own.
     __shared__ __attribute__((aligned(1024))) unsigned char xs0[kABytes];
@@ -784,8 +804,6 @@ struct GemmRing16 {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    uint32_t pm, pn;
-    tile_coords(g.x, g.y, &pm, &pn);
     const int32_t M = x.shape[0], N = y.shape[1];
     const int32_t lda = x.strides[0], ldb = y.strides[0];
     const int32_t row0 = pm * BM, col0 = pn * BN;
@@ -1197,6 +1215,13 @@ GEMM_RING_KERNEL_F16(f16_256x256x64_r4x2, 256, 256, 4, 2)
   }
 GEMM_RING16_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16, __bf16)
 GEMM_RING16_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16, _Float16)
+#define GEMM_RING16_PERSISTENT_KERNEL(NAME, BM, BN, WVM, WVN, T)                                 \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_persistent_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
+    GemmRing16<BM, BN, WVM, WVN, T, T>::run_persistent(z, x, y, m);                             \
+  }
+GEMM_RING16_PERSISTENT_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16)
+GEMM_RING16_PERSISTENT_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16)
 
 #define GEMM_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                                \
   extern "C" __global__ void __launch_bounds__(256)                                            \

@@ -395,7 +395,7 @@ def test_decode_mapped_and_fp4_launchers_on_the_recording_runtime(fake_hip):
     a, b = torch.zeros(1024, 256, dtype=torch.bfloat16), torch.zeros(256, 768, dtype=torch.bfloat16)
     ct.gemm_persistent(ct.mapped(ct.partition(z, [256, 256]), [2, 1], 5), a, b)
     rec, args = _last(ct)
-    assert rec.symbol == b"gemm_persistent_entry__bf16_256x256x64_d2x4" and tuple(rec.grid) == (5, 1, 1) and tuple(rec.block) == (512, 1, 1)
+    assert rec.symbol == b"gemm_persistent_entry__bf16_256x256x64_q2x4" and tuple(rec.grid) == (5, 1, 1) and tuple(rec.block) == (512, 1, 1)
     assert struct.unpack_from("<4i4I", args, 88) == (2, 1, 1, 2, 4, 3, 1, 12)      # map, rank, logical grid, stream items
     # NVFP4: the reference example's 16x16 tiles run on the 32x32 kernel when the launch covers the tensor
     x4, s4 = torch.zeros(16, 64, dtype=torch.uint8), torch.zeros(16, 8, dtype=torch.uint8)

@@ -313,6 +313,8 @@ def test_gpu_persistent_gemm_reference_example(ct, dev):
 @pytest.mark.parametrize("m,n,k,tile,mp,ntb,variant", [
     (1024, 1024, 512, 256, (8, 1), 16, None),                   # full grid: one item per tile block
     (1024, 768, 256, 256, (2, 1), 5, "bf16_256x256x64_d2x4"),   # a non-divisor number of tile blocks
+    (1024, 768, 256, 256, (2, 1), 5, "bf16_256x256x64_q2x4"),   # the same on the 16 x 16 x 32 ring (whole K tiles of 64)
+    (1000, 520, 192, 256, (3, 2), 1, "bf16_256x256x64_q2x4"),   # ragged edges, one tile block walks everything
     (1000, 520, 200, 256, (3, 2), 1, None),                     # ragged edges, K tail, one tile block walks everything
     (640, 384, 128, 128, (4, 1), 7, None),
     (300, 200, 96, 64, (2, 2), 6, None),                        # no matrix-core variant for 64x64 tiles: any-layout kernel
