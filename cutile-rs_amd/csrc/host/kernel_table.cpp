@@ -190,7 +190,7 @@ std::vector<KernelEntry> build_table() {
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 2);
 
   // batched GEMM (cutile-examples/examples/batch_matmul.rs): the pipelined bodies with the batch on a grid axis
-  for (const char* kind : {"q", "r"})          // rings of three a stages and two b stages (q: on v_mfma_f32_16x16x32); whole K tiles only
+  for (const char* kind : {"q", "r"})          // rings of three a stages and two b stages (q: on v_mfma_f32_16x16x32, any K; r: whole K tiles only)
     for (const char* dt : {"bf16", "f16"}) {
       std::string v = std::string(dt) + "_256x256x64_" + kind + "2x4";
       add("batch_matmul", keep(v), keep("batch_matmul_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 3);
@@ -220,7 +220,7 @@ std::vector<KernelEntry> build_table() {
     }
 
   // ---- persistent GEMM over a mapped partition: the pipelined bodies in a stream-item loop ----
-  // first the ring on v_mfma_f32_16x16x32 (whole K tiles of 64 only; the launcher skips it otherwise)
+  // first the ring on v_mfma_f32_16x16x32
   for (const char* dt : {"bf16", "f16"}) {
     std::string v = std::string(dt) + "_256x256x64_q2x4";
     add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 2);
@@ -231,6 +231,9 @@ std::vector<KernelEntry> build_table() {
     add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, (uint32_t)(t[2] * t[3] * 64),
         (uint32_t)(2 * (t[0] * 64 + 64 * t[1]) * 2), t[0], t[1], 64, 0, "bf16", 0, 2);
   }
+  // grouped GEMM over descriptor tables: first the ring on v_mfma_f32_16x16x32 (it masks a ragged last K tile itself)
+  add("group_gemm_nt_desc", "f16_256x256x64_q2x4", "group_gemm_nt_desc_entry__f16_256x256x64_q2x4", IMG_GEMM, 512,
+      (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, "f16", 0, 2);
   // f16: persistent and grouped (descriptor-table) forms of the pipelined bodies
   for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2}}) {
     std::string v = "f16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);

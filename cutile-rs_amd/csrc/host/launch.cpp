@@ -1873,13 +1873,13 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
                            k_total % 8 == 0 && extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit &&
                            extent_bytes_2d(zt) < kDescriptorLimit;   // larger operands: the any-layout kernel (64-bit addresses)
   const std::string dt = in_f32 ? "f32" : in_f16 ? "f16" : zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
-  // The ring-pipelined variants ("_r", "_q") fetch whole K tiles only.
+  // The ring-pipelined variants on 32 x 32 x 16 ("_r") fetch whole K tiles only ("_q" masks a ragged last tile).
   const int32_t k_valid = std::min(std::min(x->shape[1], y->shape[0]), k_total);
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
       if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
-          (k_valid % 64 == 0 || (strstr(e.variant, "_r") == nullptr && strstr(e.variant, "_q") == nullptr)))
+          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
         acceptable.push_back(e.variant);
   acceptable.push_back(dt + "_generic");
   Resolved res;
@@ -1942,7 +1942,7 @@ cutile_status_t cutile_launch_batch_matmul(cutile_stream_t stream, const cutile_
   if (fast_layout)
     for (const auto& e : kernel_table())
       if (strcmp(e.function, "batch_matmul") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
-          (k_valid % 64 == 0 || (strstr(e.variant, "_r") == nullptr && strstr(e.variant, "_q") == nullptr)))
+          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
         acceptable.push_back(e.variant);
   acceptable.push_back(dt + "_generic");
   Resolved res;
@@ -2128,8 +2128,7 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
-      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn &&
-          (std::min(x->shape[1], y->shape[0]) % 64 == 0 || strstr(e.variant, "_q") == nullptr))   // the ring fetches whole K tiles
+      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn)
         acceptable.push_back(e.variant);
   acceptable.push_back(std::string(dt) + "_generic");
   Resolved res;

@@ -307,8 +307,7 @@ struct Fmha {
           pf[sb * 2 + hh] = __builtin_bit_cast(vec8, w);
         }
       }
-      rs = sum_across_halves(rs);
-      if (moved) {
+      if (moved) {   // (l_i and rs are this half's share of the row sum; the halves are added after the last tile)
         const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
         l_i *= alpha;
 #pragma unroll
@@ -343,7 +342,7 @@ struct Fmha {
     // out[bh, q, d] = acc / l.  o_acc[db][e]: d = db*32 + (e/4)*8 + half*4 + e%4.
     // A row that saw no key at all (an empty key range) has l = 0 and becomes 0, as in the
     // production kernels (l_safe = max(l, 1e-8), cutile-kernels/src/attention.rs:383-386); any other row has l >= 1.
-    l_i = fmaxf(l_i, 1.0e-8f);
+    l_i = fmaxf(sum_across_halves(l_i), 1.0e-8f);
     const int32_t qr = q0 + l32;
     if (qr < out.shape[1] && qr < q_len) {
       T* orow = (T*)out.ptr + (int64_t)bh * out.strides[0] + (int64_t)qr * out.strides[1];
@@ -619,8 +618,8 @@ struct FmhaPingPong {
           pf[sb * 2 + hh] = __builtin_bit_cast(vec8, w);
         }
       }
-      rs = sum_across_halves(rs);
-      l_i += rs;
+      l_i += rs;   // this half's share of the row sum: every rescaling multiplies both halves' shares by the same
+                   // alpha, so the halves are added once, after the last tile
     };
     auto interval_end = [&]() {
       __builtin_amdgcn_sched_barrier(0);
@@ -685,6 +684,7 @@ struct FmhaPingPong {
     // out[bh, q, d] = acc / l through LDS: this wavefront's 32 rows x D as T, 16-byte
     // chunk c of row r at chunk c ^ (r & 15); then whole rows leave as 16-byte stores.
     unsigned char* band = (wave < 2 ? kb0 : wave < 4 ? kb1 : wave < 6 ? vb0 : vb1) + (wave & 1) * (32 * D * 2);
+    l_i = sum_across_halves(l_i);
     const float inv_l = 1.0f / fmaxf(l_i, 1.0e-8f);   // l = 0 only for an empty key range: the row becomes 0
 #pragma unroll
     for (int db = 0; db < DB; ++db)

@@ -814,12 +814,18 @@ struct GemmRing16 {
 
     // Global side of the fetches (per lane, K tile 0; the K advance is scalar).
     // y instruction i of this wavefront covers K rows of half i / (kBInstr/2).
+    // A lane fetches K positions k0 + 8 u .. + 7 of an x row and K row k0 + r of y: past the end of K (a ragged last
+    // tile, or a trailing fetch beyond the last one) its offset is out of range and the fetch brings zeros.  K is a
+    // multiple of 8, so a 16-byte unit is wholly inside K or wholly beyond it.
     uint32_t a_goff[kAInstr], b_goff[kBInstr];
+    int32_t a_klim[kAInstr];      // k0 < a_klim[i]  <=>  the lane's unit of instruction i lies inside K
+    const int32_t b_klim = k_valid - (int32_t)(lane / UB);   // k0 + (first row of the instruction) < b_klim  <=>  the lane's row does
 #pragma unroll
     for (int i = 0; i < kAInstr; ++i) {
       const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
       const int u = (lane & 7) ^ ((r >> 1) & 7);
       a_goff[i] = (row0 + r < M) ? (uint32_t)(((int64_t)(row0 + r) * lda + u * 8) * 2) : kOob;
+      a_klim[i] = k_valid - u * 8;
     }
 #pragma unroll
     for (int i = 0; i < kBInstr; ++i) {
@@ -827,17 +833,15 @@ struct GemmRing16 {
       const int u = (lane % UB) ^ b_swizzle(r);
       b_goff[i] = (col0 + u * 8 < N) ? (uint32_t)(((int64_t)r * ldb + col0 + u * 8) * 2) : kOob;
     }
-    // K is a whole number of tiles here (the launcher sends ragged K to the
-    // two-stage variant), so a tile is either wholly inside K or wholly beyond it;
-    // beyond it every lane's offset is out of range and the fetch reads zeros.
     auto fetch_a = [&](unsigned char* stage, int32_t k0, int i) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16,
-                                               k0 < k_valid ? a_goff[i] : kOob, k0 * 2, 0, 0);
+                                               k0 < a_klim[i] ? a_goff[i] : kOob, k0 * 2, 0, 0);
     };
     // `half` = the y half-stage receiving K rows 32*h..32*h+31, h = i / (kBInstr/2)
     auto fetch_b = [&](unsigned char* half, int32_t k0, int i) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(half + ((i % (kBInstr / 2)) * kWaves + wave) * 1024),
-                                               16, k0 < k_valid ? b_goff[i] : kOob, k0 * ldb * 2, 0, 0);
+                                               16, k0 + (i * kWaves + wave) * kBRowsPerInstr < b_klim ? b_goff[i] : kOob,
+                                               k0 * ldb * 2, 0, 0);
     };
 
     // LDS side of the operand reads (byte offsets inside a stage).  v_mfma_f32_16x16x32: a lane holds 8 consecutive K
@@ -1137,11 +1141,10 @@ GEMM_DIRECT_F16_KERNEL(f16_128x128x64_d2x2, 128, 128, 2, 2)
 // one sequence, group after group and row-major inside a group, and workgroup w computes tiles w, w + grid, ...
 // (:82-83, 106-124).  The descriptors are read from device memory by every workgroup; as in the reference they are
 // trusted: pointers 16-byte aligned, rows and columns multiples of 16, row strides multiples of 8 (:24, 47-55).
-template <int BM, int BN, int WVM, int WVN>
+template <typename G, int BM, int BN>
 __device__ __forceinline__ void group_gemm_desc(const TensorArg<1>& a_ptrs, const TensorArg<1>& b_ptrs, const TensorArg<1>& c_ptrs,
                                                 const TensorArg<2>& a_metas, const TensorArg<2>& b_metas,
                                                 const TensorArg<2>& c_metas, int32_t num_groups) {
-  using G = GemmDirect<BM, BN, WVM, WVN, _Float16, _Float16>;
   auto uniform = [](int32_t v) { return __builtin_amdgcn_readfirstlane(v); };
   auto describe = [&](const TensorArg<1>& ptrs, const TensorArg<2>& metas, int32_t g, TensorArg<2>* t) {
     const uint32_t* pp = reinterpret_cast<const uint32_t*>((const int64_t*)ptrs.ptr + (int64_t)g * ptrs.strides[0]);
@@ -1182,7 +1185,7 @@ __device__ __forceinline__ void group_gemm_desc(const TensorArg<1>& a_ptrs, cons
   extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
       group_gemm_nt_desc_entry__##NAME(TensorArg<1> a_ptrs, TensorArg<1> b_ptrs, TensorArg<1> c_ptrs, TensorArg<2> a_metas, \
                                        TensorArg<2> b_metas, TensorArg<2> c_metas, int32_t num_groups) { \
-    group_gemm_desc<BM, BN, WVM, WVN>(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups); \
+    group_gemm_desc<GemmDirect<BM, BN, WVM, WVN, _Float16, _Float16>, BM, BN>(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups); \
   }
 GROUP_GEMM_KERNEL(f16_256x256x64_d2x4, 256, 256, 2, 4)
 GROUP_GEMM_KERNEL(f16_128x128x64_d2x2, 128, 128, 2, 2)
@@ -1220,6 +1223,11 @@ GEMM_RING16_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16, _Float16)
       gemm_persistent_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
     GemmRing16<BM, BN, WVM, WVN, T, T>::run_persistent(z, x, y, m);                             \
   }
+extern "C" __global__ void __launch_bounds__(512)
+    group_gemm_nt_desc_entry__f16_256x256x64_q2x4(TensorArg<1> a_ptrs, TensorArg<1> b_ptrs, TensorArg<1> c_ptrs, TensorArg<2> a_metas,
+                                                  TensorArg<2> b_metas, TensorArg<2> c_metas, int32_t num_groups) {
+  group_gemm_desc<GemmRing16<256, 256, 2, 4, _Float16, _Float16>, 256, 256>(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups);
+}
 GEMM_RING16_PERSISTENT_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16)
 GEMM_RING16_PERSISTENT_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16)
 

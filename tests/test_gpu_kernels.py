@@ -315,6 +315,20 @@ def test_gemm_ring_pipeline_every_loop_shape(ct, dev, variant, k_tiles):
     np.testing.assert_allclose(z.float().cpu().numpy(), ref, rtol=1.6e-2, atol=2e-3)
 
 
+@pytest.mark.parametrize("k", [8, 40, 64, 72, 200, 328])
+def test_gemm_16x16x32_ring_masks_a_ragged_last_k_tile(ct, dev, k):
+    # K is any multiple of 8: the last K tile is partly (or, for K < 64, mostly) beyond K and reads zeros; y may also
+    # have fewer rows than K says
+    m, n = 300, 520
+    a, b = normal_bf16_bits((m, k), 341 + k, k ** -0.5), normal_bf16_bits((k, n), 342 + k, k ** -0.5)
+    z = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    ct.gemm(ct.partition(z, [256, 256]), to_dev_bf16(a, dev), to_dev_bf16(b, dev), k, accumulate=False, generics=["bf16", 256, 256, 8],
+            variant="bf16_256x256x64_q2x4")
+    sync()
+    ref = oracle.gemm_bf16(a, b, f32out=True)
+    np.testing.assert_allclose(z.float().cpu().numpy(), ref, rtol=1.6e-2, atol=2e-3)
+
+
 def test_gemm_ring_variant_rejects_ragged_k(ct, dev):
     m = n = 256
     k = 96

@@ -39,7 +39,7 @@ def test_group_gemm_launcher_takes_its_grid_from_num_sm(fake_hip):
     assert rec.symbol == b"group_gemm_nt_desc_entry__f16_128x128x64_d2x2" and tuple(rec.grid) == (96, 1, 1) and tuple(rec.block) == (256, 1, 1)
     ct.group_gemm_f16_nt_desc(ptrs, ptrs, ptrs, metas, metas, metas, 3, generics=[256, 256, 64], grid=(40, 1, 1))
     rec, _ = _last(ct)
-    assert rec.symbol == b"group_gemm_nt_desc_entry__f16_256x256x64_d2x4" and tuple(rec.grid) == (40, 1, 1) and tuple(rec.block) == (512, 1, 1)
+    assert rec.symbol == b"group_gemm_nt_desc_entry__f16_256x256x64_q2x4" and tuple(rec.grid) == (40, 1, 1) and tuple(rec.block) == (512, 1, 1)
     n0 = ct.lib().cutile_testing_launch_count()
     cases = [
         (lambda: ct.group_gemm_f16_nt_desc(ptrs, ptrs, ptrs, metas, metas, metas, 4), "Launch grid required"),
