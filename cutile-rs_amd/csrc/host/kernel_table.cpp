@@ -210,6 +210,12 @@ std::vector<KernelEntry> build_table() {
         (uint32_t)((64 * 17 + 16 * 65) * 4), 0, 0, 0, 0, dt, 0, 3);
 
   // ---- NVFP4 GEMM: operands expanded to f16 on the way into LDS; LDS = 2 stages x (BM + BN) rows of 128 bytes ----
+  // first (the default for 256 x 256 tiles) the forms on v_mfma_f32_16x16x32_f16 ("q"): +9 % at the power limit
+  for (auto t : {std::array<int, 2>{2, 4}, std::array<int, 2>{4, 2}})
+    for (const char* dt : {"f32", "bf16"}) {
+      std::string v = std::string(dt) + "_256x256x64_q" + std::to_string(t[0]) + "x" + std::to_string(t[1]);
+      add("linear_tile_nvfp4", keep(v), keep("linear_tile_nvfp4_entry__" + v), IMG_NVFP4, 512, (uint32_t)(2 * 512 * 128), 256, 256, 64, 0, dt, 0, 2);
+    }
   for (auto t : {std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{128, 128, 2, 2},
                  std::array<int, 4>{64, 64, 1, 1}, std::array<int, 4>{32, 32, 1, 1}})
     for (const char* dt : {"f32", "bf16"}) {
@@ -218,7 +224,6 @@ std::vector<KernelEntry> build_table() {
       add("linear_tile_nvfp4", keep(v), keep("linear_tile_nvfp4_entry__" + v), IMG_NVFP4, (uint32_t)(t[2] * t[3] * 64),
           (uint32_t)(2 * (t[0] + t[1]) * 128), t[0], t[1], 64, 0, dt, 0, 2);
     }
-
   // ---- persistent GEMM over a mapped partition: the pipelined bodies in a stream-item loop ----
   // first the ring on v_mfma_f32_16x16x32
   for (const char* dt : {"bf16", "f16"}) {

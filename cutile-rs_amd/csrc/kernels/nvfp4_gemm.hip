@@ -13,7 +13,8 @@
 // operands to f16 on their way into LDS and multiplies with v_mfma_f32_32x32x16_f16:
 // every partial product is exact in f32 and the result differs from the definition above
 // only by the order of the f32 additions.  HBM sees the packed operands (a quarter of the
-// bf16 GEMM's bytes); the matrix pipe runs at its 16-bit rate.
+// bf16 GEMM's bytes); the matrix pipe runs at its 16-bit rate.  The variants of record ("_q") use
+// v_mfma_f32_16x16x32_f16: 1241 against 1141 TFLOP/s at 8192^3 on random operands (see Nvfp4Gemm).
 //
 // Pipeline: register-staged.  For K tile kt+1 every lane fetches 16 bytes (32 values of
 // one row) of x and of y plus the two scale bytes that belong to them; while the MFMAs of
@@ -27,6 +28,8 @@
 // between individual MFMAs, hand-over before the last K step, fetches two tiles ahead) was built
 // and measured equal to this form (1138 vs 1127-1140 TFLOP/s at 8192^3), so the simple form stays.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "gemm_common.h"
 #include "kernel_args.h"
@@ -50,14 +53,19 @@ __device__ __forceinline__ u32x4 expand_fp4x8(uint32_t packed, _Float16 scale) {
   return out;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+// SHAPE16: v_mfma_f32_16x16x32_f16 instead of v_mfma_f32_32x32x16_f16 — half as many accumulator values written per
+// flop, which is worth a few per cent at the chip's power limit (see gemm_bf16.hip, GemmRing16).  Both operands are
+// K-contiguous rows here, so only the fragment addresses (row lane % 16, K group lane / 16 of a 32-wide step) and the
+// accumulator layout (a lane: row lane % 16, columns 4 (lane / 16) .. + 3 of each 16 x 16 block) change.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT, bool SHAPE16 = false>
 struct Nvfp4Gemm {
   static constexpr int BK = 64;                      // values per K tile: four scale blocks of 16
   static constexpr int kRowBytes = BK * 2;           // a stage row in f16: eight 16-byte units
   static constexpr int kWaves = WAVES_M * WAVES_N;
   static constexpr int kThreads = kWaves * 64;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int BLK = SHAPE16 ? 16 : 32;      // rows / columns of one accumulator block
+  static constexpr int TM = WM / BLK, TN = WN / BLK;
   // a piece = 32 values of one row = 16 packed bytes = two scale blocks; two pieces per row and K tile
   static constexpr int kAPieces = BM * 2 / kThreads, kBPieces = BN * 2 / kThreads;
   static constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
@@ -73,6 +81,7 @@ struct Nvfp4Gemm {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane & 31, khalf = lane >> 5;
+    const int l16 = lane & 15, grp = lane >> 4;
     uint32_t pm, pn;
     tile_coords(g.x, g.y, &pm, &pn);
     const int32_t M = x.shape[0], N = y.shape[0];
@@ -146,13 +155,16 @@ struct Nvfp4Gemm {
       for (int i = 0; i < kBPieces; ++i) expand_piece(sb, b_row[i], b_half[i], b_reg[i], b_sc[i]);
     };
 
-    f32x16 acc[TN][TM];
+    typedef float f32x4v __attribute__((ext_vector_type(4)));
+    using Acc = std::conditional_t<SHAPE16, f32x4v, f32x16>;
+    constexpr int kAccRegs = SHAPE16 ? 4 : 16;
+    Acc acc[TN][TM];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[tn][tm][v] = 0.0f;
+        for (int v = 0; v < kAccRegs; ++v) acc[tn][tm][v] = 0.0f;
 
     const int k_tiles = k_bytes / 32;
     if (k_tiles > 0) {
@@ -161,25 +173,31 @@ struct Nvfp4Gemm {
     }
     __syncthreads();
 
+    constexpr int kSteps = SHAPE16 ? 2 : 4;     // K steps of 32 or 16 values per tile
     for (int kt = 0; kt < k_tiles; ++kt) {
       const int cur = kt & 1;
       if (kt + 1 < k_tiles) load_global(kt + 1);
       const unsigned char* sa = lds + cur * kStageBytes;
       const unsigned char* sb = sa + kABytes;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
+      for (int ks = 0; ks < kSteps; ++ks) {
         f16x8 af[TM], bfr[TN];
+        const int frow = SHAPE16 ? l16 : l32, funit = SHAPE16 ? ks * 4 + grp : ks * 2 + khalf;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) af[tm] = *reinterpret_cast<const f16x8*>(sa + lds_off(wm * WM + tm * 32 + l32, ks * 2 + khalf));
+        for (int tm = 0; tm < TM; ++tm) af[tm] = *reinterpret_cast<const f16x8*>(sa + lds_off(wm * WM + tm * BLK + frow, funit));
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) bfr[tn] = *reinterpret_cast<const f16x8*>(sb + lds_off(wn * WN + tn * 32 + l32, ks * 2 + khalf));
+        for (int tn = 0; tn < TN; ++tn) bfr[tn] = *reinterpret_cast<const f16x8*>(sb + lds_off(wn * WN + tn * BLK + frow, funit));
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-          for (int tm = 0; tm < TM; ++tm)
-            acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0);
+          for (int tm = 0; tm < TM; ++tm) {
+            if constexpr (SHAPE16)
+              acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0);
+            else
+              acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfr[tn], af[tm], acc[tn][tm], 0, 0, 0);
+          }
         // the expansion of the next tile rides between the matrix instructions of the later K steps
-        if (ks == 1 && kt + 1 < k_tiles) store_lds(cur ^ 1);
+        if (ks == (SHAPE16 ? 0 : 1) && kt + 1 < k_tiles) store_lds(cur ^ 1);
       }
       __syncthreads();
     }
@@ -189,13 +207,14 @@ struct Nvfp4Gemm {
     const int32_t zM = z.shape[0], zN = z.shape[1];
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-      const int32_t r = row0 + wm * WM + tm * 32 + l32;
+      const int32_t r = row0 + wm * WM + tm * BLK + (SHAPE16 ? l16 : l32);
       if (r >= zM) continue;
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int32_t c = col0 + wn * WN + tn * 32 + q * 8 + khalf * 4;
+        for (int q = 0; q < (SHAPE16 ? 1 : 4); ++q) {
+          // the lane's 4 consecutive columns of this block: 8 q + 4 (lane / 32) of 32, or 4 (lane / 16) of 16
+          const int32_t c = col0 + wn * WN + tn * BLK + (SHAPE16 ? grp * 4 : q * 8 + khalf * 4);
           if (c >= zN) continue;
           OutT* dst = zp + (int64_t)r * ldz + c;
           float v0 = acc[tn][tm][q * 4 + 0] * alpha, v1 = acc[tn][tm][q * 4 + 1] * alpha;
@@ -224,6 +243,16 @@ struct Nvfp4Gemm {
     Nvfp4Gemm<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, xs, ys, alpha, g);                            \
   }
 
+#define NVFP4_KERNEL16(NAME, BM, BN, WVM, WVN, OUT_T)                                              \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                     \
+      linear_tile_nvfp4_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, TensorArg<2> xs, \
+                                      TensorArg<2> ys, float alpha, TileGrid g) {                  \
+    Nvfp4Gemm<BM, BN, WVM, WVN, OUT_T, true>::run(z, x, y, xs, ys, alpha, g);                      \
+  }
+NVFP4_KERNEL16(f32_256x256x64_q4x2, 256, 256, 4, 2, float)
+NVFP4_KERNEL16(f32_256x256x64_q2x4, 256, 256, 2, 4, float)
+NVFP4_KERNEL16(bf16_256x256x64_q4x2, 256, 256, 4, 2, __bf16)
+NVFP4_KERNEL16(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16)
 NVFP4_KERNEL(f32_256x256x64_w4x2, 256, 256, 4, 2, float)
 NVFP4_KERNEL(f32_256x256x64_w2x4, 256, 256, 2, 4, float)
 NVFP4_KERNEL(f32_128x128x64_w2x2, 128, 128, 2, 2, float)

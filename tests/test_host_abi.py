@@ -406,7 +406,7 @@ def test_decode_mapped_and_fp4_launchers_on_the_recording_runtime(fake_hip):
     zb = torch.zeros(512, 512)
     xb, sb = torch.zeros(512, 128, dtype=torch.uint8), torch.zeros(512, 16, dtype=torch.uint8)
     ct.linear_tile_nvfp4(ct.partition(zb, [256, 256]), xb, xb, sb, sb, 1.0)
-    assert _last(ct)[0].symbol == b"linear_tile_nvfp4_entry__f32_256x256x64_w4x2" and tuple(_last(ct)[0].grid) == (4, 1, 1)
+    assert _last(ct)[0].symbol == b"linear_tile_nvfp4_entry__f32_256x256x64_q2x4" and tuple(_last(ct)[0].grid) == (4, 1, 1)
 
     n0 = L.cutile_testing_launch_count()
     q3 = torch.zeros(8, 3, 128, dtype=h)

@@ -97,6 +97,10 @@ def test_gpu_nvfp4_reference_example(ct, dev):
     (256, 256, 256, 256, None, "f32"),
     (512, 768, 1024, 256, "f32_256x256x64_w4x2", "f32"),
     (512, 768, 1024, 256, "f32_256x256x64_w2x4", "f32"),
+    (512, 768, 1024, 256, "f32_256x256x64_q4x2", "f32"),      # the 16 x 16 x 32 forms
+    (1000, 264, 192, 256, "f32_256x256x64_q2x4", "f32"),
+    (300, 520, 64, 256, "bf16_256x256x64_q4x2", "bf16"),
+    (520, 264, 320, 256, "bf16_256x256x64_q2x4", "bf16"),
     (300, 520, 64, 256, "f32_256x256x64_w4x2", "f32"),       # one K tile
     (256, 256, 128, 256, "f32_256x256x64_w2x4", "f32"),      # two
     (1000, 264, 192, 256, "f32_256x256x64_w4x2", "f32"),     # three, ragged edges
