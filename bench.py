@@ -1117,6 +1117,16 @@ def probe_ceilings(ct, torch, flush):
             fl = flops * (2.0 if "16x16x32" in name else 1.0)     # 64 MFMAs of 16 x 16 x 32 per iteration: twice the flops of 16 of 32 x 32 x 16
             out[f"{name}_{label}"] = {"TFLOP/s": round(fl / (med * 1e-3) / 1e12, 1), "frac_of_2500": round(fl / (med * 1e-3) / 1e12 / 2500, 4),
                                       "kernel_ms": round(med, 3)}
+    # v_exp_f32 against a software exp2's multiply-adds (16 chains per lane and iteration, 2 wavefronts per SIMD,
+    # one workgroup per CU): nanoseconds per wavefront and chain
+    f = mod.function("probe_valu_exp2")
+    v_iters = 20000
+    valu = {}
+    for mode, label in ((0, "exp2_and_add"), (1, "seven_fma"), (2, "both_interleaved")):
+        med, mn = _timed(ct, torch, flush, lambda: ct.Module.launch(
+            f, (cus, 1, 1), (512, 1, 1), [C.c_void_p(sink.data_ptr()), C.c_int32(v_iters), C.c_int32(mode)]), reps=5, warm=1)
+        valu[label + "_ns"] = round(med * 1e6 / (2.0 * v_iters * 16), 2)
+    out["valu_exp2_vs_fma"] = valu
     n_bytes = 1 << 30
     n_vec = n_bytes // 16
     src = torch.empty(n_bytes // 4, dtype=torch.int32, device="cuda").fill_(0x3c003c00)

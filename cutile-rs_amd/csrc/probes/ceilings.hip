@@ -14,6 +14,7 @@
 //                      16-byte LDS fragment reads per eight MFMAs.
 //   probe_mfma16_bf16 / probe_mfma16_bf16_lds   the two loops on v_mfma_f32_16x16x32_bf16
 //                      (64 MFMAs, twice the flops, per iteration).
+//   probe_valu_exp2    v_exp_f32 against the multiply-adds of a software exp2, alone and interleaved
 //   probe_stream_read / _write / _copy   16-byte nontemporal accesses over a
 //                      buffer, the access pattern of the row kernels.
 #include <hip/hip_runtime.h>
@@ -164,6 +165,38 @@ extern "C" __global__ void __launch_bounds__(512) probe_mfma16_bf16(float* sink,
 }
 extern "C" __global__ void __launch_bounds__(512) probe_mfma16_bf16_lds(float* sink, int32_t iters, int32_t mode) {
   mfma16_loop<true>(sink, iters, mode);
+}
+// What an exponential costs the vector ALU next to multiply-adds: per iteration and lane 16 independent chains of
+// mode 0: v_exp_f32 and one add; mode 1: seven fused multiply-adds (a range reduction plus a cubic, the least a
+// software exp2 takes); mode 2: both interleaved.  Mode 2 taking the sum of modes 0 and 1 says the two share one
+// issue port; mode 1 taking longer than mode 0 says a polynomial does not relieve it.
+template <int MODE>
+__device__ __forceinline__ void valu_exp2_loop(float* sink, int32_t iters, float seed) {
+  float v[16], w[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    v[i] = seed + 0.001f * (float)(threadIdx.x + i);
+    w[i] = seed * 0.5f + (float)i;
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (MODE != 1) v[i] = __builtin_amdgcn_exp2f(v[i]) - 1.0f;
+      if (MODE != 0) {
+#pragma unroll
+        for (int f = 0; f < 7; ++f) w[i] = __builtin_fmaf(w[i], 0.999f, 0.001f);
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += v[i] + w[i];
+  sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+extern "C" __global__ void __launch_bounds__(512) probe_valu_exp2(float* sink, int32_t iters, int32_t mode) {
+  if (mode == 0) valu_exp2_loop<0>(sink, iters, 0.3f);
+  else if (mode == 1) valu_exp2_loop<1>(sink, iters, 0.3f);
+  else valu_exp2_loop<2>(sink, iters, 0.3f);
 }
 // flops per launch = gridDim.x * (blockDim.x / 64) * iters * 2 * 8 * (2 * 32 * 32 * 16); twice that for the mfma16 probes
 extern "C" __global__ void __launch_bounds__(512) probe_mfma_bf16(float* sink, int32_t iters, int32_t mode) {
