@@ -6,14 +6,17 @@
 A step is one launch of the hot-path kernel over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the bf16 GEMM at M = N = K = 8192
 (the configuration the target fractions are quoted on); every other benchmark
-configuration is measured the same way and reported under "also" in the same JSON line.
+configuration is measured the same way.  The run ends with ONE JSON line of at most 4 KB
+(headline record + every benchmark configuration in short form + the copy ceiling of the
+same run); the full records of all workloads go to gpurun_out/bench_full.json.
 
 Timing: W untimed launches, then exactly K launches between two device synchronisations
 (wall clock -> ms_per_step / value).  roofline.achieved follows the reference's do_bench
 protocol (cutile/src/bench.rs:124-211): per-launch HIP events on the launch stream, a
 512 MiB cache flush before every repetition, median reported (minimum, mean and the
-back-to-back average beside it).  The benchmark configurations are repeated in short
-form at the END of the JSON line ("baseline_configs", "ceilings").
+back-to-back average beside it; frac_back_to_back and frac_wall are the same work over
+the sustained figures).  --ceilings adds the bare-resource probes, the vendor library's
+GEMM, the kernels on zero operands and the launch-mode latencies.
 
 cpu_baseline: the CPU oracle (a port of the reference's naive CPU references), timed on
 this host's cores on a bounded sample of the same workload.  The sampled output is also
@@ -349,8 +352,13 @@ class Nvfp4Gemm(Workload):
     s = 8192
     work = 2.0 * s ** 3
     tile = 256
+    # Two roofs.  roofline.frac is against the f16 pipe this kernel computes on; frac_of_fp4_peak is the same rate
+    # against the fp4 pipe's 10.1 PFLOP/s.  The exact path needs f16: an e4m3 scale per 16 elements has a mantissa,
+    # the hardware block scale is a power of two per 32, and e2m1 x (1 + m/8) does not fit an fp8 operand.
+    other_roofs = {"mfma_fp4": 10100.0}
     config = {"workload": "NVFP4 block-scaled GEMM A[8192,8192] B[8192,8192] packed e2m1 + e4m3fn scale per 16 K, f32 out; "
-                          "matrix work runs on the f16 pipe (peak 2.5 PFLOP/s): CDNA4's fp4 pipe cannot take e4m3 scales per 16",
+                          "matrix work runs on the f16 pipe (peak 2.5 PFLOP/s; the fp4 pipe's 10.1 PFLOP/s is quoted beside it): "
+                          "CDNA4's fp4 pipe cannot take e4m3 scales per 16",
               "tile": "256x256x64"}
 
     def setup(self, ct, torch, oracle, dev):
@@ -970,14 +978,17 @@ class ExampleStream(Workload):
 
 
 def make_workloads():
+    """The default run: the benchmark configurations first, then the other kernels of the path."""
     return [Gemm(8192), Gemm(4096), GemmPersistent(8192), Fmha(False), Fmha(True), RmsNorm(), Softmax(), Saxpy(), MxGemm(), Nvfp4Gemm(),
-            Copy(), RmsNormAllF16(), SoftmaxAllF16(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv(),
-            BatchMatmul(), Matvec(), ExampleStream("relu"), ExampleStream("dropout"), ExampleStream("scale_ptr")]
+            Copy(), RmsNormAllF16(), SoftmaxAllF16(), AddRmsNorm(), SiluMul(), QkNorm(), Rope(), KvCacheUpdate(), DecodeAttention(), DecodeAttentionWide(), DecodeAttentionGrouped(), KvbmCopy(), PrefillAttention(), LmHeadArgmax(), EmbeddingBatch(), GroupGemm(), FusedQkNormRopeKv()]
 
 
-EXTRA_WORKLOADS = []  # only by name, never in the default run
+# the reference's small example programs: only by name (--workload), never in the default run
+def make_extra_workloads():
+    return [BatchMatmul(), Matvec(), ExampleStream("relu"), ExampleStream("dropout"), ExampleStream("scale_ptr")]
 
 
+WARMUP_BUDGET_S = 0.05       # untimed launches continue until this much time has passed (the reference's budget is 25 ms)
 FLUSH_BYTES = 512 << 20      # larger than the 256 MB memory-side cache and every L2
 
 
@@ -1004,6 +1015,15 @@ def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np, flush):
     for _ in range(warmup):
         w.launch()
     torch.cuda.synchronize()
+    # Warm-up by time budget on top of the W steps, as do_bench has it ("absorbs JIT and clock ramp",
+    # cutile/src/bench.rs:33-35,188-192): after tens of milliseconds without work this device needs about 30 ms of
+    # launches before they run at their steady rate (a launch of the 8192^3 GEMM takes 0.9-1.07 ms there, 0.77 ms after),
+    # and W = 5 launches of a 0.8 ms kernel end well inside that ramp.
+    t_w = time.perf_counter()
+    while time.perf_counter() - t_w < WARMUP_BUDGET_S:
+        for _ in range(4):
+            w.launch()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         w.launch()
@@ -1016,6 +1036,15 @@ def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np, flush):
     for _ in range(steps):
         dominant()
     back_to_back_ms = timer.stop() / steps
+    # the same sustained run once more with an event between every two launches: shows whether the launches of a
+    # back-to-back run slow down as the run goes on (clock management) or the first ones are slow (ramp from idle)
+    series = ct.EventSeries(steps)
+    series.mark()
+    for _ in range(steps):
+        dominant()
+        series.mark()
+    gaps = series.gaps_ms()
+    series.close()
     reps = max(10, min(steps, 40))
     times = []
     for _ in range(reps):
@@ -1035,10 +1064,16 @@ def measure(w, ct, torch, steps, warmup, with_cpu, oracle, np, flush):
         "roofline": {"bound": w.bound, "achieved": achieved, "peak": peak, "unit": punit, "frac": achieved / peak,
                      "traffic": _traffic(w.name), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)",
                      "kernel_ms": kernel_ms, "kernel_ms_min": times[0], "kernel_ms_mean": sum(times) / len(times),
-                     "kernel_ms_back_to_back": back_to_back_ms, "reps": reps,
+                     "kernel_ms_back_to_back": back_to_back_ms, "frac_back_to_back": w.work / (back_to_back_ms * 1e-3) / scale / peak,
+                     "frac_wall": w.work / (wall_ms * 1e-3) / scale / peak,
+                     "sustained_launch_ms": {"first": gaps[0], "median": _quantile(sorted(gaps), 0.5), "last": gaps[-1], "max": max(gaps)},
+                     "reps": reps,
                      "protocol": "median of per-launch HIP-event times, 512 MiB cache flush before each",
                      "algorithmic_work": w.work},
     }
+    for key, other_peak in getattr(w, "other_roofs", {}).items():      # the same rate against a second published peak
+        rec["roofline"]["frac_of_" + key.replace("mfma_", "") + "_peak"] = achieved / other_peak
+        rec["roofline"]["peak_" + key.replace("mfma_", "")] = other_peak
     try:      # which precompiled variant ran, and whether a tuning record, a pin or the table's order chose it
         got = ct.last_resolved()
         rec["kernel"] = {"variant": got["variant"], "chosen_by": got["source"], "shape_class": got["bucket"]}
@@ -1092,7 +1127,7 @@ def _timed(ct, torch, flush, launch, reps=15, warm=3):
 
 
 def probe_ceilings(ct, torch, flush):
-    """What this box sustains on the bare resources (cutile-rs_amd/csrc/probes/ceilings.hip, a code object of its own
+    """What this box sustains on the bare resources (cutile-rs_amd/bench/ceilings.hip, a code object of its own
     launched through the C ABI's module calls), under the same flush + event protocol as the workloads:
     nothing but bf16 MFMAs on register operands (ones: few bits toggle; random: the bit activity of real data), the
     same loop with the GEMM kernel's LDS operand traffic, and nontemporal read / write / copy streams of 1 GiB."""
@@ -1231,6 +1266,63 @@ def launch_modes():
 
 BASELINE_CONFIGS = ["gemm_bf16_8192", "gemm_bf16_4096", "fmha_bf16", "fmha_bf16_causal", "rms_norm_f16_16384x8192",
                     "softmax_f16_16384x8192", "saxpy_f32_16777216", "mxfp8_gemm_8192"]
+LINE_LIMIT = 4096            # bytes of the final stdout line; everything else goes to FULL_RECORD
+FULL_RECORD = os.path.join("gpurun_out", "bench_full.json")
+
+
+def _r(x, n=4):
+    return None if x is None else round(x, n)
+
+
+def compact_line(records, steps, warmup, device, ceilings=None):
+    """The one JSON line a run ends with: the headline workload's record (records[0]) with its roofline and CPU baseline,
+    every benchmark configuration in short form, and the ceilings this run measured.  At most LINE_LIMIT bytes: the
+    full records are written to a file, never into this line."""
+    h = records[0]
+    rf = h["roofline"]
+    line = {
+        "metric": METRIC, "value": _r(h["value"], 2), "unit": h["unit"], "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": _r(h["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "warmup_ms_budget": WARMUP_BUDGET_S * 1e3, "dtype": h["dtype"], "data": "synthetic (seeded host PRNG, same bytes fed to the CPU oracle)", "config": h["config"],
+        "roofline": {"bound": rf["bound"], "achieved": _r(rf["achieved"], 2), "peak": rf["peak"], "unit": rf["unit"],
+                     "frac": _r(rf["frac"]), "traffic": rf.get("traffic"), "kernel_ms": _r(rf["kernel_ms"], 5),
+                     "kernel_ms_back_to_back": _r(rf.get("kernel_ms_back_to_back"), 5),
+                     "frac_back_to_back": _r(rf.get("frac_back_to_back")), "frac_wall": _r(rf.get("frac_wall")),
+                     "protocol": "frac: median of per-launch HIP-event times, 512 MiB cache flush before each; "
+                                 "frac_back_to_back / frac_wall: K launches in a row (events / host clock)"},
+    }
+    for k in ("cpu_baseline", "parity", "kernel"):
+        if k in h:
+            line[k] = h[k]
+    line["device"] = device
+    by_name = {r["workload"]: r for r in records}
+    ceilings = ceilings or {}
+    copy_rate = ceilings.get("hbm_copy_GB/s")
+    short = {}
+    for n in BASELINE_CONFIGS:
+        if n not in by_name:
+            continue
+        r = by_name[n]["roofline"]
+        e = {"achieved": _r(r["achieved"], 1), "frac": _r(r["frac"]), "kernel_ms": _r(r["kernel_ms"]),
+             "kernel_ms_b2b": _r(r.get("kernel_ms_back_to_back")), "frac_b2b": _r(r.get("frac_back_to_back")),
+             "ms_per_step": _r(by_name[n]["ms_per_step"]), "frac_wall": _r(r.get("frac_wall")),
+             "parity_ok": all(v for k, v in by_name[n].get("parity", {}).items() if isinstance(v, bool))}
+        if r["bound"] == "hbm" and copy_rate:
+            e["frac_of_copy_ceiling"] = _r(r["achieved"] / copy_rate)
+        short[n] = e
+    line["baseline_configs"] = short
+    if ceilings:
+        line["ceilings_summary"] = ceilings
+    line["full_record"] = FULL_RECORD
+    text = json.dumps(line, separators=(",", ":"))
+    for drop in ("full_record", "kernel", "parity", "ceilings_summary"):      # never reached with real records; a guard, not a plan
+        if len(text) <= LINE_LIMIT:
+            break
+        line.pop(drop, None)
+        text = json.dumps(line, separators=(",", ":"))
+    if len(text) > LINE_LIMIT:
+        raise RuntimeError(f"bench line is {len(text)} bytes, over the {LINE_LIMIT}-byte limit")
+    return text
 
 
 def main():
@@ -1239,9 +1331,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gemm_bf16_8192")
-    ap.add_argument("--only", action="store_true", help="measure only --workload (no 'also' list)")
+    ap.add_argument("--only", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / sampled parity leg")
-    ap.add_argument("--ceilings", action="store_true", help="with --only: also run the ceiling probes and the vendor-library GEMM")
+    ap.add_argument("--ceilings", action="store_true", help="also run the ceiling probes (cutile-rs_amd/bench/ceilings.hip), the vendor-library GEMM, "
+                                                            "the kernels on zero operands and the launch-mode latencies")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel here is a one-GPU tile kernel; "
@@ -1262,10 +1355,10 @@ def main():
     workloads = make_workloads()
     head = next((w for w in workloads if w.name == args.workload), None)
     if head is None:
-        head = next((c() for c in EXTRA_WORKLOADS if c.name == args.workload), None)
+        head = next((w for w in make_extra_workloads() if w.name == args.workload), None)
         args.only = args.only or head is not None
     if head is None:
-        sys.exit(f"unknown workload {args.workload}; choose from {[w.name for w in workloads]}")
+        sys.exit(f"unknown workload {args.workload}; choose from {[w.name for w in workloads + make_extra_workloads()]}")
     order = [head] + ([] if args.only else [w for w in workloads if w is not head])
     flush = torch.empty(FLUSH_BYTES // 4, dtype=torch.int32, device=dev)
     records = []
@@ -1278,55 +1371,35 @@ def main():
             if hasattr(w.__dict__[k], "is_cuda"):
                 del w.__dict__[k]
         torch.cuda.empty_cache()
-    h = records[0]
-    line = {
-        "metric": METRIC, "value": h["value"], "unit": h["unit"], "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": h["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": h["dtype"], "data": "synthetic (seeded host PRNG, same bytes fed to the CPU oracle)",
-        "config": h["config"], "roofline": h["roofline"],
-        "device": ct.device_arch(0),
-        "tuning_records": ct.tuning_report().strip().splitlines(),
-    }
-    if "kernel" in h:
-        line["kernel"] = h["kernel"]
-    if "cpu_baseline" in h:
-        line["cpu_baseline"] = h["cpu_baseline"]
-        line["parity"] = h["parity"]
-    if len(records) > 1:
-        line["also"] = records[1:]
     by_name = {r["workload"]: r for r in records}
-    ceilings = {}
-    if "copy_f32_67108864" in by_name:
+    full = {"records": records, "tuning_records": ct.tuning_report().strip().splitlines()}
+    summary = {}
+    if "copy_f32_67108864" in by_name:      # the library's own convert kernel as a plain copy: what one read + one write reaches here
         c = by_name["copy_f32_67108864"]["roofline"]
-        ceilings["hbm_copy_stream"] = {"what": "plain copy of 2^26 f32 through the library's convert kernel (one read + one write)",
-                                       "GB/s": round(c["achieved"], 1), "frac_of_8000": round(c["frac"], 4)}
-    if not args.only or args.ceilings:
-        ceilings["library_same_box"] = library_same_box(torch, flush)
-        ceilings["probes"] = probe_ceilings(ct, torch, flush)
-        ceilings["same_kernel_zero_operands"] = same_kernel_zero_operands(ct, torch, flush)
-    if ceilings:
-        line["ceilings"] = ceilings
-    if not args.only or args.ceilings:
-        line["launch_modes"] = launch_modes()
-    # Short summaries LAST (about 1.2 kB), so that a reader who keeps only the end of the line still has every benchmark
-    # configuration (value and fraction of peak from the flushed median, wall-clock step beside it) and the ceilings
-    # this box showed in the same run.
-    line["baseline_configs"] = {
-        n: {"achieved": round(by_name[n]["roofline"]["achieved"], 1), "frac": round(by_name[n]["roofline"]["frac"], 4),
-            "kernel_ms": round(by_name[n]["roofline"]["kernel_ms"], 4), "ms_per_step": round(by_name[n]["ms_per_step"], 4),
-            "parity_ok": all(v for k, v in by_name[n].get("parity", {}).items() if isinstance(v, bool))}
-        for n in BASELINE_CONFIGS if n in by_name}
-    pr = ceilings.get("probes", {})
-    if "mfma_bf16_registers_random" in pr:
-        line["ceilings_summary"] = {
-            "TFLOP/s": {"mfma_loop_ones": pr["mfma_bf16_registers_ones"]["TFLOP/s"], "mfma_loop_random": pr["mfma_bf16_registers_random"]["TFLOP/s"],
-                        "mfma_loop_random_lds_operands": pr["mfma_bf16_lds_operands_random"]["TFLOP/s"],
-                        "mfma_16x16x32_loop_random": pr.get("mfma_16x16x32_bf16_registers_random", {}).get("TFLOP/s"),
-                        "mfma_16x16x32_loop_random_lds_operands": pr.get("mfma_16x16x32_bf16_lds_operands_random", {}).get("TFLOP/s"),
-                        "vendor_library_gemm_8192": round(ceilings["library_same_box"]["tflops"], 1),
-                        "own_kernels_zero_operands_flushed|back_to_back": {n: [v["TFLOP/s"], v["back_to_back_TFLOP/s"]] for n, v in ceilings["same_kernel_zero_operands"].items()}},
-            "GB/s": {"read": pr["hbm_read"]["GB/s"], "write": pr["hbm_write"]["GB/s"], "copy": pr["hbm_copy"]["GB/s"]}}
-    print(json.dumps(line))
+        summary["hbm_copy_GB/s"] = round(c["achieved"], 1)
+        summary["hbm_copy_frac_of_8000"] = round(c["frac"], 4)
+        summary["hbm_copy_what"] = "library convert kernel f32->f32, 2^26 elements, same flush + event protocol"
+    if args.ceilings:
+        full["library_same_box"] = library_same_box(torch, flush)
+        pr = full["probes"] = probe_ceilings(ct, torch, flush)
+        full["same_kernel_zero_operands"] = same_kernel_zero_operands(ct, torch, flush)
+        full["launch_modes"] = launch_modes()
+        if "mfma_bf16_registers_random" in pr:
+            summary["probe_TFLOP/s"] = {
+                "mfma_loop_ones": pr["mfma_bf16_registers_ones"]["TFLOP/s"], "mfma_loop_random": pr["mfma_bf16_registers_random"]["TFLOP/s"],
+                "mfma_16x16x32_random_lds_operands": pr.get("mfma_16x16x32_bf16_lds_operands_random", {}).get("TFLOP/s"),
+                "vendor_library_gemm_8192": round(full["library_same_box"]["tflops"], 1),
+                "own_kernels_zero_operands_flushed|b2b": {n: [v["TFLOP/s"], v["back_to_back_TFLOP/s"]] for n, v in full["same_kernel_zero_operands"].items()}}
+            summary["probe_GB/s"] = {"read": pr["hbm_read"]["GB/s"], "write": pr["hbm_write"]["GB/s"], "copy": pr["hbm_copy"]["GB/s"]}
+    text = compact_line(records, args.steps, args.warmup, ct.device_arch(0), summary)
+    full["line"] = json.loads(text)
+    try:
+        os.makedirs(os.path.dirname(FULL_RECORD), exist_ok=True)
+        with open(FULL_RECORD, "w") as f:
+            json.dump(full, f, indent=1)
+    except OSError as e:
+        sys.stderr.write(f"bench.py: could not write {FULL_RECORD}: {e}\n")
+    print(text, flush=True)
 
 
 if __name__ == "__main__":

@@ -1032,3 +1032,35 @@ class EventTimer:
     def close(self):
         lib().cutile_event_destroy(self.start_ev)
         lib().cutile_event_destroy(self.stop_ev)
+
+
+class EventSeries:
+    """n + 1 HIP events on one stream, recorded between n back-to-back launches: the duration of every launch of a
+    sustained run without a host synchronisation in between (the events are read after the last one completes)."""
+
+    def __init__(self, n: int, stream=None):
+        self.stream = _stream(stream)
+        self.events = []
+        for _ in range(n + 1):
+            ev = C.c_void_p()
+            check(lib().cutile_event_create(C.byref(ev)))
+            self.events.append(ev)
+        self.k = 0
+
+    def mark(self):
+        check(lib().cutile_event_record(self.events[self.k], self.stream))
+        self.k += 1
+
+    def gaps_ms(self) -> list:
+        check(lib().cutile_event_synchronize(self.events[self.k - 1]))
+        out = []
+        for a, b in zip(self.events[: self.k - 1], self.events[1: self.k]):
+            ms = C.c_float()
+            check(lib().cutile_event_elapsed_ms(a, b, C.byref(ms)))
+            out.append(ms.value)
+        return out
+
+    def close(self):
+        for ev in self.events:
+            lib().cutile_event_destroy(ev)
+        self.events = []

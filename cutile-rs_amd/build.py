@@ -132,9 +132,9 @@ PROBES_PATH = os.path.join(LIB_DIR, "probes.hsaco")
 
 
 def build_probes(force: bool = False) -> str:
-    """Ceiling probes for bench.py (bare MFMA loop, streaming reads / writes / copies): a code object of their own,
+    """Ceiling probes for `bench.py --ceilings` (bare MFMA loop, streaming reads / writes / copies): a code object of their own,
     not embedded in the host library."""
-    src = os.path.join(ROOT, "csrc", "probes", "ceilings.hip")
+    src = os.path.join(ROOT, "bench", "ceilings.hip")
     if force or not _newer(PROBES_PATH, [src]):
         _run([HIPCC] + DEVICE_FLAGS + ["-o", PROBES_PATH, src])
     return PROBES_PATH
