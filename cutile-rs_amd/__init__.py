@@ -137,6 +137,7 @@ def lib() -> C.CDLL:
             "cutile_launch_splitk_reduce_merge": [vp, P(TensorArg), P(TensorArg), P(PartitionArg), P(LaunchOpts)],
             "cutile_launch_fmha_decode_gqa_noalloc": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), f32,
                                                       P(TensorArg), i32, i32],
+            "cutile_fmha_decode_gqa_noalloc_prepare": [P(TensorArg), P(TensorArg), P(TensorArg), P(PartitionArg), P(TensorArg), i32, i32],
             "cutile_scratch_capacity": [P(C.c_size_t)],
             "cutile_launch_rope_f16": [vp, P(TensorArg), P(TensorArg), P(TensorArg), P(TensorArg), i32, P(PartitionArg),
                                        i32, P(LaunchOpts)],
@@ -574,6 +575,14 @@ def fmha_decode_gqa_noalloc(q, k, v, out: Partition, qk_scale: float, position_s
     check(lib().cutile_launch_fmha_decode_gqa_noalloc(_stream(stream), C.byref(qa), C.byref(ka), C.byref(va),
                                                       C.byref(out.arg()), C.c_float(qk_scale), C.byref(pa),
                                                       int(num_kv_splits), int(bn)))
+
+
+def fmha_decode_gqa_noalloc_prepare(q, k, v, out: Partition, position_start, num_kv_splits: int, bn: int = 64) -> None:
+    """the once-per-device-and-shape work of fmha_decode_gqa_noalloc (side library, scratch address, code objects) done
+    ahead of time, outside any stream capture; nothing is enqueued"""
+    qa, ka, va, pa = tensor_arg(q), tensor_arg(k), tensor_arg(v), tensor_arg(position_start, dtype=U32)
+    check(lib().cutile_fmha_decode_gqa_noalloc_prepare(C.byref(qa), C.byref(ka), C.byref(va), C.byref(out.arg()), C.byref(pa),
+                                                       int(num_kv_splits), int(bn)))
 
 
 def scratch_capacity() -> int:

@@ -254,26 +254,30 @@ cutile_status_t resolve_grid(const cutile_partition_arg_t* out, const cutile_lau
   return cutile_infer_launch_grid(explicit_grid, parts, 1, grid);
 }
 
-// Picks the variant: caller's hint, then the pinned preference, then `fallback`.
+// Picks the variant.  Precedence: the caller's variant, the function-wide pin set at run time
+// (cutile_kernel_set_preferred_variant), the shape class's winner (a verified tuning record or
+// cutile_kernel_set_preferred_variant_for), then `fallback` (the table's order).  A pin or a winner that does not fit
+// these arguments is passed over, not an error.
 cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* opts, const std::string& fallback,
                               const std::vector<std::string>& acceptable, Resolved* r) {
   std::string want;
   g_last_source = "caller";
   g_last_bucket = g_bucket;
+  auto fits = [&](const std::string& v) { return !v.empty() && std::find(acceptable.begin(), acceptable.end(), v) != acceptable.end(); };
   if (opts && opts->variant) want = opts->variant;
+  if (want.empty()) {
+    std::string pref = preferred_variant(function);
+    if (fits(pref)) {
+      want = pref;
+      g_last_source = "pinned";
+    }
+  }
   if (want.empty() && !g_bucket.empty()) {
     ensure_tuning_records_loaded();
     std::string pref = preferred_variant_for(function, g_bucket);
-    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) {
+    if (fits(pref)) {
       want = pref;
       g_last_source = "record:" + g_bucket;
-    }
-  }
-  if (want.empty()) {
-    std::string pref = preferred_variant(function);
-    if (!pref.empty() && std::find(acceptable.begin(), acceptable.end(), pref) != acceptable.end()) {
-      want = pref;
-      g_last_source = "pinned";
     }
   }
   if (want.empty()) {
@@ -1806,6 +1810,20 @@ cutile_status_t cutile_launch_fmha_decode_gqa_noalloc(cutile_stream_t stream, co
   return cutile_launch_splitk_reduce_merge(stream, &att.tensor, &lse.tensor, out, nullptr);
 }
 
+// Everything the entry point above does once per device and shape — opening the side library, the symbol lookup
+// (the runtime places the array then), loading the two code objects — done ahead of time: the same call in
+// compile-only mode, so every check runs and nothing is enqueued.
+cutile_status_t cutile_fmha_decode_gqa_noalloc_prepare(const cutile_tensor_arg_t* q, const cutile_tensor_arg_t* k,
+                                                       const cutile_tensor_arg_t* v, const cutile_partition_arg_t* out,
+                                                       const cutile_tensor_arg_t* position_start, int32_t num_kv_splits,
+                                                       int32_t bn) {
+  const int saved = g_launch_mode;
+  g_launch_mode = 1;
+  cutile_status_t s = cutile_launch_fmha_decode_gqa_noalloc(nullptr, q, k, v, out, 1.0f, position_start, num_kv_splits, bn);
+  g_launch_mode = saved;
+  return s;
+}
+
 cutile_status_t cutile_launch_softmax(cutile_stream_t stream, const cutile_tensor_arg_t* x,
                                       const cutile_partition_arg_t* y, const cutile_launch_opts_t* opts) {
   if (cutile_status_t s = check_tensor(x, "x", 2, 2)) return s;
@@ -1953,7 +1971,15 @@ cutile_status_t cutile_launch_batch_matmul(cutile_stream_t stream, const cutile_
   args.push_tensor(*b);
   args.push_val<int32_t>(k_total);
   args.push_tile_grid(tg);
-  uint32_t grid[3] = {tg[1] * tg[2], batches, 1};
+  // The batch rides on HIP grid axis y (z for the any-layout kernel), which holds at most 65535 workgroups; the
+  // tiles of one batch are folded into axis x.
+  CUTILE_REQUIRE(batches <= 65535u, CUTILE_ERR_KERNEL_LAUNCH,
+                 "batch_matmul: %u batches in one launch exceed the 65535 workgroups of the grid axis that carries the batch; split the launch",
+                 batches);
+  const uint64_t tiles_per_batch = (uint64_t)tg[1] * tg[2];
+  CUTILE_REQUIRE(tiles_per_batch <= 0x7fffffffull, CUTILE_ERR_KERNEL_LAUNCH,
+                 "batch_matmul: %llu output tiles per batch do not fit a launch grid axis", (unsigned long long)tiles_per_batch);
+  uint32_t grid[3] = {(uint32_t)tiles_per_batch, batches, 1};
   if (res.entry->tile[0] == 0) {   // any-layout kernel: 64x64 outputs per workgroup over the covered region of each batch
     const uint64_t cover_m = std::min<uint64_t>((uint64_t)tg[1] * bm, ct.shape[1]);
     const uint64_t cover_n = std::min<uint64_t>((uint64_t)tg[2] * bn, ct.shape[2]);
@@ -2722,7 +2748,8 @@ static cutile_status_t rng_fill(cutile_rng_t rng, const char* dtype, void* ptr, 
   // enough lanes to keep the stores streaming; each lane walks its blocks with the grid's stride
   uint32_t grid[3] = {std::max<uint32_t>(1, std::min<uint32_t>(div_up(blocks, 256), 8192)), 1, 1};
   if (cutile_status_t s = launch_packed(res.fn, grid, res.entry->block, 0, stream, args)) return s;
-  rng->offset += blocks;
+  // compile-only and specialize-only launches enqueue nothing and write no values: the stream position stays put
+  if (g_launch_mode == 0) rng->offset += blocks;
   return CUTILE_SUCCESS;
 }
 

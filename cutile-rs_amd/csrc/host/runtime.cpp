@@ -7,10 +7,12 @@
 //    device (round robin over 4 streams by default, or a single stream), a
 //    dedicated deallocator stream, an optional memory pool
 //    (cuda-async/src/device_context.rs:139-450, scheduling_policies.rs:35-87);
-//  * the completion reactor: a stream write of 1 into a pinned, device-mapped
-//    flag after the submitted work, and one scanner thread that fires the waker
-//    (cuda-async/src/reactor.rs, slot_table.rs); host-callback fallback chain as
-//    in cuda-async/src/device_future.rs:103-154.
+//  * the completion reactor: after the submitted work the stream writes a
+//    per-use stamp into a pinned, device-mapped word, and one sweeper thread
+//    fires the waker of every slot whose word shows its stamp (slot_table.h;
+//    observable behaviour of cuda-async/src/reactor.rs:68-179: 1024 slots, an
+//    out-of-slots status); host-callback fallback chain as in
+//    cuda-async/src/device_future.rs:103-154.
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -119,17 +121,17 @@ struct Waker {
   void* user;
 };
 
-struct PinnedFlags {
+struct PinnedWords {
   uint32_t* host = nullptr;
-  std::atomic<uint32_t>& flag(size_t slot) { return *reinterpret_cast<std::atomic<uint32_t>*>(host + slot); }
+  std::atomic<uint32_t>& word(size_t slot) { return *reinterpret_cast<std::atomic<uint32_t>*>(host + slot); }
 };
-static_assert(sizeof(std::atomic<uint32_t>) == sizeof(uint32_t), "flag slab is viewed as atomics");
+static_assert(sizeof(std::atomic<uint32_t>) == sizeof(uint32_t), "the pinned slab is viewed as atomics");
 
 constexpr size_t kNumSlots = 1024;     // reactor.rs:29
 constexpr uint32_t kSpinPasses = 10000;  // reactor.rs:31
 
 struct Reactor {
-  std::unique_ptr<SlotTable<Waker, PinnedFlags>> table;
+  std::unique_ptr<SlotTable<Waker, PinnedWords>> table;
   void* device_flags = nullptr;
   std::thread scanner;
   std::mutex park_mutex;
@@ -154,7 +156,7 @@ struct Reactor {
     std::vector<Waker> woken;
     uint32_t idle_passes = 0;
     while (!stop.load(std::memory_order_acquire)) {
-      table->scan_once(woken);
+      table->sweep(woken);
       if (!woken.empty()) {
         // Wakers fire outside any lock the scan held.
         for (auto& w : woken) {
@@ -165,8 +167,8 @@ struct Reactor {
         idle_passes = 0;
         continue;
       }
-      // The park gate is the armed count, not "did this pass see a bit".
-      if (table->is_idle()) {
+      // Sleep only when the pending count reads 0: a slot armed after this pass looked at it is counted already.
+      if (table->nothing_pending()) {
         park();
         idle_passes = 0;
         continue;
@@ -203,7 +205,7 @@ cutile_status_t reactor(Reactor** out) {
     } else {
       memset(host, 0, kNumSlots * sizeof(uint32_t));
       auto* r = new Reactor();
-      r->table = std::make_unique<SlotTable<Waker, PinnedFlags>>(kNumSlots, PinnedFlags{(uint32_t*)host});
+      r->table = std::make_unique<SlotTable<Waker, PinnedWords>>(kNumSlots, PinnedWords{(uint32_t*)host});
       r->device_flags = dev;
       r->scanner = std::thread([r] { r->scan_loop(); });
       g_reactor = r;
@@ -314,17 +316,17 @@ cutile_status_t cutile_reactor_register(cutile_stream_t stream, cutile_waker_fn_
   CUTILE_REQUIRE(waker, CUTILE_ERR_INVALID_ARGUMENT, "waker is null");
   Reactor* r = nullptr;
   if (cutile_status_t s = reactor(&r)) return s;
-  auto slot = r->table->claim();
-  if (!slot) return fail(CUTILE_ERR_OUT_OF_SLOTS, "reactor slot pool exhausted");
-  r->table->reset_flag(*slot);
-  void* addr = static_cast<char*>(r->device_flags) + *slot * sizeof(uint32_t);
-  cutile_status_t s = cutile_stream_write_value32(stream, addr, 1);
+  auto ticket = r->table->acquire();
+  if (!ticket) return fail(CUTILE_ERR_OUT_OF_SLOTS, "reactor slot pool exhausted");
+  // The stream stores this use's stamp; whatever an earlier use left in the word is a different value.
+  void* addr = static_cast<char*>(r->device_flags) + ticket->slot * sizeof(uint32_t);
+  cutile_status_t s = cutile_stream_write_value32(stream, addr, ticket->stamp);
   if (s != CUTILE_SUCCESS) {
-    r->table->release(*slot);
+    r->table->abandon(*ticket);
     return s;
   }
   r->registrations.fetch_add(1, std::memory_order_relaxed);
-  if (r->table->publish(*slot, Waker{waker, user})) r->unpark();
+  if (r->table->arm(*ticket, Waker{waker, user})) r->unpark();
   return CUTILE_SUCCESS;
 }
 
@@ -353,7 +355,7 @@ uint64_t cutile_reactor_wakes(void) {
 }
 int32_t cutile_reactor_armed(void) {
   std::lock_guard<std::mutex> lock(g_reactor_mutex);
-  return g_reactor ? (int32_t)g_reactor->table->armed() : 0;
+  return g_reactor ? (int32_t)g_reactor->table->pending() : 0;
 }
 
 }  // extern "C"

@@ -12,7 +12,8 @@
 // kernel table: source_hash = fingerprint of the code object that holds the kernel,
 // l2 key = fingerprint of (code object, variant symbol), toolchain fingerprint = the
 // device compiler's version text at build time, arch = gfx950.
-// The winner is applied with cutile_kernel_set_preferred_variant, which the launchers consult.
+// A winner reaches the launchers per shape class (cutile_kernel_set_preferred_variant_for, which is also how verified
+// records are applied) or function-wide (cutile_kernel_set_preferred_variant, which takes precedence over records).
 #pragma once
 #include <cstdio>
 #include <ctime>

@@ -230,8 +230,8 @@ cutile_status_t cutile_kernel_set_preferred_variant(const char* function, const 
 
 /* The same per shape class: `bucket` names the class a launcher derives from its arguments (what
  * cutile_last_resolved_bucket reports after a launch, e.g. "bf16_256x256|tiles>256" for gemm).  This is how the winners of
- * verified tuning records reach the launchers; order of precedence at a launch: the caller's variant, the bucket's
- * winner, the function-wide pin, the table's order. */
+ * verified tuning records reach the launchers; order of precedence at a launch: the caller's variant, the function-wide
+ * pin (an explicit run-time choice beats a file on disk), the bucket's winner, the table's order. */
 cutile_status_t cutile_kernel_set_preferred_variant_for(const char* function, const char* bucket, const char* variant);
 /* Tuning records (cutile/src/tune.rs:762-1016): JSON records of autotuner winners, one file per kernel, in the directory
  * `tuned` beside the library (or $CUTILE_TUNING_RECORDS; empty = none), loaded on the first launcher call.  A record is
@@ -575,6 +575,16 @@ cutile_status_t cutile_launch_fmha_decode_gqa_noalloc(cutile_stream_t stream, co
                                                       const cutile_partition_arg_t* out, float qk_scale,
                                                       const cutile_tensor_arg_t* position_start, int32_t num_kv_splits,
                                                       int32_t bn);
+/* Warm-up for the entry point above; like it, without a counterpart in the reference.  The first call of the entry
+ * point on a device opens the side library that holds the array, looks the array's address up (the runtime places the
+ * 8 MiB then) and loads two code objects: work that is neither allocation-free nor legal while a stream is being
+ * captured.  This call does all of it and enqueues nothing (the entry point in compile-only mode: the arguments are
+ * checked exactly as a launch checks them, no pointer is dereferenced).  Call it once per device and shape outside any
+ * capture; after it, cutile_launch_fmha_decode_gqa_noalloc with the same shapes only enqueues two kernels. */
+cutile_status_t cutile_fmha_decode_gqa_noalloc_prepare(const cutile_tensor_arg_t* q, const cutile_tensor_arg_t* k,
+                                                       const cutile_tensor_arg_t* v, const cutile_partition_arg_t* out,
+                                                       const cutile_tensor_arg_t* position_start, int32_t num_kv_splits,
+                                                       int32_t bn);
 /* bytes of the device-resident scratch array behind cutile_launch_fmha_decode_gqa_noalloc (needs no GPU) */
 cutile_status_t cutile_scratch_capacity(size_t* bytes);
 /* gemm<T, BM, BN, BK>(z: [BM,BN] tiles, x, y, k): z <- z + x·y with f32
@@ -771,9 +781,9 @@ cutile_status_t cutile_get_device_pool(int32_t ordinal, cutile_mempool_t* pool);
 /* Completion notification for work already submitted on `stream`.  `waker(user)`
  * is called exactly once, from another thread, after that work has completed.
  * cutile_reactor_register is the flag-write path (cuda-async/src/reactor.rs:154-179):
- * claim one of 1024 slots, enqueue a 32-bit stream write of 1 into pinned mapped
- * memory, publish the waker to the scanner thread; CUTILE_ERR_OUT_OF_SLOTS when
- * all slots are in flight.  cutile_completion_register is the chain
+ * take one of 1024 slots, enqueue a 32-bit stream write of that use's stamp into
+ * pinned mapped memory, hand the waker to the sweeper thread; CUTILE_ERR_OUT_OF_SLOTS
+ * when all slots are in flight.  cutile_completion_register is the chain
  * DeviceFuture uses (cuda-async/src/device_future.rs:103-154): reactor first,
  * hipLaunchHostFunc as fallback (or always, with CUTILE_ASYNC_HOST_SYNC=callback). */
 typedef void (*cutile_waker_fn_t)(void* user);

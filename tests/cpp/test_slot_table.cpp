@@ -1,6 +1,7 @@
-// The reactor's slot protocol under plain atomics standing in for pinned memory,
-// with a modelled "GPU" thread that completes slots — the CPU-side counterpart of
-// cuda-async/src/slot_table.rs:169-330 (MockFlags, std-thread stress 8 x 500).
+// The reactor's completion-slot protocol under plain atomics standing in for pinned memory,
+// with a modelled "GPU" thread that stores the stamps — the properties the reference checks of its own
+// table (cuda-async/src/slot_table.rs:169-330: exactly-once wake, no stale completion, exhaustion, an
+// 8 x 500 thread stress), asked of this one.
 // Built with -fsanitize=thread as well, so the ordering claims are checked by
 // the race detector and not only by the outcome.
 #include <atomic>
@@ -14,81 +15,102 @@
 
 using cutile::SlotTable;
 
-struct MockFlags {
+struct HostWords {
   std::shared_ptr<std::vector<std::atomic<uint32_t>>> cells;
-  explicit MockFlags(size_t n) : cells(std::make_shared<std::vector<std::atomic<uint32_t>>>(n)) {}
-  std::atomic<uint32_t>& flag(size_t slot) { return (*cells)[slot]; }
+  explicit HostWords(size_t n) : cells(std::make_shared<std::vector<std::atomic<uint32_t>>>(n)) {
+    for (auto& c : *cells) c.store(0);
+  }
+  std::atomic<uint32_t>& word(size_t slot) { return (*cells)[slot]; }
 };
+using Table = SlotTable<int, HostWords>;
 
-TEST(claim_publish_scan_recycle) {
-  SlotTable<int, MockFlags> t(4, MockFlags(4));
-  CHECK(t.is_idle());
-  auto s = t.claim();
-  CHECK(s && *s == 0);  // lowest index first
-  t.reset_flag(*s);
-  CHECK(t.publish(*s, 42));        // idle -> active transition reported
-  auto s2 = t.claim();
-  t.reset_flag(*s2);
-  CHECK(!t.publish(*s2, 43));      // already active
-  std::vector<int> woken;
-  CHECK(t.scan_once(woken) && woken.empty() && t.armed() == 2);  // armed, not complete: nothing retires
-  t.flags().flag(*s2).store(1);
-  CHECK(t.scan_once(woken) && woken == std::vector<int>({43}) && t.armed() == 1);
-  t.flags().flag(*s).store(1);
-  woken.clear();
-  t.scan_once(woken);
-  CHECK(woken == std::vector<int>({42}) && t.is_idle());
-  CHECK(!t.scan_once(woken));       // nothing armed any more
-  // exhaustion and release
-  std::vector<size_t> held;
-  while (auto c = t.claim()) held.push_back(*c);
-  CHECK(held.size() == 4 && !t.claim());
-  t.release(held.back());
-  CHECK(t.claim().has_value());
+TEST(acquire_arm_sweep_reuse) {
+  Table t(4, HostWords(4));
+  CHECK(t.nothing_pending());
+  auto a = t.acquire();
+  CHECK(a && a->slot == 0 && a->stamp != 0);  // lowest index first; a stamp is never the word's initial value
+  CHECK(t.arm(*a, 42));                       // nothing was pending: the sweeper has to be woken
+  auto b = t.acquire();
+  CHECK(b && b->slot == 1);
+  CHECK(!t.arm(*b, 43));                      // something already pending
+  std::vector<int> ready;
+  CHECK(t.sweep(ready) == 0 && ready.empty() && t.pending() == 2);  // armed, write not landed: nothing completes
+  t.words().word(b->slot).store(b->stamp);
+  CHECK(t.sweep(ready) == 1 && ready == std::vector<int>({43}) && t.pending() == 1);
+  t.words().word(a->slot).store(a->stamp);
+  ready.clear();
+  CHECK(t.sweep(ready) == 1 && ready == std::vector<int>({42}) && t.nothing_pending());
+  CHECK(t.sweep(ready) == 0);
+  // freed slots are handed out again, lowest first, with a new stamp
+  auto a2 = t.acquire();
+  CHECK(a2 && a2->slot == 0 && a2->stamp != a->stamp);
+  t.abandon(*a2);
+  // exhaustion, and abandon() gives a ticket back
+  std::vector<cutile::SlotTicket> held;
+  while (auto c = t.acquire()) held.push_back(*c);
+  CHECK(held.size() == 4 && !t.acquire());
+  t.abandon(held.back());
+  CHECK(t.acquire().has_value());
 }
 
-TEST(stale_flag_cannot_complete_a_reused_slot) {
-  SlotTable<int, MockFlags> t(1, MockFlags(1));
-  std::vector<int> woken;
-  auto s = *t.claim();
-  t.reset_flag(s);
-  t.publish(s, 1);
-  t.flags().flag(s).store(1);
-  t.scan_once(woken);
-  CHECK(woken.size() == 1);
-  // the flag still reads 1 from the first use; reset_flag runs before the slot is armed again
-  s = *t.claim();
-  t.reset_flag(s);
-  t.publish(s, 2);
-  woken.clear();
-  t.scan_once(woken);
-  CHECK(woken.empty() && t.armed() == 1);
+TEST(a_word_left_by_an_earlier_use_cannot_complete_the_slot) {
+  Table t(1, HostWords(1));
+  std::vector<int> ready;
+  auto a = *t.acquire();
+  t.arm(a, 1);
+  t.words().word(0).store(a.stamp);
+  CHECK(t.sweep(ready) == 1);
+  // nobody clears the word: it still holds the first use's stamp when the slot is armed again
+  auto b = *t.acquire();
+  CHECK(b.slot == 0 && b.stamp != a.stamp);
+  t.arm(b, 2);
+  ready.clear();
+  CHECK(t.sweep(ready) == 0 && ready.empty() && t.pending() == 1);
+  t.words().word(0).store(b.stamp);
+  CHECK(t.sweep(ready) == 1 && ready == std::vector<int>({2}));
+}
+
+TEST(write_that_lands_before_arm_is_found_by_the_next_sweep) {
+  Table t(2, HostWords(2));
+  std::vector<int> ready;
+  auto a = *t.acquire();
+  t.words().word(a.slot).store(a.stamp);   // the stream got there first
+  CHECK(t.sweep(ready) == 0);              // held, not armed: no payload to hand out yet
+  CHECK(t.arm(a, 7));
+  CHECK(t.sweep(ready) == 1 && ready == std::vector<int>({7}) && t.nothing_pending());
+}
+
+TEST(stamps_never_zero_and_never_repeat_back_to_back) {
+  for (uint64_t g : {uint64_t(0), uint64_t(1), uint64_t(0xfffffffeull), uint64_t(0xffffffffull), uint64_t(0x100000000ull), uint64_t(0x1fffffffeull)}) {
+    CHECK(Table::stamp_of(g) != 0);
+    CHECK(Table::stamp_of(g) != Table::stamp_of(g + 1));
+  }
 }
 
 TEST(stress_eight_registrants_one_scanner_one_device) {
   constexpr int kThreads = 8, kPerThread = 500, kSlots = 64;
-  SlotTable<int, MockFlags> t(kSlots, MockFlags(kSlots));
+  Table t(kSlots, HostWords(kSlots));
   std::mutex q_mu;
-  std::deque<size_t> device_queue;  // slots whose "stream write" is in flight
+  std::deque<cutile::SlotTicket> device_queue;  // stream writes in flight
   std::atomic<bool> stop{false};
   std::atomic<int> woken_total{0};
   std::vector<std::atomic<int>> per_payload(kThreads * kPerThread);
   for (auto& p : per_payload) p.store(0);
   std::thread device([&] {
     while (!stop.load() || !device_queue.empty()) {
-      size_t slot = SIZE_MAX;
+      cutile::SlotTicket w{SIZE_MAX, 0};
       {
         std::lock_guard<std::mutex> lock(q_mu);
-        if (!device_queue.empty()) { slot = device_queue.front(); device_queue.pop_front(); }
+        if (!device_queue.empty()) { w = device_queue.front(); device_queue.pop_front(); }
       }
-      if (slot == SIZE_MAX) { std::this_thread::yield(); continue; }
-      t.flags().flag(slot).store(1, std::memory_order_release);
+      if (w.slot == SIZE_MAX) { std::this_thread::yield(); continue; }
+      t.words().word(w.slot).store(w.stamp, std::memory_order_release);
     }
   });
   std::thread scanner([&] {
     std::vector<int> woken;
     while (woken_total.load() < kThreads * kPerThread) {
-      t.scan_once(woken);
+      t.sweep(woken);
       for (int w : woken) { per_payload[w].fetch_add(1); woken_total.fetch_add(1); }
       woken.clear();
       std::this_thread::yield();
@@ -98,14 +120,13 @@ TEST(stress_eight_registrants_one_scanner_one_device) {
   for (int th = 0; th < kThreads; ++th)
     regs.emplace_back([&, th] {
       for (int i = 0; i < kPerThread; ++i) {
-        std::optional<size_t> s;
-        while (!(s = t.claim())) std::this_thread::yield();  // pool exhausted: wait for retirements
-        t.reset_flag(*s);
+        std::optional<cutile::SlotTicket> s;
+        while (!(s = t.acquire())) std::this_thread::yield();  // all slots in use: wait for completions
         {
           std::lock_guard<std::mutex> lock(q_mu);
-          device_queue.push_back(*s);  // the device may complete it before publish: the protocol allows that
+          device_queue.push_back(*s);  // the device may store the stamp before arm(): the protocol allows that
         }
-        t.publish(*s, th * kPerThread + i);
+        t.arm(*s, th * kPerThread + i);
       }
     });
   for (auto& r : regs) r.join();
@@ -113,9 +134,9 @@ TEST(stress_eight_registrants_one_scanner_one_device) {
   stop.store(true);
   device.join();
   for (auto& p : per_payload) CHECK(p.load() == 1);  // every waker fired exactly once
-  CHECK(t.is_idle());
+  CHECK(t.nothing_pending());
   size_t free_slots = 0;
-  while (t.claim()) ++free_slots;
+  while (t.acquire()) ++free_slots;
   CHECK(free_slots == kSlots);  // nothing leaked
 }
 

@@ -292,6 +292,9 @@ def test_example_program_launchers_on_the_recording_runtime(fake_hip):
         ct.matvec(ct.partition(z.half(), [8]), xm, y, 70)
     with pytest.raises(ct.CutileError, match=r"partitioned \[1, BM, BN\]"):
         ct.batch_matmul(ct.partition(c, [3, 128, 128]), a, b, 64)
+    many = 65536                                    # one more batch than the grid axis that carries the batch can hold
+    with pytest.raises(ct.CutileError, match="65535 workgroups of the grid axis"):
+        ct.batch_matmul(ct.partition(torch.zeros(many, 8, 8), [1, 8, 8]), torch.zeros(many, 8, 8), torch.zeros(many, 8, 8), 8)
     assert ct.lib().cutile_testing_launch_count() == n
 
 
@@ -489,6 +492,20 @@ def test_rng_fills_on_the_recording_runtime(fake_hip):
     assert (n, offset, kind) == (7, 251, 0) and rng.offset == 255
     rng.set_seed(3)
     assert rng.offset == 0
+    # compile-only (1) and specialize-only (2) calls enqueue nothing, so the stream position must not move
+    L = ct.lib()
+    L.cutile_set_launch_mode.argtypes = [C.c_int32]
+    before = L.cutile_testing_launch_count()
+    for mode in (1, 2):
+        ct.check(L.cutile_set_launch_mode(mode))
+        try:
+            rng.uniform_(torch.zeros(64))
+        finally:
+            ct.check(L.cutile_set_launch_mode(0))
+        assert rng.offset == 0 and L.cutile_testing_launch_count() == before
+    rng.uniform_(torch.zeros(64))
+    assert rng.offset == 16
+    rng.set_seed(3)
     before = ct.lib().cutile_testing_launch_count()
     rng.uniform_(torch.zeros(0))                                   # nothing to fill: no launch
     assert ct.lib().cutile_testing_launch_count() == before
@@ -532,6 +549,13 @@ def test_tuning_records_choose_variants_per_shape_class_and_stale_ones_are_refus
         # the caller's variant still wins over the record
         ct.gemm(ct.partition(z, [256, 256]), a, b, 256, variant="bf16_256x256x64_w2x2")
         assert ct.last_resolved()["source"] == "caller"
+        # a function-wide pin set at run time wins over the record; taking it away gives the record back
+        ct.set_preferred_variant("gemm", "bf16_256x256x64_w2x2")
+        launch()
+        assert ct.last_resolved()["source"] == "pinned" and ct.last_resolved()["variant"] == "bf16_256x256x64_w2x2"
+        ct.set_preferred_variant("gemm", None)
+        launch()
+        assert ct.last_resolved()["source"] == "record:" + base["bucket"] and ct.last_resolved()["variant"] == "bf16_256x256x64_d2x4"
         # a record whose winner does not fit the arguments (another tile) is ignored for this launch
         ct.set_preferred_variant_for("gemm", base["bucket"], "bf16_128x128x64_d2x2")
         launch()
