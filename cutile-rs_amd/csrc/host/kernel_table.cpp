@@ -159,7 +159,7 @@ std::vector<KernelEntry> build_table() {
     std::string v = std::string(dtype) + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x" +
                     std::to_string(bk) + "_" + kind + std::to_string(wvm) + "x" + std::to_string(wvn);
     // "r" = ring of three x stages and two y stages, the others hold two stages of each
-    const uint32_t lds = kind[0] == 'r' || kind[0] == 'q' ? (uint32_t)((3 * bm * bk + 2 * bk * bn) * 2) : (uint32_t)(2 * (bm * bk + bk * bn) * 2);
+    const uint32_t lds = kind[0] == 'r' || kind[0] == 'q' || kind[0] == 'p' ? (uint32_t)((3 * bm * bk + 2 * bk * bn) * 2) : (uint32_t)(2 * (bm * bk + bk * bn) * 2);
     add("gemm", keep(v), keep("gemm_entry__" + v), IMG_GEMM, (uint32_t)(wvm * wvn * 64), lds, bm, bn, bk, 0, dtype, 0, 2);
   };
   // first entry of a tile shape = default variant; "d" = global->LDS direct, pipelined
@@ -170,6 +170,20 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 256, 256, 64, 2, 4, "r");
   gemm("bf16", 128, 128, 64, 2, 2, "r");
   gemm("bf16", 256, 256, 64, 2, 4, "q");   // "q" = the ring on v_mfma_f32_16x16x32
+  gemm("bf16", 256, 256, 64, 2, 4, "p");   // "p" = the same tile body, one workgroup per compute unit walking its tiles
+  // "s" = the same ring streaming over the output tiles a workgroup walks (one workgroup per compute unit, whole
+  // tiles only).  A family of four kernels: the variant itself reads z as the initial accumulator and moves z past
+  // the caches; "+cached" moves z through them, "+new" starts from zero.  The launcher picks the member; only the
+  // family name is a variant a caller, a pin or a tuning record can name.
+  auto stream_family = [&](const char* fn, const char* dtype, std::initializer_list<const char*> members) {
+    const std::string v = std::string(dtype) + "_256x256x64_s2x4";
+    for (const char* m : members) {
+      std::string sym = std::string(fn) + "_entry__" + v;
+      for (const char* c = m; *c; ++c) sym += *c == '+' ? '_' : *c;
+      add(fn, keep(v + m), keep(sym), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dtype, 0, 2);
+    }
+  };
+  stream_family("gemm", "bf16", {"", "+cached", "+new", "+new+cached"});
   gemm("bf16", 256, 256, 64, 4, 2);
   gemm("bf16", 256, 256, 64, 2, 4);
   gemm("bf16", 256, 256, 64, 2, 2);
@@ -182,6 +196,8 @@ std::vector<KernelEntry> build_table() {
   gemm("f16", 256, 256, 64, 4, 2, "r");
   gemm("f16", 256, 256, 64, 2, 4, "r");
   gemm("f16", 256, 256, 64, 2, 4, "q");
+  gemm("f16", 256, 256, 64, 2, 4, "p");
+  stream_family("gemm", "f16", {"", "+cached", "+new", "+new+cached"});
   gemm("bf16f32", 128, 128, 64, 2, 2);
   gemm("bf16f32", 256, 256, 64, 2, 2);
   // any tile shape, strides and extents (tile = 0: not tied to a partition shape); 64x64 outputs per workgroup
@@ -230,6 +246,7 @@ std::vector<KernelEntry> build_table() {
     std::string v = std::string(dt) + "_256x256x64_q2x4";
     add("gemm_persistent", keep(v), keep("gemm_persistent_entry__" + v), IMG_GEMM, 512, (uint32_t)((3 * 256 * 64 + 2 * 64 * 256) * 2), 256, 256, 64, 0, dt, 0, 2);
   }
+  for (const char* dt : {"bf16", "f16"}) stream_family("gemm_persistent", dt, {"", "+cached"});   // from zero accumulators always
   // 2 x 4 wavefronts first at 256 x 256: the item loop around the tile body costs the 4 x 2 form ten spilled registers (-2 %)
   for (auto t : {std::array<int, 4>{256, 256, 2, 4}, std::array<int, 4>{256, 256, 4, 2}, std::array<int, 4>{128, 128, 2, 2}}) {
     std::string v = "bf16_" + std::to_string(t[0]) + "x" + std::to_string(t[1]) + "x64_d" + std::to_string(t[2]) + "x" + std::to_string(t[3]);

@@ -304,6 +304,32 @@ cutile_status_t resolve_entry(const char* function, const cutile_launch_opts_t* 
 
 uint32_t div_up(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
 
+// The streaming GEMM variants ("..._s2x4"): a family of kernels behind one variant name.
+bool is_stream_variant(const char* variant) { return strstr(variant, "_s2x4") != nullptr; }
+// An output of this size or more is read and stored past the caches (it cannot still be cached when its consumer runs,
+// and the caches are left to the operand panels): the rule of the staged epilogue, decided on the host for this family.
+constexpr int64_t kStreamedOutputBytes = 64ll << 20;
+// Replaces the resolved family entry by the member for (z read as the initial accumulator?, z past the caches?) and
+// gives the launch grid: one workgroup per compute unit, or per tile if there are fewer tiles.
+cutile_status_t stream_member(Resolved* r, const char* function, bool accumulate, const cutile_tensor_arg_t& zt, uint64_t tiles,
+                              uint32_t* grid) {
+  const bool past_caches = (int64_t)zt.shape[0] * zt.shape[1] * (int64_t)cutile_dtype_size(zt.dtype) >= kStreamedOutputBytes;
+  std::string member = r->entry->variant;
+  if (!accumulate) member += "+new";
+  if (!past_caches) member += "+cached";
+  const KernelEntry* e = find_entry(function, member);
+  CUTILE_REQUIRE(e, CUTILE_ERR_KERNEL_NOT_FOUND, "kernel '%s' has no member '%s'", function, member.c_str());
+  int cus = 256;
+  if (g_launch_mode != 2) {
+    if (cutile_status_t s = compute_units(r->device, &cus)) return s;
+    if (e != r->entry)
+      if (cutile_status_t s = load_entry(r->device, e, &r->fn)) return s;
+    g_last_fn = r->fn;
+  }
+  *grid = (uint32_t)std::min<uint64_t>(tiles, (uint64_t)std::max(cus, 1));
+  return CUTILE_SUCCESS;
+}
+
 // Shape classes of tuning records: row lengths by the next power of two (at least 256).
 std::string pow2_class(int64_t n) {
   int64_t p = 256;
@@ -1893,17 +1919,31 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   const std::string dt = in_f32 ? "f32" : in_f16 ? "f16" : zt.dtype == CUTILE_DTYPE_BF16 ? "bf16" : "bf16f32";
   // The ring-pipelined variants on 32 x 32 x 16 ("_r") fetch whole K tiles only ("_q" masks a ragged last tile).
   const int32_t k_valid = std::min(std::min(x->shape[1], y->shape[0]), k_total);
+  // The streaming variants ("_s": one workgroup per compute unit walks its share of the tiles, the operand ring
+  // running on from tile to tile) take whole tiles in M, N and K only, and at least three K tiles.
+  const bool whole_tiles = (int64_t)tg[0] * bm == zt.shape[0] && (int64_t)tg[1] * bn == zt.shape[1] && x->shape[0] >= zt.shape[0] &&
+                           y->shape[1] >= zt.shape[1] && k_valid == k_total && k_total % 64 == 0 && k_total >= 192;
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
       if (strcmp(e.function, "gemm") == 0 && dt == e.dtype && e.tile[0] == bm && e.tile[1] == bn &&
-          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr))
+          (k_valid % 64 == 0 || strstr(e.variant, "_r") == nullptr) && strchr(e.variant, '+') == nullptr &&
+          (whole_tiles || !is_stream_variant(e.variant)))
         acceptable.push_back(e.variant);
   acceptable.push_back(dt + "_generic");
   Resolved res;
   // shape class for tuning records: the tile, and whether the tiles fit one wave of workgroups over the 256 CUs
   BucketScope bucket(dt + "_" + std::to_string(bm) + "x" + std::to_string(bn) + ((uint64_t)tg[0] * tg[1] <= 256 ? "|tiles<=256" : "|tiles>256"));
   if (cutile_status_t s = resolve_entry("gemm", opts, acceptable[0], acceptable, &res)) return s;
+  uint32_t stream_grid = 0;
+  if (is_stream_variant(res.entry->variant)) {
+    if (cutile_status_t s = stream_member(&res, "gemm", accumulate != 0, zt, (uint64_t)tg[0] * tg[1], &stream_grid)) return s;
+  } else if (strstr(res.entry->variant, "_p2x4") != nullptr) {   // the walking form: one workgroup per compute unit
+    int cus = 256;
+    if (g_launch_mode != 2)
+      if (cutile_status_t s = compute_units(res.device, &cus)) return s;
+    stream_grid = (uint32_t)std::min<uint64_t>((uint64_t)tg[0] * tg[1], (uint64_t)std::max(cus, 1));
+  }
   ArgPacker args;
   args.push_partition(*z);
   args.push_tensor(*x);
@@ -1911,7 +1951,7 @@ cutile_status_t cutile_launch_gemm(cutile_stream_t stream, const cutile_partitio
   args.push_val<int32_t>(k_total);
   args.push_tile_grid(tg);
   args.push_val<int32_t>(accumulate ? 1 : 0);
-  uint32_t grid[3] = {tg[0] * tg[1], 1, 1};
+  uint32_t grid[3] = {stream_grid ? stream_grid : tg[0] * tg[1], 1, 1};
   if (res.entry->tile[0] == 0) {   // any-layout kernel: 64x64 outputs per workgroup over the covered region
     const uint64_t cover_m = std::min<uint64_t>((uint64_t)tg[0] * bm, zt.shape[0]);
     const uint64_t cover_n = std::min<uint64_t>((uint64_t)tg[1] * bn, zt.shape[1]);
@@ -2151,14 +2191,24 @@ cutile_status_t cutile_launch_gemm_persistent(cutile_stream_t stream, const cuti
                            aligned16(zt.ptr) && x->shape[1] % 8 == 0 && y->shape[1] % 8 == 0 && zt.shape[1] % 4 == 0 &&
                            extent_bytes_2d(*x) < kDescriptorLimit && extent_bytes_2d(*y) < kDescriptorLimit &&
                            extent_bytes_2d(zt) < kDescriptorLimit;
+  // the streaming variant: whole tiles in M, N and K, at least three K tiles, the plain two-axis schedule
+  const int32_t kx = x->shape[1];
+  const bool whole_tiles = zt.shape[0] % bm == 0 && zt.shape[1] % bn == 0 && x->shape[0] >= zt.shape[0] && y->shape[1] >= zt.shape[1] &&
+                           y->shape[0] >= kx && kx % 64 == 0 && kx >= 192 && m.rank == 2;
   std::vector<std::string> acceptable;
   if (fast_layout)
     for (const auto& e : kernel_table())
-      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn)
+      if (strcmp(e.function, "gemm_persistent") == 0 && strcmp(e.dtype, dt) == 0 && e.tile[0] == bm && e.tile[1] == bn &&
+          strchr(e.variant, '+') == nullptr && (whole_tiles || !is_stream_variant(e.variant)))
         acceptable.push_back(e.variant);
   acceptable.push_back(std::string(dt) + "_generic");
   Resolved res;
   if (cutile_status_t s = resolve_entry("gemm_persistent", opts, acceptable[0], acceptable, &res)) return s;
+  if (is_stream_variant(res.entry->variant)) {
+    uint32_t unused = 0;
+    // (the member only; the launch grid stays the caller's num_tile_blocks, and the accumulators start from zero)
+    if (cutile_status_t s = stream_member(&res, "gemm_persistent", true, zt, m.total, &unused)) return s;
+  }
   ArgPacker args;
   args.push_partition(*z);
   args.push_tensor(*x);

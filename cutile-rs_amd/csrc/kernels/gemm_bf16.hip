@@ -790,6 +790,21 @@ struct GemmRing16 {
     }
   }
 
+  // gemm launched with one workgroup per compute unit ("p"): workgroup b walks the tiles b, b + gridDim.x, ... of the
+  // launch's XCD-contiguous, M-grouped order, tile after tile with the full tile body (any extents, any K, z as the
+  // initial accumulator or not).  Against one workgroup per tile it saves the workgroup starts and keeps each XCD on
+  // one contiguous eighth of the order round by round.
+  __device__ static void run_walk(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y, int32_t k_total,
+                                  const TileGrid& g, int32_t accumulate) {
+    const uint32_t total = g.x * g.y;
+    for (uint32_t item = blockIdx.x; item < total; item += gridDim.x) {
+      uint32_t pm, pn;
+      tile_of_id(item, g.x, g.y, gridDim.x, &pm, &pn);
+      run_tile(z, x, y, k_total, pm, pn, accumulate);
+      __syncthreads();   // the output bands live in the stages that the next tile refills
+    }
+  }
+
   __device__ static __forceinline__ void run_tile(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
                                                   int32_t k_total, uint32_t pm, uint32_t pn, int32_t accumulate) {
     // Separately named stages: the compiler can then tell a refill of one from
@@ -992,6 +1007,375 @@ struct GemmRing16 {
     if (wave < 6) band += (wave & 1) * kEpilogueBytesPerWave<WN>;
     store_tile_staged16<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0], z.shape[0], z.shape[1], row0 + wm * WM,
                                     col0 + wn * WN, lane, accumulate);
+  }
+};
+
+// ---- the 16 x 16 x 32 ring as one stream over many output tiles ------------------------------
+// A workgroup that computes several output tiles one after another (four per compute unit at 8192^3) pays, per tile
+// of GemmRing16, for an epilogue through LDS, a barrier because the output bands live in the operand stages, and a
+// prologue whose first fetch nothing hides.  Here the operand ring never stops:
+//  * the K tiles of a workgroup's output tiles form ONE sequence; the fetch two / three tiles ahead simply runs on
+//    into the next output tile's first K tiles (tile origin and K position are both in the scalar offset of the
+//    fetch, the per-lane offsets do not depend on the tile), so when the last MFMA of an output tile issues, the
+//    next tile's first three x tiles and two y tiles are in LDS or in flight;
+//  * the epilogue uses no LDS, so it needs no barrier and leaves the stages alone: two in-ALU exchanges
+//    (v_permlane32_swap, v_permlane16_swap) turn the accumulator layout of v_mfma_f32_16x16x32 (a lane: 4
+//    consecutive columns of one row, the four lane groups side by side, 16-column blocks in registers) into 8
+//    consecutive columns per lane with the four lane groups side by side — each store instruction then writes 16
+//    rows of 64 contiguous bytes, and the old z for `accumulate` is read in that same shape, two row blocks ahead;
+// Needs whole tiles in M, N and K (the launcher checks; everything else runs GemmRing16) and at least three K tiles.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT, typename InT = __bf16>
+struct GemmStream16 {
+  static_assert(sizeof(OutT) == 2, "16-bit outputs");
+  static constexpr int BK = 64;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 16, TN = WN / 16;
+  static constexpr int TMH = TM / 2;
+  static_assert(TM % 2 == 0 && TN % 2 == 0, "row blocks by halves, column blocks by pairs");
+  static constexpr int UB = BN / 8;
+  static constexpr int kAInstr = BM / 8 / kWaves;
+  static constexpr int kBRowsPerInstr = 64 / UB;
+  static constexpr int kBInstr = BK / kBRowsPerInstr / kWaves;
+  static constexpr int kABytes = BM * BK * 2, kBBytes = BK * BN * 2;
+  static constexpr int kLdsBytes = 3 * kABytes + 2 * kBBytes;
+  static_assert(BM % (8 * kWaves) == 0 && BK % (kBRowsPerInstr * kWaves) == 0, "tile must split evenly");
+  static_assert(UB >= 16 && UB <= 64, "y-tile row must be 16..64 units");
+  static_assert(kBInstr % 2 == 0, "each wavefront fetches the same share of both y halves");
+  static_assert(kAInstr + kBInstr <= 15, "the wait count must fit the low vmcnt field");
+
+  __device__ static __forceinline__ int a_lds_off(int r, int u) { return r * (BK * 2) + ((u ^ ((r >> 1) & 7)) << 4); }
+  __device__ static __forceinline__ int b_swizzle(int r) { return ((r & 3) << 2) | (((r >> 3) & 1) << 1); }
+  __device__ static __forceinline__ int b_lds_off(int r, int u) { return r * (BN * 2) + ((u ^ b_swizzle(r)) << 4); }
+
+  // The register that held `a` holds zeros afterwards (a tied operand: to the compiler the same value lives on, so the
+  // loop that follows accumulates where the last tile did and no second set of accumulator registers appears).
+  __device__ static __forceinline__ void clear_in_place(f32x4& a) {
+    asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+  }
+  // upper 32 lanes of a <-> lower 32 lanes of b, component by component.  (Inline assembly on purpose: through the
+  // compiler's builtin for this instruction the second result came back as a copy of the first in this kernel.)
+  __device__ static __forceinline__ void swap_halves(f32x4& a, f32x4& b) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float p = a[c], q = b[c];
+      asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(p), "+v"(q));
+      a[c] = p, b[c] = q;
+    }
+  }
+  // odd rows of 16 lanes of a <-> even rows of b
+  __device__ static __forceinline__ void swap_rows(f32x4& a, f32x4& b) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float p = a[c], q = b[c];
+      asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(p), "+v"(q));
+      a[c] = p, b[c] = q;
+    }
+  }
+
+  // `tile_of(j, &pm, &pn)`: the tile of this workgroup's j-th item, j < n_mine.  ACCUMULATE and STREAM (z read and
+  // written past the caches) are compile-time: under a run-time flag the compiler cannot pair the epilogue's loads
+  // with their uses and waits for everything in flight, the ring's fetches included.  One instantiation per kernel:
+  // the stages below are static arrays of this function.
+  template <bool ACCUMULATE, bool STREAM, class TileOf>
+  __device__ static __forceinline__ void run_items(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                                   int32_t k_total, uint32_t n_mine, TileOf tile_of) {
+    // Separately named stages: the compiler can then tell a refill of one from operand reads of another and adds no
+    // waits of its own.
+    __shared__ __attribute__((aligned(1024))) unsigned char xs0[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs1[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs2[kABytes];
+    // (the larger alignment puts the y stages first: all four then lie inside the 64 KiB that the immediate offset
+    // of an LDS read spans, so one address register per column block serves them all)
+    __shared__ __attribute__((aligned(4096))) unsigned char ys0a[kBBytes / 2];
+    __shared__ __attribute__((aligned(4096))) unsigned char ys0b[kBBytes / 2];
+    __shared__ __attribute__((aligned(4096))) unsigned char ys1a[kBBytes / 2];
+    __shared__ __attribute__((aligned(4096))) unsigned char ys1b[kBBytes / 2];
+    constexpr bool accumulate = ACCUMULATE, stream = STREAM;
+    if (n_mine == 0) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int32_t lda = x.strides[0], ldb = y.strides[0], ldz = z.strides[0];
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)(((int64_t)(x.shape[0] - 1) * lda + x.shape[1]) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)(((int64_t)(y.shape[0] - 1) * ldb + y.shape[1]) * 2));
+    const int k_tiles = k_total / BK;
+
+    // Per-lane side of the fetches: the lane's place inside ANY x tile / y tile.  Where the tile lies (its first row
+    // or column, its K position) and which of the wavefront's fetch instructions it is go into the scalar offset.
+    // x instruction i covers rows (wave * kAInstr + i) * 8 + lane / 8: the swizzle term ((row >> 1) & 7) of a lane
+    // repeats with i & 1, so two per-lane offsets serve all of them; y instruction i covers K rows
+    // (i * kWaves + wave) * kBRowsPerInstr + lane / UB, whose swizzle term does not depend on i at all: one offset.
+    static_assert(kAInstr % 2 == 0 && (kWaves * kBRowsPerInstr) % 16 == 0, "fetch offsets repeat as assumed");
+    uint32_t a_voff[2], b_voff;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_voff[i] = (uint32_t)(((int64_t)((wave * kAInstr) * 8 + (lane >> 3)) * lda + u * 8) * 2);   // row of instruction 0: the row step is scalar
+    }
+    {
+      const int r = wave * kBRowsPerInstr + lane / UB;
+      const int u = (lane % UB) ^ b_swizzle(r);
+      b_voff = (uint32_t)(((int64_t)r * ldb + u * 8) * 2);
+    }
+    const uint32_t a_istep = (uint32_t)(8 * lda * 2), b_istep = (uint32_t)(kWaves * kBRowsPerInstr * ldb * 2);
+    auto fetch_a = [&](unsigned char* stage, uint32_t soff, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(stage + (wave * kAInstr + i) * 1024), 16, a_voff[i & 1],
+                                               (int32_t)(soff + (uint32_t)i * a_istep), 0, 0);
+    };
+    auto fetch_b = [&](unsigned char* half, uint32_t soff, int i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(half + ((i % (kBInstr / 2)) * kWaves + wave) * 1024), 16, b_voff,
+                                               (int32_t)(soff + (uint32_t)i * b_istep), 0, 0);
+    };
+
+    const int grp = lane >> 4, l16 = lane & 15;
+    const int tr_row = l16 >> 2, tr_col = (l16 & 3) * 4;
+    // x: the address of K step 1 is that of K step 0 with bit 6 flipped (the K step is bit 2 of the 16-byte unit, which
+    // the swizzle only XORs); it is formed where it is used, one instruction per block, instead of living in a register
+    // of its own per 64 KiB window of LDS for the whole kernel.
+    int a_addr0, b_addr[TN];
+    a_addr0 = a_lds_off(wm * WM + l16, grp);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int n = wn * WN + tn * 16 + tr_col;
+      const int kr = grp * 8 + tr_row;
+      b_addr[tn] = b_lds_off(kr, n >> 3) + (n & 7) * 2;
+    }
+    constexpr int NB = TMH * TN;
+    auto read_a = [&](const unsigned char* xs, int a_at, int mh, bf16x8 (&into)[TMH], int i) {
+      into[i] = *reinterpret_cast<const bf16x8*>(xs + a_at + (mh * TMH + i) * (16 * BK * 2));
+    };
+    auto a_addr_of = [&](int ks) {
+      int at = a_addr0;
+      if (ks == 1) asm volatile("v_xor_b32 %0, 64, %1" : "=v"(at) : "v"(a_addr0));
+      return at;
+    };
+    auto read_b = [&](const unsigned char* yh, bf16x8 (&into)[TN], int tn) {
+      const unsigned char* p = yh + b_addr[tn];
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(p + 4 * (BN * 2)));
+      into[tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+
+    f32x4 acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[tn][tm][v] = 0.0f;
+
+    // One MFMA block, as in GemmRing16 (memory instructions dealt out one per MFMA at most); so_x / so_y are the
+    // scalar offsets of the x tile and the y tile being fetched.
+    constexpr int SLOTS = NB;
+    auto block = [&](bf16x8 (&a)[TMH], const bf16x8 (&ub)[TN], int mh, const unsigned char* rd_x, int rd_ks, int rd_mh,
+                     bool with_y, const unsigned char* rd_y, bf16x8 (&ib)[TN], bool with_fill_x, unsigned char* fill_x,
+                     unsigned char* fill_y, int fb0, int fb1, uint32_t so_x, uint32_t so_y) {
+      const int n_fill = (with_fill_x ? kAInstr : 0) + (fb1 - fb0);
+      const int rd_at = a_addr_of(rd_ks);
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int tm = j / TN, tn = j % TN;
+#pragma unroll
+        for (int i = 0; i < kAInstr + kBInstr; ++i) {
+          if (i < n_fill && i * SLOTS / n_fill == j) {
+            if (with_fill_x && i < kAInstr)
+              fetch_a(fill_x, so_x, i);
+            else
+              fetch_b(fill_y, so_y, fb0 + i - (with_fill_x ? kAInstr : 0));
+          }
+        }
+        if (with_y) {
+#pragma unroll
+          for (int q = 0; q < TN; ++q)
+            if (q * SLOTS / TN == j) read_b(rd_y, ib, q);
+        }
+        acc[tn][mh * TMH + tm] = mfma_16x16x32<InT>(ub[tn], a[tm], acc[tn][mh * TMH + tm]);
+        if (tn == TN - 1) read_a(rd_x, rd_at, rd_mh, a, tm);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+
+    // Where the current output tile and the next one lie (scalar): byte offsets of the tile's first x row / y column.
+    uint32_t pm, pn;
+    tile_of(0u, &pm, &pn);
+    uint32_t a_cur = (uint32_t)((int64_t)pm * BM * lda * 2), b_cur = pn * (BN * 2);
+    uint32_t z_row = pm * BM, z_col = pn * BN;
+    uint32_t a_nxt = a_cur, b_nxt = b_cur, z_row_nxt = z_row, z_col_nxt = z_col;
+    auto look_ahead = [&](uint32_t j) {      // the tile after item j, or item j's own once more (fetched, never used)
+      if (j + 1 < n_mine) {
+        uint32_t qm, qn;
+        tile_of(j + 1, &qm, &qn);
+        a_nxt = (uint32_t)((int64_t)qm * BM * lda * 2), b_nxt = qn * (BN * 2);
+        z_row_nxt = qm * BM, z_col_nxt = qn * BN;
+      }
+    };
+    look_ahead(0);
+    const uint32_t y_step = (uint32_t)(BK * ldb * 2);
+    // x tile / y tile number kf counted from the current output tile's first: past its last, the next tile's
+    auto so_x = [&](int kf) { return kf < k_tiles ? a_cur + (uint32_t)kf * (BK * 2) : a_nxt + (uint32_t)(kf - k_tiles) * (BK * 2); };
+    auto so_y = [&](int kf) { return kf < k_tiles ? b_cur + (uint32_t)kf * y_step : b_nxt + (uint32_t)(kf - k_tiles) * y_step; };
+
+    bf16x8 af[TMH], b0[TN], b1[TN];
+    // Prologue of the first output tile, in the issue order the steady state would have produced.
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs0, so_x(0), i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys0a, so_y(0), i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs1, so_x(1), i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys0b, so_y(0), i);
+#pragma unroll
+    for (int i = 0; i < kBInstr / 2; ++i) fetch_b(ys1a, so_y(1), i);
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) fetch_a(xs2, so_x(2), i);
+#pragma unroll
+    for (int i = kBInstr / 2; i < kBInstr; ++i) fetch_b(ys1b, so_y(1), i);
+    constexpr int kPrologueLeft = 2 * kAInstr + 3 * kBInstr / 2;
+    __builtin_amdgcn_s_waitcnt((kPrologueLeft & 15) | (7 << 4) | (0 << 8) | ((kPrologueLeft >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) read_b(ys0a, b0, tn);
+#pragma unroll
+    for (int i = 0; i < TMH; ++i) read_a(xs0, a_addr0, 0, af, i);
+
+    // K tile kt of the current output tile: GemmRing16's, with the fetches' scalar offsets running on into the next
+    // output tile.  Stores and loads share the wavefront's in-order memory counter, so in the first K tile after an
+    // epilogue these waits also wait for the older half of the epilogue's stores — by then a K tile's worth of matrix
+    // work old.  (Waits with a larger count in that K tile were built: behind a branch the compiler's own
+    // bookkeeping of what is in flight turns inexact and it adds waits of its own in front of the operand reads;
+    // as a second straight-line copy of the K tile the register allocation falls apart.)
+    constexpr int kWaitOlderLoads = (kAInstr + kBInstr) | (7 << 4) | (0 << 8);
+    auto k_tile = [&](unsigned char* x_cur, unsigned char* ya_cur, unsigned char* yb_cur, const unsigned char* x_nxt,
+                      const unsigned char* ya_nxt, int kt) {
+      block(af, b0, 0, x_cur, 0, 1, false, x_cur, b1, false, x_cur, x_cur, 0, 0, 0, 0);
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(af, b0, 1, x_cur, 1, 0, true, yb_cur, b1, false, x_cur, ya_cur, 0, kBInstr / 2, 0, so_y(kt + 2));
+      block(af, b1, 0, x_cur, 1, 1, false, x_cur, b0, false, x_cur, x_cur, 0, 0, 0, 0);
+      __builtin_amdgcn_s_waitcnt(kWaitOlderLoads);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      block(af, b1, 1, x_nxt, 0, 0, true, ya_nxt, b0, true, x_cur, yb_cur, kBInstr / 2, kBInstr, so_x(kt + 3), so_y(kt + 2));
+    };
+
+    // Epilogue of the tile at (z_row, z_col): registers only.  After the two exchanges lane (grp, l16) holds, for row
+    // block tm and column pair kp, the 8 consecutive columns kp * 32 + grp * 8 .. + 7 of row tm * 16 + l16.  z is
+    // addressed like the operands: one per-lane offset for every access, the rest in the scalar offset.
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(z.ptr, (uint32_t)(((int64_t)(z.shape[0] - 1) * ldz + z.shape[1]) * 2));
+    const uint32_t z_voff = (uint32_t)(((int64_t)l16 * ldz + grp * 8) * 2);
+    constexpr int kAux = stream ? 2 : 0;      // nt: past the caches
+    // row blocks per chunk of old z (a chunk ahead is in flight while one is added): two where the registers allow it;
+    // the f16 kernels have four registers fewer to spare and would spill in the K loop
+    constexpr int CH = __is_same(OutT, _Float16) ? 1 : 2;
+    constexpr int KP = TN / 2;
+    auto epilogue = [&]() {
+      // scalar offset of row block tm, column pair kp of this wavefront's part of the tile
+      auto z_soff = [&](int tm, int kp) {
+        return (uint32_t)(((int64_t)(z_row + wm * WM + tm * 16) * ldz + z_col + wn * WN + kp * 32) * 2);
+      };
+      u32x4 old[2][CH][KP];
+      auto load_chunk = [&](int c, u32x4 (&o)[CH][KP]) {
+#pragma unroll
+        for (int t = 0; t < CH; ++t)
+#pragma unroll
+          for (int kp = 0; kp < KP; ++kp)
+            o[t][kp] = __builtin_amdgcn_raw_buffer_load_b128(rz, z_voff, z_soff(c * CH + t, kp), kAux);
+      };
+      if (accumulate) load_chunk(0, old[0]);
+#pragma unroll
+      for (int c = 0; c < TM / CH; ++c) {
+        if (accumulate && c + 1 < TM / CH) load_chunk(c + 1, old[(c + 1) & 1]);
+#pragma unroll
+        for (int t = 0; t < CH; ++t) {
+          const int tm = c * CH + t;
+#pragma unroll
+          for (int kp = 0; kp < KP; ++kp) {
+            f32x4 lo = acc[2 * kp][tm], hi = acc[2 * kp + 1][tm];
+            swap_halves(lo, hi);
+            swap_rows(lo, hi);
+            if (accumulate) {
+              const u32x4 o = old[c & 1][t][kp];
+              lo[0] += stored_lo<OutT>(o.x), lo[1] += stored_hi<OutT>(o.x), lo[2] += stored_lo<OutT>(o.y), lo[3] += stored_hi<OutT>(o.y);
+              hi[0] += stored_lo<OutT>(o.z), hi[1] += stored_hi<OutT>(o.z), hi[2] += stored_lo<OutT>(o.w), hi[3] += stored_hi<OutT>(o.w);
+            }
+            const u32x4 w = {pack_out2<OutT>(lo[0], lo[1]), pack_out2<OutT>(lo[2], lo[3]), pack_out2<OutT>(hi[0], hi[1]),
+                             pack_out2<OutT>(hi[2], hi[3])};
+            __builtin_amdgcn_raw_buffer_store_b128(w, rz, z_voff, z_soff(tm, kp), kAux);
+            // A 16-byte store reads its data registers for a few cycles after it issues, and the compiler, which knows this
+            // hazard only for stores without a scalar offset, reuses them at once (the next block's exchange operands
+            // are moved in): two idle cycles keep the new values out of the store.
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_nop 1");
+            __builtin_amdgcn_sched_barrier(0);
+            // zero for the next tile, in place: the accumulators of the next tile are the same registers
+            clear_in_place(acc[2 * kp][tm]);
+            clear_in_place(acc[2 * kp + 1][tm]);
+          }
+        }
+      }
+    };
+
+    // The stage names repeat every 6 K tiles (3 x stages, 2 y stages); an output tile may end after any of them.
+    // After the workgroup's last tile the wavefront ends right there (this body is the whole kernel): six loop exits
+    // would be routed through one block in front of the loop header, and the compiler's bookkeeping of the fetches in
+    // flight would then see every phase's end state arrive at the first phase and add waits of its own there.
+    int left = k_tiles;       // K tiles of the current output tile still to run
+    uint32_t item = 0;
+    auto tile_end = [&]() {
+      epilogue();
+      if (++item == n_mine) {
+        __builtin_amdgcn_s_waitcnt(0);  // the look-ahead fetches must not outlive the workgroup's LDS
+        __builtin_amdgcn_endpgm();
+      }
+      a_cur = a_nxt, b_cur = b_nxt, z_row = z_row_nxt, z_col = z_col_nxt;
+      look_ahead(item);
+      left = k_tiles;
+    };
+    for (;;) {
+      k_tile(xs0, ys0a, ys0b, xs1, ys1a, k_tiles - left);
+      if (--left == 0) tile_end();
+      k_tile(xs1, ys1a, ys1b, xs2, ys0a, k_tiles - left);
+      if (--left == 0) tile_end();
+      k_tile(xs2, ys0a, ys0b, xs0, ys1a, k_tiles - left);
+      if (--left == 0) tile_end();
+      k_tile(xs0, ys1a, ys1b, xs1, ys0a, k_tiles - left);
+      if (--left == 0) tile_end();
+      k_tile(xs1, ys0a, ys0b, xs2, ys1a, k_tiles - left);
+      if (--left == 0) tile_end();
+      k_tile(xs2, ys1a, ys1b, xs0, ys0a, k_tiles - left);
+      if (--left == 0) tile_end();
+    }
+  }
+
+  // gemm: workgroup b takes the tiles b, b + gridDim.x, ... of the launch's XCD-contiguous, M-grouped order
+  template <bool ACCUMULATE, bool STREAM>
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y, int32_t k_total,
+                             const TileGrid& g) {
+    const uint32_t total = g.x * g.y;
+    const uint32_t n_mine = blockIdx.x < total ? (total - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    run_items<ACCUMULATE, STREAM>(z, x, y, k_total, n_mine, [&](uint32_t j, uint32_t* pm, uint32_t* pn) {
+      tile_of_id(blockIdx.x + j * gridDim.x, g.x, g.y, gridDim.x, pm, pn);
+    });
+  }
+  // gemm_persistent: the stream items of the mapped partition, from zero accumulators
+  template <bool STREAM>
+  __device__ static void run_persistent(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                                        const MappedArg& m) {
+    const uint32_t n_mine = blockIdx.x < m.total ? (m.total - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    run_items<false, STREAM>(z, x, y, x.shape[1], n_mine, [&](uint32_t j, uint32_t* pm, uint32_t* pn) {
+      const uint32_t it = blockIdx.x + j * gridDim.x;
+      const uint32_t pos = m.total % kNumXcd == 0 ? (it % kNumXcd) * (m.total / kNumXcd) + it / kNumXcd : it;
+      uint32_t bid[3];
+      mapped_index(m, pos, bid);
+      *pm = bid[0], *pn = bid[1];
+    });
   }
 };
 
@@ -1228,8 +1612,40 @@ extern "C" __global__ void __launch_bounds__(512)
                                                   TensorArg<2> b_metas, TensorArg<2> c_metas, int32_t num_groups) {
   group_gemm_desc<GemmRing16<256, 256, 2, 4, _Float16, _Float16>, 256, 256>(a_ptrs, b_ptrs, c_ptrs, a_metas, b_metas, c_metas, num_groups);
 }
+#define GEMM_RING16_WALK_KERNEL(NAME, BM, BN, WVM, WVN, T)                                        \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                         int32_t accumulate) {                                                  \
+    GemmRing16<BM, BN, WVM, WVN, T, T>::run_walk(z, x, y, k, g, accumulate);                    \
+  }
+GEMM_RING16_WALK_KERNEL(bf16_256x256x64_p2x4, 256, 256, 2, 4, __bf16)
+GEMM_RING16_WALK_KERNEL(f16_256x256x64_p2x4, 256, 256, 2, 4, _Float16)
 GEMM_RING16_PERSISTENT_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16)
 GEMM_RING16_PERSISTENT_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16)
+
+// the 16 x 16 x 32 ring streaming over a workgroup's output tiles ("s"): gemm launched with one workgroup per compute
+// unit, and the persistent GEMM over a mapped partition.  One kernel per (z read as the initial accumulator or not,
+// z past the caches or through them): the launcher picks; `accumulate` is part of the signature all the same.
+#define GEMM_STREAM16_KERNEL(NAME, SUFFIX, ACC, NT, BM, BN, WVM, WVN, T)                         \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_entry__##NAME##SUFFIX(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, int32_t k, TileGrid g, \
+                                 int32_t accumulate) {                                          \
+    GemmStream16<BM, BN, WVM, WVN, T, T>::template run<ACC, NT>(z, x, y, k, g);                 \
+  }
+#define GEMM_STREAM16_PERSISTENT_KERNEL(NAME, SUFFIX, NT, BM, BN, WVM, WVN, T)                   \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
+      gemm_persistent_entry__##NAME##SUFFIX(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \
+    GemmStream16<BM, BN, WVM, WVN, T, T>::template run_persistent<NT>(z, x, y, m);              \
+  }
+#define GEMM_STREAM16_FAMILY(NAME, T)                                                            \
+  GEMM_STREAM16_KERNEL(NAME, , true, true, 256, 256, 2, 4, T)                                    \
+  GEMM_STREAM16_KERNEL(NAME, _cached, true, false, 256, 256, 2, 4, T)                            \
+  GEMM_STREAM16_KERNEL(NAME, _new, false, true, 256, 256, 2, 4, T)                               \
+  GEMM_STREAM16_KERNEL(NAME, _new_cached, false, false, 256, 256, 2, 4, T)                       \
+  GEMM_STREAM16_PERSISTENT_KERNEL(NAME, , true, 256, 256, 2, 4, T)                               \
+  GEMM_STREAM16_PERSISTENT_KERNEL(NAME, _cached, false, 256, 256, 2, 4, T)
+GEMM_STREAM16_FAMILY(bf16_256x256x64_s2x4, __bf16)
+GEMM_STREAM16_FAMILY(f16_256x256x64_s2x4, _Float16)
 
 #define GEMM_ANY_LAYOUT_KERNEL(NAME, IN_T, OUT_T)                                                \
   extern "C" __global__ void __launch_bounds__(256)                                            \

@@ -101,6 +101,22 @@ __device__ __forceinline__ void tile_coords(uint32_t tiles_m, uint32_t tiles_n, 
   *pn = in_group / rows;
 }
 
+// The same order for a workgroup that walks several tiles: item `id` of a launch of `stride` workgroups (workgroup b
+// takes b, b + stride, ...).  Workgroups are dealt round-robin to the XCDs, so with stride a multiple of 8 all items of
+// a workgroup lie on its XCD, which covers one contiguous eighth of the M-grouped order round by round.
+__device__ __forceinline__ void tile_of_id(uint32_t id, uint32_t tiles_m, uint32_t tiles_n, uint32_t stride, uint32_t* pm,
+                                           uint32_t* pn) {
+  const uint32_t total = tiles_m * tiles_n;
+  if (total % kNumXcd == 0 && stride % kNumXcd == 0) id = (id % kNumXcd) * (total / kNumXcd) + id / kNumXcd;
+  const uint32_t per_group = kGroupM * tiles_n;
+  const uint32_t group = id / per_group;
+  const uint32_t first_m = group * kGroupM;
+  const uint32_t rows = min(tiles_m - first_m, (uint32_t)kGroupM);
+  const uint32_t in_group = id % per_group;
+  *pm = first_m + in_group % rows;
+  *pn = in_group / rows;
+}
+
 // Epilogue shared by the pipelined variants: accumulators -> z through LDS.
 // In the MFMA layout a lane owns 4 consecutive columns of one row, so a direct
 // store touches 32 rows with 8 or 16 bytes each and every 128-byte line of z is

@@ -615,6 +615,7 @@ inline std::vector<Config> variant_configs(const std::string& function, const st
     auto colon = e.find(':');
     if (e.substr(0, colon) != function) continue;
     std::string v = e.substr(colon + 1);
+    if (v.find('+') != std::string::npos) continue;      // a member of a kernel family: chosen by the launcher, not a variant of its own
     if (!must_contain.empty() && v.find(must_contain) == std::string::npos) continue;
     out.push_back(Config::make({{"variant", ParamValue(v)}}));
   }
