@@ -206,16 +206,32 @@ class SoftmaxAllF16(Softmax):
                 "sample": f"first {rows} of {self.m} rows (numpy, one f16 rounding per operation)"}, {"within_2_f16_steps": bool(d.max() <= 2)}
 
 
+def tuned_tile(kernel, problem, default):
+    """The tile shape the tuner's (tile, variant) sweep chose for this problem (cutile-rs_amd/tune/tune_baseline.cpp files
+    it in the kernel's tuning record under the bucket "problem|<problem>"), or `default` where no record says."""
+    path = os.path.join(ROOT, "cutile-rs_amd", "tuned", kernel + ".json")
+    try:
+        with open(path) as f:
+            for e in json.load(f).get("entries", []):
+                if e.get("bucket") == "problem|" + problem:
+                    p = e["config"]["params"]
+                    return (int(p["bm"]), int(p["bn"])), "tuning record"
+    except (OSError, ValueError, KeyError):
+        pass
+    return default, "default"
+
+
 class Gemm(Workload):
     unit, dtype, bound, peak_key = "TFLOP/s", "bf16 in / f32 acc / bf16 out", "mfma", "mfma_bf16"
-    tile = (256, 256)
 
     def __init__(self, s):
         self.s = s
         self.name = f"gemm_bf16_{s}"
         self.work = 2.0 * s ** 3
+        # the tile is the caller's choice (the partition of z): taken from the tuner's sweep over tile shapes
+        self.tile, chosen_by = tuned_tile("gemm", f"bf16|{s}x{s}x{s}", (256, 256))
         self.config = {"workload": f"GEMM bf16 M=N=K={s}, z += A·B, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 z",
-                       "tile": "256x256x64"}
+                       "tile": f"{self.tile[0]}x{self.tile[1]}x64", "tile_chosen_by": chosen_by}
 
     def setup(self, ct, torch, oracle, dev):
         import numpy as np

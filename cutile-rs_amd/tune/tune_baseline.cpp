@@ -76,6 +76,59 @@ bool tune_one(const std::string& kernel, const std::string& what, const std::fun
   return true;
 }
 
+// Tile shape AND variant for one GEMM problem: the candidates are all (tile, variant) pairs of the precompiled tiled
+// kernels (the reference's benchmark picks its tile by problem size, cutile-benchmarks/benches/gemm.rs:104-111).  The
+// tile of a launch is the caller's partition, so this winner is a record for callers: it is filed in the kernel's
+// record under the bucket "problem|<what>" with the parameters (variant, bm, bn); bench.py partitions z accordingly.
+bool tune_tiles(const std::string& kernel, const std::string& what, const std::string& dtype,
+                const std::function<Result<Unit>(int, int, const std::string&, const std::shared_ptr<Stream>&)>& launch) {
+  std::vector<tune::Config> configs;
+  for (auto& c : tune::variant_configs(kernel)) {
+    const std::string v = *c.str("variant");
+    int bm = 0, bn = 0, bk = 0;
+    char kind[16] = {0};
+    if (v.rfind(dtype + "_", 0) != 0 || sscanf(v.c_str() + dtype.size() + 1, "%dx%dx%d_%15s", &bm, &bn, &bk, kind) != 4) continue;
+    configs.push_back(tune::Config::make({{"variant", tune::ParamValue(v)}, {"bm", tune::ParamValue(bm)}, {"bn", tune::ParamValue(bn)}}));
+  }
+  printf("tuning %s  %s: %zu (tile, variant) candidates\n", kernel.c_str(), what.c_str(), configs.size());
+  bench::BenchOptions bo;
+  bo.warmup = std::chrono::milliseconds(20);
+  bo.rep = std::chrono::milliseconds(100);
+  bo.min_reps = 10;
+  bo.clear_bytes_override = 512u << 20;
+  auto tuned = tune::Autotuner(kernel + ":tiles:" + what).configs(configs).bench_options(bo).run(
+      g_stream, [&](const std::shared_ptr<Stream>& s, const tune::Config& c) -> Result<bench::BenchFn> {
+        const std::string v = *c.str("variant");
+        const int bm = (int)*c.integer("bm"), bn = (int)*c.integer("bn");
+        auto probe = launch(bm, bn, v, s);
+        if (probe.is_err()) return probe.error();
+        if (auto e = s->synchronize(); e.is_err()) return e.error();
+        return bench::BenchFn([&launch, v, bm, bn](const std::shared_ptr<Stream>& st) -> Result<Unit> { return launch(bm, bn, v, st); });
+      });
+  if (tuned.is_err() || !tuned.value().best) {
+    fprintf(stderr, "tune %s tiles (%s): no winner\n", kernel.c_str(), what.c_str());
+    return false;
+  }
+  const tune::Output& out = tuned.value();
+  const std::string best = *out.best->str("variant");
+  float best_ms = INFINITY;
+  size_t reps = 0;
+  for (auto& t : out.trials) {
+    std::string name;
+    for (auto& c : configs) if (c.id == t.config_id) name = *c.str("variant");
+    if (t.measured) printf("    %-40s median %8.4f ms  min %8.4f ms  (%zu reps)%s\n", name.c_str(), t.median_ms, t.min_ms, t.reps, name == best ? "   <- winner" : "");
+    if (t.measured && t.config_id == out.best->id && t.median_ms < best_ms) { best_ms = t.median_ms; reps = t.reps; }
+  }
+  auto it = g_records.find(kernel);
+  if (it == g_records.end()) {
+    auto ws = tune::Workspace::of_kernel(kernel, tune::space_hash(configs)).unwrap();
+    it = g_records.emplace(kernel, tune::Record(ws)).first;
+    it->second.gate = "do_bench median, 512 MiB flush, N(0,1) operands";
+  }
+  it->second.insert({"problem|" + what, *out.best, best_ms, reps, tune::variant_key(kernel, best).unwrap()});
+  return true;
+}
+
 template <class L>
 Result<Unit> enqueue(L launcher, const std::string& variant, const std::shared_ptr<Stream>& s) {
   auto r = variant.empty() ? std::move(launcher).async_on(s) : std::move(launcher).variant(variant).async_on(s);
@@ -99,6 +152,10 @@ int main(int argc, char** argv) {
     all &= tune_one("gemm", "bf16 M=N=K=" + std::to_string(s), [&](const std::string& v, const std::shared_ptr<Stream>& st) {
       return enqueue(gemm(z.partition_mut({256, 256}), x, y, s), v, st);
     });
+    all &= tune_tiles("gemm", "bf16|" + std::to_string(s) + "x" + std::to_string(s) + "x" + std::to_string(s), "bf16",
+                      [&](int bm, int bn, const std::string& v, const std::shared_ptr<Stream>& st) {
+                        return enqueue(gemm(z.partition_mut({bm, bn}), x, y, s), v, st);
+                      });
   }
   {   // GEMM f16 at 8192^3 (the operand type of the reference's own published GEMM figure)
     const int s = 8192;
