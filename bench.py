@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the tile-kernel path on one MI355X, against the kernel's roofline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--variant V] [--ceilings]
 
 A step is one launch of the hot-path kernel over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the bf16 GEMM at M = N = K = 8192
@@ -224,22 +224,24 @@ def tuned_tile(kernel, problem, default):
 class Gemm(Workload):
     unit, dtype, bound, peak_key = "TFLOP/s", "bf16 in / f32 acc / bf16 out", "mfma", "mfma_bf16"
 
-    def __init__(self, s):
-        self.s = s
-        self.name = f"gemm_bf16_{s}"
-        self.work = 2.0 * s ** 3
+    function = "gemm"          # the launcher --variant pins
+
+    def __init__(self, s, k=None, accumulate=True):
+        self.s, self.k, self.accumulate = s, k or s, accumulate
+        self.name = f"gemm_bf16_{s}" + (f"_k{k}" if k else "") + ("" if accumulate else "_new")
+        self.work = 2.0 * s * s * self.k
         # the tile is the caller's choice (the partition of z): taken from the tuner's sweep over tile shapes
-        self.tile, chosen_by = tuned_tile("gemm", f"bf16|{s}x{s}x{s}", (256, 256))
-        self.config = {"workload": f"GEMM bf16 M=N=K={s}, z += A·B, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 z",
+        self.tile, chosen_by = tuned_tile("gemm", f"bf16|{s}x{s}x{self.k}", (256, 256))
+        self.config = {"workload": f"GEMM bf16 M=N={s}, K={self.k}, z {'+=' if accumulate else '='} A·B, row-major A,B ~ N(0,1)/sqrt(K), f32 accumulate, bf16 z",
                        "tile": f"{self.tile[0]}x{self.tile[1]}x64", "tile_chosen_by": chosen_by}
 
     def setup(self, ct, torch, oracle, dev):
         import numpy as np
 
-        s = self.s
+        s, k = self.s, self.k
         self.ct = ct
-        self.ab = oracle.f32_to_bf16_bits(oracle.normal_f32((s, s), 5, 0, s ** -0.5))
-        self.bb = oracle.f32_to_bf16_bits(oracle.normal_f32((s, s), 6, 0, s ** -0.5))
+        self.ab = oracle.f32_to_bf16_bits(oracle.normal_f32((s, k), 5, 0, k ** -0.5))
+        self.bb = oracle.f32_to_bf16_bits(oracle.normal_f32((k, s), 6, 0, k ** -0.5))
         self.a, self.b = _td_bf16(torch, np, self.ab, dev), _td_bf16(torch, np, self.bb, dev)
         self.z = torch.zeros(s, s, dtype=torch.bfloat16, device=dev)
         self.zp = ct.partition(self.z, list(self.tile))
@@ -247,7 +249,7 @@ class Gemm(Workload):
     def launch(self):
         # z is read as the initial accumulator and written back, like the reference's
         # benchmark kernel (cutile-benchmarks/benches/gemm.rs:34-40: z.load(); mma...; z.store()).
-        self.ct.gemm(self.zp, self.a, self.b, self.s, accumulate=True)
+        self.ct.gemm(self.zp, self.a, self.b, self.k, accumulate=self.accumulate)
 
     def cpu_baseline(self, oracle, np, torch):
         rng = np.random.default_rng(7)
@@ -260,7 +262,7 @@ class Gemm(Workload):
         dt = time.perf_counter() - t0
         got = self.z[torch.from_numpy(rows).to(self.z.device)].float().cpu().numpy()
         rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
-        flops = 2.0 * len(rows) * self.s * self.s
+        flops = 2.0 * len(rows) * self.s * self.k
         return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
                 "sample": f"{len(rows)} of {self.s} output rows of the same problem (naive f32 loop)"}, \
                {"rel_l2_sampled_rows": rel, "tolerance": 1e-2, "ok": rel <= 1e-2}
@@ -269,6 +271,8 @@ class Gemm(Workload):
 class GemmPersistent(Gemm):
     """The reference's persistent form (cutile-examples/examples/persistent_gemm.rs): one tile block per CU walks
     the tiles of a mapped output partition in grouped order; zero initial accumulator (z is not read)."""
+
+    function = "gemm_persistent"
 
     def __init__(self, s, tile_blocks=256, group_m=8):
         super().__init__(s)
@@ -289,6 +293,7 @@ class Fmha(Workload):
     unit, dtype, bound, peak_key = "TFLOP/s", "bf16 io / f32 softmax+acc", "mfma", "mfma_bf16"
     b, h, s, d = 4, 32, 4096, 128
     bm = 256
+    function = "fmha"
 
     def __init__(self, causal):
         self.causal = causal
@@ -1001,7 +1006,10 @@ def make_workloads():
 
 # the reference's small example programs: only by name (--workload), never in the default run
 def make_extra_workloads():
-    return [BatchMatmul(), Matvec(), ExampleStream("relu"), ExampleStream("dropout"), ExampleStream("scale_ptr")]
+    # the example programs, and the GEMM at M = N = 8192 over a range of K with and without the accumulator read: the
+    # slope over K is the cost of a K tile, the intercept what a launch costs whatever its K
+    scan = [Gemm(8192, k, acc) for k in (1024, 2048, 4096) for acc in (True, False)] + [Gemm(8192, None, False)]
+    return [BatchMatmul(), Matvec(), ExampleStream("relu"), ExampleStream("dropout"), ExampleStream("scale_ptr")] + scan
 
 
 WARMUP_BUDGET_S = 0.05       # untimed launches continue until this much time has passed (the reference's budget is 25 ms)
@@ -1349,6 +1357,7 @@ def main():
     ap.add_argument("--workload", default="gemm_bf16_8192")
     ap.add_argument("--only", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / sampled parity leg")
+    ap.add_argument("--variant", default=None, help="pin this kernel variant for --workload's launcher (otherwise: tuning record, then table order)")
     ap.add_argument("--ceilings", action="store_true", help="also run the ceiling probes (cutile-rs_amd/bench/ceilings.hip), the vendor-library GEMM, "
                                                             "the kernels on zero operands and the launch-mode latencies")
     args = ap.parse_args()
@@ -1376,6 +1385,10 @@ def main():
     if head is None:
         sys.exit(f"unknown workload {args.workload}; choose from {[w.name for w in workloads + make_extra_workloads()]}")
     order = [head] + ([] if args.only else [w for w in workloads if w is not head])
+    if args.variant:
+        if not getattr(head, "function", None):
+            sys.exit(f"--variant: workload {head.name} does not name the launcher it pins")
+        ct.set_preferred_variant(head.function, args.variant)
     flush = torch.empty(FLUSH_BYTES // 4, dtype=torch.int32, device=dev)
     records = []
     for w in order:
