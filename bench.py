@@ -334,6 +334,7 @@ class Fmha(Workload):
 class MxGemm(Workload):
     name, unit, bound, peak_key = "mxfp8_gemm_8192", "TFLOP/s", "mfma", "mfma_fp8"
     dtype = "fp8 e4m3 x e8m0 block scale / f32 acc / bf16 out"
+    function = "linear_tile"
     s = 8192
     work = 2.0 * s ** 3
     tile = 256

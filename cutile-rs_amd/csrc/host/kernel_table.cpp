@@ -170,6 +170,7 @@ std::vector<KernelEntry> build_table() {
   gemm("bf16", 256, 256, 64, 2, 4, "r");
   gemm("bf16", 128, 128, 64, 2, 2, "r");
   gemm("bf16", 256, 256, 64, 2, 4, "q");   // "q" = the ring on v_mfma_f32_16x16x32
+  gemm("bf16", 128, 128, 64, 2, 2, "q");   // 80 KiB of stages: two workgroups per compute unit
   gemm("bf16", 256, 256, 64, 2, 4, "p");   // "p" = the same tile body, one workgroup per compute unit walking its tiles
   // "s" = the same ring streaming over the output tiles a workgroup walks (one workgroup per compute unit, whole
   // tiles only).  A family of four kernels: the variant itself reads z as the initial accumulator and moves z past
@@ -196,6 +197,7 @@ std::vector<KernelEntry> build_table() {
   gemm("f16", 256, 256, 64, 4, 2, "r");
   gemm("f16", 256, 256, 64, 2, 4, "r");
   gemm("f16", 256, 256, 64, 2, 4, "q");
+  gemm("f16", 128, 128, 64, 2, 2, "q");
   gemm("f16", 256, 256, 64, 2, 4, "p");
   stream_family("gemm", "f16", {"", "+cached", "+new", "+new+cached"});
   gemm("bf16f32", 128, 128, 64, 2, 2);
@@ -330,16 +332,18 @@ std::vector<KernelEntry> build_table() {
   add("splitk_reduce_merge", "f16", "splitk_reduce_merge_entry__f16", IMG_FMHA, 256, 0, 0, 0, 0, 0, "f16", 0, 3);
 
   // ---- MXFP8 GEMM: LDS = 2 stages x (BM + BN) x 128 bytes ----
-  // "d" = global->LDS direct, pipelined; scales staged in blocks of four K tiles (16 bytes per row, two blocks)
+  // "d", "e" = global->LDS direct, pipelined; scales staged in blocks of four K tiles (16 bytes per row, two blocks)
   auto mx = [&](const char* out, int bm, int bn, int wvm, int wvn, const char* kind = "w") {
     std::string v = std::string("mxfp8_") + out + "_" + std::to_string(bm) + "x" + std::to_string(bn) + "x128_" + kind +
                     std::to_string(wvm) + "x" + std::to_string(wvn);
     add("linear_tile", keep(v), keep("linear_tile_entry__" + v), IMG_MXGEMM, (uint32_t)(wvm * wvn * 64),
-        (uint32_t)(2 * (bm + bn) * (128 + (kind[0] == 'd' ? 16 : 0))), bm, bn, 128, 0, out, 0, 2);
+        (uint32_t)(2 * (bm + bn) * (128 + (kind[0] == 'd' || kind[0] == 'e' ? 16 : 0))), bm, bn, 128, 0, out, 0, 2);
   };
   mx("bf16", 256, 256, 4, 2, "d");
   mx("bf16", 256, 256, 2, 4, "d");
   mx("f32", 256, 256, 2, 4, "d");
+  mx("bf16", 256, 256, 4, 2, "e");   // "e" = the direct pipeline on v_mfma_scale_f32_16x16x128_f8f6f4
+  mx("f32", 256, 256, 4, 2, "e");
   mx("bf16", 256, 256, 2, 2);
   mx("bf16", 256, 256, 2, 4);
   mx("bf16", 128, 128, 2, 2);

@@ -1602,6 +1602,10 @@ GEMM_RING_KERNEL_F16(f16_256x256x64_r4x2, 256, 256, 4, 2)
   }
 GEMM_RING16_KERNEL(bf16_256x256x64_q2x4, 256, 256, 2, 4, __bf16, __bf16)
 GEMM_RING16_KERNEL(f16_256x256x64_q2x4, 256, 256, 2, 4, _Float16, _Float16)
+// 128 x 128 tiles on four wavefronts: 80 KiB of stages, so two workgroups share a compute unit and one's main loop
+// runs under the other's prologue and epilogue (for launches of about one 256 x 256 tile per compute unit)
+GEMM_RING16_KERNEL(bf16_128x128x64_q2x2, 128, 128, 2, 2, __bf16, __bf16)
+GEMM_RING16_KERNEL(f16_128x128x64_q2x2, 128, 128, 2, 2, _Float16, _Float16)
 #define GEMM_RING16_PERSISTENT_KERNEL(NAME, BM, BN, WVM, WVN, T)                                 \
   extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                  \
       gemm_persistent_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, MappedArg m) { \

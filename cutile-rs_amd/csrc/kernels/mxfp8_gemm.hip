@@ -487,6 +487,242 @@ struct MxGemmDirect {
   }
 };
 
+// ---- the direct pipeline on v_mfma_scale_f32_16x16x128_f8f6f4 ("e") ------------------------------------
+// The matrix kernels here run against the chip's power limit, and per flop the 16 x 16 x 128 form writes half as many
+// accumulator values as 32 x 32 x 64: a loop of nothing but scaled fp8 MFMAs on random operand bits sustains 4250
+// TFLOP/s with it against 3810 (equal, 4960 - 4990, on constant operands).  Operand layout (measured on gfx950 with
+// one-hot products): a lane (row r = lane % 16, group g = lane / 16) holds 32 bytes of its row; the first 16 are K
+// positions 16 g .. 16 g + 15 of the instruction's 128, the last 16 are 64 + 16 g .. 64 + 16 g + 15; lane group s
+// supplies, in byte 0 of its scale register, the scale of K block s (positions 32 s .. 32 s + 31) of its row.  The
+// result is laid out like v_mfma_f32_16x16x32's.
+// One instruction covers a whole K tile, so a tile is 32 MFMAs (4 x row blocks by 8 y row blocks of 16): for each y
+// block in turn, the four x blocks.  Registers hold the four x fragments and two y fragments (slot = y block % 2): a
+// y fragment is reloaded with y block tn + 2 as its last MFMA issues, the x fragments with the next tile's during the
+// last y block, four MFMAs (the other wavefront of the SIMD issues as many in between) before their next use.
+// Hand-over of the stages five MFMAs before the end of the tile; the refill of the stage just drained is dealt out over
+// those MFMAs.
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+struct MxGemmDirect16 {
+  static constexpr int BK = 128;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 16, TN = WN / 16;
+  static constexpr int kAInstr = BM / 8 / kWaves, kBInstr = BN / 8 / kWaves;   // 1 KiB = 8 rows of 128 bytes
+  static constexpr int kSInstr = (BM + BN) / 64 / kWaves;                     // 1 KiB = 64 rows x 16 scale bytes
+  static constexpr int kABytes = BM * BK, kBBytes = BN * BK;
+  static constexpr int kScaleBytes = (BM + BN) * 16;                          // 4 K tiles of scales per row
+  static constexpr int kStageBytes = kABytes + kBBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes + 2 * kScaleBytes;
+  static constexpr int NB = TM * TN;
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0 && (BM + BN) % (64 * kWaves) == 0 && BM % 64 == 0,
+                "tile must split evenly");
+  static_assert(TN % 2 == 0 && TN >= 4 && TM >= 2, "two y fragment slots: an even number of y blocks keeps a block in its slot from tile to tile");
+
+  __device__ static __forceinline__ int lds_off(int r, int u) { return r * BK + ((u ^ ((r >> 1) & 7)) << 4); }
+
+  __device__ static void run(const PartitionArg<2>& z, const TensorArg<2>& x, const TensorArg<2>& y,
+                             const TensorArg<2>& xs, const TensorArg<2>& ys, float alpha, const TileGrid& g) {
+    // The y stages come first in LDS (the larger alignment sorts them to the front): every y fragment read then
+    // reaches its 16 rows through the instruction's 16-bit offset from ONE pair of per-lane addresses, whichever the
+    // stage.  The x stages lie beyond that reach; their four fragments per tile add the stage's address to the lane's
+    // offset at each read (an opaque copy keeps the compiler from carrying one address register per fragment and stage).
+    __shared__ __attribute__((aligned(4096))) unsigned char ys0[kBBytes];
+    __shared__ __attribute__((aligned(4096))) unsigned char ys1[kBBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs0[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char xs1[kABytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char scales0[kScaleBytes];   // scale blocks 0, 2, 4 ...
+    __shared__ __attribute__((aligned(1024))) unsigned char scales1[kScaleBytes];   // scale blocks 1, 3, 5 ...
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l16 = lane & 15, grp = lane >> 4;
+    uint32_t pm, pn;
+    tile_coords(g.x, g.y, &pm, &pn);
+    const int32_t M = x.shape[0], N = y.shape[0], K = min(x.shape[1], y.shape[1]);
+    const int32_t lda = x.strides[0], ldb = y.strides[0];
+    const int32_t ldsa = xs.strides[0], ldsb = ys.strides[0];
+    const int32_t row0 = pm * BM, col0 = pn * BN;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(x.ptr, (uint32_t)((int64_t)(M - 1) * lda + x.shape[1]));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(y.ptr, (uint32_t)((int64_t)(N - 1) * ldb + y.shape[1]));
+    const __amdgpu_buffer_rsrc_t rsa = make_rsrc(xs.ptr, (uint32_t)((int64_t)(xs.shape[0] - 1) * ldsa + xs.shape[1]));
+    const __amdgpu_buffer_rsrc_t rsb = make_rsrc(ys.ptr, (uint32_t)((int64_t)(ys.shape[0] - 1) * ldsb + ys.shape[1]));
+    constexpr uint32_t kOob = 0x80000000u;
+    const int k_tiles = K / BK;
+
+    // Global side of the fetches: as in MxGemmDirect (per lane, K tile 0; the K advance is scalar).
+    uint32_t a_goff[kAInstr], b_goff[kBInstr], s_goff[kSInstr];
+#pragma unroll
+    for (int i = 0; i < kAInstr; ++i) {
+      const int r = (wave * kAInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      a_goff[i] = (row0 + r < M) ? (uint32_t)((int64_t)(row0 + r) * lda + u * 16) : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < kBInstr; ++i) {
+      const int r = (wave * kBInstr + i) * 8 + (lane >> 3);
+      const int u = (lane & 7) ^ ((r >> 1) & 7);
+      b_goff[i] = (col0 + r < N) ? (uint32_t)((int64_t)(col0 + r) * ldb + u * 16) : kOob;
+    }
+#pragma unroll
+    for (int i = 0; i < kSInstr; ++i) {
+      const int sidx = wave * kSInstr + i;
+      const bool is_x = sidx < BM / 64;
+      const int r = (is_x ? sidx : sidx - BM / 64) * 64 + lane;
+      s_goff[i] = is_x ? ((row0 + r < M) ? (uint32_t)((int64_t)(row0 + r) * ldsa) : kOob)
+                       : ((col0 + r < N) ? (uint32_t)((int64_t)(col0 + r) * ldsb) : kOob);
+    }
+    constexpr int NF = kAInstr + kBInstr;
+    auto scale_block = [&](int32_t tile) -> unsigned char* { return ((tile >> 2) & 1) ? scales1 : scales0; };
+    auto fetch_one = [&](unsigned char* xs, unsigned char* ys, int32_t kt, int i) {
+      const bool wanted = kt < k_tiles;   // past the last tile: out-of-range offsets, zeros
+      const int32_t k0 = wanted ? kt * BK : 0;
+      if (i < kAInstr) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (LDS_PTR(void))(xs + (wave * kAInstr + i) * 1024), 16,
+                                                 wanted ? a_goff[i] : kOob, k0, 0, 0);
+      } else if (i < kAInstr + kBInstr) {
+        const int b = i - kAInstr;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (LDS_PTR(void))(ys + (wave * kBInstr + b) * 1024), 16,
+                                                 wanted ? b_goff[b] : kOob, k0, 0, 0);
+      } else {
+        const int si = i - kAInstr - kBInstr;
+        const int sidx = wave * kSInstr + si;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(sidx < BM / 64 ? rsa : rsb,
+                                                 (LDS_PTR(void))(scale_block(kt) + sidx * 1024), 16,
+                                                 wanted ? s_goff[si] : kOob, k0 / 32, 0, 0);
+      }
+    };
+
+    // LDS side: the lane's two 16-byte units of its row (K positions 16 g .. and 64 + 16 g ..) and its scale byte.
+    const int a_lo = lds_off(wm * WM + l16, grp), a_hi = lds_off(wm * WM + l16, 4 + grp);               // + tm * 16 rows
+    const int b_lo = lds_off(wn * WN + l16, grp), b_hi = lds_off(wn * WN + l16, 4 + grp);                 // + tn * 16 rows
+    const int sa_addr = (wm * WM + l16) * 16 + grp;                                 // + tm * 16 rows, + 4 * (tile % 4)
+    const int sb_addr = BM * 16 + (wn * WN + l16) * 16 + grp;                       // + tn * 16 rows
+    auto read_frag = [&](const unsigned char* stage, int lo, int hi, int blk, bool far) -> i32x8 {
+      if (far) asm volatile("" : "+v"(lo), "+v"(hi));
+      u32x4 l = *reinterpret_cast<const u32x4*>(stage + lo + blk * 16 * BK);
+      u32x4 h = *reinterpret_cast<const u32x4*>(stage + hi + blk * 16 * BK);
+      return i32x8{(int)l.x, (int)l.y, (int)l.z, (int)l.w, (int)h.x, (int)h.y, (int)h.z, (int)h.w};
+    };
+
+    f32x4_acc acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[tn][tm][v] = 0.0f;
+
+    i32x8 af[TM], bfr[2];       // x fragments of the tile; y fragments (slot = y block % 2)
+    int sa[TM], sb[2];          // their scales (byte 0)
+    // A fragment's scale is one byte read straight from the staged scale rows (lane group g reads byte g of the row's
+    // dword for the tile: no shift) by an instruction the compiler does not see as a memory access: the scale rows
+    // sit in two buffers picked at run time, and a visible read of "either" would be made to wait for every fetch in
+    // flight.  The reads are ordered by the hand-over like all the others, and each is issued in front of its
+    // fragment's own reads, whose wait covers it.  `base` = the scale block's LDS address plus the lane's row and
+    // byte; the row block and the tile's place in the scale block are the instruction's offset.
+    // (The four lane groups read four bytes of one dword, which the LDS counts as a bank conflict, two cycles a read;
+    // reading the dwords instead, all twelve of a tile behind the hand-over, packed with v_perm_b32 and picked by the
+    // MFMA's op_sel, was built and measured slower: the same conflicts, and a tile's worth of LDS latency exposed.)
+    auto read_scale = [&](uint32_t base, int off) -> int {
+      int v;
+      asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(v) : "v"(base), "n"(off));
+      return v;
+    };
+    auto scale_base = [&](const unsigned char* blk, int lane_addr) -> uint32_t { return (uint32_t)(uintptr_t)blk + (uint32_t)lane_addr; };
+    auto load_a = [&](const unsigned char* xs, uint32_t sbase, int ph, int tm) {
+      sa[tm] = read_scale(sbase, tm * 16 * 16 + 4 * ph);
+      af[tm] = read_frag(xs, a_lo, a_hi, tm, true);
+    };
+    auto load_b = [&](const unsigned char* ys, uint32_t sbase, int ph, int tn) {
+      sb[tn & 1] = read_scale(sbase, tn * 16 * 16 + 4 * ph);
+      bfr[tn & 1] = read_frag(ys, b_lo, b_hi, tn, false);
+    };
+
+    // Prologue: tile 0 (and 1) on their way, the first fragments and scales in registers.
+    if (k_tiles > 0) {
+#pragma unroll
+      for (int i = 0; i < NF + kSInstr; ++i) fetch_one(xs0, ys0, 0, i);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < NF; ++i) fetch_one(xs1, ys1, 1, i);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) load_a(xs0, scale_base(scales0, sa_addr), 0, tm);
+#pragma unroll
+      for (int tn = 0; tn < 2; ++tn) load_b(ys0, scale_base(scales0, sb_addr), 0, tn);
+    }
+    // The hand-over sits before the last MFMA of the last y block but one: the reload behind that MFMA is the first
+    // read of the next tile's stage, and the last read of the current one (y block TN - 1, requested behind the MFMAs of
+    // block TN - 3) has had a block's MFMAs to complete, so the wait in front of the barrier finds it done.
+    constexpr int kHandOverAt = (TN - 1) * TM - 1;
+    constexpr int kFetchSlots = NB - kHandOverAt;
+    // `with_scales`: tile kt+2 opens a scale block (kt + 2 is a multiple of 4).
+    // `phase` = kt % 4 (the tile's place in its scale block), known where the call is written.
+    auto k_tile = [&](unsigned char* x_cur, unsigned char* y_cur, const unsigned char* x_nxt, const unsigned char* y_nxt, int kt,
+                      auto with_scales, auto phase) {
+      constexpr int PH = decltype(phase)::value;
+      constexpr int NFT = NF + (decltype(with_scales)::value ? kSInstr : 0);
+      constexpr int PHN = (PH + 1) & 3;
+      const uint32_t sb_cur = scale_base(scale_block(kt), sb_addr);
+      const uint32_t sa_nxt = scale_base(scale_block(kt + 1), sa_addr), sb_nxt = scale_base(scale_block(kt + 1), sb_addr);
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          const int j = tn * TM + tm;
+          if (j == kHandOverAt) {
+            __builtin_amdgcn_s_waitcnt(0);   // own reads of `cur` done, own share of tile kt+1 landed
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (j >= kHandOverAt) {
+#pragma unroll
+            for (int i = 0; i < NFT; ++i)
+              if (i * kFetchSlots / NFT == j - kHandOverAt) fetch_one(x_cur, y_cur, kt + 2, i);
+          }
+          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfr[tn & 1], af[tm], acc[tn][tm], 0, 0, 0, sb[tn & 1], 0, sa[tm]);
+          __builtin_amdgcn_sched_barrier(0);   // a reload must follow the last reader, or it needs registers of its own
+          if (tn == TN - 1) load_a(x_nxt, sa_nxt, PHN, tm);       // x block tm has done its last MFMA of this tile
+          if (tm == TM - 1) {                                       // so has y block tn: its slot takes y block tn + 2
+            if (tn + 2 < TN) load_b(y_cur, sb_cur, PH, tn + 2);
+            else load_b(y_nxt, sb_nxt, PHN, tn + 2 - TN);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    };
+    int kt = 0;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
+    using P3 = std::integral_constant<int, 3>;
+    for (; kt + 4 <= k_tiles; kt += 4) {
+      k_tile(xs0, ys0, xs1, ys1, kt, std::false_type{}, P0{});
+      k_tile(xs1, ys1, xs0, ys0, kt + 1, std::false_type{}, P1{});
+      k_tile(xs0, ys0, xs1, ys1, kt + 2, std::true_type{}, P2{});
+      k_tile(xs1, ys1, xs0, ys0, kt + 3, std::false_type{}, P3{});
+    }
+    if (kt < k_tiles) k_tile(xs0, ys0, xs1, ys1, kt, std::false_type{}, P0{});
+    if (kt + 1 < k_tiles) k_tile(xs1, ys1, xs0, ys0, kt + 1, std::false_type{}, P1{});
+    if (kt + 2 < k_tiles) k_tile(xs0, ys0, xs1, ys1, kt + 2, std::true_type{}, P2{});
+
+    // Every wavefront is past its operand reads and every fetch has landed: the stages are free to carry the output.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[tn][tm][v] *= alpha;
+    static_assert(kWaves == 8 && 2 * kEpilogueBytesPerWave<WN> <= kABytes && 2 * kEpilogueBytesPerWave<WN> <= kBBytes, "two output bands per stage array");
+    unsigned char* band = (wave < 2 ? ys0 : wave < 4 ? ys1 : wave < 6 ? xs0 : xs1) + (wave & 1) * kEpilogueBytesPerWave<WN>;
+    store_tile_staged16<TM, TN, OutT>(acc, band, (OutT*)z.ptr, z.strides[0], z.shape[0], z.shape[1], row0 + wm * WM,
+                                      col0 + wn * WN, lane, 0);
+  }
+};
+
 }  // namespace
 
 #define MX_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                                   \
@@ -514,3 +750,13 @@ MX_KERNEL(mxfp8_f32_64x64x128_w1x1, 64, 64, 1, 1, float)
 MX_DIRECT_KERNEL(mxfp8_bf16_256x256x128_d2x4, 256, 256, 2, 4, __bf16)
 MX_DIRECT_KERNEL(mxfp8_bf16_256x256x128_d4x2, 256, 256, 4, 2, __bf16)
 MX_DIRECT_KERNEL(mxfp8_f32_256x256x128_d2x4, 256, 256, 2, 4, float)
+
+#define MX_DIRECT16_KERNEL(NAME, BM, BN, WVM, WVN, OUT_T)                                          \
+  extern "C" __global__ void __launch_bounds__(WVM* WVN * 64)                                     \
+      linear_tile_entry__##NAME(PartitionArg<2> z, TensorArg<2> x, TensorArg<2> y, TensorArg<2> xs, \
+                                TensorArg<2> ys, float alpha, TileGrid g) {                        \
+    MxGemmDirect16<BM, BN, WVM, WVN, OUT_T>::run(z, x, y, xs, ys, alpha, g);                       \
+  }
+
+MX_DIRECT16_KERNEL(mxfp8_bf16_256x256x128_e4x2, 256, 256, 4, 2, __bf16)
+MX_DIRECT16_KERNEL(mxfp8_f32_256x256x128_e4x2, 256, 256, 4, 2, float)

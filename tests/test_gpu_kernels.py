@@ -281,7 +281,7 @@ def test_softmax_f32(ct, dev, m, n, bm, bn):
 
 
 # ---- K4: bf16 GEMM --------------------------------------------------------------------------
-GEMM_VARIANTS = ["bf16_256x256x64_q2x4", "bf16_256x256x64_r2x4", "bf16_256x256x64_r4x2", "bf16_128x128x64_r2x2", "bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
+GEMM_VARIANTS = ["bf16_256x256x64_q2x4", "bf16_128x128x64_q2x2", "bf16_256x256x64_r2x4", "bf16_256x256x64_r4x2", "bf16_128x128x64_r2x2", "bf16_256x256x64_d4x2", "bf16_256x256x64_d2x4", "bf16_128x128x64_d2x2", "bf16_256x256x64_w2x2", "bf16_256x256x64_w2x4", "bf16_256x256x64_w4x2", "bf16_256x128x64_w2x2",
                  "bf16_128x256x64_w2x2", "bf16_128x128x64_w2x2", "bf16_64x128x64_w2x2"]
 
 
@@ -300,7 +300,7 @@ def test_gemm_bf16_variants(ct, dev, variant):
     np.testing.assert_allclose(got, ref, rtol=1.6e-2, atol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["bf16_256x256x64_q2x4", "bf16_256x256x64_r2x4", "bf16_128x128x64_r2x2"])
+@pytest.mark.parametrize("variant", ["bf16_256x256x64_q2x4", "bf16_128x128x64_q2x2", "bf16_256x256x64_r2x4", "bf16_128x128x64_r2x2"])
 @pytest.mark.parametrize("k_tiles", [1, 2, 3, 6, 7, 13])
 def test_gemm_ring_pipeline_every_loop_shape(ct, dev, variant, k_tiles):
     # the ring pipeline repeats its stage names every 6 K tiles: cover the unrolled
@@ -495,6 +495,14 @@ def test_mxfp8_all_ones_known_answer(ct, dev):
     (328, 520, 384, 256, torch.float32, "mxfp8_f32_256x256x128_d2x4"),
     (520, 328, 896, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_d2x4"),
     (328, 520, 896, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_d4x2"),
+    # the 16 x 16 x 128 matrix instruction: one, two, three, five and eight K tiles (every place in a scale block,
+    # the loop of four and its remainders); M, N off the tile
+    (256, 256, 128, 256, torch.float32, "mxfp8_f32_256x256x128_e4x2"),
+    (256, 512, 256, 256, torch.float32, "mxfp8_f32_256x256x128_e4x2"),
+    (328, 520, 384, 256, torch.float32, "mxfp8_f32_256x256x128_e4x2"),
+    (520, 328, 640, 256, torch.float32, "mxfp8_f32_256x256x128_e4x2"),
+    (328, 520, 896, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_e4x2"),
+    (512, 768, 1024, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_e4x2"),
     (512, 512, 1024, 256, torch.bfloat16, "mxfp8_bf16_256x256x128_w2x2"),
 ])
 def test_mxfp8_random_blocks(ct, dev, m, n, k, tile, out_dtype, variant):
