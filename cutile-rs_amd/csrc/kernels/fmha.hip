@@ -409,7 +409,10 @@ struct FmhaPingPong {
     __shared__ __attribute__((aligned(1024))) unsigned char vb1[kTileBytes];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const bool late = wave >= kWaves / 2;   // the half of the workgroup that runs one interval behind
+    // The half of the workgroup that runs one interval behind.  Causal: the upper rows (wavefronts 0-3), which see
+    // fewer keys: they finish their last tile while the lower rows still have diagonal tiles to do, and what is left
+    // of the workgroup's run is the leading half's alone (see tc_h below).
+    const bool late = causal ? wave < kWaves / 2 : wave >= kWaves / 2;
     const int l32 = lane & 31, half = lane >> 5;
     const int grp = lane >> 4, l16 = lane & 15;
 
@@ -451,12 +454,17 @@ struct FmhaPingPong {
       qf[ks] = __builtin_bit_cast(vec8, w);
     }
 
-    int32_t tc = (k_len + BN - 1) / BN;
+    // tc: KV tiles the workgroup fetches.  tc_h: those this half of it (128 query rows) multiplies; under a causal mask
+    // the upper half's rows end up to two tiles of keys before the lower half's, and a tile whose keys no row of the
+    // half sees adds nothing to it.  mask_start: the first tile in which some key is hidden from some row of the half.
+    int32_t tc = (k_len + BN - 1) / BN, tc_h = tc;
     int32_t mask_start = k_len / BN;
     if (causal) {
       const int32_t m_end = input_pos + (q_tile + 1) * BM;
-      mask_start = min((input_pos + q_tile * BM) / BN, k_len / BN);
       tc = (min(m_end, k_len) + BN - 1) / BN;
+      const int32_t h0 = input_pos + q_tile * BM + (wave / (kWaves / 2)) * (BM / 2);   // position of the half's first query
+      mask_start = min(h0 / BN, k_len / BN);
+      tc_h = (min(h0 + BM / 2, k_len) + BN - 1) / BN;
     }
 
     // Global side of the tile fetches: the LDS side of a direct load is lane
@@ -642,13 +650,26 @@ struct FmhaPingPong {
           fetch_k(kc, j + 2, j + 2 < tc);
           fetch_v(vn, j + 1);
         };
-        if (LATE && !LAST) refill();
+        // (the late half's last tile may not be the workgroup's: its share of the fetches goes on)
+        const bool fetch_on = !LAST || (LATE && j + 1 < tc);
+        if (LATE && fetch_on) refill();
         softmax_segment(j);
         if (!LATE) wait_fetches();
         interval_end();
         if (!LATE && !LAST) refill();
         matrix_segment(vc, kn, std::integral_constant<bool, !LAST>{});
-        if (LATE && !LAST) wait_fetches();
+        if (LATE && fetch_on) wait_fetches();
+        interval_end();
+      };
+      // A tile the late half fetches its share of and does not multiply: the same requests, waits and barriers.
+      auto idle_tile = [&](int32_t j, unsigned char* kc, unsigned char* vn) {
+        const bool fetch_on = j + 1 < tc;
+        if (fetch_on) {
+          fetch_k(kc, j + 2, j + 2 < tc);
+          fetch_v(vn, j + 1);
+        }
+        interval_end();
+        if (fetch_on) wait_fetches();
         interval_end();
       };
       fetch_k(kb1, 1, tc > 1);
@@ -657,16 +678,22 @@ struct FmhaPingPong {
       first_segment(kb0);
       if (LATE) wait_fetches();
       interval_end();
+      const int32_t mine = LATE ? tc_h : tc;   // the leading half's rows reach the workgroup's last tile
       int32_t j = 0;
-      for (; j + 2 < tc; j += 2) {
+      for (; j + 2 < mine; j += 2) {
         tile(j, kb0, kb1, vb0, vb1, std::false_type{});
         tile(j + 1, kb1, kb0, vb1, vb0, std::false_type{});
       }
-      if (tc - j == 2) {
+      if (mine - j == 2) {
         tile(j, kb0, kb1, vb0, vb1, std::false_type{});
         tile(j + 1, kb1, kb0, vb1, vb0, std::true_type{});
       } else {
         tile(j, kb0, kb1, vb0, vb1, std::true_type{});
+      }
+      if (LATE) {
+        for (j = mine; j < tc; ++j) {
+          if (j & 1) idle_tile(j, kb1, vb0); else idle_tile(j, kb0, vb1);
+        }
       }
       if (!LATE) interval_end();         // pairs with the late half's last interval
     };
