@@ -449,6 +449,14 @@ def test_fmha_pingpong_every_loop_shape(ct, dev, s, causal, input_pos):
     assert _fmha_case(ct, dev, 1, 4, 2, s, 128, 256, causal, input_pos, variant="bf16_256x64x128_pp", seed=431) <= 2e-2
 
 
+@pytest.mark.parametrize("s,input_pos", [(256, 0), (320, 0), (448, 64), (512, 40), (704, 100), (832, 130), (576, 200)])
+def test_fmha_pingpong_causal_halves_stop_at_their_own_last_tile(ct, dev, s, input_pos):
+    # under a causal mask the upper 128 rows of a 256-row query tile run as the trailing half of the workgroup and
+    # multiply only the KV tiles they can see (zero, one or two fewer than the lower rows, at either parity of the
+    # unrolled-by-two pipeline); positions that start inside a KV tile, and key ranges that end before the queries do
+    assert _fmha_case(ct, dev, 1, 2, 1, s, 128, 256, True, input_pos, variant="bf16_256x64x128_pp", seed=451 + s) <= 2e-2
+
+
 def test_fmha_pingpong_f16(ct, dev):
     assert _fmha_case(ct, dev, 1, 2, 2, 640, 128, 256, True, 0, dtype=torch.float16, variant="f16_256x64x128_pp") <= 2e-2
 
