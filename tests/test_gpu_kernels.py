@@ -329,6 +329,24 @@ def test_gemm_16x16x32_ring_masks_a_ragged_last_k_tile(ct, dev, k):
     np.testing.assert_allclose(z.float().cpu().numpy(), ref, rtol=1.6e-2, atol=2e-3)
 
 
+@pytest.mark.parametrize("variant,k,accumulate", [("bf16_128x128x64_q2x2", 200, False), ("bf16_128x128x64_q2x2", 448, True),
+                                                  ("f16_128x128x64_q2x2", 328, True)])
+def test_gemm_16x16x32_ring_at_128x128(ct, dev, variant, k, accumulate):
+    # the same ring on four wavefronts (two workgroups to a compute unit): ragged K, ragged M and N, z as the initial
+    # accumulator, both 16-bit operand types
+    f16 = variant.startswith("f16")
+    bits, to_dev, to_f32 = (normal_f16_bits, to_dev_f16, oracle.f16_bits_to_f32) if f16 else (normal_bf16_bits, to_dev_bf16, oracle.bf16_bits_to_f32)
+    m, n = 300, 520
+    a, b = bits((m, k), 351 + k, k ** -0.5), bits((k, n), 352 + k, k ** -0.5)
+    z0 = bits((m, n), 353 + k, 0.5)
+    z = to_dev(z0, dev).clone()
+    ct.gemm(ct.partition(z, [128, 128]), to_dev(a, dev), to_dev(b, dev), k, accumulate=accumulate, generics=["f16" if f16 else "bf16", 128, 128, 8],
+            variant=variant)
+    sync()
+    ref = to_f32(a).astype(np.float64) @ to_f32(b).astype(np.float64) + (to_f32(z0) if accumulate else 0.0)
+    np.testing.assert_allclose(z.float().cpu().numpy(), ref, rtol=1.6e-2, atol=4e-3)
+
+
 def test_gemm_ring_variant_rejects_ragged_k(ct, dev):
     m = n = 256
     k = 96
